@@ -1,0 +1,318 @@
+#!/usr/bin/env python3
+"""Benchmark of the row-wise operator kernels on one MI355X.
+
+Default run (the line the driver records): the Llama-7B token shape —
+RMSNorm forward + backward, bf16, 32768 packed tokens x hidden 4096, eps 1e-6.
+One "step" is one forward + one backward over that batch, inputs resident in
+HBM.  `value` is algorithmic GB/s of the whole step (every input read once,
+every output written once).  The `roofline` object is for the dominant kernel
+of the step (the backward row kernel), timed with HIP events recorded around
+that kernel on its stream; `cpu_baseline` is the oracle's fp32 CPU port timed
+on a bounded sample of the same rows.
+
+`--all` additionally times every kernel of every BASELINE configuration and
+adds the table as `kernels` (also printed to stderr).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+IGNORE = -100
+
+
+def _load():
+    hk = importlib.import_module("hotspa-ae_amd")
+    hk.lib()  # fails loudly when the HIP library has not been built
+    return hk
+
+
+# ---------------------------------------------------------------------------
+# cases: each builds `nsets` rotating buffer sets and returns (launch(i), bytes, rows, main-kernel name)
+# ---------------------------------------------------------------------------
+def _randn(torch, shape, dtype, std=1.0, seed=0):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    n = 1
+    for s in shape:
+        n *= s
+    out = torch.empty(shape, dtype=dtype, device="cuda")
+    flat = out.view(-1)
+    step = 1 << 26
+    for o in range(0, n, step):  # chunked: no full-size fp32 temporary
+        m = min(step, n - o)
+        flat[o:o + m] = (torch.randn(m, generator=g, device="cuda", dtype=torch.float32) * std).to(dtype)
+    return out
+
+
+def _uniform(torch, shape, dtype, lo, hi, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return (torch.rand(shape, generator=g, device="cuda", dtype=torch.float32) * (hi - lo) + lo).to(dtype)
+
+
+def case_rmsnorm(hk, torch, nsets, which):
+    rows, cols, eps = 32768, 4096, 1e-6
+    bf = torch.bfloat16
+    sets = []
+    for i in range(nsets):
+        s = dict(x=_randn(torch, (rows, cols), bf, 1.0, 402 + 10 * i), dz=_randn(torch, (rows, cols), bf, 1.0, 404 + 10 * i),
+                 z=torch.empty((rows, cols), dtype=bf, device="cuda"), dx=torch.empty((rows, cols), dtype=bf, device="cuda"),
+                 mu=torch.empty(rows, device="cuda"), rs=torch.empty(rows, device="cuda"))
+        sets.append(s)
+    w = _uniform(torch, (cols,), bf, 0.8, 1.2, 403)
+    dg, db = torch.empty_like(w), torch.empty_like(w)
+    ws = torch.empty(max(1, hk.norm_bwd_workspace_bytes(8, rows, cols) // 4), device="cuda")
+    for s in sets:
+        hk.dropout_add_ln_fwd(s["x"], None, w, None, s["z"], None, s["mu"], s["rs"], eps, True)
+    fwd_bytes = 2 * rows * cols * 2 + cols * 2 + rows * 4 + rows * 4
+    bwd_bytes = 3 * rows * cols * 2 + rows * 4 + cols * 2 + 2 * cols * 2
+
+    def fwd(i):
+        s = sets[i % nsets]
+        hk.dropout_add_ln_fwd(s["x"], None, w, None, s["z"], None, s["mu"], s["rs"], eps, True)
+
+    def bwd(i):
+        s = sets[i % nsets]
+        hk.dropout_add_ln_bwd(s["dz"], None, s["x"], s["mu"], s["rs"], w, s["dx"], None, dg, db, True, workspace=ws)
+
+    if which == "fwd":
+        return fwd, fwd_bytes, rows
+    if which == "bwd":
+        return bwd, bwd_bytes, rows
+    return (lambda i: (fwd(i), bwd(i))), fwd_bytes + bwd_bytes, rows
+
+
+def case_layernorm(hk, torch, nsets, which, cfg):
+    if cfg == "C1":
+        rows, cols, dt, eps = 8192, 4096, torch.float32, 1e-5
+    else:
+        rows, cols, dt, eps = 16384, 5120, torch.bfloat16, 1e-5
+    es = 4 if dt == torch.float32 else 2
+    sets = []
+    for i in range(nsets):
+        sets.append(dict(x=_randn(torch, (rows, cols), dt, 1.0, 101 + 10 * i), dy=_randn(torch, (rows, cols), dt, 1.0, 514 + 10 * i),
+                         y=torch.empty((rows, cols), dtype=dt, device="cuda"), dx=torch.empty((rows, cols), dtype=dt, device="cuda"),
+                         mean=torch.empty(rows, device="cuda"), rstd=torch.empty(rows, device="cuda")))
+    g = _uniform(torch, (cols,), dt, 0.5, 1.5, 102)
+    b = (_randn(torch, (cols,), torch.float32, 0.1, 103)).to(dt)
+    dg, db = torch.empty_like(g), torch.empty_like(g)
+    ws = torch.empty(max(1, hk.norm_bwd_workspace_bytes(hk.dtype_code(g), rows, cols) // 4), device="cuda")
+    for s in sets:
+        hk.layer_norm_fwd(s["x"], g, b, s["y"], s["mean"], s["rstd"], eps, stat_kind=1)
+    fwd_bytes = 2 * rows * cols * es + 2 * cols * es + 2 * rows * 4
+    bwd_bytes = 3 * rows * cols * es + 2 * rows * 4 + cols * es + 2 * cols * es
+
+    def fwd(i):
+        s = sets[i % nsets]
+        hk.layer_norm_fwd(s["x"], g, b, s["y"], s["mean"], s["rstd"], eps, stat_kind=1)
+
+    def bwd(i):
+        s = sets[i % nsets]
+        hk.layer_norm_bwd(s["dy"], s["x"], g, b, s["mean"], s["rstd"], s["dx"], dg, db, eps, stat_kind=1,
+                          clamp_gamma=True, workspace=ws)
+
+    return (fwd, fwd_bytes, rows) if which == "fwd" else (bwd, bwd_bytes, rows)
+
+
+def case_softmax(hk, torch, nsets, which):
+    shape = (4, 32, 2048, 2048)
+    rows = 4 * 32 * 2048
+    bf = torch.bfloat16
+    sets = []
+    for i in range(nsets):
+        s = dict(x=_randn(torch, shape, bf, 3.0, 201 + 10 * i), y=torch.empty(shape, dtype=bf, device="cuda"))
+        hk.softmax_fwd(s["x"], s["y"])
+        if which == "bwd":
+            s["dy"] = _randn(torch, shape, bf, 1.0, 202 + 10 * i)
+            s["dx"] = s.pop("x")  # reuse the storage: x is not read by backward
+        sets.append(s)
+    n = rows * 2048 * 2
+    if which == "fwd":
+        return (lambda i: hk.softmax_fwd(sets[i % nsets]["x"], sets[i % nsets]["y"])), 2 * n, rows
+    return (lambda i: hk.softmax_bwd(sets[i % nsets]["y"], sets[i % nsets]["dy"], sets[i % nsets]["dx"])), 3 * n, rows
+
+
+def case_sce(hk, torch, nsets, which):
+    rows, cols = 16384, 32000
+    bf = torch.bfloat16
+    g = torch.Generator(device="cuda").manual_seed(502)
+    labels = torch.randint(0, cols, (rows,), generator=g, device="cuda", dtype=torch.int64)
+    drop = torch.rand(rows, generator=g, device="cuda") < 0.05
+    labels[drop] = IGNORE
+    sets = []
+    for i in range(nsets):
+        s = dict(x=_randn(torch, (rows, cols), bf, 2.0, 501 + 10 * i))
+        if which == "bwd":
+            s["dx"] = torch.empty((rows, cols), dtype=bf, device="cuda")
+        sets.append(s)
+    loss = torch.empty(rows, dtype=bf, device="cuda")
+    gl = torch.full((rows,), 1.0 / rows, dtype=bf, device="cuda")
+    n = rows * cols * 2
+    if which == "fwd":
+        return (lambda i: hk.sce_sparse_fwd(sets[i % nsets]["x"], labels, loss, IGNORE)), n + rows * 8 + rows * 2, rows
+    return (lambda i: hk.sce_sparse_bwd(sets[i % nsets]["x"], labels, gl, sets[i % nsets]["dx"], IGNORE)), \
+        2 * n + rows * 8 + rows * 2, rows
+
+
+def case_reduce(hk, torch, nsets, axes, op, three_d=False):
+    rows, cols = 32768, 4096
+    bf = torch.bfloat16
+    sets = [_randn(torch, (rows, cols), bf, 1.0, 301 + 10 * i) for i in range(nsets)]
+    if three_d:
+        sets = [t.view(64, 512, 4096) for t in sets]
+    nout = cols if 0 in axes else rows
+    out = torch.empty(nout, dtype=bf, device="cuda")
+    shape, strides = list(sets[0].shape), list(sets[0].stride())
+    ws = torch.empty(max(1, hk.reduce_workspace_bytes(8, shape, strides, list(axes)) // 4), device="cuda")
+    return (lambda i: hk.reduce(sets[i % nsets], out, list(axes), op, workspace=ws)), rows * cols * 2 + nout * 2, \
+        (rows if 1 in axes and not three_d else cols)
+
+
+def case_copy(hk, torch, nsets):
+    n = 1 << 28
+    src = [torch.empty(n, dtype=torch.uint8, device="cuda").zero_() for _ in range(nsets)]
+    dst = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(nsets)]
+    return (lambda i: hk.copy_kernel(dst[i % nsets], src[i % nsets])), 2 * n, 1
+
+
+CASES = [
+    ("C1 layernorm fwd fp32 [8192x4096]", lambda hk, t, n: case_layernorm(hk, t, n, "fwd", "C1")),
+    ("C2 softmax fwd bf16 [4,32,2048,2048]", lambda hk, t, n: case_softmax(hk, t, 2, "fwd")),
+    ("C2 softmax bwd bf16 [4,32,2048,2048]", lambda hk, t, n: case_softmax(hk, t, 2, "bwd")),
+    ("C3 reduce sum axis0 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (0,), "sum")),
+    ("C3 reduce mean axis0 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (0,), "mean")),
+    ("C3 reduce sum axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "sum")),
+    ("C3 reduce mean axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "mean")),
+    ("C3 reduce sum axes(0,1) bf16 [64x512x4096]", lambda hk, t, n: case_reduce(hk, t, n, (0, 1), "sum", True)),
+    ("C4 rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "fwd")),
+    ("C4 rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "bwd")),
+    ("C5 sce fwd bf16 [16384x32000]", lambda hk, t, n: case_sce(hk, t, 2, "fwd")),
+    ("C5 sce bwd bf16 [16384x32000]", lambda hk, t, n: case_sce(hk, t, 2, "bwd")),
+    ("C5 layernorm fwd bf16 [16384x5120]", lambda hk, t, n: case_layernorm(hk, t, n, "fwd", "C5")),
+    ("C5 layernorm bwd bf16 [16384x5120]", lambda hk, t, n: case_layernorm(hk, t, n, "bwd", "C5")),
+    ("copy kernel 256 MiB (calibration)", lambda hk, t, n: case_copy(hk, t, n)),
+]
+
+
+def time_case(hk, torch, launch, steps, warmup, profile_main=True):
+    """Returns (ms per step over the whole region, mean us of the main kernel from bracketing events)."""
+    for i in range(warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    pairs = [(hk.Event(), hk.Event()) for _ in range(steps)] if profile_main else []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        if profile_main:
+            hk.check(hk.lib().hk_profile_next_kernel(pairs[i][0].h, pairs[i][1].h))
+        launch(i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    hk.lib().hk_profile_next_kernel(None, None)
+    main_us = None
+    if profile_main:
+        main_us = sum(b.elapsed_ns_since(a) for a, b in pairs) / 1000.0 / steps
+    return (t1 - t0) * 1000.0 / steps, main_us
+
+
+def cpu_baseline(sample_rows=2048, cols=4096, reps=3):
+    """fp32 CPU port of the step (oracle's refcpu_rmsnorm_*), all host threads, on `sample_rows` rows."""
+    import ctypes
+    import numpy as np
+    import oracle
+    lib = oracle.lib()
+    cores = min(int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1), 64)
+    lib.refcpu_set_num_threads(ctypes.c_int(cores))
+    g = np.random.default_rng(402)
+    x = g.standard_normal((sample_rows, cols), dtype=np.float32)
+    dz = g.standard_normal((sample_rows, cols), dtype=np.float32)
+    w = (g.random(cols, dtype=np.float32) * 0.4 + 0.8).astype(np.float32)
+    z = np.empty_like(x); dx = np.empty_like(x); rs = np.empty(sample_rows, dtype=np.float32)
+    dg = np.empty(cols, dtype=np.float32)
+    fp = ctypes.POINTER(ctypes.c_float)
+    P = lambda a: a.ctypes.data_as(fp)
+    best = None
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        lib.refcpu_rmsnorm_fwd_f32(P(x), P(w), ctypes.c_int64(sample_rows), ctypes.c_int64(cols), ctypes.c_float(1e-6), P(z), P(rs))
+        lib.refcpu_rmsnorm_bwd_f32(P(dz), P(x), P(w), P(rs), ctypes.c_int64(sample_rows), ctypes.c_int64(cols), P(dx), P(dg))
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    algo = sample_rows * (5 * cols * 2 + 12)  # same bf16 accounting as the GPU step, per row
+    return {"value": round(algo / best / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "%d of 32768 rows, fwd+bwd, fp32 arithmetic, best of %d; RMSNorm has no CPU kernel in the "
+                      "reference, this is the oracle formula" % (sample_rows, reps)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--all", action="store_true", help="also time every kernel of every configuration")
+    ap.add_argument("--only", default="", help="substring filter for --all")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--nsets", type=int, default=3, help="rotating buffer sets (working set > cache)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus 1); no multi-GPU path exists", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    hk = _load()
+    torch.cuda.set_device(0)
+
+    kernels = []
+    if args.all:
+        for name, make in CASES:
+            if args.only and args.only not in name:
+                continue
+            launch, nbytes, rows = make(hk, torch, args.nsets)
+            ms, main_us = time_case(hk, torch, launch, args.steps, args.warmup)
+            rec = {"case": name, "us": round(ms * 1000, 2), "main_kernel_us": round(main_us, 2),
+                   "GBps": round(nbytes / ms / 1e6, 1), "frac_of_8TBps": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                   "main_kernel_frac": round(nbytes / main_us / 1e3 / HBM_PEAK_GBS, 4),
+                   "rows_per_s": round(rows / ms * 1e3), "bytes": nbytes}
+            kernels.append(rec)
+            print("%-46s %9.2f us (main %8.2f us) %8.1f GB/s  %5.1f%% (main %5.1f%%)" % (
+                name, rec["us"], rec["main_kernel_us"], rec["GBps"], 100 * rec["frac_of_8TBps"],
+                100 * rec["main_kernel_frac"]), file=sys.stderr, flush=True)
+            del launch
+            torch.cuda.empty_cache()
+
+    # headline: fwd + bwd at the Llama-7B token shape
+    step, step_bytes, rows = case_rmsnorm(hk, torch, args.nsets, "both")
+    ms, _ = time_case(hk, torch, step, args.steps, args.warmup, profile_main=False)
+    bwd, bwd_bytes, _ = case_rmsnorm(hk, torch, args.nsets, "bwd")
+    _, bwd_us = time_case(hk, torch, bwd, args.steps, args.warmup, profile_main=True)
+    achieved = bwd_bytes / bwd_us / 1e3
+    out = {
+        "metric": "HBM GB/s, RMSNorm fwd+bwd at Llama-7B token shape (algorithmic bytes / step time)",
+        "value": round(step_bytes / ms / 1e6, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16 storage, fp32 arithmetic", "data": "synthetic",
+        "config": {"workload": "C4 RMSNorm fwd+bwd bf16 [32768 packed tokens x 4096], eps 1e-6, weight U(0.8,1.2)",
+                   "rows": rows, "hidden": 4096, "us_fwd_plus_bwd": round(ms * 1000, 2),
+                   "rows_per_s": round(rows / ms * 1e3), "frac_of_hbm_peak": round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)},
+        "roofline": {"bound": "hbm", "kernel": "norm_bwd_kernel<bf16> (RMSNorm backward, dx + dgamma/dbeta partials)",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_us": round(bwd_us, 2)},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    if kernels:
+        out["kernels"] = kernels
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

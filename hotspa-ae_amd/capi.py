@@ -1,0 +1,254 @@
+"""ctypes bindings of include/hk_rowwise.h operating on torch CUDA tensors.
+
+torch is used for device memory and streams only; every computation goes
+through the C-ABI entry points.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "lib", "libhk_rowwise.so")
+_lib = None
+
+HK_FLOAT16, HK_FLOAT32, HK_FLOAT64, HK_BFLOAT16, HK_INT64 = 5, 6, 7, 8, 4
+HK_STAT_VAR, HK_STAT_RSTD = 0, 1
+HK_REDUCE_SUM, HK_REDUCE_MEAN = 0, 1
+
+DTYPES = {"uint8": 0, "int8": 1, "int16": 2, "int32": 3, "int64": 4, "fp16": 5, "fp32": 6,
+          "fp64": 7, "bf16": 8, "bool": 9}
+
+
+class HkError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("hk error %d: %s" % (code, message))
+        self.code = code
+
+
+def lib_path():
+    return _LIB
+
+
+def lib():
+    """Loads libhk_rowwise.so; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            raise HkError(-100, "native library %s is missing: run __graft_entry__.build() "
+                                "(or python hotspa-ae_amd/build.py) first" % _LIB)
+        _lib = ctypes.CDLL(_LIB)
+        _lib.hk_last_error.restype = ctypes.c_char_p
+        _lib.hk_version.restype = ctypes.c_char_p
+        _lib.hk_tune_keys.restype = ctypes.c_char_p
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise HkError(rc, lib().hk_last_error().decode("utf-8", "replace"))
+
+
+def dtype_code(t):
+    import torch
+    return {torch.float16: 5, torch.float32: 6, torch.float64: 7, torch.bfloat16: 8, torch.int64: 4,
+            torch.int32: 3, torch.int16: 2, torch.int8: 1, torch.uint8: 0, torch.bool: 9}[t.dtype]
+
+
+def torch_dtype(name):
+    import torch
+    return {"fp16": torch.float16, "fp32": torch.float32, "fp64": torch.float64, "bf16": torch.bfloat16,
+            "int64": torch.int64, "int32": torch.int32, "int16": torch.int16, "int8": torch.int8,
+            "uint8": torch.uint8}[name]
+
+
+def _ptr(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def current_stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def _arr(vals):
+    vals = list(vals)
+    return (ctypes.c_int64 * max(len(vals), 1))(*vals)
+
+
+def tune_set(key, value):
+    check(lib().hk_tune_set(key.encode(), ctypes.c_int(int(value))))
+
+
+class Event:
+    """hipEvent through the C-ABI, recorded on torch's current stream."""
+
+    def __init__(self):
+        self.h = ctypes.c_void_p()
+        check(lib().hk_event_create(ctypes.byref(self.h), ctypes.c_int(1)))
+
+    def record(self, stream=None):
+        check(lib().hk_event_record(self.h, stream if stream is not None else current_stream()))
+
+    def sync(self):
+        check(lib().hk_event_sync(self.h))
+
+    def elapsed_ns_since(self, start):
+        ns = ctypes.c_int64()
+        check(lib().hk_event_elapsed_ns(start.h, self.h, ctypes.byref(ns)))
+        return ns.value
+
+    def __del__(self):
+        try:
+            if self.h:
+                lib().hk_event_destroy(self.h)
+        except Exception:
+            pass
+
+
+# ---------------------------------------------------------------------------
+# operators: tensors are torch CUDA tensors, dense, already allocated
+# ---------------------------------------------------------------------------
+def layer_norm_fwd(x, gamma, beta, y, mean, stat, eps, stat_kind=HK_STAT_RSTD, stream=None):
+    rows = x.numel() // x.shape[-1] if x.numel() else 0
+    cols = x.shape[-1]
+    check(lib().hk_layer_norm_fwd(dtype_code(x), _ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _ptr(mean), _ptr(stat),
+                                  dtype_code(mean if mean is not None else stat), ctypes.c_int(stat_kind),
+                                  _i64(rows), _i64(cols), ctypes.c_float(eps),
+                                  stream if stream is not None else current_stream()))
+
+
+def norm_bwd_workspace_bytes(dtype, rows, cols):
+    n = ctypes.c_size_t()
+    check(lib().hk_norm_bwd_workspace_bytes(ctypes.c_int(dtype), _i64(rows), _i64(cols), ctypes.byref(n)))
+    return n.value
+
+
+def _workspace(nbytes, device):
+    import torch
+    if nbytes == 0:
+        return None
+    return torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=device)
+
+
+def layer_norm_bwd(dy, x_or_y, gamma, beta, mean, stat, dx, dgamma, dbeta, eps, stat_kind=HK_STAT_RSTD,
+                   memory_efficient=False, clamp_gamma=False, workspace=None, stream=None):
+    cols = dy.shape[-1]
+    rows = dy.numel() // cols if dy.numel() else 0
+    if workspace is None:
+        workspace = _workspace(norm_bwd_workspace_bytes(dtype_code(dy), rows, cols), dy.device)
+    wsb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(lib().hk_layer_norm_bwd(dtype_code(dy), _ptr(dy), _ptr(x_or_y), _ptr(gamma), _ptr(beta), _ptr(mean),
+                                  _ptr(stat), dtype_code(stat), ctypes.c_int(stat_kind), _ptr(dx), _ptr(dgamma),
+                                  _ptr(dbeta), _i64(rows), _i64(cols), ctypes.c_float(eps),
+                                  ctypes.c_int(int(memory_efficient)), ctypes.c_int(int(clamp_gamma)),
+                                  _ptr(workspace), ctypes.c_size_t(wsb),
+                                  stream if stream is not None else current_stream()))
+    return workspace
+
+
+def dropout_add_ln_fwd(x0, residual, gamma, beta, z, x_out, mu, rsigma, eps, is_rms, stream=None):
+    rows, cols = x0.shape
+    rtype = dtype_code(residual) if residual is not None else dtype_code(x0)
+    check(lib().hk_dropout_add_ln_fwd(dtype_code(x0), rtype, dtype_code(gamma), _ptr(x0), _ptr(residual),
+                                      _ptr(gamma), _ptr(beta), _ptr(z), _ptr(x_out), _ptr(mu), _ptr(rsigma),
+                                      _i64(rows), _i64(cols), ctypes.c_float(eps), ctypes.c_int(int(is_rms)),
+                                      stream if stream is not None else current_stream()))
+
+
+def dropout_add_ln_bwd(dz, dx_in, x, mu, rsigma, gamma, dx0, dresidual, dgamma, dbeta, is_rms,
+                       workspace=None, stream=None):
+    rows, cols = x.shape
+    if workspace is None:
+        workspace = _workspace(norm_bwd_workspace_bytes(dtype_code(dz), rows, cols), dz.device)
+    wsb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(lib().hk_dropout_add_ln_bwd(dtype_code(dz), dtype_code(x), dtype_code(gamma), _ptr(dz), _ptr(dx_in),
+                                      _ptr(x), _ptr(mu), _ptr(rsigma), _ptr(gamma), _ptr(dx0), _ptr(dresidual),
+                                      _ptr(dgamma), _ptr(dbeta), _i64(rows), _i64(cols), ctypes.c_int(int(is_rms)),
+                                      _ptr(workspace), ctypes.c_size_t(wsb),
+                                      stream if stream is not None else current_stream()))
+    return workspace
+
+
+def _odi(shape, dim):
+    dim = dim % len(shape)
+    outer = 1
+    for s in shape[:dim]:
+        outer *= s
+    inner = 1
+    for s in shape[dim + 1:]:
+        inner *= s
+    return outer, shape[dim], inner
+
+
+def softmax_fwd(x, y, dim=-1, stream=None):
+    o, d, i = _odi(list(x.shape), dim)
+    check(lib().hk_softmax_fwd(dtype_code(x), _ptr(x), _ptr(y), _i64(o), _i64(d), _i64(i),
+                               stream if stream is not None else current_stream()))
+
+
+def softmax_bwd(y, dy, dx, dim=-1, stream=None):
+    o, d, i = _odi(list(y.shape), dim)
+    check(lib().hk_softmax_bwd(dtype_code(y), _ptr(y), _ptr(dy), _ptr(dx), _i64(o), _i64(d), _i64(i),
+                               stream if stream is not None else current_stream()))
+
+
+def sce_sparse_fwd(logits, labels, loss, ignored_index, stream=None):
+    cols = logits.shape[-1]
+    rows = logits.numel() // cols if logits.numel() else 0
+    check(lib().hk_sce_sparse_fwd(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(loss), _i64(rows), _i64(cols),
+                                  _i64(ignored_index), stream if stream is not None else current_stream()))
+
+
+def sce_sparse_bwd(logits, labels, grad_loss, dlogits, ignored_index, stream=None):
+    cols = logits.shape[-1]
+    rows = logits.numel() // cols if logits.numel() else 0
+    check(lib().hk_sce_sparse_bwd(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(grad_loss), _ptr(dlogits),
+                                  _i64(rows), _i64(cols), _i64(ignored_index),
+                                  stream if stream is not None else current_stream()))
+
+
+def sce_dense_fwd(logits, labels, loss, stream=None):
+    cols = logits.shape[-1]
+    rows = logits.numel() // cols if logits.numel() else 0
+    check(lib().hk_sce_dense_fwd(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(loss), _i64(rows), _i64(cols),
+                                 stream if stream is not None else current_stream()))
+
+
+def sce_dense_bwd(logits, labels, grad_loss, dlogits, stream=None):
+    cols = logits.shape[-1]
+    rows = logits.numel() // cols if logits.numel() else 0
+    check(lib().hk_sce_dense_bwd(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(grad_loss), _ptr(dlogits),
+                                 _i64(rows), _i64(cols), stream if stream is not None else current_stream()))
+
+
+def reduce_workspace_bytes(dtype, shape, strides, axes):
+    n = ctypes.c_size_t()
+    check(lib().hk_reduce_workspace_bytes(ctypes.c_int(dtype), ctypes.c_int(len(shape)), _arr(shape), _arr(strides),
+                                          ctypes.c_int(len(axes)), _arr(axes), ctypes.byref(n)))
+    return n.value
+
+
+def reduce(x, out, axes, op="sum", workspace=None, stream=None):
+    """x may be any strided torch view; axes already wrapped to [0, ndim)."""
+    shape, strides = list(x.shape), list(x.stride())
+    if workspace is None:
+        workspace = _workspace(reduce_workspace_bytes(dtype_code(x), shape, strides, axes), x.device)
+    wsb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(lib().hk_reduce(dtype_code(x), dtype_code(out), _ptr(x), _ptr(out), ctypes.c_int(len(shape)), _arr(shape),
+                          _arr(strides), ctypes.c_int(len(axes)), _arr(axes),
+                          ctypes.c_int(HK_REDUCE_MEAN if op == "mean" else HK_REDUCE_SUM), _ptr(workspace),
+                          ctypes.c_size_t(wsb), stream if stream is not None else current_stream()))
+    return workspace
+
+
+def copy_kernel(dst, src, stream=None):
+    check(lib().hk_copy_kernel(_ptr(dst), _ptr(src), ctypes.c_size_t(src.numel() * src.element_size()),
+                               stream if stream is not None else current_stream()))
+
+
+def strided_copy(src, dst, stream=None):
+    check(lib().hk_strided_copy(dtype_code(src), _ptr(src), _ptr(dst), ctypes.c_int(src.dim()), _arr(src.shape),
+                                _arr(src.stride()), stream if stream is not None else current_stream()))

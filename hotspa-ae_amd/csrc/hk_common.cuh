@@ -1,0 +1,369 @@
+// Device-side building blocks shared by every row-wise kernel: 128-bit vector
+// I/O for fp32 / bf16 / fp16 rows, wave64 DPP reductions, LDS cross-wave
+// combine, and the host-side launch/error helpers of the C-ABI layer.
+//
+// Written for gfx950 (CDNA4) only: wave size is 64, DPP row_bcast modes and the
+// v_cvt_pk_bf16_f32 conversion are assumed.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "hk_rowwise.h"
+
+namespace hk {
+
+constexpr int kWave = 64;
+constexpr int kMaxBlock = 1024;
+constexpr int kMaxWaves = kMaxBlock / kWave;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// Storage element tags. bf16 / fp16 are carried as raw 16-bit patterns; all
+// arithmetic is done in fp32 after unpacking.
+struct bf16 { uint16_t bits; };
+struct fp16 { uint16_t bits; };
+
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// ---------------------------------------------------------------------------
+// Scalar conversions
+// ---------------------------------------------------------------------------
+template <typename T> struct Cvt;
+
+template <> struct Cvt<float> {
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+};
+
+template <> struct Cvt<bf16> {
+  static __device__ __forceinline__ float load(const bf16* p) {
+    return u2f(uint32_t(p->bits) << 16);
+  }
+  static __device__ __forceinline__ void store(bf16* p, float v) {
+    // round-to-nearest-even through the hardware packed converter
+    f32x2 f = {v, 0.f};
+    bf16x2 b = __builtin_convertvector(f, bf16x2);
+    p->bits = uint16_t(__builtin_bit_cast(uint32_t, b) & 0xffffu);
+  }
+};
+
+template <> struct Cvt<fp16> {
+  static __device__ __forceinline__ float load(const fp16* p) {
+    return float(__builtin_bit_cast(_Float16, p->bits));
+  }
+  static __device__ __forceinline__ void store(fp16* p, float v) {
+    p->bits = __builtin_bit_cast(uint16_t, _Float16(v));
+  }
+};
+
+template <> struct Cvt<double> {
+  static __device__ __forceinline__ double load(const double* p) { return *p; }
+  static __device__ __forceinline__ void store(double* p, double v) { *p = v; }
+};
+
+// ---------------------------------------------------------------------------
+// 16-byte vectors: N elements of T <-> N floats
+// ---------------------------------------------------------------------------
+template <typename T> struct VecIO;
+
+template <> struct VecIO<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void unpack(const u32x4& r, float* f) {
+    f[0] = u2f(r.x); f[1] = u2f(r.y); f[2] = u2f(r.z); f[3] = u2f(r.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* f) {
+    u32x4 r = {f2u(f[0]), f2u(f[1]), f2u(f[2]), f2u(f[3])};
+    return r;
+  }
+};
+
+template <> struct VecIO<bf16> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void unpack(const u32x4& r, float* f) {
+    f[0] = u2f(r.x << 16); f[1] = u2f(r.x & 0xffff0000u);
+    f[2] = u2f(r.y << 16); f[3] = u2f(r.y & 0xffff0000u);
+    f[4] = u2f(r.z << 16); f[5] = u2f(r.z & 0xffff0000u);
+    f[6] = u2f(r.w << 16); f[7] = u2f(r.w & 0xffff0000u);
+  }
+  static __device__ __forceinline__ uint32_t pk(float a, float b) {
+    f32x2 f = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* f) {
+    u32x4 r = {pk(f[0], f[1]), pk(f[2], f[3]), pk(f[4], f[5]), pk(f[6], f[7])};
+    return r;
+  }
+};
+
+template <> struct VecIO<fp16> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void up(uint32_t w, float* f) {
+    f32x2 v = __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
+    f[0] = v.x; f[1] = v.y;
+  }
+  static __device__ __forceinline__ void unpack(const u32x4& r, float* f) {
+    up(r.x, f); up(r.y, f + 2); up(r.z, f + 4); up(r.w, f + 6);
+  }
+  static __device__ __forceinline__ uint32_t pk(float a, float b) {
+    f32x2 f = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* f) {
+    u32x4 r = {pk(f[0], f[1]), pk(f[2], f[3]), pk(f[4], f[5]), pk(f[6], f[7])};
+    return r;
+  }
+};
+
+__device__ __forceinline__ u32x4 ld16(const void* p) {
+  return *reinterpret_cast<const u32x4*>(p);
+}
+__device__ __forceinline__ void st16(void* p, const u32x4& v) {
+  *reinterpret_cast<u32x4*>(p) = v;
+}
+// Streaming store for write-once outputs (bypasses cache residency).
+__device__ __forceinline__ void st16_stream(void* p, const u32x4& v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
+__device__ __forceinline__ u32x4 ld16_stream(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+
+// ---------------------------------------------------------------------------
+// wave64 reductions through DPP (no LDS traffic).  After the call every lane
+// holds the result.
+// ---------------------------------------------------------------------------
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_f(float v, float old = 0.f) {
+  return u2f(uint32_t(__builtin_amdgcn_update_dpp(
+      int(f2u(old)), int(f2u(v)), CTRL, ROW_MASK, 0xf, false)));
+}
+
+constexpr int kDppXor1 = 0xB1;        // quad_perm:[1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // row_half_mirror
+constexpr int kDppMirror = 0x140;     // row_mirror
+constexpr int kDppBcast15 = 0x142;    // row_bcast:15
+constexpr int kDppBcast31 = 0x143;    // row_bcast:31
+
+__device__ __forceinline__ float readlane_f(float v, int lane) {
+  return u2f(uint32_t(__builtin_amdgcn_readlane(int(f2u(v)), lane)));
+}
+
+struct OpSum {
+  static __device__ __forceinline__ float identity() { return 0.f; }
+  static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
+};
+struct OpMax {
+  static __device__ __forceinline__ float identity() { return -__builtin_huge_valf(); }
+  static __device__ __forceinline__ float apply(float a, float b) { return fmaxf(a, b); }
+};
+
+template <typename Op>
+__device__ __forceinline__ float wave_allreduce(float v) {
+  v = Op::apply(v, dpp_f<kDppXor1>(v, v));
+  v = Op::apply(v, dpp_f<kDppXor2>(v, v));
+  v = Op::apply(v, dpp_f<kDppHalfMirror>(v, v));
+  v = Op::apply(v, dpp_f<kDppMirror>(v, v));
+  // every lane of a 16-lane row now holds that row's result; fold the 4 rows
+  float r0 = readlane_f(v, 0), r1 = readlane_f(v, 16);
+  float r2 = readlane_f(v, 32), r3 = readlane_f(v, 48);
+  return Op::apply(Op::apply(r0, r1), Op::apply(r2, r3));
+}
+
+__device__ __forceinline__ float wave_sum(float v) { return wave_allreduce<OpSum>(v); }
+__device__ __forceinline__ float wave_max(float v) { return wave_allreduce<OpMax>(v); }
+
+// Shuffle through DPP for the 16-lane-local steps of a butterfly, and through
+// the cross-lane network only for the 16 / 32 strides.  Used by reductions on
+// tuples (Chan merge, online softmax) where the combine is not a plain op.
+template <int STRIDE>
+__device__ __forceinline__ float lane_xor(float v) {
+  if constexpr (STRIDE == 1) return dpp_f<kDppXor1>(v, v);
+  else if constexpr (STRIDE == 2) return dpp_f<kDppXor2>(v, v);
+  else return __shfl_xor(v, STRIDE, kWave);
+}
+
+// ---------------------------------------------------------------------------
+// Block-level combine: waves [w0, w0+nw) of a workgroup cooperate on one row.
+// `scratch` holds kMaxWaves floats per slot in LDS.  All threads of the block
+// must call (contains __syncthreads).
+// ---------------------------------------------------------------------------
+template <typename Op>
+__device__ __forceinline__ float block_allreduce(float v, float* scratch, int nwaves) {
+  v = wave_allreduce<Op>(v);
+  const int w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) scratch[w] = v;
+  __syncthreads();
+  float r = Op::identity();
+  for (int i = 0; i < nwaves; ++i) r = Op::apply(r, scratch[i]);
+  return r;
+}
+
+// ---------------------------------------------------------------------------
+// Tuple reductions.  P is a struct with `float v[P::K]` and
+// `static P merge(P, P)` (commutative up to rounding).  The wave version
+// leaves the same value in every lane; the group version combines the waves
+// [first_wave, first_wave + nwaves) of a workgroup through `scratch`
+// (kMaxWaves * K floats) and contains one __syncthreads().
+// ---------------------------------------------------------------------------
+template <typename P>
+__device__ __forceinline__ P wave_allreduce_tuple(P a) {
+  P b;
+#pragma unroll
+  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_f<kDppXor1>(a.v[k], a.v[k]);
+  a = P::merge(a, b);
+#pragma unroll
+  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_f<kDppXor2>(a.v[k], a.v[k]);
+  a = P::merge(a, b);
+#pragma unroll
+  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_f<kDppHalfMirror>(a.v[k], a.v[k]);
+  a = P::merge(a, b);
+#pragma unroll
+  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_f<kDppMirror>(a.v[k], a.v[k]);
+  a = P::merge(a, b);
+  P r[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int k = 0; k < P::K; ++k) r[j].v[k] = readlane_f(a.v[k], 16 * j);
+  return P::merge(P::merge(r[0], r[1]), P::merge(r[2], r[3]));
+}
+
+template <typename P>
+__device__ __forceinline__ P group_allreduce_tuple(P a, float* scratch, int first_wave,
+                                                    int nwaves) {
+  a = wave_allreduce_tuple<P>(a);
+  if (nwaves == 1) return a;
+  const int w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int k = 0; k < P::K; ++k) scratch[w * P::K + k] = a.v[k];
+  }
+  __syncthreads();
+  P r;
+#pragma unroll
+  for (int k = 0; k < P::K; ++k) r.v[k] = scratch[first_wave * P::K + k];
+  for (int i = 1; i < nwaves; ++i) {
+    P o;
+#pragma unroll
+    for (int k = 0; k < P::K; ++k) o.v[k] = scratch[(first_wave + i) * P::K + k];
+    r = P::merge(r, o);
+  }
+  return r;
+}
+
+// plain sums of K values
+template <int KK>
+struct SumTuple {
+  static constexpr int K = KK;
+  float v[KK];
+  static __device__ __forceinline__ SumTuple merge(SumTuple a, const SumTuple& b) {
+#pragma unroll
+    for (int k = 0; k < KK; ++k) a.v[k] += b.v[k];
+    return a;
+  }
+};
+
+// (count, mean, M2) with Chan's parallel update of Welford's statistics
+struct MomentTuple {
+  static constexpr int K = 3;
+  float v[3];
+  static __device__ __forceinline__ MomentTuple merge(const MomentTuple& a, const MomentTuple& b) {
+    MomentTuple r;
+    const float n = a.v[0] + b.v[0];
+    const float inv = n > 0.f ? __builtin_amdgcn_rcpf(n) : 0.f;
+    const float delta = b.v[1] - a.v[1];
+    const float wb = b.v[0] * inv;
+    r.v[0] = n;
+    r.v[1] = a.v[1] + delta * wb;
+    r.v[2] = a.v[2] + b.v[2] + delta * delta * a.v[0] * wb;
+    return r;
+  }
+};
+
+// (running max, sum of exp(x - max)) for the online softmax
+struct MaxSumTuple {
+  static constexpr int K = 2;
+  float v[2];
+  static __device__ __forceinline__ MaxSumTuple merge(const MaxSumTuple& a, const MaxSumTuple& b) {
+    constexpr float kLog2e = 1.4426950408889634f;
+    MaxSumTuple r;
+    const float m = fmaxf(a.v[0], b.v[0]);
+    // an empty side has max = -inf and sum = 0; keep exp2(-inf - -inf) out of the result
+    const float ms = (m == -__builtin_huge_valf()) ? 0.f : m;
+    r.v[0] = m;
+    r.v[1] = a.v[1] * __builtin_amdgcn_exp2f((a.v[0] - ms) * kLog2e) +
+             b.v[1] * __builtin_amdgcn_exp2f((b.v[0] - ms) * kLog2e);
+    return r;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// host helpers
+// ---------------------------------------------------------------------------
+void set_last_error(const char* fmt, ...);
+
+#define HK_CHECK_HIP(expr)                                                     \
+  do {                                                                         \
+    hipError_t _e = (expr);                                                    \
+    if (_e != hipSuccess) {                                                    \
+      ::hk::set_last_error("%s failed: %s (%s:%d)", #expr,                     \
+                           hipGetErrorString(_e), __FILE__, __LINE__);         \
+      return HK_ERR_HIP;                                                       \
+    }                                                                          \
+  } while (0)
+
+#define HK_REQUIRE(cond, code, ...)                                            \
+  do {                                                                         \
+    if (!(cond)) {                                                             \
+      ::hk::set_last_error(__VA_ARGS__);                                       \
+      return (code);                                                           \
+    }                                                                          \
+  } while (0)
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline hipStream_t as_hip(hkStream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Tunable launch parameters (0 = automatic); values are set through
+// hk_tune_set().  The order matches the name table in hk_device.hip.
+enum TuneKey {
+  TUNE_NORM_FWD_THREADS = 0,
+  TUNE_NORM_BWD_THREADS,
+  TUNE_NORM_BWD_BLOCKS,
+  TUNE_SOFTMAX_THREADS,
+  TUNE_SCE_THREADS,
+  TUNE_REDUCE_INNER_THREADS,
+  TUNE_REDUCE_OUTER_ROW_BLOCKS,
+  TUNE_STREAM_STORES,
+  TUNE_NORM_BWD_ROWS_PER_BLOCK,
+  TUNE_NUM_KEYS
+};
+int tune_get(int key);
+int device_cu_count();
+
+inline size_t dtype_size(int dtype) {
+  switch (dtype) {
+    case HK_UINT8: case HK_INT8: case HK_BOOL: return 1;
+    case HK_INT16: case HK_FLOAT16: case HK_BFLOAT16: return 2;
+    case HK_INT32: case HK_FLOAT32: return 4;
+    case HK_INT64: case HK_FLOAT64: return 8;
+    default: return 0;
+  }
+}
+
+int launch_check(const char* what);
+
+// Brackets the main kernel of an operator with the events armed through
+// hk_profile_next_kernel(); no-ops when nothing is armed.
+void profile_before(hipStream_t s);
+void profile_after(hipStream_t s);
+
+} // namespace hk

@@ -1,0 +1,351 @@
+// Device / memory / stream / event entry points of the C-ABI, plus the small
+// utility kernels (fill, streaming copy, strided gather) and the tuning table.
+#include "hk_common.cuh"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+
+namespace hk {
+
+static thread_local char g_last_error[512] = "";
+
+void set_last_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+}
+
+int launch_check(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_last_error("launch of %s failed: %s", what, hipGetErrorString(e));
+    return HK_ERR_HIP;
+  }
+  return HK_OK;
+}
+
+static thread_local hipEvent_t g_prof_before = nullptr;
+static thread_local hipEvent_t g_prof_after = nullptr;
+
+void profile_before(hipStream_t s) {
+  if (g_prof_before) { (void)hipEventRecord(g_prof_before, s); g_prof_before = nullptr; }
+}
+void profile_after(hipStream_t s) {
+  if (g_prof_after) { (void)hipEventRecord(g_prof_after, s); g_prof_after = nullptr; }
+}
+
+// ---------------------------------------------------------------------------
+// tuning table
+// ---------------------------------------------------------------------------
+static const char* const kTuneNames[] = {
+  "norm_fwd_threads",   // threads cooperating on one row (64 = one wavefront per row)
+  "norm_bwd_threads",
+  "norm_bwd_blocks",    // persistent grid size of the backward kernels
+  "softmax_threads",
+  "sce_threads",
+  "reduce_inner_threads",
+  "reduce_outer_row_blocks",
+  "stream_stores",      // 1: non-temporal stores for write-once outputs, 2: plain stores
+  "norm_bwd_rows_per_block",
+};
+constexpr int kNumTune = sizeof(kTuneNames) / sizeof(kTuneNames[0]);
+static_assert(kNumTune == TUNE_NUM_KEYS, "tune name table out of sync with TuneKey");
+static int g_tune[kNumTune] = {0};
+
+int tune_get(int key) { return (key >= 0 && key < kNumTune) ? g_tune[key] : 0; }
+
+// Compute-unit count of the current device, cached per device index.
+int device_cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+// ---------------------------------------------------------------------------
+// utility kernels
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fill_bytes_kernel(uint8_t* dst, uint32_t word, size_t bytes) {
+  // head/tail bytes individually, the aligned middle as 16-byte stores
+  const size_t tid = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t nthreads = size_t(gridDim.x) * blockDim.x;
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(dst);
+  size_t head = (16 - (addr & 15)) & 15;
+  if (head > bytes) head = bytes;
+  const size_t nvec = (bytes - head) / 16;
+  const size_t tail_begin = head + nvec * 16;
+  const uint8_t b = uint8_t(word & 0xff);
+  if (tid < head) dst[tid] = b;
+  u32x4 v = {word, word, word, word};
+  u32x4* mid = reinterpret_cast<u32x4*>(dst + head);
+  for (size_t i = tid; i < nvec; i += nthreads) mid[i] = v;
+  if (tid < bytes - tail_begin) dst[tail_begin + tid] = b;
+}
+
+template <int UNROLL>
+__global__ __launch_bounds__(256) void copy16_kernel(u32x4* __restrict__ dst,
+                                                     const u32x4* __restrict__ src, size_t nvec) {
+  const size_t base = (size_t(blockIdx.x) * UNROLL) * 256 + threadIdx.x;
+  u32x4 v[UNROLL];
+#pragma unroll
+  for (int i = 0; i < UNROLL; ++i) {
+    size_t idx = base + size_t(i) * 256;
+    if (idx < nvec) v[i] = src[idx];
+  }
+#pragma unroll
+  for (int i = 0; i < UNROLL; ++i) {
+    size_t idx = base + size_t(i) * 256;
+    if (idx < nvec) dst[idx] = v[i];
+  }
+}
+
+struct StridedMeta {
+  int ndim;
+  int64_t shape[8];
+  int64_t stride[8];
+};
+
+template <typename W>
+__global__ __launch_bounds__(256) void strided_copy_kernel(const W* __restrict__ src,
+                                                           W* __restrict__ dst, StridedMeta m,
+                                                           int64_t numel) {
+  int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t step = int64_t(gridDim.x) * blockDim.x;
+  for (; i < numel; i += step) {
+    int64_t rem = i, off = 0;
+    for (int d = m.ndim - 1; d >= 0; --d) {
+      int64_t q = rem / m.shape[d];
+      off += (rem - q * m.shape[d]) * m.stride[d];
+      rem = q;
+    }
+    dst[i] = src[off];
+  }
+}
+
+} // namespace hk
+
+using namespace hk;
+
+extern "C" {
+
+const char* hk_last_error(void) { return g_last_error; }
+const char* hk_version(void) { return "hk_rowwise 0.1 (gfx950)"; }
+
+int hk_device_count(int* count) {
+  HK_REQUIRE(count, HK_ERR_INVALID, "hk_device_count: null output");
+  HK_CHECK_HIP(hipGetDeviceCount(count));
+  return HK_OK;
+}
+int hk_set_device(int device) { HK_CHECK_HIP(hipSetDevice(device)); return HK_OK; }
+int hk_get_device(int* device) {
+  HK_REQUIRE(device, HK_ERR_INVALID, "hk_get_device: null output");
+  HK_CHECK_HIP(hipGetDevice(device));
+  return HK_OK;
+}
+int hk_device_sync(void) { HK_CHECK_HIP(hipDeviceSynchronize()); return HK_OK; }
+int hk_mem_get_info(size_t* free_bytes, size_t* total_bytes) {
+  HK_REQUIRE(free_bytes && total_bytes, HK_ERR_INVALID, "hk_mem_get_info: null output");
+  HK_CHECK_HIP(hipMemGetInfo(free_bytes, total_bytes));
+  return HK_OK;
+}
+int hk_device_cu_count(int device, int* cus) {
+  HK_REQUIRE(cus, HK_ERR_INVALID, "hk_device_cu_count: null output");
+  HK_CHECK_HIP(hipDeviceGetAttribute(cus, hipDeviceAttributeMultiprocessorCount, device));
+  return HK_OK;
+}
+
+int hk_malloc(void** ptr, size_t bytes) {
+  HK_REQUIRE(ptr, HK_ERR_INVALID, "hk_malloc: null output");
+  *ptr = nullptr;
+  if (bytes == 0) return HK_OK;
+  HK_CHECK_HIP(hipMalloc(ptr, bytes));
+  return HK_OK;
+}
+int hk_free(void* ptr) {
+  if (ptr) HK_CHECK_HIP(hipFree(ptr));
+  return HK_OK;
+}
+int hk_host_malloc(void** ptr, size_t bytes) {
+  HK_REQUIRE(ptr, HK_ERR_INVALID, "hk_host_malloc: null output");
+  *ptr = nullptr;
+  if (bytes == 0) return HK_OK;
+  HK_CHECK_HIP(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+  return HK_OK;
+}
+int hk_host_free(void* ptr) {
+  if (ptr) HK_CHECK_HIP(hipHostFree(ptr));
+  return HK_OK;
+}
+int hk_memcpy_h2d(void* dst, const void* src, size_t bytes, hkStream_t stream) {
+  if (bytes == 0) return HK_OK;
+  HK_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_hip(stream)));
+  return HK_OK;
+}
+int hk_memcpy_d2h(void* dst, const void* src, size_t bytes, hkStream_t stream) {
+  if (bytes == 0) return HK_OK;
+  HK_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_hip(stream)));
+  return HK_OK;
+}
+int hk_memcpy_d2d(void* dst, const void* src, size_t bytes, hkStream_t stream) {
+  if (bytes == 0) return HK_OK;
+  HK_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_hip(stream)));
+  return HK_OK;
+}
+int hk_memset(void* dst, int value, size_t bytes, hkStream_t stream) {
+  if (bytes == 0) return HK_OK;
+  HK_REQUIRE(dst, HK_ERR_INVALID, "hk_memset: null destination");
+  uint32_t b = uint32_t(value) & 0xff;
+  uint32_t word = b | (b << 8) | (b << 16) | (b << 24);
+  size_t nvec = bytes / 16 + 1;
+  size_t blocks = (nvec + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fill_bytes_kernel, dim3(unsigned(blocks)), dim3(256), 0, as_hip(stream),
+                     static_cast<uint8_t*>(dst), word, bytes);
+  return launch_check("fill_bytes_kernel");
+}
+
+int hk_stream_create(hkStream_t* stream) {
+  HK_REQUIRE(stream, HK_ERR_INVALID, "hk_stream_create: null output");
+  hipStream_t s;
+  HK_CHECK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream = reinterpret_cast<hkStream_t>(s);
+  return HK_OK;
+}
+int hk_stream_destroy(hkStream_t stream) {
+  if (stream) HK_CHECK_HIP(hipStreamDestroy(as_hip(stream)));
+  return HK_OK;
+}
+int hk_stream_sync(hkStream_t stream) {
+  HK_CHECK_HIP(hipStreamSynchronize(as_hip(stream)));
+  return HK_OK;
+}
+int hk_stream_wait_event(hkStream_t stream, hkEvent_t event) {
+  HK_REQUIRE(event, HK_ERR_INVALID, "hk_stream_wait_event: null event");
+  HK_CHECK_HIP(hipStreamWaitEvent(as_hip(stream), reinterpret_cast<hipEvent_t>(event), 0));
+  return HK_OK;
+}
+
+int hk_event_create(hkEvent_t* event, int enable_timing) {
+  HK_REQUIRE(event, HK_ERR_INVALID, "hk_event_create: null output");
+  hipEvent_t e;
+  HK_CHECK_HIP(hipEventCreateWithFlags(&e, enable_timing ? hipEventDefault : hipEventDisableTiming));
+  *event = reinterpret_cast<hkEvent_t>(e);
+  return HK_OK;
+}
+int hk_event_destroy(hkEvent_t event) {
+  if (event) HK_CHECK_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
+  return HK_OK;
+}
+int hk_event_record(hkEvent_t event, hkStream_t stream) {
+  HK_REQUIRE(event, HK_ERR_INVALID, "hk_event_record: null event");
+  HK_CHECK_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(event), as_hip(stream)));
+  return HK_OK;
+}
+int hk_event_sync(hkEvent_t event) {
+  HK_REQUIRE(event, HK_ERR_INVALID, "hk_event_sync: null event");
+  HK_CHECK_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(event)));
+  return HK_OK;
+}
+int hk_event_query(hkEvent_t event, int* done) {
+  HK_REQUIRE(event && done, HK_ERR_INVALID, "hk_event_query: null argument");
+  hipError_t e = hipEventQuery(reinterpret_cast<hipEvent_t>(event));
+  if (e == hipSuccess) { *done = 1; return HK_OK; }
+  if (e == hipErrorNotReady) { *done = 0; (void)hipGetLastError(); return HK_OK; }
+  set_last_error("hipEventQuery failed: %s", hipGetErrorString(e));
+  return HK_ERR_HIP;
+}
+int hk_event_elapsed_ns(hkEvent_t start, hkEvent_t stop, int64_t* ns) {
+  HK_REQUIRE(start && stop && ns, HK_ERR_INVALID, "hk_event_elapsed_ns: null argument");
+  float ms = 0.f;
+  HK_CHECK_HIP(hipEventElapsedTime(&ms, reinterpret_cast<hipEvent_t>(start),
+                                   reinterpret_cast<hipEvent_t>(stop)));
+  *ns = int64_t(double(ms) * 1.0e6);
+  return HK_OK;
+}
+
+int hk_profile_next_kernel(hkEvent_t before, hkEvent_t after) {
+  g_prof_before = reinterpret_cast<hipEvent_t>(before);
+  g_prof_after = reinterpret_cast<hipEvent_t>(after);
+  return HK_OK;
+}
+
+int hk_tune_set(const char* key, int value) {
+  HK_REQUIRE(key, HK_ERR_INVALID, "hk_tune_set: null key");
+  for (int i = 0; i < kNumTune; ++i) {
+    if (std::strcmp(key, kTuneNames[i]) == 0) {
+      g_tune[i] = value;
+      return HK_OK;
+    }
+  }
+  set_last_error("hk_tune_set: unknown key '%s'", key);
+  return HK_ERR_INVALID;
+}
+
+const char* hk_tune_keys(void) {
+  static std::string keys;
+  static std::once_flag once;
+  std::call_once(once, [] {
+    for (int i = 0; i < kNumTune; ++i) {
+      if (i) keys += ",";
+      keys += kTuneNames[i];
+    }
+  });
+  return keys.c_str();
+}
+
+int hk_copy_kernel(void* dst, const void* src, size_t bytes, hkStream_t stream) {
+  if (bytes == 0) return HK_OK;
+  HK_REQUIRE(dst && src, HK_ERR_INVALID, "hk_copy_kernel: null pointer");
+  HK_REQUIRE(bytes % 16 == 0 && aligned16(dst) && aligned16(src), HK_ERR_INVALID,
+             "hk_copy_kernel: needs 16-byte aligned pointers and size");
+  constexpr int UNROLL = 4;
+  size_t nvec = bytes / 16;
+  size_t blocks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
+  HK_REQUIRE(blocks <= 0x7fffffffu, HK_ERR_INVALID, "hk_copy_kernel: size too large");
+  hipLaunchKernelGGL(copy16_kernel<UNROLL>, dim3(unsigned(blocks)), dim3(256), 0, as_hip(stream),
+                     static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), nvec);
+  return launch_check("copy16_kernel");
+}
+
+int hk_strided_copy(int dtype, const void* src, void* dst, int ndim, const int64_t* shape,
+                    const int64_t* src_strides, hkStream_t stream) {
+  HK_REQUIRE(ndim >= 0 && ndim <= 8, HK_ERR_INVALID, "hk_strided_copy: ndim %d not in [0, 8]", ndim);
+  HK_REQUIRE(ndim == 0 || (shape && src_strides), HK_ERR_INVALID, "hk_strided_copy: null meta");
+  size_t es = dtype_size(dtype);
+  HK_REQUIRE(es != 0, HK_ERR_UNSUPPORTED, "hk_strided_copy: unknown dtype %d", dtype);
+  StridedMeta m;
+  m.ndim = ndim;
+  int64_t numel = 1;
+  for (int d = 0; d < ndim; ++d) {
+    HK_REQUIRE(shape[d] >= 0, HK_ERR_INVALID, "hk_strided_copy: negative extent");
+    m.shape[d] = shape[d];
+    m.stride[d] = src_strides[d];
+    numel *= shape[d];
+  }
+  if (numel == 0) return HK_OK;
+  HK_REQUIRE(src && dst, HK_ERR_INVALID, "hk_strided_copy: null pointer");
+  int64_t blocks = (numel + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  dim3 g{unsigned(blocks)}, b{256};
+  hipStream_t s = as_hip(stream);
+  switch (es) {
+    case 1: hipLaunchKernelGGL(strided_copy_kernel<uint8_t>, g, b, 0, s, (const uint8_t*)src, (uint8_t*)dst, m, numel); break;
+    case 2: hipLaunchKernelGGL(strided_copy_kernel<uint16_t>, g, b, 0, s, (const uint16_t*)src, (uint16_t*)dst, m, numel); break;
+    case 4: hipLaunchKernelGGL(strided_copy_kernel<uint32_t>, g, b, 0, s, (const uint32_t*)src, (uint32_t*)dst, m, numel); break;
+    default: hipLaunchKernelGGL(strided_copy_kernel<uint64_t>, g, b, 0, s, (const uint64_t*)src, (uint64_t*)dst, m, numel); break;
+  }
+  return launch_check("strided_copy_kernel");
+}
+
+} // extern "C"

@@ -1,0 +1,605 @@
+// Reduce sum / mean over arbitrary axes for gfx950.
+//
+// The host merges neighbouring dimensions of the same kind (reduced / kept)
+// that are contiguous in memory, then picks one of three kernels:
+//   inner   [rows, C] -> [rows]   : the reduced extent is the unit-stride one;
+//           a wavefront or workgroup streams a row with 128-bit loads, DPP +
+//           LDS fold.  Long rows are split over several workgroups.
+//   outer   [B, R, C] -> [B, C]   : the kept extent is the unit-stride one;
+//           every lane owns one 128-bit column vector, the waves of a
+//           workgroup take interleaved rows, rows are split over many
+//           workgroups, fp32 partials are folded by a second small launch.
+//   generic any strided layout    : one thread per output element.
+// bf16 / fp16 accumulate in fp32; mean multiplies the final sum by
+// float(1 / reduce_num).
+#include "hk_common.cuh"
+
+#include <algorithm>
+#include <type_traits>
+#include <vector>
+
+namespace hk {
+
+// ---------------------------------------------------------------------------
+// element access for the scalar paths
+// ---------------------------------------------------------------------------
+template <typename T> struct AccOf { using type = T; };
+template <> struct AccOf<bf16> { using type = float; };
+template <> struct AccOf<fp16> { using type = float; };
+template <> struct AccOf<bool> { using type = int64_t; };
+
+template <typename T, typename ACC>
+__device__ __forceinline__ ACC ld_acc(const T* p) {
+  if constexpr (std::is_same<T, bf16>::value || std::is_same<T, fp16>::value) return ACC(Cvt<T>::load(p));
+  else return ACC(*p);
+}
+template <typename T, typename ACC>
+__device__ __forceinline__ void st_acc(T* p, ACC v) {
+  if constexpr (std::is_same<T, bf16>::value || std::is_same<T, fp16>::value) Cvt<T>::store(p, float(v));
+  else *p = T(v);
+}
+// sum -> output value (mean applies the fp32 factor, ReduceMean.cu:9-22)
+template <typename ACC>
+__device__ __forceinline__ ACC project(ACC v, float factor, int is_mean) {
+  if (!is_mean) return v;
+  if constexpr (std::is_floating_point<ACC>::value) return v * ACC(factor);
+  else return ACC(float(v) * factor);
+}
+
+template <typename ACC>
+__device__ __forceinline__ ACC block_sum_lds(ACC v, ACC* lds) {
+  const int tid = threadIdx.x;
+  lds[tid] = v;
+  __syncthreads();
+  for (int s = blockDim.x >> 1; s > 0; s >>= 1) {
+    if (tid < s) lds[tid] += lds[tid + s];
+    __syncthreads();
+  }
+  ACC r = lds[0];
+  __syncthreads();
+  return r;
+}
+
+// ---------------------------------------------------------------------------
+// inner reduction, vector path (fp32 / bf16 / fp16 input, fp32 accumulate)
+// grid = (row groups, nsplit); a group of `tpr` threads takes one row chunk
+// ---------------------------------------------------------------------------
+struct InnerArgs {
+  const void* in;
+  void* out;          // OUT_T [rows] when nsplit == 1, else float [rows, nsplit]
+  int64_t rows;
+  int64_t row_stride; // elements
+  int64_t cols;
+  int64_t chunk;      // columns per split (multiple of the vector width)
+  int nsplit;
+  float factor;
+  int is_mean;
+};
+
+template <typename T, typename OUT_T, bool WAVE_ROW>
+__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
+void reduce_inner_vec_kernel(InnerArgs a) {
+  constexpr int VEC = VecIO<T>::N;
+  constexpr int U = 8;
+  __shared__ float red[kMaxWaves];
+  const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
+  const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
+  const int64_t row = WAVE_ROW
+      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)
+      : int64_t(blockIdx.x);
+  if (WAVE_ROW && row >= a.rows) return;
+  const int split = blockIdx.y;
+  const int64_t c0 = int64_t(split) * a.chunk;
+  const int64_t c1 = (c0 + a.chunk < a.cols) ? c0 + a.chunk : a.cols;
+  const T* p = static_cast<const T*>(a.in) + row * a.row_stride + c0;
+  const int64_t nvec = (c1 - c0) / VEC;
+
+  float acc[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) acc[u] = 0.f;
+  int64_t v = t;
+  for (; v + int64_t(U - 1) * tpr < nvec; v += int64_t(U) * tpr) {
+    u32x4 r[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) r[u] = ld16(p + (v + int64_t(u) * tpr) * VEC);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float f[VEC];
+      VecIO<T>::unpack(r[u], f);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[u] += f[j];
+    }
+  }
+  for (; v < nvec; v += tpr) {
+    float f[VEC];
+    VecIO<T>::unpack(ld16(p + v * VEC), f);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[0] += f[j];
+  }
+  // scalar tail of the last split
+  for (int64_t c = c0 + nvec * VEC + t; c < c1; c += tpr)
+    acc[1] += Cvt<T>::load(static_cast<const T*>(a.in) + row * a.row_stride + c);
+  float s = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+  if constexpr (WAVE_ROW) {
+    s = wave_sum(s);
+  } else {
+    s = block_allreduce<OpSum>(s, red, int(blockDim.x >> 6));
+  }
+  if (t == 0) {
+    if (a.nsplit == 1) st_acc<OUT_T, float>(static_cast<OUT_T*>(a.out) + row, project<float>(s, a.factor, a.is_mean));
+    else static_cast<float*>(a.out)[row * a.nsplit + split] = s;
+  }
+}
+
+// inner reduction, scalar path: any dtype / alignment; one workgroup per row
+template <typename T, typename ACC, typename OUT_T>
+__global__ __launch_bounds__(256)
+void reduce_inner_scalar_kernel(const T* in, OUT_T* out, int64_t rows, int64_t row_stride,
+                                int64_t cols, float factor, int is_mean) {
+  __shared__ ACC lds[256];
+  const int64_t row = blockIdx.x;
+  const T* p = in + row * row_stride;
+  ACC acc = ACC(0);
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) acc += ld_acc<T, ACC>(p + c);
+  acc = block_sum_lds<ACC>(acc, lds);
+  if (threadIdx.x == 0) st_acc<OUT_T, ACC>(out + row, project<ACC>(acc, factor, is_mean));
+}
+
+// ---------------------------------------------------------------------------
+// outer reduction, vector path: in [B, R, C] (C unit stride), out [B, C]
+// grid = (column tiles of 64 vectors, row splits, B); block = 64 x WY
+// ---------------------------------------------------------------------------
+struct OuterArgs {
+  const void* in;
+  void* out;            // OUT_T [B, C] when rsplit == 1, else float [rsplit, B, C]
+  int64_t B, R, C;
+  int64_t b_stride, r_stride;   // elements
+  int64_t rows_per_split;
+  int rsplit;
+  float factor;
+  int is_mean;
+};
+
+template <typename T, typename OUT_T>
+__global__ __launch_bounds__(1024)
+void reduce_outer_vec_kernel(OuterArgs a) {
+  constexpr int VEC = VecIO<T>::N;
+  constexpr int U = 8;
+  extern __shared__ float lds[];   // [WY][64 * VEC]
+  const int lane = threadIdx.x & 63;
+  const int w = threadIdx.x >> 6;
+  const int wy = blockDim.x >> 6;
+  const int64_t cv = int64_t(blockIdx.x) * kWave + lane;   // column vector index
+  const int64_t c = cv * VEC;
+  const bool col_ok = c < a.C;                              // C is a multiple of VEC here
+  const int split = blockIdx.y;
+  const int64_t b = blockIdx.z;
+  const int64_t r0 = int64_t(split) * a.rows_per_split;
+  const int64_t r1 = (r0 + a.rows_per_split < a.R) ? r0 + a.rows_per_split : a.R;
+  const T* p = static_cast<const T*>(a.in) + b * a.b_stride + c;
+
+  float acc[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+  if (col_ok) {
+    int64_t r = r0 + w;
+    for (; r + int64_t(U - 1) * wy < r1; r += int64_t(U) * wy) {
+      u32x4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = ld16(p + (r + int64_t(u) * wy) * a.r_stride);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        float f[VEC];
+        VecIO<T>::unpack(v[u], f);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += f[j];
+      }
+    }
+    for (; r < r1; r += wy) {
+      float f[VEC];
+      VecIO<T>::unpack(ld16(p + r * a.r_stride), f);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += f[j];
+    }
+  }
+  // fold the waves of the block: lane-major layout keeps LDS accesses conflict-free
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) lds[(w * VEC + j) * kWave + lane] = acc[j];
+  __syncthreads();
+  // thread (w, lane) finishes element j = w, w + wy, ... of its lane's vector
+  for (int j = w; j < VEC; j += wy) {
+    float s = 0.f;
+    for (int k = 0; k < wy; ++k) s += lds[(k * VEC + j) * kWave + lane];
+    if (col_ok) {
+      if (a.rsplit == 1)
+        st_acc<OUT_T, float>(static_cast<OUT_T*>(a.out) + b * a.C + c + j, project<float>(s, a.factor, a.is_mean));
+      else
+        static_cast<float*>(a.out)[(int64_t(split) * a.B + b) * a.C + c + j] = s;
+    }
+  }
+}
+
+// folds float partials [nparts, n] -> OUT_T [n]
+template <typename OUT_T>
+__global__ __launch_bounds__(256)
+void reduce_fold_partials_kernel(const float* part, OUT_T* out, int nparts, int64_t n, float factor,
+                                 int is_mean) {
+  const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int k = 0; k < nparts; ++k) s += part[int64_t(k) * n + i];
+  st_acc<OUT_T, float>(out + i, project<float>(s, factor, is_mean));
+}
+
+// outer reduction, scalar path: one thread per output column, any dtype
+template <typename T, typename ACC, typename OUT_T>
+__global__ __launch_bounds__(256)
+void reduce_outer_scalar_kernel(const T* in, OUT_T* out, int64_t B, int64_t R, int64_t C,
+                                int64_t b_stride, int64_t r_stride, float factor, int is_mean) {
+  const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= B * C) return;
+  const int64_t b = i / C, c = i - b * C;
+  const T* p = in + b * b_stride + c;
+  ACC acc = ACC(0);
+  for (int64_t r = 0; r < R; ++r) acc += ld_acc<T, ACC>(p + r * r_stride);
+  st_acc<OUT_T, ACC>(out + i, project<ACC>(acc, factor, is_mean));
+}
+
+// ---------------------------------------------------------------------------
+// generic strided reduction: one thread per output element
+// ---------------------------------------------------------------------------
+constexpr int kMaxDims = 8;
+struct GenericMeta {
+  int n_keep, n_red;
+  int64_t keep_size[kMaxDims], keep_stride[kMaxDims];   // outermost first
+  int64_t red_size[kMaxDims], red_stride[kMaxDims];     // outermost first
+  int64_t n_out, n_red_total;
+};
+
+template <typename T, typename ACC, typename OUT_T>
+__global__ __launch_bounds__(256)
+void reduce_generic_kernel(const T* in, OUT_T* out, GenericMeta m, float factor, int is_mean) {
+  const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= m.n_out) return;
+  int64_t rem = i, base = 0;
+  for (int d = m.n_keep - 1; d >= 0; --d) {
+    const int64_t q = rem / m.keep_size[d];
+    base += (rem - q * m.keep_size[d]) * m.keep_stride[d];
+    rem = q;
+  }
+  ACC acc = ACC(0);
+  for (int64_t k = 0; k < m.n_red_total; ++k) {
+    int64_t r = k, off = base;
+    for (int d = m.n_red - 1; d >= 0; --d) {
+      const int64_t q = r / m.red_size[d];
+      off += (r - q * m.red_size[d]) * m.red_stride[d];
+      r = q;
+    }
+    acc += ld_acc<T, ACC>(in + off);
+  }
+  st_acc<OUT_T, ACC>(out + i, project<ACC>(acc, factor, is_mean));
+}
+
+// ---------------------------------------------------------------------------
+// host-side planning
+// ---------------------------------------------------------------------------
+struct MergedDim { int64_t size, stride; bool reduce; };
+
+enum PlanKind { PLAN_EMPTY, PLAN_COPYLIKE, PLAN_INNER, PLAN_OUTER, PLAN_GENERIC };
+
+struct ReducePlan {
+  PlanKind kind = PLAN_GENERIC;
+  std::vector<MergedDim> dims;     // outermost first, extents > 1 only
+  int64_t n_out = 1, n_red = 1;
+  // inner
+  int64_t rows = 1, row_stride = 0, cols = 1;
+  // outer
+  int64_t B = 1, R = 1, C = 1, b_stride = 0, r_stride = 0;
+};
+
+// Same merging rule as the reference planner: walk from the innermost
+// dimension outwards and fuse a dimension into its inner neighbour when both
+// are reduced or both are kept and stride[i] == stride[i+1] * shape[i+1].
+static int make_plan(int ndim, const int64_t* shape, const int64_t* strides, int naxes,
+                     const int64_t* axes, ReducePlan* plan, const char* who) {
+  HK_REQUIRE(ndim >= 0 && ndim <= kMaxDims, HK_ERR_INVALID, "%s: ndim %d not in [0, %d]", who, ndim, kMaxDims);
+  HK_REQUIRE(naxes >= 0, HK_ERR_INVALID, "%s: negative axis count", who);
+  HK_REQUIRE(ndim == 0 || (shape && strides), HK_ERR_INVALID, "%s: null shape/strides", who);
+  HK_REQUIRE(naxes == 0 || axes, HK_ERR_INVALID, "%s: null axes", who);
+  bool red[kMaxDims] = {false};
+  for (int i = 0; i < naxes; ++i) {
+    HK_REQUIRE(axes[i] >= 0 && axes[i] < ndim, HK_ERR_INVALID, "%s: axis %lld out of range for %d dims",
+               who, (long long)axes[i], ndim);
+    red[axes[i]] = true;     // duplicates collapse, order is irrelevant
+  }
+  plan->dims.clear();
+  plan->n_out = 1;
+  plan->n_red = 1;
+  for (int d = 0; d < ndim; ++d) {
+    HK_REQUIRE(shape[d] >= 0, HK_ERR_INVALID, "%s: negative extent", who);
+    if (red[d]) plan->n_red *= shape[d]; else plan->n_out *= shape[d];
+  }
+  if (plan->n_out == 0) { plan->kind = PLAN_EMPTY; return HK_OK; }
+  std::vector<MergedDim> rev;   // innermost first
+  for (int d = ndim - 1; d >= 0; --d) {
+    if (shape[d] == 1) continue;
+    if (!rev.empty() && rev.back().reduce == red[d] &&
+        strides[d] == rev.back().stride * rev.back().size) {
+      rev.back().size *= shape[d];
+    } else {
+      rev.push_back(MergedDim{shape[d], strides[d], red[d]});
+    }
+  }
+  plan->dims.assign(rev.rbegin(), rev.rend());
+  std::vector<MergedDim> keep, rd;
+  for (auto& d : plan->dims) (d.reduce ? rd : keep).push_back(d);
+  if (rd.empty() || plan->n_red == 1) {
+    plan->kind = PLAN_COPYLIKE;   // nothing to add up: generic kernel copies / scales
+    return HK_OK;
+  }
+  if (plan->n_red == 0) { plan->kind = PLAN_GENERIC; return HK_OK; }  // sum over nothing = 0
+  const auto& dims = plan->dims;
+  if (rd.size() == 1 && rd[0].stride == 1 && keep.size() <= 1) {
+    plan->kind = PLAN_INNER;
+    plan->cols = rd[0].size;
+    plan->rows = keep.empty() ? 1 : keep[0].size;
+    plan->row_stride = keep.empty() ? 0 : keep[0].stride;
+    return HK_OK;
+  }
+  if (rd.size() == 1 && !dims.back().reduce && dims.back().stride == 1 && keep.size() <= 2 &&
+      dims.size() >= 2 && dims[dims.size() - 2].reduce) {
+    plan->kind = PLAN_OUTER;
+    plan->C = dims.back().size;
+    plan->R = rd[0].size;
+    plan->r_stride = rd[0].stride;
+    plan->B = keep.size() == 2 ? keep[0].size : 1;
+    plan->b_stride = keep.size() == 2 ? keep[0].stride : 0;
+    return HK_OK;
+  }
+  plan->kind = PLAN_GENERIC;
+  return HK_OK;
+}
+
+struct InnerShape { int tpr; int nsplit; int64_t chunk; bool vec; };
+struct OuterShape { int wy; int rsplit; int64_t rows_per_split; bool vec; };
+
+template <typename T>
+static InnerShape shape_inner(const ReducePlan& p, const void* in) {
+  constexpr int VEC = 16 / sizeof(T);
+  InnerShape s{};
+  s.vec = aligned16(in) && (p.rows == 1 || p.row_stride % VEC == 0);
+  const int64_t nvec = p.cols / VEC;
+  int tpr = tune_get(TUNE_REDUCE_INNER_THREADS);
+  if (tpr <= 0) tpr = nvec <= 64 * 16 ? 64 : (nvec <= 256 * 16 ? 256 : 1024);
+  tpr = std::min(1024, std::max(64, (tpr + 63) / 64 * 64));
+  s.tpr = tpr;
+  // few long rows: split columns so that ~4 workgroups per CU exist
+  const int64_t want_blocks = int64_t(device_cu_count()) * 4;
+  int64_t groups = tpr == 64 ? (p.rows + 3) / 4 : p.rows;
+  int64_t nsplit = 1;
+  if (groups < want_blocks && nvec > int64_t(tpr) * 32) {
+    nsplit = std::min<int64_t>((want_blocks + groups - 1) / groups, nvec / (int64_t(tpr) * 16));
+    nsplit = std::max<int64_t>(1, std::min<int64_t>(nsplit, 1024));
+  }
+  int64_t chunk_vec = (nvec + nsplit - 1) / nsplit;
+  if (chunk_vec == 0) chunk_vec = 1;
+  s.chunk = chunk_vec * VEC;
+  s.nsplit = int((p.cols + s.chunk - 1) / s.chunk);
+  if (s.nsplit < 1) s.nsplit = 1;
+  return s;
+}
+
+template <typename T>
+static OuterShape shape_outer(const ReducePlan& p, const void* in) {
+  constexpr int VEC = 16 / sizeof(T);
+  OuterShape s{};
+  s.vec = aligned16(in) && p.C % VEC == 0 && p.r_stride % VEC == 0 && (p.B == 1 || p.b_stride % VEC == 0);
+  const int64_t col_tiles = (p.C / VEC + 63) / 64;
+  // waves per block: enough rows per wave to keep 8 loads in flight
+  int wy = 16;
+  while (wy > 1 && p.R < int64_t(wy) * 8) wy >>= 1;
+  s.wy = wy;
+  int rsplit = tune_get(TUNE_REDUCE_OUTER_ROW_BLOCKS);
+  if (rsplit <= 0) {
+    const int64_t want_blocks = int64_t(device_cu_count()) * 2;
+    const int64_t have = col_tiles * p.B;
+    rsplit = int(std::max<int64_t>(1, (want_blocks + have - 1) / have));
+  }
+  const int64_t max_split = std::max<int64_t>(1, p.R / (int64_t(wy) * 8));
+  rsplit = int(std::min<int64_t>(rsplit, max_split));
+  rsplit = std::min(rsplit, 65535);
+  s.rows_per_split = (p.R + rsplit - 1) / rsplit;
+  s.rsplit = int((p.R + s.rows_per_split - 1) / s.rows_per_split);
+  return s;
+}
+
+template <typename T>
+static size_t workspace_for(const ReducePlan& p, const void* in) {
+  if (p.kind == PLAN_INNER) {
+    InnerShape s = shape_inner<T>(p, in);
+    return (s.vec && s.nsplit > 1) ? size_t(p.rows) * s.nsplit * sizeof(float) : 0;
+  }
+  if (p.kind == PLAN_OUTER) {
+    OuterShape s = shape_outer<T>(p, in);
+    return (s.vec && s.rsplit > 1) ? size_t(s.rsplit) * p.B * p.C * sizeof(float) : 0;
+  }
+  return 0;
+}
+
+static GenericMeta generic_meta(const ReducePlan& p) {
+  GenericMeta m{};
+  m.n_keep = 0; m.n_red = 0;
+  for (auto& d : p.dims) {
+    if (d.reduce) { m.red_size[m.n_red] = d.size; m.red_stride[m.n_red] = d.stride; ++m.n_red; }
+    else { m.keep_size[m.n_keep] = d.size; m.keep_stride[m.n_keep] = d.stride; ++m.n_keep; }
+  }
+  m.n_out = p.n_out;
+  m.n_red_total = p.n_red;
+  return m;
+}
+
+// fast kernels: T in {float, bf16, fp16}, fp32 accumulation
+template <typename T, typename OUT_T>
+static int reduce_fast(const ReducePlan& p, const void* in, void* out, float factor, int is_mean,
+                       void* ws, size_t ws_bytes, hipStream_t st, bool* handled) {
+  *handled = false;
+  if (p.kind == PLAN_INNER) {
+    InnerShape s = shape_inner<T>(p, in);
+    if (!s.vec) return HK_OK;
+    *handled = true;
+    InnerArgs a{};
+    a.in = in; a.rows = p.rows; a.row_stride = p.row_stride; a.cols = p.cols; a.chunk = s.chunk;
+    a.nsplit = s.nsplit; a.factor = factor; a.is_mean = is_mean;
+    if (s.nsplit > 1) {
+      const size_t need = size_t(p.rows) * s.nsplit * sizeof(float);
+      HK_REQUIRE(ws && ws_bytes >= need, HK_ERR_WORKSPACE, "hk_reduce: workspace of %zu bytes needed, %zu given", need, ws_bytes);
+      a.out = ws;
+    } else {
+      a.out = out;
+    }
+    HK_REQUIRE(p.rows <= 0x7fffffffLL, HK_ERR_INVALID, "hk_reduce: too many rows");
+    profile_before(st);
+    if (s.tpr == 64) {
+      dim3 grid(unsigned((p.rows + 3) / 4), unsigned(s.nsplit)), block(256);
+      hipLaunchKernelGGL((reduce_inner_vec_kernel<T, OUT_T, true>), grid, block, 0, st, a);
+    } else {
+      dim3 grid(unsigned(p.rows), unsigned(s.nsplit)), block{unsigned(s.tpr)};
+      hipLaunchKernelGGL((reduce_inner_vec_kernel<T, OUT_T, false>), grid, block, 0, st, a);
+    }
+    profile_after(st);
+    int rc = launch_check("reduce_inner_vec_kernel");
+    if (rc != HK_OK || s.nsplit == 1) return rc;
+    // second pass over the fp32 partials [rows, nsplit]
+    hipLaunchKernelGGL((reduce_inner_scalar_kernel<float, float, OUT_T>), dim3(unsigned(p.rows)), dim3(256), 0, st,
+                       static_cast<const float*>(ws), static_cast<OUT_T*>(out), p.rows, int64_t(s.nsplit),
+                       int64_t(s.nsplit), factor, is_mean);
+    return launch_check("reduce_inner_scalar_kernel");
+  }
+  if (p.kind == PLAN_OUTER) {
+    OuterShape s = shape_outer<T>(p, in);
+    if (!s.vec) return HK_OK;
+    *handled = true;
+    constexpr int VEC = 16 / sizeof(T);
+    OuterArgs a{};
+    a.in = in; a.B = p.B; a.R = p.R; a.C = p.C; a.b_stride = p.b_stride; a.r_stride = p.r_stride;
+    a.rows_per_split = s.rows_per_split; a.rsplit = s.rsplit; a.factor = factor; a.is_mean = is_mean;
+    if (s.rsplit > 1) {
+      const size_t need = size_t(s.rsplit) * p.B * p.C * sizeof(float);
+      HK_REQUIRE(ws && ws_bytes >= need, HK_ERR_WORKSPACE, "hk_reduce: workspace of %zu bytes needed, %zu given", need, ws_bytes);
+      a.out = ws;
+    } else {
+      a.out = out;
+    }
+    HK_REQUIRE(p.B <= 65535, HK_ERR_UNSUPPORTED, "hk_reduce: batch extent %lld too large for the column kernel", (long long)p.B);
+    const int64_t col_tiles = (p.C / VEC + 63) / 64;
+    dim3 grid(unsigned(col_tiles), unsigned(s.rsplit), unsigned(p.B)), block{unsigned(64 * s.wy)};
+    const size_t lds = size_t(s.wy) * 64 * VEC * sizeof(float);
+    profile_before(st);
+    hipLaunchKernelGGL((reduce_outer_vec_kernel<T, OUT_T>), grid, block, lds, st, a);
+    profile_after(st);
+    int rc = launch_check("reduce_outer_vec_kernel");
+    if (rc != HK_OK || s.rsplit == 1) return rc;
+    const int64_t n = p.B * p.C;
+    hipLaunchKernelGGL((reduce_fold_partials_kernel<OUT_T>), dim3(unsigned((n + 255) / 256)), dim3(256), 0, st,
+                       static_cast<const float*>(ws), static_cast<OUT_T*>(out), s.rsplit, n, factor, is_mean);
+    return launch_check("reduce_fold_partials_kernel");
+  }
+  return HK_OK;
+}
+
+template <typename T, typename ACC, typename OUT_T>
+static int reduce_slow(const ReducePlan& p, const void* in, void* out, float factor, int is_mean,
+                       hipStream_t st) {
+  const T* ip = static_cast<const T*>(in);
+  OUT_T* op = static_cast<OUT_T*>(out);
+  if (p.kind == PLAN_INNER) {
+    HK_REQUIRE(p.rows <= 0x7fffffffLL, HK_ERR_INVALID, "hk_reduce: too many rows");
+    hipLaunchKernelGGL((reduce_inner_scalar_kernel<T, ACC, OUT_T>), dim3(unsigned(p.rows)), dim3(256), 0, st, ip, op,
+                       p.rows, p.row_stride, p.cols, factor, is_mean);
+    return launch_check("reduce_inner_scalar_kernel");
+  }
+  if (p.kind == PLAN_OUTER) {
+    const int64_t n = p.B * p.C;
+    hipLaunchKernelGGL((reduce_outer_scalar_kernel<T, ACC, OUT_T>), dim3(unsigned((n + 255) / 256)), dim3(256), 0, st,
+                       ip, op, p.B, p.R, p.C, p.b_stride, p.r_stride, factor, is_mean);
+    return launch_check("reduce_outer_scalar_kernel");
+  }
+  GenericMeta m = generic_meta(p);
+  hipLaunchKernelGGL((reduce_generic_kernel<T, ACC, OUT_T>), dim3(unsigned((m.n_out + 255) / 256)), dim3(256), 0, st,
+                     ip, op, m, factor, is_mean);
+  return launch_check("reduce_generic_kernel");
+}
+
+template <typename T, typename OUT_T>
+static int reduce_float_like(const ReducePlan& p, const void* in, void* out, float factor, int is_mean,
+                             void* ws, size_t ws_bytes, hipStream_t st) {
+  bool handled = false;
+  int rc = reduce_fast<T, OUT_T>(p, in, out, factor, is_mean, ws, ws_bytes, st, &handled);
+  if (rc != HK_OK || handled) return rc;
+  return reduce_slow<T, float, OUT_T>(p, in, out, factor, is_mean, st);
+}
+
+} // namespace hk
+
+using namespace hk;
+
+extern "C" {
+
+int hk_reduce_workspace_bytes(int in_dtype, int ndim, const int64_t* shape, const int64_t* strides,
+                              int naxes, const int64_t* axes, size_t* bytes) {
+  HK_REQUIRE(bytes, HK_ERR_INVALID, "hk_reduce_workspace_bytes: null output");
+  *bytes = 0;
+  ReducePlan p;
+  int rc = make_plan(ndim, shape, strides, naxes, axes, &p, "hk_reduce_workspace_bytes");
+  if (rc != HK_OK) return rc;
+  // alignment of the data pointer is unknown here: assume the vector path
+  const void* aligned = reinterpret_cast<const void*>(uintptr_t(16));
+  switch (in_dtype) {
+    case HK_FLOAT32: *bytes = workspace_for<float>(p, aligned); break;
+    case HK_BFLOAT16: case HK_FLOAT16: *bytes = workspace_for<uint16_t>(p, aligned); break;
+    default: break;
+  }
+  return HK_OK;
+}
+
+int hk_reduce(int in_dtype, int out_dtype, const void* in, void* out, int ndim, const int64_t* shape,
+              const int64_t* strides, int naxes, const int64_t* axes, int op, void* workspace,
+              size_t workspace_bytes, hkStream_t stream) {
+  HK_REQUIRE(op == HK_REDUCE_SUM || op == HK_REDUCE_MEAN, HK_ERR_UNSUPPORTED, "hk_reduce: reduction %d not implemented", op);
+  ReducePlan p;
+  int rc = make_plan(ndim, shape, strides, naxes, axes, &p, "hk_reduce");
+  if (rc != HK_OK) return rc;
+  if (naxes == 0 || p.kind == PLAN_EMPTY) return HK_OK;   // nothing to reduce / nothing to write
+  HK_REQUIRE(in && out, HK_ERR_INVALID, "hk_reduce: null input/output");
+  HK_REQUIRE((p.n_out + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_reduce: output too large");
+  const int is_mean = op == HK_REDUCE_MEAN;
+  const float factor = is_mean ? 1.0f / float(size_t(p.n_red)) : 1.0f;
+  hipStream_t st = as_hip(stream);
+  const bool in16 = in_dtype == HK_BFLOAT16 || in_dtype == HK_FLOAT16;
+  HK_REQUIRE(out_dtype == in_dtype || (in16 && out_dtype == HK_FLOAT32), HK_ERR_UNSUPPORTED,
+             "hk_reduce: output dtype %d not implemented for input dtype %d", out_dtype, in_dtype);
+  ReducePlan q = p;
+  if (p.kind == PLAN_COPYLIKE) q.kind = PLAN_GENERIC;
+#define HK_RED_SLOW(T) return reduce_slow<T, AccOf<T>::type, T>(q, in, out, factor, is_mean, st)
+  switch (in_dtype) {
+    case HK_FLOAT32: return reduce_float_like<float, float>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
+    case HK_BFLOAT16:
+      if (out_dtype == HK_FLOAT32) return reduce_float_like<bf16, float>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
+      return reduce_float_like<bf16, bf16>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
+    case HK_FLOAT16:
+      if (out_dtype == HK_FLOAT32) return reduce_float_like<fp16, float>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
+      return reduce_float_like<fp16, fp16>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
+    case HK_FLOAT64: HK_RED_SLOW(double);
+    case HK_UINT8: HK_RED_SLOW(uint8_t);
+    case HK_INT8: HK_RED_SLOW(int8_t);
+    case HK_INT16: HK_RED_SLOW(int16_t);
+    case HK_INT32: HK_RED_SLOW(int32_t);
+    case HK_INT64: HK_RED_SLOW(int64_t);
+    default:
+      set_last_error("hk_reduce: not implemented for dtype %d", in_dtype);
+      return HK_ERR_UNSUPPORTED;
+  }
+#undef HK_RED_SLOW
+}
+
+} // extern "C"

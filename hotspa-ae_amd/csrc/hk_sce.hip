@@ -1,0 +1,499 @@
+// Fused softmax cross-entropy forward / backward for gfx950 (sparse int64
+// labels with an ignored index, and dense labels).
+//
+// A logits row is read from HBM once and kept in registers; each thread folds
+// its elements into a (max, sum-of-exp) pair, pairs are merged online across
+// lanes (DPP) and waves (LDS).  Forward writes one loss per row; backward
+// rescales the stored exponentials into (softmax - onehot) * grad_loss and
+// writes the row once.  Rows whose label equals the ignored index are not read
+// at all: loss 0 / a zero gradient row is written.
+#include "hk_common.cuh"
+
+#include <algorithm>
+
+namespace hk {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kNegInf = -__builtin_huge_valf();
+
+struct SceArgs {
+  const void* logits;
+  const int64_t* labels;   // sparse
+  const void* dlabels;     // dense labels (same shape as logits)
+  const void* grad_loss;   // backward
+  void* out;               // forward: loss [rows]; backward: dlogits
+  int64_t rows;
+  int cols;
+  int nvec;
+  int64_t ignored_index;
+  int stream_store;
+};
+
+template <bool WAVE_ROW>
+__device__ __forceinline__ void row_coords(int& tpr, int& t, int64_t& row, int& nwaves) {
+  tpr = WAVE_ROW ? kWave : int(blockDim.x);
+  t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
+  row = WAVE_ROW ? int64_t(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6) : int64_t(blockIdx.x);
+  nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
+}
+
+// ------------------------------- sparse forward ----------------------------
+template <typename T, int NV, bool WAVE_ROW>
+__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
+void sce_sparse_fwd_kernel(SceArgs a) {
+  constexpr int VEC = VecIO<T>::N;
+  __shared__ float red[kMaxWaves * 2];
+  int tpr, t, nwaves;
+  int64_t row;
+  row_coords<WAVE_ROW>(tpr, t, row, nwaves);
+  if (WAVE_ROW && row >= a.rows) return;
+
+  T* loss = static_cast<T*>(a.out);
+  const int64_t label = a.labels[row];
+  if (label == a.ignored_index) {          // uniform over the row's threads
+    if (t == 0) Cvt<T>::store(loss + row, 0.f);
+    return;
+  }
+  const T* xr = static_cast<const T*>(a.logits) + row * int64_t(a.cols);
+  u32x4 raw[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * tpr + t;
+    raw[i] = u32x4{0, 0, 0, 0};
+    if (v < a.nvec) raw[i] = ld16(xr + v * VEC);
+  }
+  float m = kNegInf;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (i * tpr + t < a.nvec) {
+      float f[VEC];
+      VecIO<T>::unpack(raw[i], f);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) m = fmaxf(m, f[j]);
+    }
+  }
+  const float ms = (m == kNegInf) ? 0.f : m;
+  const float off = -ms * kLog2e;
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (i * tpr + t < a.nvec) {
+      float f[VEC];
+      VecIO<T>::unpack(raw[i], f);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) s += __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, off));
+    }
+  }
+  MaxSumTuple p;
+  p.v[0] = m; p.v[1] = s;
+  p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);
+  if (t == 0) {
+    float r;
+    if (label >= 0 && label < a.cols) {
+      const float xl = Cvt<T>::load(xr + label);
+      r = (__builtin_amdgcn_logf(p.v[1]) * kLn2 + p.v[0]) - xl;
+    } else {
+      r = __builtin_nanf("");  // label outside [0, cols): no logit to gather
+    }
+    Cvt<T>::store(loss + row, r);
+  }
+}
+
+// ------------------------------- sparse backward ---------------------------
+template <typename T, int NV, bool WAVE_ROW>
+__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
+void sce_sparse_bwd_kernel(SceArgs a) {
+  constexpr int VEC = VecIO<T>::N;
+  __shared__ float red[kMaxWaves * 2];
+  int tpr, t, nwaves;
+  int64_t row;
+  row_coords<WAVE_ROW>(tpr, t, row, nwaves);
+  if (WAVE_ROW && row >= a.rows) return;
+
+  T* dxr = static_cast<T*>(a.out) + row * int64_t(a.cols);
+  const int64_t label = a.labels[row];
+  if (label == a.ignored_index) {
+    const u32x4 z = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = i * tpr + t;
+      if (v < a.nvec) {
+        if (a.stream_store) st16_stream(dxr + v * VEC, z);
+        else st16(dxr + v * VEC, z);
+      }
+    }
+    return;
+  }
+  const T* xr = static_cast<const T*>(a.logits) + row * int64_t(a.cols);
+  u32x4 raw[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * tpr + t;
+    raw[i] = u32x4{0, 0, 0, 0};
+    if (v < a.nvec) raw[i] = ld16(xr + v * VEC);
+  }
+  const float g = Cvt<T>::load(static_cast<const T*>(a.grad_loss) + row);
+  float e[NV * VEC];
+  float m = kNegInf;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const bool ok = i * tpr + t < a.nvec;
+    VecIO<T>::unpack(raw[i], &e[i * VEC]);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      if (!ok) e[i * VEC + j] = kNegInf;
+      m = fmaxf(m, e[i * VEC + j]);
+    }
+  }
+  const float ms = (m == kNegInf) ? 0.f : m;
+  const float off = -ms * kLog2e;
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV * VEC; ++k) {
+    e[k] = __builtin_amdgcn_exp2f(fmaf(e[k], kLog2e, off));
+    s += e[k];
+  }
+  MaxSumTuple p;
+  p.v[0] = m; p.v[1] = s;
+  p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);
+  const float M = (p.v[0] == kNegInf) ? 0.f : p.v[0];
+  const float scale = __builtin_amdgcn_exp2f((ms - M) * kLog2e) / p.v[1] * g;
+  const int lvec = int(label / VEC), lsub = int(label - int64_t(lvec) * VEC);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * tpr + t;
+    if (v < a.nvec) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) e[i * VEC + j] *= scale;
+      if (label >= 0 && v == lvec) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+          if (j == lsub) e[i * VEC + j] -= g;
+      }
+      const u32x4 o = VecIO<T>::pack(&e[i * VEC]);
+      if (a.stream_store) st16_stream(dxr + v * VEC, o);
+      else st16(dxr + v * VEC, o);
+    }
+  }
+}
+
+// ------------------------------- dense labels ------------------------------
+// loss = (M + log S) * sum(l) - sum(l * x);  dx = (softmax - l) * g
+template <typename T, int NV, bool WAVE_ROW, bool BWD>
+__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
+void sce_dense_kernel(SceArgs a) {
+  constexpr int VEC = VecIO<T>::N;
+  __shared__ float red[kMaxWaves * 2];
+  __shared__ float red2[kMaxWaves * 2];
+  int tpr, t, nwaves;
+  int64_t row;
+  row_coords<WAVE_ROW>(tpr, t, row, nwaves);
+  if (WAVE_ROW && row >= a.rows) return;
+
+  const T* xr = static_cast<const T*>(a.logits) + row * int64_t(a.cols);
+  const T* lr = static_cast<const T*>(a.dlabels) + row * int64_t(a.cols);
+  u32x4 rx[NV], rl[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * tpr + t;
+    rx[i] = u32x4{0, 0, 0, 0};
+    rl[i] = u32x4{0, 0, 0, 0};
+    if (v < a.nvec) { rx[i] = ld16(xr + v * VEC); rl[i] = ld16(lr + v * VEC); }
+  }
+  float m = kNegInf;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (i * tpr + t < a.nvec) {
+      float f[VEC];
+      VecIO<T>::unpack(rx[i], f);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) m = fmaxf(m, f[j]);
+    }
+  }
+  const float ms = (m == kNegInf) ? 0.f : m;
+  const float off = -ms * kLog2e;
+  float s = 0.f;
+  SumTuple<2> ls;
+  ls.v[0] = 0.f; ls.v[1] = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (i * tpr + t < a.nvec) {
+      float f[VEC], l[VEC];
+      VecIO<T>::unpack(rx[i], f);
+      VecIO<T>::unpack(rl[i], l);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        s += __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, off));
+        if constexpr (!BWD) { ls.v[0] += l[j]; ls.v[1] = fmaf(l[j], f[j], ls.v[1]); }
+      }
+    }
+  }
+  MaxSumTuple p;
+  p.v[0] = m; p.v[1] = s;
+  p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);
+  if constexpr (!BWD) {
+    ls = WAVE_ROW ? wave_allreduce_tuple(ls) : group_allreduce_tuple(ls, red2, 0, nwaves);
+    if (t == 0) {
+      const float lse = __builtin_amdgcn_logf(p.v[1]) * kLn2 + p.v[0];
+      Cvt<T>::store(static_cast<T*>(a.out) + row, lse * ls.v[0] - ls.v[1]);
+    }
+  } else {
+    const float g = Cvt<T>::load(static_cast<const T*>(a.grad_loss) + row);
+    const float M = (p.v[0] == kNegInf) ? 0.f : p.v[0];
+    const float inv = 1.0f / p.v[1];
+    const float off2 = -M * kLog2e;
+    T* dxr = static_cast<T*>(a.out) + row * int64_t(a.cols);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = i * tpr + t;
+      if (v < a.nvec) {
+        float f[VEC], l[VEC];
+        VecIO<T>::unpack(rx[i], f);
+        VecIO<T>::unpack(rl[i], l);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+          f[j] = (__builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, off2)) * inv - l[j]) * g;
+        const u32x4 o = VecIO<T>::pack(f);
+        if (a.stream_store) st16_stream(dxr + v * VEC, o);
+        else st16(dxr + v * VEC, o);
+      }
+    }
+  }
+}
+
+// ------------------------------- fallback ----------------------------------
+// Any cols / alignment / dtype: one workgroup per row, strided passes.
+template <typename T, typename CT>
+struct SceIO {
+  static __device__ __forceinline__ CT ld(const T* p) { return CT(Cvt<T>::load(p)); }
+  static __device__ __forceinline__ void st(T* p, CT v) { Cvt<T>::store(p, v); }
+};
+template <typename CT> __device__ __forceinline__ CT sce_exp(CT v);
+template <> __device__ __forceinline__ float sce_exp<float>(float v) { return __builtin_amdgcn_exp2f(v * kLog2e); }
+template <> __device__ __forceinline__ double sce_exp<double>(double v) { return exp(v); }
+template <typename CT> __device__ __forceinline__ CT sce_log(CT v);
+template <> __device__ __forceinline__ float sce_log<float>(float v) { return __builtin_amdgcn_logf(v) * kLn2; }
+template <> __device__ __forceinline__ double sce_log<double>(double v) { return log(v); }
+
+template <typename CT>
+__device__ __forceinline__ CT sce_block_reduce(CT v, CT* lds, bool is_max) {
+  const int tid = threadIdx.x;
+  lds[tid] = v;
+  __syncthreads();
+  for (int s = blockDim.x >> 1; s > 0; s >>= 1) {
+    if (tid < s) lds[tid] = is_max ? (lds[tid] > lds[tid + s] ? lds[tid] : lds[tid + s])
+                                   : lds[tid] + lds[tid + s];
+    __syncthreads();
+  }
+  CT r = lds[0];
+  __syncthreads();
+  return r;
+}
+
+// MODE 0: sparse fwd, 1: sparse bwd, 2: dense fwd, 3: dense bwd
+template <typename T, typename CT, int MODE>
+__global__ __launch_bounds__(256)
+void sce_generic_kernel(SceArgs a) {
+  __shared__ CT lds[256];
+  const int64_t row = blockIdx.x;
+  const int64_t cols = a.cols;
+  const T* xr = static_cast<const T*>(a.logits) + row * cols;
+  int64_t label = 0;
+  if (MODE < 2) {
+    label = a.labels[row];
+    if (label == a.ignored_index) {
+      if (MODE == 0) {
+        if (threadIdx.x == 0) SceIO<T, CT>::st(static_cast<T*>(a.out) + row, CT(0));
+      } else {
+        T* dxr = static_cast<T*>(a.out) + row * cols;
+        for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) SceIO<T, CT>::st(dxr + c, CT(0));
+      }
+      return;
+    }
+  }
+  CT m = -__builtin_huge_val();
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+    const CT v = SceIO<T, CT>::ld(xr + c);
+    m = v > m ? v : m;
+  }
+  m = sce_block_reduce<CT>(m, lds, true);
+  CT s = 0;
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) s += sce_exp<CT>(SceIO<T, CT>::ld(xr + c) - m);
+  s = sce_block_reduce<CT>(s, lds, false);
+  if (MODE == 0) {
+    if (threadIdx.x == 0) {
+      CT r;
+      if (label >= 0 && label < cols) r = (sce_log<CT>(s) + m) - SceIO<T, CT>::ld(xr + label);
+      else r = CT(__builtin_nanf(""));
+      SceIO<T, CT>::st(static_cast<T*>(a.out) + row, r);
+    }
+  } else if (MODE == 2) {
+    const T* lr = static_cast<const T*>(a.dlabels) + row * cols;
+    CT sl = 0, slx = 0;
+    for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+      const CT l = SceIO<T, CT>::ld(lr + c);
+      sl += l;
+      slx += l * SceIO<T, CT>::ld(xr + c);
+    }
+    sl = sce_block_reduce<CT>(sl, lds, false);
+    slx = sce_block_reduce<CT>(slx, lds, false);
+    if (threadIdx.x == 0)
+      SceIO<T, CT>::st(static_cast<T*>(a.out) + row, (sce_log<CT>(s) + m) * sl - slx);
+  } else {
+    const CT g = SceIO<T, CT>::ld(static_cast<const T*>(a.grad_loss) + row);
+    const CT inv = CT(1) / s;
+    T* dxr = static_cast<T*>(a.out) + row * cols;
+    const T* lr = MODE == 3 ? static_cast<const T*>(a.dlabels) + row * cols : nullptr;
+    for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+      CT pr = sce_exp<CT>(SceIO<T, CT>::ld(xr + c) - m) * inv;
+      if (MODE == 1) pr = (c == label) ? (pr * g - g) : pr * g;
+      else pr = (pr - SceIO<T, CT>::ld(lr + c)) * g;
+      SceIO<T, CT>::st(dxr + c, pr);
+    }
+  }
+}
+
+static inline int pow2_ceil_sce(int v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+static bool pick_sce_shape(int nvec, int max_nv_wave, int max_nv, int* threads, int* nv) {
+  const int forced = tune_get(TUNE_SCE_THREADS);
+  if (forced > 0) {
+    int t = std::min(1024, std::max(64, (forced + 63) / 64 * 64));
+    int n = pow2_ceil_sce((nvec + t - 1) / t);
+    if (n > max_nv) return false;
+    *threads = t; *nv = n;
+    return true;
+  }
+  if (nvec <= 64 * max_nv_wave) {
+    *threads = 64;
+    *nv = pow2_ceil_sce((nvec + 63) / 64);
+    return true;
+  }
+  for (int n = 4; n <= max_nv; n <<= 1) {
+    int t = ((nvec + n - 1) / n + 63) / 64 * 64;
+    if (t <= 1024) { *threads = t; *nv = n; return true; }
+  }
+  return false;
+}
+
+// MODE as in sce_generic_kernel
+template <typename T, int MODE, bool WAVE_ROW>
+static int launch_sce_nv(const SceArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
+#define HK_SCE_LAUNCH(N)                                                                         \
+  do {                                                                                           \
+    if constexpr (MODE == 0) hipLaunchKernelGGL((sce_sparse_fwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a); \
+    else if constexpr (MODE == 1) hipLaunchKernelGGL((sce_sparse_bwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a); \
+    else if constexpr (MODE == 2) hipLaunchKernelGGL((sce_dense_kernel<T, N, WAVE_ROW, false>), grid, block, 0, s, a); \
+    else hipLaunchKernelGGL((sce_dense_kernel<T, N, WAVE_ROW, true>), grid, block, 0, s, a);       \
+  } while (0)
+  profile_before(s);
+  switch (nv) {
+    case 1: HK_SCE_LAUNCH(1); break;
+    case 2: HK_SCE_LAUNCH(2); break;
+    case 4: HK_SCE_LAUNCH(4); break;
+    case 8:
+      if constexpr (MODE == 0 || VecIO<T>::N == 4) { HK_SCE_LAUNCH(8); break; }
+      [[fallthrough]];
+    default:
+      set_last_error("softmax cross-entropy: no kernel for %d vectors per thread", nv);
+      return HK_ERR_UNSUPPORTED;
+  }
+#undef HK_SCE_LAUNCH
+  profile_after(s);
+  return launch_check("sce kernel");
+}
+
+template <typename T, int MODE>
+static int sce_typed(SceArgs a, hipStream_t s) {
+  constexpr int VEC = VecIO<T>::N;
+  const bool vec_ok = a.cols % VEC == 0 && aligned16(a.logits) && aligned16(a.dlabels) &&
+                      (MODE == 0 || MODE == 2 || aligned16(a.out));
+  a.nvec = a.cols / VEC;
+  // sparse forward only keeps the packed row; the others keep 32 floats or two rows
+  const int max_nv = (MODE == 0) ? 8 : 32 / VEC;
+  const int max_nv_wave = (MODE == 0) ? 8 : 32 / VEC;
+  int threads = 0, nv = 0;
+  if (vec_ok && pick_sce_shape(a.nvec, max_nv_wave, max_nv, &threads, &nv)) {
+    if (threads == 64) {
+      dim3 grid(unsigned((a.rows + 3) / 4)), block(256);
+      return launch_sce_nv<T, MODE, true>(a, nv, grid, block, s);
+    }
+    dim3 grid{unsigned(a.rows)}, block{unsigned(threads)};
+    return launch_sce_nv<T, MODE, false>(a, nv, grid, block, s);
+  }
+  hipLaunchKernelGGL((sce_generic_kernel<T, float, MODE>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
+  return launch_check("sce_generic_kernel");
+}
+
+template <int MODE>
+static int sce_dispatch(int dtype, SceArgs& a, hipStream_t s, const char* who) {
+  HK_REQUIRE(a.rows >= 0 && a.cols >= 0, HK_ERR_INVALID, "%s: negative shape", who);
+  if (a.rows == 0) return HK_OK;
+  HK_REQUIRE(a.cols > 0, HK_ERR_INVALID, "%s: rows without classes", who);
+  HK_REQUIRE(a.rows <= 0x7fffffffLL, HK_ERR_INVALID, "%s: too many rows", who);
+  HK_REQUIRE(a.logits && a.out, HK_ERR_INVALID, "%s: null input/output", who);
+  HK_REQUIRE(MODE >= 2 || a.labels, HK_ERR_INVALID, "%s: null labels", who);
+  HK_REQUIRE(MODE < 2 || a.dlabels, HK_ERR_INVALID, "%s: null labels", who);
+  HK_REQUIRE((MODE & 1) == 0 || a.grad_loss, HK_ERR_INVALID, "%s: null grad_loss", who);
+  a.stream_store = tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1;
+  switch (dtype) {
+    case HK_FLOAT32: return sce_typed<float, MODE>(a, s);
+    case HK_BFLOAT16: return sce_typed<bf16, MODE>(a, s);
+    case HK_FLOAT16: return sce_typed<fp16, MODE>(a, s);
+    case HK_FLOAT64:
+      hipLaunchKernelGGL((sce_generic_kernel<double, double, MODE>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
+      return launch_check("sce_generic_kernel<double>");
+    default:
+      set_last_error("%s: not implemented for dtype %d", who, dtype);
+      return HK_ERR_UNSUPPORTED;
+  }
+}
+
+} // namespace hk
+
+using namespace hk;
+
+extern "C" {
+
+int hk_sce_sparse_fwd(int dtype, const void* logits, const int64_t* labels, void* loss, int64_t rows,
+                      int64_t cols, int64_t ignored_index, hkStream_t stream) {
+  HK_REQUIRE(cols <= 0x3fffffff, HK_ERR_INVALID, "hk_sce_sparse_fwd: cols too large");
+  SceArgs a{};
+  a.logits = logits; a.labels = labels; a.out = loss; a.rows = rows; a.cols = int(cols);
+  a.ignored_index = ignored_index;
+  return sce_dispatch<0>(dtype, a, as_hip(stream), "hk_sce_sparse_fwd");
+}
+
+int hk_sce_sparse_bwd(int dtype, const void* logits, const int64_t* labels, const void* grad_loss,
+                      void* dlogits, int64_t rows, int64_t cols, int64_t ignored_index,
+                      hkStream_t stream) {
+  HK_REQUIRE(cols <= 0x3fffffff, HK_ERR_INVALID, "hk_sce_sparse_bwd: cols too large");
+  SceArgs a{};
+  a.logits = logits; a.labels = labels; a.grad_loss = grad_loss; a.out = dlogits; a.rows = rows;
+  a.cols = int(cols); a.ignored_index = ignored_index;
+  return sce_dispatch<1>(dtype, a, as_hip(stream), "hk_sce_sparse_bwd");
+}
+
+int hk_sce_dense_fwd(int dtype, const void* logits, const void* labels, void* loss, int64_t rows,
+                     int64_t cols, hkStream_t stream) {
+  HK_REQUIRE(cols <= 0x3fffffff, HK_ERR_INVALID, "hk_sce_dense_fwd: cols too large");
+  SceArgs a{};
+  a.logits = logits; a.dlabels = labels; a.out = loss; a.rows = rows; a.cols = int(cols);
+  return sce_dispatch<2>(dtype, a, as_hip(stream), "hk_sce_dense_fwd");
+}
+
+int hk_sce_dense_bwd(int dtype, const void* logits, const void* labels, const void* grad_loss,
+                     void* dlogits, int64_t rows, int64_t cols, hkStream_t stream) {
+  HK_REQUIRE(cols <= 0x3fffffff, HK_ERR_INVALID, "hk_sce_dense_bwd: cols too large");
+  SceArgs a{};
+  a.logits = logits; a.dlabels = labels; a.grad_loss = grad_loss; a.out = dlogits; a.rows = rows;
+  a.cols = int(cols);
+  return sce_dispatch<3>(dtype, a, as_hip(stream), "hk_sce_dense_bwd");
+}
+
+} // extern "C"

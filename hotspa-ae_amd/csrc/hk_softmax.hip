@@ -1,0 +1,395 @@
+// Softmax forward / backward for gfx950.
+//
+// Last-dimension softmax keeps the row in registers (one HBM read, one write):
+// every thread folds its elements into a (max, sum-of-exp) pair, the pairs are
+// merged online across lanes (DPP) and waves (LDS), and the stored exponentials
+// are rescaled on the way out, so exp is evaluated once per element.
+// One wavefront per row for short rows, one workgroup per row for long rows.
+#include "hk_common.cuh"
+
+#include <algorithm>
+
+namespace hk {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kNegInf = -__builtin_huge_valf();
+
+struct SoftmaxArgs {
+  const void* x;    // forward: input;  backward: y
+  const void* dy;   // backward only
+  void* out;        // forward: y;      backward: dx
+  int64_t rows;
+  int cols;
+  int nvec;
+  int stream_store;
+};
+
+template <typename T, int NV, bool WAVE_ROW>
+__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
+void softmax_fwd_kernel(SoftmaxArgs a) {
+  constexpr int VEC = VecIO<T>::N;
+  __shared__ float red[kMaxWaves * 2];
+  const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
+  const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
+  const int64_t row = WAVE_ROW
+      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)
+      : int64_t(blockIdx.x);
+  if (WAVE_ROW && row >= a.rows) return;
+  const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
+
+  const T* xr = static_cast<const T*>(a.x) + row * int64_t(a.cols);
+  u32x4 raw[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * tpr + t;
+    raw[i] = u32x4{0, 0, 0, 0};
+    if (v < a.nvec) raw[i] = ld16(xr + v * VEC);
+  }
+  float e[NV * VEC];
+  float m = kNegInf;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const bool ok = i * tpr + t < a.nvec;
+    VecIO<T>::unpack(raw[i], &e[i * VEC]);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      if (!ok) e[i * VEC + j] = kNegInf;
+      m = fmaxf(m, e[i * VEC + j]);
+    }
+  }
+  const float ms = (m == kNegInf) ? 0.f : m;
+  const float off = -ms * kLog2e;
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV * VEC; ++k) {
+    e[k] = __builtin_amdgcn_exp2f(fmaf(e[k], kLog2e, off));
+    s += e[k];
+  }
+  MaxSumTuple p;
+  p.v[0] = m; p.v[1] = s;
+  p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);
+  const float M = (p.v[0] == kNegInf) ? 0.f : p.v[0];
+  const float scale = __builtin_amdgcn_exp2f((ms - M) * kLog2e) / p.v[1];
+
+  T* yr = static_cast<T*>(a.out) + row * int64_t(a.cols);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * tpr + t;
+    if (v < a.nvec) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) e[i * VEC + j] *= scale;
+      const u32x4 o = VecIO<T>::pack(&e[i * VEC]);
+      if (a.stream_store) st16_stream(yr + v * VEC, o);
+      else st16(yr + v * VEC, o);
+    }
+  }
+}
+
+template <typename T, int NV, bool WAVE_ROW>
+__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
+void softmax_bwd_kernel(SoftmaxArgs a) {
+  constexpr int VEC = VecIO<T>::N;
+  __shared__ float red[kMaxWaves];
+  const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
+  const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
+  const int64_t row = WAVE_ROW
+      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)
+      : int64_t(blockIdx.x);
+  if (WAVE_ROW && row >= a.rows) return;
+  const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
+
+  const T* yr = static_cast<const T*>(a.x) + row * int64_t(a.cols);
+  const T* dyr = static_cast<const T*>(a.dy) + row * int64_t(a.cols);
+  u32x4 ry[NV], rdy[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * tpr + t;
+    ry[i] = u32x4{0, 0, 0, 0};
+    rdy[i] = u32x4{0, 0, 0, 0};
+    if (v < a.nvec) { ry[i] = ld16(yr + v * VEC); rdy[i] = ld16(dyr + v * VEC); }
+  }
+  SumTuple<1> s;
+  s.v[0] = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    float y[VEC], d[VEC];
+    VecIO<T>::unpack(ry[i], y);
+    VecIO<T>::unpack(rdy[i], d);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) s.v[0] = fmaf(y[j], d[j], s.v[0]);  // padding is zero
+  }
+  s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red, 0, nwaves);
+  const float dot = s.v[0];
+  T* dxr = static_cast<T*>(a.out) + row * int64_t(a.cols);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * tpr + t;
+    if (v < a.nvec) {
+      float y[VEC], d[VEC];
+      VecIO<T>::unpack(ry[i], y);
+      VecIO<T>::unpack(rdy[i], d);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) d[j] = y[j] * (d[j] - dot);
+      const u32x4 o = VecIO<T>::pack(d);
+      if (a.stream_store) st16_stream(dxr + v * VEC, o);
+      else st16(dxr + v * VEC, o);
+    }
+  }
+}
+
+// Softmax along a dimension of extent `dim` with element stride `inner`
+// (inner == 1: rows too long or too unaligned for the register kernels).
+// One thread walks one (outer, inner) position, threads of a wave sit on
+// neighbouring inner positions; for inner == 1 one workgroup takes one row.
+template <typename T, typename CT>
+struct SmIO {
+  static __device__ __forceinline__ CT ld(const T* p) { return CT(Cvt<T>::load(p)); }
+  static __device__ __forceinline__ void st(T* p, CT v) { Cvt<T>::store(p, v); }
+};
+
+template <typename CT> __device__ __forceinline__ CT exp_ct(CT v);
+template <> __device__ __forceinline__ float exp_ct<float>(float v) { return __builtin_amdgcn_exp2f(v * kLog2e); }
+template <> __device__ __forceinline__ double exp_ct<double>(double v) { return exp(v); }
+
+template <typename T, typename CT>
+__global__ __launch_bounds__(256)
+void softmax_fwd_strided_kernel(const T* x, T* y, int64_t outer, int64_t dim, int64_t inner) {
+  const int64_t pos = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (pos >= outer * inner) return;
+  const int64_t o = pos / inner, in = pos - o * inner;
+  const T* xp = x + o * dim * inner + in;
+  T* yp = y + o * dim * inner + in;
+  CT m = -__builtin_huge_val(), s = 0;
+  for (int64_t k = 0; k < dim; ++k) {
+    const CT v = SmIO<T, CT>::ld(xp + k * inner);
+    m = v > m ? v : m;
+  }
+  for (int64_t k = 0; k < dim; ++k) s += exp_ct<CT>(SmIO<T, CT>::ld(xp + k * inner) - m);
+  const CT inv = CT(1) / s;
+  for (int64_t k = 0; k < dim; ++k)
+    SmIO<T, CT>::st(yp + k * inner, exp_ct<CT>(SmIO<T, CT>::ld(xp + k * inner) - m) * inv);
+}
+
+template <typename T, typename CT>
+__global__ __launch_bounds__(256)
+void softmax_bwd_strided_kernel(const T* y, const T* dy, T* dx, int64_t outer, int64_t dim,
+                                int64_t inner) {
+  const int64_t pos = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (pos >= outer * inner) return;
+  const int64_t o = pos / inner, in = pos - o * inner;
+  const int64_t base = o * dim * inner + in;
+  CT dot = 0;
+  for (int64_t k = 0; k < dim; ++k)
+    dot += SmIO<T, CT>::ld(y + base + k * inner) * SmIO<T, CT>::ld(dy + base + k * inner);
+  for (int64_t k = 0; k < dim; ++k) {
+    const CT yv = SmIO<T, CT>::ld(y + base + k * inner);
+    SmIO<T, CT>::st(dx + base + k * inner, yv * (SmIO<T, CT>::ld(dy + base + k * inner) - dot));
+  }
+}
+
+template <typename CT>
+__device__ __forceinline__ CT block_reduce_generic(CT v, CT* lds, bool is_max) {
+  const int tid = threadIdx.x;
+  lds[tid] = v;
+  __syncthreads();
+  for (int s = blockDim.x >> 1; s > 0; s >>= 1) {
+    if (tid < s) lds[tid] = is_max ? (lds[tid] > lds[tid + s] ? lds[tid] : lds[tid + s])
+                                   : lds[tid] + lds[tid + s];
+    __syncthreads();
+  }
+  CT r = lds[0];
+  __syncthreads();
+  return r;
+}
+
+template <typename T, typename CT>
+__global__ __launch_bounds__(256)
+void softmax_fwd_longrow_kernel(const T* x, T* y, int64_t cols) {
+  __shared__ CT lds[256];
+  const T* xr = x + int64_t(blockIdx.x) * cols;
+  T* yr = y + int64_t(blockIdx.x) * cols;
+  CT m = -__builtin_huge_val();
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+    const CT v = SmIO<T, CT>::ld(xr + c);
+    m = v > m ? v : m;
+  }
+  m = block_reduce_generic<CT>(m, lds, true);
+  CT s = 0;
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) s += exp_ct<CT>(SmIO<T, CT>::ld(xr + c) - m);
+  s = block_reduce_generic<CT>(s, lds, false);
+  const CT inv = CT(1) / s;
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x)
+    SmIO<T, CT>::st(yr + c, exp_ct<CT>(SmIO<T, CT>::ld(xr + c) - m) * inv);
+}
+
+template <typename T, typename CT>
+__global__ __launch_bounds__(256)
+void softmax_bwd_longrow_kernel(const T* y, const T* dy, T* dx, int64_t cols) {
+  __shared__ CT lds[256];
+  const int64_t base = int64_t(blockIdx.x) * cols;
+  CT dot = 0;
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x)
+    dot += SmIO<T, CT>::ld(y + base + c) * SmIO<T, CT>::ld(dy + base + c);
+  dot = block_reduce_generic<CT>(dot, lds, false);
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+    const CT yv = SmIO<T, CT>::ld(y + base + c);
+    SmIO<T, CT>::st(dx + base + c, yv * (SmIO<T, CT>::ld(dy + base + c) - dot));
+  }
+}
+
+static inline int pow2_ceil_sm(int v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+// threads per row / vectors per thread for a row of nvec 16-byte vectors
+static bool pick_softmax_shape(int nvec, int max_nv_wave, int max_nv, int* threads, int* nv) {
+  const int forced = tune_get(TUNE_SOFTMAX_THREADS);
+  if (forced > 0) {
+    int t = std::min(1024, std::max(64, (forced + 63) / 64 * 64));
+    int n = pow2_ceil_sm((nvec + t - 1) / t);
+    if (n > max_nv) return false;
+    *threads = t; *nv = n;
+    return true;
+  }
+  if (nvec <= 64 * max_nv_wave) {
+    *threads = 64;
+    *nv = pow2_ceil_sm((nvec + 63) / 64);
+    return true;
+  }
+  for (int n = 4; n <= max_nv; n <<= 1) {
+    int t = ((nvec + n - 1) / n + 63) / 64 * 64;
+    if (t <= 1024) { *threads = t; *nv = n; return true; }
+  }
+  return false;
+}
+
+template <typename T, bool BWD, bool WAVE_ROW>
+static int launch_softmax_nv(const SoftmaxArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
+#define HK_SM_CASE(N)                                                                      \
+  case N:                                                                                  \
+    if constexpr (BWD) hipLaunchKernelGGL((softmax_bwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a); \
+    else hipLaunchKernelGGL((softmax_fwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a);   \
+    break;
+  profile_before(s);
+  switch (nv) {
+    HK_SM_CASE(1) HK_SM_CASE(2) HK_SM_CASE(4) HK_SM_CASE(8)
+    case 16:
+      if constexpr (VecIO<T>::N == 4 && !BWD) {
+        hipLaunchKernelGGL((softmax_fwd_kernel<T, 16, WAVE_ROW>), grid, block, 0, s, a);
+        break;
+      }
+      [[fallthrough]];
+    default:
+      set_last_error("softmax: no kernel for %d vectors per thread", nv);
+      return HK_ERR_UNSUPPORTED;
+  }
+#undef HK_SM_CASE
+  profile_after(s);
+  return launch_check(BWD ? "softmax_bwd_kernel" : "softmax_fwd_kernel");
+}
+
+template <typename T, bool BWD>
+static int softmax_lastdim_typed(SoftmaxArgs a, hipStream_t s) {
+  constexpr int VEC = VecIO<T>::N;
+  const bool vec_ok = a.cols % VEC == 0 && aligned16(a.x) && aligned16(a.dy) && aligned16(a.out);
+  a.nvec = a.cols / VEC;
+  // forward keeps NV*VEC exponentials per thread: at most 64 floats
+  // backward holds y and dy: at most 4 vectors of each per thread
+  const int max_nv = BWD ? 4 : 64 / VEC;
+  const int max_nv_wave = BWD ? 4 : std::min(8, 64 / VEC);
+  int threads = 0, nv = 0;
+  if (vec_ok && pick_softmax_shape(a.nvec, max_nv_wave, max_nv, &threads, &nv)) {
+    if (threads == 64) {
+      dim3 grid(unsigned((a.rows + 3) / 4)), block(256);
+      return launch_softmax_nv<T, BWD, true>(a, nv, grid, block, s);
+    }
+    dim3 grid{unsigned(a.rows)}, block{unsigned(threads)};
+    return launch_softmax_nv<T, BWD, false>(a, nv, grid, block, s);
+  }
+  if constexpr (BWD) {
+    hipLaunchKernelGGL((softmax_bwd_longrow_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s,
+                       static_cast<const T*>(a.x), static_cast<const T*>(a.dy), static_cast<T*>(a.out),
+                       int64_t(a.cols));
+    return launch_check("softmax_bwd_longrow_kernel");
+  } else {
+    hipLaunchKernelGGL((softmax_fwd_longrow_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s,
+                       static_cast<const T*>(a.x), static_cast<T*>(a.out), int64_t(a.cols));
+    return launch_check("softmax_fwd_longrow_kernel");
+  }
+}
+
+template <typename T, typename CT, bool BWD>
+static int softmax_strided_typed(const void* x, const void* dy, void* out, int64_t outer, int64_t dim,
+                                 int64_t inner, hipStream_t s) {
+  if (inner == 1) {
+    if constexpr (BWD) {
+      hipLaunchKernelGGL((softmax_bwd_longrow_kernel<T, CT>), dim3(unsigned(outer)), dim3(256), 0, s,
+                         static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<T*>(out), dim);
+    } else {
+      hipLaunchKernelGGL((softmax_fwd_longrow_kernel<T, CT>), dim3(unsigned(outer)), dim3(256), 0, s,
+                         static_cast<const T*>(x), static_cast<T*>(out), dim);
+    }
+    return launch_check("softmax_longrow_kernel");
+  }
+  const int64_t npos = outer * inner;
+  const int64_t blocks = (npos + 255) / 256;
+  if constexpr (BWD) {
+    hipLaunchKernelGGL((softmax_bwd_strided_kernel<T, CT>), dim3(unsigned(blocks)), dim3(256), 0, s,
+                       static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<T*>(out), outer,
+                       dim, inner);
+  } else {
+    hipLaunchKernelGGL((softmax_fwd_strided_kernel<T, CT>), dim3(unsigned(blocks)), dim3(256), 0, s,
+                       static_cast<const T*>(x), static_cast<T*>(out), outer, dim, inner);
+  }
+  return launch_check("softmax_strided_kernel");
+}
+
+template <bool BWD>
+static int softmax_dispatch(int dtype, const void* x, const void* dy, void* out, int64_t outer,
+                            int64_t dim, int64_t inner, hipStream_t s, const char* who) {
+  HK_REQUIRE(outer >= 0 && dim >= 0 && inner >= 0, HK_ERR_INVALID, "%s: negative extent", who);
+  if (outer == 0 || dim == 0 || inner == 0) return HK_OK;
+  HK_REQUIRE(x && out && (!BWD || dy), HK_ERR_INVALID, "%s: null input/output", who);
+  HK_REQUIRE(outer <= 0x7fffffffLL && (outer * inner + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID,
+             "%s: too many rows", who);
+  if (inner == 1 && dim <= 0x3fffffff && dtype != HK_FLOAT64) {
+    SoftmaxArgs a{};
+    a.x = x; a.dy = dy; a.out = out; a.rows = outer; a.cols = int(dim);
+    a.stream_store = tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1;
+    switch (dtype) {
+      case HK_FLOAT32: return softmax_lastdim_typed<float, BWD>(a, s);
+      case HK_BFLOAT16: return softmax_lastdim_typed<bf16, BWD>(a, s);
+      case HK_FLOAT16: return softmax_lastdim_typed<fp16, BWD>(a, s);
+      default: break;
+    }
+  }
+  switch (dtype) {
+    case HK_FLOAT32: return softmax_strided_typed<float, float, BWD>(x, dy, out, outer, dim, inner, s);
+    case HK_BFLOAT16: return softmax_strided_typed<bf16, float, BWD>(x, dy, out, outer, dim, inner, s);
+    case HK_FLOAT16: return softmax_strided_typed<fp16, float, BWD>(x, dy, out, outer, dim, inner, s);
+    case HK_FLOAT64: return softmax_strided_typed<double, double, BWD>(x, dy, out, outer, dim, inner, s);
+    default:
+      set_last_error("%s: not implemented for dtype %d", who, dtype);
+      return HK_ERR_UNSUPPORTED;
+  }
+}
+
+} // namespace hk
+
+using namespace hk;
+
+extern "C" {
+
+int hk_softmax_fwd(int dtype, const void* x, void* y, int64_t outer, int64_t dim, int64_t inner,
+                   hkStream_t stream) {
+  return softmax_dispatch<false>(dtype, x, nullptr, y, outer, dim, inner, as_hip(stream), "hk_softmax_fwd");
+}
+
+int hk_softmax_bwd(int dtype, const void* y, const void* dy, void* dx, int64_t outer, int64_t dim,
+                   int64_t inner, hkStream_t stream) {
+  return softmax_dispatch<true>(dtype, y, dy, dx, outer, dim, inner, as_hip(stream), "hk_softmax_bwd");
+}
+
+} // extern "C"

@@ -1,0 +1,252 @@
+/*
+ * hk_rowwise.h — C-ABI of the gfx950 (MI355X) device layer for Hetu's row-wise
+ * operator kernels: LayerNorm / RMSNorm forward+backward, Softmax
+ * forward+backward, fused SoftmaxCrossEntropy (sparse int64 labels and dense
+ * labels) forward+backward, Reduce sum/mean over arbitrary axes, plus the
+ * stream / event / memory calls the host-side wrappers need.
+ *
+ * Everything here is `extern "C"`, plain pointers and sizes.  All device
+ * pointers are HIP device addresses on the current device; `hkStream_t` is a
+ * `hipStream_t` (NULL = the null stream).  Every function returns HK_OK (0) or
+ * a negative error code and never throws; `hk_last_error()` gives the message
+ * of the calling thread's last failure.  Kernels are launched asynchronously
+ * on the given stream; no entry point synchronises the device.
+ *
+ * dtype codes equal the numeric values of hetu::DataType
+ * (hetu/core/dtype.h:9-22) so the C++ layer can pass them through.
+ */
+#ifndef HK_ROWWISE_H_
+#define HK_ROWWISE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HK_API __attribute__((visibility("default")))
+
+/* ---- error codes -------------------------------------------------------- */
+enum {
+  HK_OK = 0,
+  HK_ERR_INVALID = -1,      /* bad argument (null pointer, negative size, bad axis ...) */
+  HK_ERR_UNSUPPORTED = -2,  /* dtype / feature not implemented (HT_NOT_IMPLEMENTED upstream) */
+  HK_ERR_HIP = -3,          /* a HIP runtime call failed */
+  HK_ERR_WORKSPACE = -4     /* workspace missing or too small */
+};
+
+/* ---- dtype codes: hetu/core/dtype.h:9-22 -------------------------------- */
+enum {
+  HK_UINT8 = 0,
+  HK_INT8 = 1,
+  HK_INT16 = 2,
+  HK_INT32 = 3,
+  HK_INT64 = 4,
+  HK_FLOAT16 = 5,
+  HK_FLOAT32 = 6,
+  HK_FLOAT64 = 7,
+  HK_BFLOAT16 = 8,
+  HK_BOOL = 9
+};
+
+/* ---- reduction codes: hetu/core/reduction_type.h:7-15 (kSUM, kMEAN) ------ */
+enum { HK_REDUCE_SUM = 0, HK_REDUCE_MEAN = 1 };
+
+/* second per-row statistic written/read by the LayerNorm entries */
+enum {
+  HK_STAT_VAR = 0,  /* biased variance   — LayerNormCuda,      LayerNorm.cu:43-50   */
+  HK_STAT_RSTD = 1  /* 1/sqrt(var + eps) — FusedLayerNormCuda, FusedLayerNorm.cu:422 */
+};
+
+typedef struct ihipStream_t* hkStream_t;
+typedef struct ihipEvent_t* hkEvent_t;
+
+HK_API const char* hk_last_error(void);
+HK_API const char* hk_version(void);
+
+/* ======================================================================== *
+ * Device / memory / stream / event layer.
+ * Replaces the raw CUDA calls under hetu/impl/stream/CUDAStream.{h,cc},
+ * hetu/impl/memory/CUDACachingMemoryPool.cu and hetu/impl/utils/cuda_utils.h.
+ * ======================================================================== */
+HK_API int hk_device_count(int* count);                 /* cuda_utils.h: GetDeviceCount      */
+HK_API int hk_set_device(int device);                   /* cuda_utils.h:103-127 device guard  */
+HK_API int hk_get_device(int* device);
+HK_API int hk_device_sync(void);
+HK_API int hk_mem_get_info(size_t* free_bytes, size_t* total_bytes);
+HK_API int hk_device_cu_count(int device, int* cus);    /* Device::dprop().multiProcessorCount */
+
+HK_API int hk_malloc(void** ptr, size_t bytes);         /* CUDACachingMemoryPool.cu: cudaMalloc */
+HK_API int hk_free(void* ptr);
+HK_API int hk_host_malloc(void** ptr, size_t bytes);    /* pinned host memory */
+HK_API int hk_host_free(void* ptr);
+HK_API int hk_memcpy_h2d(void* dst, const void* src, size_t bytes, hkStream_t stream);
+HK_API int hk_memcpy_d2h(void* dst, const void* src, size_t bytes, hkStream_t stream);
+HK_API int hk_memcpy_d2d(void* dst, const void* src, size_t bytes, hkStream_t stream);
+/* fill with a byte value through a kernel (safe under graph capture) */
+HK_API int hk_memset(void* dst, int value, size_t bytes, hkStream_t stream);
+
+/* CUDAStream.cc:28-40 — non-blocking streams at default priority */
+HK_API int hk_stream_create(hkStream_t* stream);
+HK_API int hk_stream_destroy(hkStream_t stream);
+HK_API int hk_stream_sync(hkStream_t stream);           /* CUDAStream.cc:62-64 */
+HK_API int hk_stream_wait_event(hkStream_t stream, hkEvent_t event); /* CUDAEvent::Block */
+
+/* CUDAStream.h:50-114 — CUDAEvent */
+HK_API int hk_event_create(hkEvent_t* event, int enable_timing);
+HK_API int hk_event_destroy(hkEvent_t event);
+HK_API int hk_event_record(hkEvent_t event, hkStream_t stream);
+HK_API int hk_event_sync(hkEvent_t event);
+HK_API int hk_event_query(hkEvent_t event, int* done);
+/* nanoseconds from `start` to `stop` (CUDAEvent::TimeSince, CUDAStream.h:96-109) */
+HK_API int hk_event_elapsed_ns(hkEvent_t start, hkEvent_t stop, int64_t* ns);
+
+/* Launch-shape overrides for tuning sweeps; key names are listed in
+ * hk_tune_keys().  value 0 restores the automatic choice. */
+HK_API int hk_tune_set(const char* key, int value);
+HK_API const char* hk_tune_keys(void);
+
+/* Measurement hook: the next launch of an operator's main kernel (the one that
+ * streams the rows; not the small fold / finalize launches) made by the calling
+ * thread records `before` and `after` around that kernel on its stream, then the
+ * hook clears itself.  Pass NULLs to cancel. */
+HK_API int hk_profile_next_kernel(hkEvent_t before, hkEvent_t after);
+
+/* Plain streaming copy kernel of `bytes` (multiple of 16, 16-byte aligned):
+ * calibration reference for bandwidth counters and timings. */
+HK_API int hk_copy_kernel(void* dst, const void* src, size_t bytes, hkStream_t stream);
+
+/* Gathers a strided view into a dense row-major array (what the reference's
+ * OffsetCalculator does per element, hetu/impl/utils/offset_calculator.cuh:16-68).
+ * shape/strides in elements, ndim <= 8. */
+HK_API int hk_strided_copy(int dtype, const void* src, void* dst, int ndim,
+                           const int64_t* shape, const int64_t* src_strides,
+                           hkStream_t stream);
+
+/* ======================================================================== *
+ * LayerNorm.
+ * x, y: [rows, cols] dense, dtype `dtype` (fp32 / bf16 / fp16); gamma, beta:
+ * [cols] same dtype (either may be NULL: gamma=1 / beta=0).
+ * mean, stat: [rows] of `stats_dtype` (HK_FLOAT32 or `dtype`).
+ *
+ * Replaces LayerNormCuda (hetu/impl/kernel/LayerNorm.cu:66-121; stat_kind
+ * HK_STAT_VAR, stats_dtype = dtype) and FusedLayerNormCuda
+ * (hetu/impl/kernel/FusedLayerNorm.cu:967-1004; HK_STAT_RSTD, HK_FLOAT32).
+ * ======================================================================== */
+HK_API int hk_layer_norm_fwd(int dtype, const void* x, const void* gamma, const void* beta,
+                             void* y, void* mean, void* stat, int stats_dtype, int stat_kind,
+                             int64_t rows, int64_t cols, float eps, hkStream_t stream);
+
+/* Bytes of scratch hk_layer_norm_bwd / hk_dropout_add_ln_bwd need for the
+ * column-sum partials of dgamma / dbeta. */
+HK_API int hk_norm_bwd_workspace_bytes(int dtype, int64_t rows, int64_t cols, size_t* bytes);
+
+/* LayerNorm backward.  dy, x_or_y, dx: [rows, cols]; dgamma, dbeta: [cols] of
+ * `dtype` (either may be NULL).  mean/stat as written by hk_layer_norm_fwd.
+ *  memory_efficient = 0: x_or_y is the forward input x.
+ *  memory_efficient = 1: x_or_y is the forward OUTPUT y and x_hat is recomputed
+ *    as (y - beta) / clamp_by_magnitude(gamma, eps)  (FusedLayerNorm.cu:486-503).
+ *  clamp_gamma: apply clamp_by_magnitude(gamma, eps) to gamma in dx, as
+ *    cuComputeGradInput does unconditionally (FusedLayerNorm.cu:911-938).
+ * Replaces LayerNormGradientCuda (LayerNorm.cu:235-337) and
+ * FusedLayerNormGradientCuda (FusedLayerNorm.cu:1006-1144). */
+HK_API int hk_layer_norm_bwd(int dtype, const void* dy, const void* x_or_y, const void* gamma,
+                             const void* beta, const void* mean, const void* stat,
+                             int stats_dtype, int stat_kind, void* dx, void* dgamma,
+                             void* dbeta, int64_t rows, int64_t cols, float eps,
+                             int memory_efficient, int clamp_gamma, void* workspace,
+                             size_t workspace_bytes, hkStream_t stream);
+
+/* ======================================================================== *
+ * Dropout-add-LayerNorm / RMSNorm (flash-attention layer_norm path).
+ * Replaces DropoutAddLnFwdCuda (hetu/impl/kernel/RMSNorm.cu:91-264) and
+ * DropoutAddLnBwdCuda (RMSNorm.cu:266-470) for the configuration Hetu's
+ * RMSNorm / LayerNorm modules use: dropout_p = 0, no rowscale / colscale /
+ * subset.  x0: [rows, cols] `itype`; residual (optional, may be NULL): [rows,
+ * cols] `rtype`; gamma, beta (beta optional): [cols] `wtype`; z: [rows, cols]
+ * `itype`; x_out (optional): the pre-norm sum x0 + residual in `rtype`, written
+ * when non-NULL; mu, rsigma: [rows] fp32.
+ *   rs = rsqrt(m2/cols + eps + (is_rms ? mu^2 : 0)),  z = gamma*rs*(x - (is_rms?0:mu)) + beta
+ *   (flash-attn csrc/layer_norm ln_fwd_kernels.cuh:155-177).
+ * ======================================================================== */
+HK_API int hk_dropout_add_ln_fwd(int itype, int rtype, int wtype, const void* x0,
+                                 const void* residual, const void* gamma, const void* beta,
+                                 void* z, void* x_out, void* mu, void* rsigma, int64_t rows,
+                                 int64_t cols, float eps, int is_rms_norm, hkStream_t stream);
+
+/* dz: [rows, cols] `itype`; dx_in (optional): upstream gradient of the
+ * pre-norm sum (`rtype`), added to dx; x: [rows, cols] `rtype`; dx0: [rows,
+ * cols] `itype`; dresidual (optional): `rtype`; dgamma, dbeta: [cols] `wtype`
+ * (dbeta may be NULL).  (ln_bwd_kernels.cuh:126-221, finalize :301-442) */
+HK_API int hk_dropout_add_ln_bwd(int itype, int rtype, int wtype, const void* dz,
+                                 const void* dx_in, const void* x, const void* mu,
+                                 const void* rsigma, const void* gamma, void* dx0,
+                                 void* dresidual, void* dgamma, void* dbeta, int64_t rows,
+                                 int64_t cols, int is_rms_norm, void* workspace,
+                                 size_t workspace_bytes, hkStream_t stream);
+
+/* ======================================================================== *
+ * Softmax along one dimension of a dense array viewed as [outer, dim, inner].
+ * Replaces SoftmaxCuda (hetu/impl/kernel/Softmax.cu:250-310) and
+ * SoftmaxGradientCuda (Softmax.cu:364-404): dx = dy*y - y*sum(dy*y).
+ * ======================================================================== */
+HK_API int hk_softmax_fwd(int dtype, const void* x, void* y, int64_t outer, int64_t dim,
+                          int64_t inner, hkStream_t stream);
+HK_API int hk_softmax_bwd(int dtype, const void* y, const void* dy, void* dx, int64_t outer,
+                          int64_t dim, int64_t inner, hkStream_t stream);
+
+/* ======================================================================== *
+ * Fused softmax cross-entropy, sparse int64 labels.
+ * logits: [rows, cols]; labels: [rows] int64; loss: [rows] `dtype`.
+ *   loss[r] = (labels[r] == ignored_index) ? 0 : logsumexp(x[r,:]) - x[r, labels[r]]
+ * Replaces SoftmaxCrossEntropySparseCuda
+ * (hetu/impl/kernel/SoftmaxCrossEntropySparse.cu:239-274).
+ * ======================================================================== */
+HK_API int hk_sce_sparse_fwd(int dtype, const void* logits, const int64_t* labels, void* loss,
+                             int64_t rows, int64_t cols, int64_t ignored_index,
+                             hkStream_t stream);
+/* dlogits[r, c] = (softmax(x[r,:])[c] - [c == labels[r]]) * grad_loss[r]; rows
+ * whose label equals ignored_index are written as zeros, as the CPU twin and
+ * softmax_cross_entropy_sparse_gradient_kernel do
+ * (SoftmaxCrossEntropySparse.cc:49-55, .cu:93-140).
+ * Replaces SoftmaxCrossEntropySparseGradientCuda (.cu:276-318). */
+HK_API int hk_sce_sparse_bwd(int dtype, const void* logits, const int64_t* labels,
+                             const void* grad_loss, void* dlogits, int64_t rows, int64_t cols,
+                             int64_t ignored_index, hkStream_t stream);
+
+/* Dense (soft / one-hot) labels of the logits' shape:
+ *   loss[r] = -sum_c labels[r,c] * log_softmax(x[r,:])[c]
+ *   dlogits = (softmax(x) - labels) * grad_loss[r]
+ * Replaces SoftmaxCrossEntropyCuda / SoftmaxCrossEntropyGradientCuda
+ * (hetu/impl/kernel/SoftmaxCrossEntropy.cu:13-73, 91-171). */
+HK_API int hk_sce_dense_fwd(int dtype, const void* logits, const void* labels, void* loss,
+                            int64_t rows, int64_t cols, hkStream_t stream);
+HK_API int hk_sce_dense_bwd(int dtype, const void* logits, const void* labels,
+                            const void* grad_loss, void* dlogits, int64_t rows, int64_t cols,
+                            hkStream_t stream);
+
+/* ======================================================================== *
+ * Reduce sum / mean over a set of axes of a (possibly strided) array.
+ * shape / strides (in elements) describe the input; axes must already be
+ * wrapped to [0, ndim), may be unsorted or repeated (sorted + de-duplicated
+ * inside, hetu/impl/kernel/Reduce.cuh:765-768).  The output is written dense,
+ * kept dims in their original order.  bf16 / fp16 accumulate in fp32; mean is
+ * sum * (1.0f / reduce_num) (hetu/impl/kernel/ReduceMean.cu:9-33).
+ * out_dtype may be HK_FLOAT32 for bf16 / fp16 input (ReduceSum.cu:28-37).
+ * Replaces ReduceSumCuda / ReduceMeanCuda (ReduceSum.cu:25-42,
+ * ReduceMean.cu:35-55) and launch_reduce_kernel (Reduce.cuh:757-844).
+ * ======================================================================== */
+HK_API int hk_reduce_workspace_bytes(int in_dtype, int ndim, const int64_t* shape,
+                                     const int64_t* strides, int naxes, const int64_t* axes,
+                                     size_t* bytes);
+HK_API int hk_reduce(int in_dtype, int out_dtype, const void* in, void* out, int ndim,
+                     const int64_t* shape, const int64_t* strides, int naxes,
+                     const int64_t* axes, int op, void* workspace, size_t workspace_bytes,
+                     hkStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* HK_ROWWISE_H_ */

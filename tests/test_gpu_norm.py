@@ -1,0 +1,248 @@
+"""GPU parity of LayerNorm / RMSNorm forward and backward against the oracle,
+through the C-ABI (hk_layer_norm_*, hk_dropout_add_ln_*)."""
+import numpy as np
+import pytest
+
+import helpers
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(7, 64), (33, 256), (5, 1000), (64, 4096), (16, 5120), (3, 8192), (9, 1024 + 8),
+          (4, 7), (2, 20000), (1, 40000)]
+
+
+def _inputs(rows, cols, dtype, seed):
+    x = helpers.draw(seed, (rows, cols), dtype=dtype)
+    gamma = helpers.draw(seed + 1, (cols,), "uniform", 0.5, 1.5, dtype)
+    beta = helpers.draw(seed + 2, (cols,), "normal", 0.0, 0.1, dtype)
+    dy = helpers.draw(seed + 3, (rows, cols), dtype=dtype)
+    return x, gamma, beta, dy
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("kind", ["var", "rstd"])
+def test_layer_norm_fwd(hk, cuda, dtype, shape, kind):
+    import torch
+    rows, cols = shape
+    eps = 1e-5
+    x, gamma, beta, _ = _inputs(rows, cols, dtype, 1000 + cols)
+    ey, emean, evar, erstd = oracle.layernorm_fwd(x, gamma, beta, eps)
+    tx, tg, tb = (helpers.to_torch(v, dtype, cuda) for v in (x, gamma, beta))
+    ty = torch.empty_like(tx)
+    # LayerNormCuda keeps (mean, var) in the data dtype; FusedLayerNormCuda (mean, rstd) in fp32
+    sdt = tx.dtype if kind == "var" else torch.float32
+    tmean = torch.empty(rows, dtype=sdt, device=cuda)
+    tstat = torch.empty(rows, dtype=sdt, device=cuda)
+    hk.layer_norm_fwd(tx, tg, tb, ty, tmean, tstat, eps, stat_kind=0 if kind == "var" else 1)
+    torch.cuda.synchronize()
+    helpers.assert_close(ty, ey, dtype, "y")
+    sdtype = dtype if kind == "var" else "fp32"
+    helpers.assert_close(tmean, emean, sdtype, "mean", scale=float(np.sqrt(np.mean(x.astype(np.float64) ** 2))))
+    helpers.assert_close(tstat, evar if kind == "var" else erstd, sdtype, kind)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_layer_norm_bwd(hk, cuda, dtype, shape):
+    import torch
+    rows, cols = shape
+    eps = 1e-5
+    x, gamma, beta, dy = _inputs(rows, cols, dtype, 2000 + cols)
+    _, mean, _, rstd = oracle.layernorm_fwd(x, gamma, beta, eps)
+    mean32, rstd32 = mean.astype(np.float32), rstd.astype(np.float32)
+    edx, edg, edb = oracle.layernorm_bwd(dy, x, gamma, mean32, rstd32, eps, clamp_gamma=True)
+    tx, tg, tb, tdy = (helpers.to_torch(v, dtype, cuda) for v in (x, gamma, beta, dy))
+    tmean = helpers.to_torch(mean32, "fp32", cuda)
+    trstd = helpers.to_torch(rstd32, "fp32", cuda)
+    tdx = torch.empty_like(tx)
+    tdg = torch.empty_like(tg)
+    tdb = torch.empty_like(tg)
+    hk.layer_norm_bwd(tdy, tx, tg, tb, tmean, trstd, tdx, tdg, tdb, eps, stat_kind=1, clamp_gamma=True)
+    torch.cuda.synchronize()
+    helpers.assert_close(tdx, edx, dtype, "dx")
+    helpers.assert_close(tdg, edg, dtype, "dgamma")
+    helpers.assert_close(tdb, edb, dtype, "dbeta")
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("shape", [(33, 256), (16, 5120), (4, 7)])
+def test_layer_norm_bwd_from_var(hk, cuda, dtype, shape):
+    """LayerNormGradientCuda's form: statistics are (mean, var) in the data dtype."""
+    import torch
+    rows, cols = shape
+    eps = 1e-5
+    x, gamma, beta, dy = _inputs(rows, cols, dtype, 2500 + cols)
+    _, mean, var, _ = oracle.layernorm_fwd(x, gamma, beta, eps)
+    mean_s, var_s = oracle.round_to(mean, dtype), oracle.round_to(var, dtype)
+    rstd = 1.0 / np.sqrt(var_s.astype(np.float64) + eps)
+    edx, edg, edb = oracle.layernorm_bwd(dy, x, gamma, mean_s, rstd, eps, clamp_gamma=False)
+    tx, tg, tb, tdy = (helpers.to_torch(v, dtype, cuda) for v in (x, gamma, beta, dy))
+    tmean, tvar = helpers.to_torch(mean_s, dtype, cuda), helpers.to_torch(var_s, dtype, cuda)
+    tdx, tdg, tdb = torch.empty_like(tx), torch.empty_like(tg), torch.empty_like(tg)
+    hk.layer_norm_bwd(tdy, tx, tg, tb, tmean, tvar, tdx, tdg, tdb, eps, stat_kind=0, clamp_gamma=False)
+    torch.cuda.synchronize()
+    helpers.assert_close(tdx, edx, dtype, "dx")
+    helpers.assert_close(tdg, edg, dtype, "dgamma")
+    helpers.assert_close(tdb, edb, dtype, "dbeta")
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("shape", [(33, 256), (16, 5120), (5, 1000), (4, 7)])
+def test_layer_norm_bwd_memory_efficient(hk, cuda, dtype, shape):
+    """FusedLayerNormGradient with inplace=true: x_hat is rebuilt from the forward output."""
+    import torch
+    rows, cols = shape
+    eps = 1e-5
+    x, gamma, beta, dy = _inputs(rows, cols, dtype, 2700 + cols)
+    # a few tiny gammas exercise clamp_by_magnitude
+    gamma[:3] = oracle.round_to(np.array([1e-7, -1e-7, 0.0], dtype=np.float32), dtype)
+    y64, _, _, rstd = oracle.layernorm_fwd(x, gamma, beta, eps)
+    y = oracle.round_to(y64, dtype)
+    rstd32 = rstd.astype(np.float32)
+    edx, edg, edb = oracle.layernorm_bwd_memeff(dy, y, gamma, beta, rstd32, eps)
+    ty, tg, tb, tdy = (helpers.to_torch(v, dtype, cuda) for v in (y, gamma, beta, dy))
+    trstd = helpers.to_torch(rstd32, "fp32", cuda)
+    tdx, tdg, tdb = torch.empty_like(ty), torch.empty_like(tg), torch.empty_like(tg)
+    hk.layer_norm_bwd(tdy, ty, tg, tb, None, trstd, tdx, tdg, tdb, eps, stat_kind=1, memory_efficient=True)
+    torch.cuda.synchronize()
+    helpers.assert_close(tdx, edx, dtype, "dx")
+    helpers.assert_close(tdg, edg, dtype, "dgamma")
+    helpers.assert_close(tdb, edb, dtype, "dbeta")
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(7, 64), (40, 4096), (16, 5120), (3, 8192), (5, 1000), (4, 7)])
+@pytest.mark.parametrize("is_rms", [True, False])
+@pytest.mark.parametrize("residual", [False, True])
+def test_dropout_add_ln(hk, cuda, dtype, shape, is_rms, residual):
+    import torch
+    rows, cols = shape
+    eps = 1e-6
+    x0, gamma, beta, dz = _inputs(rows, cols, dtype, 3000 + cols)
+    if is_rms:
+        gamma = helpers.draw(77, (cols,), "uniform", 0.8, 1.2, dtype)
+    res = helpers.draw(3100 + cols, (rows, cols), dtype=dtype) if residual else None
+    ez, exo, emu, ers = oracle.dropout_add_ln_fwd(x0, res, gamma, None if is_rms else beta, eps, is_rms)
+    tx0, tg, tb, tdz = (helpers.to_torch(v, dtype, cuda) for v in (x0, gamma, beta, dz))
+    tres = helpers.to_torch(res, dtype, cuda) if residual else None
+    tz = torch.empty_like(tx0)
+    txo = torch.empty_like(tx0) if residual else None
+    tmu = torch.empty(rows, dtype=torch.float32, device=cuda)
+    trs = torch.empty(rows, dtype=torch.float32, device=cuda)
+    hk.dropout_add_ln_fwd(tx0, tres, tg, None if is_rms else tb, tz, txo, tmu, trs, eps, is_rms)
+    torch.cuda.synchronize()
+    helpers.assert_close(tz, ez, dtype, "z")
+    helpers.assert_close(trs, ers, "fp32", "rsigma")
+    helpers.assert_close(tmu, emu, "fp32", "mu", scale=1.0)
+    if residual:
+        helpers.assert_close(txo, exo, dtype, "x")
+
+    # backward on the saved x (rounded to the storage dtype) and the saved statistics
+    x = oracle.round_to(exo, dtype) if residual else x0
+    mu32, rs32 = helpers.to_numpy(tmu), helpers.to_numpy(trs)
+    dxin = helpers.draw(3200 + cols, (rows, cols), dtype=dtype) if residual else None
+    edx, edg, edb = oracle.dropout_add_ln_bwd(dz, dxin, x, mu32, rs32, gamma, is_rms)
+    tx = helpers.to_torch(x, dtype, cuda)
+    tdxin = helpers.to_torch(dxin, dtype, cuda) if residual else None
+    tdx0 = torch.empty_like(tx)
+    tdres = torch.empty_like(tx) if residual else None
+    tdg, tdb = torch.empty_like(tg), torch.empty_like(tg)
+    hk.dropout_add_ln_bwd(tdz, tdxin, tx, tmu, trs, tg, tdx0, tdres, tdg, tdb, is_rms)
+    torch.cuda.synchronize()
+    helpers.assert_close(tdx0, edx, dtype, "dx0")
+    if residual:
+        assert torch.equal(tdres, tdx0)
+    helpers.assert_close(tdg, edg, dtype, "dgamma")
+    helpers.assert_close(tdb, edb, dtype, "dbeta")
+
+
+def test_rmsnorm_bwd_identity(hk, cuda):
+    """sum_cols dx*x = eps * rs^3 * sum_cols (gamma*dz)*x per row: pins where eps sits."""
+    import torch
+    rows, cols, eps = 64, 4096, 1e-2
+    x, gamma, _, dz = _inputs(rows, cols, "fp32", 4242)
+    tx, tg, tdz = (helpers.to_torch(v, "fp32", cuda) for v in (x, gamma, dz))
+    tz, tmu, trs = torch.empty_like(tx), torch.empty(rows, device=cuda), torch.empty(rows, device=cuda)
+    hk.dropout_add_ln_fwd(tx, None, tg, None, tz, None, tmu, trs, eps, True)
+    tdx, tdg, tdb = torch.empty_like(tx), torch.empty_like(tg), torch.empty_like(tg)
+    hk.dropout_add_ln_bwd(tdz, None, tx, tmu, trs, tg, tdx, None, tdg, tdb, True)
+    torch.cuda.synchronize()
+    lhs = (tdx.double() * tx.double()).sum(1).cpu().numpy()
+    rhs = eps * trs.double().cpu().numpy() ** 3 * (gamma.astype(np.float64) * dz * x).sum(1)
+    assert np.max(np.abs(lhs - rhs)) <= 1e-4 * (np.abs(rhs).max() + 1.0)
+
+
+def test_constant_rows_and_empty(hk, cuda):
+    import torch
+    rows, cols = 8, 512
+    x = np.full((rows, cols), 3.25, dtype=np.float32)
+    gamma = helpers.draw(1, (cols,), "uniform", 0.5, 1.5)
+    beta = helpers.draw(2, (cols,), "normal", 0.0, 0.1)
+    tx, tg, tb = (helpers.to_torch(v, "fp32", cuda) for v in (x, gamma, beta))
+    ty = torch.empty_like(tx)
+    tmean, tvar = torch.empty(rows, device=cuda), torch.empty(rows, device=cuda)
+    hk.layer_norm_fwd(tx, tg, tb, ty, tmean, tvar, 1e-5, stat_kind=0)
+    torch.cuda.synchronize()
+    assert torch.all(tvar == 0)                      # variance never goes negative
+    assert torch.all(tmean == 3.25)
+    assert torch.equal(ty, tb.expand(rows, cols))   # y == beta
+    # empty input: returns without touching anything
+    e = torch.empty((0, cols), device=cuda)
+    hk.layer_norm_fwd(e, tg, tb, e, tmean[:0], tvar[:0], 1e-5)
+    torch.cuda.synchronize()
+
+
+def test_unsupported_and_bad_arguments(hk, cuda):
+    import torch
+    t = torch.zeros((4, 64), dtype=torch.int32, device=cuda)
+    s = torch.zeros(4, dtype=torch.float32, device=cuda)
+    with pytest.raises(hk.HkError) as e:
+        hk.layer_norm_fwd(t, None, None, t, s, s, 1e-5)
+    assert e.value.code == -2        # HK_ERR_UNSUPPORTED, the HT_NOT_IMPLEMENTED of the dtype switch
+    x = torch.zeros((4, 4096), dtype=torch.bfloat16, device=cuda)
+    g = torch.ones(4096, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(hk.HkError) as e:
+        hk.layer_norm_bwd(x, x, g, g, s, s, x, g, g, 1e-5, workspace=torch.zeros(4, device=cuda))
+    assert e.value.code == -4        # HK_ERR_WORKSPACE
+
+
+@pytest.mark.parametrize("cfg", ["C1", "C4", "C5"])
+def test_full_size_configs(hk, cuda, cfg):
+    """The benchmark shapes: GPU on the whole tensor, oracle on a sample of rows
+    (rows are independent) plus float64 column sums for the weight gradients."""
+    import torch
+    if cfg == "C1":
+        rows, cols, dtype, eps, is_rms = 8192, 4096, "fp32", 1e-5, False
+    elif cfg == "C4":
+        rows, cols, dtype, eps, is_rms = 32768, 4096, "bf16", 1e-6, True
+    else:
+        rows, cols, dtype, eps, is_rms = 16384, 5120, "bf16", 1e-5, False
+    x = helpers.draw(402, (rows, cols), dtype=dtype)
+    gamma = helpers.draw(403, (cols,), "uniform", 0.8 if is_rms else 0.5, 1.2 if is_rms else 1.5, dtype)
+    beta = helpers.draw(513, (cols,), "normal", 0.0, 0.1, dtype)
+    dz = helpers.draw(404, (rows, cols), dtype=dtype)
+    tx, tg, tb, tdz = (helpers.to_torch(v, dtype, cuda) for v in (x, gamma, beta, dz))
+    tz = torch.empty_like(tx)
+    tmu, trs = torch.empty(rows, device=cuda), torch.empty(rows, device=cuda)
+    hk.dropout_add_ln_fwd(tx, None, tg, None if is_rms else tb, tz, None, tmu, trs, eps, is_rms)
+    tdx, tdg, tdb = torch.empty_like(tx), torch.empty_like(tg), torch.empty_like(tg)
+    hk.dropout_add_ln_bwd(tdz, None, tx, tmu, trs, tg, tdx, None, tdg, tdb, is_rms)
+    torch.cuda.synchronize()
+    sel = np.sort(helpers.rng(5).choice(rows, 48, replace=False))
+    ez, _, emu, ers = oracle.dropout_add_ln_fwd(x[sel], None, gamma, None if is_rms else beta, eps, is_rms)
+    helpers.assert_close(tz[sel], ez, dtype, "z")
+    helpers.assert_close(trs[sel], ers, "fp32", "rsigma")
+    mu32, rs32 = helpers.to_numpy(tmu), helpers.to_numpy(trs)
+    edx, _, _ = oracle.dropout_add_ln_bwd(dz[sel], None, x[sel], mu32[sel], rs32[sel], gamma, is_rms)
+    helpers.assert_close(tdx[sel], edx, dtype, "dx")
+    # weight gradients over all rows in float64
+    xd, dzd = x.astype(np.float64), dz.astype(np.float64)
+    yhat = (xd - (0.0 if is_rms else mu32.astype(np.float64)[:, None])) * rs32.astype(np.float64)[:, None]
+    helpers.assert_close(tdg, (dzd * yhat).sum(0), dtype, "dgamma")
+    helpers.assert_close(tdb, dzd.sum(0), dtype, "dbeta")
+    # per-row invariant of LayerNorm: sum_cols dx == 0 (up to rounding of the stored dx)
+    if not is_rms:
+        rowsum = tdx.float().sum(1).abs().max().item()
+        assert rowsum <= 1e-2 * cols ** 0.5

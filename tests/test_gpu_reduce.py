@@ -1,0 +1,105 @@
+"""GPU parity of Reduce sum / mean over arbitrary axes (hk_reduce)."""
+import itertools
+
+import numpy as np
+import pytest
+
+import helpers
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(hk, cuda, tx, axes, op, out_dtype=None):
+    import torch
+    red = sorted(set(axes))
+    out_shape = [s for d, s in enumerate(tx.shape) if d not in red] or [1]
+    out = torch.full(out_shape, -7, dtype=out_dtype or tx.dtype, device=cuda)
+    hk.reduce(tx, out, list(axes), op)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_every_axis_subset_is_exact(hk, cuda, dtype):
+    """Small integers make every fp32 partial sum exact: results are known bit for bit,
+    whatever order the kernels add in.  Covers the dimension-merging rule."""
+    shape = (3, 4, 5, 6)
+    x = helpers.rng(7).integers(-3, 4, size=shape).astype(np.float32)
+    tx = helpers.to_torch(x, dtype, cuda)
+    for k in range(1, 5):
+        for axes in itertools.combinations(range(4), k):
+            want = x.astype(np.float64).sum(axis=axes)
+            got = _run(hk, cuda, tx, axes, "sum")
+            assert np.array_equal(helpers.to_numpy(got).astype(np.float64).reshape(want.shape or (1,)),
+                                  want.reshape(want.shape or (1,))), axes
+    # unsorted and repeated axes are sorted and de-duplicated
+    got = _run(hk, cuda, tx, [2, 0, 2], "sum")
+    assert np.array_equal(helpers.to_numpy(got), x.sum(axis=(0, 2)))
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("shape,axes", [((512, 4096), (0,)), ((512, 4096), (1,)), ((8, 64, 4096), (0, 1)),
+                                        ((6, 300, 520), (1,)), ((5, 1000), (1,)), ((1000, 5), (0,)),
+                                        ((3, 100000), (1,)), ((70000,), (0,)), ((4, 33, 7), (0, 2)),
+                                        ((33, 264), (0,)), ((2, 2, 1 << 20), (2,))])
+@pytest.mark.parametrize("op", ["sum", "mean"])
+def test_reduce_parity(hk, cuda, dtype, shape, axes, op):
+    x = helpers.draw(301, shape, dtype=dtype)
+    want = oracle.reduce(x, list(axes), op)
+    tx = helpers.to_torch(x, dtype, cuda)
+    got = _run(hk, cuda, tx, axes, op)
+    n = int(np.prod([shape[a] for a in axes]))
+    helpers.assert_close(got, want, dtype, "%s %s" % (op, axes), scale=float(np.sqrt(n)) / (n if op == "mean" else 1))
+
+
+def test_mean_rounding_order(hk, cuda):
+    """mean = fp32 sum * float(1/n): integer inputs make the sum exact, so the result is known bit for bit."""
+    x = helpers.rng(11).integers(-8, 9, size=(64, 3000)).astype(np.float32)
+    tx = helpers.to_torch(x, "fp32", cuda)
+    got = helpers.to_numpy(_run(hk, cuda, tx, (1,), "mean"))
+    want = oracle.reduce(x, [1], "mean", mean_mode=1).astype(np.float32)
+    assert np.array_equal(got, want)
+
+
+def test_strided_views_and_fp32_output(hk, cuda):
+    import torch
+    x = helpers.draw(302, (16, 24, 40), dtype="bf16")
+    tx = helpers.to_torch(x, "bf16", cuda)
+    for view, nview in ((tx.permute(2, 0, 1), x.transpose(2, 0, 1)), (tx[:, ::2, 3:35], x[:, ::2, 3:35]),
+                        (tx.transpose(0, 1), x.transpose(1, 0, 2))):
+        for axes in ((0,), (1,), (2,), (0, 2), (0, 1, 2)):
+            want = oracle.reduce(np.ascontiguousarray(nview), list(axes), "sum")
+            got = _run(hk, cuda, view, axes, "sum", out_dtype=torch.float32)
+            helpers.assert_close(got, want, "fp32", "strided %s" % (axes,), scale=float(np.abs(want).max()), rtol=1e-5)
+
+
+@pytest.mark.parametrize("tdt", ["int64", "int32", "fp64", "uint8"])
+def test_integer_and_double(hk, cuda, tdt):
+    import torch
+    x = helpers.rng(5).integers(0, 5, size=(17, 33, 9))
+    tx = torch.from_numpy(x).to(hk.torch_dtype(tdt)).to(cuda)
+    for axes in ((0,), (1, 2), (0, 1, 2), (2,)):
+        got = _run(hk, cuda, tx, axes, "sum")
+        want = x.sum(axis=axes)
+        if tdt == "uint8":
+            want = want % 256
+        assert np.array_equal(got.cpu().numpy().astype(np.int64).reshape(-1), np.asarray(want).reshape(-1))
+
+
+def test_full_size_configs(hk, cuda):
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(301)
+    tx = torch.randn((32768, 4096), generator=g, dtype=torch.float32).to(torch.bfloat16).to(cuda)
+    xd = tx.double()
+    for axes, op in (((0,), "sum"), ((0,), "mean"), ((1,), "sum"), ((1,), "mean")):
+        want = (xd.sum(axes[0]) if op == "sum" else xd.mean(axes[0])).cpu().numpy()
+        got = _run(hk, cuda, tx, axes, op)
+        n = tx.shape[axes[0]]
+        helpers.assert_close(got, want, "bf16", "%s %s" % (op, axes), scale=float(np.sqrt(n)) / (n if op == "mean" else 1))
+    t3 = tx.view(64, 512, 4096)
+    got = _run(hk, cuda, t3, (0, 1), "sum")
+    helpers.assert_close(got, xd.sum(0).cpu().numpy(), "bf16", "sum (0,1)", scale=float(np.sqrt(32768)))
+    # linearity: sum(2x) == 2 sum(x) exactly in bf16 (scaling by two is exact)
+    got2 = _run(hk, cuda, (tx * 2), (0,), "sum")
+    assert torch.equal(got2.float(), _run(hk, cuda, tx, (0,), "sum").float() * 2)

@@ -29,6 +29,23 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 struct bf16 { uint16_t bits; };
 struct fp16 { uint16_t bits; };
 
+// Index of the calling wavefront inside its workgroup as a scalar: everything
+// derived from it (row number, row pointers) then lives in SGPRs and row loads
+// use one scalar base plus a per-lane offset.
+__device__ __forceinline__ int wave_index() {
+  return __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6));
+}
+
+// Makes the compiler forget what it knows about a packed vector without
+// emitting an instruction.  Used between two passes over the same registers so
+// that the second pass re-derives its fp32 values from the packed data instead
+// of keeping every unpacked intermediate of the first pass alive.
+__device__ __forceinline__ void launder(uint32_t __attribute__((ext_vector_type(4))) & v) {
+  uint32_t a = v.x, b = v.y, c = v.z, d = v.w;
+  asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+  v.x = a; v.y = b; v.z = c; v.w = d;
+}
+
 __device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
 
@@ -121,7 +138,13 @@ template <> struct VecIO<fp16> {
   }
 };
 
+// Row data is read exactly once: non-temporal loads keep it from displacing
+// reusable lines and stream measurably faster.  Small reused vectors (gamma,
+// beta) go through ld16_keep.
 __device__ __forceinline__ u32x4 ld16(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+__device__ __forceinline__ u32x4 ld16_keep(const void* p) {
   return *reinterpret_cast<const u32x4*>(p);
 }
 __device__ __forceinline__ void st16(void* p, const u32x4& v) {
@@ -344,6 +367,7 @@ enum TuneKey {
   TUNE_REDUCE_OUTER_ROW_BLOCKS,
   TUNE_STREAM_STORES,
   TUNE_NORM_BWD_ROWS_PER_BLOCK,
+  TUNE_NORM_BWD_PREFETCH,
   TUNE_NUM_KEYS
 };
 int tune_get(int key);

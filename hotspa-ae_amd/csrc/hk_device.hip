@@ -52,6 +52,7 @@ static const char* const kTuneNames[] = {
   "reduce_outer_row_blocks",
   "stream_stores",      // 1: non-temporal stores for write-once outputs, 2: plain stores
   "norm_bwd_rows_per_block",
+  "norm_bwd_prefetch",  // rows loaded ahead by the backward kernel (1..3)
 };
 constexpr int kNumTune = sizeof(kTuneNames) / sizeof(kTuneNames[0]);
 static_assert(kNumTune == TUNE_NUM_KEYS, "tune name table out of sync with TuneKey");
@@ -313,8 +314,10 @@ int hk_copy_kernel(void* dst, const void* src, size_t bytes, hkStream_t stream) 
   size_t nvec = bytes / 16;
   size_t blocks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
   HK_REQUIRE(blocks <= 0x7fffffffu, HK_ERR_INVALID, "hk_copy_kernel: size too large");
+  profile_before(as_hip(stream));
   hipLaunchKernelGGL(copy16_kernel<UNROLL>, dim3(unsigned(blocks)), dim3(256), 0, as_hip(stream),
                      static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), nvec);
+  profile_after(as_hip(stream));
   return launch_check("copy16_kernel");
 }
 

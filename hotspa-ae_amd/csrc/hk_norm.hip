@@ -12,6 +12,7 @@
 #include "hk_common.cuh"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace hk {
 
@@ -63,7 +64,7 @@ void norm_fwd_kernel(NormFwdArgs a) {
   const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
   const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
   const int64_t row = WAVE_ROW
-      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)
+      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index()
       : int64_t(blockIdx.x);
   if (WAVE_ROW && row >= a.rows) return;  // wave-uniform; no block barrier in this mode
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
@@ -172,12 +173,12 @@ void norm_fwd_kernel(NormFwdArgs a) {
     if (v < a.nvec) {
       float f[VEC], g[VEC], b[VEC];
       get(i, f);
-      if (gp) VecIO<T>::unpack(ld16(gp + v * VEC), g);
+      if (gp) VecIO<T>::unpack(ld16_keep(gp + v * VEC), g);
       else {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) g[j] = 1.f;
       }
-      if (bp) VecIO<T>::unpack(ld16(bp + v * VEC), b);
+      if (bp) VecIO<T>::unpack(ld16_keep(bp + v * VEC), b);
       else {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) b[j] = 0.f;
@@ -312,13 +313,23 @@ static bool pick_row_shape(int nvec, int forced_threads, int max_nv, int wave_ro
     return true;
   }
   // short rows: one wavefront per row
-  if (nvec <= 64 * wave_row_max_nv) {
+  if (nvec <= 64 * wave_row_max_nv && nvec <= 256) {
     *threads = 64;
     *nv = pow2_ceil((nvec + 63) / 64);
     return true;
   }
+  // medium rows (measured on MI355X: 4096 / 5120 bf16 columns, 4096 fp32
+  // columns): small workgroups of 128..256 threads per row stream fastest
+  for (int n = 2; n <= max_nv; n <<= 1) {
+    int t = ((nvec + n - 1) / n + 63) / 64 * 64;
+    if (t <= 256) {
+      *threads = t;
+      *nv = n;
+      return true;
+    }
+  }
   // long rows: one workgroup per row, smallest power-of-two vector count that
-  // keeps the block within 1024 threads, starting from 4 vectors per thread
+  // keeps the block within 1024 threads
   for (int n = 4; n <= max_nv; n <<= 1) {
     int t = ((nvec + n - 1) / n + 63) / 64 * 64;
     if (t <= 1024) {
@@ -413,36 +424,43 @@ __device__ __forceinline__ float clamp_by_magnitude(float g, float eps) {
   return g > -eps ? -eps : g;
 }
 
-template <typename T, int NV, int MODE>
-__global__ __launch_bounds__(1024)
+// Column-owner backward kernel.  A group of `tpr` threads walks rows; thread t
+// owns the same columns in every row, so its dgamma / dbeta sums stay in
+// registers.  With xc = x - mu (x for RMSNorm), t = dy * gamma and
+// m2 = mean(t * xc):   dx = rs * t - rs * mean(t) - xc * rs^3 * m2,
+// two fused multiply-adds per element once the row sums are known.
+template <typename T, int NV, int MODE, int PF>
+__global__ __launch_bounds__(NV == 1 ? 1024 : 512)
 void norm_bwd_kernel(NormBwdArgs a) {
   constexpr int VEC = VecIO<T>::N;
   constexpr int NE = NV * VEC;
   extern __shared__ float lds[];           // [rows_per_block, cols] column-sum staging
   __shared__ float red[2][kMaxWaves * 2];  // double-buffered by iteration parity
 
-  const int tpr = a.tpr;
+  const int tpr = a.tpr;                   // multiple of 64: a wavefront never straddles two rows
   const int rpb = int(blockDim.x) / tpr;
-  const int group = int(threadIdx.x) / tpr;
+  const int group = __builtin_amdgcn_readfirstlane(int(threadIdx.x) / tpr);
   const int t = int(threadIdx.x) - group * tpr;
   const int waves_per_group = tpr >> 6;
   const int first_wave = group * waves_per_group;
 
-  const T* gp = static_cast<const T*>(a.gamma);
-  const T* bp = static_cast<const T*>(a.beta);
-  // gamma (and beta) stay packed; a missing gamma is all ones
-  u32x4 gmp[NV];
-  [[maybe_unused]] u32x4 btp[MODE == BWD_LN_MEMEFF ? NV : 1];
+  // gamma (and beta) of this thread's columns as fp32; a missing gamma is all ones
+  float gm[NE];
+  [[maybe_unused]] float bt[MODE == BWD_LN_MEMEFF ? NE : 1];
   {
-    float ones[VEC], zeros[VEC];
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) { ones[j] = 1.f; zeros[j] = 0.f; }
+    const T* gp = static_cast<const T*>(a.gamma);
+    const T* bp = static_cast<const T*>(a.beta);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = i * tpr + t;
-      gmp[i] = (v < a.nvec && gp) ? ld16(gp + v * VEC) : VecIO<T>::pack(ones);
-      if constexpr (MODE == BWD_LN_MEMEFF)
-        btp[i] = (v < a.nvec && bp) ? ld16(bp + v * VEC) : VecIO<T>::pack(zeros);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) gm[i * VEC + j] = 1.f;
+      if (v < a.nvec && gp) VecIO<T>::unpack(ld16_keep(gp + v * VEC), &gm[i * VEC]);
+      if constexpr (MODE == BWD_LN_MEMEFF) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) bt[i * VEC + j] = 0.f;
+        if (v < a.nvec && bp) VecIO<T>::unpack(ld16_keep(bp + v * VEC), &bt[i * VEC]);
+      }
     }
   }
   const bool clamp = a.clamp_gamma != 0 || MODE == BWD_LN_MEMEFF;
@@ -452,92 +470,108 @@ void norm_bwd_kernel(NormBwdArgs a) {
   for (int e = 0; e < NE; ++e) { dg[e] = 0.f; db[e] = 0.f; }
 
   const int64_t stride = int64_t(gridDim.x) * rpb;
-  // rows are kept packed; cx/cdy hold the row being processed, nx/ndy the
-  // prefetched next row of this group
-  u32x4 cx[NV], cdy[NV], nx[NV], ndy[NV];
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    cx[i] = u32x4{0, 0, 0, 0}; cdy[i] = u32x4{0, 0, 0, 0};
-    nx[i] = u32x4{0, 0, 0, 0}; ndy[i] = u32x4{0, 0, 0, 0};
-  }
+  // nx / ndy: the next PF rows of this group, packed, oldest first
+  u32x4 nx[PF][NV], ndy[PF][NV];
   int64_t row = int64_t(blockIdx.x) * rpb + group;
-  if (row < a.rows) {
-    const T* xr = static_cast<const T*>(a.x) + row * int64_t(a.cols);
-    const T* dyr = static_cast<const T*>(a.dy) + row * int64_t(a.cols);
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int v = i * tpr + t;
-      if (v < a.nvec) { nx[i] = ld16(xr + v * VEC); ndy[i] = ld16(dyr + v * VEC); }
-    }
-  }
-
-  // xhat and the per-element dy*gamma term of one vector
-  auto elem = [&](const u32x4& px, const u32x4& pdy, int i, float mu, float rs, float* xhat,
-                  float* dyv, float* yb, float* gm) {
-    float xv[VEC];
-    VecIO<T>::unpack(px, xv);
-    VecIO<T>::unpack(pdy, dyv);
-    VecIO<T>::unpack(gmp[i], gm);
-    [[maybe_unused]] float bt[VEC];
-    if constexpr (MODE == BWD_LN_MEMEFF) VecIO<T>::unpack(btp[i], bt);
+  for (int d = 0; d < PF; ++d) {
+    const int64_t r = row + d * stride;
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      if constexpr (MODE == BWD_LN_MEMEFF) {
-        yb[j] = xv[j] - bt[j];
-        xhat[j] = yb[j] / clamp_by_magnitude(gm[j], a.eps);
-      } else {
-        xhat[j] = (MODE == BWD_RMS) ? rs * xv[j] : rs * (xv[j] - mu);
+    for (int i = 0; i < NV; ++i) { nx[d][i] = u32x4{0, 0, 0, 0}; ndy[d][i] = u32x4{0, 0, 0, 0}; }
+    if (r < a.rows) {
+      const T* xr = static_cast<const T*>(a.x) + r * int64_t(a.cols);
+      const T* dyr = static_cast<const T*>(a.dy) + r * int64_t(a.cols);
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int v = i * tpr + t;
+        if (v < a.nvec) { nx[d][i] = ld16(xr + v * VEC); ndy[d][i] = ld16(dyr + v * VEC); }
       }
     }
-  };
+  }
 
   int parity = 0;
   for (int64_t base = int64_t(blockIdx.x) * rpb; base < a.rows; base += stride, parity ^= 1) {
     const bool valid = row < a.rows;
-#pragma unroll
-    for (int i = 0; i < NV; ++i) { cx[i] = nx[i]; cdy[i] = ndy[i]; }
+    float xs[NE], ts[NE];                 // xc (x_hat in the memory-efficient mode) and dy * gamma
     float mu = 0.f, rs = 0.f;
-    if (valid) {
-      if (MODE == BWD_LN) mu = load_stat<T>(a.mean, row, a.stats_f32);
-      const float sv = load_stat<T>(a.stat, row, a.stats_f32);
-      rs = a.stat_kind == HK_STAT_VAR ? 1.0f / sqrtf(sv + a.eps) : sv;
-    }
-    // prefetch the next row of this group while this one is reduced
-    const int64_t next = row + stride;
-    if (next < a.rows) {
-      const T* xr = static_cast<const T*>(a.x) + next * int64_t(a.cols);
-      const T* dyr = static_cast<const T*>(a.dy) + next * int64_t(a.cols);
-#pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        const int v = i * tpr + t;
-        if (v < a.nvec) { nx[i] = ld16(xr + v * VEC); ndy[i] = ld16(dyr + v * VEC); }
-      }
-    }
-
     SumTuple<2> s;
     s.v[0] = 0.f; s.v[1] = 0.f;
     if (valid) {
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
-        if (i * tpr + t < a.nvec) {
-          float xhat[VEC], dyv[VEC], yb[VEC], gm[VEC];
-          elem(cx[i], cdy[i], i, mu, rs, xhat, dyv, yb, gm);
+        VecIO<T>::unpack(nx[0][i], &xs[i * VEC]);
+        VecIO<T>::unpack(ndy[0][i], &ts[i * VEC]);
+      }
+      if (MODE == BWD_LN) mu = load_stat<T>(a.mean, row, a.stats_f32);
+      const float sv = load_stat<T>(a.stat, row, a.stats_f32);
+      rs = a.stat_kind == HK_STAT_VAR ? 1.0f / sqrtf(sv + a.eps) : sv;
+    }
+    // rotate the prefetch ring and issue the loads of the row PF steps ahead
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            const int e = i * VEC + j;
-            if constexpr (MODE == BWD_LN_MEMEFF) s.v[1] = fmaf(dyv[j], yb[j], s.v[1]);
-            else s.v[1] = fmaf(dyv[j] * gm[j], xhat[j], s.v[1]);
-            if (MODE != BWD_RMS) s.v[0] = fmaf(dyv[j], gm[j], s.v[0]);
-            dg[e] = fmaf(dyv[j], xhat[j], dg[e]);
-            db[e] += dyv[j];
-          }
+    for (int d = 0; d + 1 < PF; ++d) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) { nx[d][i] = nx[d + 1][i]; ndy[d][i] = ndy[d + 1][i]; }
+    }
+    const int64_t next = row + stride;
+    {
+      const int64_t far = row + int64_t(PF) * stride;
+      if (far < a.rows) {
+        const T* xr = static_cast<const T*>(a.x) + far * int64_t(a.cols);
+        const T* dyr = static_cast<const T*>(a.dy) + far * int64_t(a.cols);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          const int v = i * tpr + t;
+          if (v < a.nvec) { nx[PF - 1][i] = ld16(xr + v * VEC); ndy[PF - 1][i] = ld16(dyr + v * VEC); }
         }
       }
     }
+    if (valid) {
+      // padding vectors hold zeros in ts (dy), so they add nothing anywhere.
+      // q = dy * rs * gamma is both the dx term and, summed, rs * sum(dy * gamma).
+      auto accumulate = [&](auto clamped) {
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+          const float dz = ts[e];
+          if constexpr (MODE == BWD_LN_MEMEFF) {
+            const float yb = xs[e] - bt[e];
+            const float kg = clamp_by_magnitude(gm[e], a.eps);
+            const float xhat = yb / kg;
+            s.v[0] = fmaf(dz, gm[e], s.v[0]);
+            s.v[1] = fmaf(dz, yb, s.v[1]);
+            dg[e] = fmaf(dz, xhat, dg[e]);
+            db[e] += dz;
+            xs[e] = xhat;
+            ts[e] = dz * kg;
+          } else {
+            const float xc = (MODE == BWD_RMS) ? xs[e] : xs[e] - mu;
+            const float dzr = dz * rs;
+            const float q = dzr * gm[e];
+            s.v[1] = fmaf(q, xc, s.v[1]);
+            if (MODE != BWD_RMS) s.v[0] += q;
+            dg[e] = fmaf(dzr, xc, dg[e]);
+            db[e] += dz;
+            xs[e] = xc;
+            // the per-element term of dx uses the clamped gamma when asked to
+            if constexpr (decltype(clamped)::value) ts[e] = dzr * clamp_by_magnitude(gm[e], a.eps);
+            else ts[e] = q;
+          }
+        }
+      };
+      if (clamp) accumulate(std::true_type{});   // uniform
+      else accumulate(std::false_type{});
+    }
     s = group_allreduce_tuple(s, red[parity], first_wave, waves_per_group);
     if (valid) {
-      const float c1 = (MODE == BWD_RMS) ? 0.f : s.v[0] * a.inv_cols;
-      const float c2 = s.v[1] * a.inv_cols;
+      // plain modes: s0 = rs * sum(dy g), s1 = rs * sum(dy g xc);  dx = q - s0/n - xc * rs^2 * s1/n
+      // memory-efficient: s0 = sum(dy g), s1 = sum(dy (y - beta));   dx = rs * (dy kg - s0/n - xhat * s1/n)
+      float rc1, k3;
+      if constexpr (MODE == BWD_LN_MEMEFF) {
+        rc1 = rs * s.v[0] * a.inv_cols;
+        k3 = rs * s.v[1] * a.inv_cols;
+      } else {
+        rc1 = (MODE == BWD_RMS) ? 0.f : s.v[0] * a.inv_cols;
+        k3 = rs * rs * s.v[1] * a.inv_cols;
+      }
       T* dxr = static_cast<T*>(a.dx) + row * int64_t(a.cols);
       T* drr = a.dres ? static_cast<T*>(a.dres) + row * int64_t(a.cols) : nullptr;
       const T* dir = a.dx_in ? static_cast<const T*>(a.dx_in) + row * int64_t(a.cols) : nullptr;
@@ -545,12 +579,12 @@ void norm_bwd_kernel(NormBwdArgs a) {
       for (int i = 0; i < NV; ++i) {
         const int v = i * tpr + t;
         if (v < a.nvec) {
-          float xhat[VEC], dyv[VEC], yb[VEC], gm[VEC], o[VEC];
-          elem(cx[i], cdy[i], i, mu, rs, xhat, dyv, yb, gm);
+          float o[VEC];
 #pragma unroll
           for (int j = 0; j < VEC; ++j) {
-            const float kg = clamp ? clamp_by_magnitude(gm[j], a.eps) : gm[j];
-            o[j] = rs * (fmaf(dyv[j], kg, -c1) - xhat[j] * c2);
+            const float base = (MODE == BWD_LN_MEMEFF) ? fmaf(ts[i * VEC + j], rs, -rc1)
+                                                       : ts[i * VEC + j] - rc1;
+            o[j] = fmaf(-xs[i * VEC + j], k3, base);
           }
           if (dir) {
             float u[VEC];
@@ -605,32 +639,48 @@ void norm_bwd_kernel(NormBwdArgs a) {
 }
 
 // Folds the [nparts, cols] fp32 partial rows into dgamma / dbeta of type T.
-// One workgroup per 64 columns; wave w sums partial rows w, w+16, ...
+// blockIdx.y picks dgamma / dbeta; a block covers 128 columns as 32 float4
+// column groups x 16 row slices, every slice keeps 8 independent loads in
+// flight, slices are folded through LDS.
 template <typename T>
-__global__ __launch_bounds__(1024)
+__global__ __launch_bounds__(512)
 void norm_bwd_finalize_kernel(const float* __restrict__ part_dgamma,
                               const float* __restrict__ part_dbeta, T* dgamma, T* dbeta,
                               int nparts, int cols) {
-  __shared__ float lds[2][kMaxWaves][kWave];
-  const int lane = threadIdx.x & 63;
-  const int w = threadIdx.x >> 6;
-  const int nw = blockDim.x >> 6;
-  const int c = blockIdx.x * kWave + lane;
-  float sg = 0.f, sb = 0.f;
-  if (c < cols) {
-    for (int r = w; r < nparts; r += nw) {
-      if (part_dgamma) sg += part_dgamma[int64_t(r) * cols + c];
-      if (part_dbeta) sb += part_dbeta[int64_t(r) * cols + c];
+  constexpr int U = 8;
+  __shared__ float lds[16][32][4];
+  const float* part = blockIdx.y == 0 ? part_dgamma : part_dbeta;
+  T* out = blockIdx.y == 0 ? dgamma : dbeta;
+  if (part == nullptr || out == nullptr) return;     // uniform over the block
+  const int cg = threadIdx.x & 31, slice = threadIdx.x >> 5;
+  const int c = (blockIdx.x * 32 + cg) * 4;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (c < cols) {                                     // cols is a multiple of 4 on this path
+    int r = slice;
+    for (; r + (U - 1) * 16 < nparts; r += U * 16) {
+      u32x4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = ld16_keep(part + int64_t(r + u * 16) * cols + c);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        acc[0] += u2f(v[u].x); acc[1] += u2f(v[u].y); acc[2] += u2f(v[u].z); acc[3] += u2f(v[u].w);
+      }
+    }
+    for (; r < nparts; r += 16) {
+      const u32x4 v = ld16_keep(part + int64_t(r) * cols + c);
+      acc[0] += u2f(v.x); acc[1] += u2f(v.y); acc[2] += u2f(v.z); acc[3] += u2f(v.w);
     }
   }
-  lds[0][w][lane] = sg;
-  lds[1][w][lane] = sb;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) lds[slice][cg][k] = acc[k];
   __syncthreads();
-  if (w == 0 && c < cols) {
-    float tg = 0.f, tb = 0.f;
-    for (int i = 0; i < nw; ++i) { tg += lds[0][i][lane]; tb += lds[1][i][lane]; }
-    if (dgamma && part_dgamma) Cvt<T>::store(dgamma + c, tg);
-    if (dbeta && part_dbeta) Cvt<T>::store(dbeta + c, tb);
+  if (threadIdx.x < 128) {
+    const int g = threadIdx.x >> 2, k = threadIdx.x & 3;
+    const int oc = (blockIdx.x * 32 + g) * 4 + k;
+    float s = 0.f;
+#pragma unroll
+    for (int sl = 0; sl < 16; ++sl) s += lds[sl][g][k];
+    if (oc < cols) Cvt<T>::store(out + oc, s);
   }
 }
 
@@ -748,6 +798,7 @@ void norm_bwd_generic_cols_kernel(NormBwdArgs a, int mode, T* dgamma, T* dbeta) 
 struct BwdPlan {
   bool reg_path;
   int tpr, nv, rpb, grid;
+  int block;
   size_t lds_bytes;
   size_t ws_bytes;
 };
@@ -759,8 +810,8 @@ static BwdPlan plan_norm_bwd(int64_t rows, int cols, bool aligned) {
   p.reg_path = false;
   if (!aligned || cols % VEC != 0) return p;
   const int nvec = cols / VEC;
-  // the dgamma / dbeta accumulators of a thread must stay in registers: 8
-  // columns per thread by default, 16 when a thread count is forced
+  // column-owner kernel: the dgamma / dbeta accumulators of a thread must stay
+  // in registers: 8 columns per thread by default, 16 when a thread count is forced
   const int max_nv = (tune_get(TUNE_NORM_BWD_THREADS) > 0 ? 16 : 8) / VEC;
   int tpr = tune_get(TUNE_NORM_BWD_THREADS);
   int nv;
@@ -775,18 +826,21 @@ static BwdPlan plan_norm_bwd(int64_t rows, int cols, bool aligned) {
     tpr = ((nvec + nv - 1) / nv + 63) / 64 * 64;
     if (tpr > 1024) return p;
   }
+  // kernels with more than one vector per thread are built for 512-thread blocks
+  const int max_block = nv == 1 ? 1024 : 512;
+  if (tpr > max_block) return p;
   int rpb = tune_get(TUNE_NORM_BWD_ROWS_PER_BLOCK);
-  if (rpb <= 0) rpb = 1024 / tpr;
-  rpb = std::max(1, std::min(rpb, 1024 / tpr));
+  if (rpb <= 0) rpb = std::max(1, max_block / tpr);
+  rpb = std::max(1, std::min(rpb, max_block / tpr));
   // staging buffer of the final fold must fit 64 KiB of LDS
   while (rpb > 1 && size_t(rpb) * cols * sizeof(float) > 65536) --rpb;
   int grid = tune_get(TUNE_NORM_BWD_BLOCKS);
-  if (grid <= 0) grid = device_cu_count();
+  if (grid <= 0) grid = device_cu_count();   // one 1024-thread workgroup per CU measured fastest
   const int64_t max_useful = (rows + rpb - 1) / rpb;
   if (grid > max_useful) grid = int(max_useful);
   if (grid < 1) grid = 1;
   p.reg_path = true;
-  p.tpr = tpr; p.nv = nv; p.rpb = rpb; p.grid = grid;
+  p.tpr = tpr; p.nv = nv; p.rpb = rpb; p.grid = grid; p.block = tpr * rpb;
   p.lds_bytes = rpb > 1 ? size_t(rpb) * cols * sizeof(float) : 0;
   p.ws_bytes = size_t(2) * grid * cols * sizeof(float);
   return p;
@@ -794,21 +848,29 @@ static BwdPlan plan_norm_bwd(int64_t rows, int cols, bool aligned) {
 
 template <typename T, int MODE>
 static int launch_norm_bwd_nv(const NormBwdArgs& a, const BwdPlan& p, hipStream_t s) {
-  dim3 grid{unsigned(p.grid)}, block{unsigned(p.tpr * p.rpb)};
+  dim3 grid{unsigned(p.grid)}, block{unsigned(p.block)};
   profile_before(s);
+  int pf = tune_get(TUNE_NORM_BWD_PREFETCH);
+  if (pf <= 0) pf = 1;   // deeper rings measured slower
+#define HK_BWD_LAUNCH(N, P) hipLaunchKernelGGL((norm_bwd_kernel<T, N, MODE, P>), grid, block, p.lds_bytes, s, a)
+#define HK_BWD_PF(N)                                   \
+  do {                                                 \
+    if (pf == 1) HK_BWD_LAUNCH(N, 1);                  \
+    else if (pf == 2) HK_BWD_LAUNCH(N, 2);             \
+    else HK_BWD_LAUNCH(N, 3);                          \
+  } while (0)
   switch (p.nv) {
-    case 1: hipLaunchKernelGGL((norm_bwd_kernel<T, 1, MODE>), grid, block, p.lds_bytes, s, a); break;
-    case 2: hipLaunchKernelGGL((norm_bwd_kernel<T, 2, MODE>), grid, block, p.lds_bytes, s, a); break;
+    case 1: HK_BWD_PF(1); break;
+    case 2: HK_BWD_PF(2); break;
     case 4:
-      if constexpr (VecIO<T>::N == 4) {
-        hipLaunchKernelGGL((norm_bwd_kernel<T, 4, MODE>), grid, block, p.lds_bytes, s, a);
-        break;
-      }
+      if constexpr (VecIO<T>::N == 4) { HK_BWD_PF(4); break; }
       [[fallthrough]];
     default:
       set_last_error("norm_bwd: no kernel for %d vectors per thread", p.nv);
       return HK_ERR_UNSUPPORTED;
   }
+#undef HK_BWD_PF
+#undef HK_BWD_LAUNCH
   profile_after(s);
   return launch_check("norm_bwd_kernel");
 }
@@ -850,7 +912,7 @@ static int norm_bwd_typed(NormBwdArgs a, int mode, void* dgamma, void* dbeta, vo
     default: rc = launch_norm_bwd_nv<T, BWD_LN_MEMEFF>(a, p, s); break;
   }
   if (rc != HK_OK || !want_cols) return rc;
-  hipLaunchKernelGGL((norm_bwd_finalize_kernel<T>), dim3(unsigned((a.cols + 63) / 64)), dim3(1024), 0, s,
+  hipLaunchKernelGGL((norm_bwd_finalize_kernel<T>), dim3(unsigned((a.cols + 127) / 128), 2), dim3(512), 0, s,
                      a.part_dgamma, a.part_dbeta, static_cast<T*>(dgamma), static_cast<T*>(dbeta),
                      p.grid, a.cols);
   return launch_check("norm_bwd_finalize_kernel");

@@ -85,7 +85,7 @@ void reduce_inner_vec_kernel(InnerArgs a) {
   const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
   const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
   const int64_t row = WAVE_ROW
-      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)
+      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index()
       : int64_t(blockIdx.x);
   if (WAVE_ROW && row >= a.rows) return;
   const int split = blockIdx.y;
@@ -224,11 +224,30 @@ template <typename OUT_T>
 __global__ __launch_bounds__(256)
 void reduce_fold_partials_kernel(const float* part, OUT_T* out, int nparts, int64_t n, float factor,
                                  int is_mean) {
-  const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  float s = 0.f;
-  for (int k = 0; k < nparts; ++k) s += part[int64_t(k) * n + i];
-  st_acc<OUT_T, float>(out + i, project<float>(s, factor, is_mean));
+  // 64 outputs per block; the 4 waves take interleaved partial rows with 8
+  // independent loads in flight each, then fold through LDS
+  constexpr int U = 8;
+  __shared__ float lds[4][kWave];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int64_t i = int64_t(blockIdx.x) * kWave + lane;
+  float acc = 0.f;
+  if (i < n) {
+    int k = w;
+    for (; k + (U - 1) * 4 < nparts; k += U * 4) {
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = part[int64_t(k + u * 4) * n + i];
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc += v[u];
+    }
+    for (; k < nparts; k += 4) acc += part[int64_t(k) * n + i];
+  }
+  lds[w][lane] = acc;
+  __syncthreads();
+  if (w == 0 && i < n) {
+    const float s = (lds[0][lane] + lds[1][lane]) + (lds[2][lane] + lds[3][lane]);
+    st_acc<OUT_T, float>(out + i, project<float>(s, factor, is_mean));
+  }
 }
 
 // outer reduction, scalar path: one thread per output column, any dtype
@@ -370,7 +389,7 @@ static InnerShape shape_inner(const ReducePlan& p, const void* in) {
   s.vec = aligned16(in) && (p.rows == 1 || p.row_stride % VEC == 0);
   const int64_t nvec = p.cols / VEC;
   int tpr = tune_get(TUNE_REDUCE_INNER_THREADS);
-  if (tpr <= 0) tpr = nvec <= 64 * 16 ? 64 : (nvec <= 256 * 16 ? 256 : 1024);
+  if (tpr <= 0) tpr = nvec <= 64 * 32 ? 64 : (nvec <= 256 * 32 ? 256 : 1024);
   tpr = std::min(1024, std::max(64, (tpr + 63) / 64 * 64));
   s.tpr = tpr;
   // few long rows: split columns so that ~4 workgroups per CU exist
@@ -394,14 +413,16 @@ static OuterShape shape_outer(const ReducePlan& p, const void* in) {
   constexpr int VEC = 16 / sizeof(T);
   OuterShape s{};
   s.vec = aligned16(in) && p.C % VEC == 0 && p.r_stride % VEC == 0 && (p.B == 1 || p.b_stride % VEC == 0);
-  const int64_t col_tiles = (p.C / VEC + 63) / 64;
+  s.wy = 1; s.rsplit = 1; s.rows_per_split = p.R;
+  if (!s.vec) return s;
+  const int64_t col_tiles = std::max<int64_t>(1, (p.C / VEC + 63) / 64);
   // waves per block: enough rows per wave to keep 8 loads in flight
   int wy = 16;
   while (wy > 1 && p.R < int64_t(wy) * 8) wy >>= 1;
   s.wy = wy;
   int rsplit = tune_get(TUNE_REDUCE_OUTER_ROW_BLOCKS);
   if (rsplit <= 0) {
-    const int64_t want_blocks = int64_t(device_cu_count()) * 2;
+    const int64_t want_blocks = int64_t(device_cu_count());   // one workgroup per CU measured fastest
     const int64_t have = col_tiles * p.B;
     rsplit = int(std::max<int64_t>(1, (want_blocks + have - 1) / have));
   }
@@ -500,7 +521,7 @@ static int reduce_fast(const ReducePlan& p, const void* in, void* out, float fac
     int rc = launch_check("reduce_outer_vec_kernel");
     if (rc != HK_OK || s.rsplit == 1) return rc;
     const int64_t n = p.B * p.C;
-    hipLaunchKernelGGL((reduce_fold_partials_kernel<OUT_T>), dim3(unsigned((n + 255) / 256)), dim3(256), 0, st,
+    hipLaunchKernelGGL((reduce_fold_partials_kernel<OUT_T>), dim3(unsigned((n + 63) / 64)), dim3(256), 0, st,
                        static_cast<const float*>(ws), static_cast<OUT_T*>(out), s.rsplit, n, factor, is_mean);
     return launch_check("reduce_fold_partials_kernel");
   }

@@ -34,7 +34,7 @@ template <bool WAVE_ROW>
 __device__ __forceinline__ void row_coords(int& tpr, int& t, int64_t& row, int& nwaves) {
   tpr = WAVE_ROW ? kWave : int(blockDim.x);
   t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
-  row = WAVE_ROW ? int64_t(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6) : int64_t(blockIdx.x);
+  row = WAVE_ROW ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index() : int64_t(blockIdx.x);
   nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
 }
 
@@ -374,7 +374,13 @@ static bool pick_sce_shape(int nvec, int max_nv_wave, int max_nv, int* threads, 
     *nv = pow2_ceil_sce((nvec + 63) / 64);
     return true;
   }
-  for (int n = 4; n <= max_nv; n <<= 1) {
+  // long rows, measured at 32000 bf16 columns: the widest vector count the
+  // kernel is built for wins (512 threads x 8 vectors beat 1024 x 4 forward)
+  for (int n = max_nv; n >= 1; n >>= 1) {
+    int t = ((nvec + n - 1) / n + 63) / 64 * 64;
+    if (t <= 1024 && (t >= 256 || n == 1)) { *threads = t; *nv = n; return true; }
+  }
+  for (int n = 1; n <= max_nv; n <<= 1) {
     int t = ((nvec + n - 1) / n + 63) / 64 * 64;
     if (t <= 1024) { *threads = t; *nv = n; return true; }
   }

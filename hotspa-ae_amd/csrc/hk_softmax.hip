@@ -32,7 +32,7 @@ void softmax_fwd_kernel(SoftmaxArgs a) {
   const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
   const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
   const int64_t row = WAVE_ROW
-      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)
+      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index()
       : int64_t(blockIdx.x);
   if (WAVE_ROW && row >= a.rows) return;
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
@@ -93,7 +93,7 @@ void softmax_bwd_kernel(SoftmaxArgs a) {
   const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
   const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
   const int64_t row = WAVE_ROW
-      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)
+      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index()
       : int64_t(blockIdx.x);
   if (WAVE_ROW && row >= a.rows) return;
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
@@ -244,7 +244,7 @@ static inline int pow2_ceil_sm(int v) {
 }
 
 // threads per row / vectors per thread for a row of nvec 16-byte vectors
-static bool pick_softmax_shape(int nvec, int max_nv_wave, int max_nv, int* threads, int* nv) {
+static bool pick_softmax_shape(int nvec, int max_nv_wave, int max_nv, bool bwd, int* threads, int* nv) {
   const int forced = tune_get(TUNE_SOFTMAX_THREADS);
   if (forced > 0) {
     int t = std::min(1024, std::max(64, (forced + 63) / 64 * 64));
@@ -253,12 +253,15 @@ static bool pick_softmax_shape(int nvec, int max_nv_wave, int max_nv, int* threa
     *threads = t; *nv = n;
     return true;
   }
-  if (nvec <= 64 * max_nv_wave) {
+  // measured on MI355X at 2048 bf16 columns: forward is fastest with two
+  // vectors per thread (128 threads per row), backward with one (256 threads)
+  const int want = bwd ? 1 : 2;
+  if (nvec <= 64 * want) {
     *threads = 64;
     *nv = pow2_ceil_sm((nvec + 63) / 64);
-    return true;
+    return *nv <= max_nv_wave;
   }
-  for (int n = 4; n <= max_nv; n <<= 1) {
+  for (int n = want; n <= max_nv; n <<= 1) {
     int t = ((nvec + n - 1) / n + 63) / 64 * 64;
     if (t <= 1024) { *threads = t; *nv = n; return true; }
   }
@@ -300,7 +303,7 @@ static int softmax_lastdim_typed(SoftmaxArgs a, hipStream_t s) {
   const int max_nv = BWD ? 4 : 64 / VEC;
   const int max_nv_wave = BWD ? 4 : std::min(8, 64 / VEC);
   int threads = 0, nv = 0;
-  if (vec_ok && pick_softmax_shape(a.nvec, max_nv_wave, max_nv, &threads, &nv)) {
+  if (vec_ok && pick_softmax_shape(a.nvec, max_nv_wave, max_nv, BWD, &threads, &nv)) {
     if (threads == 64) {
       dim3 grid(unsigned((a.rows + 3) / 4)), block(256);
       return launch_softmax_nv<T, BWD, true>(a, nv, grid, block, s);

@@ -48,3 +48,23 @@ def test_missing_library_fails_loudly(hk, monkeypatch, tmp_path):
         assert "missing" in str(e)
     else:
         raise AssertionError("loading a missing library must raise")
+
+
+def test_planners_survive_odd_shapes(hk):
+    """Host-side launch planning (no kernel is launched): every axis subset of small,
+    odd and degenerate shapes, with dense and permuted strides."""
+    import itertools
+    import numpy as np
+    g = np.random.default_rng(0)
+    for shape in ([3, 4, 5, 6], [1, 7], [6], [2, 1, 3], [0, 5], [5, 0], [33, 264], [1000, 5], [4, 33, 7],
+                  [2, 2, 1 << 20], [70000], [1, 1, 1]):
+        dense = [int(np.prod(shape[i + 1:], dtype=np.int64)) for i in range(len(shape))]
+        for strides in (dense, list(reversed(dense)), [s * 2 for s in dense]):
+            for k in range(0, len(shape) + 1):
+                for axes in itertools.combinations(range(len(shape)), k):
+                    for dt in (6, 8, 4):
+                        assert hk.reduce_workspace_bytes(dt, shape, strides, list(axes)) >= 0
+    for dt in (5, 6, 8):
+        for _ in range(200):
+            rows, cols = int(g.integers(0, 70000)), int(g.integers(0, 70000))
+            assert hk.norm_bwd_workspace_bytes(dt, rows, cols) >= 0

@@ -53,7 +53,8 @@ def test_sce_sparse(hk, cuda, dtype, shape):
 
 def test_label_gather_is_exact(hk, cuda):
     """Rows built so that loss is exactly representable: a zero logit at one
-    position, -2^k elsewhere (their exponentials vanish next to exp(0))."""
+    position (the maximum), -8192 elsewhere and -2^(r+4) under the label; every
+    other exponential vanishes next to exp(0) at the precision of the result."""
     import torch
     cols = 32000
     labs = np.array([0, 1, 7, 8, 255, 4095, 31999, 16000, 12345], dtype=np.int64)
@@ -62,14 +63,14 @@ def test_label_gather_is_exact(hk, cuda):
         x = np.full((rows, cols), -8192.0, dtype=np.float32)
         for r in range(rows):
             x[r, (int(labs[r]) + 3) % cols] = 0.0        # the row maximum
-            x[r, labs[r]] = -float(2 ** (r + 1))         # distinct value under the label
+            x[r, labs[r]] = -float(2 ** (r + 4))         # distinct value under the label
         tx = helpers.to_torch(x, dtype, cuda)
         tl = torch.from_numpy(labs).to(cuda)
         tloss = torch.empty(rows, dtype=tdt, device=cuda)
         hk.sce_sparse_fwd(tx, tl, tloss, IGN)
         torch.cuda.synchronize()
         got = tloss.float().cpu().numpy()
-        assert np.array_equal(got, np.array([float(2 ** (r + 1)) for r in range(rows)], dtype=np.float32))
+        assert np.array_equal(got, np.array([float(2 ** (r + 4)) for r in range(rows)], dtype=np.float32))
 
 
 def test_out_of_range_label_is_nan(hk, cuda):

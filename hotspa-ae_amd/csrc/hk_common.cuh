@@ -311,22 +311,31 @@ struct MomentTuple {
   }
 };
 
-// (running max, sum of exp(x - max)) for the online softmax
-struct MaxSumTuple {
-  static constexpr int K = 2;
-  float v[2];
-  static __device__ __forceinline__ MaxSumTuple merge(const MaxSumTuple& a, const MaxSumTuple& b) {
-    constexpr float kLog2e = 1.4426950408889634f;
-    MaxSumTuple r;
+// Online softmax state.  v[0] = ml, the running maximum ALREADY multiplied by
+// log2(e) and rounded to fp32 once; v[1] = sum of exp2(x * log2e - ml).  Every
+// exponential of a thread is taken against the thread's own rounded ml and
+// re-based by exp2(ml_a - ml_b), a difference of two fp32 numbers, so the
+// rounding of ml is a common factor of numerator and denominator and cancels:
+// results do not degrade when the logits carry a large common offset.
+// K3 variant: v[2] additionally tracks the maximum itself (for log-sum-exp).
+template <int KK>
+struct OnlineSoftmaxTuple {
+  static constexpr int K = KK;
+  float v[KK];
+  static __device__ __forceinline__ OnlineSoftmaxTuple merge(const OnlineSoftmaxTuple& a,
+                                                              const OnlineSoftmaxTuple& b) {
+    OnlineSoftmaxTuple r;
     const float m = fmaxf(a.v[0], b.v[0]);
-    // an empty side has max = -inf and sum = 0; keep exp2(-inf - -inf) out of the result
+    // an empty side has ml = -inf and sum = 0; keep exp2(-inf - -inf) out of the result
     const float ms = (m == -__builtin_huge_valf()) ? 0.f : m;
     r.v[0] = m;
-    r.v[1] = a.v[1] * __builtin_amdgcn_exp2f((a.v[0] - ms) * kLog2e) +
-             b.v[1] * __builtin_amdgcn_exp2f((b.v[0] - ms) * kLog2e);
+    r.v[1] = a.v[1] * __builtin_amdgcn_exp2f(a.v[0] - ms) + b.v[1] * __builtin_amdgcn_exp2f(b.v[0] - ms);
+    if constexpr (KK == 3) r.v[2] = fmaxf(a.v[2], b.v[2]);
     return r;
   }
 };
+using MaxSumTuple = OnlineSoftmaxTuple<2>;
+using MaxSumMaxTuple = OnlineSoftmaxTuple<3>;
 
 // ---------------------------------------------------------------------------
 // host helpers

@@ -43,7 +43,7 @@ template <typename T, int NV, bool WAVE_ROW>
 __global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
 void sce_sparse_fwd_kernel(SceArgs a) {
   constexpr int VEC = VecIO<T>::N;
-  __shared__ float red[kMaxWaves * 2];
+  __shared__ float red[kMaxWaves * 3];
   int tpr, t, nwaves;
   int64_t row;
   row_coords<WAVE_ROW>(tpr, t, row, nwaves);
@@ -73,8 +73,8 @@ void sce_sparse_fwd_kernel(SceArgs a) {
       for (int j = 0; j < VEC; ++j) m = fmaxf(m, f[j]);
     }
   }
-  const float ms = (m == kNegInf) ? 0.f : m;
-  const float off = -ms * kLog2e;
+  // ml: this thread's maximum in the log2 domain, rounded once (see OnlineSoftmaxTuple)
+  const float ml = (m == kNegInf) ? 0.f : m * kLog2e;
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -82,17 +82,20 @@ void sce_sparse_fwd_kernel(SceArgs a) {
       float f[VEC];
       VecIO<T>::unpack(raw[i], f);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) s += __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, off));
+      for (int j = 0; j < VEC; ++j) s += __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, -ml));
     }
   }
-  MaxSumTuple p;
-  p.v[0] = m; p.v[1] = s;
+  MaxSumMaxTuple p;
+  p.v[0] = (m == kNegInf) ? kNegInf : ml; p.v[1] = s; p.v[2] = m;
   p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);
   if (t == 0) {
     float r;
     if (label >= 0 && label < a.cols) {
       const float xl = Cvt<T>::load(xr + label);
-      r = (__builtin_amdgcn_logf(p.v[1]) * kLn2 + p.v[0]) - xl;
+      // sum exp(x - M) = S * 2^(ML - M * log2e); the fma recovers the rounding of ML exactly
+      const float M = p.v[2];
+      const float log2s = __builtin_amdgcn_logf(p.v[1]) - fmaf(M, kLog2e, -p.v[0]);
+      r = (log2s * kLn2 + M) - xl;
     } else {
       r = __builtin_nanf("");  // label outside [0, cols): no logit to gather
     }
@@ -146,19 +149,18 @@ void sce_sparse_bwd_kernel(SceArgs a) {
       m = fmaxf(m, e[i * VEC + j]);
     }
   }
-  const float ms = (m == kNegInf) ? 0.f : m;
-  const float off = -ms * kLog2e;
+  const float ml = (m == kNegInf) ? 0.f : m * kLog2e;
   float s = 0.f;
 #pragma unroll
   for (int k = 0; k < NV * VEC; ++k) {
-    e[k] = __builtin_amdgcn_exp2f(fmaf(e[k], kLog2e, off));
+    e[k] = __builtin_amdgcn_exp2f(fmaf(e[k], kLog2e, -ml));
     s += e[k];
   }
   MaxSumTuple p;
-  p.v[0] = m; p.v[1] = s;
+  p.v[0] = (m == kNegInf) ? kNegInf : ml; p.v[1] = s;
   p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);
-  const float M = (p.v[0] == kNegInf) ? 0.f : p.v[0];
-  const float scale = __builtin_amdgcn_exp2f((ms - M) * kLog2e) / p.v[1] * g;
+  const float ML = (p.v[0] == kNegInf) ? 0.f : p.v[0];
+  const float scale = __builtin_amdgcn_exp2f(ml - ML) / p.v[1] * g;
   const int lvec = int(label / VEC), lsub = int(label - int64_t(lvec) * VEC);
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -184,7 +186,7 @@ template <typename T, int NV, bool WAVE_ROW, bool BWD>
 __global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
 void sce_dense_kernel(SceArgs a) {
   constexpr int VEC = VecIO<T>::N;
-  __shared__ float red[kMaxWaves * 2];
+  __shared__ float red[kMaxWaves * 3];
   __shared__ float red2[kMaxWaves * 2];
   int tpr, t, nwaves;
   int64_t row;
@@ -211,8 +213,7 @@ void sce_dense_kernel(SceArgs a) {
       for (int j = 0; j < VEC; ++j) m = fmaxf(m, f[j]);
     }
   }
-  const float ms = (m == kNegInf) ? 0.f : m;
-  const float off = -ms * kLog2e;
+  const float ml = (m == kNegInf) ? 0.f : m * kLog2e;
   float s = 0.f;
   SumTuple<2> ls;
   ls.v[0] = 0.f; ls.v[1] = 0.f;
@@ -224,25 +225,26 @@ void sce_dense_kernel(SceArgs a) {
       VecIO<T>::unpack(rl[i], l);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        s += __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, off));
+        s += __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, -ml));
         if constexpr (!BWD) { ls.v[0] += l[j]; ls.v[1] = fmaf(l[j], f[j], ls.v[1]); }
       }
     }
   }
-  MaxSumTuple p;
-  p.v[0] = m; p.v[1] = s;
+  MaxSumMaxTuple p;
+  p.v[0] = (m == kNegInf) ? kNegInf : ml; p.v[1] = s; p.v[2] = m;
   p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);
   if constexpr (!BWD) {
     ls = WAVE_ROW ? wave_allreduce_tuple(ls) : group_allreduce_tuple(ls, red2, 0, nwaves);
     if (t == 0) {
-      const float lse = __builtin_amdgcn_logf(p.v[1]) * kLn2 + p.v[0];
+      const float M = p.v[2];
+      const float log2s = __builtin_amdgcn_logf(p.v[1]) - fmaf(M, kLog2e, -p.v[0]);
+      const float lse = log2s * kLn2 + M;
       Cvt<T>::store(static_cast<T*>(a.out) + row, lse * ls.v[0] - ls.v[1]);
     }
   } else {
     const float g = Cvt<T>::load(static_cast<const T*>(a.grad_loss) + row);
-    const float M = (p.v[0] == kNegInf) ? 0.f : p.v[0];
+    const float ML = (p.v[0] == kNegInf) ? 0.f : p.v[0];
     const float inv = 1.0f / p.v[1];
-    const float off2 = -M * kLog2e;
     T* dxr = static_cast<T*>(a.out) + row * int64_t(a.cols);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -253,7 +255,7 @@ void sce_dense_kernel(SceArgs a) {
         VecIO<T>::unpack(rl[i], l);
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
-          f[j] = (__builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, off2)) * inv - l[j]) * g;
+          f[j] = (__builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, -ML)) * inv - l[j]) * g;
         const u32x4 o = VecIO<T>::pack(f);
         if (a.stream_store) st16_stream(dxr + v * VEC, o);
         else st16(dxr + v * VEC, o);

@@ -57,19 +57,19 @@ void softmax_fwd_kernel(SoftmaxArgs a) {
       m = fmaxf(m, e[i * VEC + j]);
     }
   }
-  const float ms = (m == kNegInf) ? 0.f : m;
-  const float off = -ms * kLog2e;
+  // ml: this thread's maximum in the log2 domain, rounded once (see OnlineSoftmaxTuple)
+  const float ml = (m == kNegInf) ? 0.f : m * kLog2e;
   float s = 0.f;
 #pragma unroll
   for (int k = 0; k < NV * VEC; ++k) {
-    e[k] = __builtin_amdgcn_exp2f(fmaf(e[k], kLog2e, off));
+    e[k] = __builtin_amdgcn_exp2f(fmaf(e[k], kLog2e, -ml));
     s += e[k];
   }
   MaxSumTuple p;
-  p.v[0] = m; p.v[1] = s;
+  p.v[0] = (m == kNegInf) ? kNegInf : ml; p.v[1] = s;
   p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);
-  const float M = (p.v[0] == kNegInf) ? 0.f : p.v[0];
-  const float scale = __builtin_amdgcn_exp2f((ms - M) * kLog2e) / p.v[1];
+  const float ML = (p.v[0] == kNegInf) ? 0.f : p.v[0];
+  const float scale = __builtin_amdgcn_exp2f(ml - ML) / p.v[1];
 
   T* yr = static_cast<T*>(a.out) + row * int64_t(a.cols);
 #pragma unroll

@@ -137,3 +137,21 @@ def test_sce_full_size_bf16(hk, cuda):
     mean_all = tloss.float().sum().item() / rows
     n_valid = int((lab != IGN).sum())
     assert abs(mean_all - tloss.float()[~ign].mean().item() * n_valid / rows) <= 1e-4
+
+
+def test_large_common_offset(hk, cuda):
+    """Logits around +1000 / -3000 in fp32: the shift must cancel exactly, no precision is lost."""
+    import torch
+    for shift in (1000.0, -3000.0):
+        x = (helpers.draw(77, (16, 4096), "normal", 0.0, 2.0) + np.float32(shift)).astype(np.float32)
+        lab = _labels(16, 4096, 78, 0.0)
+        tx, tl = helpers.to_torch(x, "fp32", cuda), torch.from_numpy(lab).to(cuda)
+        tloss = torch.empty(16, device=cuda)
+        hk.sce_sparse_fwd(tx, tl, tloss, IGN)
+        g = np.full(16, 1.0, dtype=np.float32)
+        tdx = torch.empty_like(tx)
+        hk.sce_sparse_bwd(tx, tl, helpers.to_torch(g, "fp32", cuda), tdx, IGN)
+        torch.cuda.synchronize()
+        helpers.assert_close(tloss, oracle.sce_sparse_fwd(x, lab, IGN), "fp32", "loss")
+        edx = oracle.sce_sparse_bwd(x, lab, g, IGN)
+        helpers.assert_close(tdx, edx, "fp32", "dlogits", scale=float(np.abs(edx).max()) * 1e-2)

@@ -70,20 +70,41 @@ def build_device(verbose=True):
 
 
 def build_host(verbose=True):
-    if not os.path.isdir(HOST):
-        return None
+    """g++: every .cc under hetu/ -> lib/libhetu_rowwise.so, then the host
+    self-test tests/cpp/host_selftest.cc -> lib/hetu_host_selftest."""
     srcs = []
     for dirpath, _, files in os.walk(HOST):
         srcs += [os.path.join(dirpath, f) for f in files if f.endswith(".cc")]
     if not srcs:
-        return None
+        raise RuntimeError("no host sources under " + HOST)
+    os.makedirs(LIB, exist_ok=True)
+    objdir = os.path.join(OBJ, "host")
+    os.makedirs(objdir, exist_ok=True)
+    cxx = ["g++", "-O2", "-std=c++17", "-fPIC", "-pthread", "-I" + INCLUDE, "-I" + HERE]
+    srcs = sorted(srcs)
+    objs = [os.path.join(objdir, os.path.relpath(s, HOST).replace(os.sep, "_")[:-3] + ".o") for s in srcs]
+
+    def one(pair):
+        src, obj = pair
+        _run(cxx + ["-c", src, "-o", obj])
+        return src
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
+        for src in pool.map(one, zip(srcs, objs)):
+            if verbose:
+                print("[build] compiled", os.path.relpath(src, ROOT), flush=True)
     out = os.path.join(LIB, "libhetu_rowwise.so")
-    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-pthread", "-fvisibility=default",
-           "-I" + INCLUDE, "-I" + HERE, "-o", out] + sorted(srcs) + [
-           "-L" + LIB, "-lhk_rowwise", "-Wl,-rpath,$ORIGIN"]
-    _run(cmd)
+    _run(["g++", "-shared", "-pthread", "-o", out] + objs +
+         ["-L" + LIB, "-lhk_rowwise", "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("[build] linked", out, flush=True)
+    selftest = os.path.join(ROOT, "tests", "cpp", "host_selftest.cc")
+    if os.path.exists(selftest):
+        exe = os.path.join(LIB, "hetu_host_selftest")
+        _run(cxx + [selftest, "-o", exe, "-L" + LIB, "-lhetu_rowwise", "-lhk_rowwise",
+                    "-Wl,-rpath,$ORIGIN"])
+        if verbose:
+            print("[build] linked", exe, flush=True)
     return out
 
 

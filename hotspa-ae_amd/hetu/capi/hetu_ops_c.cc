@@ -1,0 +1,294 @@
+// extern "C" face of the operator layer (declared in hetu_ops_c.h).
+#include "hetu_ops_c.h"
+
+#include <string>
+
+#include "hetu/graph/ops/kernel_links.h"
+#include "hetu/impl/memory/CachingMemoryPool.h"
+#include "hetu/impl/stream/HIPStream.h"
+
+using namespace hetu;
+
+namespace {
+
+thread_local std::string g_error;
+
+template <typename F>
+int guarded(F&& fn) {
+  try {
+    fn();
+    g_error.clear();
+    return HT_OK;
+  } catch (const hetu::not_implemented& e) {
+    g_error = e.what();
+    return HT_ERR_NOT_IMPLEMENTED;
+  } catch (const hetu::assertion_error& e) {
+    g_error = e.what();
+    return HT_ERR_ASSERTION;
+  } catch (const hetu::value_error& e) {
+    g_error = e.what();
+    return HT_ERR_VALUE;
+  } catch (const hetu::bad_alloc& e) {
+    g_error = e.what();
+    return HT_ERR_BAD_ALLOC;
+  } catch (const hetu::hetu_exception& e) {
+    g_error = e.what();
+    return HT_ERR_RUNTIME;
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return HT_ERR_OTHER;
+  }
+}
+
+Device device_of(const HtArray* a) {
+  return a->device_type == HT_DEVICE_ACCEL ? Device(kCUDA, DeviceIndex(a->device_index)) : Device(kCPU);
+}
+
+NDArray wrap(const HtArray* a) {
+  if (a == nullptr) return NDArray();
+  HT_VALUE_ERROR_IF(a->ndim < 0 || a->ndim > HT_C_MAX_NDIM) << "array rank " << a->ndim << " out of range";
+  HTShape shape(a->shape, a->shape + a->ndim);
+  HTStride stride(a->stride, a->stride + a->ndim);
+  return NDArray::borrow(a->data, shape, device_of(a), static_cast<DataType>(a->dtype), stride);
+}
+
+Stream stream_of(const HtArray* a, int stream_index) {
+  return Stream(device_of(a), StreamIndex(stream_index));
+}
+
+// dense device-to-device copy of an operator result into caller memory
+void copy_out(const NDArray& result, HtArray* out, const Stream& stream) {
+  NDArray dst = wrap(out);
+  HT_ASSERT(dst->is_contiguous()) << "result buffers must be dense";
+  HT_ASSERT(dst->numel() == result->numel() && dst->dtype() == result->dtype())
+    << "result " << result->meta() << " does not fit the buffer " << dst->meta();
+  if (result->numel() == 0) return;
+  NDArray src = NDArray::contiguous(result, stream.stream_index());
+  hetu::impl::HIPStream hs(stream);
+  hetu::hip::DeviceGuard guard(hs.device_id());
+  HK_CALL(hk_memcpy_d2d(dst->raw_data_ptr(), src->raw_data_ptr(), src->numel() * DataType2Size(src->dtype()), hs));
+  NDArray::MarkUsedBy({src, dst}, stream);
+  stream.Sync();   // the caller owns dst and may read it right away
+}
+
+hetu::impl::CachingMemoryPool& caching_pool(int device_index) {
+  auto pool = GetMemoryPool(Device(kCUDA, DeviceIndex(device_index)));
+  auto* cp = dynamic_cast<hetu::impl::CachingMemoryPool*>(pool.get());
+  HT_ASSERT(cp != nullptr) << "device pool is not the caching pool";
+  return *cp;
+}
+
+} // namespace
+
+extern "C" {
+
+const char* ht_last_error(void) { return g_error.c_str(); }
+
+int ht_layer_norm(const HtArray* in, const HtArray* scale, const HtArray* bias, HtArray* mean, HtArray* var,
+                  HtArray* out, int64_t reduce_dims, float eps, int stream_index) {
+  return guarded([&] {
+    NDArray m = wrap(mean), v = wrap(var), o = wrap(out);
+    hetu::impl::LayerNormCuda(wrap(in), wrap(scale), wrap(bias), m, v, o, reduce_dims, eps,
+                              stream_of(in, stream_index));
+  });
+}
+
+int ht_layer_norm_gradient(const HtArray* out_grads, const HtArray* in, const HtArray* scale, HtArray* grad_in,
+                           HtArray* grad_scale, HtArray* grad_bias, const HtArray* mean, const HtArray* var,
+                           int64_t reduce_dims, float eps, int stream_index) {
+  return guarded([&] {
+    NDArray gi = wrap(grad_in), gs = wrap(grad_scale), gb = wrap(grad_bias);
+    hetu::impl::LayerNormGradientCuda(wrap(out_grads), wrap(in), wrap(scale), gi, gs, gb, wrap(mean), wrap(var),
+                                      reduce_dims, eps, stream_of(in, stream_index));
+  });
+}
+
+int ht_fused_layer_norm(const HtArray* in, const HtArray* scale, const HtArray* bias, HtArray* mean,
+                        HtArray* invvar, HtArray* out, int64_t reduce_dims, float eps, int stream_index) {
+  return guarded([&] {
+    NDArray m = wrap(mean), v = wrap(invvar), o = wrap(out);
+    hetu::impl::FusedLayerNormCuda(wrap(in), wrap(scale), wrap(bias), m, v, o, reduce_dims, eps,
+                                   stream_of(in, stream_index));
+  });
+}
+
+int ht_fused_layer_norm_gradient(const HtArray* out_grads, const HtArray* x_or_y, const HtArray* scale,
+                                 const HtArray* bias, HtArray* grad_in, HtArray* grad_scale, HtArray* grad_bias,
+                                 const HtArray* mean, const HtArray* invvar, int64_t reduce_dims, float eps,
+                                 int inplace, int stream_index) {
+  return guarded([&] {
+    NDArray gi = wrap(grad_in), gs = wrap(grad_scale), gb = wrap(grad_bias);
+    hetu::impl::FusedLayerNormGradientCuda(wrap(out_grads), wrap(x_or_y), wrap(scale), wrap(bias), gi, gs, gb,
+                                           wrap(mean), wrap(invvar), reduce_dims, eps, inplace != 0,
+                                           stream_of(x_or_y, stream_index));
+  });
+}
+
+int ht_dropout_add_ln_fwd(const HtArray* x0, const HtArray* residual, const HtArray* gamma, const HtArray* beta,
+                          const HtArray* rowscale, const HtArray* colscale, HtArray* z, HtArray* x, HtArray* mu,
+                          HtArray* rsigma, float dropout_p, float epsilon, int residual_in_fp32, int is_rms_norm,
+                          int stream_index) {
+  return guarded([&] {
+    NDArray zz = wrap(z), xx = wrap(x), m = wrap(mu), r = wrap(rsigma), dmask, none;
+    hetu::impl::DropoutAddLnFwdCuda(wrap(x0), wrap(residual), wrap(gamma), wrap(beta), wrap(rowscale),
+                                    wrap(colscale), none, none, zz, xx, dmask, m, r, dropout_p, epsilon, 1.0f, 0,
+                                    residual_in_fp32 != 0, is_rms_norm != 0, stream_of(x0, stream_index));
+  });
+}
+
+int ht_dropout_add_ln_bwd(const HtArray* dz, const HtArray* dx, const HtArray* x, const HtArray* mu,
+                          const HtArray* rsigma, const HtArray* gamma, const HtArray* rowscale,
+                          const HtArray* colscale, HtArray* dx0, HtArray* dresidual, HtArray* dgamma,
+                          HtArray* dbeta, float dropout_p, int has_residual, int is_rms_norm, int stream_index) {
+  return guarded([&] {
+    NDArray d0 = wrap(dx0), dr = wrap(dresidual), dg = wrap(dgamma), db = wrap(dbeta), none, p1, p2, p3, p4;
+    hetu::impl::DropoutAddLnBwdCuda(wrap(dz), wrap(dx), wrap(x), none, none, wrap(mu), wrap(rsigma), wrap(gamma),
+                                    wrap(rowscale), wrap(colscale), none, none, d0, dr, dg, db, p1, p2, p3, p4,
+                                    dropout_p, 1.0f, 0, has_residual != 0, is_rms_norm != 0,
+                                    stream_of(dz, stream_index));
+  });
+}
+
+int ht_softmax(const HtArray* in, HtArray* out, int64_t dim, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(out);
+    hetu::impl::SoftmaxCuda(wrap(in), o, dim, stream_of(in, stream_index));
+  });
+}
+
+int ht_softmax_gradient(const HtArray* y, const HtArray* dy, HtArray* dx, int64_t dim, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(dx);
+    hetu::impl::SoftmaxGradientCuda(wrap(y), wrap(dy), o, dim, stream_of(y, stream_index));
+  });
+}
+
+int ht_softmax_cross_entropy(const HtArray* pred, const HtArray* label, HtArray* loss, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(loss);
+    hetu::impl::SoftmaxCrossEntropyCuda(wrap(pred), wrap(label), o, stream_of(pred, stream_index));
+  });
+}
+
+int ht_softmax_cross_entropy_gradient(const HtArray* pred, const HtArray* label, const HtArray* grad_loss,
+                                      HtArray* out, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(out);
+    hetu::impl::SoftmaxCrossEntropyGradientCuda(wrap(pred), wrap(label), wrap(grad_loss), o,
+                                                stream_of(pred, stream_index));
+  });
+}
+
+int ht_softmax_cross_entropy_sparse(const HtArray* pred, const HtArray* label, HtArray* loss,
+                                    int64_t ignored_index, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(loss);
+    hetu::impl::SoftmaxCrossEntropySparseCuda(wrap(pred), wrap(label), o, ignored_index,
+                                              stream_of(pred, stream_index));
+  });
+}
+
+int ht_softmax_cross_entropy_sparse_gradient(const HtArray* pred, const HtArray* label, const HtArray* grad_loss,
+                                             HtArray* out, int64_t ignored_index, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(out);
+    hetu::impl::SoftmaxCrossEntropySparseGradientCuda(wrap(pred), wrap(label), wrap(grad_loss), o, ignored_index,
+                                                      stream_of(pred, stream_index));
+  });
+}
+
+int ht_reduce(const HtArray* in, HtArray* out, const int64_t* axes, int naxes, int red_type, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(out);
+    HTAxes ax(axes, axes + naxes);
+    hetu::impl::ReduceCuda(wrap(in), o, ax, static_cast<ReductionType>(red_type), stream_of(in, stream_index));
+  });
+}
+
+int ht_ndarray_reduce(const HtArray* in, int red_type, const int64_t* axes, int naxes, int keepdims, HtArray* out,
+                      int stream_index) {
+  return guarded([&] {
+    HTAxes ax(axes, axes + naxes);
+    NDArray r = NDArray::reduce(wrap(in), static_cast<ReductionType>(red_type), ax, keepdims != 0, stream_index);
+    copy_out(r, out, stream_of(in, stream_index));
+  });
+}
+
+int ht_ndarray_softmax(const HtArray* in, int64_t dim, HtArray* out, int stream_index) {
+  return guarded([&] {
+    NDArray r = NDArray::softmax(wrap(in), dim, stream_index);
+    copy_out(r, out, stream_of(in, stream_index));
+  });
+}
+
+int ht_ndarray_layernorm(const HtArray* in, const HtArray* scale, const HtArray* bias, int normalized_ndim,
+                         double eps, int fused, HtArray* out, HtArray* mean, HtArray* var, int stream_index) {
+  return guarded([&] {
+    NDArray x = wrap(in);
+    HT_VALUE_ERROR_IF(normalized_ndim < 1 || size_t(normalized_ndim) > x->ndim()) << "bad normalized_ndim";
+    HTShape normalized(x->shape().end() - normalized_ndim, x->shape().end());
+    NDArrayList r = fused ? NDArray::fused_layernorm(x, wrap(scale), wrap(bias), normalized, eps, stream_index)
+                          : NDArray::layernorm(x, wrap(scale), wrap(bias), normalized, eps, stream_index);
+    const Stream s = stream_of(in, stream_index);
+    copy_out(r[0], out, s);
+    if (mean) copy_out(r[1], mean, s);
+    if (var) copy_out(r[2], var, s);
+  });
+}
+
+int ht_ndarray_sceloss(const HtArray* preds, const HtArray* labels, int sparse, int64_t ignored_index,
+                       int reduction, HtArray* out, int stream_index) {
+  return guarded([&] {
+    const auto red = static_cast<ReductionType>(reduction);
+    NDArray r = sparse ? NDArray::sceloss(wrap(preds), wrap(labels), ignored_index, red, stream_index)
+                       : NDArray::sceloss(wrap(preds), wrap(labels), red, stream_index);
+    copy_out(r, out, stream_of(preds, stream_index));
+  });
+}
+
+int ht_stream_sync(int device_index, int stream_index) {
+  return guarded([&] { Stream(Device(kCUDA, DeviceIndex(device_index)), StreamIndex(stream_index)).Sync(); });
+}
+
+int ht_synchronize_all(void) {
+  return guarded([&] { SynchronizeAllStreams(); });
+}
+
+int ht_pool_alloc(int device_index, size_t bytes, int stream_index, void** ptr, uint64_t* id,
+                  size_t* granted_bytes) {
+  return guarded([&] {
+    const Device dev(kCUDA, DeviceIndex(device_index));
+    DataPtr p = AllocFromMemoryPool(dev, bytes, Stream(dev, StreamIndex(stream_index)));
+    *ptr = p.ptr;
+    *id = p.id;
+    *granted_bytes = p.size;
+  });
+}
+
+int ht_pool_free(int device_index, void* ptr, uint64_t id, size_t granted_bytes) {
+  return guarded([&] { FreeToMemoryPool(DataPtr(ptr, granted_bytes, Device(kCUDA, DeviceIndex(device_index)), id)); });
+}
+
+int ht_pool_mark_used(int device_index, void* ptr, uint64_t id, size_t granted_bytes, int stream_index) {
+  return guarded([&] {
+    const Device dev(kCUDA, DeviceIndex(device_index));
+    GetMemoryPool(dev)->MarkDataSpaceUsedByStream(DataPtr(ptr, granted_bytes, dev, id),
+                                                  Stream(dev, StreamIndex(stream_index)));
+  });
+}
+
+int ht_pool_empty_cache(int device_index) {
+  return guarded([&] { GetMemoryPool(Device(kCUDA, DeviceIndex(device_index)))->EmptyCache(); });
+}
+
+int ht_pool_stats(int device_index, uint64_t* values, int n_values) {
+  return guarded([&] {
+    auto s = caching_pool(device_index).stats();
+    const uint64_t all[14] = {s.allocated, s.peak_allocated, s.reserved, s.peak_reserved, s.alloc_cnt, s.free_cnt,
+                              s.mark_cnt, s.segment_allocs, s.segment_frees, s.cache_hits, s.cross_stream_takes,
+                              s.parked, s.splits, s.merges};
+    for (int i = 0; i < n_values && i < 14; ++i) values[i] = all[i];
+  });
+}
+
+} // extern "C"

@@ -1,0 +1,94 @@
+// Declarations of the kernel entry points of the row-wise operator path and the
+// device switch that picks them (hetu/graph/ops/kernel_links.h:12-21, 125-135,
+// 168-175, 199-206, 260-269, 296-308, 362-397 of the reference).  The names
+// `KERNEL##Cuda` / `KERNEL##Cpu` are produced by token pasting in the dispatch
+// macros, so they are the link contract; the `Cuda` entries here are the
+// gfx950 implementations.
+#pragma once
+
+#include "hetu/core/ndarray.h"
+#include "hetu/core/stream.h"
+
+namespace hetu {
+namespace impl {
+
+#define DECLARE_KERNEL(KERNEL, DEVICE, ...) extern void KERNEL##DEVICE(__VA_ARGS__)
+#define DECLARE_KERNEL_CPU(KERNEL, ...) DECLARE_KERNEL(KERNEL, Cpu, __VA_ARGS__)
+#define DECLARE_KERNEL_CUDA(KERNEL, ...) DECLARE_KERNEL(KERNEL, Cuda, __VA_ARGS__)
+#define DECLARE_KERNEL_CPU_AND_CUDA(KERNEL, ...)                                                    \
+  DECLARE_KERNEL_CPU(KERNEL, __VA_ARGS__);                                                          \
+  DECLARE_KERNEL_CUDA(KERNEL, __VA_ARGS__)
+
+// x0, residual_, gamma, beta_, rowscale_, colscale_, x0_subset_, z_subset_, z, x, dmask, mu, rsigma,
+// dropout_p, epsilon, rowscale_const, z_numrows, residual_in_fp32, is_rms_norm
+DECLARE_KERNEL_CUDA(DropoutAddLnFwd, const NDArray&, const NDArray&, const NDArray&, const NDArray&,
+                    const NDArray&, const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&, NDArray&,
+                    NDArray&, NDArray&, const float, const float, const float, const int64_t, bool, bool,
+                    const Stream&);
+// dz, dx_, x, x0_, dmask_, mu, rsigma, gamma, rowscale_, colscale_, x0_subset_, z_subset_, dx0, dresidual,
+// dgamma, dbeta, dgamma_part, dbeta_part, dcolscale, dcolscale_part, dropout_p, rowscale_const,
+// x0_numrows, has_residual, is_rms_norm
+DECLARE_KERNEL_CUDA(DropoutAddLnBwd, const NDArray&, const NDArray&, const NDArray&, const NDArray&,
+                    const NDArray&, const NDArray&, const NDArray&, const NDArray&, const NDArray&, const NDArray&,
+                    const NDArray&, const NDArray&, NDArray&, NDArray&, NDArray&, NDArray&, NDArray&, NDArray&,
+                    NDArray&, NDArray&, const float, const float, const int64_t, const bool, bool, const Stream&);
+// in, scale, bias, mean, invvar, out, reduce_dims, eps
+DECLARE_KERNEL_CUDA(FusedLayerNorm, const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&, NDArray&,
+                    int64_t, float, const Stream&);
+// dy, x_or_y, scale, bias, dx, dscale, dbias, mean, invvar, reduce_dims, eps, inplace
+DECLARE_KERNEL_CUDA(FusedLayerNormGradient, const NDArray&, const NDArray&, const NDArray&, const NDArray&,
+                    NDArray&, NDArray&, NDArray&, const NDArray&, const NDArray&, int64_t, float, bool,
+                    const Stream&);
+// in, scale, bias, mean, var, out, reduce_dims, eps
+DECLARE_KERNEL_CPU_AND_CUDA(LayerNorm, const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&,
+                            NDArray&, int64_t, float, const Stream&);
+// dy, x, scale, dx, dscale, dbias, mean, var, reduce_dims, eps
+DECLARE_KERNEL_CPU_AND_CUDA(LayerNormGradient, const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&,
+                            NDArray&, const NDArray&, const NDArray&, int64_t, float, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(Reduce, const NDArray&, NDArray&, const HTAxes&, ReductionType, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(ReduceMean, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(ReduceSum, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(Softmax, const NDArray&, NDArray&, int64_t, const Stream&);
+// y, dy, dx, dim
+DECLARE_KERNEL_CPU_AND_CUDA(SoftmaxGradient, const NDArray&, const NDArray&, NDArray&, int64_t, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(SoftmaxCrossEntropy, const NDArray&, const NDArray&, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(SoftmaxCrossEntropyGradient, const NDArray&, const NDArray&, const NDArray&, NDArray&,
+                            const Stream&);
+// pred, label, loss, ignored_index
+DECLARE_KERNEL_CPU_AND_CUDA(SoftmaxCrossEntropySparse, const NDArray&, const NDArray&, NDArray&, const int64_t,
+                            const Stream&);
+// pred, label, grad_loss, output, ignored_index
+DECLARE_KERNEL_CPU_AND_CUDA(SoftmaxCrossEntropySparseGradient, const NDArray&, const NDArray&, const NDArray&,
+                            NDArray&, const int64_t, const Stream&);
+
+#define HT_DISPATCH_KERNEL_CASE_CPU(KERNEL, ...)                                                    \
+  case kCPU: {                                                                                      \
+    KERNEL##Cpu(__VA_ARGS__);                                                                       \
+    break;                                                                                          \
+  }
+#define HT_DISPATCH_KERNEL_CASE_CUDA(KERNEL, ...)                                                   \
+  case kCUDA: {                                                                                     \
+    KERNEL##Cuda(__VA_ARGS__);                                                                      \
+    break;                                                                                          \
+  }
+#define HT_DISPATCH_KERNEL_SWITCH(DEVICE_TYPE, OP_TYPE, ...)                                        \
+  do {                                                                                              \
+    const auto& _device_type = DEVICE_TYPE;                                                         \
+    switch (_device_type) {                                                                         \
+      __VA_ARGS__                                                                                   \
+      default:                                                                                      \
+        HT_NOT_IMPLEMENTED << "\"" << OP_TYPE << "\" is not implemented for \""                     \
+                           << DeviceType2Str(_device_type) << "\"";                                 \
+    }                                                                                               \
+  } while (0)
+#define HT_DISPATCH_KERNEL_CPU_AND_CUDA(DEVICE_TYPE, OP_TYPE, KERNEL, ...)                          \
+  HT_DISPATCH_KERNEL_SWITCH(DEVICE_TYPE, OP_TYPE,                                                   \
+                            HT_DISPATCH_KERNEL_CASE_CPU(KERNEL, __VA_ARGS__)                        \
+                              HT_DISPATCH_KERNEL_CASE_CUDA(KERNEL, __VA_ARGS__))
+#define HT_DISPATCH_KERNEL_CPU_ONLY(DEVICE_TYPE, OP_TYPE, KERNEL, ...)                              \
+  HT_DISPATCH_KERNEL_SWITCH(DEVICE_TYPE, OP_TYPE, HT_DISPATCH_KERNEL_CASE_CPU(KERNEL, __VA_ARGS__))
+#define HT_DISPATCH_KERNEL_CUDA_ONLY(DEVICE_TYPE, OP_TYPE, KERNEL, ...)                             \
+  HT_DISPATCH_KERNEL_SWITCH(DEVICE_TYPE, OP_TYPE, HT_DISPATCH_KERNEL_CASE_CUDA(KERNEL, __VA_ARGS__))
+
+} // namespace impl
+} // namespace hetu

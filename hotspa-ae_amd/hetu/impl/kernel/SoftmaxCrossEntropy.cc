@@ -1,0 +1,76 @@
+// SoftmaxCrossEntropyCuda / ...GradientCuda (dense labels of the predictions'
+// shape): arguments and meaning of hetu/impl/kernel/SoftmaxCrossEntropy.cu:13-73
+// and :91-171 of the reference, as one fused pass instead of the reference's
+// cuDNN softmax + elementwise + cuDNN reduce.
+#include "hetu/graph/ops/kernel_links.h"
+#include "hetu/impl/kernel/kernel_utils.h"
+
+namespace hetu {
+namespace impl {
+
+void SoftmaxCrossEntropyCuda(const NDArray& input, const NDArray& label, NDArray& output, const Stream& stream) {
+  HT_ASSERT_CUDA_DEVICE(input);
+  HT_ASSERT_SAME_DEVICE(input, label);
+  HT_ASSERT_SAME_DEVICE(input, output);
+  const size_t indim = input->ndim();
+  HT_ASSERT(indim >= 1 && indim == label->ndim() && (indim == output->ndim() + 1 || (indim == 1 && output->ndim() == 1)))
+    << "Indim is " << indim << ", Label dim is " << label->ndim() << ", Output dim is " << output->ndim();
+  HT_ASSERT_SAME_SHAPE(input, label);
+  HT_ASSERT_SAME_DTYPE(input, label);
+  HT_ASSERT_SAME_DTYPE(input, output);
+  HT_ASSERT_CONTIGUOUS(output);
+  int64_t rows = 1;
+  for (size_t i = 0; i + 1 < indim; ++i) rows *= input->shape(i);
+  const int64_t cols = input->shape(indim - 1);
+  HT_ASSERT(int64_t(output->numel()) == rows) << "loss " << output->shape() << " must hold one value per row";
+  if (rows * cols == 0) return;
+
+  HIPStream hip_stream(stream);
+  hip::DeviceGuard guard(hip_stream.device_id());
+  NDArray x = Dense(input, stream), l = Dense(label, stream);
+  HK_CALL(hk_sce_dense_fwd(int(input->dtype()), x->raw_data_ptr(), l->raw_data_ptr(), output->raw_data_ptr(), rows,
+                           cols, hip_stream));
+  NDArray::MarkUsedBy({x, l, output}, stream);
+}
+
+void SoftmaxCrossEntropyGradientCuda(const NDArray& input_y, const NDArray& label, const NDArray& grad,
+                                     NDArray& output, const Stream& stream) {
+  HT_ASSERT_CUDA_DEVICE(input_y);
+  HT_ASSERT_SAME_DEVICE(input_y, label);
+  HT_ASSERT_SAME_DEVICE(input_y, grad);
+  HT_ASSERT_SAME_DEVICE(input_y, output);
+  const size_t indim = input_y->ndim();
+  HT_ASSERT(indim >= 1 && indim == label->ndim() && indim == output->ndim() &&
+            (indim == grad->ndim() + 1 || (indim == 1 && grad->ndim() == 1)))
+    << "Indim is " << indim << ", Label dim is " << label->ndim() << ", Output dim is " << output->ndim();
+  HT_ASSERT_SAME_SHAPE(input_y, label);
+  HT_ASSERT_SAME_SHAPE(input_y, output);
+  HT_ASSERT_SAME_DTYPE(input_y, label);
+  HT_ASSERT_SAME_DTYPE(input_y, grad);
+  HT_ASSERT_SAME_DTYPE(input_y, output);
+  HT_ASSERT_CONTIGUOUS(output);
+  int64_t rows = 1;
+  for (size_t i = 0; i + 1 < indim; ++i) rows *= input_y->shape(i);
+  const int64_t cols = input_y->shape(indim - 1);
+  HT_ASSERT(int64_t(grad->numel()) == rows) << "grad " << grad->shape() << " must hold one value per row";
+  if (rows * cols == 0) return;
+
+  HIPStream hip_stream(stream);
+  hip::DeviceGuard guard(hip_stream.device_id());
+  NDArray x = Dense(input_y, stream), l = Dense(label, stream), g = Dense(grad, stream);
+  HK_CALL(hk_sce_dense_bwd(int(input_y->dtype()), x->raw_data_ptr(), l->raw_data_ptr(), g->raw_data_ptr(),
+                           output->raw_data_ptr(), rows, cols, hip_stream));
+  NDArray::MarkUsedBy({x, l, g, output}, stream);
+}
+
+void SoftmaxCrossEntropyCpu(const NDArray&, const NDArray&, NDArray&, const Stream&) {
+  HT_NOT_IMPLEMENTED << "SoftmaxCrossEntropy has no host kernel in this build; move the arrays to the accelerator";
+}
+
+void SoftmaxCrossEntropyGradientCpu(const NDArray&, const NDArray&, const NDArray&, NDArray&, const Stream&) {
+  HT_NOT_IMPLEMENTED << "SoftmaxCrossEntropyGradient has no host kernel in this build; move the arrays to the "
+                        "accelerator";
+}
+
+} // namespace impl
+} // namespace hetu

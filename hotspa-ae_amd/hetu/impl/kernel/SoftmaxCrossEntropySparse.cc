@@ -1,0 +1,81 @@
+// SoftmaxCrossEntropySparseCuda / ...GradientCuda: arguments and meaning of
+// hetu/impl/kernel/SoftmaxCrossEntropySparse.cu:239-274 and :276-318 of the
+// reference.  Labels are int64 class ids, one per row; a row whose label equals
+// `ignored_index` has loss 0 and a zero gradient row.
+#include "hetu/graph/ops/kernel_links.h"
+#include "hetu/impl/kernel/kernel_utils.h"
+
+namespace hetu {
+namespace impl {
+
+namespace {
+void RowsCols(const NDArray& pred, int64_t& rows, int64_t& cols) {
+  HT_ASSERT(pred->ndim() >= 1) << "predictions need at least one dimension";
+  rows = 1;
+  for (size_t i = 0; i + 1 < pred->ndim(); ++i) rows *= pred->shape(i);
+  cols = pred->shape(pred->ndim() - 1);
+}
+} // namespace
+
+void SoftmaxCrossEntropySparseCuda(const NDArray& pred, const NDArray& label, NDArray& loss,
+                                   const int64_t ignored_index, const Stream& stream) {
+  HT_ASSERT_CUDA_DEVICE(pred);
+  HT_ASSERT_SAME_DEVICE(pred, label);
+  HT_ASSERT_SAME_DEVICE(pred, loss);
+  HT_ASSERT_SAME_DTYPE(pred, loss);
+  HT_ASSERT(label->dtype() == kInt64) << "labels must be int64 class ids, got " << label->dtype();
+  HT_ASSERT_CONTIGUOUS(loss);
+  int64_t rows, cols;
+  RowsCols(pred, rows, cols);
+  HT_ASSERT(int64_t(label->numel()) == rows && int64_t(loss->numel()) == rows)
+    << "labels " << label->shape() << " / loss " << loss->shape() << " must hold one value per row of "
+    << pred->shape();
+  if (rows == 0) return;
+  HT_VALUE_ERROR_IF(cols == 0) << "cross entropy over zero classes";
+
+  HIPStream hip_stream(stream);
+  hip::DeviceGuard guard(hip_stream.device_id());
+  NDArray p = Dense(pred, stream), l = Dense(label, stream);
+  HK_CALL(hk_sce_sparse_fwd(int(pred->dtype()), p->raw_data_ptr(), l->data_ptr<int64_t>(), loss->raw_data_ptr(), rows,
+                            cols, ignored_index, hip_stream));
+  NDArray::MarkUsedBy({p, l, loss}, stream);
+}
+
+void SoftmaxCrossEntropySparseGradientCuda(const NDArray& pred, const NDArray& label, const NDArray& grad_loss,
+                                           NDArray& output, const int64_t ignored_index, const Stream& stream) {
+  HT_ASSERT_CUDA_DEVICE(pred);
+  HT_ASSERT_SAME_DEVICE(pred, label);
+  HT_ASSERT_SAME_DEVICE(pred, grad_loss);
+  HT_ASSERT_SAME_DEVICE(pred, output);
+  HT_ASSERT_SAME_SHAPE(pred, output);
+  HT_ASSERT_SAME_DTYPE(pred, output);
+  HT_ASSERT_SAME_DTYPE(pred, grad_loss);
+  HT_ASSERT(label->dtype() == kInt64) << "labels must be int64 class ids, got " << label->dtype();
+  HT_ASSERT_CONTIGUOUS(output);
+  int64_t rows, cols;
+  RowsCols(pred, rows, cols);
+  HT_ASSERT(int64_t(label->numel()) == rows && int64_t(grad_loss->numel()) == rows)
+    << "labels " << label->shape() << " / grad_loss " << grad_loss->shape() << " must hold one value per row of "
+    << pred->shape();
+  if (rows == 0 || cols == 0) return;
+
+  HIPStream hip_stream(stream);
+  hip::DeviceGuard guard(hip_stream.device_id());
+  NDArray p = Dense(pred, stream), l = Dense(label, stream), g = Dense(grad_loss, stream);
+  HK_CALL(hk_sce_sparse_bwd(int(pred->dtype()), p->raw_data_ptr(), l->data_ptr<int64_t>(), g->raw_data_ptr(),
+                            output->raw_data_ptr(), rows, cols, ignored_index, hip_stream));
+  NDArray::MarkUsedBy({p, l, g, output}, stream);
+}
+
+void SoftmaxCrossEntropySparseCpu(const NDArray&, const NDArray&, NDArray&, const int64_t, const Stream&) {
+  HT_NOT_IMPLEMENTED << "SoftmaxCrossEntropySparse has no host kernel in this build; move the arrays to the accelerator";
+}
+
+void SoftmaxCrossEntropySparseGradientCpu(const NDArray&, const NDArray&, const NDArray&, NDArray&, const int64_t,
+                                          const Stream&) {
+  HT_NOT_IMPLEMENTED << "SoftmaxCrossEntropySparseGradient has no host kernel in this build; move the arrays to the "
+                        "accelerator";
+}
+
+} // namespace impl
+} // namespace hetu

@@ -1,0 +1,254 @@
+"""ctypes bindings of include/hetu_ops_c.h: the C++ operator layer
+(libhetu_rowwise.so) called with torch tensors as borrowed arrays.
+
+Errors of the C++ layer come back as Python exceptions named after the C++
+ones (AssertionError_, NotImplemented_, ValueError_, RuntimeError_).
+"""
+import ctypes
+import os
+
+from . import capi
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "lib", "libhetu_rowwise.so")
+_lib = None
+
+MAX_NDIM = 8
+RED = {"sum": 0, "mean": 1, "max": 2, "min": 3, "prod": 4, "none": 5}
+DEFAULT_STREAM = 1   # hetu::kComputingStream
+
+
+class HetuError(RuntimeError):
+    kind = "other"
+
+
+class AssertionError_(HetuError):
+    kind = "assertion_error"
+
+
+class NotImplemented_(HetuError):
+    kind = "not_implemented"
+
+
+class ValueError_(HetuError):
+    kind = "value_error"
+
+
+class RuntimeError_(HetuError):
+    kind = "runtime_error"
+
+
+class BadAlloc_(HetuError):
+    kind = "bad_alloc"
+
+
+_KINDS = {1: AssertionError_, 2: NotImplemented_, 3: ValueError_, 4: RuntimeError_, 5: BadAlloc_}
+
+
+class HtArray(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("dtype", ctypes.c_int32), ("ndim", ctypes.c_int32),
+                ("shape", ctypes.c_int64 * MAX_NDIM), ("stride", ctypes.c_int64 * MAX_NDIM),
+                ("device_type", ctypes.c_int32), ("device_index", ctypes.c_int32)]
+
+
+def lib_path():
+    return _LIB
+
+
+def lib():
+    """Loads libhetu_rowwise.so; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            raise HetuError("native library %s is missing: run __graft_entry__.build() first" % _LIB)
+        capi.lib()   # libhk_rowwise.so first, so the dependency resolves from the same folder
+        _lib = ctypes.CDLL(_LIB)
+        _lib.ht_last_error.restype = ctypes.c_char_p
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise _KINDS.get(rc, HetuError)(lib().ht_last_error().decode("utf-8", "replace"))
+
+
+def desc(t):
+    """HtArray borrowing a torch tensor (None -> NULL = undefined NDArray)."""
+    if t is None:
+        return None
+    assert t.dim() <= MAX_NDIM
+    a = HtArray()
+    a.data = t.data_ptr()
+    a.dtype = capi.dtype_code(t)
+    a.ndim = t.dim()
+    for i in range(t.dim()):
+        a.shape[i] = t.shape[i]
+        a.stride[i] = t.stride(i)
+    a.device_type = 1 if t.is_cuda else 0
+    a.device_index = t.device.index or 0 if t.is_cuda else 0
+    a._keep = t
+    return a
+
+
+def _p(a):
+    return ctypes.byref(a) if a is not None else None
+
+
+def _call(name, *args):
+    conv = []
+    for v in args:
+        if isinstance(v, HtArray) or v is None:
+            conv.append(_p(v))
+        else:
+            conv.append(v)
+    check(getattr(lib(), name)(*conv))
+
+
+def _i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def _f(v):
+    return ctypes.c_float(float(v))
+
+
+def _axes(axes):
+    axes = list(axes)
+    return (ctypes.c_int64 * max(len(axes), 1))(*axes), ctypes.c_int(len(axes))
+
+
+def stream_sync(stream=DEFAULT_STREAM, device=0):
+    check(lib().ht_stream_sync(ctypes.c_int(device), ctypes.c_int(stream)))
+
+
+def synchronize_all():
+    check(lib().ht_synchronize_all())
+
+
+# ---- kernel entry points --------------------------------------------------
+def layer_norm(x, scale, bias, mean, var, out, reduce_dims, eps, stream=DEFAULT_STREAM):
+    _call("ht_layer_norm", desc(x), desc(scale), desc(bias), desc(mean), desc(var), desc(out), _i64(reduce_dims),
+          _f(eps), ctypes.c_int(stream))
+
+
+def layer_norm_gradient(dy, x, scale, dx, dscale, dbias, mean, var, reduce_dims, eps, stream=DEFAULT_STREAM):
+    _call("ht_layer_norm_gradient", desc(dy), desc(x), desc(scale), desc(dx), desc(dscale), desc(dbias), desc(mean),
+          desc(var), _i64(reduce_dims), _f(eps), ctypes.c_int(stream))
+
+
+def fused_layer_norm(x, scale, bias, mean, invvar, out, reduce_dims, eps, stream=DEFAULT_STREAM):
+    _call("ht_fused_layer_norm", desc(x), desc(scale), desc(bias), desc(mean), desc(invvar), desc(out),
+          _i64(reduce_dims), _f(eps), ctypes.c_int(stream))
+
+
+def fused_layer_norm_gradient(dy, x_or_y, scale, bias, dx, dscale, dbias, mean, invvar, reduce_dims, eps, inplace,
+                              stream=DEFAULT_STREAM):
+    _call("ht_fused_layer_norm_gradient", desc(dy), desc(x_or_y), desc(scale), desc(bias), desc(dx), desc(dscale),
+          desc(dbias), desc(mean), desc(invvar), _i64(reduce_dims), _f(eps), ctypes.c_int(int(inplace)),
+          ctypes.c_int(stream))
+
+
+def dropout_add_ln_fwd(x0, residual, gamma, beta, z, x, mu, rsigma, eps, is_rms_norm, dropout_p=0.0,
+                       rowscale=None, colscale=None, residual_in_fp32=False, stream=DEFAULT_STREAM):
+    _call("ht_dropout_add_ln_fwd", desc(x0), desc(residual), desc(gamma), desc(beta), desc(rowscale),
+          desc(colscale), desc(z), desc(x), desc(mu), desc(rsigma), _f(dropout_p), _f(eps),
+          ctypes.c_int(int(residual_in_fp32)), ctypes.c_int(int(is_rms_norm)), ctypes.c_int(stream))
+
+
+def dropout_add_ln_bwd(dz, dx, x, mu, rsigma, gamma, dx0, dresidual, dgamma, dbeta, has_residual, is_rms_norm,
+                       dropout_p=0.0, rowscale=None, colscale=None, stream=DEFAULT_STREAM):
+    _call("ht_dropout_add_ln_bwd", desc(dz), desc(dx), desc(x), desc(mu), desc(rsigma), desc(gamma),
+          desc(rowscale), desc(colscale), desc(dx0), desc(dresidual), desc(dgamma), desc(dbeta), _f(dropout_p),
+          ctypes.c_int(int(has_residual)), ctypes.c_int(int(is_rms_norm)), ctypes.c_int(stream))
+
+
+def softmax(x, out, dim, stream=DEFAULT_STREAM):
+    _call("ht_softmax", desc(x), desc(out), _i64(dim), ctypes.c_int(stream))
+
+
+def softmax_gradient(y, dy, dx, dim, stream=DEFAULT_STREAM):
+    _call("ht_softmax_gradient", desc(y), desc(dy), desc(dx), _i64(dim), ctypes.c_int(stream))
+
+
+def softmax_cross_entropy(pred, label, loss, stream=DEFAULT_STREAM):
+    _call("ht_softmax_cross_entropy", desc(pred), desc(label), desc(loss), ctypes.c_int(stream))
+
+
+def softmax_cross_entropy_gradient(pred, label, grad_loss, out, stream=DEFAULT_STREAM):
+    _call("ht_softmax_cross_entropy_gradient", desc(pred), desc(label), desc(grad_loss), desc(out),
+          ctypes.c_int(stream))
+
+
+def softmax_cross_entropy_sparse(pred, label, loss, ignored_index, stream=DEFAULT_STREAM):
+    _call("ht_softmax_cross_entropy_sparse", desc(pred), desc(label), desc(loss), _i64(ignored_index),
+          ctypes.c_int(stream))
+
+
+def softmax_cross_entropy_sparse_gradient(pred, label, grad_loss, out, ignored_index, stream=DEFAULT_STREAM):
+    _call("ht_softmax_cross_entropy_sparse_gradient", desc(pred), desc(label), desc(grad_loss), desc(out),
+          _i64(ignored_index), ctypes.c_int(stream))
+
+
+def reduce(x, out, axes, red_type, stream=DEFAULT_STREAM):
+    ax, n = _axes(axes)
+    _call("ht_reduce", desc(x), desc(out), ax, n, ctypes.c_int(RED[red_type]), ctypes.c_int(stream))
+
+
+# ---- NDArray statics ------------------------------------------------------
+def ndarray_reduce(x, red_type, axes, keepdims, out, stream=DEFAULT_STREAM):
+    ax, n = _axes(axes)
+    _call("ht_ndarray_reduce", desc(x), ctypes.c_int(RED[red_type]), ax, n, ctypes.c_int(int(keepdims)), desc(out),
+          ctypes.c_int(stream))
+
+
+def ndarray_softmax(x, dim, out, stream=DEFAULT_STREAM):
+    _call("ht_ndarray_softmax", desc(x), _i64(dim), desc(out), ctypes.c_int(stream))
+
+
+def ndarray_layernorm(x, scale, bias, normalized_ndim, eps, fused, out, mean=None, var=None,
+                      stream=DEFAULT_STREAM):
+    _call("ht_ndarray_layernorm", desc(x), desc(scale), desc(bias), ctypes.c_int(normalized_ndim),
+          ctypes.c_double(eps), ctypes.c_int(int(fused)), desc(out), desc(mean), desc(var), ctypes.c_int(stream))
+
+
+def ndarray_sceloss(preds, labels, out, reduction="mean", ignored_index=None, stream=DEFAULT_STREAM):
+    sparse = ignored_index is not None
+    _call("ht_ndarray_sceloss", desc(preds), desc(labels), ctypes.c_int(int(sparse)),
+          _i64(ignored_index if sparse else 0), ctypes.c_int(RED[reduction]), desc(out), ctypes.c_int(stream))
+
+
+# ---- device memory pool ---------------------------------------------------
+class PoolBlock:
+    def __init__(self, ptr, ident, size, device):
+        self.ptr, self.id, self.size, self.device = ptr, ident, size, device
+
+
+def pool_alloc(nbytes, stream=DEFAULT_STREAM, device=0):
+    ptr, ident, granted = ctypes.c_void_p(), ctypes.c_uint64(), ctypes.c_size_t()
+    check(lib().ht_pool_alloc(ctypes.c_int(device), ctypes.c_size_t(nbytes), ctypes.c_int(stream),
+                              ctypes.byref(ptr), ctypes.byref(ident), ctypes.byref(granted)))
+    return PoolBlock(ptr.value or 0, ident.value, granted.value, device)
+
+
+def pool_free(block):
+    check(lib().ht_pool_free(ctypes.c_int(block.device), ctypes.c_void_p(block.ptr), ctypes.c_uint64(block.id),
+                             ctypes.c_size_t(block.size)))
+
+
+def pool_mark_used(block, stream):
+    check(lib().ht_pool_mark_used(ctypes.c_int(block.device), ctypes.c_void_p(block.ptr), ctypes.c_uint64(block.id),
+                                  ctypes.c_size_t(block.size), ctypes.c_int(stream)))
+
+
+def pool_empty_cache(device=0):
+    check(lib().ht_pool_empty_cache(ctypes.c_int(device)))
+
+
+_STAT_NAMES = ["allocated", "peak_allocated", "reserved", "peak_reserved", "alloc_cnt", "free_cnt", "mark_cnt",
+               "segment_allocs", "segment_frees", "cache_hits", "cross_stream_takes", "parked", "splits", "merges"]
+
+
+def pool_stats(device=0):
+    vals = (ctypes.c_uint64 * len(_STAT_NAMES))()
+    check(lib().ht_pool_stats(ctypes.c_int(device), vals, ctypes.c_int(len(_STAT_NAMES))))
+    return dict(zip(_STAT_NAMES, [int(v) for v in vals]))

@@ -1,0 +1,115 @@
+/* C entry points over the C++ operator layer (libhetu_rowwise.so): the
+ * `<Kernel>Cuda` functions declared in hetu/graph/ops/kernel_links.h of the
+ * reference and the NDArray statics that dispatch to them, callable from any
+ * language with a C FFI.  Arrays are described, not owned: every HtArray
+ * borrows caller memory for the duration of the call.  A NULL HtArray pointer
+ * stands for an undefined NDArray (an optional operand left out).
+ *
+ * Every function returns HT_OK or the kind of C++ exception the layer threw;
+ * ht_last_error() holds its message (thread-local).
+ */
+#ifndef HETU_OPS_C_H_
+#define HETU_OPS_C_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HT_API __attribute__((visibility("default")))
+
+enum {
+  HT_OK = 0,
+  HT_ERR_ASSERTION = 1,       /* hetu::assertion_error   (HT_ASSERT*)        */
+  HT_ERR_NOT_IMPLEMENTED = 2, /* hetu::not_implemented   (HT_NOT_IMPLEMENTED) */
+  HT_ERR_VALUE = 3,           /* hetu::value_error       (HT_VALUE_ERROR)     */
+  HT_ERR_RUNTIME = 4,         /* hetu::runtime_error, HIP failures            */
+  HT_ERR_BAD_ALLOC = 5,       /* hetu::bad_alloc                              */
+  HT_ERR_OTHER = 6
+};
+
+enum { HT_DEVICE_CPU = 0, HT_DEVICE_ACCEL = 1 };   /* hetu::DeviceType kCPU / kCUDA */
+enum { HT_RED_SUM = 0, HT_RED_MEAN = 1, HT_RED_MAX = 2, HT_RED_MIN = 3, HT_RED_PROD = 4, HT_RED_NONE = 5 };
+
+#define HT_C_MAX_NDIM 8
+
+typedef struct HtArray {
+  void* data;
+  int32_t dtype;                 /* hetu::DataType value (HK_FLOAT32 ...)      */
+  int32_t ndim;
+  int64_t shape[HT_C_MAX_NDIM];
+  int64_t stride[HT_C_MAX_NDIM];   /* in elements                                 */
+  int32_t device_type;           /* HT_DEVICE_*                                 */
+  int32_t device_index;
+} HtArray;
+
+HT_API const char* ht_last_error(void);
+
+/* ---- kernel entry points (one per `<Kernel>Cuda` symbol) ---- */
+HT_API int ht_layer_norm(const HtArray* in, const HtArray* scale, const HtArray* bias, HtArray* mean,
+                         HtArray* var, HtArray* out, int64_t reduce_dims, float eps, int stream_index);
+HT_API int ht_layer_norm_gradient(const HtArray* out_grads, const HtArray* in, const HtArray* scale,
+                                  HtArray* grad_in, HtArray* grad_scale, HtArray* grad_bias,
+                                  const HtArray* mean, const HtArray* var, int64_t reduce_dims, float eps,
+                                  int stream_index);
+HT_API int ht_fused_layer_norm(const HtArray* in, const HtArray* scale, const HtArray* bias, HtArray* mean,
+                               HtArray* invvar, HtArray* out, int64_t reduce_dims, float eps,
+                               int stream_index);
+HT_API int ht_fused_layer_norm_gradient(const HtArray* out_grads, const HtArray* x_or_y, const HtArray* scale,
+                                        const HtArray* bias, HtArray* grad_in, HtArray* grad_scale,
+                                        HtArray* grad_bias, const HtArray* mean, const HtArray* invvar,
+                                        int64_t reduce_dims, float eps, int inplace, int stream_index);
+HT_API int ht_dropout_add_ln_fwd(const HtArray* x0, const HtArray* residual, const HtArray* gamma,
+                                 const HtArray* beta, const HtArray* rowscale, const HtArray* colscale,
+                                 HtArray* z, HtArray* x, HtArray* mu, HtArray* rsigma, float dropout_p,
+                                 float epsilon, int residual_in_fp32, int is_rms_norm, int stream_index);
+HT_API int ht_dropout_add_ln_bwd(const HtArray* dz, const HtArray* dx, const HtArray* x, const HtArray* mu,
+                                 const HtArray* rsigma, const HtArray* gamma, const HtArray* rowscale,
+                                 const HtArray* colscale, HtArray* dx0, HtArray* dresidual, HtArray* dgamma,
+                                 HtArray* dbeta, float dropout_p, int has_residual, int is_rms_norm,
+                                 int stream_index);
+HT_API int ht_softmax(const HtArray* in, HtArray* out, int64_t dim, int stream_index);
+HT_API int ht_softmax_gradient(const HtArray* y, const HtArray* dy, HtArray* dx, int64_t dim, int stream_index);
+HT_API int ht_softmax_cross_entropy(const HtArray* pred, const HtArray* label, HtArray* loss, int stream_index);
+HT_API int ht_softmax_cross_entropy_gradient(const HtArray* pred, const HtArray* label, const HtArray* grad_loss,
+                                             HtArray* out, int stream_index);
+HT_API int ht_softmax_cross_entropy_sparse(const HtArray* pred, const HtArray* label, HtArray* loss,
+                                           int64_t ignored_index, int stream_index);
+HT_API int ht_softmax_cross_entropy_sparse_gradient(const HtArray* pred, const HtArray* label,
+                                                    const HtArray* grad_loss, HtArray* out,
+                                                    int64_t ignored_index, int stream_index);
+HT_API int ht_reduce(const HtArray* in, HtArray* out, const int64_t* axes, int naxes, int red_type,
+                     int stream_index);
+
+/* ---- NDArray statics: device dispatch + output allocation from the pool ----
+ * `out` (and mean / var) describe caller memory the result is written to. */
+HT_API int ht_ndarray_reduce(const HtArray* in, int red_type, const int64_t* axes, int naxes, int keepdims,
+                             HtArray* out, int stream_index);
+HT_API int ht_ndarray_softmax(const HtArray* in, int64_t dim, HtArray* out, int stream_index);
+HT_API int ht_ndarray_layernorm(const HtArray* in, const HtArray* scale, const HtArray* bias,
+                                int normalized_ndim, double eps, int fused, HtArray* out, HtArray* mean,
+                                HtArray* var, int stream_index);
+/* sparse = 1: int64 labels + ignored_index; sparse = 0: dense labels. */
+HT_API int ht_ndarray_sceloss(const HtArray* preds, const HtArray* labels, int sparse, int64_t ignored_index,
+                              int reduction, HtArray* out, int stream_index);
+
+/* ---- streams and the device memory pool ---- */
+HT_API int ht_stream_sync(int device_index, int stream_index);
+HT_API int ht_synchronize_all(void);
+HT_API int ht_pool_alloc(int device_index, size_t bytes, int stream_index, void** ptr, uint64_t* id,
+                         size_t* granted_bytes);
+HT_API int ht_pool_free(int device_index, void* ptr, uint64_t id, size_t granted_bytes);
+HT_API int ht_pool_mark_used(int device_index, void* ptr, uint64_t id, size_t granted_bytes, int stream_index);
+HT_API int ht_pool_empty_cache(int device_index);
+/* allocated, peak_allocated, reserved, peak_reserved, alloc_cnt, free_cnt,
+ * mark_cnt, segment_allocs, segment_frees, cache_hits, cross_stream_takes,
+ * parked, splits, merges: 14 values */
+HT_API int ht_pool_stats(int device_index, uint64_t* values, int n_values);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* HETU_OPS_C_H_ */

@@ -1,0 +1,461 @@
+// Host-side checks of the C++ operator layer that need no GPU: dtypes, devices,
+// streams, axis parsing, exceptions, the host pool, NDArray views, the device
+// switch, and the caching pool's policy driven through a scripted backend.
+// Prints one line per check; exit status is the number of failed checks.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <set>
+#include <string>
+
+#include "hetu/core/ndarray.h"
+#include "hetu/graph/ops/kernel_links.h"
+#include "hetu/impl/memory/CachingMemoryPool.h"
+#include "hetu/impl/utils/dispatch.h"
+
+using namespace hetu;
+using hetu::impl::CachingMemoryPool;
+using hetu::impl::PoolBackend;
+
+static int g_failed = 0, g_run = 0;
+
+#define CHECK(cond)                                                                    \
+  do {                                                                                 \
+    if (!(cond)) {                                                                     \
+      std::printf("    CHECK FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);          \
+      throw std::runtime_error("check failed");                                        \
+    }                                                                                  \
+  } while (0)
+
+template <typename E, typename F>
+static bool throws(F&& f, const char* needle = nullptr) {
+  try {
+    f();
+  } catch (const E& e) {
+    return needle == nullptr || std::string(e.what()).find(needle) != std::string::npos;
+  } catch (...) {
+    return false;
+  }
+  return false;
+}
+
+static void run(const char* name, const std::function<void()>& body) {
+  ++g_run;
+  try {
+    body();
+    std::printf("[ OK ] %s\n", name);
+  } catch (const std::exception& e) {
+    ++g_failed;
+    std::printf("[FAIL] %s: %s\n", name, e.what());
+  }
+  std::fflush(stdout);
+}
+
+// ---- scripted device: addresses are never dereferenced ----
+struct FakeDevice : PoolBackend {
+  size_t capacity;
+  size_t in_use = 0;
+  uintptr_t next_addr = uintptr_t(1) << 32;
+  std::map<void*, size_t> live;
+  struct Ev { Stream stream; bool done; };
+  std::vector<Ev*> events;
+  std::vector<std::pair<PackedStreamId, PackedStreamId>> waits;   // (waiting stream, recorded-on stream)
+  int device_syncs = 0, stream_syncs = 0;
+  bool auto_complete = false;
+
+  explicit FakeDevice(size_t cap) : capacity(cap) {}
+  ~FakeDevice() override { for (auto* e : events) delete e; }
+  void* RawAlloc(size_t bytes) override {
+    if (in_use + bytes > capacity) return nullptr;
+    void* p = reinterpret_cast<void*>(next_addr);
+    next_addr += (bytes + (size_t(2) << 20) - 1) / (size_t(2) << 20) * (size_t(2) << 20) + (size_t(2) << 20);
+    live[p] = bytes;
+    in_use += bytes;
+    return p;
+  }
+  void RawFree(void* ptr) override {
+    auto it = live.find(ptr);
+    if (it == live.end()) throw std::runtime_error("RawFree of unknown pointer");
+    in_use -= it->second;
+    live.erase(it);
+  }
+  void* EventRecord(const Stream& s) override {
+    auto* e = new Ev{s, auto_complete};
+    events.push_back(e);
+    return e;
+  }
+  bool EventDone(void* e) override { return static_cast<Ev*>(e)->done; }
+  void EventSync(void* e) override { static_cast<Ev*>(e)->done = true; }
+  void EventRelease(void*) override {}
+  void StreamWaitEvent(const Stream& s, void* e) override {
+    waits.emplace_back(s.pack(), static_cast<Ev*>(e)->stream.pack());
+  }
+  void StreamSync(const Stream&) override { ++stream_syncs; }
+  void DeviceSync() override { ++device_syncs; }
+  void complete_all() { for (auto* e : events) e->done = true; }
+};
+
+static const size_t MiB = size_t(1) << 20;
+
+struct PoolFixture {
+  FakeDevice* dev;
+  std::unique_ptr<CachingMemoryPool> pool;
+  Stream s1{Device(kCUDA, 0), 1}, s2{Device(kCUDA, 0), 2}, s3{Device(kCUDA, 0), 3};
+  explicit PoolFixture(size_t capacity = 4096 * MiB, size_t max_split = 200 * MiB, size_t max_frag = 20 * MiB) {
+    dev = new FakeDevice(capacity);
+    pool.reset(new CachingMemoryPool(Device(kCUDA, 0), "TestPool", std::unique_ptr<PoolBackend>(dev), max_split,
+                                     max_frag));
+  }
+};
+
+int main() {
+  run("dtype sizes and names", [] {
+    CHECK(DataType2Size(kFloat32) == 4 && DataType2Size(kBFloat16) == 2 && DataType2Size(kFloat16) == 2);
+    CHECK(DataType2Size(kFloat64) == 8 && DataType2Size(kInt64) == 8 && DataType2Size(kUInt8) == 1);
+    CHECK(int(kFloat16) == 5 && int(kFloat32) == 6 && int(kFloat64) == 7 && int(kBFloat16) == 8 && int(kInt64) == 4);
+    CHECK(DataType2Str(kBFloat16) == "bfloat16");
+  });
+
+  run("bfloat16 rounds to nearest even and keeps NaN", [] {
+    CHECK(bfloat16(1.0f).val == 0x3F80);
+    // 1 + 2^-8 is the midpoint between 1 and the next bf16: ties go to even (1.0)
+    CHECK(bfloat16(1.0f + 0.00390625f).val == 0x3F80);
+    // 1 + 3*2^-8 is the midpoint between 0x3F81 and 0x3F82: even is 0x3F82
+    CHECK(bfloat16(1.0f + 3 * 0.00390625f).val == 0x3F82);
+    CHECK(bfloat16(std::nanf("")).val == 0x7FC0);
+    CHECK(float(bfloat16(-2.5f)) == -2.5f);
+    CHECK(std::isinf(float(bfloat16(3.4e38f))));
+  });
+
+  run("float16 round trip of every finite half", [] {
+    for (uint32_t h = 0; h < 65536; ++h) {
+      float16 a;
+      a.val = uint16_t(h);
+      const bool nan = ((h & 0x7C00) == 0x7C00) && (h & 0x3FF);
+      if (nan) { CHECK(std::isnan(float(a))); continue; }
+      CHECK(float16(float(a)).val == h);
+    }
+    CHECK(float16(65520.f).val == 0x7C00 && float16(65519.f).val == 0x7BFF);
+    CHECK(float16(1.0f + 0.00048828125f).val == 0x3C00);   // tie -> even
+  });
+
+  run("device and stream handles", [] {
+    Device d(kCUDA, 3), c(kCPU, 5);
+    CHECK(d.is_cuda() && d.index() == 3 && c.is_cpu() && c.index() == 0);
+    CHECK(throws<assertion_error>([] { Device(kCUDA, 16); }));
+    for (int dev = 0; dev < 16; ++dev)
+      for (int id = 0; id < HT_NUM_STREAMS_PER_DEVICE; ++id) {
+        Stream s(Device(kCUDA, DeviceIndex(dev)), id);
+        CHECK(Stream::unpack(s.pack()) == s);
+      }
+    CHECK(Stream::unpack(Stream(Device(kCPU), 0).pack()) == Stream(Device(kCPU), 0));
+    CHECK(throws<assertion_error>([] { Stream(Device(kCUDA, 0), 16); }));
+    CHECK(throws<assertion_error>([] { Stream(Device(kCUDA, 0), -1); }));
+    CHECK(!Stream().is_defined() && Stream(Device(kCUDA, 0)).is_blocking());
+    CHECK(kBlockingStream == 0 && kComputingStream == 1 && NDArray::DEFAULT_STREAM == kComputingStream);
+  });
+
+  run("exceptions carry kind and message", [] {
+    CHECK(throws<assertion_error>([] { HT_ASSERT(1 == 2) << "custom text " << 42; }, "custom text 42"));
+    CHECK(throws<not_implemented>([] { HT_NOT_IMPLEMENTED << "nope"; }, "nope"));
+    CHECK(throws<value_error>([] { HT_VALUE_ERROR_IF(true) << "bad value"; }, "bad value"));
+    CHECK(throws<runtime_error>([] { HT_RUNTIME_ERROR << "rt"; }, "rt"));
+    CHECK(throws<hetu_exception>([] { HT_ASSERT_EQ(1, 2) << "eq"; }));
+    bool ran = false;
+    HT_ASSERT(true) << "never evaluated";
+    HT_VALUE_ERROR_IF(false) << "never";
+    ran = true;
+    CHECK(ran);
+  });
+
+  run("axis parsing and reduced shapes", [] {
+    CHECK(NDArrayMeta::ParseAxis(-1, 3) == 2 && NDArrayMeta::ParseAxis(0, 3) == 0);
+    CHECK(throws<assertion_error>([] { NDArrayMeta::ParseAxis(3, 3); }));
+    CHECK(throws<assertion_error>([] { NDArrayMeta::ParseAxis(-4, 3); }));
+    CHECK((NDArrayMeta::ParseAxes({}, 3) == HTAxes{0, 1, 2}));
+    CHECK((NDArrayMeta::ParseAxes({-1, 0, 2, 0}, 3) == HTAxes{0, 2}));
+    CHECK((NDArrayMeta::Reduce({4, 5, 6}, {1}, false) == HTShape{4, 6}));
+    CHECK((NDArrayMeta::Reduce({4, 5, 6}, {1}, true) == HTShape{4, 1, 6}));
+    CHECK((NDArrayMeta::Reduce({4, 5, 6}, {}, false) == HTShape{1}));
+    CHECK((NDArrayMeta::Reduce({4, 5, 6}, {0, -1}, false) == HTShape{5}));
+    CHECK((NDArrayMeta::Reduce({4, 5, 6}, {}, true) == HTShape{1, 1, 1}));
+  });
+
+  run("meta strides and contiguity", [] {
+    NDArrayMeta m({2, 3, 4}, kFloat32, Device(kCPU));
+    CHECK((m.stride == HTStride{12, 4, 1}) && m.is_contiguous() && m.numel() == 24);
+    m.set_stride({1, 2, 6});
+    CHECK(!m.is_contiguous());
+    CHECK(throws<assertion_error>([&] { m.set_stride({1, 2}); }));
+    NDArrayMeta one({1, 1}, kFloat32, Device(kCPU), {7, 9});
+    CHECK(one.is_contiguous());
+  });
+
+  run("dtype switch macros", [] {
+    size_t size = 0;
+    HT_DISPATCH_FLOATING_TYPES(kBFloat16, spec_t, "probe", [&]() { size = sizeof(spec_t); });
+    CHECK(size == 2);
+    HT_DISPATCH_INTEGER_AND_FLOATING_TYPES(kInt64, spec_t, "probe", [&]() { size = sizeof(spec_t); });
+    CHECK(size == 8);
+    CHECK(throws<not_implemented>(
+      [&] { HT_DISPATCH_FLOATING_TYPES(kInt32, spec_t, "probe", [&]() { size = sizeof(spec_t); }); }, "probe"));
+  });
+
+  run("host pool: allocate, borrow, free", [] {
+    auto pool = GetMemoryPool(Device(kCPU));
+    DataPtr a = pool->AllocDataSpace(100);
+    CHECK(a.ptr != nullptr && a.size >= 100 && (reinterpret_cast<uintptr_t>(a.ptr) % 64) == 0);
+    std::memset(a.ptr, 0xAB, 100);
+    pool->FreeDataSpace(a);
+    CHECK(throws<value_error>([&] { pool->FreeDataSpace(a); }));
+    DataPtr z = pool->AllocDataSpace(0);
+    CHECK(z.ptr == nullptr && z.size == 0);
+    pool->FreeDataSpace(z);
+    int deleted = 0;
+    float mine[4] = {1, 2, 3, 4};
+    DataPtr b = pool->BorrowDataSpace(mine, sizeof(mine), [&](DataPtr) { ++deleted; });
+    CHECK(b.ptr == mine);
+    pool->FreeDataSpace(b);
+    CHECK(deleted == 1 && mine[2] == 3.f);
+  });
+
+  run("host NDArray: views, permute, slice, contiguous", [] {
+    NDArray a = NDArray::empty({2, 3, 4}, Device(kCPU), kFloat32);
+    float* p = a->data_ptr<float>();
+    for (int i = 0; i < 24; ++i) p[i] = float(i);
+    NDArray v = NDArray::view(a, {6, -1});
+    CHECK((v->shape() == HTShape{6, 4}) && v->data_ptr<float>() == p);
+    CHECK(throws<value_error>([&] { NDArray::view(a, {5, -1}); }));
+    NDArray t = NDArray::permute(a, {2, 0, 1});
+    CHECK((t->shape() == HTShape{4, 2, 3}) && (t->stride() == HTStride{1, 12, 4}) && !t->is_contiguous());
+    NDArray tc = NDArray::contiguous(t);
+    CHECK(tc->is_contiguous() && tc->data_ptr<float>() != p);
+    // tc[k][i][j] = a[i][j][k]
+    for (int k = 0; k < 4; ++k)
+      for (int i = 0; i < 2; ++i)
+        for (int j = 0; j < 3; ++j) CHECK(tc->data_ptr<float>()[(k * 2 + i) * 3 + j] == float((i * 3 + j) * 4 + k));
+    NDArray s = NDArray::slice(a, {1, 1, 0}, {1, 2, 4});
+    CHECK(s->storage_offset() == 16 && s->data_ptr<float>()[0] == 16.f);
+    CHECK(throws<value_error>([&] { NDArray::slice(a, {1, 2, 0}, {1, 2, 4}); }));
+    CHECK(throws<value_error>([&] { NDArray::permute(a, {0, 0, 1}); }));
+    NDArray z = NDArray::zeros({5}, Device(kCPU), kInt64);
+    for (int i = 0; i < 5; ++i) CHECK(z->data_ptr<int64_t>()[i] == 0);
+    NDArray e = NDArray::empty({0, 7}, Device(kCPU), kFloat32);
+    CHECK(e->numel() == 0 && e->is_contiguous());
+    // a view that reaches past its storage (96 B, held in 128) is refused
+    CHECK(throws<assertion_error>([&] { NDArray::as_strided(a, {2, 3, 4}, {12, 4, 1}, 9); }));
+  });
+
+  run("device switch: host arrays have no kernels on this path", [] {
+    NDArray a = NDArray::zeros({4, 8}, Device(kCPU), kFloat32);
+    NDArray g = NDArray::zeros({8}, Device(kCPU), kFloat32);
+    CHECK(throws<not_implemented>([&] { NDArray::softmax(a, 1); }));
+    CHECK(throws<not_implemented>([&] { NDArray::sum(a, {0}); }));
+    CHECK(throws<not_implemented>([&] { NDArray::layernorm(a, g, g, {8}); }));
+    // the fused variant exists for the accelerator only: the switch itself refuses
+    CHECK(throws<not_implemented>([&] { NDArray::fused_layernorm(a, g, g, {8}); }, "cpu"));
+    NDArray lab = NDArray::zeros({4}, Device(kCPU), kInt64);
+    CHECK(throws<not_implemented>([&] { NDArray::sceloss(a, lab, int64_t(-1)); }));
+    // an accelerator kernel handed host arrays fails its device assertion
+    NDArray out = NDArray::empty_like(a);
+    CHECK(throws<assertion_error>([&] { hetu::impl::SoftmaxCuda(a, out, 1, Stream(Device(kCUDA, 0), 1)); }));
+    CHECK(throws<assertion_error>(
+      [&] { hetu::impl::ReduceCuda(a, out, {0}, kSUM, Stream(Device(kCUDA, 0), 1)); }));
+  });
+
+  // ------------------------------------------------------------------ pool policy
+  run("pool: rounding, carving small requests from one segment", [] {
+    PoolFixture f;
+    CHECK(CachingMemoryPool::RoundRequest(1) == 256 && CachingMemoryPool::RoundRequest(256) == 256 &&
+          CachingMemoryPool::RoundRequest(257) == 512);
+    DataPtr a = f.pool->AllocDataSpace(1000, f.s1), b = f.pool->AllocDataSpace(1000, f.s1);
+    CHECK(a.size == 1024 && b.size == 1024 && a.is_new_malloc && !b.is_new_malloc);
+    CHECK(static_cast<uint8_t*>(b.ptr) == static_cast<uint8_t*>(a.ptr) + 1024);
+    auto s = f.pool->stats();
+    CHECK(s.segment_allocs == 1 && s.reserved == 2 * MiB && s.allocated == 2048 && s.alloc_cnt == 2);
+    DataPtr z = f.pool->AllocDataSpace(0, f.s1);
+    CHECK(z.ptr == nullptr && z.size == 0);
+    f.pool->FreeDataSpace(z);
+    f.pool->FreeDataSpace(a);
+    f.pool->FreeDataSpace(b);
+    CHECK(throws<value_error>([&] { f.pool->FreeDataSpace(b); }, "freed twice"));
+  });
+
+  run("pool: same-stream reuse needs no event, neighbours merge back", [] {
+    PoolFixture f;
+    DataPtr a = f.pool->AllocDataSpace(4096, f.s1);
+    void* first = a.ptr;
+    f.pool->FreeDataSpace(a);
+    DataPtr b = f.pool->AllocDataSpace(4096, f.s1);
+    CHECK(b.ptr == first && f.dev->events.empty() && f.pool->stats().cache_hits == 1);
+    DataPtr c = f.pool->AllocDataSpace(8192, f.s1);
+    f.pool->FreeDataSpace(b);
+    f.pool->FreeDataSpace(c);
+    // everything merged: the whole 2 MiB segment can be handed out again
+    DataPtr whole = f.pool->AllocDataSpace(2 * MiB, f.s1);
+    CHECK(whole.ptr == first && f.pool->stats().segment_allocs == 1 && f.pool->stats().merges >= 2);
+    f.pool->FreeDataSpace(whole);
+  });
+
+  run("pool: another stream takes a cached block behind an event", [] {
+    PoolFixture f;
+    DataPtr a = f.pool->AllocDataSpace(3 * MiB, f.s1);
+    void* first = a.ptr;
+    f.pool->FreeDataSpace(a);
+    DataPtr b = f.pool->AllocDataSpace(3 * MiB, f.s2);
+    CHECK(b.ptr == first && f.pool->stats().cross_stream_takes == 1 && f.pool->stats().segment_allocs == 1);
+    CHECK(f.dev->waits.size() == 1 && f.dev->waits[0].first == f.s2.pack() && f.dev->waits[0].second == f.s1.pack());
+    // now owned by s2: freeing and reusing on s2 needs nothing more
+    f.pool->FreeDataSpace(b);
+    DataPtr c = f.pool->AllocDataSpace(3 * MiB, f.s2);
+    CHECK(c.ptr == first && f.dev->waits.size() == 1);
+    f.pool->FreeDataSpace(c);
+  });
+
+  run("pool: a block other streams used is parked until their events pass", [] {
+    PoolFixture f;
+    DataPtr a = f.pool->AllocDataSpace(4 * MiB, f.s1);
+    void* first = a.ptr;
+    f.pool->MarkDataSpaceUsedByStream(a, f.s1);   // the owner itself: nothing to record
+    CHECK(f.pool->stats().mark_cnt == 0);
+    f.pool->MarkDataSpaceUsedByStream(a, f.s2);
+    f.pool->MarkDataSpaceUsedByStream(a, f.s2);
+    f.pool->MarkDataSpaceUsedByStream(a, f.s3);
+    CHECK(f.pool->stats().mark_cnt == 2);
+    f.pool->FreeDataSpace(a);
+    CHECK(f.pool->stats().parked == 1 && f.dev->events.size() == 2);
+    DataPtr b = f.pool->AllocDataSpace(4 * MiB, f.s1);
+    CHECK(b.ptr != first && f.pool->stats().segment_allocs == 2);   // still parked
+    f.dev->events[0]->done = true;
+    DataPtr c = f.pool->AllocDataSpace(4 * MiB, f.s1);
+    CHECK(c.ptr != first);                                           // one event still pending
+    f.dev->events[1]->done = true;
+    DataPtr d = f.pool->AllocDataSpace(4 * MiB, f.s1);
+    CHECK(d.ptr == first);
+    f.pool->FreeDataSpace(b);
+    f.pool->FreeDataSpace(c);
+    f.pool->FreeDataSpace(d);
+  });
+
+  run("pool: large blocks are not split, bounded waste", [] {
+    PoolFixture f;
+    DataPtr big = f.pool->AllocDataSpace(300 * MiB, f.s1);
+    void* first = big.ptr;
+    f.pool->FreeDataSpace(big);
+    DataPtr small = f.pool->AllocDataSpace(100 * MiB, f.s1);     // would waste 200 MiB: new segment
+    CHECK(small.ptr != first);
+    DataPtr close = f.pool->AllocDataSpace(290 * MiB, f.s1);     // wastes 10 MiB <= 20 MiB: whole block
+    CHECK(close.ptr == first && close.size == 300 * MiB);
+    f.pool->FreeDataSpace(small);
+    // 100 MiB <= max split: it is split for a 10 MiB request
+    DataPtr part = f.pool->AllocDataSpace(10 * MiB, f.s1);
+    CHECK(part.ptr == small.ptr && part.size == 10 * MiB);
+    f.pool->FreeDataSpace(part);
+    f.pool->FreeDataSpace(close);
+  });
+
+  run("pool: out of memory releases the cache and retries, then reports", [] {
+    PoolFixture f(/*capacity=*/64 * MiB);
+    DataPtr a = f.pool->AllocDataSpace(40 * MiB, f.s1);
+    f.pool->FreeDataSpace(a);
+    // cached 40 MiB on s1 does not fit a 50 MiB request; the device has 24 MiB left
+    DataPtr b = f.pool->AllocDataSpace(50 * MiB, f.s1);
+    CHECK(b.ptr != nullptr && f.pool->stats().retries_after_oom == 1 && f.pool->stats().segment_frees == 1);
+    CHECK(f.dev->device_syncs >= 1 && f.dev->in_use == 50 * MiB);
+    CHECK(throws<runtime_error>([&] { f.pool->AllocDataSpace(32 * MiB, f.s1); }, "out of memory"));
+    f.pool->FreeDataSpace(b);
+    f.pool->EmptyCache();
+    CHECK(f.pool->stats().reserved == 0 && f.dev->in_use == 0 && f.dev->live.empty());
+  });
+
+  run("pool: EmptyCache waits for parked blocks and keeps live ones", [] {
+    PoolFixture f;
+    DataPtr keep = f.pool->AllocDataSpace(5 * MiB, f.s1);
+    DataPtr gone = f.pool->AllocDataSpace(5 * MiB, f.s1);
+    f.pool->MarkDataSpaceUsedByStream(gone, f.s2);
+    f.pool->FreeDataSpace(gone);
+    f.pool->EmptyCache();
+    auto s = f.pool->stats();
+    CHECK(s.reserved == 6 * MiB && s.allocated == 5 * MiB && f.dev->live.size() == 1);
+    f.pool->FreeDataSpace(keep);
+  });
+
+  run("pool: borrowed memory runs its deleter once, after marked streams drain", [] {
+    PoolFixture f;
+    int deleted = 0;
+    char mine[64];
+    DataPtr b = f.pool->BorrowDataSpace(mine, sizeof(mine), [&](DataPtr) { ++deleted; });
+    f.pool->MarkDataSpaceUsedByStream(b, f.s2);
+    f.pool->FreeDataSpace(b);
+    CHECK(deleted == 1 && f.dev->stream_syncs == 1 && f.pool->stats().reserved == 0);
+    CHECK(throws<value_error>([&] { f.pool->BorrowDataSpace(nullptr, 8, nullptr); }));
+  });
+
+  run("pool: WaitDataSpace drains owner and user streams", [] {
+    PoolFixture f;
+    DataPtr a = f.pool->AllocDataSpace(1 * MiB, f.s1);
+    f.pool->MarkDataSpaceUsedByStream(a, f.s3);
+    f.pool->WaitDataSpace(a, false).get();
+    CHECK(f.dev->stream_syncs == 2);
+    f.pool->WaitDataSpace(a, true).get();
+    CHECK(f.dev->stream_syncs == 4);
+    f.pool->FreeDataSpace(a);
+  });
+
+  run("pool: randomized alloc/free never overlaps live blocks", [] {
+    PoolFixture f(/*capacity=*/512 * MiB, /*max_split=*/16 * MiB, /*max_frag=*/2 * MiB);
+    f.dev->auto_complete = true;
+    struct Live { DataPtr p; };
+    std::vector<Live> live;
+    uint64_t rng = 0x9E3779B97F4A7C15ull;
+    auto next = [&] { rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17; return rng; };
+    const Stream streams[3] = {f.s1, f.s2, f.s3};
+    for (int step = 0; step < 4000; ++step) {
+      const bool do_alloc = live.empty() || (next() % 100 < 55 && live.size() < 64);
+      if (do_alloc) {
+        const size_t cls = next() % 3;
+        const size_t bytes = cls == 0 ? 1 + next() % 4096 : cls == 1 ? 1 + next() % (3 * MiB) : 1 + next() % (24 * MiB);
+        DataPtr p;
+        try {
+          p = f.pool->AllocDataSpace(bytes, streams[next() % 3]);
+        } catch (const runtime_error&) {
+          continue;   // scripted device full: allowed
+        }
+        CHECK(p.size >= bytes && reinterpret_cast<uintptr_t>(p.ptr) % 256 == 0);
+        for (auto& l : live) {
+          auto* a0 = static_cast<uint8_t*>(l.p.ptr);
+          auto* b0 = static_cast<uint8_t*>(p.ptr);
+          CHECK(a0 + l.p.size <= b0 || b0 + p.size <= a0);
+        }
+        if (next() % 4 == 0) f.pool->MarkDataSpaceUsedByStream(p, streams[next() % 3]);
+        live.push_back({p});
+      } else {
+        const size_t i = next() % live.size();
+        f.pool->FreeDataSpace(live[i].p);
+        live[i] = live.back();
+        live.pop_back();
+      }
+    }
+    size_t sum = 0;
+    for (auto& l : live) sum += l.p.size;
+    CHECK(f.pool->stats().allocated == sum && f.pool->stats().reserved >= sum);
+    for (auto& l : live) f.pool->FreeDataSpace(l.p);
+    f.pool->EmptyCache();
+    CHECK(f.pool->stats().allocated == 0 && f.pool->stats().reserved == 0 && f.dev->live.empty());
+  });
+
+  run("pool knobs from the environment", [] {
+    setenv("HETU_TEST_KNOB_MB", "64", 1);
+    CHECK(hetu::impl::ParsePoolKnobMB("HETU_TEST_KNOB_MB", 200) == 64 * MiB);
+    setenv("HETU_TEST_KNOB_MB", "sixty", 1);
+    CHECK(hetu::impl::ParsePoolKnobMB("HETU_TEST_KNOB_MB", 200) == 200 * MiB);
+    setenv("HETU_TEST_KNOB_MB", "-3", 1);
+    CHECK(hetu::impl::ParsePoolKnobMB("HETU_TEST_KNOB_MB", 20) == 20 * MiB);
+    unsetenv("HETU_TEST_KNOB_MB");
+    CHECK(hetu::impl::ParsePoolKnobMB("HETU_TEST_KNOB_MB", 20) == 20 * MiB);
+  });
+
+  std::printf("%d checks, %d failed\n", g_run, g_failed);
+  return g_failed;
+}

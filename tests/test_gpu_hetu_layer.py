@@ -1,0 +1,463 @@
+"""GPU parity of the C++ operator layer (hetu::impl::<Kernel>Cuda entry points and
+the NDArray statics) against the oracle, called through include/hetu_ops_c.h with
+torch tensors as borrowed arrays.  The layer runs on its own HIP streams, so each
+test drains torch's stream before the call and the layer's stream after it."""
+import importlib
+
+import numpy as np
+import pytest
+
+import helpers
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops(hk):
+    return importlib.import_module("hotspa-ae_amd.hetu_ops")
+
+
+def _sync_in():
+    import torch
+    torch.cuda.synchronize()
+
+
+def _dev(vals, dtype, cuda):
+    return [helpers.to_torch(v, dtype, cuda) for v in vals]
+
+
+def _norm_inputs(shape, cols, dtype, seed):
+    x = helpers.draw(seed, shape, dtype=dtype)
+    gamma = helpers.draw(seed + 1, (cols,), "uniform", 0.5, 1.5, dtype)
+    beta = helpers.draw(seed + 2, (cols,), "normal", 0.0, 0.1, dtype)
+    dy = helpers.draw(seed + 3, shape, dtype=dtype)
+    return x, gamma, beta, dy
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("shape,reduce_dims", [((6, 5, 256), 1), ((3, 4, 16, 64), 2), ((33, 1000), 1)])
+def test_layer_norm_and_gradient(ops, cuda, dtype, shape, reduce_dims):
+    import torch
+    cols = int(np.prod(shape[len(shape) - reduce_dims:]))
+    rows = int(np.prod(shape)) // cols
+    eps = 1e-5
+    x, gamma, beta, dy = _norm_inputs(shape, cols, dtype, 11 + cols)
+    ey, emean, evar, erstd = oracle.layernorm_fwd(x.reshape(rows, cols), gamma, beta, eps)
+    tx, tg, tb, tdy = _dev((x, gamma, beta, dy), dtype, cuda)
+    tg = tg.reshape(shape[len(shape) - reduce_dims:])
+    tb = tb.reshape(shape[len(shape) - reduce_dims:])
+    stat_shape = tuple(shape[:len(shape) - reduce_dims]) + (1,) * reduce_dims
+    ty = torch.empty_like(tx)
+    tmean = torch.empty(stat_shape, dtype=tx.dtype, device=cuda)
+    tvar = torch.empty(stat_shape, dtype=tx.dtype, device=cuda)
+    _sync_in()
+    ops.layer_norm(tx, tg, tb, tmean, tvar, ty, reduce_dims, eps)
+    ops.stream_sync()
+    helpers.assert_close(ty, ey.reshape(shape), dtype, "y")
+    helpers.assert_close(tvar.reshape(rows), evar, dtype, "var")
+    # gradient from the statistics the forward stored (rounded to the data dtype, as the reference keeps them)
+    mean_r = helpers.to_numpy(tmean).reshape(rows).astype(np.float64)
+    var_r = helpers.to_numpy(tvar).reshape(rows).astype(np.float64)
+    rstd_r = 1.0 / np.sqrt(var_r + eps)
+    edx, edg, edb = oracle.layernorm_bwd(dy.reshape(rows, cols), x.reshape(rows, cols), gamma,
+                                         mean_r.astype(np.float32), rstd_r.astype(np.float32))
+    tdx = torch.empty_like(tx)
+    tdg = torch.empty_like(tg)
+    tdb = torch.empty_like(tg)
+    _sync_in()
+    ops.layer_norm_gradient(tdy, tx, tg, tdx, tdg, tdb, tmean, tvar, reduce_dims, eps)
+    ops.stream_sync()
+    helpers.assert_close(tdx, edx.reshape(shape), dtype, "dx")
+    helpers.assert_close(tdg.reshape(cols), edg, dtype, "dscale")
+    helpers.assert_close(tdb.reshape(cols), edb, dtype, "dbias")
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("inplace", [False, True])
+def test_fused_layer_norm_and_gradient(ops, cuda, dtype, inplace):
+    import torch
+    shape, cols = (4, 9, 512), 512
+    rows = 36
+    eps = 1e-5
+    x, gamma, beta, dy = _norm_inputs(shape, cols, dtype, 77)
+    ey, emean, _, erstd = oracle.layernorm_fwd(x.reshape(rows, cols), gamma, beta, eps)
+    tx, tg, tb, tdy = _dev((x, gamma, beta, dy), dtype, cuda)
+    ty = torch.empty_like(tx)
+    tmean = torch.empty((4, 9, 1), dtype=torch.float32, device=cuda)
+    trstd = torch.empty((4, 9, 1), dtype=torch.float32, device=cuda)
+    _sync_in()
+    ops.fused_layer_norm(tx, tg, tb, tmean, trstd, ty, 1, eps)
+    ops.stream_sync()
+    helpers.assert_close(ty, ey.reshape(shape), dtype, "y")
+    helpers.assert_close(trstd.reshape(rows), erstd, "fp32", "rstd")
+    mean32 = helpers.to_numpy(tmean).reshape(rows)
+    rstd32 = helpers.to_numpy(trstd).reshape(rows)
+    tdx, tdg, tdb = torch.empty_like(tx), torch.empty_like(tg), torch.empty_like(tg)
+    if inplace:
+        y_stored = helpers.to_numpy(ty).reshape(rows, cols)
+        edx, edg, edb = oracle.layernorm_bwd_memeff(dy.reshape(rows, cols), y_stored, gamma, beta, rstd32, eps)
+        _sync_in()
+        ops.fused_layer_norm_gradient(tdy, ty, tg, tb, tdx, tdg, tdb, tmean, trstd, 1, eps, True)
+    else:
+        edx, edg, edb = oracle.layernorm_bwd(dy.reshape(rows, cols), x.reshape(rows, cols), gamma, mean32, rstd32,
+                                             eps, clamp_gamma=True)
+        _sync_in()
+        ops.fused_layer_norm_gradient(tdy, tx, tg, tb, tdx, tdg, tdb, tmean, trstd, 1, eps, False)
+    ops.stream_sync()
+    helpers.assert_close(tdx, edx.reshape(shape), dtype, "dx")
+    helpers.assert_close(tdg, edg, dtype, "dscale")
+    helpers.assert_close(tdb, edb, dtype, "dbias")
+    # statistics must be float32 for the fused variant
+    with pytest.raises(ops.AssertionError_, match="float32"):
+        ops.fused_layer_norm(tx, tg, tb, tmean.to(tx.dtype) if dtype != "fp32" else tmean.double(), trstd, ty, 1, eps)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("is_rms", [True, False])
+@pytest.mark.parametrize("with_residual", [False, True])
+def test_dropout_add_ln(ops, cuda, dtype, is_rms, with_residual):
+    import torch
+    rows, cols = 48, 4096
+    eps = 1e-6
+    x0, gamma, beta, dz = _norm_inputs((rows, cols), cols, dtype, 300 + int(is_rms))
+    res = helpers.draw(305, (rows, cols), dtype=dtype) if with_residual else None
+    ez, ex, emu, ers = oracle.dropout_add_ln_fwd(x0, res, gamma, None if is_rms else beta, eps, is_rms)
+    tx0, tg, tb, tdz = _dev((x0, gamma, beta, dz), dtype, cuda)
+    tres = helpers.to_torch(res, dtype, cuda) if with_residual else None
+    tz = torch.empty_like(tx0)
+    tx = torch.empty_like(tx0) if with_residual else None
+    tmu = torch.empty(rows, dtype=torch.float32, device=cuda)
+    trs = torch.empty(rows, dtype=torch.float32, device=cuda)
+    _sync_in()
+    ops.dropout_add_ln_fwd(tx0, tres, tg, None if is_rms else tb, tz, tx, tmu, trs, eps, is_rms)
+    ops.stream_sync()
+    helpers.assert_close(tz, ez, dtype, "z")
+    helpers.assert_close(trs, ers, "fp32", "rsigma")
+    if with_residual:
+        helpers.assert_close(tx, ex, dtype, "x")
+    x_saved = helpers.to_numpy(tx) if with_residual else x0
+    mu32, rs32 = helpers.to_numpy(tmu), helpers.to_numpy(trs)
+    edx0, edg, edb = oracle.dropout_add_ln_bwd(dz, None, x_saved, mu32, rs32, gamma, is_rms)
+    tdx0 = torch.empty_like(tx0)
+    tdres = torch.empty_like(tx0) if with_residual else None
+    tdg, tdb = torch.empty_like(tg), torch.empty_like(tg)
+    _sync_in()
+    ops.dropout_add_ln_bwd(tdz, None, tx if with_residual else tx0, tmu, trs, tg, tdx0, tdres, tdg, tdb,
+                           with_residual, is_rms)
+    ops.stream_sync()
+    helpers.assert_close(tdx0, edx0, dtype, "dx0")
+    helpers.assert_close(tdg, edg, dtype, "dgamma")
+    helpers.assert_close(tdb, edb, dtype, "dbeta")
+    if with_residual:
+        helpers.assert_close(tdres, edx0, dtype, "dresidual")
+
+
+def test_dropout_add_ln_refuses_what_it_does_not_compute(ops, cuda):
+    import torch
+    rows, cols = 8, 256
+    x0 = torch.zeros(rows, cols, device=cuda)
+    g = torch.ones(cols, device=cuda)
+    z = torch.empty_like(x0)
+    mu = torch.empty(rows, device=cuda)
+    rs = torch.empty(rows, device=cuda)
+    _sync_in()
+    with pytest.raises(ops.NotImplemented_, match="dropout"):
+        ops.dropout_add_ln_fwd(x0, None, g, None, z, None, mu, rs, 1e-6, True, dropout_p=0.1)
+    with pytest.raises(ops.NotImplemented_, match="scaling"):
+        ops.dropout_add_ln_fwd(x0, None, g, None, z, None, mu, rs, 1e-6, True, colscale=g)
+    with pytest.raises(ops.AssertionError_, match="multiple of 8"):
+        ops.dropout_add_ln_fwd(x0[:, :252].contiguous(), None, g[:252].contiguous(), None,
+                               z[:, :252].contiguous(), None, mu, rs, 1e-6, True)
+    with pytest.raises(ops.AssertionError_):     # x0 must be dense
+        ops.dropout_add_ln_fwd(x0.t(), None, g, None, z, None, mu, rs, 1e-6, True)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("shape,dim", [((4, 6, 300), -1), ((5, 64, 33), 1), ((16, 2048), 1), ((7, 3, 5, 9), 0)])
+def test_softmax_and_gradient(ops, cuda, dtype, shape, dim):
+    import torch
+    x = helpers.draw(51, shape, "normal", 0.0, 2.0, dtype)
+    dy = helpers.draw(52, shape, dtype=dtype)
+    ey = oracle.softmax_fwd(x, dim)
+    tx, tdy = _dev((x, dy), dtype, cuda)
+    ty = torch.empty_like(tx)
+    _sync_in()
+    ops.softmax(tx, ty, dim)
+    ops.stream_sync()
+    helpers.assert_close(ty, ey, dtype, "y")
+    y_stored = helpers.to_numpy(ty)
+    edx = oracle.softmax_bwd(y_stored, dy, dim)
+    tdx = torch.empty_like(tx)
+    _sync_in()
+    ops.softmax_gradient(ty, tdy, tdx, dim)
+    ops.stream_sync()
+    helpers.assert_close(tdx, edx, dtype, "dx")
+
+
+def test_softmax_of_a_permuted_view(ops, cuda):
+    """Inputs of any stride are accepted (made dense inside); outputs must be dense."""
+    import torch
+    x = helpers.draw(61, (12, 40, 24), "normal", 0.0, 2.0, "fp32")
+    tx = helpers.to_torch(x, "fp32", cuda).permute(2, 0, 1)       # [24, 12, 40], not dense
+    ey = oracle.softmax_fwd(np.ascontiguousarray(x.transpose(2, 0, 1)), -1)
+    ty = torch.empty((24, 12, 40), device=cuda)
+    _sync_in()
+    ops.softmax(tx, ty, -1)
+    ops.stream_sync()
+    helpers.assert_close(ty, ey, "fp32", "y")
+    with pytest.raises(ops.AssertionError_, match="not contiguous"):
+        ops.softmax(tx, torch.empty((12, 40, 24), device=cuda).permute(2, 0, 1), -1)
+    with pytest.raises(ops.AssertionError_, match="Invalid dimension"):
+        ops.softmax(tx, ty, 3)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_sparse_cross_entropy_and_gradient(ops, cuda, dtype):
+    import torch
+    shape, cols = (6, 11, 1000), 1000
+    rows = 66
+    ignored = -100
+    x = helpers.draw(71, shape, "normal", 0.0, 3.0, dtype)
+    g = helpers.rng(72)
+    labels = g.integers(0, cols, size=shape[:-1]).astype(np.int64)
+    labels.reshape(-1)[::7] = ignored
+    gl = helpers.draw(73, shape[:-1], dtype=dtype)
+    eloss = oracle.sce_sparse_fwd(x.reshape(rows, cols), labels.reshape(rows), ignored)
+    egrad = oracle.sce_sparse_bwd(x.reshape(rows, cols), labels.reshape(rows), gl.reshape(rows), ignored)
+    tx, tgl = _dev((x, gl), dtype, cuda)
+    tl = torch.from_numpy(labels).to(cuda)
+    tloss = torch.empty(shape[:-1], dtype=tx.dtype, device=cuda)
+    tgrad = torch.empty_like(tx)
+    _sync_in()
+    ops.softmax_cross_entropy_sparse(tx, tl, tloss, ignored)
+    ops.softmax_cross_entropy_sparse_gradient(tx, tl, tgl, tgrad, ignored)
+    ops.stream_sync()
+    helpers.assert_close(tloss.reshape(rows), eloss, dtype, "loss")
+    helpers.assert_close(tgrad.reshape(rows, cols), egrad, dtype, "grad")
+    got = helpers.to_numpy(tloss).reshape(rows)
+    assert np.all(got[labels.reshape(rows) == ignored] == 0.0)
+    assert np.all(helpers.to_numpy(tgrad).reshape(rows, cols)[labels.reshape(rows) == ignored] == 0.0)
+    with pytest.raises(ops.AssertionError_, match="int64"):
+        ops.softmax_cross_entropy_sparse(tx, tl.int(), tloss, ignored)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_dense_cross_entropy_and_gradient(ops, cuda, dtype):
+    import torch
+    rows, cols = 40, 777
+    x = helpers.draw(81, (rows, cols), "normal", 0.0, 3.0, dtype)
+    lab = helpers.rng(82).random((rows, cols)).astype(np.float32)
+    lab = oracle.round_to(lab / lab.sum(axis=1, keepdims=True), dtype)
+    gl = helpers.draw(83, (rows,), dtype=dtype)
+    eloss = oracle.sce_dense_fwd(x, lab)
+    egrad = oracle.sce_dense_bwd(x, lab, gl)
+    tx, tlab, tgl = _dev((x, lab, gl), dtype, cuda)
+    tloss = torch.empty(rows, dtype=tx.dtype, device=cuda)
+    tgrad = torch.empty_like(tx)
+    _sync_in()
+    ops.softmax_cross_entropy(tx, tlab, tloss)
+    ops.softmax_cross_entropy_gradient(tx, tlab, tgl, tgrad)
+    ops.stream_sync()
+    helpers.assert_close(tloss, eloss, dtype, "loss")
+    helpers.assert_close(tgrad, egrad, dtype, "grad")
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp64", "int64"])
+@pytest.mark.parametrize("axes", [[0], [1], [-1], [0, 2], [], [2, 0, 0]])
+@pytest.mark.parametrize("red", ["sum", "mean"])
+def test_reduce_kernel_entry(ops, cuda, dtype, axes, red):
+    import torch
+    shape = (9, 130, 24)
+    if dtype == "int64":
+        x = helpers.rng(91).integers(-1000, 1000, size=shape).astype(np.int64)
+        tx = torch.from_numpy(x).to(cuda)
+    else:
+        x = helpers.draw(91, shape, dtype=dtype if dtype != "fp64" else "fp32")
+        tx = helpers.to_torch(x, dtype, cuda)
+    nd = len(shape)
+    norm_axes = sorted(set(a % nd for a in axes)) if axes else list(range(nd))
+    out_shape = [s for i, s in enumerate(shape) if i not in norm_axes] or [1]
+    tout = torch.empty(out_shape, dtype=tx.dtype, device=cuda)
+    _sync_in()
+    ops.reduce(tx, tout, axes, red)
+    ops.stream_sync()
+    if dtype == "int64":
+        e = x.sum(axis=tuple(norm_axes))
+        if red == "mean":
+            n = int(np.prod([shape[a] for a in norm_axes]))
+            # integer mean: the sum times float(1/n), truncated back to the integer type
+            e = (e.astype(np.float64) * float(np.float32(1.0) / np.float32(n))).astype(np.int64)
+            assert np.all(np.abs(tout.cpu().numpy().reshape(e.shape) - e) <= 1)
+        else:
+            assert np.array_equal(tout.cpu().numpy().reshape(e.shape), e)
+    else:
+        e = oracle.reduce(x, norm_axes, red)
+        # the mean is the sum times float(1/n): its factor carries fp32 rounding even for fp64 data
+        rtol = 1e-6 if (dtype == "fp64" and red == "mean") else None
+        helpers.assert_close(tout, np.asarray(e).reshape(out_shape), dtype, "%s over %s" % (red, axes), rtol=rtol)
+
+
+def test_reduce_rejects_what_is_not_on_the_path(ops, cuda):
+    import torch
+    x = torch.ones(4, 8, device=cuda)
+    _sync_in()
+    with pytest.raises(ops.NotImplemented_, match="max"):
+        ops.reduce(x, torch.empty(8, device=cuda), [0], "max")
+    with pytest.raises(ops.NotImplemented_, match="none"):
+        ops.reduce(x, torch.empty(8, device=cuda), [0], "none")
+    with pytest.raises(ops.AssertionError_, match="Invalid dimension"):
+        ops.reduce(x, torch.empty(8, device=cuda), [2], "sum")
+    with pytest.raises(ops.AssertionError_, match="kept elements"):
+        ops.reduce(x, torch.empty(5, device=cuda), [0], "sum")
+
+
+def test_reduce_of_a_strided_view_needs_no_copy(ops, cuda):
+    import torch
+    x = helpers.draw(95, (64, 48, 20), dtype="fp32")
+    tx = helpers.to_torch(x, "fp32", cuda)
+    view = tx.permute(1, 2, 0)[:, ::2, :]            # [48, 10, 64], strides (20, 2, 960)
+    e = np.ascontiguousarray(x.transpose(1, 2, 0)[:, ::2, :]).astype(np.float64).sum(axis=(0, 2))
+    tout = torch.empty(10, device=cuda)
+    before = ops.pool_stats()["alloc_cnt"]
+    _sync_in()
+    ops.reduce(view, tout, [0, 2], "sum")
+    ops.stream_sync()
+    helpers.assert_close(tout, e, "fp32", "strided sum")
+    assert ops.pool_stats()["alloc_cnt"] - before <= 1      # at most the partials scratch, never a dense copy of x
+
+
+def test_ndarray_statics_allocate_and_dispatch(ops, cuda):
+    import torch
+    dtype = "bf16"
+    shape, cols = (8, 16, 1024), 1024
+    rows = 128
+    x, gamma, beta, _ = _norm_inputs(shape, cols, dtype, 400)
+    tx, tg, tb = _dev((x, gamma, beta), dtype, cuda)
+    _sync_in()
+    # reduce: sum / mean with keepdims
+    tsum = torch.empty((8, 1, 1024), dtype=tx.dtype, device=cuda)
+    ops.ndarray_reduce(tx, "mean", [1], True, tsum)
+    helpers.assert_close(tsum, np.asarray(oracle.reduce(x, [1], "mean")).reshape(8, 1, 1024), dtype, "mean")
+    # softmax
+    tsm = torch.empty_like(tx)
+    ops.ndarray_softmax(tx, -1, tsm)
+    helpers.assert_close(tsm, oracle.softmax_fwd(x, -1), dtype, "softmax")
+    # layernorm (stats in the data dtype) and fused layernorm (fp32 stats)
+    ey, emean, evar, erstd = oracle.layernorm_fwd(x.reshape(rows, cols), gamma, beta, 1e-5)
+    ty = torch.empty_like(tx)
+    tmean = torch.empty((8, 16, 1), dtype=tx.dtype, device=cuda)
+    tvar = torch.empty((8, 16, 1), dtype=tx.dtype, device=cuda)
+    ops.ndarray_layernorm(tx, tg, tb, 1, 1e-5, False, ty, tmean, tvar)
+    helpers.assert_close(ty, ey.reshape(shape), dtype, "layernorm")
+    helpers.assert_close(tvar.reshape(rows), evar, dtype, "var")
+    tmean32 = torch.empty((8, 16, 1), dtype=torch.float32, device=cuda)
+    trstd32 = torch.empty((8, 16, 1), dtype=torch.float32, device=cuda)
+    ops.ndarray_layernorm(tx, tg, tb, 1, 1e-5, True, ty, tmean32, trstd32)
+    helpers.assert_close(ty, ey.reshape(shape), dtype, "fused layernorm")
+    helpers.assert_close(trstd32.reshape(rows), erstd, "fp32", "rstd")
+
+
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
+def test_ndarray_sceloss_reductions(ops, cuda, reduction):
+    """kMEAN divides by ALL rows, ignored ones included (it is a plain mean over the per-row losses)."""
+    import torch
+    rows, cols, ignored = 96, 512, -1
+    x = helpers.draw(500, (rows, cols), "normal", 0.0, 2.0, "fp32")
+    labels = helpers.rng(501).integers(0, cols, size=rows).astype(np.int64)
+    labels[::5] = ignored
+    per_row = oracle.sce_sparse_fwd(x, labels, ignored)
+    tx = helpers.to_torch(x, "fp32", cuda)
+    tl = torch.from_numpy(labels).to(cuda)
+    _sync_in()
+    if reduction == "none":
+        out = torch.empty(rows, device=cuda)
+        ops.ndarray_sceloss(tx, tl, out, "none", ignored_index=ignored)
+        helpers.assert_close(out, per_row, "fp32", "per-row loss")
+    else:
+        out = torch.empty(1, device=cuda)
+        ops.ndarray_sceloss(tx, tl, out, reduction, ignored_index=ignored)
+        e = per_row.sum() / rows if reduction == "mean" else per_row.sum()
+        helpers.assert_close(out, np.array([e]), "fp32", reduction)
+    # dense labels through the same static
+    lab = np.zeros((rows, cols), dtype=np.float32)
+    keep = labels != ignored
+    lab[np.arange(rows)[keep], labels[keep]] = 1.0
+    out = torch.empty(rows, device=cuda)
+    ops.ndarray_sceloss(tx, helpers.to_torch(lab, "fp32", cuda), out, "none")
+    helpers.assert_close(out, per_row, "fp32", "one-hot dense labels equal sparse labels")
+
+
+def test_empty_arrays_are_no_ops(ops, cuda):
+    import torch
+    x = torch.empty((0, 64), device=cuda)
+    g = torch.ones(64, device=cuda)
+    _sync_in()
+    ops.softmax(x, torch.empty_like(x), -1)
+    ops.layer_norm(x, g, g, torch.empty((0, 1), device=cuda), torch.empty((0, 1), device=cuda),
+                   torch.empty_like(x), 1, 1e-5)
+    dg = torch.full((64,), 7.0, device=cuda)
+    db = torch.full((64,), 7.0, device=cuda)
+    _sync_in()
+    ops.layer_norm_gradient(x, x, g, torch.empty_like(x), dg, db, torch.empty((0, 1), device=cuda),
+                            torch.empty((0, 1), device=cuda), 1, 1e-5)
+    ops.stream_sync()
+    assert float(dg.abs().sum()) == 0.0 and float(db.abs().sum()) == 0.0     # empty column sums
+    ops.softmax_cross_entropy_sparse(x, torch.empty(0, dtype=torch.int64, device=cuda),
+                                     torch.empty(0, device=cuda), -1)
+    out = torch.full((64,), 3.0, device=cuda)
+    _sync_in()
+    ops.reduce(x, out, [0], "sum")
+    ops.stream_sync()
+    assert float(out.abs().sum()) == 0.0
+
+
+def test_device_pool_reuses_and_orders_across_streams(ops, cuda):
+    """The real pool on the GPU: same-stream reuse, cross-stream take, parking, EmptyCache."""
+    ops.synchronize_all()
+    ops.pool_empty_cache()
+    s0 = ops.pool_stats()
+    a = ops.pool_alloc(5 << 20, stream=1)
+    assert a.ptr % 256 == 0 and a.size == 5 << 20
+    ops.pool_free(a)
+    b = ops.pool_alloc(5 << 20, stream=1)
+    assert b.ptr == a.ptr
+    ops.pool_free(b)
+    c = ops.pool_alloc(5 << 20, stream=2)                # taken from stream 1's cache behind an event
+    assert c.ptr == a.ptr
+    ops.pool_mark_used(c, 3)
+    ops.pool_free(c)                                     # parked behind an event on stream 3 (idle: passes at once)
+    d = ops.pool_alloc(5 << 20, stream=2)
+    s1 = ops.pool_stats()
+    assert s1["segment_allocs"] - s0["segment_allocs"] <= 2
+    assert s1["cross_stream_takes"] - s0["cross_stream_takes"] >= 1
+    assert s1["parked"] - s0["parked"] == 1
+    ops.pool_free(d)
+    small = [ops.pool_alloc(1000, stream=1) for _ in range(8)]
+    assert len({blk.ptr for blk in small}) == 8
+    assert max(blk.ptr for blk in small) - min(blk.ptr for blk in small) < (2 << 20)    # one segment
+    for blk in small:
+        ops.pool_free(blk)
+    with pytest.raises(ops.ValueError_, match="freed twice"):
+        ops.pool_free(small[0])
+    ops.pool_empty_cache()
+    s2 = ops.pool_stats()
+    assert s2["allocated"] == 0 and s2["reserved"] == 0
+
+
+def test_operators_leave_no_memory_behind(ops, cuda):
+    import torch
+    x = torch.randn(256, 4096, device=cuda, dtype=torch.bfloat16)
+    g = torch.ones(4096, device=cuda, dtype=torch.bfloat16)
+    dx, dg, db = torch.empty_like(x), torch.empty_like(g), torch.empty_like(g)
+    mu = torch.empty(256, device=cuda)
+    rs = torch.empty(256, device=cuda)
+    z = torch.empty_like(x)
+    _sync_in()
+    for _ in range(3):
+        ops.dropout_add_ln_fwd(x, None, g, None, z, None, mu, rs, 1e-6, True)
+        ops.dropout_add_ln_bwd(x, None, x, mu, rs, g, dx, None, dg, db, False, True)
+    ops.stream_sync()
+    s = ops.pool_stats()
+    assert s["allocated"] == 0                 # scratch went back to the pool
+    assert s["cache_hits"] >= 2                # and was reused by the later iterations

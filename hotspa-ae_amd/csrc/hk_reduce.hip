@@ -590,8 +590,20 @@ int hk_reduce(int in_dtype, int out_dtype, const void* in, void* out, int ndim, 
   ReducePlan p;
   int rc = make_plan(ndim, shape, strides, naxes, axes, &p, "hk_reduce");
   if (rc != HK_OK) return rc;
-  if (naxes == 0 || p.kind == PLAN_EMPTY) return HK_OK;   // nothing to reduce / nothing to write
-  HK_REQUIRE(in && out, HK_ERR_INVALID, "hk_reduce: null input/output");
+  if (p.kind == PLAN_EMPTY) return HK_OK;   // nothing to write
+  HK_REQUIRE(out, HK_ERR_INVALID, "hk_reduce: null output");
+  if (naxes == 0) {   // nothing to reduce: the dense copy of the input
+    HK_REQUIRE(out_dtype == in_dtype, HK_ERR_UNSUPPORTED, "hk_reduce: a reduction over no axes cannot change the dtype");
+    return hk_strided_copy(in_dtype, in, out, ndim, shape, strides, stream);
+  }
+  if (p.n_red == 0) {
+    // empty sums are 0; an empty mean is 0 * (1/0) = NaN for floating types (all-ones bytes are a NaN in each)
+    const bool floating = out_dtype == HK_FLOAT16 || out_dtype == HK_BFLOAT16 || out_dtype == HK_FLOAT32 || out_dtype == HK_FLOAT64;
+    const size_t es = dtype_size(out_dtype);
+    HK_REQUIRE(es > 0, HK_ERR_UNSUPPORTED, "hk_reduce: dtype %d not implemented", out_dtype);
+    return hk_memset(out, (op == HK_REDUCE_MEAN && floating) ? 0xFF : 0, size_t(p.n_out) * es, stream);
+  }
+  HK_REQUIRE(in, HK_ERR_INVALID, "hk_reduce: null input");
   HK_REQUIRE((p.n_out + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_reduce: output too large");
   const int is_mean = op == HK_REDUCE_MEAN;
   const float factor = is_mean ? 1.0f / float(size_t(p.n_red)) : 1.0f;

@@ -234,6 +234,8 @@ HK_API int hk_sce_dense_bwd(int dtype, const void* logits, const void* labels,
  * kept dims in their original order.  bf16 / fp16 accumulate in fp32; mean is
  * sum * (1.0f / reduce_num) (hetu/impl/kernel/ReduceMean.cu:9-33).
  * out_dtype may be HK_FLOAT32 for bf16 / fp16 input (ReduceSum.cu:28-37).
+ * naxes = 0 writes the dense copy of the input; a reduced extent of 0 writes
+ * the empty sum 0 (mean: NaN for floating types); no kept element, no write.
  * Replaces ReduceSumCuda / ReduceMeanCuda (ReduceSum.cu:25-42,
  * ReduceMean.cu:35-55) and launch_reduce_kernel (Reduce.cuh:757-844).
  * ======================================================================== */

@@ -103,3 +103,26 @@ def test_full_size_configs(hk, cuda):
     # linearity: sum(2x) == 2 sum(x) exactly in bf16 (scaling by two is exact)
     got2 = _run(hk, cuda, (tx * 2), (0,), "sum")
     assert torch.equal(got2.float(), _run(hk, cuda, tx, (0,), "sum").float() * 2)
+
+
+def test_degenerate_reductions(hk, cuda):
+    """No axes = a dense copy (also of a strided view); a reduced extent of 0 gives
+    the empty sum 0 and the empty mean NaN; nothing kept = nothing written."""
+    import torch
+    x = helpers.draw(11, (6, 10), dtype="fp32")
+    tx = helpers.to_torch(x, "fp32", cuda)
+    got = _run(hk, cuda, tx, (), "sum")
+    assert np.array_equal(helpers.to_numpy(got), x)
+    view = tx.t()
+    out = torch.full((10, 6), -7.0, device=cuda)
+    hk.reduce(view, out, [], "sum")
+    torch.cuda.synchronize()
+    assert np.array_equal(helpers.to_numpy(out), x.T)
+    empty = torch.empty((0, 10), device=cuda)
+    assert np.array_equal(helpers.to_numpy(_run(hk, cuda, empty, (0,), "sum")), np.zeros(10, dtype=np.float32))
+    assert np.all(np.isnan(helpers.to_numpy(_run(hk, cuda, empty, (0,), "mean"))))
+    assert np.all(np.isnan(helpers.to_numpy(_run(hk, cuda, empty.bfloat16(), (0,), "mean"))))
+    untouched = torch.full((1,), -7.0, device=cuda)
+    hk.reduce(torch.empty((10, 0), device=cuda), torch.empty((0,), device=cuda), [0], "sum")
+    torch.cuda.synchronize()
+    assert float(untouched[0]) == -7.0

@@ -200,6 +200,12 @@ CASES = [
 ]
 
 
+# HBM bytes one launch of the RMSNorm backward kernel moves at the headline shape: rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE read 262764.1 and 270336.0 KiB per dispatch; a 256 MiB copy kernel calibrates the counters at
+# x2.000 (FETCH_SIZE reads 131082 KiB for 262144 KiB fetched) and x1.000 (WRITE_SIZE).
+NORM_BWD_TRAFFIC_BYTES = int((262764.1 * 2.0 + 270336.0 * 1.0) * 1024)
+
+
 def time_case(hk, torch, launch, steps, warmup, profile_main=True):
     """Returns (ms per step over a plain timed region, mean us of the main kernel measured in a
     second region with HIP events recorded around that kernel on its stream)."""
@@ -300,13 +306,13 @@ def main():
         "metric": "HBM GB/s, RMSNorm fwd+bwd at Llama-7B token shape (algorithmic bytes / step time)",
         "value": round(step_bytes / ms / 1e6, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16 storage, fp32 arithmetic", "data": "synthetic",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "C4 RMSNorm fwd+bwd bf16 [32768 packed tokens x 4096], eps 1e-6, weight U(0.8,1.2)",
-                   "rows": rows, "hidden": 4096, "us_fwd_plus_bwd": round(ms * 1000, 2),
+                   "rows": rows, "hidden": 4096, "storage": "bf16", "accumulate": "fp32", "us_fwd_plus_bwd": round(ms * 1000, 2),
                    "rows_per_s": round(rows / ms * 1e3), "frac_of_hbm_peak": round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "kernel": "norm_bwd_kernel<bf16> (RMSNorm backward, dx + dgamma/dbeta partials)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": NORM_BWD_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_us": round(bwd_us, 2)},
     }
     if not args.no_cpu:

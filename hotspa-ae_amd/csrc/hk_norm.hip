@@ -472,13 +472,19 @@ void norm_bwd_kernel(NormBwdArgs a) {
   const int64_t stride = int64_t(gridDim.x) * rpb;
   // nx / ndy: the next PF rows of this group, packed, oldest first
   u32x4 nx[PF][NV], ndy[PF][NV];
+  // the row statistics travel in the same ring: a load issued when they are needed
+  // would put a full memory round trip on every iteration's critical path
+  float nmu[PF], nsv[PF];
   int64_t row = int64_t(blockIdx.x) * rpb + group;
 #pragma unroll
   for (int d = 0; d < PF; ++d) {
     const int64_t r = row + d * stride;
 #pragma unroll
     for (int i = 0; i < NV; ++i) { nx[d][i] = u32x4{0, 0, 0, 0}; ndy[d][i] = u32x4{0, 0, 0, 0}; }
+    nmu[d] = 0.f; nsv[d] = 0.f;
     if (r < a.rows) {
+      if (MODE == BWD_LN) nmu[d] = load_stat<T>(a.mean, r, a.stats_f32);
+      nsv[d] = load_stat<T>(a.stat, r, a.stats_f32);
       const T* xr = static_cast<const T*>(a.x) + r * int64_t(a.cols);
       const T* dyr = static_cast<const T*>(a.dy) + r * int64_t(a.cols);
 #pragma unroll
@@ -502,8 +508,8 @@ void norm_bwd_kernel(NormBwdArgs a) {
         VecIO<T>::unpack(nx[0][i], &xs[i * VEC]);
         VecIO<T>::unpack(ndy[0][i], &ts[i * VEC]);
       }
-      if (MODE == BWD_LN) mu = load_stat<T>(a.mean, row, a.stats_f32);
-      const float sv = load_stat<T>(a.stat, row, a.stats_f32);
+      mu = nmu[0];
+      const float sv = nsv[0];
       rs = a.stat_kind == HK_STAT_VAR ? 1.0f / sqrtf(sv + a.eps) : sv;
     }
     // rotate the prefetch ring and issue the loads of the row PF steps ahead
@@ -511,6 +517,7 @@ void norm_bwd_kernel(NormBwdArgs a) {
     for (int d = 0; d + 1 < PF; ++d) {
 #pragma unroll
       for (int i = 0; i < NV; ++i) { nx[d][i] = nx[d + 1][i]; ndy[d][i] = ndy[d + 1][i]; }
+      nmu[d] = nmu[d + 1]; nsv[d] = nsv[d + 1];
     }
     const int64_t next = row + stride;
     {
@@ -523,6 +530,8 @@ void norm_bwd_kernel(NormBwdArgs a) {
           const int v = i * tpr + t;
           if (v < a.nvec) { nx[PF - 1][i] = ld16(xr + v * VEC); ndy[PF - 1][i] = ld16(dyr + v * VEC); }
         }
+        if (MODE == BWD_LN) nmu[PF - 1] = load_stat<T>(a.mean, far, a.stats_f32);
+        nsv[PF - 1] = load_stat<T>(a.stat, far, a.stats_f32);
       }
     }
     if (valid) {

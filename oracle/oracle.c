@@ -12,7 +12,7 @@
  *   refcpu_*   fp32 ports of the reference's CPU kernels with the same pass
  *              structure; they are what the bench times as "cpu_baseline".
  *
- * Pinning (see tests/test_oracle_*.py): closed forms and invariants, brute
+ * Pinning (see tests/test_oracle.py): closed forms and invariants, brute
  * force on tiny inputs, finite differences for every backward, and
  * cross-checks against an independent library (torch CPU, float64).  The
  * reference repository holds no tests, golden vectors or fixtures for these

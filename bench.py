@@ -261,8 +261,9 @@ def cpu_baseline(sample_rows=2048, cols=4096, reps=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=300,
+                    help="untimed steps; a few hundred let the clocks settle after idle")
     ap.add_argument("--all", action="store_true", help="also time every kernel of every configuration")
     ap.add_argument("--only", default="", help="substring filter for --all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

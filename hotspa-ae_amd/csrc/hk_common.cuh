@@ -7,6 +7,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <type_traits>
+#include <utility>
 #include <stdint.h>
 #include <stddef.h>
 
@@ -137,6 +139,29 @@ template <> struct VecIO<fp16> {
     return r;
   }
 };
+
+// max(a, b, c) in one instruction.  Written as inline assembly because fmaxf() on values that were
+// assembled from integer bits makes the compiler canonicalise each operand first (one extra v_max per
+// element); the instruction itself already returns the non-NaN operand when one operand is a NaN.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+// A 16-byte vector whose every element is -infinity in T: padding that leaves a
+// maximum and a sum of exponentials untouched, so kernels need no per-vector
+// predicate in their arithmetic.
+template <typename T> __device__ __forceinline__ u32x4 neg_inf_vec();
+template <> __device__ __forceinline__ u32x4 neg_inf_vec<float>() {
+  return u32x4{0xff800000u, 0xff800000u, 0xff800000u, 0xff800000u};
+}
+template <> __device__ __forceinline__ u32x4 neg_inf_vec<bf16>() {
+  return u32x4{0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u};
+}
+template <> __device__ __forceinline__ u32x4 neg_inf_vec<fp16>() {
+  return u32x4{0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u};
+}
 
 // Row data is read exactly once: non-temporal loads keep it from displacing
 // reusable lines and stream measurably faster.  Small reused vectors (gamma,
@@ -280,6 +305,17 @@ __device__ __forceinline__ P group_allreduce_tuple(P a, float* scratch, int firs
     r = P::merge(r, o);
   }
   return r;
+}
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}): a loop whose index is a
+// compile-time constant in every iteration
+template <typename F, int... D>
+__device__ __forceinline__ void static_for_impl(F& f, std::integer_sequence<int, D...>) {
+  (f(std::integral_constant<int, D>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 // plain sums of K values

@@ -125,36 +125,37 @@ void norm_fwd_kernel(NormFwdArgs a) {
     var = fmaxf(ms - mu * mu, 0.f);
     rs = 1.0f / sqrtf(ms + a.eps);
   } else {
-    // thread-local moments over the registers, then Chan merge
-    float s = 0.f;
-    int cnt = 0;
+    // the row sits in registers, so the textbook two-pass variance costs no memory traffic: sum -> mean,
+    // then sum of squared distances to that mean.  Two plain sum reductions (six DPP adds each, one LDS
+    // round when several waves share the row) are far shorter than one reduction of Welford triples, whose
+    // every merge step carries a division on the critical path.
+    SumTuple<1> s;
+    s.v[0] = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       if (i * tpr + t < a.nvec) {
         float f[VEC];
         get(i, f);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) s += f[j];
-        cnt += VEC;
+        for (int j = 0; j < VEC; ++j) s.v[0] += f[j];
       }
     }
-    MomentTuple m;
-    m.v[0] = float(cnt);
-    m.v[1] = cnt > 0 ? s / float(cnt) : 0.f;
-    float m2 = 0.f;
+    s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red, 0, nwaves);
+    mu = s.v[0] * a.inv_cols;
+    SumTuple<1> q;
+    q.v[0] = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       if (i * tpr + t < a.nvec) {
         float f[VEC];
         get(i, f);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) { const float d = f[j] - m.v[1]; m2 = fmaf(d, d, m2); }
+        for (int j = 0; j < VEC; ++j) { const float d = f[j] - mu; q.v[0] = fmaf(d, d, q.v[0]); }
       }
     }
-    m.v[2] = m2;
-    m = WAVE_ROW ? wave_allreduce_tuple(m) : group_allreduce_tuple(m, red, 0, nwaves);
-    mu = m.v[1];
-    var = m.v[2] * a.inv_cols;
+    // a second LDS region: waves still reading the first sums must not see them overwritten
+    q = WAVE_ROW ? wave_allreduce_tuple(q) : group_allreduce_tuple(q, red + kMaxWaves, 0, nwaves);
+    var = q.v[0] * a.inv_cols;
     rs = 1.0f / sqrtf(var + a.eps);
   }
 
@@ -470,18 +471,15 @@ void norm_bwd_kernel(NormBwdArgs a) {
   for (int e = 0; e < NE; ++e) { dg[e] = 0.f; db[e] = 0.f; }
 
   const int64_t stride = int64_t(gridDim.x) * rpb;
-  // nx / ndy: the next PF rows of this group, packed, oldest first
+  // A ring of PF rows in flight per thread group: slot d holds row0 + d * stride, packed, together with
+  // that row's statistics (a statistics load issued when the value is needed would put a full memory
+  // round trip on every step's critical path).  The loop body is unrolled over the slots, so a slot is a
+  // fixed set of registers: moving a slot's registers while its loads are still outstanding would stall
+  // on them and flatten the ring to depth one.
   u32x4 nx[PF][NV], ndy[PF][NV];
-  // the row statistics travel in the same ring: a load issued when they are needed
-  // would put a full memory round trip on every iteration's critical path
   float nmu[PF], nsv[PF];
-  int64_t row = int64_t(blockIdx.x) * rpb + group;
-#pragma unroll
-  for (int d = 0; d < PF; ++d) {
-    const int64_t r = row + d * stride;
-#pragma unroll
-    for (int i = 0; i < NV; ++i) { nx[d][i] = u32x4{0, 0, 0, 0}; ndy[d][i] = u32x4{0, 0, 0, 0}; }
-    nmu[d] = 0.f; nsv[d] = 0.f;
+  auto issue = [&](auto slot, int64_t r) {
+    constexpr int d = decltype(slot)::value;
     if (r < a.rows) {
       if (MODE == BWD_LN) nmu[d] = load_stat<T>(a.mean, r, a.stats_f32);
       nsv[d] = load_stat<T>(a.stat, r, a.stats_f32);
@@ -493,10 +491,20 @@ void norm_bwd_kernel(NormBwdArgs a) {
         if (v < a.nvec) { nx[d][i] = ld16(xr + v * VEC); ndy[d][i] = ld16(dyr + v * VEC); }
       }
     }
+  };
+  int64_t row0 = int64_t(blockIdx.x) * rpb + group;
+#pragma unroll
+  for (int d = 0; d < PF; ++d) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) { nx[d][i] = u32x4{0, 0, 0, 0}; ndy[d][i] = u32x4{0, 0, 0, 0}; }
+    nmu[d] = 0.f; nsv[d] = 0.f;
   }
+  static_for<PF>([&](auto slot) { issue(slot, row0 + decltype(slot)::value * stride); });
 
   int parity = 0;
-  for (int64_t base = int64_t(blockIdx.x) * rpb; base < a.rows; base += stride, parity ^= 1) {
+  auto step = [&](auto slot) {
+    constexpr int d = decltype(slot)::value;
+    const int64_t row = row0 + d * stride;
     const bool valid = row < a.rows;
     float xs[NE], ts[NE];                 // xc (x_hat in the memory-efficient mode) and dy * gamma
     float mu = 0.f, rs = 0.f;
@@ -505,35 +513,15 @@ void norm_bwd_kernel(NormBwdArgs a) {
     if (valid) {
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
-        VecIO<T>::unpack(nx[0][i], &xs[i * VEC]);
-        VecIO<T>::unpack(ndy[0][i], &ts[i * VEC]);
+        VecIO<T>::unpack(nx[d][i], &xs[i * VEC]);
+        VecIO<T>::unpack(ndy[d][i], &ts[i * VEC]);
       }
-      mu = nmu[0];
-      const float sv = nsv[0];
+      mu = nmu[d];
+      const float sv = nsv[d];
       rs = a.stat_kind == HK_STAT_VAR ? 1.0f / sqrtf(sv + a.eps) : sv;
     }
-    // rotate the prefetch ring and issue the loads of the row PF steps ahead
-#pragma unroll
-    for (int d = 0; d + 1 < PF; ++d) {
-#pragma unroll
-      for (int i = 0; i < NV; ++i) { nx[d][i] = nx[d + 1][i]; ndy[d][i] = ndy[d + 1][i]; }
-      nmu[d] = nmu[d + 1]; nsv[d] = nsv[d + 1];
-    }
-    const int64_t next = row + stride;
-    {
-      const int64_t far = row + int64_t(PF) * stride;
-      if (far < a.rows) {
-        const T* xr = static_cast<const T*>(a.x) + far * int64_t(a.cols);
-        const T* dyr = static_cast<const T*>(a.dy) + far * int64_t(a.cols);
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-          const int v = i * tpr + t;
-          if (v < a.nvec) { nx[PF - 1][i] = ld16(xr + v * VEC); ndy[PF - 1][i] = ld16(dyr + v * VEC); }
-        }
-        if (MODE == BWD_LN) nmu[PF - 1] = load_stat<T>(a.mean, far, a.stats_f32);
-        nsv[PF - 1] = load_stat<T>(a.stat, far, a.stats_f32);
-      }
-    }
+    // the slot is free again: refill it with the row PF steps ahead
+    issue(slot, row + int64_t(PF) * stride);
     if (valid) {
       // padding vectors hold zeros in ts (dy), so they add nothing anywhere.
       // q = dy * rs * gamma is both the dx term and, summed, rs * sum(dy * gamma).
@@ -570,6 +558,7 @@ void norm_bwd_kernel(NormBwdArgs a) {
       else accumulate(std::false_type{});
     }
     s = group_allreduce_tuple(s, red[parity], first_wave, waves_per_group);
+    parity ^= 1;
     if (valid) {
       // plain modes: s0 = rs * sum(dy g), s1 = rs * sum(dy g xc);  dx = q - s0/n - xc * rs^2 * s1/n
       // memory-efficient: s0 = sum(dy g), s1 = sum(dy (y - beta));   dx = rs * (dy kg - s0/n - xhat * s1/n)
@@ -608,7 +597,12 @@ void norm_bwd_kernel(NormBwdArgs a) {
         }
       }
     }
-    row = next;
+  };
+  // every thread of the block takes the same number of steps (the bound is block-uniform), so the
+  // barrier inside the group reduction is reached by all of them
+  for (int64_t base = int64_t(blockIdx.x) * rpb; base < a.rows; base += int64_t(PF) * stride) {
+    static_for<PF>(step);
+    row0 += int64_t(PF) * stride;
   }
 
   // fold the row groups of this block, then write one partial row per block
@@ -860,13 +854,14 @@ static int launch_norm_bwd_nv(const NormBwdArgs& a, const BwdPlan& p, hipStream_
   dim3 grid{unsigned(p.grid)}, block{unsigned(p.block)};
   profile_before(s);
   int pf = tune_get(TUNE_NORM_BWD_PREFETCH);
-  if (pf <= 0) pf = 1;   // deeper rings measured slower
+  if (pf <= 0) pf = 2;
 #define HK_BWD_LAUNCH(N, P) hipLaunchKernelGGL((norm_bwd_kernel<T, N, MODE, P>), grid, block, p.lds_bytes, s, a)
 #define HK_BWD_PF(N)                                   \
   do {                                                 \
     if (pf == 1) HK_BWD_LAUNCH(N, 1);                  \
     else if (pf == 2) HK_BWD_LAUNCH(N, 2);             \
-    else HK_BWD_LAUNCH(N, 3);                          \
+    else if (pf == 3) HK_BWD_LAUNCH(N, 3);             \
+    else HK_BWD_LAUNCH(N, 4);                          \
   } while (0)
   switch (p.nv) {
     case 1: HK_BWD_PF(1); break;

@@ -389,11 +389,16 @@ static InnerShape shape_inner(const ReducePlan& p, const void* in) {
   s.vec = aligned16(in) && (p.rows == 1 || p.row_stride % VEC == 0);
   const int64_t nvec = p.cols / VEC;
   int tpr = tune_get(TUNE_REDUCE_INNER_THREADS);
-  if (tpr <= 0) tpr = nvec <= 64 * 32 ? 64 : (nvec <= 256 * 32 ? 256 : 1024);
+  const int64_t want_blocks = int64_t(device_cu_count()) * 4;
+  if (tpr <= 0) {
+    tpr = nvec <= 64 * 32 ? 64 : (nvec <= 256 * 32 ? 256 : 1024);
+    // too few rows to fill the chip: widen the group until a thread has at most one round of 8 loads,
+    // so that a short row costs one memory round trip instead of several dependent ones
+    if (p.rows < want_blocks) tpr = int(std::max<int64_t>(tpr, std::min<int64_t>(1024, (nvec + 7) / 8)));
+  }
   tpr = std::min(1024, std::max(64, (tpr + 63) / 64 * 64));
   s.tpr = tpr;
   // few long rows: split columns so that ~4 workgroups per CU exist
-  const int64_t want_blocks = int64_t(device_cu_count()) * 4;
   int64_t groups = tpr == 64 ? (p.rows + 3) / 4 : p.rows;
   int64_t nsplit = 1;
   if (groups < want_blocks && nvec > int64_t(tpr) * 32) {

@@ -56,35 +56,35 @@ void sce_sparse_fwd_kernel(SceArgs a) {
     return;
   }
   const T* xr = static_cast<const T*>(a.logits) + row * int64_t(a.cols);
-  u32x4 raw[NV];
+  // slots past the row's end hold -inf: they change neither the maximum nor the sum
+  float f[NV * VEC];
+  {
+    u32x4 raw[NV];
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int v = i * tpr + t;
-    raw[i] = u32x4{0, 0, 0, 0};
-    if (v < a.nvec) raw[i] = ld16(xr + v * VEC);
-  }
-  float m = kNegInf;
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    if (i * tpr + t < a.nvec) {
-      float f[VEC];
-      VecIO<T>::unpack(raw[i], f);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) m = fmaxf(m, f[j]);
+    for (int i = 0; i < NV; ++i) {
+      const int v = i * tpr + t;
+      if ((i + 1) * tpr <= a.nvec) {       // uniform: every thread's slot i is inside the row
+        raw[i] = ld16(xr + v * VEC);
+      } else {
+        raw[i] = neg_inf_vec<T>();
+        if (v < a.nvec) raw[i] = ld16(xr + v * VEC);
+      }
     }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) VecIO<T>::unpack(raw[i], &f[i * VEC]);
   }
+  float m = f[0];
+  static_assert((NV * VEC) % 2 == 0, "pairs of elements per max3");
+  m = fmaxf(m, f[1]);
+#pragma unroll
+  for (int e = 2; e < NV * VEC; e += 2) m = max3(m, f[e], f[e + 1]);
   // ml: this thread's maximum in the log2 domain, rounded once (see OnlineSoftmaxTuple)
   const float ml = (m == kNegInf) ? 0.f : m * kLog2e;
-  float s = 0.f;
+  // four independent chains: the exponential unit's latency is not serialised behind one accumulator
+  float s4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    if (i * tpr + t < a.nvec) {
-      float f[VEC];
-      VecIO<T>::unpack(raw[i], f);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) s += __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, -ml));
-    }
-  }
+  for (int e = 0; e < NV * VEC; ++e) s4[e & 3] += __builtin_amdgcn_exp2f(fmaf(f[e], kLog2e, -ml));
+  const float s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
   MaxSumMaxTuple p;
   p.v[0] = (m == kNegInf) ? kNegInf : ml; p.v[1] = s; p.v[2] = m;
   p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);

@@ -58,6 +58,7 @@ template <typename T> struct Cvt;
 
 template <> struct Cvt<float> {
   static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ float to_float(float v) { return v; }
   static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
 };
 
@@ -65,6 +66,7 @@ template <> struct Cvt<bf16> {
   static __device__ __forceinline__ float load(const bf16* p) {
     return u2f(uint32_t(p->bits) << 16);
   }
+  static __device__ __forceinline__ float to_float(bf16 v) { return u2f(uint32_t(v.bits) << 16); }
   static __device__ __forceinline__ void store(bf16* p, float v) {
     // round-to-nearest-even through the hardware packed converter
     f32x2 f = {v, 0.f};
@@ -77,6 +79,7 @@ template <> struct Cvt<fp16> {
   static __device__ __forceinline__ float load(const fp16* p) {
     return float(__builtin_bit_cast(_Float16, p->bits));
   }
+  static __device__ __forceinline__ float to_float(fp16 v) { return float(__builtin_bit_cast(_Float16, v.bits)); }
   static __device__ __forceinline__ void store(fp16* p, float v) {
     p->bits = __builtin_bit_cast(uint16_t, _Float16(v));
   }

@@ -430,13 +430,24 @@ __device__ __forceinline__ float clamp_by_magnitude(float g, float eps) {
 // registers.  With xc = x - mu (x for RMSNorm), t = dy * gamma and
 // m2 = mean(t * xc):   dx = rs * t - rs * mean(t) - xc * rs^3 * m2,
 // two fused multiply-adds per element once the row sums are known.
-template <typename T, int NV, int MODE, int PF>
+//
+// PF rows per thread group are in flight at any time (a ring of register slots,
+// refilled as soon as a slot has been unpacked).  The steady-state loop is
+// written without a single branch around a memory instruction: out-of-range
+// rows are clamped instead of skipped, EXACT says that no thread has a column
+// past the row's end, STATS_F32 fixes the statistics' type.  Only then does the
+// compiler count outstanding loads exactly; any branch in the loop makes it
+// wait for all of them at every step, which flattens the ring to depth one.
+// Rows that do not fill a whole round of PF steps go through the same step with
+// its guards switched on.
+template <typename T, int NV, int MODE, int PF, bool EXACT, bool STATS_F32>
 __global__ __launch_bounds__(NV == 1 ? 1024 : 512)
 void norm_bwd_kernel(NormBwdArgs a) {
   constexpr int VEC = VecIO<T>::N;
   constexpr int NE = NV * VEC;
+  using StatT = typename std::conditional<STATS_F32, float, T>::type;
   extern __shared__ float lds[];           // [rows_per_block, cols] column-sum staging
-  __shared__ float red[2][kMaxWaves * 2];  // double-buffered by iteration parity
+  __shared__ float red[2][kMaxWaves * 2];  // double-buffered by step parity
 
   const int tpr = a.tpr;                   // multiple of 64: a wavefront never straddles two rows
   const int rpb = int(blockDim.x) / tpr;
@@ -444,6 +455,17 @@ void norm_bwd_kernel(NormBwdArgs a) {
   const int t = int(threadIdx.x) - group * tpr;
   const int waves_per_group = tpr >> 6;
   const int first_wave = group * waves_per_group;
+
+  // column vectors of this thread; a thread past the row's end (only when !EXACT) reads the last vector
+  // again and has its dy forced to zero, so it adds nothing and stores nothing
+  int vidx[NV];
+  bool vin[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * tpr + t;
+    vin[i] = EXACT || v < a.nvec;
+    vidx[i] = vin[i] ? v : a.nvec - 1;
+  }
 
   // gamma (and beta) of this thread's columns as fp32; a missing gamma is all ones
   float gm[NE];
@@ -453,14 +475,13 @@ void norm_bwd_kernel(NormBwdArgs a) {
     const T* bp = static_cast<const T*>(a.beta);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int v = i * tpr + t;
 #pragma unroll
       for (int j = 0; j < VEC; ++j) gm[i * VEC + j] = 1.f;
-      if (v < a.nvec && gp) VecIO<T>::unpack(ld16_keep(gp + v * VEC), &gm[i * VEC]);
+      if (gp) VecIO<T>::unpack(ld16_keep(gp + vidx[i] * VEC), &gm[i * VEC]);
       if constexpr (MODE == BWD_LN_MEMEFF) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) bt[i * VEC + j] = 0.f;
-        if (v < a.nvec && bp) VecIO<T>::unpack(ld16_keep(bp + v * VEC), &bt[i * VEC]);
+        if (bp) VecIO<T>::unpack(ld16_keep(bp + vidx[i] * VEC), &bt[i * VEC]);
       }
     }
   }
@@ -471,92 +492,88 @@ void norm_bwd_kernel(NormBwdArgs a) {
   for (int e = 0; e < NE; ++e) { dg[e] = 0.f; db[e] = 0.f; }
 
   const int64_t stride = int64_t(gridDim.x) * rpb;
-  // A ring of PF rows in flight per thread group: slot d holds row0 + d * stride, packed, together with
-  // that row's statistics (a statistics load issued when the value is needed would put a full memory
-  // round trip on every step's critical path).  The loop body is unrolled over the slots, so a slot is a
-  // fixed set of registers: moving a slot's registers while its loads are still outstanding would stall
-  // on them and flatten the ring to depth one.
+  const int64_t last_row = a.rows - 1;
   u32x4 nx[PF][NV], ndy[PF][NV];
-  float nmu[PF], nsv[PF];
+  StatT nmu[PF], nsv[PF];
+  const StatT* meanp = static_cast<const StatT*>(a.mean);
+  const StatT* statp = static_cast<const StatT*>(a.stat);
+  // loads of row r into slot d; r past the end re-reads the last row (its results are never used)
   auto issue = [&](auto slot, int64_t r) {
     constexpr int d = decltype(slot)::value;
-    if (r < a.rows) {
-      if (MODE == BWD_LN) nmu[d] = load_stat<T>(a.mean, r, a.stats_f32);
-      nsv[d] = load_stat<T>(a.stat, r, a.stats_f32);
-      const T* xr = static_cast<const T*>(a.x) + r * int64_t(a.cols);
-      const T* dyr = static_cast<const T*>(a.dy) + r * int64_t(a.cols);
+    const int64_t rc = r < last_row ? r : last_row;
+    if constexpr (MODE == BWD_LN) nmu[d] = meanp[rc];
+    nsv[d] = statp[rc];
+    const T* xr = static_cast<const T*>(a.x) + rc * int64_t(a.cols);
+    const T* dyr = static_cast<const T*>(a.dy) + rc * int64_t(a.cols);
 #pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        const int v = i * tpr + t;
-        if (v < a.nvec) { nx[d][i] = ld16(xr + v * VEC); ndy[d][i] = ld16(dyr + v * VEC); }
-      }
+    for (int i = 0; i < NV; ++i) {
+      nx[d][i] = ld16(xr + vidx[i] * VEC);
+      ndy[d][i] = ld16(dyr + vidx[i] * VEC);
     }
   };
   int64_t row0 = int64_t(blockIdx.x) * rpb + group;
-#pragma unroll
-  for (int d = 0; d < PF; ++d) {
-#pragma unroll
-    for (int i = 0; i < NV; ++i) { nx[d][i] = u32x4{0, 0, 0, 0}; ndy[d][i] = u32x4{0, 0, 0, 0}; }
-    nmu[d] = 0.f; nsv[d] = 0.f;
-  }
   static_for<PF>([&](auto slot) { issue(slot, row0 + decltype(slot)::value * stride); });
 
   int parity = 0;
-  auto step = [&](auto slot) {
+  // guarded: check that the slot's row exists (the tail); otherwise it is known to
+  auto step = [&](auto slot, auto guarded) {
     constexpr int d = decltype(slot)::value;
+    constexpr bool GUARD = decltype(guarded)::value;
     const int64_t row = row0 + d * stride;
-    const bool valid = row < a.rows;
+    const bool valid = !GUARD || row < a.rows;
     float xs[NE], ts[NE];                 // xc (x_hat in the memory-efficient mode) and dy * gamma
-    float mu = 0.f, rs = 0.f;
-    SumTuple<2> s;
-    s.v[0] = 0.f; s.v[1] = 0.f;
-    if (valid) {
 #pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        VecIO<T>::unpack(nx[d][i], &xs[i * VEC]);
-        VecIO<T>::unpack(ndy[d][i], &ts[i * VEC]);
+    for (int i = 0; i < NV; ++i) {
+      VecIO<T>::unpack(nx[d][i], &xs[i * VEC]);
+      VecIO<T>::unpack(ndy[d][i], &ts[i * VEC]);
+      if (!EXACT) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) ts[i * VEC + j] = vin[i] ? ts[i * VEC + j] : 0.f;
       }
-      mu = nmu[d];
-      const float sv = nsv[d];
-      rs = a.stat_kind == HK_STAT_VAR ? 1.0f / sqrtf(sv + a.eps) : sv;
     }
+    [[maybe_unused]] float mu = 0.f;
+    if constexpr (MODE == BWD_LN) mu = Cvt<StatT>::to_float(nmu[d]);
+    const float sv = Cvt<StatT>::to_float(nsv[d]);
+    const float rs = a.stat_kind == HK_STAT_VAR ? 1.0f / sqrtf(sv + a.eps) : sv;
     // the slot is free again: refill it with the row PF steps ahead
     issue(slot, row + int64_t(PF) * stride);
-    if (valid) {
-      // padding vectors hold zeros in ts (dy), so they add nothing anywhere.
-      // q = dy * rs * gamma is both the dx term and, summed, rs * sum(dy * gamma).
-      auto accumulate = [&](auto clamped) {
+
+    SumTuple<2> s;
+    s.v[0] = 0.f; s.v[1] = 0.f;
+    // new column sums go to copies first: a guarded step of a missing row must leave dg / db alone
+    // without a branch around the arithmetic
+    auto accumulate = [&](auto clamped) {
 #pragma unroll
-        for (int e = 0; e < NE; ++e) {
-          const float dz = ts[e];
-          if constexpr (MODE == BWD_LN_MEMEFF) {
-            const float yb = xs[e] - bt[e];
-            const float kg = clamp_by_magnitude(gm[e], a.eps);
-            const float xhat = yb / kg;
-            s.v[0] = fmaf(dz, gm[e], s.v[0]);
-            s.v[1] = fmaf(dz, yb, s.v[1]);
-            dg[e] = fmaf(dz, xhat, dg[e]);
-            db[e] += dz;
-            xs[e] = xhat;
-            ts[e] = dz * kg;
-          } else {
-            const float xc = (MODE == BWD_RMS) ? xs[e] : xs[e] - mu;
-            const float dzr = dz * rs;
-            const float q = dzr * gm[e];
-            s.v[1] = fmaf(q, xc, s.v[1]);
-            if (MODE != BWD_RMS) s.v[0] += q;
-            dg[e] = fmaf(dzr, xc, dg[e]);
-            db[e] += dz;
-            xs[e] = xc;
-            // the per-element term of dx uses the clamped gamma when asked to
-            if constexpr (decltype(clamped)::value) ts[e] = dzr * clamp_by_magnitude(gm[e], a.eps);
-            else ts[e] = q;
-          }
+      for (int e = 0; e < NE; ++e) {
+        const float dz = (GUARD && !valid) ? 0.f : ts[e];
+        if constexpr (MODE == BWD_LN_MEMEFF) {
+          const float yb = xs[e] - bt[e];
+          const float kg = clamp_by_magnitude(gm[e], a.eps);
+          const float xhat = yb / kg;
+          s.v[0] = fmaf(dz, gm[e], s.v[0]);
+          s.v[1] = fmaf(dz, yb, s.v[1]);
+          dg[e] = fmaf(dz, xhat, dg[e]);
+          db[e] += dz;
+          xs[e] = xhat;
+          ts[e] = dz * kg;
+        } else {
+          const float xc = (MODE == BWD_RMS) ? xs[e] : xs[e] - mu;
+          const float dzr = dz * rs;
+          const float q = dzr * gm[e];
+          s.v[1] = fmaf(q, xc, s.v[1]);
+          if (MODE != BWD_RMS) s.v[0] += q;
+          dg[e] = fmaf(dzr, xc, dg[e]);
+          db[e] += dz;
+          xs[e] = xc;
+          // the per-element term of dx uses the clamped gamma when asked to
+          if constexpr (decltype(clamped)::value) ts[e] = dzr * clamp_by_magnitude(gm[e], a.eps);
+          else ts[e] = q;
         }
-      };
-      if (clamp) accumulate(std::true_type{});   // uniform
-      else accumulate(std::false_type{});
-    }
+      }
+    };
+    if (clamp) accumulate(std::true_type{});   // uniform
+    else accumulate(std::false_type{});
+
     s = group_allreduce_tuple(s, red[parity], first_wave, waves_per_group);
     parity ^= 1;
     if (valid) {
@@ -575,8 +592,8 @@ void norm_bwd_kernel(NormBwdArgs a) {
       const T* dir = a.dx_in ? static_cast<const T*>(a.dx_in) + row * int64_t(a.cols) : nullptr;
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
-        const int v = i * tpr + t;
-        if (v < a.nvec) {
+        if (EXACT || vin[i]) {
+          const int v = vidx[i];
           float o[VEC];
 #pragma unroll
           for (int j = 0; j < VEC; ++j) {
@@ -598,11 +615,20 @@ void norm_bwd_kernel(NormBwdArgs a) {
       }
     }
   };
-  // every thread of the block takes the same number of steps (the bound is block-uniform), so the
-  // barrier inside the group reduction is reached by all of them
-  for (int64_t base = int64_t(blockIdx.x) * rpb; base < a.rows; base += int64_t(PF) * stride) {
-    static_for<PF>(step);
-    row0 += int64_t(PF) * stride;
+  // Every thread of the block takes the same number of steps (both loop bounds are block-uniform), so
+  // the barrier inside the group reduction is reached by all of them.
+  int64_t base = int64_t(blockIdx.x) * rpb;
+  const int64_t round = int64_t(PF) * stride;
+  // rounds in which every slot of every group of this block holds an existing row
+#pragma nounroll
+  for (; base + int64_t(PF - 1) * stride + rpb <= a.rows; base += round) {
+    static_for<PF>([&](auto slot) { step(slot, std::false_type{}); });
+    row0 += round;
+  }
+#pragma nounroll
+  for (; base < a.rows; base += round) {
+    static_for<PF>([&](auto slot) { step(slot, std::true_type{}); });
+    row0 += round;
   }
 
   // fold the row groups of this block, then write one partial row per block
@@ -854,14 +880,35 @@ static int launch_norm_bwd_nv(const NormBwdArgs& a, const BwdPlan& p, hipStream_
   dim3 grid{unsigned(p.grid)}, block{unsigned(p.block)};
   profile_before(s);
   int pf = tune_get(TUNE_NORM_BWD_PREFETCH);
-  if (pf <= 0) pf = 2;
-#define HK_BWD_LAUNCH(N, P) hipLaunchKernelGGL((norm_bwd_kernel<T, N, MODE, P>), grid, block, p.lds_bytes, s, a)
+  // two rows in flight where the registers allow it (RMSNorm); the LayerNorm modes carry the mean as well
+  // and start spilling at depth two under the 128-register cap of 1024-thread blocks
+  if (pf <= 0) pf = (MODE == BWD_RMS) ? 2 : 1;
+  const bool exact = int64_t(p.nv) * p.tpr == a.nvec;
+  const bool f32 = a.stats_f32 != 0;
+  // statistics in the data dtype only ever come with the plain LayerNorm backward
+  if (!f32 && MODE != BWD_LN) {
+    set_last_error("norm_bwd: this mode keeps its statistics in float32");
+    return HK_ERR_INVALID;
+  }
+#define HK_BWD_LAUNCH(N, P, E, F) \
+  hipLaunchKernelGGL((norm_bwd_kernel<T, N, MODE, P, E, F>), grid, block, p.lds_bytes, s, a)
+#define HK_BWD_EF(N, P)                                                    \
+  do {                                                                     \
+    if constexpr (MODE == BWD_LN) {                                        \
+      if (exact && f32) HK_BWD_LAUNCH(N, P, true, true);                   \
+      else if (exact) HK_BWD_LAUNCH(N, P, true, false);                    \
+      else if (f32) HK_BWD_LAUNCH(N, P, false, true);                      \
+      else HK_BWD_LAUNCH(N, P, false, false);                              \
+    } else {                                                               \
+      if (exact) HK_BWD_LAUNCH(N, P, true, true);                          \
+      else HK_BWD_LAUNCH(N, P, false, true);                               \
+    }                                                                      \
+  } while (0)
 #define HK_BWD_PF(N)                                   \
   do {                                                 \
-    if (pf == 1) HK_BWD_LAUNCH(N, 1);                  \
-    else if (pf == 2) HK_BWD_LAUNCH(N, 2);             \
-    else if (pf == 3) HK_BWD_LAUNCH(N, 3);             \
-    else HK_BWD_LAUNCH(N, 4);                          \
+    if (pf == 1) HK_BWD_EF(N, 1);                      \
+    else if (pf == 2) HK_BWD_EF(N, 2);                 \
+    else HK_BWD_EF(N, 3);                              \
   } while (0)
   switch (p.nv) {
     case 1: HK_BWD_PF(1); break;
@@ -873,6 +920,7 @@ static int launch_norm_bwd_nv(const NormBwdArgs& a, const BwdPlan& p, hipStream_
       set_last_error("norm_bwd: no kernel for %d vectors per thread", p.nv);
       return HK_ERR_UNSUPPORTED;
   }
+#undef HK_BWD_EF
 #undef HK_BWD_PF
 #undef HK_BWD_LAUNCH
   profile_after(s);

@@ -181,6 +181,33 @@ def case_copy(hk, torch, nsets):
     return (lambda i: hk.copy_kernel(dst[i % nsets], src[i % nsets])), 2 * n, 1
 
 
+def case_fill(hk, torch, nsets):
+    import ctypes
+    n = 1 << 28
+    dst = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(nsets)]
+    lib = hk.lib()
+
+    def launch(i):
+        hk.check(lib.hk_memset(ctypes.c_void_p(dst[i % nsets].data_ptr()), ctypes.c_int(0), ctypes.c_size_t(n),
+                               hk.current_stream()))
+    return launch, n, 1
+
+
+def case_torch_add(hk, torch, nsets):
+    """torch's own elementwise add (two reads, one write per element): an independent yardstick for what
+    a plain streaming kernel with this read/write mix reaches on the same GPU."""
+    rows, cols = 32768, 4096
+    bf = torch.bfloat16
+    a = [_randn(torch, (rows, cols), bf, 1.0, 901 + i) for i in range(nsets)]
+    b = [_randn(torch, (rows, cols), bf, 1.0, 951 + i) for i in range(nsets)]
+    o = [torch.empty((rows, cols), dtype=bf, device="cuda") for _ in range(nsets)]
+
+    def launch(i):
+        torch.add(a[i % nsets], b[i % nsets], out=o[i % nsets])
+    launch.no_hook = True
+    return launch, 3 * rows * cols * 2, rows
+
+
 CASES = [
     ("C1 layernorm fwd fp32 [8192x4096]", lambda hk, t, n: case_layernorm(hk, t, n, "fwd", "C1")),
     ("C2 softmax fwd bf16 [4,32,2048,2048]", lambda hk, t, n: case_softmax(hk, t, 2, "fwd")),
@@ -197,6 +224,8 @@ CASES = [
     ("C5 layernorm fwd bf16 [16384x5120]", lambda hk, t, n: case_layernorm(hk, t, n, "fwd", "C5")),
     ("C5 layernorm bwd bf16 [16384x5120]", lambda hk, t, n: case_layernorm(hk, t, n, "bwd", "C5")),
     ("copy kernel 256 MiB (calibration)", lambda hk, t, n: case_copy(hk, t, n)),
+    ("fill kernel 256 MiB (write-only calibration)", lambda hk, t, n: case_fill(hk, t, n)),
+    ("torch.add bf16 [32768x4096] (2R:1W yardstick)", lambda hk, t, n: case_torch_add(hk, t, n)),
 ]
 
 
@@ -293,7 +322,10 @@ def main():
             if args.only and args.only not in name:
                 continue
             launch, nbytes, rows = make(hk, torch, args.nsets)
-            ms, main_us = time_case(hk, torch, launch, args.steps, args.warmup)
+            ms, main_us = time_case(hk, torch, launch, args.steps, args.warmup,
+                                    profile_main=not getattr(launch, "no_hook", False))
+            if main_us is None:
+                main_us = ms * 1000
             rec = {"case": name, "us": round(ms * 1000, 2), "main_kernel_us": round(main_us, 2),
                    "GBps": round(nbytes / ms / 1e6, 1), "frac_of_8TBps": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
                    "main_kernel_frac": round(nbytes / main_us / 1e3 / HBM_PEAK_GBS, 4),

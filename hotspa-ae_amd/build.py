@@ -46,7 +46,18 @@ def _hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def build_device(verbose=True):
+def _stale(src, obj):
+    if not os.path.exists(obj):
+        return True
+    own = os.path.getmtime(os.path.join(CSRC, src))
+    common = os.path.getmtime(os.path.join(CSRC, "hk_common.cuh"))
+    header = max(os.path.getmtime(os.path.join(INCLUDE, f)) for f in os.listdir(INCLUDE))
+    return os.path.getmtime(obj) < max(own, common, header)
+
+
+def build_device(verbose=True, incremental=False):
+    """hipcc: every .hip under csrc/ -> lib/libhk_rowwise.so.  incremental=True skips
+    sources whose object is newer than the source and the shared headers."""
     os.makedirs(LIB, exist_ok=True)
     os.makedirs(OBJ, exist_ok=True)
     hipcc = _hipcc()
@@ -55,6 +66,8 @@ def build_device(verbose=True):
 
     def one(pair):
         src, obj = pair
+        if incremental and not _stale(src, obj):
+            return src + " (up to date)"
         _run([hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
         return src
 
@@ -108,11 +121,11 @@ def build_host(verbose=True):
     return out
 
 
-def build_all(verbose=True):
-    build_device(verbose)
+def build_all(verbose=True, incremental=False):
+    build_device(verbose, incremental)
     build_host(verbose)
 
 
 if __name__ == "__main__":
-    build_all()
+    build_all(incremental="--incremental" in sys.argv[1:])
     sys.exit(0)

@@ -78,20 +78,27 @@ int device_cu_count() {
 // utility kernels
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void fill_bytes_kernel(uint8_t* dst, uint32_t word, size_t bytes) {
-  // head/tail bytes individually, the aligned middle as 16-byte stores
-  const size_t tid = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  const size_t nthreads = size_t(gridDim.x) * blockDim.x;
+  // head / tail bytes individually (first workgroup), the aligned middle as 16-byte stores: every
+  // workgroup writes 4 KiB-strided vectors once and retires, the shape that streams fastest here
+  constexpr int UNROLL = 4;
   const uintptr_t addr = reinterpret_cast<uintptr_t>(dst);
   size_t head = (16 - (addr & 15)) & 15;
   if (head > bytes) head = bytes;
   const size_t nvec = (bytes - head) / 16;
   const size_t tail_begin = head + nvec * 16;
   const uint8_t b = uint8_t(word & 0xff);
-  if (tid < head) dst[tid] = b;
-  u32x4 v = {word, word, word, word};
+  if (blockIdx.x == 0) {
+    if (threadIdx.x < head) dst[threadIdx.x] = b;
+    if (threadIdx.x < bytes - tail_begin) dst[tail_begin + threadIdx.x] = b;
+  }
+  const u32x4 v = {word, word, word, word};
   u32x4* mid = reinterpret_cast<u32x4*>(dst + head);
-  for (size_t i = tid; i < nvec; i += nthreads) mid[i] = v;
-  if (tid < bytes - tail_begin) dst[tail_begin + tid] = b;
+  const size_t base = (size_t(blockIdx.x) * UNROLL) * 256 + threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < UNROLL; ++i) {
+    const size_t idx = base + size_t(i) * 256;
+    if (idx < nvec) mid[idx] = v;
+  }
 }
 
 template <int UNROLL>
@@ -209,10 +216,12 @@ int hk_memset(void* dst, int value, size_t bytes, hkStream_t stream) {
   uint32_t b = uint32_t(value) & 0xff;
   uint32_t word = b | (b << 8) | (b << 16) | (b << 24);
   size_t nvec = bytes / 16 + 1;
-  size_t blocks = (nvec + 255) / 256;
-  if (blocks > 4096) blocks = 4096;
+  size_t blocks = (nvec + 1023) / 1024;
+  HK_REQUIRE(blocks <= 0x7fffffffu, HK_ERR_INVALID, "hk_memset: size too large");
+  profile_before(as_hip(stream));
   hipLaunchKernelGGL(fill_bytes_kernel, dim3(unsigned(blocks)), dim3(256), 0, as_hip(stream),
                      static_cast<uint8_t*>(dst), word, bytes);
+  profile_after(as_hip(stream));
   return launch_check("fill_bytes_kernel");
 }
 

@@ -1,0 +1,95 @@
+"""GPU checks of the device layer of the C-ABI: fill, copies, streams and events."""
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_memset_any_alignment_and_size(hk, cuda):
+    import torch
+    lib = hk.lib()
+    buf = torch.zeros(1 << 16, dtype=torch.uint8, device=cuda)
+    for off, n in [(0, 0), (0, 1), (1, 1), (3, 13), (5, 16), (15, 17), (16, 4096), (7, 4099), (1, 40000), (9, 1 << 15)]:
+        buf.fill_(0x11)
+        torch.cuda.synchronize()
+        hk.check(lib.hk_memset(ctypes.c_void_p(buf.data_ptr() + off), ctypes.c_int(0xAB), ctypes.c_size_t(n),
+                               hk.current_stream()))
+        torch.cuda.synchronize()
+        got = buf.cpu().numpy()
+        want = np.full(1 << 16, 0x11, dtype=np.uint8)
+        want[off:off + n] = 0xAB
+        assert np.array_equal(got, want), (off, n)
+    big = torch.empty((1 << 26) + 3, dtype=torch.uint8, device=cuda)
+    hk.check(lib.hk_memset(ctypes.c_void_p(big.data_ptr()), ctypes.c_int(0x5A), ctypes.c_size_t(big.numel()),
+                           hk.current_stream()))
+    torch.cuda.synchronize()
+    assert int(big.min()) == 0x5A and int(big.max()) == 0x5A
+    assert lib.hk_memset(None, 0, ctypes.c_size_t(8), hk.current_stream()) == -1
+
+
+def test_copy_and_strided_copy(hk, cuda):
+    import torch
+    src = torch.arange(1 << 20, dtype=torch.int32, device=cuda)
+    dst = torch.zeros_like(src)
+    hk.copy_kernel(dst.view(torch.uint8), src.view(torch.uint8))
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)
+    for dt in (torch.float32, torch.bfloat16, torch.int64, torch.uint8, torch.float64):
+        x = (torch.arange(7 * 12 * 5, device=cuda) % 120).to(dt).reshape(7, 12, 5)
+        view = x.permute(2, 0, 1)[:, ::2, 1:]
+        out = torch.empty(view.shape, dtype=dt, device=cuda)
+        hk.strided_copy(view, out)
+        torch.cuda.synchronize()
+        assert torch.equal(out, view.contiguous()), dt
+
+
+def test_streams_events_and_ordering(hk, cuda):
+    import torch
+    lib = hk.lib()
+    s1, s2 = ctypes.c_void_p(), ctypes.c_void_p()
+    hk.check(lib.hk_stream_create(ctypes.byref(s1)))
+    hk.check(lib.hk_stream_create(ctypes.byref(s2)))
+    a = torch.zeros(1 << 24, dtype=torch.uint8, device=cuda)
+    b = torch.zeros_like(a)
+    torch.cuda.synchronize()
+    e0, e1 = hk.Event(), hk.Event()
+    e0.record(s1)
+    hk.check(lib.hk_memset(ctypes.c_void_p(a.data_ptr()), ctypes.c_int(7), ctypes.c_size_t(a.numel()), s1))
+    e1.record(s1)
+    # s2 copies a -> b only after s1's fill: ordered by the event, not by the host
+    hk.check(lib.hk_stream_wait_event(s2, e1.h))
+    hk.check(lib.hk_copy_kernel(ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(a.data_ptr()),
+                                ctypes.c_size_t(a.numel()), s2))
+    hk.check(lib.hk_stream_sync(s2))
+    assert int(b.min()) == 7 and int(b.max()) == 7
+    e1.sync()
+    done = ctypes.c_int(0)
+    hk.check(lib.hk_event_query(e1.h, ctypes.byref(done)))
+    assert done.value == 1
+    ns = e1.elapsed_ns_since(e0)
+    assert 0 < ns < 50_000_000            # a 16 MiB fill takes microseconds, not 50 ms
+    hk.check(lib.hk_stream_destroy(s1))
+    hk.check(lib.hk_stream_destroy(s2))
+
+
+def test_device_queries(hk, cuda):
+    lib = hk.lib()
+    n = ctypes.c_int()
+    hk.check(lib.hk_device_count(ctypes.byref(n)))
+    assert n.value >= 1
+    cus = ctypes.c_int()
+    hk.check(lib.hk_device_cu_count(0, ctypes.byref(cus)))
+    assert cus.value >= 64
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    hk.check(lib.hk_mem_get_info(ctypes.byref(free), ctypes.byref(total)))
+    assert 0 < free.value <= total.value and total.value > (64 << 30)
+    p = ctypes.c_void_p()
+    hk.check(lib.hk_malloc(ctypes.byref(p), ctypes.c_size_t(1 << 20)))
+    assert p.value and p.value % 256 == 0
+    hk.check(lib.hk_free(p))
+    h = ctypes.c_void_p()
+    hk.check(lib.hk_host_malloc(ctypes.byref(h), ctypes.c_size_t(4096)))
+    assert h.value
+    hk.check(lib.hk_host_free(h))

@@ -217,6 +217,9 @@ CASES = [
     ("C3 reduce sum axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "sum")),
     ("C3 reduce mean axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "mean")),
     ("C3 reduce sum axes(0,1) bf16 [64x512x4096]", lambda hk, t, n: case_reduce(hk, t, n, (0, 1), "sum", True)),
+    ("next: reduce max axis0 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (0,), "max")),
+    ("next: reduce max axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "max")),
+    ("next: reduce prod axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "prod")),
     ("C4 rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "fwd")),
     ("C4 rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "bwd")),
     ("C5 sce fwd bf16 [16384x32000]", lambda hk, t, n: case_sce(hk, t, 2, "fwd")),

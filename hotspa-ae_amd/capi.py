@@ -12,7 +12,8 @@ _lib = None
 
 HK_FLOAT16, HK_FLOAT32, HK_FLOAT64, HK_BFLOAT16, HK_INT64 = 5, 6, 7, 8, 4
 HK_STAT_VAR, HK_STAT_RSTD = 0, 1
-HK_REDUCE_SUM, HK_REDUCE_MEAN = 0, 1
+HK_REDUCE_SUM, HK_REDUCE_MEAN, HK_REDUCE_MAX, HK_REDUCE_MIN, HK_REDUCE_PROD = 0, 1, 2, 3, 4
+REDUCE_OPS = {"sum": 0, "mean": 1, "max": 2, "min": 3, "prod": 4}
 
 DTYPES = {"uint8": 0, "int8": 1, "int16": 2, "int32": 3, "int64": 4, "fp16": 5, "fp32": 6,
           "fp64": 7, "bf16": 8, "bool": 9}
@@ -239,7 +240,7 @@ def reduce(x, out, axes, op="sum", workspace=None, stream=None):
     wsb = 0 if workspace is None else workspace.numel() * workspace.element_size()
     check(lib().hk_reduce(dtype_code(x), dtype_code(out), _ptr(x), _ptr(out), ctypes.c_int(len(shape)), _arr(shape),
                           _arr(strides), ctypes.c_int(len(axes)), _arr(axes),
-                          ctypes.c_int(HK_REDUCE_MEAN if op == "mean" else HK_REDUCE_SUM), _ptr(workspace),
+                          ctypes.c_int(REDUCE_OPS[op]), _ptr(workspace),
                           ctypes.c_size_t(wsb), stream if stream is not None else current_stream()))
     return workspace
 

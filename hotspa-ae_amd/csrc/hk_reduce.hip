@@ -1,4 +1,4 @@
-// Reduce sum / mean over arbitrary axes for gfx950.
+// Reduce sum / mean / max / min / product over arbitrary axes for gfx950.
 //
 // The host merges neighbouring dimensions of the same kind (reduced / kept)
 // that are contiguous in memory, then picks one of three kernels:
@@ -11,10 +11,12 @@
 //           workgroups, fp32 partials are folded by a second small launch.
 //   generic any strided layout    : one thread per output element.
 // bf16 / fp16 accumulate in fp32; mean multiplies the final sum by
-// float(1 / reduce_num).
+// float(1 / reduce_num).  Every kernel takes the reduction (identity + combine)
+// as a type, so all five share the same planning and memory access.
 #include "hk_common.cuh"
 
 #include <algorithm>
+#include <limits>
 #include <type_traits>
 #include <vector>
 
@@ -46,13 +48,53 @@ __device__ __forceinline__ ACC project(ACC v, float factor, int is_mean) {
   else return ACC(float(v) * factor);
 }
 
-template <typename ACC>
-__device__ __forceinline__ ACC block_sum_lds(ACC v, ACC* lds) {
+// The reductions: identity element and combine.  Max / min return a NaN as soon as one operand is a NaN,
+// as (isnan(a) || a > b) ? a : b does in the reference (ReduceMax.cu:10-14, ReduceMin.cu:10-14); their
+// identities are -inf / +inf (the integer type's extremes for integers); the product starts from 1
+// (ReduceProd.cu:8-24).
+template <typename A> __device__ __forceinline__ bool is_nan(A v) {
+  if constexpr (std::is_floating_point<A>::value) return v != v;
+  else return false;
+}
+struct RSum {
+  template <typename A> static __device__ __forceinline__ A identity() { return A(0); }
+  template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return a + b; }
+};
+struct RProd {
+  template <typename A> static __device__ __forceinline__ A identity() { return A(1); }
+  template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return a * b; }
+};
+struct RMax {
+  template <typename A> static __device__ __forceinline__ A identity() {
+    if constexpr (std::is_floating_point<A>::value) return -std::numeric_limits<A>::infinity();
+    else return std::numeric_limits<A>::lowest();
+  }
+  template <typename A> static __device__ __forceinline__ A apply(A a, A b) {
+    return (is_nan(a) || a > b) ? a : (is_nan(b) ? b : (a > b ? a : b));
+  }
+};
+struct RMin {
+  template <typename A> static __device__ __forceinline__ A identity() {
+    if constexpr (std::is_floating_point<A>::value) return std::numeric_limits<A>::infinity();
+    else return std::numeric_limits<A>::max();
+  }
+  template <typename A> static __device__ __forceinline__ A apply(A a, A b) {
+    return (is_nan(a) || a < b) ? a : (is_nan(b) ? b : (a < b ? a : b));
+  }
+};
+// the float face the wave / block reduction helpers expect
+template <typename R> struct AsFloatOp {
+  static __device__ __forceinline__ float identity() { return R::template identity<float>(); }
+  static __device__ __forceinline__ float apply(float a, float b) { return R::template apply<float>(a, b); }
+};
+
+template <typename R, typename ACC>
+__device__ __forceinline__ ACC block_reduce_lds(ACC v, ACC* lds) {
   const int tid = threadIdx.x;
   lds[tid] = v;
   __syncthreads();
   for (int s = blockDim.x >> 1; s > 0; s >>= 1) {
-    if (tid < s) lds[tid] += lds[tid + s];
+    if (tid < s) lds[tid] = R::template apply<ACC>(lds[tid], lds[tid + s]);
     __syncthreads();
   }
   ACC r = lds[0];
@@ -76,7 +118,7 @@ struct InnerArgs {
   int is_mean;
 };
 
-template <typename T, typename OUT_T, bool WAVE_ROW>
+template <typename T, typename OUT_T, bool WAVE_ROW, typename R>
 __global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
 void reduce_inner_vec_kernel(InnerArgs a) {
   constexpr int VEC = VecIO<T>::N;
@@ -96,7 +138,7 @@ void reduce_inner_vec_kernel(InnerArgs a) {
 
   float acc[U];
 #pragma unroll
-  for (int u = 0; u < U; ++u) acc[u] = 0.f;
+  for (int u = 0; u < U; ++u) acc[u] = R::template identity<float>();
   int64_t v = t;
   for (; v + int64_t(U - 1) * tpr < nvec; v += int64_t(U) * tpr) {
     u32x4 r[U];
@@ -107,23 +149,24 @@ void reduce_inner_vec_kernel(InnerArgs a) {
       float f[VEC];
       VecIO<T>::unpack(r[u], f);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[u] += f[j];
+      for (int j = 0; j < VEC; ++j) acc[u] = R::apply(acc[u], f[j]);
     }
   }
   for (; v < nvec; v += tpr) {
     float f[VEC];
     VecIO<T>::unpack(ld16(p + v * VEC), f);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[0] += f[j];
+    for (int j = 0; j < VEC; ++j) acc[0] = R::apply(acc[0], f[j]);
   }
   // scalar tail of the last split
   for (int64_t c = c0 + nvec * VEC + t; c < c1; c += tpr)
-    acc[1] += Cvt<T>::load(static_cast<const T*>(a.in) + row * a.row_stride + c);
-  float s = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+    acc[1] = R::apply(acc[1], Cvt<T>::load(static_cast<const T*>(a.in) + row * a.row_stride + c));
+  float s = R::apply(R::apply(R::apply(acc[0], acc[1]), R::apply(acc[2], acc[3])),
+                     R::apply(R::apply(acc[4], acc[5]), R::apply(acc[6], acc[7])));
   if constexpr (WAVE_ROW) {
-    s = wave_sum(s);
+    s = wave_allreduce<AsFloatOp<R>>(s);
   } else {
-    s = block_allreduce<OpSum>(s, red, int(blockDim.x >> 6));
+    s = block_allreduce<AsFloatOp<R>>(s, red, int(blockDim.x >> 6));
   }
   if (t == 0) {
     if (a.nsplit == 1) st_acc<OUT_T, float>(static_cast<OUT_T*>(a.out) + row, project<float>(s, a.factor, a.is_mean));
@@ -132,16 +175,16 @@ void reduce_inner_vec_kernel(InnerArgs a) {
 }
 
 // inner reduction, scalar path: any dtype / alignment; one workgroup per row
-template <typename T, typename ACC, typename OUT_T>
+template <typename T, typename ACC, typename OUT_T, typename R>
 __global__ __launch_bounds__(256)
 void reduce_inner_scalar_kernel(const T* in, OUT_T* out, int64_t rows, int64_t row_stride,
                                 int64_t cols, float factor, int is_mean) {
   __shared__ ACC lds[256];
   const int64_t row = blockIdx.x;
   const T* p = in + row * row_stride;
-  ACC acc = ACC(0);
-  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) acc += ld_acc<T, ACC>(p + c);
-  acc = block_sum_lds<ACC>(acc, lds);
+  ACC acc = R::template identity<ACC>();
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) acc = R::template apply<ACC>(acc, ld_acc<T, ACC>(p + c));
+  acc = block_reduce_lds<R, ACC>(acc, lds);
   if (threadIdx.x == 0) st_acc<OUT_T, ACC>(out + row, project<ACC>(acc, factor, is_mean));
 }
 
@@ -160,7 +203,7 @@ struct OuterArgs {
   int is_mean;
 };
 
-template <typename T, typename OUT_T>
+template <typename T, typename OUT_T, typename R>
 __global__ __launch_bounds__(1024)
 void reduce_outer_vec_kernel(OuterArgs a) {
   constexpr int VEC = VecIO<T>::N;
@@ -180,7 +223,7 @@ void reduce_outer_vec_kernel(OuterArgs a) {
 
   float acc[VEC];
 #pragma unroll
-  for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+  for (int j = 0; j < VEC; ++j) acc[j] = R::template identity<float>();
   if (col_ok) {
     int64_t r = r0 + w;
     for (; r + int64_t(U - 1) * wy < r1; r += int64_t(U) * wy) {
@@ -192,14 +235,14 @@ void reduce_outer_vec_kernel(OuterArgs a) {
         float f[VEC];
         VecIO<T>::unpack(v[u], f);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] += f[j];
+        for (int j = 0; j < VEC; ++j) acc[j] = R::apply(acc[j], f[j]);
       }
     }
     for (; r < r1; r += wy) {
       float f[VEC];
       VecIO<T>::unpack(ld16(p + r * a.r_stride), f);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] += f[j];
+      for (int j = 0; j < VEC; ++j) acc[j] = R::apply(acc[j], f[j]);
     }
   }
   // fold the waves of the block: lane-major layout keeps LDS accesses conflict-free
@@ -208,8 +251,8 @@ void reduce_outer_vec_kernel(OuterArgs a) {
   __syncthreads();
   // thread (w, lane) finishes element j = w, w + wy, ... of its lane's vector
   for (int j = w; j < VEC; j += wy) {
-    float s = 0.f;
-    for (int k = 0; k < wy; ++k) s += lds[(k * VEC + j) * kWave + lane];
+    float s = R::template identity<float>();
+    for (int k = 0; k < wy; ++k) s = R::apply(s, lds[(k * VEC + j) * kWave + lane]);
     if (col_ok) {
       if (a.rsplit == 1)
         st_acc<OUT_T, float>(static_cast<OUT_T*>(a.out) + b * a.C + c + j, project<float>(s, a.factor, a.is_mean));
@@ -220,7 +263,7 @@ void reduce_outer_vec_kernel(OuterArgs a) {
 }
 
 // folds float partials [nparts, n] -> OUT_T [n]
-template <typename OUT_T>
+template <typename OUT_T, typename R>
 __global__ __launch_bounds__(256)
 void reduce_fold_partials_kernel(const float* part, OUT_T* out, int nparts, int64_t n, float factor,
                                  int is_mean) {
@@ -230,7 +273,7 @@ void reduce_fold_partials_kernel(const float* part, OUT_T* out, int nparts, int6
   __shared__ float lds[4][kWave];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int64_t i = int64_t(blockIdx.x) * kWave + lane;
-  float acc = 0.f;
+  float acc = R::template identity<float>();
   if (i < n) {
     int k = w;
     for (; k + (U - 1) * 4 < nparts; k += U * 4) {
@@ -238,29 +281,29 @@ void reduce_fold_partials_kernel(const float* part, OUT_T* out, int nparts, int6
 #pragma unroll
       for (int u = 0; u < U; ++u) v[u] = part[int64_t(k + u * 4) * n + i];
 #pragma unroll
-      for (int u = 0; u < U; ++u) acc += v[u];
+      for (int u = 0; u < U; ++u) acc = R::apply(acc, v[u]);
     }
-    for (; k < nparts; k += 4) acc += part[int64_t(k) * n + i];
+    for (; k < nparts; k += 4) acc = R::apply(acc, part[int64_t(k) * n + i]);
   }
   lds[w][lane] = acc;
   __syncthreads();
   if (w == 0 && i < n) {
-    const float s = (lds[0][lane] + lds[1][lane]) + (lds[2][lane] + lds[3][lane]);
+    const float s = R::apply(R::apply(lds[0][lane], lds[1][lane]), R::apply(lds[2][lane], lds[3][lane]));
     st_acc<OUT_T, float>(out + i, project<float>(s, factor, is_mean));
   }
 }
 
 // outer reduction, scalar path: one thread per output column, any dtype
-template <typename T, typename ACC, typename OUT_T>
+template <typename T, typename ACC, typename OUT_T, typename R>
 __global__ __launch_bounds__(256)
-void reduce_outer_scalar_kernel(const T* in, OUT_T* out, int64_t B, int64_t R, int64_t C,
+void reduce_outer_scalar_kernel(const T* in, OUT_T* out, int64_t B, int64_t NR, int64_t C,
                                 int64_t b_stride, int64_t r_stride, float factor, int is_mean) {
   const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= B * C) return;
   const int64_t b = i / C, c = i - b * C;
   const T* p = in + b * b_stride + c;
-  ACC acc = ACC(0);
-  for (int64_t r = 0; r < R; ++r) acc += ld_acc<T, ACC>(p + r * r_stride);
+  ACC acc = R::template identity<ACC>();
+  for (int64_t r = 0; r < NR; ++r) acc = R::template apply<ACC>(acc, ld_acc<T, ACC>(p + r * r_stride));
   st_acc<OUT_T, ACC>(out + i, project<ACC>(acc, factor, is_mean));
 }
 
@@ -275,7 +318,7 @@ struct GenericMeta {
   int64_t n_out, n_red_total;
 };
 
-template <typename T, typename ACC, typename OUT_T>
+template <typename T, typename ACC, typename OUT_T, typename R>
 __global__ __launch_bounds__(256)
 void reduce_generic_kernel(const T* in, OUT_T* out, GenericMeta m, float factor, int is_mean) {
   const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -286,7 +329,7 @@ void reduce_generic_kernel(const T* in, OUT_T* out, GenericMeta m, float factor,
     base += (rem - q * m.keep_size[d]) * m.keep_stride[d];
     rem = q;
   }
-  ACC acc = ACC(0);
+  ACC acc = R::template identity<ACC>();
   for (int64_t k = 0; k < m.n_red_total; ++k) {
     int64_t r = k, off = base;
     for (int d = m.n_red - 1; d >= 0; --d) {
@@ -294,7 +337,7 @@ void reduce_generic_kernel(const T* in, OUT_T* out, GenericMeta m, float factor,
       off += (r - q * m.red_size[d]) * m.red_stride[d];
       r = q;
     }
-    acc += ld_acc<T, ACC>(in + off);
+    acc = R::template apply<ACC>(acc, ld_acc<T, ACC>(in + off));
   }
   st_acc<OUT_T, ACC>(out + i, project<ACC>(acc, factor, is_mean));
 }
@@ -465,7 +508,7 @@ static GenericMeta generic_meta(const ReducePlan& p) {
 }
 
 // fast kernels: T in {float, bf16, fp16}, fp32 accumulation
-template <typename T, typename OUT_T>
+template <typename T, typename OUT_T, typename R>
 static int reduce_fast(const ReducePlan& p, const void* in, void* out, float factor, int is_mean,
                        void* ws, size_t ws_bytes, hipStream_t st, bool* handled) {
   *handled = false;
@@ -487,16 +530,16 @@ static int reduce_fast(const ReducePlan& p, const void* in, void* out, float fac
     profile_before(st);
     if (s.tpr == 64) {
       dim3 grid(unsigned((p.rows + 3) / 4), unsigned(s.nsplit)), block(256);
-      hipLaunchKernelGGL((reduce_inner_vec_kernel<T, OUT_T, true>), grid, block, 0, st, a);
+      hipLaunchKernelGGL((reduce_inner_vec_kernel<T, OUT_T, true, R>), grid, block, 0, st, a);
     } else {
       dim3 grid(unsigned(p.rows), unsigned(s.nsplit)), block{unsigned(s.tpr)};
-      hipLaunchKernelGGL((reduce_inner_vec_kernel<T, OUT_T, false>), grid, block, 0, st, a);
+      hipLaunchKernelGGL((reduce_inner_vec_kernel<T, OUT_T, false, R>), grid, block, 0, st, a);
     }
     profile_after(st);
     int rc = launch_check("reduce_inner_vec_kernel");
     if (rc != HK_OK || s.nsplit == 1) return rc;
     // second pass over the fp32 partials [rows, nsplit]
-    hipLaunchKernelGGL((reduce_inner_scalar_kernel<float, float, OUT_T>), dim3(unsigned(p.rows)), dim3(256), 0, st,
+    hipLaunchKernelGGL((reduce_inner_scalar_kernel<float, float, OUT_T, R>), dim3(unsigned(p.rows)), dim3(256), 0, st,
                        static_cast<const float*>(ws), static_cast<OUT_T*>(out), p.rows, int64_t(s.nsplit),
                        int64_t(s.nsplit), factor, is_mean);
     return launch_check("reduce_inner_scalar_kernel");
@@ -521,48 +564,74 @@ static int reduce_fast(const ReducePlan& p, const void* in, void* out, float fac
     dim3 grid(unsigned(col_tiles), unsigned(s.rsplit), unsigned(p.B)), block{unsigned(64 * s.wy)};
     const size_t lds = size_t(s.wy) * 64 * VEC * sizeof(float);
     profile_before(st);
-    hipLaunchKernelGGL((reduce_outer_vec_kernel<T, OUT_T>), grid, block, lds, st, a);
+    hipLaunchKernelGGL((reduce_outer_vec_kernel<T, OUT_T, R>), grid, block, lds, st, a);
     profile_after(st);
     int rc = launch_check("reduce_outer_vec_kernel");
     if (rc != HK_OK || s.rsplit == 1) return rc;
     const int64_t n = p.B * p.C;
-    hipLaunchKernelGGL((reduce_fold_partials_kernel<OUT_T>), dim3(unsigned((n + 63) / 64)), dim3(256), 0, st,
+    hipLaunchKernelGGL((reduce_fold_partials_kernel<OUT_T, R>), dim3(unsigned((n + 63) / 64)), dim3(256), 0, st,
                        static_cast<const float*>(ws), static_cast<OUT_T*>(out), s.rsplit, n, factor, is_mean);
     return launch_check("reduce_fold_partials_kernel");
   }
   return HK_OK;
 }
 
-template <typename T, typename ACC, typename OUT_T>
+template <typename T, typename ACC, typename OUT_T, typename R>
 static int reduce_slow(const ReducePlan& p, const void* in, void* out, float factor, int is_mean,
                        hipStream_t st) {
   const T* ip = static_cast<const T*>(in);
   OUT_T* op = static_cast<OUT_T*>(out);
   if (p.kind == PLAN_INNER) {
     HK_REQUIRE(p.rows <= 0x7fffffffLL, HK_ERR_INVALID, "hk_reduce: too many rows");
-    hipLaunchKernelGGL((reduce_inner_scalar_kernel<T, ACC, OUT_T>), dim3(unsigned(p.rows)), dim3(256), 0, st, ip, op,
+    hipLaunchKernelGGL((reduce_inner_scalar_kernel<T, ACC, OUT_T, R>), dim3(unsigned(p.rows)), dim3(256), 0, st, ip, op,
                        p.rows, p.row_stride, p.cols, factor, is_mean);
     return launch_check("reduce_inner_scalar_kernel");
   }
   if (p.kind == PLAN_OUTER) {
     const int64_t n = p.B * p.C;
-    hipLaunchKernelGGL((reduce_outer_scalar_kernel<T, ACC, OUT_T>), dim3(unsigned((n + 255) / 256)), dim3(256), 0, st,
+    hipLaunchKernelGGL((reduce_outer_scalar_kernel<T, ACC, OUT_T, R>), dim3(unsigned((n + 255) / 256)), dim3(256), 0, st,
                        ip, op, p.B, p.R, p.C, p.b_stride, p.r_stride, factor, is_mean);
     return launch_check("reduce_outer_scalar_kernel");
   }
   GenericMeta m = generic_meta(p);
-  hipLaunchKernelGGL((reduce_generic_kernel<T, ACC, OUT_T>), dim3(unsigned((m.n_out + 255) / 256)), dim3(256), 0, st,
+  hipLaunchKernelGGL((reduce_generic_kernel<T, ACC, OUT_T, R>), dim3(unsigned((m.n_out + 255) / 256)), dim3(256), 0, st,
                      ip, op, m, factor, is_mean);
   return launch_check("reduce_generic_kernel");
 }
 
-template <typename T, typename OUT_T>
+template <typename T, typename OUT_T, typename R>
 static int reduce_float_like(const ReducePlan& p, const void* in, void* out, float factor, int is_mean,
                              void* ws, size_t ws_bytes, hipStream_t st) {
   bool handled = false;
-  int rc = reduce_fast<T, OUT_T>(p, in, out, factor, is_mean, ws, ws_bytes, st, &handled);
+  int rc = reduce_fast<T, OUT_T, R>(p, in, out, factor, is_mean, ws, ws_bytes, st, &handled);
   if (rc != HK_OK || handled) return rc;
-  return reduce_slow<T, float, OUT_T>(p, in, out, factor, is_mean, st);
+  return reduce_slow<T, float, OUT_T, R>(p, in, out, factor, is_mean, st);
+}
+
+// every dtype of one reduction
+template <typename R>
+static int reduce_typed(const ReducePlan& q, int in_dtype, int out_dtype, const void* in, void* out, float factor,
+                        int is_mean, void* workspace, size_t workspace_bytes, hipStream_t st) {
+#define HK_RED_SLOW(T) return reduce_slow<T, AccOf<T>::type, T, R>(q, in, out, factor, is_mean, st)
+  switch (in_dtype) {
+    case HK_FLOAT32: return reduce_float_like<float, float, R>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
+    case HK_BFLOAT16:
+      if (out_dtype == HK_FLOAT32) return reduce_float_like<bf16, float, R>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
+      return reduce_float_like<bf16, bf16, R>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
+    case HK_FLOAT16:
+      if (out_dtype == HK_FLOAT32) return reduce_float_like<fp16, float, R>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
+      return reduce_float_like<fp16, fp16, R>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
+    case HK_FLOAT64: HK_RED_SLOW(double);
+    case HK_UINT8: HK_RED_SLOW(uint8_t);
+    case HK_INT8: HK_RED_SLOW(int8_t);
+    case HK_INT16: HK_RED_SLOW(int16_t);
+    case HK_INT32: HK_RED_SLOW(int32_t);
+    case HK_INT64: HK_RED_SLOW(int64_t);
+    default:
+      set_last_error("hk_reduce: not implemented for dtype %d", in_dtype);
+      return HK_ERR_UNSUPPORTED;
+  }
+#undef HK_RED_SLOW
 }
 
 } // namespace hk
@@ -591,7 +660,8 @@ int hk_reduce_workspace_bytes(int in_dtype, int ndim, const int64_t* shape, cons
 int hk_reduce(int in_dtype, int out_dtype, const void* in, void* out, int ndim, const int64_t* shape,
               const int64_t* strides, int naxes, const int64_t* axes, int op, void* workspace,
               size_t workspace_bytes, hkStream_t stream) {
-  HK_REQUIRE(op == HK_REDUCE_SUM || op == HK_REDUCE_MEAN, HK_ERR_UNSUPPORTED, "hk_reduce: reduction %d not implemented", op);
+  HK_REQUIRE(op == HK_REDUCE_SUM || op == HK_REDUCE_MEAN || op == HK_REDUCE_MAX || op == HK_REDUCE_MIN ||
+             op == HK_REDUCE_PROD, HK_ERR_UNSUPPORTED, "hk_reduce: reduction %d not implemented", op);
   ReducePlan p;
   int rc = make_plan(ndim, shape, strides, naxes, axes, &p, "hk_reduce");
   if (rc != HK_OK) return rc;
@@ -601,43 +671,33 @@ int hk_reduce(int in_dtype, int out_dtype, const void* in, void* out, int ndim, 
     HK_REQUIRE(out_dtype == in_dtype, HK_ERR_UNSUPPORTED, "hk_reduce: a reduction over no axes cannot change the dtype");
     return hk_strided_copy(in_dtype, in, out, ndim, shape, strides, stream);
   }
-  if (p.n_red == 0) {
+  const bool additive = op == HK_REDUCE_SUM || op == HK_REDUCE_MEAN;
+  if (p.n_red == 0 && additive) {
     // empty sums are 0; an empty mean is 0 * (1/0) = NaN for floating types (all-ones bytes are a NaN in each)
     const bool floating = out_dtype == HK_FLOAT16 || out_dtype == HK_BFLOAT16 || out_dtype == HK_FLOAT32 || out_dtype == HK_FLOAT64;
     const size_t es = dtype_size(out_dtype);
     HK_REQUIRE(es > 0, HK_ERR_UNSUPPORTED, "hk_reduce: dtype %d not implemented", out_dtype);
     return hk_memset(out, (op == HK_REDUCE_MEAN && floating) ? 0xFF : 0, size_t(p.n_out) * es, stream);
   }
-  HK_REQUIRE(in, HK_ERR_INVALID, "hk_reduce: null input");
+  HK_REQUIRE(in || p.n_red == 0, HK_ERR_INVALID, "hk_reduce: null input");
   HK_REQUIRE((p.n_out + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_reduce: output too large");
   const int is_mean = op == HK_REDUCE_MEAN;
   const float factor = is_mean ? 1.0f / float(size_t(p.n_red)) : 1.0f;
   hipStream_t st = as_hip(stream);
   const bool in16 = in_dtype == HK_BFLOAT16 || in_dtype == HK_FLOAT16;
-  HK_REQUIRE(out_dtype == in_dtype || (in16 && out_dtype == HK_FLOAT32), HK_ERR_UNSUPPORTED,
-             "hk_reduce: output dtype %d not implemented for input dtype %d", out_dtype, in_dtype);
+  // a wider output exists for sums and products of 16-bit data (ReduceSum.cu:28-37, ReduceProd.cu:26-37)
+  const bool widen_ok = in16 && out_dtype == HK_FLOAT32 && op != HK_REDUCE_MAX && op != HK_REDUCE_MIN;
+  HK_REQUIRE(out_dtype == in_dtype || widen_ok, HK_ERR_UNSUPPORTED,
+             "hk_reduce: output dtype %d not implemented for input dtype %d and reduction %d", out_dtype, in_dtype, op);
   ReducePlan q = p;
-  if (p.kind == PLAN_COPYLIKE) q.kind = PLAN_GENERIC;
-#define HK_RED_SLOW(T) return reduce_slow<T, AccOf<T>::type, T>(q, in, out, factor, is_mean, st)
-  switch (in_dtype) {
-    case HK_FLOAT32: return reduce_float_like<float, float>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
-    case HK_BFLOAT16:
-      if (out_dtype == HK_FLOAT32) return reduce_float_like<bf16, float>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
-      return reduce_float_like<bf16, bf16>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
-    case HK_FLOAT16:
-      if (out_dtype == HK_FLOAT32) return reduce_float_like<fp16, float>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
-      return reduce_float_like<fp16, fp16>(q, in, out, factor, is_mean, workspace, workspace_bytes, st);
-    case HK_FLOAT64: HK_RED_SLOW(double);
-    case HK_UINT8: HK_RED_SLOW(uint8_t);
-    case HK_INT8: HK_RED_SLOW(int8_t);
-    case HK_INT16: HK_RED_SLOW(int16_t);
-    case HK_INT32: HK_RED_SLOW(int32_t);
-    case HK_INT64: HK_RED_SLOW(int64_t);
-    default:
-      set_last_error("hk_reduce: not implemented for dtype %d", in_dtype);
-      return HK_ERR_UNSUPPORTED;
+  // an empty reduced extent (max / min / prod) writes the identity: the one-thread-per-output kernel does that
+  if (p.kind == PLAN_COPYLIKE || p.n_red == 0) q.kind = PLAN_GENERIC;
+  switch (op) {
+    case HK_REDUCE_MAX: return reduce_typed<RMax>(q, in_dtype, out_dtype, in, out, factor, 0, workspace, workspace_bytes, st);
+    case HK_REDUCE_MIN: return reduce_typed<RMin>(q, in_dtype, out_dtype, in, out, factor, 0, workspace, workspace_bytes, st);
+    case HK_REDUCE_PROD: return reduce_typed<RProd>(q, in_dtype, out_dtype, in, out, factor, 0, workspace, workspace_bytes, st);
+    default: return reduce_typed<RSum>(q, in_dtype, out_dtype, in, out, factor, is_mean, workspace, workspace_bytes, st);
   }
-#undef HK_RED_SLOW
 }
 
 } // extern "C"

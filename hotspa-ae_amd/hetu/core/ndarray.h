@@ -133,6 +133,18 @@ class NDArray {
                       StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY) {
     return reduce(input, kMEAN, axes, keepdims, stream_id, output);
   }
+  static NDArray max(const NDArray& input, const HTAxes& axes = HTAxes(), bool keepdims = false,
+                     StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY) {
+    return reduce(input, kMAX, axes, keepdims, stream_id, output);
+  }
+  static NDArray min(const NDArray& input, const HTAxes& axes = HTAxes(), bool keepdims = false,
+                     StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY) {
+    return reduce(input, kMIN, axes, keepdims, stream_id, output);
+  }
+  static NDArray prod(const NDArray& input, const HTAxes& axes = HTAxes(), bool keepdims = false,
+                      StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY) {
+    return reduce(input, kPROD, axes, keepdims, stream_id, output);
+  }
   static NDArrayList layernorm(const NDArray& input, const NDArray& bn_scale, const NDArray& bn_bias,
                                const HTShape& normalized_shape, double eps = 0.01,
                                StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY,

@@ -48,6 +48,9 @@ DECLARE_KERNEL_CPU_AND_CUDA(LayerNormGradient, const NDArray&, const NDArray&, c
 DECLARE_KERNEL_CPU_AND_CUDA(Reduce, const NDArray&, NDArray&, const HTAxes&, ReductionType, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(ReduceMean, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(ReduceSum, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(ReduceMax, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(ReduceMin, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(ReduceProd, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(Softmax, const NDArray&, NDArray&, int64_t, const Stream&);
 // y, dy, dx, dim
 DECLARE_KERNEL_CPU_AND_CUDA(SoftmaxGradient, const NDArray&, const NDArray&, NDArray&, int64_t, const Stream&);

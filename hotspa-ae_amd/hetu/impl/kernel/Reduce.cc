@@ -1,8 +1,8 @@
-// ReduceCuda / ReduceSumCuda / ReduceMeanCuda: arguments and meaning of
-// hetu/impl/kernel/Reduce.cu:21-59, ReduceSum.cu:25-42 and ReduceMean.cu:35-55
-// of the reference.  The input may have any strides (the kernel plans on shape
-// and strides); the output is written dense.  Max / min / prod are not on this
-// path and raise not_implemented.
+// ReduceCuda / ReduceSumCuda / ReduceMeanCuda / ReduceMaxCuda / ReduceMinCuda /
+// ReduceProdCuda: arguments and meaning of hetu/impl/kernel/Reduce.cu:21-59,
+// ReduceSum.cu:25-42, ReduceMean.cu:35-55, ReduceMax.cu:28-41, ReduceMin.cu:28-41
+// and ReduceProd.cu:26-45 of the reference.  The input may have any strides (the
+// kernel plans on shape and strides); the output is written dense.
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
 
@@ -52,6 +52,21 @@ void ReduceMeanCuda(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes
   LaunchReduce(in_arr, out_arr, axes, num_ax, HK_REDUCE_MEAN, stream);
 }
 
+void ReduceMaxCuda(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax,
+                   const Stream& stream) {
+  LaunchReduce(in_arr, out_arr, axes, num_ax, HK_REDUCE_MAX, stream);
+}
+
+void ReduceMinCuda(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax,
+                   const Stream& stream) {
+  LaunchReduce(in_arr, out_arr, axes, num_ax, HK_REDUCE_MIN, stream);
+}
+
+void ReduceProdCuda(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax,
+                    const Stream& stream) {
+  LaunchReduce(in_arr, out_arr, axes, num_ax, HK_REDUCE_PROD, stream);
+}
+
 void ReduceCuda(const NDArray& input, NDArray& output, const HTAxes& axes, ReductionType red_type,
                 const Stream& stream) {
   HT_ASSERT_CUDA_DEVICE(input);
@@ -60,9 +75,9 @@ void ReduceCuda(const NDArray& input, NDArray& output, const HTAxes& axes, Reduc
   switch (red_type) {
     case kSUM: ReduceSumCuda(input, output, parsed_axes.data(), int64_t(parsed_axes.size()), stream); break;
     case kMEAN: ReduceMeanCuda(input, output, parsed_axes.data(), int64_t(parsed_axes.size()), stream); break;
-    case kMAX:
-    case kMIN:
-    case kPROD: HT_NOT_IMPLEMENTED << "Reduction " << red_type << " is not part of the row-wise kernel set"; break;
+    case kMAX: ReduceMaxCuda(input, output, parsed_axes.data(), int64_t(parsed_axes.size()), stream); break;
+    case kMIN: ReduceMinCuda(input, output, parsed_axes.data(), int64_t(parsed_axes.size()), stream); break;
+    case kPROD: ReduceProdCuda(input, output, parsed_axes.data(), int64_t(parsed_axes.size()), stream); break;
     case kNONE: HT_NOT_IMPLEMENTED << "Reduction type cannot be none"; break;
     default: HT_VALUE_ERROR << "Unknown reduction type: " << static_cast<int32_t>(red_type);
   }
@@ -77,6 +92,15 @@ void ReduceSumCpu(const NDArray&, NDArray&, const int64_t*, int64_t, const Strea
 }
 void ReduceMeanCpu(const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&) {
   HT_NOT_IMPLEMENTED << "ReduceMean has no host kernel in this build; move the arrays to the accelerator";
+}
+void ReduceMaxCpu(const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&) {
+  HT_NOT_IMPLEMENTED << "ReduceMax has no host kernel in this build; move the arrays to the accelerator";
+}
+void ReduceMinCpu(const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&) {
+  HT_NOT_IMPLEMENTED << "ReduceMin has no host kernel in this build; move the arrays to the accelerator";
+}
+void ReduceProdCpu(const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&) {
+  HT_NOT_IMPLEMENTED << "ReduceProd has no host kernel in this build; move the arrays to the accelerator";
 }
 
 } // namespace impl

@@ -51,7 +51,8 @@ enum {
 };
 
 /* ---- reduction codes: hetu/core/reduction_type.h:7-15 (kSUM, kMEAN) ------ */
-enum { HK_REDUCE_SUM = 0, HK_REDUCE_MEAN = 1 };
+/* values of hetu::ReductionType (hetu/core/reduction_type.h:7-15) */
+enum { HK_REDUCE_SUM = 0, HK_REDUCE_MEAN = 1, HK_REDUCE_MAX = 2, HK_REDUCE_MIN = 3, HK_REDUCE_PROD = 4 };
 
 /* second per-row statistic written/read by the LayerNorm entries */
 enum {
@@ -227,7 +228,8 @@ HK_API int hk_sce_dense_bwd(int dtype, const void* logits, const void* labels,
                             hkStream_t stream);
 
 /* ======================================================================== *
- * Reduce sum / mean over a set of axes of a (possibly strided) array.
+ * Reduce sum / mean / max / min / product over a set of axes of a (possibly
+ * strided) array.
  * shape / strides (in elements) describe the input; axes must already be
  * wrapped to [0, ndim), may be unsorted or repeated (sorted + de-duplicated
  * inside, hetu/impl/kernel/Reduce.cuh:765-768).  The output is written dense,
@@ -236,8 +238,14 @@ HK_API int hk_sce_dense_bwd(int dtype, const void* logits, const void* labels,
  * out_dtype may be HK_FLOAT32 for bf16 / fp16 input (ReduceSum.cu:28-37).
  * naxes = 0 writes the dense copy of the input; a reduced extent of 0 writes
  * the empty sum 0 (mean: NaN for floating types); no kept element, no write.
- * Replaces ReduceSumCuda / ReduceMeanCuda (ReduceSum.cu:25-42,
- * ReduceMean.cu:35-55) and launch_reduce_kernel (Reduce.cuh:757-844).
+ * Max / min return a NaN once one has been seen and start from -inf / +inf (the
+ * type's extremes for integers); the product starts from 1; an empty reduced
+ * extent writes those identities (ReduceMax.cu:10-25, ReduceMin.cu:10-25,
+ * ReduceProd.cu:8-24).  A widened fp32 output exists for sum, mean and product.
+ * Replaces ReduceSumCuda / ReduceMeanCuda / ReduceMaxCuda / ReduceMinCuda /
+ * ReduceProdCuda (ReduceSum.cu:25-42, ReduceMean.cu:35-55, ReduceMax.cu:28-41,
+ * ReduceMin.cu:28-41, ReduceProd.cu:26-45) and launch_reduce_kernel
+ * (Reduce.cuh:757-844).
  * ======================================================================== */
 HK_API int hk_reduce_workspace_bytes(int in_dtype, int ndim, const int64_t* shape,
                                      const int64_t* strides, int naxes, const int64_t* axes,

@@ -221,7 +221,7 @@ def strided_reduce(buf, shape, strides, axes, op="sum", mean_mode=0):
     out_shape = [shape[d] for d in range(ndim) if d not in red]
     out = np.empty(int(np.prod(out_shape, dtype=np.int64)) if out_shape else 1)
     rc = lib().oracle_reduce(_p(buf.reshape(-1), c_f64p), ctypes.c_int(ndim), sh, st, ctypes.c_int(len(axes)), ax,
-                             ctypes.c_int(1 if op == "mean" else 0), ctypes.c_int(mean_mode), _p(out, c_f64p))
+                             ctypes.c_int({"sum": 0, "mean": 1, "max": 2, "min": 3, "prod": 4}[op]), ctypes.c_int(mean_mode), _p(out, c_f64p))
     if rc != 0:
         raise ValueError("oracle_reduce: bad arguments")
     return out.reshape(out_shape if out_shape else [1])

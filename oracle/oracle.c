@@ -387,7 +387,10 @@ ORACLE_API int oracle_reduce(const double* in, int ndim, const int64_t* shape,
       rem /= shape[d];
       base += idx[d] * strides[d];
     }
-    double s = 0.0;
+    /* is_mean doubles as the reduction selector: 0 sum, 1 mean, 2 max, 3 min, 4 product
+     * (hetu::ReductionType order).  Max / min return a NaN once one has been seen and start from
+     * -inf / +inf (ReduceMax.cu:10-25, ReduceMin.cu:10-25); the product starts from 1 (ReduceProd.cu:8-24). */
+    double s = is_mean == 2 ? -INFINITY : is_mean == 3 ? INFINITY : is_mean == 4 ? 1.0 : 0.0;
     for (int64_t k = 0; k < n_red; ++k) {
       int64_t r = k, off = base;
       for (int d = ndim - 1; d >= 0; --d) {
@@ -395,9 +398,13 @@ ORACLE_API int oracle_reduce(const double* in, int ndim, const int64_t* shape,
         off += (r % shape[d]) * strides[d];
         r /= shape[d];
       }
-      s += in[off];
+      const double v = in[off];
+      if (is_mean == 2) s = (isnan(s) || s > v) ? s : v;
+      else if (is_mean == 3) s = (isnan(s) || s < v) ? s : v;
+      else if (is_mean == 4) s *= v;
+      else s += v;
     }
-    if (is_mean) {
+    if (is_mean == 1) {
       if (mean_mode == 1) {
         const float factor = 1.0f / (float)(size_t)n_red;
         s = (double)((float)s * factor);

@@ -302,8 +302,15 @@ def test_reduce_rejects_what_is_not_on_the_path(ops, cuda):
     import torch
     x = torch.ones(4, 8, device=cuda)
     _sync_in()
-    with pytest.raises(ops.NotImplemented_, match="max"):
-        ops.reduce(x, torch.empty(8, device=cuda), [0], "max")
+    out = torch.empty(8, device=cuda)
+    x3, x2 = x * 3, x * 2
+    _sync_in()
+    ops.reduce(x3, out, [0], "max")
+    ops.stream_sync()
+    assert float(out.min()) == 3.0 and float(out.max()) == 3.0
+    ops.reduce(x2, out, [0], "prod")
+    ops.stream_sync()
+    assert float(out.min()) == 16.0
     with pytest.raises(ops.NotImplemented_, match="none"):
         ops.reduce(x, torch.empty(8, device=cuda), [0], "none")
     with pytest.raises(ops.AssertionError_, match="Invalid dimension"):

@@ -126,3 +126,79 @@ def test_degenerate_reductions(hk, cuda):
     hk.reduce(torch.empty((10, 0), device=cuda), torch.empty((0,), device=cuda), [0], "sum")
     torch.cuda.synchronize()
     assert float(untouched[0]) == -7.0
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("op", ["max", "min"])
+def test_max_min_are_exact_selections(hk, cuda, dtype, op):
+    """A maximum / minimum is one of the inputs: the result is known bit for bit in every dtype, whatever
+    order the kernels combine in.  Covers the row, column, split and generic kernels."""
+    import itertools
+    shape = (3, 4, 5, 6)
+    x = helpers.draw(21, shape, dtype=dtype)
+    tx = helpers.to_torch(x, dtype, cuda)
+    f = np.max if op == "max" else np.min
+    for k in range(1, 5):
+        for axes in itertools.combinations(range(4), k):
+            got = helpers.to_numpy(_run(hk, cuda, tx, axes, op)).astype(np.float64)
+            assert np.array_equal(got.reshape(-1), np.asarray(f(x.astype(np.float64), axis=axes)).reshape(-1)), axes
+    for shp, axes in (((257, 4096), (0,)), ((257, 4096), (1,)), ((3, 70000), (1,)), ((20000, 72), (0,)),
+                      ((64, 33, 40), (0, 2)), ((5, 1000, 24), (1,)), ((1, 16384), (1,)), ((9, 1031), (1,))):
+        x = helpers.draw(22 + len(shp), shp, dtype=dtype)
+        tx = helpers.to_torch(x, dtype, cuda)
+        got = helpers.to_numpy(_run(hk, cuda, tx, axes, op)).astype(np.float64)
+        assert np.array_equal(got.reshape(-1), np.asarray(f(x.astype(np.float64), axis=axes)).reshape(-1)), (shp, axes)
+    # a strided view
+    base = helpers.to_torch(helpers.draw(29, (48, 20, 64), dtype=dtype), dtype, cuda)
+    view = base.permute(1, 2, 0)[:, ::2, :]
+    want = f(helpers.to_numpy(view.contiguous()).astype(np.float64), axis=(0, 2))
+    assert np.array_equal(helpers.to_numpy(_run(hk, cuda, view, (0, 2), op)).astype(np.float64).reshape(-1), want.reshape(-1))
+
+
+@pytest.mark.parametrize("op", ["max", "min"])
+def test_max_min_nan_and_infinities(hk, cuda, op):
+    import torch
+    x = helpers.draw(31, (64, 4096), dtype="fp32")
+    x[3, 100] = np.nan
+    x[5, 7] = np.inf
+    x[6, 9] = -np.inf
+    tx = helpers.to_torch(x, "fp32", cuda)
+    for axes in ((1,), (0,)):
+        got = helpers.to_numpy(_run(hk, cuda, tx, axes, op)).astype(np.float64).reshape(-1)
+        want = np.asarray(oracle.reduce(x, list(axes), op)).reshape(-1)
+        assert np.array_equal(np.isnan(got), np.isnan(want)) and np.isnan(want).sum() == 1
+        assert np.array_equal(got[~np.isnan(got)], want[~np.isnan(want)])
+    # an empty reduced extent writes the identity
+    empty = torch.empty((0, 10), device=cuda)
+    ident = -np.inf if op == "max" else np.inf
+    assert np.all(helpers.to_numpy(_run(hk, cuda, empty, (0,), op)) == ident)
+    assert np.all(helpers.to_numpy(_run(hk, cuda, empty.bfloat16(), (0,), op)).astype(np.float64) == ident)
+    # integers: exact, identities are the type's extremes
+    xi = helpers.rng(32).integers(-1000, 1000, size=(17, 33, 9))
+    for tdt in ("int64", "int32", "uint8"):
+        ti = torch.from_numpy(xi).to(hk.torch_dtype(tdt)).to(cuda)
+        ref = ti.cpu().numpy()
+        got = _run(hk, cuda, ti, (0, 2), op).cpu().numpy()
+        assert np.array_equal(got, (ref.max(axis=(0, 2)) if op == "max" else ref.min(axis=(0, 2)))), tdt
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_prod_parity_and_widened_output(hk, cuda, dtype):
+    import torch
+    # factors near 1 keep long products in range; fp32 accumulation against the float64 oracle
+    for shp, axes in (((300, 512), (1,)), ((300, 512), (0,)), ((7, 40, 24), (0, 2)), ((2, 3), (0, 1))):
+        x = helpers.draw(41 + len(shp), shp, "uniform", 0.97, 1.03, dtype)
+        tx = helpers.to_torch(x, dtype, cuda)
+        want = np.asarray(oracle.reduce(x, list(axes), "prod"))
+        helpers.assert_close(_run(hk, cuda, tx, axes, "prod"), want, dtype, "prod %s %s" % (shp, axes))
+        if dtype == "bf16":
+            helpers.assert_close(_run(hk, cuda, tx, axes, "prod", out_dtype=torch.float32), want, "fp32",
+                                 "prod to fp32 %s %s" % (shp, axes), rtol=2e-5)
+    # small integers: exact
+    xi = helpers.rng(43).integers(1, 4, size=(6, 5)).astype(np.float32)
+    got = helpers.to_numpy(_run(hk, cuda, helpers.to_torch(xi, "fp32", cuda), (1,), "prod"))
+    assert np.array_equal(got, xi.prod(axis=1))
+    assert np.all(helpers.to_numpy(_run(hk, cuda, torch.empty((4, 0), device=cuda), (1,), "prod")) == 1.0)
+    # max / min have no widened output
+    with pytest.raises(hk.HkError):
+        _run(hk, cuda, helpers.to_torch(xi, "bf16", cuda), (1,), "max", out_dtype=torch.float32)

@@ -284,6 +284,33 @@ def test_reduce_mean_rounding_modes():
     assert np.allclose(ref, exact, rtol=2e-7)
 
 
+def test_reduce_max_min_prod_against_numpy_and_nan_rule():
+    """Selections are exact; a NaN anywhere in the reduced set wins (numpy's max / min have the same rule);
+    identities are -inf, +inf and 1 (an empty reduced extent); products against numpy float64."""
+    import itertools
+    g = np.random.default_rng(14)
+    x = g.standard_normal((3, 4, 5, 6))
+    for k in range(1, 5):
+        for axes in itertools.combinations(range(4), k):
+            for op, f in (("max", np.max), ("min", np.min)):
+                assert np.array_equal(oracle.reduce(x, list(axes), op).reshape(-1), np.asarray(f(x, axis=axes)).reshape(-1))
+            assert np.allclose(oracle.reduce(x, list(axes), "prod").reshape(-1), np.asarray(np.prod(x, axis=axes)).reshape(-1), **F64)
+    y = x.copy()
+    y[1, 2, 3, 4] = np.nan
+    for op, f in (("max", np.max), ("min", np.min)):
+        got, want = oracle.reduce(y, [1, 3], op), f(y, axis=(1, 3))
+        assert np.array_equal(np.isnan(got), np.isnan(want)) and np.isnan(got).sum() == 1
+        assert np.array_equal(got[~np.isnan(got)], want[~np.isnan(want)])
+    empty = np.zeros((4, 0))
+    assert np.all(oracle.reduce(empty, [1], "max") == -np.inf)
+    assert np.all(oracle.reduce(empty, [1], "min") == np.inf)
+    assert np.all(oracle.reduce(empty, [1], "prod") == 1.0)
+    assert np.all(oracle.reduce(empty, [1], "sum") == 0.0)
+    # all-equal and single-element rows
+    assert np.array_equal(oracle.reduce(np.full((3, 7), -2.5), [1], "max"), np.full(3, -2.5))
+    assert np.array_equal(oracle.reduce(x[:, :1], [1], "min").reshape(-1), x[:, 0].reshape(-1))
+
+
 # ---------------------------------------------------------------------------
 # fp32 CPU ports (the timed baseline) agree with the float64 oracle
 # ---------------------------------------------------------------------------

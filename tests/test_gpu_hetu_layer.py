@@ -468,3 +468,45 @@ def test_operators_leave_no_memory_behind(ops, cuda):
     s = ops.pool_stats()
     assert s["allocated"] == 0                 # scratch went back to the pool
     assert s["cache_hits"] >= 2                # and was reused by the later iterations
+
+
+def test_two_streams_share_the_pool_without_corruption(ops, cuda):
+    """Operators alternate between two of the layer's streams while their scratch and temporaries come
+    from the same pool: blocks freed on one stream are taken by the other behind an event.  Every result
+    is checked, so a block reused before its previous user finished would show up as a wrong answer."""
+    import torch
+    rows, cols = 2048, 4096
+    xs = [helpers.draw(700 + i, (rows, cols), dtype="bf16") for i in range(2)]
+    dys = [helpers.draw(710 + i, (rows, cols), dtype="bf16") for i in range(2)]
+    gamma = helpers.draw(720, (cols,), "uniform", 0.8, 1.2, "bf16")
+    want = []
+    for x, dy in zip(xs, dys):
+        z, _, mu, rs = oracle.dropout_add_ln_fwd(x, None, gamma, None, 1e-6, True)
+        dx0, dg, _ = oracle.dropout_add_ln_bwd(dy, None, x, mu.astype(np.float32), rs.astype(np.float32), gamma, True)
+        want.append((z, dx0, dg, np.asarray(oracle.reduce(x, [0], "sum"))))
+    tg = helpers.to_torch(gamma, "bf16", cuda)
+    dev = []
+    for x, dy in zip(xs, dys):
+        tx, tdy = helpers.to_torch(x, "bf16", cuda), helpers.to_torch(dy, "bf16", cuda)
+        dev.append(dict(x=tx, dy=tdy, z=torch.empty_like(tx), dx=torch.empty_like(tx), dg=torch.empty_like(tg),
+                        db=torch.empty_like(tg), mu=torch.empty(rows, device=cuda), rs=torch.empty(rows, device=cuda),
+                        colsum=torch.empty(cols, dtype=tx.dtype, device=cuda)))
+    _sync_in()
+    before = ops.pool_stats()
+    for it in range(6):
+        for k, stream in enumerate((1, 2)):
+            d = dev[(k + it) % 2]          # the two data sets swap streams every iteration
+            ops.dropout_add_ln_fwd(d["x"], None, tg, None, d["z"], None, d["mu"], d["rs"], 1e-6, True, stream=stream)
+            ops.dropout_add_ln_bwd(d["dy"], None, d["x"], d["mu"], d["rs"], tg, d["dx"], None, d["dg"], d["db"],
+                                   False, True, stream=stream)
+            ops.reduce(d["x"], d["colsum"], [0], "sum", stream=stream)
+        ops.stream_sync(1)
+        ops.stream_sync(2)
+    for d, (z, dx0, dg, colsum) in zip(dev, want):
+        helpers.assert_close(d["z"], z, "bf16", "z")
+        helpers.assert_close(d["dx"], dx0, "bf16", "dx0")
+        helpers.assert_close(d["dg"], dg, "bf16", "dgamma")
+        helpers.assert_close(d["colsum"], colsum, "bf16", "column sums", scale=float(np.sqrt(rows)))
+    after = ops.pool_stats()
+    assert after["allocated"] == before["allocated"]
+    assert after["segment_allocs"] - before["segment_allocs"] <= 6      # scratch is recycled, not re-allocated

@@ -59,7 +59,7 @@ template <typename T, int NV, bool WAVE_ROW, bool HAS_RES>
 __global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
 void norm_fwd_kernel(NormFwdArgs a) {
   constexpr int VEC = VecIO<T>::N;
-  __shared__ float red[kMaxWaves * 3];
+  __shared__ float red[kMaxWaves * 4];
 
   const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
   const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
@@ -125,37 +125,48 @@ void norm_fwd_kernel(NormFwdArgs a) {
     var = fmaxf(ms - mu * mu, 0.f);
     rs = 1.0f / sqrtf(ms + a.eps);
   } else {
-    // the row sits in registers, so the textbook two-pass variance costs no memory traffic: sum -> mean,
-    // then sum of squared distances to that mean.  Two plain sum reductions (six DPP adds each, one LDS
-    // round when several waves share the row) are far shorter than one reduction of Welford triples, whose
-    // every merge step carries a division on the critical path.
-    SumTuple<1> s;
-    s.v[0] = 0.f;
+    // One reduction in the common case: sums of (x - K) and (x - K)^2 with K = the row's first element, a
+    // sample of the row, so the two terms of var = E[(x-K)^2] - (E[x-K])^2 are both of the size of the
+    // variance and cancel harmlessly.  When K turns out to be far from the mean (more than 4 standard
+    // deviations: an outlier in column 0) the cancellation would cost digits; the row is still in
+    // registers, so that row alone takes the textbook second pass over (x - mean)^2.
+    float K = Cvt<T>::load(xr);
+    if constexpr (HAS_RES) K += Cvt<T>::load(static_cast<const T*>(a.residual) + row * int64_t(a.cols));
+    SumTuple<2> s;
+    s.v[0] = 0.f; s.v[1] = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       if (i * tpr + t < a.nvec) {
         float f[VEC];
         get(i, f);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) s.v[0] += f[j];
+        for (int j = 0; j < VEC; ++j) { const float d = f[j] - K; s.v[0] += d; s.v[1] = fmaf(d, d, s.v[1]); }
       }
     }
     s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red, 0, nwaves);
-    mu = s.v[0] * a.inv_cols;
-    SumTuple<1> q;
-    q.v[0] = 0.f;
+    const float dm = s.v[0] * a.inv_cols;
+    mu = K + dm;
+    var = fmaxf(fmaf(-dm, dm, s.v[1] * a.inv_cols), 0.f);
+    if (dm * dm > 16.f * var) {   // the same value in every thread of the row: a uniform branch
+      // corrected two-pass: distances to the first estimate of the mean; their sum refines the mean
+      // (the large shift cost it digits too) and corrects the sum of squares
+      SumTuple<2> q;
+      q.v[0] = 0.f; q.v[1] = 0.f;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      if (i * tpr + t < a.nvec) {
-        float f[VEC];
-        get(i, f);
+      for (int i = 0; i < NV; ++i) {
+        if (i * tpr + t < a.nvec) {
+          float f[VEC];
+          get(i, f);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) { const float d = f[j] - mu; q.v[0] = fmaf(d, d, q.v[0]); }
+          for (int j = 0; j < VEC; ++j) { const float d = f[j] - mu; q.v[0] += d; q.v[1] = fmaf(d, d, q.v[1]); }
+        }
       }
+      // a second LDS region: waves still reading the first sums must not see them overwritten
+      q = WAVE_ROW ? wave_allreduce_tuple(q) : group_allreduce_tuple(q, red + kMaxWaves * 2, 0, nwaves);
+      const float dc = q.v[0] * a.inv_cols;
+      mu += dc;
+      var = fmaxf(fmaf(-dc, dc, q.v[1] * a.inv_cols), 0.f);
     }
-    // a second LDS region: waves still reading the first sums must not see them overwritten
-    q = WAVE_ROW ? wave_allreduce_tuple(q) : group_allreduce_tuple(q, red + kMaxWaves, 0, nwaves);
-    var = q.v[0] * a.inv_cols;
     rs = 1.0f / sqrtf(var + a.eps);
   }
 
@@ -166,6 +177,8 @@ void norm_fwd_kernel(NormFwdArgs a) {
 
   const float shift = a.is_rms ? 0.f : mu;
   T* yr = static_cast<T*>(a.y) + row * int64_t(a.cols);
+  // gamma / beta are fetched here, after the reduction: holding them in registers across it was measured
+  // slower (fewer resident waves) than these cache hits
   const T* gp = static_cast<const T*>(a.gamma);
   const T* bp = static_cast<const T*>(a.beta);
 #pragma unroll

@@ -246,3 +246,39 @@ def test_full_size_configs(hk, cuda, cfg):
     if not is_rms:
         rowsum = tdx.float().sum(1).abs().max().item()
         assert rowsum <= 1e-2 * cols ** 0.5
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("cols", [256, 4096, 5120])
+def test_layer_norm_statistics_conditioning(hk, cuda, dtype, cols):
+    """Rows whose first element is an outlier, rows riding on a large common offset, and rows that are
+    constant apart from one element: the variance must stay accurate in all of them."""
+    import torch
+    rows = 24
+    eps = 1e-5
+    x = helpers.draw(900 + cols, (rows, cols), dtype="fp32").astype(np.float64)
+    x[0:6, 0] = 3000.0                      # first column far from the row mean
+    x[6:12] += 300.0                        # mean >> standard deviation
+    x[12:16] = 7.0
+    x[12:16, 5] = 7.5                       # almost constant
+    x[16:18] = -2.0                         # constant: variance exactly 0
+    x[18, 0] = -1e4
+    x = oracle.round_to(x.astype(np.float32), dtype)
+    gamma = helpers.draw(1, (cols,), "uniform", 0.5, 1.5, dtype)
+    beta = helpers.draw(2, (cols,), "normal", 0.0, 0.1, dtype)
+    ey, emean, evar, erstd = oracle.layernorm_fwd(x, gamma, beta, eps)
+    tx, tg, tb = (helpers.to_torch(v, dtype, cuda) for v in (x, gamma, beta))
+    ty = torch.empty_like(tx)
+    tmean = torch.empty(rows, dtype=torch.float32, device=cuda)
+    trstd = torch.empty(rows, dtype=torch.float32, device=cuda)
+    hk.layer_norm_fwd(tx, tg, tb, ty, tmean, trstd, eps, stat_kind=1)
+    torch.cuda.synchronize()
+    got_rstd = helpers.to_numpy(trstd).astype(np.float64)
+    got_mean = helpers.to_numpy(tmean).astype(np.float64)
+    # statistics are fp32 whatever the data type: judge them at fp32 accuracy, row by row
+    assert np.all(np.abs(got_rstd - erstd) <= 2e-5 * np.abs(erstd)), np.max(np.abs(got_rstd - erstd) / np.abs(erstd))
+    assert np.all(np.abs(got_mean - emean) <= 2e-6 * (np.abs(emean) + np.sqrt(evar) + 1e-3))
+    assert np.all(got_rstd[16:18] == np.float32(1.0 / np.sqrt(np.float32(eps))))
+    # a mean near 300 is only known to half an fp32 ulp (1.5e-5) in fp32 arithmetic, and x - mean inherits
+    # that: the fp32 bound for y is loosened accordingly in this stress case
+    helpers.assert_close(ty, ey, dtype, "y", rtol=1e-4 if dtype == "fp32" else None)

@@ -298,6 +298,73 @@ def cpu_baseline(rows=32768, cols=4096, budget_s=12.0):
                       "formula" % (rows, reps, reps * dt)}
 
 
+def cpu_kernels(budget_s=1.5):
+    """fp32 CPU ports of the reference's CPU kernels (oracle's refcpu_*: the pass structure of
+    LayerNormCpu, the softmax / cross-entropy loops, the reductions), timed on all host threads and,
+    for the serial loops of the reference, on one; bytes counted in the ports' own fp32 storage."""
+    import ctypes
+    import numpy as np
+    import oracle
+    lib = oracle.lib()
+    cores = min(int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1), 64)
+    g = np.random.default_rng(7)
+    fp = ctypes.POINTER(ctypes.c_float)
+    P = lambda a: a.ctypes.data_as(fp)
+    I = ctypes.c_int64
+
+    def block(rows, cols):
+        b = g.standard_normal((min(rows, 512), cols), dtype=np.float32)
+        return np.tile(b, ((rows + b.shape[0] - 1) // b.shape[0], 1))[:rows].copy()
+
+    def timed(fn, nbytes, threads):
+        lib.refcpu_set_num_threads(ctypes.c_int(threads))
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while reps < 2 or time.perf_counter() - t0 < budget_s:
+            fn()
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        return round(dt * 1e6, 1), round(nbytes / dt / 1e9, 2), reps
+
+    out = []
+
+    def add(name, fn, nbytes, sample, serial_too=False):
+        us, gbs, reps = timed(fn, nbytes, cores)
+        rec = {"case": name, "us": us, "GBps": gbs, "cores": cores, "sample": sample, "reps": reps}
+        if serial_too:
+            us1, gbs1, _ = timed(fn, nbytes, 1)
+            rec["us_1_thread"], rec["GBps_1_thread"] = us1, gbs1
+        out.append(rec)
+
+    rows, cols = 8192, 4096
+    x = block(rows, cols); y = np.empty_like(x)
+    gm = np.ones(cols, np.float32); bt = np.zeros(cols, np.float32)
+    mean = np.empty(rows, np.float32); var = np.empty(rows, np.float32)
+    add("C1 layernorm fwd fp32 [8192x4096] (LayerNormCpu pass structure)",
+        lambda: lib.refcpu_layernorm_fwd_f32(P(x), P(gm), P(bt), I(rows), I(cols), ctypes.c_float(1e-5), P(y), P(mean), P(var)),
+        2 * rows * cols * 4, "full size", serial_too=True)
+    rows, cols = 16384, 2048
+    x = block(rows, cols); y = np.empty_like(x); dx = np.empty_like(x)
+    add("C2 softmax fwd fp32 [16384 of 262144 rows x 2048]",
+        lambda: lib.refcpu_softmax_fwd_f32(P(x), I(rows), I(cols), P(y)), 2 * rows * cols * 4, "1/16 of the rows")
+    add("C2 softmax bwd fp32 [16384 of 262144 rows x 2048]",
+        lambda: lib.refcpu_softmax_bwd_f32(P(y), P(x), I(rows), I(cols), P(dx)), 3 * rows * cols * 4, "1/16 of the rows")
+    rows, cols = 8192, 4096
+    x = block(rows, cols); o0 = np.empty(cols, np.float32); o1 = np.empty(rows, np.float32)
+    add("C3 reduce sum axis1 fp32 [8192 of 32768 rows x 4096]",
+        lambda: lib.refcpu_reduce_sum_axis1_f32(P(x), I(rows), I(cols), P(o1)), rows * cols * 4, "1/4 of the rows")
+    add("C3 reduce sum axis0 fp32 [8192 of 32768 rows x 4096] (serial loop)",
+        lambda: lib.refcpu_reduce_sum_axis0_f32(P(x), I(rows), I(cols), P(o0)), rows * cols * 4, "1/4 of the rows")
+    rows, cols = 1024, 32000
+    x = block(rows, cols); loss = np.empty(rows, np.float32)
+    lab = (np.arange(rows, dtype=np.int64) * 31) % cols
+    add("C5 sce fwd fp32 [1024 of 16384 rows x 32000]",
+        lambda: lib.refcpu_sce_sparse_fwd_f32(P(x), lab.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)), I(rows), I(cols),
+                                              I(-100), P(loss)), rows * cols * 4, "1/16 of the rows")
+    lib.refcpu_set_num_threads(ctypes.c_int(cores))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -363,6 +430,11 @@ def main():
         out["cpu_baseline"] = cpu_baseline()
     if kernels:
         out["kernels"] = kernels
+        if not args.no_cpu:
+            out["cpu_kernels"] = cpu_kernels()
+            for rec in out["cpu_kernels"]:
+                print("cpu  %-66s %10.1f us %8.2f GB/s (%d threads)" % (rec["case"], rec["us"], rec["GBps"], rec["cores"]),
+                      file=sys.stderr, flush=True)
     print(json.dumps(out), flush=True)
 
 

@@ -287,10 +287,19 @@ __device__ __forceinline__ P wave_allreduce_tuple(P a) {
   return P::merge(P::merge(r[0], r[1]), P::merge(r[2], r[3]));
 }
 
+// the cross-wave half of group_allreduce_tuple: `a` is already the same in every lane of a wave
+template <typename P>
+__device__ __forceinline__ P group_combine_tuple(P a, float* scratch, int first_wave, int nwaves);
+
 template <typename P>
 __device__ __forceinline__ P group_allreduce_tuple(P a, float* scratch, int first_wave,
                                                     int nwaves) {
   a = wave_allreduce_tuple<P>(a);
+  return group_combine_tuple<P>(a, scratch, first_wave, nwaves);
+}
+
+template <typename P>
+__device__ __forceinline__ P group_combine_tuple(P a, float* scratch, int first_wave, int nwaves) {
   if (nwaves == 1) return a;
   const int w = threadIdx.x >> 6;
   if ((threadIdx.x & 63) == 0) {
@@ -346,6 +355,21 @@ struct MomentTuple {
     r.v[0] = n;
     r.v[1] = a.v[1] + delta * wb;
     r.v[2] = a.v[2] + b.v[2] + delta * delta * a.v[0] * wb;
+    return r;
+  }
+};
+
+// The same update when both sides are known to hold the SAME number of elements (every step of a
+// butterfly over lanes that started with equal counts): the weights are 1/2, no reciprocal is needed.
+struct EqualMomentTuple {
+  static constexpr int K = 3;
+  float v[3];
+  static __device__ __forceinline__ EqualMomentTuple merge(const EqualMomentTuple& a, const EqualMomentTuple& b) {
+    EqualMomentTuple r;
+    const float delta = b.v[1] - a.v[1];
+    r.v[0] = a.v[0] + a.v[0];
+    r.v[1] = fmaf(delta, 0.5f, a.v[1]);
+    r.v[2] = fmaf(delta * delta, 0.5f * a.v[0], a.v[2] + b.v[2]);
     return r;
   }
 };

@@ -1,8 +1,9 @@
 // LayerNorm / RMSNorm forward and backward for gfx950.
 //
 // Forward: a row lives in registers as packed 128-bit vectors (one HBM read),
-// statistics are Welford moments merged with Chan's update across lanes (DPP)
-// and waves (LDS), output is written with 128-bit stores.  One wavefront per
+// statistics are Welford moments merged with Chan's update across lanes (DPP,
+// equal-count form when the row fills every lane) and waves (LDS), output is
+// written with 128-bit stores.  One wavefront per
 // row for short rows, one workgroup per row for long rows.
 //
 // Backward: a persistent grid walks the rows; every thread owns a fixed set of
@@ -59,7 +60,7 @@ template <typename T, int NV, bool WAVE_ROW, bool HAS_RES>
 __global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
 void norm_fwd_kernel(NormFwdArgs a) {
   constexpr int VEC = VecIO<T>::N;
-  __shared__ float red[kMaxWaves * 4];
+  __shared__ float red[kMaxWaves * 3];
 
   const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
   const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
@@ -125,48 +126,48 @@ void norm_fwd_kernel(NormFwdArgs a) {
     var = fmaxf(ms - mu * mu, 0.f);
     rs = 1.0f / sqrtf(ms + a.eps);
   } else {
-    // One reduction in the common case: sums of (x - K) and (x - K)^2 with K = the row's first element, a
-    // sample of the row, so the two terms of var = E[(x-K)^2] - (E[x-K])^2 are both of the size of the
-    // variance and cancel harmlessly.  When K turns out to be far from the mean (more than 4 standard
-    // deviations: an outlier in column 0) the cancellation would cost digits; the row is still in
-    // registers, so that row alone takes the textbook second pass over (x - mean)^2.
-    float K = Cvt<T>::load(xr);
-    if constexpr (HAS_RES) K += Cvt<T>::load(static_cast<const T*>(a.residual) + row * int64_t(a.cols));
-    SumTuple<2> s;
-    s.v[0] = 0.f; s.v[1] = 0.f;
+    // Welford statistics, merged with Chan's parallel update: each thread forms (count, mean, M2) of the
+    // elements it holds in registers, lanes merge through a DPP butterfly, waves through LDS.  When every
+    // thread holds the same count (the row fills all vector slots: a uniform test) each butterfly step
+    // merges equal-sized halves and needs no reciprocal; a ragged row takes the general update.
+    float s = 0.f;
+    int cnt = 0;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       if (i * tpr + t < a.nvec) {
         float f[VEC];
         get(i, f);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) { const float d = f[j] - K; s.v[0] += d; s.v[1] = fmaf(d, d, s.v[1]); }
+        for (int j = 0; j < VEC; ++j) s += f[j];
+        cnt += VEC;
       }
     }
-    s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red, 0, nwaves);
-    const float dm = s.v[0] * a.inv_cols;
-    mu = K + dm;
-    var = fmaxf(fmaf(-dm, dm, s.v[1] * a.inv_cols), 0.f);
-    if (dm * dm > 16.f * var) {   // the same value in every thread of the row: a uniform branch
-      // corrected two-pass: distances to the first estimate of the mean; their sum refines the mean
-      // (the large shift cost it digits too) and corrects the sum of squares
-      SumTuple<2> q;
-      q.v[0] = 0.f; q.v[1] = 0.f;
+    const bool even = a.nvec == NV * tpr;                    // uniform
+    const float mean_t = even ? s * (1.0f / float(NV * VEC)) : (cnt > 0 ? s / float(cnt) : 0.f);
+    float m2 = 0.f;
 #pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        if (i * tpr + t < a.nvec) {
-          float f[VEC];
-          get(i, f);
+    for (int i = 0; i < NV; ++i) {
+      if (i * tpr + t < a.nvec) {
+        float f[VEC];
+        get(i, f);
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) { const float d = f[j] - mu; q.v[0] += d; q.v[1] = fmaf(d, d, q.v[1]); }
-        }
+        for (int j = 0; j < VEC; ++j) { const float d = f[j] - mean_t; m2 = fmaf(d, d, m2); }
       }
-      // a second LDS region: waves still reading the first sums must not see them overwritten
-      q = WAVE_ROW ? wave_allreduce_tuple(q) : group_allreduce_tuple(q, red + kMaxWaves * 2, 0, nwaves);
-      const float dc = q.v[0] * a.inv_cols;
-      mu += dc;
-      var = fmaxf(fmaf(-dc, dc, q.v[1] * a.inv_cols), 0.f);
     }
+    MomentTuple m;
+    m.v[0] = float(cnt); m.v[1] = mean_t; m.v[2] = m2;
+    if (even) {
+      EqualMomentTuple e;
+      e.v[0] = m.v[0]; e.v[1] = m.v[1]; e.v[2] = m.v[2];
+      e = wave_allreduce_tuple(e);
+      m.v[0] = e.v[0]; m.v[1] = e.v[1]; m.v[2] = e.v[2];
+    } else {
+      m = wave_allreduce_tuple(m);
+    }
+    // waves are merged one after the other (growing count on one side): the general update
+    if (!WAVE_ROW) m = group_combine_tuple(m, red, 0, nwaves);
+    mu = m.v[1];
+    var = m.v[2] * a.inv_cols;
     rs = 1.0f / sqrtf(var + a.eps);
   }
 
@@ -303,7 +304,10 @@ static int launch_norm_fwd_nv(const NormFwdArgs& a, int nv, dim3 grid, dim3 bloc
   switch (nv) {
     case 1: hipLaunchKernelGGL((norm_fwd_kernel<T, 1, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
     case 2: hipLaunchKernelGGL((norm_fwd_kernel<T, 2, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 3: hipLaunchKernelGGL((norm_fwd_kernel<T, 3, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
     case 4: hipLaunchKernelGGL((norm_fwd_kernel<T, 4, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 5: hipLaunchKernelGGL((norm_fwd_kernel<T, 5, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 6: hipLaunchKernelGGL((norm_fwd_kernel<T, 6, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
     case 8: hipLaunchKernelGGL((norm_fwd_kernel<T, 8, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
     case 16: hipLaunchKernelGGL((norm_fwd_kernel<T, 16, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
     default:
@@ -333,7 +337,20 @@ static bool pick_row_shape(int nvec, int forced_threads, int max_nv, int wave_ro
     return true;
   }
   // medium rows (measured on MI355X: 4096 / 5120 bf16 columns, 4096 fp32
-  // columns): small workgroups of 128..256 threads per row stream fastest
+  // columns): small workgroups of 128..256 threads per row stream fastest.
+  // First choice: the fewest vectors per thread that fill every lane exactly
+  // (5120 bf16 columns = 640 vectors = 128 threads x 5): no idle lanes, and the
+  // statistics merge takes its equal-count form.
+  static const int kCounts[] = {2, 3, 4, 5, 6, 8};
+  for (int n : kCounts) {
+    if (n > max_nv) break;
+    int t = ((nvec + n - 1) / n + 63) / 64 * 64;
+    if (t <= 256 && n * t == nvec) {
+      *threads = t;
+      *nv = n;
+      return true;
+    }
+  }
   for (int n = 2; n <= max_nv; n <<= 1) {
     int t = ((nvec + n - 1) / n + 63) / 64 * 64;
     if (t <= 256) {

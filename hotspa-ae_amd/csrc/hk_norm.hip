@@ -889,7 +889,12 @@ static BwdPlan plan_norm_bwd(int64_t rows, int cols, bool aligned) {
   const int max_block = nv == 1 ? 1024 : 512;
   if (tpr > max_block) return p;
   int rpb = tune_get(TUNE_NORM_BWD_ROWS_PER_BLOCK);
-  if (rpb <= 0) rpb = std::max(1, max_block / tpr);
+  if (rpb <= 0) {
+    rpb = std::max(1, max_block / tpr);
+    // 512 threads already stream a whole 4096-column row per step; pairing two such groups in one
+    // workgroup only adds waves to every barrier (measured 2-3 % slower than one group per workgroup)
+    if (tpr >= 512) rpb = 1;
+  }
   rpb = std::max(1, std::min(rpb, max_block / tpr));
   // staging buffer of the final fold must fit 64 KiB of LDS
   while (rpb > 1 && size_t(rpb) * cols * sizeof(float) > 65536) --rpb;

@@ -84,7 +84,7 @@ def build_device(verbose=True, incremental=False):
 
 def build_host(verbose=True):
     """g++: every .cc under hetu/ -> lib/libhetu_rowwise.so, then the host
-    self-test tests/cpp/host_selftest.cc -> lib/hetu_host_selftest."""
+    self-tests tests/cpp/{host,gpu}_selftest.cc -> lib/hetu_{host,gpu}_selftest."""
     srcs = []
     for dirpath, _, files in os.walk(HOST):
         srcs += [os.path.join(dirpath, f) for f in files if f.endswith(".cc")]
@@ -111,13 +111,14 @@ def build_host(verbose=True):
          ["-L" + LIB, "-lhk_rowwise", "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("[build] linked", out, flush=True)
-    selftest = os.path.join(ROOT, "tests", "cpp", "host_selftest.cc")
-    if os.path.exists(selftest):
-        exe = os.path.join(LIB, "hetu_host_selftest")
-        _run(cxx + [selftest, "-o", exe, "-L" + LIB, "-lhetu_rowwise", "-lhk_rowwise",
-                    "-Wl,-rpath,$ORIGIN"])
-        if verbose:
-            print("[build] linked", exe, flush=True)
+    for name in ("host_selftest", "gpu_selftest"):
+        selftest = os.path.join(ROOT, "tests", "cpp", name + ".cc")
+        if os.path.exists(selftest):
+            exe = os.path.join(LIB, "hetu_" + name)
+            _run(cxx + [selftest, "-o", exe, "-L" + LIB, "-lhetu_rowwise", "-lhk_rowwise",
+                        "-Wl,-rpath,$ORIGIN"])
+            if verbose:
+                print("[build] linked", exe, flush=True)
     return out
 
 

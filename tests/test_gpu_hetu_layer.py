@@ -510,3 +510,16 @@ def test_two_streams_share_the_pool_without_corruption(ops, cuda):
     after = ops.pool_stats()
     assert after["allocated"] == before["allocated"]
     assert after["segment_allocs"] - before["segment_allocs"] <= 6      # scratch is recycled, not re-allocated
+
+
+def test_native_cpp_gpu_selftest(cuda):
+    """tests/cpp/gpu_selftest.cc: the layer driven from C++ (NDArray::cuda / cpu / zeros, the operator
+    statics, events, the pool) and checked against double-precision loops inside the binary."""
+    import os
+    import subprocess
+    exe = os.path.join(helpers.ROOT, "hotspa-ae_amd", "lib", "hetu_gpu_selftest")
+    assert os.path.exists(exe), "run __graft_entry__.build() first"
+    proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    failed = [l for l in proc.stdout.splitlines() if l.startswith("[FAIL]")]
+    assert proc.returncode == 0 and not failed, proc.stdout[-4000:]
+    assert sum(l.startswith("[ OK ]") for l in proc.stdout.splitlines()) >= 8

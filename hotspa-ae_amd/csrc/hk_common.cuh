@@ -38,16 +38,6 @@ __device__ __forceinline__ int wave_index() {
   return __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6));
 }
 
-// Makes the compiler forget what it knows about a packed vector without
-// emitting an instruction.  Used between two passes over the same registers so
-// that the second pass re-derives its fp32 values from the packed data instead
-// of keeping every unpacked intermediate of the first pass alive.
-__device__ __forceinline__ void launder(uint32_t __attribute__((ext_vector_type(4))) & v) {
-  uint32_t a = v.x, b = v.y, c = v.z, d = v.w;
-  asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-  v.x = a; v.y = b; v.z = c; v.w = d;
-}
-
 __device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
 
@@ -207,15 +197,7 @@ __device__ __forceinline__ float readlane_f(float v, int lane) {
   return u2f(uint32_t(__builtin_amdgcn_readlane(int(f2u(v)), lane)));
 }
 
-struct OpSum {
-  static __device__ __forceinline__ float identity() { return 0.f; }
-  static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
-};
-struct OpMax {
-  static __device__ __forceinline__ float identity() { return -__builtin_huge_valf(); }
-  static __device__ __forceinline__ float apply(float a, float b) { return fmaxf(a, b); }
-};
-
+// Op: a struct with `static float identity()` and `static float apply(float, float)`.
 template <typename Op>
 __device__ __forceinline__ float wave_allreduce(float v) {
   v = Op::apply(v, dpp_f<kDppXor1>(v, v));
@@ -228,8 +210,6 @@ __device__ __forceinline__ float wave_allreduce(float v) {
   return Op::apply(Op::apply(r0, r1), Op::apply(r2, r3));
 }
 
-__device__ __forceinline__ float wave_sum(float v) { return wave_allreduce<OpSum>(v); }
-__device__ __forceinline__ float wave_max(float v) { return wave_allreduce<OpMax>(v); }
 
 // Shuffle through DPP for the 16-lane-local steps of a butterfly, and through
 // the cross-lane network only for the 16 / 32 strides.  Used by reductions on

@@ -160,6 +160,28 @@ def case_sce(hk, torch, nsets, which):
         2 * n + rows * 8 + rows * 2, rows
 
 
+def case_nll_bwd(hk, torch, nsets):
+    rows, cols = 16384, 32000
+    bf = torch.bfloat16
+    g = torch.Generator(device="cuda").manual_seed(602)
+    labels = torch.randint(0, cols, (rows,), generator=g, device="cuda", dtype=torch.int64)
+    gl = torch.full((rows,), 1.0 / rows, dtype=bf, device="cuda")
+    outs = [torch.empty((rows, cols), dtype=bf, device="cuda") for _ in range(2)]
+    return (lambda i: hk.nll_loss_bwd(labels, gl, outs[i % 2])), rows * cols * 2 + rows * 10, rows
+
+
+def case_instance_norm(hk, torch, nsets):
+    # [N=256, C=256, H=32, W=32] bf16: 65536 planes of 1024 elements, no scale / bias
+    rows, cols = 256 * 256, 32 * 32
+    bf = torch.bfloat16
+    xs = [_randn(torch, (rows, cols), bf, 1.0, 611 + i) for i in range(nsets)]
+    ys = [torch.empty((rows, cols), dtype=bf, device="cuda") for _ in range(nsets)]
+    mean = torch.empty(rows, dtype=bf, device="cuda")
+    var = torch.empty(rows, dtype=bf, device="cuda")
+    return (lambda i: hk.layer_norm_fwd(xs[i % nsets], None, None, ys[i % nsets], mean, var, 1e-5, stat_kind=0)), \
+        2 * rows * cols * 2 + 2 * rows * 2, rows
+
+
 def case_reduce(hk, torch, nsets, axes, op, three_d=False):
     rows, cols = 32768, 4096
     bf = torch.bfloat16
@@ -220,6 +242,8 @@ CASES = [
     ("next: reduce max axis0 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (0,), "max")),
     ("next: reduce max axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "max")),
     ("next: reduce prod axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "prod")),
+    ("next: nll loss bwd bf16 [16384x32000] (write only)", lambda hk, t, n: case_nll_bwd(hk, t, n)),
+    ("next: instance norm fwd bf16 [256,256,32,32]", lambda hk, t, n: case_instance_norm(hk, t, n)),
     ("C4 rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "fwd")),
     ("C4 rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "bwd")),
     ("C5 sce fwd bf16 [16384x32000]", lambda hk, t, n: case_sce(hk, t, 2, "fwd")),

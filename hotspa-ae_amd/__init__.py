@@ -19,7 +19,7 @@ from .capi import (  # noqa: F401
     layer_norm_fwd, layer_norm_bwd, norm_bwd_workspace_bytes,
     dropout_add_ln_fwd, dropout_add_ln_bwd,
     softmax_fwd, softmax_bwd,
-    sce_sparse_fwd, sce_sparse_bwd, sce_dense_fwd, sce_dense_bwd,
+    sce_sparse_fwd, sce_sparse_bwd, sce_dense_fwd, sce_dense_bwd, nll_loss_fwd, nll_loss_bwd,
     reduce, reduce_workspace_bytes, tune_set, copy_kernel, strided_copy,
     Event, current_stream,
 )

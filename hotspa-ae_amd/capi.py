@@ -225,6 +225,20 @@ def sce_dense_bwd(logits, labels, grad_loss, dlogits, stream=None):
                                  _i64(rows), _i64(cols), stream if stream is not None else current_stream()))
 
 
+def nll_loss_fwd(pred, labels, loss, stream=None):
+    cols = pred.shape[-1]
+    rows = pred.numel() // cols if pred.numel() else 0
+    check(lib().hk_nll_loss_fwd(dtype_code(pred), _ptr(pred), _ptr(labels), _ptr(loss), _i64(rows), _i64(cols),
+                                stream if stream is not None else current_stream()))
+
+
+def nll_loss_bwd(labels, grad_loss, out, stream=None):
+    cols = out.shape[-1]
+    rows = out.numel() // cols if out.numel() else 0
+    check(lib().hk_nll_loss_bwd(dtype_code(out), _ptr(labels), _ptr(grad_loss), _ptr(out), _i64(rows), _i64(cols),
+                                stream if stream is not None else current_stream()))
+
+
 def reduce_workspace_bytes(dtype, shape, strides, axes):
     n = ctypes.c_size_t()
     check(lib().hk_reduce_workspace_bytes(ctypes.c_int(dtype), ctypes.c_int(len(shape)), _arr(shape), _arr(strides),

@@ -149,6 +149,22 @@ int ht_dropout_add_ln_bwd(const HtArray* dz, const HtArray* dx, const HtArray* x
   });
 }
 
+int ht_instance_norm(const HtArray* in, HtArray* mean, HtArray* var, HtArray* out, float eps, int stream_index) {
+  return guarded([&] {
+    NDArray m = wrap(mean), v = wrap(var), o = wrap(out);
+    hetu::impl::InstanceNormCuda(wrap(in), m, v, o, eps, stream_of(in, stream_index));
+  });
+}
+
+int ht_instance_norm_gradient(const HtArray* out_grads, const HtArray* in, HtArray* grad_in, const HtArray* mean,
+                              const HtArray* var, float eps, int stream_index) {
+  return guarded([&] {
+    NDArray g = wrap(grad_in);
+    hetu::impl::InstanceNormGradientCuda(wrap(out_grads), wrap(in), g, wrap(mean), wrap(var), eps,
+                                         stream_of(in, stream_index));
+  });
+}
+
 int ht_softmax(const HtArray* in, HtArray* out, int64_t dim, int stream_index) {
   return guarded([&] {
     NDArray o = wrap(out);
@@ -194,6 +210,21 @@ int ht_softmax_cross_entropy_sparse_gradient(const HtArray* pred, const HtArray*
     NDArray o = wrap(out);
     hetu::impl::SoftmaxCrossEntropySparseGradientCuda(wrap(pred), wrap(label), wrap(grad_loss), o, ignored_index,
                                                       stream_of(pred, stream_index));
+  });
+}
+
+int ht_nll_loss(const HtArray* pred, const HtArray* label, HtArray* loss, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(loss);
+    hetu::impl::NLLLossCuda(wrap(pred), wrap(label), o, stream_of(pred, stream_index));
+  });
+}
+
+int ht_nll_loss_gradient(const HtArray* pred, const HtArray* label, const HtArray* grad_loss, HtArray* out,
+                         int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(out);
+    hetu::impl::NLLLossGradientCuda(wrap(pred), wrap(label), wrap(grad_loss), o, stream_of(pred, stream_index));
   });
 }
 

@@ -1,6 +1,6 @@
 // Declarations of the kernel entry points of the row-wise operator path and the
 // device switch that picks them (hetu/graph/ops/kernel_links.h:12-21, 125-135,
-// 168-175, 199-206, 260-269, 296-308, 362-397 of the reference).  The names
+// 168-175, 185-189, 199-206, 239-243, 260-269, 296-308, 362-397 of the reference).  The names
 // `KERNEL##Cuda` / `KERNEL##Cpu` are produced by token pasting in the dispatch
 // macros, so they are the link contract; the `Cuda` entries here are the
 // gfx950 implementations.
@@ -39,12 +39,20 @@ DECLARE_KERNEL_CUDA(FusedLayerNorm, const NDArray&, const NDArray&, const NDArra
 DECLARE_KERNEL_CUDA(FusedLayerNormGradient, const NDArray&, const NDArray&, const NDArray&, const NDArray&,
                     NDArray&, NDArray&, NDArray&, const NDArray&, const NDArray&, int64_t, float, bool,
                     const Stream&);
+// in, mean, var, out, eps   /   out_grads, in, grad_in, mean, var, eps
+DECLARE_KERNEL_CPU_AND_CUDA(InstanceNorm, const NDArray&, NDArray&, NDArray&, NDArray&, float, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(InstanceNormGradient, const NDArray&, const NDArray&, NDArray&, const NDArray&,
+                            const NDArray&, float, const Stream&);
 // in, scale, bias, mean, var, out, reduce_dims, eps
 DECLARE_KERNEL_CPU_AND_CUDA(LayerNorm, const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&,
                             NDArray&, int64_t, float, const Stream&);
 // dy, x, scale, dx, dscale, dbias, mean, var, reduce_dims, eps
 DECLARE_KERNEL_CPU_AND_CUDA(LayerNormGradient, const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&,
                             NDArray&, const NDArray&, const NDArray&, int64_t, float, const Stream&);
+// pred, label, loss   /   pred, label, grad_loss, output
+DECLARE_KERNEL_CPU_AND_CUDA(NLLLoss, const NDArray&, const NDArray&, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(NLLLossGradient, const NDArray&, const NDArray&, const NDArray&, NDArray&,
+                            const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(Reduce, const NDArray&, NDArray&, const HTAxes&, ReductionType, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(ReduceMean, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(ReduceSum, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);

@@ -162,6 +162,15 @@ def dropout_add_ln_bwd(dz, dx, x, mu, rsigma, gamma, dx0, dresidual, dgamma, dbe
           ctypes.c_int(int(has_residual)), ctypes.c_int(int(is_rms_norm)), ctypes.c_int(stream))
 
 
+def instance_norm(x, mean, var, out, eps, stream=DEFAULT_STREAM):
+    _call("ht_instance_norm", desc(x), desc(mean), desc(var), desc(out), _f(eps), ctypes.c_int(stream))
+
+
+def instance_norm_gradient(dy, x, dx, mean, var, eps, stream=DEFAULT_STREAM):
+    _call("ht_instance_norm_gradient", desc(dy), desc(x), desc(dx), desc(mean), desc(var), _f(eps),
+          ctypes.c_int(stream))
+
+
 def softmax(x, out, dim, stream=DEFAULT_STREAM):
     _call("ht_softmax", desc(x), desc(out), _i64(dim), ctypes.c_int(stream))
 
@@ -187,6 +196,14 @@ def softmax_cross_entropy_sparse(pred, label, loss, ignored_index, stream=DEFAUL
 def softmax_cross_entropy_sparse_gradient(pred, label, grad_loss, out, ignored_index, stream=DEFAULT_STREAM):
     _call("ht_softmax_cross_entropy_sparse_gradient", desc(pred), desc(label), desc(grad_loss), desc(out),
           _i64(ignored_index), ctypes.c_int(stream))
+
+
+def nll_loss(pred, label, loss, stream=DEFAULT_STREAM):
+    _call("ht_nll_loss", desc(pred), desc(label), desc(loss), ctypes.c_int(stream))
+
+
+def nll_loss_gradient(pred, label, grad_loss, out, stream=DEFAULT_STREAM):
+    _call("ht_nll_loss_gradient", desc(pred), desc(label), desc(grad_loss), desc(out), ctypes.c_int(stream))
 
 
 def reduce(x, out, axes, red_type, stream=DEFAULT_STREAM):

@@ -70,6 +70,10 @@ HT_API int ht_dropout_add_ln_bwd(const HtArray* dz, const HtArray* dx, const HtA
                                  const HtArray* colscale, HtArray* dx0, HtArray* dresidual, HtArray* dgamma,
                                  HtArray* dbeta, float dropout_p, int has_residual, int is_rms_norm,
                                  int stream_index);
+HT_API int ht_instance_norm(const HtArray* in, HtArray* mean, HtArray* var, HtArray* out, float eps,
+                            int stream_index);
+HT_API int ht_instance_norm_gradient(const HtArray* out_grads, const HtArray* in, HtArray* grad_in,
+                                     const HtArray* mean, const HtArray* var, float eps, int stream_index);
 HT_API int ht_softmax(const HtArray* in, HtArray* out, int64_t dim, int stream_index);
 HT_API int ht_softmax_gradient(const HtArray* y, const HtArray* dy, HtArray* dx, int64_t dim, int stream_index);
 HT_API int ht_softmax_cross_entropy(const HtArray* pred, const HtArray* label, HtArray* loss, int stream_index);
@@ -80,6 +84,9 @@ HT_API int ht_softmax_cross_entropy_sparse(const HtArray* pred, const HtArray* l
 HT_API int ht_softmax_cross_entropy_sparse_gradient(const HtArray* pred, const HtArray* label,
                                                     const HtArray* grad_loss, HtArray* out,
                                                     int64_t ignored_index, int stream_index);
+HT_API int ht_nll_loss(const HtArray* pred, const HtArray* label, HtArray* loss, int stream_index);
+HT_API int ht_nll_loss_gradient(const HtArray* pred, const HtArray* label, const HtArray* grad_loss,
+                                HtArray* out, int stream_index);
 HT_API int ht_reduce(const HtArray* in, HtArray* out, const int64_t* axes, int naxes, int red_type,
                      int stream_index);
 

@@ -228,6 +228,18 @@ HK_API int hk_sce_dense_bwd(int dtype, const void* logits, const void* labels,
                             hkStream_t stream);
 
 /* ======================================================================== *
+ * Negative log-likelihood loss on log-probabilities, int64 class labels.
+ *   loss[r] = -pred[r, labels[r]]                    (0 for a label outside [0, cols))
+ *   out[r, c] = (c == labels[r]) ? -grad_loss[r] * cols : 0     (every element written once)
+ * Replaces NLLLossCuda / NLLLossGradientCuda (hetu/impl/kernel/NLLLoss.cu:43-86,
+ * :88-128; the "* cols" factor is the reference's, :39).
+ * ======================================================================== */
+HK_API int hk_nll_loss_fwd(int dtype, const void* pred, const int64_t* labels, void* loss,
+                           int64_t rows, int64_t cols, hkStream_t stream);
+HK_API int hk_nll_loss_bwd(int dtype, const int64_t* labels, const void* grad_loss, void* out,
+                           int64_t rows, int64_t cols, hkStream_t stream);
+
+/* ======================================================================== *
  * Reduce sum / mean / max / min / product over a set of axes of a (possibly
  * strided) array.
  * shape / strides (in elements) describe the input; axes must already be

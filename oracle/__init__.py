@@ -225,3 +225,27 @@ def strided_reduce(buf, shape, strides, axes, op="sum", mean_mode=0):
     if rc != 0:
         raise ValueError("oracle_reduce: bad arguments")
     return out.reshape(out_shape if out_shape else [1])
+
+
+def nll_loss_fwd(pred, labels):
+    """loss[r] = -pred[r, label[r]], 0 for a label outside [0, cols)
+    (hetu/impl/kernel/NLLLoss.cu:8-22).  Plain numpy: a gather has no arithmetic to restate in C."""
+    pred = np.asarray(pred, dtype=np.float64)
+    rows, cols = pred.shape
+    lab = np.asarray(labels, dtype=np.int64)
+    ok = (lab >= 0) & (lab < cols)
+    out = np.zeros(rows)
+    out[ok] = -pred[np.arange(rows)[ok], lab[ok]]
+    return out
+
+
+def nll_loss_bwd(labels, grad_loss, cols):
+    """out[r, c] = -grad_loss[r] * cols at c = label[r] (if inside [0, cols)), 0 elsewhere
+    (hetu/impl/kernel/NLLLoss.cu:24-41: the array is cleared first, :116, and the factor cols is the reference's)."""
+    lab = np.asarray(labels, dtype=np.int64)
+    g = np.asarray(grad_loss, dtype=np.float64)
+    rows = lab.shape[0]
+    out = np.zeros((rows, cols))
+    ok = (lab >= 0) & (lab < cols)
+    out[np.arange(rows)[ok], lab[ok]] = -g[ok] * cols
+    return out

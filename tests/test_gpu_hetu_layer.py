@@ -523,3 +523,38 @@ def test_native_cpp_gpu_selftest(cuda):
     failed = [l for l in proc.stdout.splitlines() if l.startswith("[FAIL]")]
     assert proc.returncode == 0 and not failed, proc.stdout[-4000:]
     assert sum(l.startswith("[ OK ]") for l in proc.stdout.splitlines()) >= 8
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("shape", [(3, 5, 16, 16), (2, 4, 28, 36), (1, 2, 7, 9)])
+def test_instance_norm_and_gradient(ops, cuda, dtype, shape):
+    """An instance norm is a layer norm without scale and bias over each [H, W] plane."""
+    import torch
+    n, c, h, w = shape
+    rows, cols, eps = n * c, h * w, 1e-5
+    x = helpers.draw(800 + cols, shape, "normal", 0.5, 2.0, dtype)
+    dy = helpers.draw(801 + cols, shape, dtype=dtype)
+    ones, zeros = np.ones(cols, np.float32), np.zeros(cols, np.float32)
+    ey, emean, evar, erstd = oracle.layernorm_fwd(x.reshape(rows, cols), ones, zeros, eps)
+    tx, tdy = _dev((x, dy), dtype, cuda)
+    ty = torch.empty_like(tx)
+    tmean = torch.empty((n, c, 1, 1), dtype=tx.dtype, device=cuda)
+    tvar = torch.empty((n, c, 1, 1), dtype=tx.dtype, device=cuda)
+    _sync_in()
+    ops.instance_norm(tx, tmean, tvar, ty, eps)
+    ops.stream_sync()
+    helpers.assert_close(ty, ey.reshape(shape), dtype, "y")
+    helpers.assert_close(tvar.reshape(rows), evar, dtype, "var")
+    mean_r = helpers.to_numpy(tmean).reshape(rows).astype(np.float64)
+    rstd_r = 1.0 / np.sqrt(helpers.to_numpy(tvar).reshape(rows).astype(np.float64) + eps)
+    edx, _, _ = oracle.layernorm_bwd(dy.reshape(rows, cols), x.reshape(rows, cols), ones, mean_r.astype(np.float32),
+                                     rstd_r.astype(np.float32))
+    tdx = torch.empty_like(tx)
+    before = ops.pool_stats()["alloc_cnt"]
+    _sync_in()
+    ops.instance_norm_gradient(tdy, tx, tdx, tmean, tvar, eps)
+    ops.stream_sync()
+    helpers.assert_close(tdx, edx.reshape(shape), dtype, "dx")
+    assert ops.pool_stats()["alloc_cnt"] == before          # no column sums, so no scratch
+    with pytest.raises(ops.AssertionError_, match="N, C, H, W"):
+        ops.instance_norm(tx.reshape(n * c, h, w), tmean, tvar, ty.reshape(n * c, h, w), eps)

@@ -311,6 +311,25 @@ def test_reduce_max_min_prod_against_numpy_and_nan_rule():
     assert np.array_equal(oracle.reduce(x[:, :1], [1], "min").reshape(-1), x[:, 0].reshape(-1))
 
 
+def test_nll_loss_is_the_cross_entropy_of_log_softmax():
+    """NLL(log_softmax(x)) is the sparse cross-entropy; its gradient routed through the reference's
+    scaling (-grad * cols at the label) is a one-hot pattern; out-of-range labels give 0 / an all-zero row."""
+    import torch
+    g = np.random.default_rng(15)
+    x = g.standard_normal((9, 40))
+    lab = g.integers(0, 40, size=9)
+    logp = torch.log_softmax(torch.from_numpy(x), dim=1).numpy()
+    assert np.allclose(oracle.nll_loss_fwd(logp, lab), oracle.sce_sparse_fwd(x.astype(np.float32).astype(np.float64).astype(np.float32), lab, -100), rtol=1e-5, atol=1e-6)
+    assert np.allclose(oracle.nll_loss_fwd(logp, lab), torch.nn.functional.nll_loss(torch.from_numpy(logp), torch.from_numpy(lab), reduction="none").numpy(), **F64)
+    lab2 = lab.copy(); lab2[0] = -1; lab2[1] = 40
+    assert oracle.nll_loss_fwd(logp, lab2)[0] == 0.0 and oracle.nll_loss_fwd(logp, lab2)[1] == 0.0
+    gl = g.standard_normal(9)
+    out = oracle.nll_loss_bwd(lab2, gl, 40)
+    assert np.count_nonzero(out) == 7 and not out[0].any() and not out[1].any()
+    for r in range(2, 9):
+        assert out[r, lab2[r]] == -gl[r] * 40
+
+
 # ---------------------------------------------------------------------------
 # fp32 CPU ports (the timed baseline) agree with the float64 oracle
 # ---------------------------------------------------------------------------

@@ -17,7 +17,7 @@ The directory name contains a hyphen, so import it with
 from .capi import (  # noqa: F401
     HkError, lib, lib_path, check, DTYPES, dtype_code, torch_dtype,
     layer_norm_fwd, layer_norm_bwd, norm_bwd_workspace_bytes,
-    dropout_add_ln_fwd, dropout_add_ln_bwd,
+    dropout_add_ln_fwd, dropout_add_ln_bwd, dropout_add_ln_fwd_ex, dropout_add_ln_bwd_ex,
     softmax_fwd, softmax_bwd,
     sce_sparse_fwd, sce_sparse_bwd, sce_dense_fwd, sce_dense_bwd, nll_loss_fwd, nll_loss_bwd,
     reduce, reduce_workspace_bytes, tune_set, copy_kernel, strided_copy,

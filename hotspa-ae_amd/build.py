@@ -19,7 +19,8 @@ LIB = os.path.join(HERE, "lib")
 OBJ = os.path.join(HERE, "build")
 INCLUDE = os.path.join(ROOT, "include")
 
-HIP_SOURCES = ["hk_device.hip", "hk_norm.hip", "hk_softmax.hip", "hk_sce.hip", "hk_reduce.hip", "hk_nll.hip"]
+HIP_SOURCES = ["hk_device.hip", "hk_norm.hip", "hk_softmax.hip", "hk_sce.hip", "hk_reduce.hip", "hk_nll.hip",
+               "hk_dropout_ln.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fvisibility=hidden",

@@ -173,6 +173,92 @@ def dropout_add_ln_bwd(dz, dx_in, x, mu, rsigma, gamma, dx0, dresidual, dgamma, 
     return workspace
 
 
+class DropoutAddLnFwdParams(ctypes.Structure):
+    """hkDropoutAddLnFwdParams of include/hk_rowwise.h"""
+    _fields_ = [("itype", ctypes.c_int), ("rtype", ctypes.c_int), ("wtype", ctypes.c_int),
+                ("rows", ctypes.c_int64), ("cols", ctypes.c_int64), ("x0_numrows", ctypes.c_int64),
+                ("z_numrows", ctypes.c_int64)] + \
+               [(n, ctypes.c_void_p) for n in ("x0", "x1", "residual", "gamma", "beta", "gamma1", "beta1",
+                                               "rowscale", "colscale", "x0_subset", "z_subset", "z", "z1", "x",
+                                               "dmask", "dmask1", "mu", "rs")] + \
+               [("dropout_p", ctypes.c_float), ("epsilon", ctypes.c_float), ("rowscale_const", ctypes.c_float),
+                ("is_rms_norm", ctypes.c_int), ("seed", ctypes.c_uint64), ("offset", ctypes.c_uint64)]
+
+
+class DropoutAddLnBwdParams(ctypes.Structure):
+    """hkDropoutAddLnBwdParams of include/hk_rowwise.h"""
+    _fields_ = [("itype", ctypes.c_int), ("rtype", ctypes.c_int), ("wtype", ctypes.c_int),
+                ("rows", ctypes.c_int64), ("cols", ctypes.c_int64), ("x0_numrows", ctypes.c_int64),
+                ("z_numrows", ctypes.c_int64)] + \
+               [(n, ctypes.c_void_p) for n in ("dz", "dz1", "dx", "x", "x0", "dmask", "dmask1", "mu", "rs", "gamma",
+                                               "gamma1", "rowscale", "colscale", "x0_subset", "z_subset", "dx0",
+                                               "dx1", "dresidual", "dgamma", "dbeta", "dgamma1", "dbeta1",
+                                               "dcolscale", "workspace")] + \
+               [("workspace_bytes", ctypes.c_size_t), ("dropout_p", ctypes.c_float),
+                ("rowscale_const", ctypes.c_float), ("is_rms_norm", ctypes.c_int)]
+
+
+def _addr(t):
+    return None if t is None else t.data_ptr()
+
+
+def dropout_add_ln_fwd_ex(x0, gamma, z, mu, rs, *, x1=None, residual=None, beta=None, gamma1=None, beta1=None,
+                          rowscale=None, colscale=None, x0_subset=None, z_subset=None, z1=None, x=None,
+                          dmask=None, dmask1=None, dropout_p=0.0, eps=1e-5, rowscale_const=1.0, is_rms=False,
+                          seed=0, offset=0, rtype=None, stream=None):
+    """hk_dropout_add_ln_fwd_ex on torch tensors; rows is the length of the subsets when they are given.
+    rtype (a dtype code) names the residual type when neither residual nor x is passed."""
+    p = DropoutAddLnFwdParams()
+    p.itype = dtype_code(x0)
+    p.wtype = dtype_code(gamma)
+    if residual is not None:
+        p.rtype = dtype_code(residual)
+    elif x is not None:
+        p.rtype = dtype_code(x)
+    else:
+        p.rtype = p.itype if rtype is None else rtype
+    p.cols = x0.shape[1]
+    p.rows = x0.shape[0] if x0_subset is None else x0_subset.numel()
+    p.x0_numrows = x0.shape[0]
+    p.z_numrows = z.shape[0]
+    for name, t in (("x0", x0), ("x1", x1), ("residual", residual), ("gamma", gamma), ("beta", beta),
+                    ("gamma1", gamma1), ("beta1", beta1), ("rowscale", rowscale), ("colscale", colscale),
+                    ("x0_subset", x0_subset), ("z_subset", z_subset), ("z", z), ("z1", z1), ("x", x),
+                    ("dmask", dmask), ("dmask1", dmask1), ("mu", mu), ("rs", rs)):
+        setattr(p, name, _addr(t))
+    p.dropout_p = dropout_p; p.epsilon = eps; p.rowscale_const = rowscale_const
+    p.is_rms_norm = int(is_rms); p.seed = seed; p.offset = offset
+    check(lib().hk_dropout_add_ln_fwd_ex(ctypes.byref(p), stream if stream is not None else current_stream()))
+
+
+def dropout_add_ln_bwd_ex(dz, x, mu, rs, gamma, dx0, *, dz1=None, dx=None, x0=None, dmask=None, dmask1=None,
+                          gamma1=None, rowscale=None, colscale=None, x0_subset=None, z_subset=None, dx1=None,
+                          dresidual=None, dgamma=None, dbeta=None, dgamma1=None, dbeta1=None, dcolscale=None,
+                          dropout_p=0.0, rowscale_const=1.0, is_rms=False, workspace=None, stream=None):
+    """hk_dropout_add_ln_bwd_ex on torch tensors; allocates the workspace when none is passed."""
+    p = DropoutAddLnBwdParams()
+    p.itype = dtype_code(dz); p.rtype = dtype_code(x); p.wtype = dtype_code(gamma)
+    p.rows, p.cols = x.shape
+    p.x0_numrows = dx0.shape[0]
+    p.z_numrows = dz.shape[0]
+    for name, t in (("dz", dz), ("dz1", dz1), ("dx", dx), ("x", x), ("x0", x0), ("dmask", dmask),
+                    ("dmask1", dmask1), ("mu", mu), ("rs", rs), ("gamma", gamma), ("gamma1", gamma1),
+                    ("rowscale", rowscale), ("colscale", colscale), ("x0_subset", x0_subset),
+                    ("z_subset", z_subset), ("dx0", dx0), ("dx1", dx1), ("dresidual", dresidual),
+                    ("dgamma", dgamma), ("dbeta", dbeta), ("dgamma1", dgamma1), ("dbeta1", dbeta1),
+                    ("dcolscale", dcolscale)):
+        setattr(p, name, _addr(t))
+    p.dropout_p = dropout_p; p.rowscale_const = rowscale_const; p.is_rms_norm = int(is_rms)
+    if workspace is None:
+        need = ctypes.c_size_t(0)
+        check(lib().hk_dropout_add_ln_bwd_ex_workspace_bytes(ctypes.byref(p), ctypes.byref(need)))
+        workspace = _workspace(need.value, dz.device)
+    p.workspace = _addr(workspace)
+    p.workspace_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(lib().hk_dropout_add_ln_bwd_ex(ctypes.byref(p), stream if stream is not None else current_stream()))
+    return workspace
+
+
 def _odi(shape, dim):
     dim = dim % len(shape)
     outer = 1

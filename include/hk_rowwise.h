@@ -187,6 +187,110 @@ HK_API int hk_dropout_add_ln_bwd(int itype, int rtype, int wtype, const void* dz
                                  int64_t cols, int is_rms_norm, void* workspace,
                                  size_t workspace_bytes, hkStream_t stream);
 
+/* ------------------------------------------------------------------------ *
+ * The same interface with every feature of the flash-attention layer_norm
+ * kernels the reference vendors: dropout, per-row and per-column scaling, row
+ * subsets, mixed input / residual / weight types and the parallel-residual form
+ * (two inputs, two affine outputs of one normalisation).  The parameter blocks
+ * mirror layer_norm::FwdParams / BwdParams (flash-attn csrc/layer_norm ln.h:29-175),
+ * which is what DropoutAddLnFwdCuda / DropoutAddLnBwdCuda (RMSNorm.cu:91-264,
+ * 266-470) and DropoutAddLnParallelResidualFwdCuda / ...BwdCuda (RMSNorm.cu:474-826)
+ * fill before calling the launcher.  Arithmetic: ln_fwd_kernels.cuh:97-182,
+ * ln_bwd_kernels.cuh:93-221, ln_parallel_residual_{fwd,bwd}_kernels.cuh.
+ *
+ * Types.  itype: x0, x1, z, z1, rowscale, dz, dz1, dx0, dx1.  rtype: residual,
+ * x, dx, dresidual.  wtype: gamma, beta, gamma1, beta1, colscale and their
+ * gradients.  mu, rs: fp32.  dmask, dmask1: uint8.  x0_subset, z_subset: int32.
+ * Accepted (wtype, itype, rtype), the combinations the reference registers
+ * (ln_fwd_4096.cu:6-15): all equal (fp32 / fp16 / bf16); (fp32, 16-bit, fp32);
+ * (16-bit, same 16-bit, fp32); (fp32, 16-bit, same 16-bit); (fp16, fp32, fp32).
+ * cols must be a multiple of 8 and at most 8192 (RMSNorm.cu:187).  Data
+ * pointers must be 16-byte aligned, dmask pointers 8-byte aligned.
+ *
+ * Shapes.  rows = rows of x / residual / mu / rs (the length of the subsets when
+ * given).  Without subsets x0, dmask, z, dz, dx0 have `rows` rows.  With
+ * subsets (both or neither): x0, dmask, dx0 have x0_numrows rows, z and dz have
+ * z_numrows rows; x0_subset[r] / z_subset[r] are 1-based row numbers, 0 means
+ * "row r reads no x0" / "row r writes no z"; numbers outside [0, numrows] are
+ * treated as 0; rowscale is ignored and rowscale_const used instead
+ * (ln_fwd_kernels.cuh:99).  The parallel form (x1, gamma1, z1, dz1, dx1 ...)
+ * excludes rowscale, colscale and subsets.
+ *
+ * Dropout.  keep-mask bytes are written to dmask (dmask1 for x1) by the forward
+ * and read back by the backward.  The mask is a pure function of (seed, offset,
+ * element index e in x0): word e % 4 of Philox4x32-10 with key = seed and counter
+ * = (2 * (e / 4) + (0 for x0, 1 for x1), offset), mapped to (0, 1] as
+ * float(bits) * 2^-32 + 2^-33 and kept when <= 1 - dropout_p.  (The reference
+ * keys its stream by the CUDA thread index of a grid sized from the SM count,
+ * ln_fwd_kernels.cuh:66-73, so its mask depends on the device it runs on.)
+ *
+ * Optional pointers may be NULL.  x is written when non-NULL.  Gradients of the
+ * weights are written when non-NULL; they need the workspace reported by
+ * hk_dropout_add_ln_bwd_ex_workspace_bytes.
+ * ------------------------------------------------------------------------ */
+typedef struct hkDropoutAddLnFwdParams {
+  int itype, rtype, wtype;
+  int64_t rows, cols, x0_numrows, z_numrows;
+  const void* x0;        /* [rows | x0_numrows, cols] itype */
+  const void* x1;        /* parallel form: second input */
+  const void* residual;  /* [rows, cols] rtype */
+  const void* gamma;     /* [cols] wtype */
+  const void* beta;
+  const void* gamma1;    /* parallel form: second affine pair (NULL: one output) */
+  const void* beta1;
+  const void* rowscale;  /* [rows] itype */
+  const void* colscale;  /* [cols] wtype */
+  const int32_t* x0_subset;
+  const int32_t* z_subset;
+  void* z;               /* [rows | z_numrows, cols] itype */
+  void* z1;
+  void* x;               /* [rows, cols] rtype: the pre-norm sum */
+  uint8_t* dmask;        /* x0's shape; required when dropout_p > 0 */
+  uint8_t* dmask1;       /* required when dropout_p > 0 and x1 is given */
+  float* mu;             /* [rows] */
+  float* rs;             /* [rows] */
+  float dropout_p, epsilon, rowscale_const;
+  int is_rms_norm;
+  uint64_t seed, offset;
+} hkDropoutAddLnFwdParams;
+
+typedef struct hkDropoutAddLnBwdParams {
+  int itype, rtype, wtype;
+  int64_t rows, cols, x0_numrows, z_numrows;
+  const void* dz;        /* [rows | z_numrows, cols] itype */
+  const void* dz1;       /* parallel form, with gamma1 */
+  const void* dx;        /* [rows, cols] rtype: upstream gradient of the pre-norm sum */
+  const void* x;         /* [rows, cols] rtype */
+  const void* x0;        /* itype; required with colscale */
+  const uint8_t* dmask;  /* required when dropout_p > 0 */
+  const uint8_t* dmask1;
+  const float* mu;
+  const float* rs;
+  const void* gamma;
+  const void* gamma1;
+  const void* rowscale;
+  const void* colscale;
+  const int32_t* x0_subset;
+  const int32_t* z_subset;
+  void* dx0;             /* [rows | x0_numrows, cols] itype */
+  void* dx1;             /* parallel form: gradient of x1 */
+  void* dresidual;       /* [rows, cols] rtype */
+  void* dgamma;          /* [cols] wtype */
+  void* dbeta;
+  void* dgamma1;
+  void* dbeta1;
+  void* dcolscale;
+  void* workspace;
+  size_t workspace_bytes;
+  float dropout_p, rowscale_const;
+  int is_rms_norm;
+} hkDropoutAddLnBwdParams;
+
+HK_API int hk_dropout_add_ln_fwd_ex(const hkDropoutAddLnFwdParams* params, hkStream_t stream);
+HK_API int hk_dropout_add_ln_bwd_ex_workspace_bytes(const hkDropoutAddLnBwdParams* params,
+                                                    size_t* bytes);
+HK_API int hk_dropout_add_ln_bwd_ex(const hkDropoutAddLnBwdParams* params, hkStream_t stream);
+
 /* ======================================================================== *
  * Softmax along one dimension of a dense array viewed as [outer, dim, inner].
  * Replaces SoftmaxCuda (hetu/impl/kernel/Softmax.cu:250-310) and

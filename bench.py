@@ -182,6 +182,44 @@ def case_instance_norm(hk, torch, nsets):
         2 * rows * cols * 2 + 2 * rows * 2, rows
 
 
+def case_dropout_ln(hk, torch, nsets, which):
+    """Pre-norm residual block at the headline shape: x = dropout(x0, 0.1) + residual, z = RMSNorm(x); the
+    backward takes the gradients of z and of the residual stream and returns those of x0 and the residual."""
+    rows, cols, eps, p = 32768, 4096, 1e-6, 0.1
+    bf = torch.bfloat16
+    n = rows * cols
+    sets = []
+    for i in range(nsets):
+        s = dict(x0=_randn(torch, (rows, cols), bf, 1.0, 702 + 10 * i), res=_randn(torch, (rows, cols), bf, 1.0, 703 + 10 * i),
+                 z=torch.empty((rows, cols), dtype=bf, device="cuda"), x=torch.empty((rows, cols), dtype=bf, device="cuda"),
+                 m=torch.empty((rows, cols), dtype=torch.uint8, device="cuda"),
+                 mu=torch.empty(rows, device="cuda"), rs=torch.empty(rows, device="cuda"))
+        sets.append(s)
+    w = _uniform(torch, (cols,), bf, 0.8, 1.2, 704)
+    dg, db = torch.empty_like(w), torch.empty_like(w)
+
+    def fwd(i):
+        s = sets[i % nsets]
+        hk.dropout_add_ln_fwd_ex(s["x0"], w, s["z"], s["mu"], s["rs"], residual=s["res"], x=s["x"], dmask=s["m"],
+                                 dropout_p=p, eps=eps, is_rms=True, seed=1234, offset=i)
+
+    for i in range(nsets):
+        fwd(i)
+    if which == "fwd":
+        return fwd, n * (2 + 2 + 2 + 2 + 1) + cols * 2 + rows * 8, rows
+    # backward reuses x0 / res storage for its outputs (they are not read by it)
+    dz = [_randn(torch, (rows, cols), bf, 1.0, 705 + 10 * i) for i in range(nsets)]
+    ws = hk.dropout_add_ln_bwd_ex(dz[0], sets[0]["x"], sets[0]["mu"], sets[0]["rs"], w, sets[0]["x0"], dx=sets[0]["z"],
+                                  dmask=sets[0]["m"], dresidual=sets[0]["res"], dgamma=dg, dbeta=db, dropout_p=p,
+                                  is_rms=True)
+
+    def bwd(i):
+        s = sets[i % nsets]
+        hk.dropout_add_ln_bwd_ex(dz[i % nsets], s["x"], s["mu"], s["rs"], w, s["x0"], dx=s["z"], dmask=s["m"],
+                                 dresidual=s["res"], dgamma=dg, dbeta=db, dropout_p=p, is_rms=True, workspace=ws)
+    return bwd, n * (2 + 2 + 2 + 1 + 2 + 2) + rows * 4 + cols * 6, rows
+
+
 def case_reduce(hk, torch, nsets, axes, op, three_d=False):
     rows, cols = 32768, 4096
     bf = torch.bfloat16
@@ -244,6 +282,8 @@ CASES = [
     ("next: reduce prod axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "prod")),
     ("next: nll loss bwd bf16 [16384x32000] (write only)", lambda hk, t, n: case_nll_bwd(hk, t, n)),
     ("next: instance norm fwd bf16 [256,256,32,32]", lambda hk, t, n: case_instance_norm(hk, t, n)),
+    ("next: dropout(0.1)+residual+rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_dropout_ln(hk, t, 2, "fwd")),
+    ("next: dropout(0.1)+residual+rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_dropout_ln(hk, t, 2, "bwd")),
     ("C4 rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "fwd")),
     ("C4 rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "bwd")),
     ("C5 sce fwd bf16 [16384x32000]", lambda hk, t, n: case_sce(hk, t, 2, "fwd")),

@@ -557,9 +557,12 @@ static BwdShape plan_dal_bwd(int64_t rows, int cols) {
   const int nchunks = cols / kChunk;
   p.tpr = (nchunks + 63) / 64 * 64;
   p.rpb = p.tpr > 512 ? 1 : 512 / p.tpr;
+  const int forced_rpb = tune_get(TUNE_NORM_BWD_ROWS_PER_BLOCK);
+  if (forced_rpb > 0) p.rpb = std::max(1, std::min(forced_rpb, 1024 / p.tpr));
   p.block = p.tpr * p.rpb;
   // two 512-thread workgroups (one of 1024) per compute unit
   int64_t grid = int64_t(device_cu_count()) * (p.block > 512 ? 1 : 2);
+  if (tune_get(TUNE_NORM_BWD_BLOCKS) > 0) grid = tune_get(TUNE_NORM_BWD_BLOCKS);
   const int64_t useful = (rows + p.rpb - 1) / p.rpb;
   if (grid > useful) grid = useful;
   if (grid < 1) grid = 1;

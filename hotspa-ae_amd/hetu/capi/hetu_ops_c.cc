@@ -4,6 +4,7 @@
 #include <string>
 
 #include "hetu/graph/ops/kernel_links.h"
+#include "hetu/impl/random/CPURandomState.h"
 #include "hetu/impl/memory/CachingMemoryPool.h"
 #include "hetu/impl/stream/HIPStream.h"
 
@@ -125,28 +126,71 @@ int ht_fused_layer_norm_gradient(const HtArray* out_grads, const HtArray* x_or_y
 }
 
 int ht_dropout_add_ln_fwd(const HtArray* x0, const HtArray* residual, const HtArray* gamma, const HtArray* beta,
-                          const HtArray* rowscale, const HtArray* colscale, HtArray* z, HtArray* x, HtArray* mu,
-                          HtArray* rsigma, float dropout_p, float epsilon, int residual_in_fp32, int is_rms_norm,
-                          int stream_index) {
+                          const HtArray* rowscale, const HtArray* colscale, const HtArray* x0_subset,
+                          const HtArray* z_subset, HtArray* z, HtArray* x, HtArray* dmask, HtArray* mu,
+                          HtArray* rsigma, float dropout_p, float epsilon, float rowscale_const, int64_t z_numrows,
+                          int residual_in_fp32, int is_rms_norm, int stream_index) {
   return guarded([&] {
-    NDArray zz = wrap(z), xx = wrap(x), m = wrap(mu), r = wrap(rsigma), dmask, none;
+    NDArray zz = wrap(z), xx = wrap(x), dm = wrap(dmask), m = wrap(mu), r = wrap(rsigma);
     hetu::impl::DropoutAddLnFwdCuda(wrap(x0), wrap(residual), wrap(gamma), wrap(beta), wrap(rowscale),
-                                    wrap(colscale), none, none, zz, xx, dmask, m, r, dropout_p, epsilon, 1.0f, 0,
-                                    residual_in_fp32 != 0, is_rms_norm != 0, stream_of(x0, stream_index));
+                                    wrap(colscale), wrap(x0_subset), wrap(z_subset), zz, xx, dm, m, r, dropout_p,
+                                    epsilon, rowscale_const, z_numrows, residual_in_fp32 != 0, is_rms_norm != 0,
+                                    stream_of(x0, stream_index));
   });
 }
 
-int ht_dropout_add_ln_bwd(const HtArray* dz, const HtArray* dx, const HtArray* x, const HtArray* mu,
-                          const HtArray* rsigma, const HtArray* gamma, const HtArray* rowscale,
-                          const HtArray* colscale, HtArray* dx0, HtArray* dresidual, HtArray* dgamma,
-                          HtArray* dbeta, float dropout_p, int has_residual, int is_rms_norm, int stream_index) {
+int ht_dropout_add_ln_bwd(const HtArray* dz, const HtArray* dx, const HtArray* x, const HtArray* x0,
+                          const HtArray* dmask, const HtArray* mu, const HtArray* rsigma, const HtArray* gamma,
+                          const HtArray* rowscale, const HtArray* colscale, const HtArray* x0_subset,
+                          const HtArray* z_subset, HtArray* dx0, HtArray* dresidual, HtArray* dgamma,
+                          HtArray* dbeta, HtArray* dcolscale, float dropout_p, float rowscale_const,
+                          int64_t x0_numrows, int has_residual, int is_rms_norm, int stream_index) {
   return guarded([&] {
-    NDArray d0 = wrap(dx0), dr = wrap(dresidual), dg = wrap(dgamma), db = wrap(dbeta), none, p1, p2, p3, p4;
-    hetu::impl::DropoutAddLnBwdCuda(wrap(dz), wrap(dx), wrap(x), none, none, wrap(mu), wrap(rsigma), wrap(gamma),
-                                    wrap(rowscale), wrap(colscale), none, none, d0, dr, dg, db, p1, p2, p3, p4,
-                                    dropout_p, 1.0f, 0, has_residual != 0, is_rms_norm != 0,
-                                    stream_of(dz, stream_index));
+    NDArray d0 = wrap(dx0), dr = wrap(dresidual), dg = wrap(dgamma), db = wrap(dbeta), dc = wrap(dcolscale);
+    NDArray p1, p2, p3;
+    hetu::impl::DropoutAddLnBwdCuda(wrap(dz), wrap(dx), wrap(x), wrap(x0), wrap(dmask), wrap(mu), wrap(rsigma),
+                                    wrap(gamma), wrap(rowscale), wrap(colscale), wrap(x0_subset), wrap(z_subset),
+                                    d0, dr, dg, db, p1, p2, dc, p3, dropout_p, rowscale_const, x0_numrows,
+                                    has_residual != 0, is_rms_norm != 0, stream_of(dz, stream_index));
   });
+}
+
+int ht_dropout_add_ln_parallel_residual_fwd(const HtArray* x0, const HtArray* x1, const HtArray* residual,
+                                            const HtArray* gamma0, const HtArray* beta0, const HtArray* gamma1,
+                                            const HtArray* beta1, HtArray* z0, HtArray* z1, HtArray* x,
+                                            HtArray* dmask0, HtArray* dmask1, HtArray* mu, HtArray* rsigma,
+                                            float dropout_p, float epsilon, int residual_in_fp32, int is_rms_norm,
+                                            int stream_index) {
+  return guarded([&] {
+    NDArray a0 = wrap(z0), a1 = wrap(z1), xx = wrap(x), m0 = wrap(dmask0), m1 = wrap(dmask1), m = wrap(mu),
+            r = wrap(rsigma);
+    hetu::impl::DropoutAddLnParallelResidualFwdCuda(wrap(x0), wrap(x1), wrap(residual), wrap(gamma0), wrap(beta0),
+                                                    wrap(gamma1), wrap(beta1), a0, a1, xx, m0, m1, m, r, dropout_p,
+                                                    epsilon, residual_in_fp32 != 0, is_rms_norm != 0,
+                                                    stream_of(x0, stream_index));
+  });
+}
+
+int ht_dropout_add_ln_parallel_residual_bwd(const HtArray* dz0, const HtArray* dz1, const HtArray* dx,
+                                            const HtArray* x, const HtArray* dmask0, const HtArray* dmask1,
+                                            const HtArray* mu, const HtArray* rsigma, const HtArray* gamma0,
+                                            const HtArray* gamma1, HtArray* dx0, HtArray* dx1, HtArray* dresidual,
+                                            HtArray* dgamma0, HtArray* dbeta0, HtArray* dgamma1, HtArray* dbeta1,
+                                            float dropout_p, int has_x1, int has_residual, int is_rms_norm,
+                                            int stream_index) {
+  return guarded([&] {
+    NDArray d0 = wrap(dx0), d1 = wrap(dx1), dr = wrap(dresidual), g0 = wrap(dgamma0), b0 = wrap(dbeta0),
+            g1 = wrap(dgamma1), b1 = wrap(dbeta1), p1, p2, p3, p4;
+    hetu::impl::DropoutAddLnParallelResidualBwdCuda(wrap(dz0), wrap(dz1), wrap(dx), wrap(x), wrap(dmask0),
+                                                    wrap(dmask1), wrap(mu), wrap(rsigma), wrap(gamma0), wrap(gamma1),
+                                                    d0, d1, dr, g0, b0, g1, b1, p1, p2, p3, p4, dropout_p,
+                                                    has_x1 != 0, has_residual != 0, is_rms_norm != 0,
+                                                    stream_of(dz0, stream_index));
+  });
+}
+
+int ht_set_random_seed(uint64_t seed) {
+  return guarded([&] { hetu::impl::SetCPURandomSeed(seed); });
 }
 
 int ht_instance_norm(const HtArray* in, HtArray* mean, HtArray* var, HtArray* out, float eps, int stream_index) {

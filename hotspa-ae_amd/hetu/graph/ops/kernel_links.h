@@ -32,6 +32,18 @@ DECLARE_KERNEL_CUDA(DropoutAddLnBwd, const NDArray&, const NDArray&, const NDArr
                     const NDArray&, const NDArray&, const NDArray&, const NDArray&, const NDArray&, const NDArray&,
                     const NDArray&, const NDArray&, NDArray&, NDArray&, NDArray&, NDArray&, NDArray&, NDArray&,
                     NDArray&, NDArray&, const float, const float, const int64_t, const bool, bool, const Stream&);
+// x0, x1_, residual_, gamma0, beta0_, gamma1_, beta1_, z0, z1, x, dmask0, dmask1, mu, rsigma, dropout_p,
+// epsilon, residual_in_fp32, is_rms_norm
+DECLARE_KERNEL_CUDA(DropoutAddLnParallelResidualFwd, const NDArray&, const NDArray&, const NDArray&,
+                    const NDArray&, const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&, NDArray&,
+                    NDArray&, NDArray&, NDArray&, NDArray&, const float, const float, bool, bool, const Stream&);
+// dz0, dz1_, dx_, x, dmask0_, dmask1_, mu, rsigma, gamma0, gamma1_, dx0, dx1, dresidual, dgamma0, dbeta0,
+// dgamma1, dbeta1, dgamma0_part, dbeta0_part, dgamma1_part, dbeta1_part, dropout_p, has_x1, has_residual,
+// is_rms_norm
+DECLARE_KERNEL_CUDA(DropoutAddLnParallelResidualBwd, const NDArray&, const NDArray&, const NDArray&,
+                    const NDArray&, const NDArray&, const NDArray&, const NDArray&, const NDArray&, const NDArray&,
+                    const NDArray&, NDArray&, NDArray&, NDArray&, NDArray&, NDArray&, NDArray&, NDArray&, NDArray&,
+                    NDArray&, NDArray&, NDArray&, const float, const bool, const bool, bool, const Stream&);
 // in, scale, bias, mean, invvar, out, reduce_dims, eps
 DECLARE_KERNEL_CUDA(FusedLayerNorm, const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&, NDArray&,
                     int64_t, float, const Stream&);

@@ -149,17 +149,43 @@ def fused_layer_norm_gradient(dy, x_or_y, scale, bias, dx, dscale, dbias, mean, 
 
 
 def dropout_add_ln_fwd(x0, residual, gamma, beta, z, x, mu, rsigma, eps, is_rms_norm, dropout_p=0.0,
-                       rowscale=None, colscale=None, residual_in_fp32=False, stream=DEFAULT_STREAM):
+                       rowscale=None, colscale=None, residual_in_fp32=False, x0_subset=None, z_subset=None,
+                       dmask=None, rowscale_const=1.0, z_numrows=0, stream=DEFAULT_STREAM):
     _call("ht_dropout_add_ln_fwd", desc(x0), desc(residual), desc(gamma), desc(beta), desc(rowscale),
-          desc(colscale), desc(z), desc(x), desc(mu), desc(rsigma), _f(dropout_p), _f(eps),
-          ctypes.c_int(int(residual_in_fp32)), ctypes.c_int(int(is_rms_norm)), ctypes.c_int(stream))
+          desc(colscale), desc(x0_subset), desc(z_subset), desc(z), desc(x), desc(dmask), desc(mu), desc(rsigma),
+          _f(dropout_p), _f(eps), _f(rowscale_const), _i64(z_numrows), ctypes.c_int(int(residual_in_fp32)),
+          ctypes.c_int(int(is_rms_norm)), ctypes.c_int(stream))
 
 
 def dropout_add_ln_bwd(dz, dx, x, mu, rsigma, gamma, dx0, dresidual, dgamma, dbeta, has_residual, is_rms_norm,
-                       dropout_p=0.0, rowscale=None, colscale=None, stream=DEFAULT_STREAM):
-    _call("ht_dropout_add_ln_bwd", desc(dz), desc(dx), desc(x), desc(mu), desc(rsigma), desc(gamma),
-          desc(rowscale), desc(colscale), desc(dx0), desc(dresidual), desc(dgamma), desc(dbeta), _f(dropout_p),
+                       dropout_p=0.0, rowscale=None, colscale=None, x0=None, dmask=None, x0_subset=None,
+                       z_subset=None, dcolscale=None, rowscale_const=1.0, x0_numrows=0, stream=DEFAULT_STREAM):
+    _call("ht_dropout_add_ln_bwd", desc(dz), desc(dx), desc(x), desc(x0), desc(dmask), desc(mu), desc(rsigma),
+          desc(gamma), desc(rowscale), desc(colscale), desc(x0_subset), desc(z_subset), desc(dx0),
+          desc(dresidual), desc(dgamma), desc(dbeta), desc(dcolscale), _f(dropout_p), _f(rowscale_const),
+          _i64(x0_numrows), ctypes.c_int(int(has_residual)), ctypes.c_int(int(is_rms_norm)), ctypes.c_int(stream))
+
+
+def dropout_add_ln_parallel_residual_fwd(x0, x1, residual, gamma0, beta0, gamma1, beta1, z0, z1, x, dmask0, dmask1,
+                                         mu, rsigma, dropout_p, eps, residual_in_fp32=False, is_rms_norm=False,
+                                         stream=DEFAULT_STREAM):
+    _call("ht_dropout_add_ln_parallel_residual_fwd", desc(x0), desc(x1), desc(residual), desc(gamma0), desc(beta0),
+          desc(gamma1), desc(beta1), desc(z0), desc(z1), desc(x), desc(dmask0), desc(dmask1), desc(mu),
+          desc(rsigma), _f(dropout_p), _f(eps), ctypes.c_int(int(residual_in_fp32)),
+          ctypes.c_int(int(is_rms_norm)), ctypes.c_int(stream))
+
+
+def dropout_add_ln_parallel_residual_bwd(dz0, dz1, dx, x, dmask0, dmask1, mu, rsigma, gamma0, gamma1, dx0, dx1,
+                                         dresidual, dgamma0, dbeta0, dgamma1, dbeta1, dropout_p, has_x1,
+                                         has_residual, is_rms_norm=False, stream=DEFAULT_STREAM):
+    _call("ht_dropout_add_ln_parallel_residual_bwd", desc(dz0), desc(dz1), desc(dx), desc(x), desc(dmask0),
+          desc(dmask1), desc(mu), desc(rsigma), desc(gamma0), desc(gamma1), desc(dx0), desc(dx1), desc(dresidual),
+          desc(dgamma0), desc(dbeta0), desc(dgamma1), desc(dbeta1), _f(dropout_p), ctypes.c_int(int(has_x1)),
           ctypes.c_int(int(has_residual)), ctypes.c_int(int(is_rms_norm)), ctypes.c_int(stream))
+
+
+def set_random_seed(seed):
+    _call("ht_set_random_seed", ctypes.c_uint64(seed))
 
 
 def instance_norm(x, mean, var, out, eps, stream=DEFAULT_STREAM):

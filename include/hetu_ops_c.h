@@ -61,15 +61,37 @@ HT_API int ht_fused_layer_norm_gradient(const HtArray* out_grads, const HtArray*
                                         const HtArray* bias, HtArray* grad_in, HtArray* grad_scale,
                                         HtArray* grad_bias, const HtArray* mean, const HtArray* invvar,
                                         int64_t reduce_dims, float eps, int inplace, int stream_index);
+/* DropoutAddLnFwdCuda / DropoutAddLnBwdCuda with their full argument lists (hetu/impl/kernel/RMSNorm.cu:91-110,
+ * 266-292; the *_part outputs of the backward are internal scratch here).  Optional arrays may be NULL. */
 HT_API int ht_dropout_add_ln_fwd(const HtArray* x0, const HtArray* residual, const HtArray* gamma,
                                  const HtArray* beta, const HtArray* rowscale, const HtArray* colscale,
-                                 HtArray* z, HtArray* x, HtArray* mu, HtArray* rsigma, float dropout_p,
-                                 float epsilon, int residual_in_fp32, int is_rms_norm, int stream_index);
-HT_API int ht_dropout_add_ln_bwd(const HtArray* dz, const HtArray* dx, const HtArray* x, const HtArray* mu,
-                                 const HtArray* rsigma, const HtArray* gamma, const HtArray* rowscale,
-                                 const HtArray* colscale, HtArray* dx0, HtArray* dresidual, HtArray* dgamma,
-                                 HtArray* dbeta, float dropout_p, int has_residual, int is_rms_norm,
+                                 const HtArray* x0_subset, const HtArray* z_subset, HtArray* z, HtArray* x,
+                                 HtArray* dmask, HtArray* mu, HtArray* rsigma, float dropout_p, float epsilon,
+                                 float rowscale_const, int64_t z_numrows, int residual_in_fp32, int is_rms_norm,
                                  int stream_index);
+HT_API int ht_dropout_add_ln_bwd(const HtArray* dz, const HtArray* dx, const HtArray* x, const HtArray* x0,
+                                 const HtArray* dmask, const HtArray* mu, const HtArray* rsigma,
+                                 const HtArray* gamma, const HtArray* rowscale, const HtArray* colscale,
+                                 const HtArray* x0_subset, const HtArray* z_subset, HtArray* dx0,
+                                 HtArray* dresidual, HtArray* dgamma, HtArray* dbeta, HtArray* dcolscale,
+                                 float dropout_p, float rowscale_const, int64_t x0_numrows, int has_residual,
+                                 int is_rms_norm, int stream_index);
+/* DropoutAddLnParallelResidualFwdCuda / ...BwdCuda (RMSNorm.cu:474-493, 642-668) */
+HT_API int ht_dropout_add_ln_parallel_residual_fwd(const HtArray* x0, const HtArray* x1, const HtArray* residual,
+                                                   const HtArray* gamma0, const HtArray* beta0,
+                                                   const HtArray* gamma1, const HtArray* beta1, HtArray* z0,
+                                                   HtArray* z1, HtArray* x, HtArray* dmask0, HtArray* dmask1,
+                                                   HtArray* mu, HtArray* rsigma, float dropout_p, float epsilon,
+                                                   int residual_in_fp32, int is_rms_norm, int stream_index);
+HT_API int ht_dropout_add_ln_parallel_residual_bwd(const HtArray* dz0, const HtArray* dz1, const HtArray* dx,
+                                                   const HtArray* x, const HtArray* dmask0, const HtArray* dmask1,
+                                                   const HtArray* mu, const HtArray* rsigma, const HtArray* gamma0,
+                                                   const HtArray* gamma1, HtArray* dx0, HtArray* dx1,
+                                                   HtArray* dresidual, HtArray* dgamma0, HtArray* dbeta0,
+                                                   HtArray* dgamma1, HtArray* dbeta1, float dropout_p, int has_x1,
+                                                   int has_residual, int is_rms_norm, int stream_index);
+/* SetCPURandomSeed (hetu/impl/random/CPURandomState.cc:13-18): seeds the source of dropout seeds; 0 is ignored */
+HT_API int ht_set_random_seed(uint64_t seed);
 HT_API int ht_instance_norm(const HtArray* in, HtArray* mean, HtArray* var, HtArray* out, float eps,
                             int stream_index);
 HT_API int ht_instance_norm_gradient(const HtArray* out_grads, const HtArray* in, HtArray* grad_in,

@@ -12,6 +12,7 @@
 #include "hetu/core/ndarray.h"
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/memory/CachingMemoryPool.h"
+#include "hetu/impl/random/CPURandomState.h"
 #include "hetu/impl/utils/dispatch.h"
 
 using namespace hetu;
@@ -115,6 +116,20 @@ int main() {
     CHECK(DataType2Size(kFloat64) == 8 && DataType2Size(kInt64) == 8 && DataType2Size(kUInt8) == 1);
     CHECK(int(kFloat16) == 5 && int(kFloat32) == 6 && int(kFloat64) == 7 && int(kBFloat16) == 8 && int(kInt64) == 4);
     CHECK(DataType2Str(kBFloat16) == "bfloat16");
+  });
+
+  run("seed source: unseeded follows the clock, seeded replays a 64-bit Mersenne Twister", [] {
+    using hetu::impl::GenNextRandomSeed;
+    using hetu::impl::SetCPURandomSeed;
+    CHECK(GenNextRandomSeed() != 0);
+    SetCPURandomSeed(0);                                     // ignored
+    SetCPURandomSeed(5489);                                  // the generator's own default seed
+    CHECK(GenNextRandomSeed() == 14514284786278117030ull);   // its documented first output
+    uint64_t v = 0;
+    for (int i = 1; i < 10000; ++i) v = GenNextRandomSeed();
+    CHECK(v == 9981545732273789042ull);                      // and its 10000th (the C++ standard's check value)
+    SetCPURandomSeed(5489);
+    CHECK(GenNextRandomSeed() == 14514284786278117030ull);
   });
 
   run("bfloat16 rounds to nearest even and keeps NaN", [] {

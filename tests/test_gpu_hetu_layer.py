@@ -153,7 +153,7 @@ def test_dropout_add_ln(ops, cuda, dtype, is_rms, with_residual):
         helpers.assert_close(tdres, edx0, dtype, "dresidual")
 
 
-def test_dropout_add_ln_refuses_what_it_does_not_compute(ops, cuda):
+def test_dropout_add_ln_checks(ops, cuda):
     import torch
     rows, cols = 8, 256
     x0 = torch.zeros(rows, cols, device=cuda)
@@ -162,15 +162,171 @@ def test_dropout_add_ln_refuses_what_it_does_not_compute(ops, cuda):
     mu = torch.empty(rows, device=cuda)
     rs = torch.empty(rows, device=cuda)
     _sync_in()
-    with pytest.raises(ops.NotImplemented_, match="dropout"):
+    with pytest.raises(ops.AssertionError_, match="x must be given"):       # dropout keeps the pre-norm sum
         ops.dropout_add_ln_fwd(x0, None, g, None, z, None, mu, rs, 1e-6, True, dropout_p=0.1)
-    with pytest.raises(ops.NotImplemented_, match="scaling"):
-        ops.dropout_add_ln_fwd(x0, None, g, None, z, None, mu, rs, 1e-6, True, colscale=g)
+    with pytest.raises(ops.AssertionError_, match="dmask must be given"):
+        ops.dropout_add_ln_fwd(x0, None, g, None, z, torch.empty_like(x0), mu, rs, 1e-6, True, dropout_p=0.1)
+    with pytest.raises(ops.AssertionError_, match="z_subset"):
+        ops.dropout_add_ln_fwd(x0, None, g, None, z, torch.empty_like(x0), mu, rs, 1e-6, True,
+                               x0_subset=torch.ones(rows, dtype=torch.int32, device=cuda))
+    with pytest.raises(ops.NotImplemented_, match="no kernel for weight dtype"):   # bf16 weights, fp32 input
+        ops.dropout_add_ln_fwd(x0, None, g.bfloat16(), None, z, torch.empty_like(x0), mu, rs, 1e-6, True,
+                               colscale=g.bfloat16())
     with pytest.raises(ops.AssertionError_, match="multiple of 8"):
         ops.dropout_add_ln_fwd(x0[:, :252].contiguous(), None, g[:252].contiguous(), None,
                                z[:, :252].contiguous(), None, mu, rs, 1e-6, True)
     with pytest.raises(ops.AssertionError_):     # x0 must be dense
         ops.dropout_add_ln_fwd(x0.t(), None, g, None, z, None, mu, rs, 1e-6, True)
+
+
+MT19937_64_FIRST_OF_5489 = 14514284786278117030   # first output of std::mt19937_64 seeded with its default 5489
+
+
+@pytest.mark.parametrize("is_rms", [False, True])
+def test_dropout_add_ln_full_feature_set(ops, cuda, is_rms):
+    """Dropout + rowscale + colscale + residual in fp32 with bf16 input through DropoutAddLnFwdCuda / BwdCuda.
+    The seed comes from the layer's seeded generator, so the mask is known in advance."""
+    import torch
+    from oracle import dropout_add_ln as dal
+    rows, cols, eps, p = 40, 1024, 1e-5, 0.2
+    x0 = helpers.draw(1, (rows, cols), dtype="bf16"); residual = helpers.draw(2, (rows, cols), dtype="fp32")
+    gamma = helpers.draw(3, (cols,), "uniform", 0.5, 1.5, "fp32"); beta = helpers.draw(4, (cols,), "normal", 0, 0.1, "fp32")
+    rowscale = helpers.draw(5, (rows,), "uniform", 0.5, 2.0, "bf16")
+    colscale = helpers.draw(6, (cols,), "uniform", 0.5, 2.0, "fp32")
+    dz = helpers.draw(7, (rows, cols), dtype="bf16"); dx_in = helpers.draw(8, (rows, cols), dtype="fp32")
+    emask = dal.dropout_keep(MT19937_64_FIRST_OF_5489, 0, rows * cols, np.float32(1) - np.float32(p)).reshape(rows, cols)
+    ez, ex, emu, ers = dal.fwd(x0, residual, gamma, None if is_rms else beta, rowscale, colscale, dmask=emask,
+                               dropout_p=p, eps=eps, is_rms=is_rms)
+    tx0, trow, tdz = _dev((x0, rowscale, dz), "bf16", cuda)
+    tres, tg, tb, tcol, tdxin = _dev((residual, gamma, beta, colscale, dx_in), "fp32", cuda)
+    tz = torch.empty_like(tx0); tx = torch.empty_like(tres)
+    tm = torch.zeros(rows, cols, dtype=torch.uint8, device=cuda)
+    tmu = torch.empty(rows, device=cuda); trs = torch.empty(rows, device=cuda)
+    _sync_in()
+    ops.set_random_seed(5489)
+    ops.dropout_add_ln_fwd(tx0, tres, tg, None if is_rms else tb, tz, tx, tmu, trs, eps, is_rms, dropout_p=p,
+                           rowscale=trow, colscale=tcol, dmask=tm)
+    ops.stream_sync()
+    assert np.array_equal(tm.cpu().numpy(), emask)
+    helpers.assert_close(tz, ez, "bf16", "z")
+    helpers.assert_close(tx, ex, "fp32", "x")
+    helpers.assert_close(trs, ers, "fp32", "rsigma")
+    # the generator moves on: a second call draws another mask; reseeding brings the first one back
+    tm2 = torch.zeros_like(tm)
+    ops.dropout_add_ln_fwd(tx0, tres, tg, None if is_rms else tb, tz, tx, tmu, trs, eps, is_rms, dropout_p=p,
+                           rowscale=trow, colscale=tcol, dmask=tm2)
+    ops.stream_sync()
+    assert 0.2 < (tm2 != tm).float().mean().item() < 0.45
+    ops.set_random_seed(5489)
+    ops.dropout_add_ln_fwd(tx0, tres, tg, None if is_rms else tb, tz, tx, tmu, trs, eps, is_rms, dropout_p=p,
+                           rowscale=trow, colscale=tcol, dmask=tm2)
+    ops.stream_sync()
+    assert torch.equal(tm2, tm)
+
+    xs = helpers.to_numpy(tx); mu32 = helpers.to_numpy(tmu); rs32 = helpers.to_numpy(trs)
+    edx0, edres, edg, edb, edcol = dal.bwd(dz, dx_in, xs, x0, emask, mu32, rs32, gamma, rowscale, colscale,
+                                           dropout_p=p, is_rms=is_rms)
+    tdx0 = torch.empty_like(tx0); tdres = torch.empty_like(tres)
+    tdg, tdb, tdcol = torch.empty_like(tg), torch.empty_like(tg), torch.empty_like(tg)
+    _sync_in()
+    ops.dropout_add_ln_bwd(tdz, tdxin, tx, tmu, trs, tg, tdx0, tdres, tdg, tdb, True, is_rms, dropout_p=p,
+                           rowscale=trow, colscale=tcol, x0=tx0, dmask=tm, dcolscale=tdcol)
+    ops.stream_sync()
+    helpers.assert_close(tdx0, edx0, "bf16", "dx0")
+    helpers.assert_close(tdres, edres, "fp32", "dresidual")
+    helpers.assert_close(tdg, edg, "fp32", "dgamma")
+    helpers.assert_close(tdb, edb, "fp32", "dbeta")
+    helpers.assert_close(tdcol, edcol, "fp32", "dcolscale")
+
+
+def test_dropout_add_ln_row_subsets(ops, cuda):
+    import torch
+    from oracle import dropout_add_ln as dal
+    rows, x0_rows, z_rows, cols, eps, rsc = 12, 7, 5, 512, 1e-5, 0.5
+    x0_subset = np.array([1, 0, 2, 3, 0, 4, 0, 5, 6, 0, 7, 0], dtype=np.int32)
+    z_subset = np.array([0, 1, 0, 2, 3, 0, 4, 0, 0, 5, 0, 0], dtype=np.int32)
+    x0 = helpers.draw(1, (x0_rows, cols), dtype="fp16"); residual = helpers.draw(2, (rows, cols), dtype="fp16")
+    gamma = helpers.draw(3, (cols,), "uniform", 0.5, 1.5, "fp16"); beta = helpers.draw(4, (cols,), "normal", 0, 0.1, "fp16")
+    dz = helpers.draw(5, (z_rows, cols), dtype="fp16")
+    ez, ex, emu, ers = dal.fwd(x0, residual, gamma, beta, None, None, x0_subset, z_subset, None, 0.0, eps, rsc,
+                               z_rows, False)
+    tx0, tres, tg, tb, tdz = _dev((x0, residual, gamma, beta, dz), "fp16", cuda)
+    sx0, sz = helpers.to_torch(x0_subset, "int32", cuda), helpers.to_torch(z_subset, "int32", cuda)
+    tz = torch.empty(z_rows, cols, dtype=torch.float16, device=cuda); tx = torch.empty_like(tres)
+    tmu = torch.empty(rows, device=cuda); trs = torch.empty(rows, device=cuda)
+    _sync_in()
+    ops.dropout_add_ln_fwd(tx0, tres, tg, tb, tz, tx, tmu, trs, eps, False, x0_subset=sx0, z_subset=sz,
+                           rowscale_const=rsc, z_numrows=z_rows)
+    ops.stream_sync()
+    helpers.assert_close(tz, ez, "fp16", "z")
+    helpers.assert_close(tx, ex, "fp16", "x")
+    xs = helpers.to_numpy(tx); mu32 = helpers.to_numpy(tmu); rs32 = helpers.to_numpy(trs)
+    edx0, edres, edg, edb, _ = dal.bwd(dz, None, xs, x0, None, mu32, rs32, gamma, None, None, x0_subset, z_subset,
+                                       0.0, rsc, x0_rows, False)
+    tdx0 = torch.empty_like(tx0); tdres = torch.empty_like(tres)
+    tdg, tdb = torch.empty_like(tg), torch.empty_like(tg)
+    _sync_in()
+    ops.dropout_add_ln_bwd(tdz, None, tx, tmu, trs, tg, tdx0, tdres, tdg, tdb, True, False, x0_subset=sx0,
+                           z_subset=sz, rowscale_const=rsc, x0_numrows=x0_rows)
+    ops.stream_sync()
+    helpers.assert_close(tdx0, edx0, "fp16", "dx0")
+    helpers.assert_close(tdres, edres, "fp16", "dresidual")
+    helpers.assert_close(tdg, edg, "fp16", "dgamma")
+    helpers.assert_close(tdb, edb, "fp16", "dbeta")
+    with pytest.raises(ops.AssertionError_, match="z must have shape"):
+        ops.dropout_add_ln_fwd(tx0, tres, tg, tb, tz, tx, tmu, trs, eps, False, x0_subset=sx0, z_subset=sz,
+                               rowscale_const=rsc, z_numrows=z_rows + 1)
+
+
+@pytest.mark.parametrize("tied", [False, True])
+def test_dropout_add_ln_parallel_residual(ops, cuda, tied):
+    import torch
+    from oracle import dropout_add_ln as dal
+    rows, cols, eps, p = 24, 2048, 1e-5, 0.1
+    dt = "bf16"
+    x0 = helpers.draw(1, (rows, cols), dtype=dt); x1 = helpers.draw(2, (rows, cols), dtype=dt)
+    residual = helpers.draw(3, (rows, cols), dtype=dt)
+    g0 = helpers.draw(4, (cols,), "uniform", 0.5, 1.5, dt); b0 = helpers.draw(5, (cols,), "normal", 0, 0.1, dt)
+    g1 = None if tied else helpers.draw(6, (cols,), "uniform", 0.5, 1.5, dt)
+    b1 = None if tied else helpers.draw(7, (cols,), "normal", 0, 0.1, dt)
+    dz0 = helpers.draw(8, (rows, cols), dtype=dt); dz1 = None if tied else helpers.draw(9, (rows, cols), dtype=dt)
+    keep = np.float32(1) - np.float32(p)
+    m0 = dal.dropout_keep(MT19937_64_FIRST_OF_5489, 0, rows * cols, keep, 0).reshape(rows, cols)
+    m1 = dal.dropout_keep(MT19937_64_FIRST_OF_5489, 0, rows * cols, keep, 1).reshape(rows, cols)
+    ez0, ez1, ex, emu, ers = dal.parallel_fwd(x0, x1, residual, g0, b0, g1, b1, m0, m1, p, eps, False)
+    T = lambda a: None if a is None else helpers.to_torch(a, dt, cuda)
+    tx0, tx1, tres, tg0, tb0, tg1, tb1, tdz0, tdz1 = map(T, (x0, x1, residual, g0, b0, g1, b1, dz0, dz1))
+    tz0 = torch.empty_like(tx0); tz1 = None if tied else torch.empty_like(tx0); tx = torch.empty_like(tx0)
+    tm0 = torch.zeros(rows, cols, dtype=torch.uint8, device=cuda); tm1 = torch.zeros_like(tm0)
+    tmu = torch.empty(rows, device=cuda); trs = torch.empty(rows, device=cuda)
+    _sync_in()
+    ops.set_random_seed(5489)
+    ops.dropout_add_ln_parallel_residual_fwd(tx0, tx1, tres, tg0, tb0, tg1, tb1, tz0, tz1, tx, tm0, tm1, tmu, trs,
+                                             p, eps)
+    ops.stream_sync()
+    assert np.array_equal(tm0.cpu().numpy(), m0) and np.array_equal(tm1.cpu().numpy(), m1)
+    helpers.assert_close(tz0, ez0, dt, "z0")
+    if not tied:
+        helpers.assert_close(tz1, ez1, dt, "z1")
+    helpers.assert_close(tx, ex, dt, "x")
+    xs = helpers.to_numpy(tx); mu32 = helpers.to_numpy(tmu); rs32 = helpers.to_numpy(trs)
+    edx0, edx1, edres, edg0, edb0, edg1, edb1 = dal.parallel_bwd(dz0, dz1, None, xs, m0, m1, mu32, rs32, g0, g1, p,
+                                                                 True, False)
+    tdx0, tdx1, tdres = torch.empty_like(tx0), torch.empty_like(tx0), torch.empty_like(tx0)
+    tdg0, tdb0 = torch.empty_like(tg0), torch.empty_like(tg0)
+    tdg1 = None if tied else torch.empty_like(tg0); tdb1 = None if tied else torch.empty_like(tg0)
+    _sync_in()
+    ops.dropout_add_ln_parallel_residual_bwd(tdz0, tdz1, None, tx, tm0, tm1, tmu, trs, tg0, tg1, tdx0, tdx1, tdres,
+                                             tdg0, tdb0, tdg1, tdb1, p, True, True)
+    ops.stream_sync()
+    helpers.assert_close(tdx0, edx0, dt, "dx0")
+    helpers.assert_close(tdx1, edx1, dt, "dx1")
+    helpers.assert_close(tdres, edres, dt, "dresidual")
+    helpers.assert_close(tdg0, edg0, dt, "dgamma0")
+    helpers.assert_close(tdb0, edb0, dt, "dbeta0")
+    if not tied:
+        helpers.assert_close(tdg1, edg1, dt, "dgamma1")
+        helpers.assert_close(tdb1, edb1, dt, "dbeta1")
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])

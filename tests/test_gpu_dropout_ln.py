@@ -237,6 +237,47 @@ def test_parallel_residual(hk, cuda, combo, has_x1, tied, p, is_rms, shape):
         helpers.assert_close(tdb1, edb1, wt, "dbeta1")
 
 
+@pytest.mark.parametrize("combo", COMBOS, ids=lambda c: "w%s-i%s-r%s" % c)
+@pytest.mark.parametrize("rows,cols,blocks", [(1, 512, 0), (61, 512, 2), (50, 4096, 3), (2500, 4096, 0),
+                                               (37, 5120, 5), (19, 8192, 4), (23, 1000, 2)])
+@pytest.mark.parametrize("is_rms", [False, True])
+def test_prenorm_block_backward(hk, cuda, combo, rows, cols, blocks, is_rms):
+    """Dropout + incoming and outgoing residual-stream gradients and nothing else: the form with a kernel of
+    its own when the row fills every thread (cols = 1000 does not and takes the general kernel).  A forced
+    small grid makes every thread group walk many rows, through full rounds and the guarded tail."""
+    import torch
+    wt, it, rt = combo
+    p = 0.15
+    seed = 8100 + rows + cols
+    x = helpers.draw(seed, (rows, cols), dtype=rt)
+    gamma = helpers.draw(seed + 1, (cols,), "uniform", 0.5, 1.5, wt)
+    dz = helpers.draw(seed + 2, (rows, cols), dtype=it)
+    dx_in = helpers.draw(seed + 3, (rows, cols), dtype=rt)
+    mask = _mask(rows * cols, p).reshape(rows, cols)
+    xd = x.astype(np.float64)
+    mu = xd.mean(axis=1)
+    rs = 1.0 / np.sqrt((xd * xd).mean(axis=1) + 1e-5) if is_rms else 1.0 / np.sqrt(xd.var(axis=1) + 1e-5)
+    mu32, rs32 = mu.astype(np.float32), rs.astype(np.float32)
+    edx0, edres, edg, edb, _ = dal.bwd(dz, dx_in, x, None, mask, mu32, rs32, gamma, dropout_p=p, is_rms=is_rms)
+    tx, tdxin = _tt(x, rt, cuda), _tt(dx_in, rt, cuda)
+    tdz, tg = _tt(dz, it, cuda), _tt(gamma, wt, cuda)
+    tdx0 = torch.empty_like(tdz); tdres = torch.empty_like(tx)
+    tdg, tdb = torch.empty_like(tg), torch.empty_like(tg)
+    hk.tune_set("norm_bwd_blocks", blocks)
+    try:
+        hk.dropout_add_ln_bwd_ex(tdz, tx, _tt(mu32, "fp32", cuda), _tt(rs32, "fp32", cuda), tg, tdx0, dx=tdxin,
+                                 dmask=_tt(mask, "uint8", cuda), dresidual=tdres, dgamma=tdg, dbeta=tdb,
+                                 dropout_p=p, is_rms=is_rms)
+        torch.cuda.synchronize()
+    finally:
+        hk.tune_set("norm_bwd_blocks", 0)
+    helpers.assert_close(tdx0, edx0, it, "dx0")
+    helpers.assert_close(tdres, edres, rt, "dresidual")
+    helpers.assert_close(tdg, edg, wt, "dgamma")
+    helpers.assert_close(tdb, edb, wt, "dbeta")
+    assert (helpers.to_numpy(tdx0)[mask == 0] == 0).all()
+
+
 def test_plain_call_matches_the_plain_entry_point(hk, cuda):
     """No feature and uniform types: the call is handed to the tuned kernels, bit for bit."""
     import torch

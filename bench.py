@@ -436,7 +436,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=300,
                     help="untimed steps; a few hundred let the clocks settle after idle")
     ap.add_argument("--all", action="store_true", help="also time every kernel of every configuration")
-    ap.add_argument("--only", default="", help="substring filter for --all")
+    ap.add_argument("--only", default="", help="substring filter for --all (comma-separated: any of them)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--nsets", type=int, default=3, help="rotating buffer sets (working set > cache)")
     args = ap.parse_args()
@@ -453,7 +453,7 @@ def main():
     kernels = []
     if args.all:
         for name, make in CASES:
-            if args.only and args.only not in name:
+            if args.only and not any(part in name for part in args.only.split(",")):
                 continue
             launch, nbytes, rows = make(hk, torch, args.nsets)
             ms, main_us = time_case(hk, torch, launch, args.steps, args.warmup,

@@ -259,6 +259,46 @@ def dropout_add_ln_bwd_ex(dz, x, mu, rs, gamma, dx0, *, dz1=None, dx=None, x0=No
     return workspace
 
 
+UNARY_OPS = {"exp": 0, "log": 1, "neg": 2, "sqrt": 3}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+
+
+def unary(op, x, out, stream=None):
+    """hk_unary: out = op(x), dense arrays of one dtype (out may be x)."""
+    check(lib().hk_unary(UNARY_OPS[op], dtype_code(x), _ptr(x), _ptr(out), _i64(x.numel()),
+                         stream if stream is not None else current_stream()))
+
+
+def binary_const(op, x, scalar, out, scalar_first=False, stream=None):
+    """hk_binary_const: out = x op scalar (scalar op x when scalar_first)."""
+    check(lib().hk_binary_const(BINARY_OPS[op], dtype_code(x), _ptr(x), ctypes.c_double(scalar),
+                                ctypes.c_int(int(scalar_first)), _ptr(out), _i64(x.numel()),
+                                stream if stream is not None else current_stream()))
+
+
+def binary(op, a, b, out, stream=None):
+    """hk_binary: out = a op b, broadcasting a and b (any strides) to out's shape; out is dense."""
+    shape = list(out.shape)
+    sa = list(a.expand(shape).stride())
+    sb = list(b.expand(shape).stride())
+    check(lib().hk_binary(BINARY_OPS[op], dtype_code(out), _ptr(a), _ptr(b), _ptr(out), ctypes.c_int(len(shape)),
+                          _arr(shape), _arr(sa), _arr(sb), stream if stream is not None else current_stream()))
+
+
+def vocab_parallel_ce_gather(logits, labels, vocab_start, vocab_end, ignored_index, picked, lse, stream=None):
+    rows, cols = logits.shape
+    check(lib().hk_vocab_parallel_ce_gather(dtype_code(logits), _ptr(logits), _ptr(labels), _i64(rows), _i64(cols),
+                                            _i64(vocab_start), _i64(vocab_end), _i64(ignored_index), _ptr(picked),
+                                            _ptr(lse), stream if stream is not None else current_stream()))
+
+
+def vocab_parallel_ce_bwd(softmax, labels, grad_loss, out, vocab_start, stream=None):
+    rows, cols = softmax.shape
+    check(lib().hk_vocab_parallel_ce_bwd(dtype_code(softmax), _ptr(softmax), _ptr(labels), _ptr(grad_loss),
+                                         _ptr(out), _i64(rows), _i64(cols), _i64(vocab_start),
+                                         stream if stream is not None else current_stream()))
+
+
 def _odi(shape, dim):
     dim = dim % len(shape)
     outer = 1

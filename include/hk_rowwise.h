@@ -344,6 +344,54 @@ HK_API int hk_nll_loss_bwd(int dtype, const int64_t* labels, const void* grad_lo
                            int64_t rows, int64_t cols, hkStream_t stream);
 
 /* ======================================================================== *
+ * Local kernels of the vocabulary-parallel cross-entropy: this device holds the
+ * columns [vocab_start, vocab_end) of the logits, [rows, cols] dense.
+ *   gather: picked[r] = logits[r, labels[r] - vocab_start] when the label lies in
+ *     the shard, else 0; a row whose label is ignored_index gets picked = 0 AND
+ *     lse = 0; lse of every other row is left untouched (the caller has put
+ *     log(sum(exp)) there).
+ *   bwd: out[r, c] = (softmax[r, c] - [c == labels[r] - vocab_start]) * grad_loss[r];
+ *     the column test is on unsigned 64-bit values, so labels outside the shard
+ *     and negative labels match nothing; ignored rows are not special-cased (the
+ *     caller zeroes their grad_loss).  out may alias softmax.
+ * Replaces VocabParallelCrossEntropyCuda / VocabParallelCrossEntropyGradientCuda
+ * (hetu/impl/kernel/VocabParallelCrossEntropyLoss.cu:14-64, 69-119).
+ * ======================================================================== */
+HK_API int hk_vocab_parallel_ce_gather(int dtype, const void* logits, const int64_t* labels,
+                                       int64_t rows, int64_t cols, int64_t vocab_start,
+                                       int64_t vocab_end, int64_t ignored_index, void* picked,
+                                       void* lse, hkStream_t stream);
+HK_API int hk_vocab_parallel_ce_bwd(int dtype, const void* softmax, const int64_t* labels,
+                                    const void* grad_loss, void* out, int64_t rows, int64_t cols,
+                                    int64_t vocab_start, hkStream_t stream);
+
+/* ======================================================================== *
+ * Element-wise operators on dense arrays of fp32 / bf16 / fp16 / fp64 (16-bit
+ * types compute in fp32 and round once).  out may alias an input of its shape.
+ *   hk_unary: exp, log, negate, sqrt.  Replaces ExpCuda, LogCuda, OppositeCuda,
+ *     SqrtCuda (hetu/impl/kernel/Exp.cu:12-29, Log.cu, Opposite.cu, Sqrt.cu).
+ *   hk_binary_const: x op c, or c op x when scalar_first != 0 (sub, div); the
+ *     constant is first rounded to the array's type.  Replaces AddConstCuda,
+ *     SubConstCuda (c - x), MulConstCuda, DivConstCuda (c / x)
+ *     (hetu/impl/kernel/BinaryConst.cu:10-53).
+ *   hk_binary: out = a op b with broadcasting.  out is dense with shape
+ *     out_shape[ndim] (ndim <= 8); a_strides / b_strides are the operands'
+ *     element strides aligned to out_shape, 0 along a broadcast dimension.
+ *     Replaces AddElewiseCuda, SubElewiseCuda, MulElewiseCuda, DivElewiseCuda
+ *     (hetu/impl/kernel/BinaryElewise.cu) and the launch_loop_kernel /
+ *     vectorize_broadcast_loop_kernel family they run on (Vectorized.cuh).
+ * Integer arrays are not implemented (HK_ERR_UNSUPPORTED).
+ * ======================================================================== */
+enum { HK_UNARY_EXP = 0, HK_UNARY_LOG = 1, HK_UNARY_NEG = 2, HK_UNARY_SQRT = 3 };
+enum { HK_BINARY_ADD = 0, HK_BINARY_SUB = 1, HK_BINARY_MUL = 2, HK_BINARY_DIV = 3 };
+HK_API int hk_unary(int op, int dtype, const void* in, void* out, int64_t numel, hkStream_t stream);
+HK_API int hk_binary_const(int op, int dtype, const void* in, double scalar, int scalar_first,
+                           void* out, int64_t numel, hkStream_t stream);
+HK_API int hk_binary(int op, int dtype, const void* a, const void* b, void* out, int ndim,
+                     const int64_t* out_shape, const int64_t* a_strides, const int64_t* b_strides,
+                     hkStream_t stream);
+
+/* ======================================================================== *
  * Reduce sum / mean / max / min / product over a set of axes of a (possibly
  * strided) array.
  * shape / strides (in elements) describe the input; axes must already be

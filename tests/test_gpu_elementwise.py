@@ -1,0 +1,239 @@
+"""GPU parity of the element-wise operators (hk_unary, hk_binary_const, hk_binary) and of the
+vocabulary-parallel cross-entropy's local kernels (hk_vocab_parallel_ce_gather / _bwd) through the C-ABI.
+The expected values are numpy float64 one-liners of the operator's definition (np.exp, a - b, ...), rounded
+nowhere; tolerances 1e-5 (fp32) / 1e-2 (bf16, fp16) / 1e-12 (fp64)."""
+import numpy as np
+import pytest
+
+import helpers
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["fp32", "bf16", "fp16", "fp64"]
+NP_UNARY = {"exp": np.exp, "log": np.log, "neg": np.negative, "sqrt": np.sqrt}
+NP_BINARY = {"add": np.add, "sub": np.subtract, "mul": np.multiply, "div": np.divide}
+
+
+def _draw(seed, shape, dtype, positive=False):
+    g = helpers.rng(seed)
+    v = g.standard_normal(shape) if not positive else g.uniform(0.5, 4.0, shape)
+    return v.astype(np.float64) if dtype == "fp64" else oracle.round_to(v.astype(np.float32), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("op", ["exp", "log", "neg", "sqrt"])
+@pytest.mark.parametrize("n", [1, 7, 4096, 100003, 1 << 20])
+def test_unary(hk, cuda, dtype, op, n):
+    import torch
+    x = _draw(11 + n, (n,), dtype, positive=op in ("log", "sqrt"))
+    tx = helpers.to_torch(x, dtype, cuda)
+    ty = torch.empty_like(tx)
+    hk.unary(op, tx, ty)
+    torch.cuda.synchronize()
+    helpers.assert_close(ty, NP_UNARY[op](x.astype(np.float64)), dtype, op)
+    # in place, and from an address that is not 16-byte aligned
+    if n > 8:
+        tv = tx[1:]
+        hk.unary(op, tv, tv)
+        torch.cuda.synchronize()
+        helpers.assert_close(tv, NP_UNARY[op](x[1:].astype(np.float64)), dtype, op + " in place")
+
+
+def test_unary_special_values(hk, cuda):
+    import torch
+    x = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), float("nan"), 88.0, -80.0, 1e-30], device=cuda)
+    y = torch.empty_like(x)
+    hk.unary("exp", x, y)
+    torch.cuda.synchronize()
+    assert torch.allclose(y, torch.exp(x), rtol=1e-6, atol=0, equal_nan=True)
+    hk.unary("log", x, y)
+    torch.cuda.synchronize()
+    assert torch.allclose(y, torch.log(x), rtol=1e-6, atol=0, equal_nan=True)
+    hk.unary("sqrt", x, y)
+    torch.cuda.synchronize()
+    assert torch.allclose(y, torch.sqrt(x), rtol=1e-6, atol=0, equal_nan=True)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("op,first", [("add", False), ("mul", False), ("sub", True), ("div", True), ("sub", False),
+                                      ("div", False)])
+@pytest.mark.parametrize("n", [5, 8192, 100003])
+def test_binary_const(hk, cuda, dtype, op, first, n):
+    import torch
+    x = _draw(21 + n, (n,), dtype, positive=True)
+    c = 1.0 / 3.0
+    # the constant enters rounded to the array's type (static_cast<spec_t>(value) in the reference)
+    cr = c if dtype == "fp64" else float(oracle.round_to(np.array([c], np.float32), dtype)[0])
+    xd = x.astype(np.float64)
+    want = NP_BINARY[op](cr, xd) if first else NP_BINARY[op](xd, cr)
+    tx = helpers.to_torch(x, dtype, cuda)
+    ty = torch.empty_like(tx)
+    hk.binary_const(op, tx, c, ty, scalar_first=first)
+    torch.cuda.synchronize()
+    helpers.assert_close(ty, want, dtype, op)
+    if dtype == "bf16" and op == "mul" and n >= 8192:
+        # one fp32 product, one rounding: bit-exact with the constant rounded to bf16 first (bf16(1/3) lies 2e-3
+        # above 1/3), and visibly different from the product with the unrounded constant
+        got = helpers.to_numpy(ty)
+        assert np.array_equal(got, oracle.round_to(x.astype(np.float32) * np.float32(cr), "bf16"))
+        assert (got != oracle.round_to(x.astype(np.float32) * np.float32(c), "bf16")).mean() > 0.2
+
+
+BROADCASTS = [
+    ((64, 4096), (64, 4096)),          # same shape
+    ((64, 4096), (64, 1)),             # per-row value (logits - row maximum)
+    ((64, 4096), (4096,)),             # per-column vector
+    ((64, 1), (1, 4096)),              # outer combination
+    ((64, 4096), ()),                  # single value
+    ((3, 5, 7, 16), (5, 1, 16)),       # merges to nothing two-dimensional: generic kernel
+    ((6, 10, 256), (6, 10, 1)),        # leading dims merge: [60, 256] op [60, 1]
+    ((33, 1001), (33, 1)),             # odd row length: scalar path
+    ((1,), (1,)),
+    ((2, 3, 4, 5, 6, 2, 3, 2), (2, 1, 4, 1, 6, 1, 3, 1)),   # eight dims
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+@pytest.mark.parametrize("shapes", BROADCASTS, ids=lambda s: "%sx%s" % s)
+def test_binary_broadcast(hk, cuda, dtype, op, shapes):
+    import torch
+    sa, sb = shapes
+    a = _draw(31, sa, dtype, positive=True)
+    b = _draw(32, sb, dtype, positive=True)
+    want = NP_BINARY[op](a.astype(np.float64), b.astype(np.float64))
+    ta, tb = helpers.to_torch(a, dtype, cuda), helpers.to_torch(b, dtype, cuda)
+    out = torch.empty(want.shape, dtype=ta.dtype, device=cuda)
+    hk.binary(op, ta, tb, out)
+    torch.cuda.synchronize()
+    helpers.assert_close(out, want, dtype, op)
+    # operands swapped (the broadcast one on the left)
+    hk.binary(op, tb, ta, out)
+    torch.cuda.synchronize()
+    helpers.assert_close(out, NP_BINARY[op](b.astype(np.float64), a.astype(np.float64)), dtype, op + " swapped")
+
+
+def test_binary_strided_operands_and_in_place(hk, cuda):
+    import torch
+    a = torch.randn(48, 512, device=cuda)
+    b = torch.randn(512, 48, device=cuda)
+    out = torch.empty(48, 512, device=cuda)
+    hk.binary("add", a, b.t(), out)                       # transposed view: generic kernel
+    torch.cuda.synchronize()
+    assert torch.allclose(out, a + b.t(), rtol=1e-6, atol=1e-6)
+    half = torch.empty(48, 256, device=cuda)
+    hk.binary("mul", a[:, ::2], a[:, 1::2], half)         # column-strided views
+    torch.cuda.synchronize()
+    assert torch.allclose(half, a[:, ::2] * a[:, 1::2], rtol=1e-6, atol=1e-6)
+    s = torch.rand(48, 1, device=cuda) + 0.5
+    want = a / s
+    hk.binary("div", a, s, a)                             # in place, as the loss op divides exp by its row sum
+    torch.cuda.synchronize()
+    assert torch.allclose(a, want, rtol=1e-6, atol=0)
+    e = torch.empty(0, 16, device=cuda)
+    hk.binary("add", e, e, e)                             # empty: nothing to do
+    with pytest.raises(hk.HkError) as err:
+        hk.binary("add", a.long(), a.long(), a.long())
+    assert err.value.code == -2
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cols", [1000, 4096, 50257])
+def test_vocab_parallel_local_kernels(hk, cuda, dtype, cols):
+    import torch
+    rows, ignored = 77, -100
+    start = 3 * cols
+    g = helpers.rng(5 + cols)
+    logits = _draw(41 + cols, (rows, cols), dtype)
+    labels = g.integers(0, 8 * cols, rows).astype(np.int64)          # most labels lie in other shards
+    labels[::5] = g.integers(start, start + cols, len(labels[::5]))  # every fifth in this one
+    labels[3] = ignored; labels[10] = start; labels[11] = start + cols - 1; labels[12] = start + cols
+    labels[13] = start - 1
+    tl = helpers.to_torch(logits, dtype, cuda); tlab = torch.from_numpy(labels).to(cuda)
+    picked = torch.full((rows,), 7.0, dtype=tl.dtype, device=cuda)
+    lse = torch.full((rows,), 5.0, dtype=tl.dtype, device=cuda)
+    hk.vocab_parallel_ce_gather(tl, tlab, start, start + cols, ignored, picked, lse)
+    torch.cuda.synchronize()
+    inside = (labels >= start) & (labels < start + cols) & (labels != ignored)
+    want = np.where(inside, logits[np.arange(rows), np.clip(labels - start, 0, cols - 1)], 0.0)
+    assert np.array_equal(helpers.to_numpy(picked).astype(np.float64), want.astype(np.float64))   # a gather: exact
+    want_lse = np.where(labels == ignored, 0.0, 5.0)
+    assert np.array_equal(helpers.to_numpy(lse).astype(np.float64), want_lse)
+
+    sm = np.abs(_draw(43 + cols, (rows, cols), dtype)) / cols
+    gl = _draw(44, (rows,), dtype)
+    onehot = np.zeros((rows, cols)); onehot[np.flatnonzero(inside), (labels - start)[inside]] = 1.0
+    want_grad = (sm.astype(np.float64) - onehot) * gl.astype(np.float64)[:, None]
+    tsm, tgl = helpers.to_torch(sm, dtype, cuda), helpers.to_torch(gl, dtype, cuda)
+    out = torch.empty_like(tsm)
+    hk.vocab_parallel_ce_bwd(tsm, tlab, tgl, out, start)
+    torch.cuda.synchronize()
+    helpers.assert_close(out, want_grad, dtype, "gradient")
+    hk.vocab_parallel_ce_bwd(tsm, tlab, tgl, tsm, start)   # in place
+    torch.cuda.synchronize()
+    assert torch.equal(tsm, out)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_vocab_parallel_loss_over_two_shards_equals_the_fused_loss(hk, cuda, dtype):
+    """The loss op's sequence (VocabParallelCrossEntropyLoss.cc:51-108) on two column shards held by this one
+    GPU, the three cross-device reductions replaced by max / sum over the two partial results: row maximum,
+    logits - maximum, exp, row sum, divide (softmax kept), log, gather, subtract.  Its per-row loss and its
+    gradient must equal the fused sparse cross-entropy of the whole matrix."""
+    import torch
+    rows, cols, ignored = 96, 4096, -100
+    half = cols // 2
+    g = helpers.rng(77)
+    logits = _draw(51, (rows, cols), dtype) * 3
+    labels = g.integers(0, cols, rows).astype(np.int64); labels[::9] = ignored
+    full = helpers.to_torch(logits, dtype, cuda); tlab = torch.from_numpy(labels).to(cuda)
+    loss_ref = oracle.sce_sparse_fwd(logits, labels, ignored)
+    gl = np.where(labels == ignored, 0.0, 1.0 / rows)
+    grad_ref = oracle.sce_sparse_bwd(logits, labels, gl.astype(np.float32), ignored)
+
+    shards = [full[:, :half].contiguous(), full[:, half:].contiguous()]
+    tdt = full.dtype
+    col = lambda: torch.empty(rows, 1, dtype=tdt, device=cuda)
+    part_max = []
+    for x in shards:
+        m = col()
+        hk.reduce(x, m.view(rows), [1], "max")
+        part_max.append(m)
+    row_max = torch.maximum(part_max[0], part_max[1])                 # all-reduce(max)
+    exps, part_sum = [], []
+    for x in shards:
+        v = torch.empty_like(x)
+        hk.binary("sub", x, row_max, v)
+        hk.unary("exp", v, v)
+        s = col()
+        hk.reduce(v, s.view(rows), [1], "sum")
+        exps.append(v); part_sum.append(s)
+    row_sum = part_sum[0] + part_sum[1]                               # all-reduce(sum)
+    lse = col()
+    hk.unary("log", row_sum, lse)
+    picked_total = torch.zeros(rows, 1, dtype=torch.float32, device=cuda)
+    grads = []
+    tgl = helpers.to_torch(gl, dtype, cuda).view(rows, 1)
+    for k, x in enumerate(shards):
+        shifted = torch.empty_like(x)
+        hk.binary("sub", x, row_max, shifted)
+        picked = col()
+        lse_k = lse.clone()
+        hk.vocab_parallel_ce_gather(shifted, tlab, k * half, (k + 1) * half, ignored, picked.view(rows),
+                                    lse_k.view(rows))
+        picked_total += picked.float()                                # all-reduce(sum)
+        hk.binary("div", exps[k], row_sum, exps[k])                   # softmax, in place
+        out = torch.empty_like(x)
+        hk.vocab_parallel_ce_bwd(exps[k], tlab, tgl.view(rows), out, k * half)
+        grads.append(out)
+        lse_final = lse_k
+    loss = torch.empty(rows, 1, dtype=tdt, device=cuda)
+    hk.binary("sub", lse_final, picked_total.to(tdt), loss)
+    torch.cuda.synchronize()
+    # In bf16 the unfused sequence rounds logits - maximum (up to ~25 in magnitude here) to 8 bits before the
+    # exponential: an absolute error of up to 0.06 in the exponent, i.e. several percent in softmax.  That is the
+    # arithmetic of the sequence itself (every step below is within 1e-2 of its own definition, tested above).
+    helpers.assert_close(loss.view(rows), loss_ref, dtype, "loss", rtol=2e-2 if dtype == "bf16" else 1e-5)
+    helpers.assert_close(torch.cat(grads, dim=1), grad_ref, dtype, "gradient",
+                         rtol=1e-1 if dtype == "bf16" else 1e-5)

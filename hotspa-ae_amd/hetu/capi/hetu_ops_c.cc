@@ -280,6 +280,102 @@ int ht_reduce(const HtArray* in, HtArray* out, const int64_t* axes, int naxes, i
   });
 }
 
+int ht_binary(int op, const HtArray* a, const HtArray* b, HtArray* out, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(out);
+    const Stream st = stream_of(a, stream_index);
+    switch (op) {
+      case 0: hetu::impl::AddElewiseCuda(wrap(a), wrap(b), o, st); break;
+      case 1: hetu::impl::SubElewiseCuda(wrap(a), wrap(b), o, st); break;
+      case 2: hetu::impl::MulElewiseCuda(wrap(a), wrap(b), o, st); break;
+      case 3: hetu::impl::DivElewiseCuda(wrap(a), wrap(b), o, st); break;
+      default: HT_VALUE_ERROR << "unknown binary op " << op;
+    }
+  });
+}
+
+int ht_binary_const(int op, const HtArray* in, double value, HtArray* out, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(out);
+    const Stream st = stream_of(in, stream_index);
+    switch (op) {
+      case 0: hetu::impl::AddConstCuda(wrap(in), value, o, st); break;
+      case 1: hetu::impl::SubConstCuda(wrap(in), value, o, st); break;
+      case 2: hetu::impl::MulConstCuda(wrap(in), value, o, st); break;
+      case 3: hetu::impl::DivConstCuda(wrap(in), value, o, st); break;
+      default: HT_VALUE_ERROR << "unknown binary op " << op;
+    }
+  });
+}
+
+int ht_unary(int op, const HtArray* in, HtArray* out, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(out);
+    const Stream st = stream_of(in, stream_index);
+    switch (op) {
+      case 0: hetu::impl::ExpCuda(wrap(in), o, st); break;
+      case 1: hetu::impl::LogCuda(wrap(in), o, st); break;
+      case 2: hetu::impl::OppositeCuda(wrap(in), o, st); break;
+      case 3: hetu::impl::SqrtCuda(wrap(in), o, st); break;
+      default: HT_VALUE_ERROR << "unknown unary op " << op;
+    }
+  });
+}
+
+int ht_ndarray_binary(int op, const HtArray* a, const HtArray* b, HtArray* out, int in_place, int stream_index) {
+  return guarded([&] {
+    NDArray x = wrap(a), y = wrap(b), r, none;
+    NDArray& dst = in_place ? x : none;
+    switch (op) {
+      case 0: r = NDArray::add(x, y, stream_index, dst); break;
+      case 1: r = NDArray::sub(x, y, stream_index, dst); break;
+      case 2: r = NDArray::mul(x, y, stream_index, dst); break;
+      case 3: r = NDArray::div(x, y, stream_index, dst); break;
+      default: HT_VALUE_ERROR << "unknown binary op " << op;
+    }
+    if (!in_place) copy_out(r, out, stream_of(a, stream_index));
+  });
+}
+
+int ht_ndarray_unary(int op, const HtArray* in, HtArray* out, int in_place, int stream_index) {
+  return guarded([&] {
+    NDArray x = wrap(in), r, none;
+    NDArray& dst = in_place ? x : none;
+    switch (op) {
+      case 0: r = NDArray::exp(x, stream_index, dst); break;
+      case 1: r = NDArray::log(x, stream_index, dst); break;
+      case 2: r = NDArray::neg(x, stream_index, dst); break;
+      case 3: r = NDArray::sqrt(x, stream_index, dst); break;
+      default: HT_VALUE_ERROR << "unknown unary op " << op;
+    }
+    if (!in_place) copy_out(r, out, stream_of(in, stream_index));
+  });
+}
+
+int ht_vocab_parallel_cross_entropy(const HtArray* vocab_parallel_logits, const HtArray* labels,
+                                    int64_t vocab_start_index, int64_t vocab_end_index, int64_t ignored_index,
+                                    HtArray* predicted_logits_partial, HtArray* log_sum_exp_logits,
+                                    int stream_index) {
+  return guarded([&] {
+    NDArray p = wrap(predicted_logits_partial), l = wrap(log_sum_exp_logits);
+    hetu::impl::VocabParallelCrossEntropyCuda(wrap(vocab_parallel_logits), wrap(labels), vocab_start_index,
+                                              vocab_end_index, ignored_index, p, l,
+                                              stream_of(vocab_parallel_logits, stream_index));
+  });
+}
+
+int ht_vocab_parallel_cross_entropy_gradient(const HtArray* softmax, const HtArray* labels,
+                                             int64_t vocab_start_index, int64_t vocab_end_index,
+                                             int64_t ignored_index, const HtArray* grad_loss, HtArray* output,
+                                             int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(output);
+    hetu::impl::VocabParallelCrossEntropyGradientCuda(wrap(softmax), wrap(labels), vocab_start_index,
+                                                      vocab_end_index, ignored_index, wrap(grad_loss), o,
+                                                      stream_of(softmax, stream_index));
+  });
+}
+
 int ht_ndarray_reduce(const HtArray* in, int red_type, const int64_t* axes, int naxes, int keepdims, HtArray* out,
                       int stream_index) {
   return guarded([&] {

@@ -233,6 +233,66 @@ NDArrayList NDArray::fused_layernorm(const NDArray& input, const NDArray& bn_sca
   return {out, savemean, savevar};
 }
 
+// ---- element-wise arithmetic ------------------------------------------------
+#define HT_NDARRAY_BINARY(fn, Kernel)                                                                       \
+  NDArray NDArray::fn(const NDArray& x, const NDArray& y, StreamIndex stream_id, NDArray& output) {         \
+    auto output_shape = NDArrayMeta::Broadcast(x->shape(), y->shape());                                     \
+    HT_ASSERT(!output_shape.empty())                                                                        \
+      << "Shapes cannot be broadcast together: " << x->shape() << " vs. " << y->shape();                    \
+    NDArray out = output.is_defined() ? output : NDArray::empty(output_shape, x->device(), x->dtype(),      \
+                                                                stream_id);                                 \
+    Stream stream(x->device(), stream_id);                                                                  \
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(x->device().type(), __FUNCTION__, hetu::impl::Kernel, x, y, out,        \
+                                    stream);                                                                \
+    return out;                                                                                             \
+  }
+HT_NDARRAY_BINARY(add, AddElewise)
+HT_NDARRAY_BINARY(sub, SubElewise)
+HT_NDARRAY_BINARY(mul, MulElewise)
+HT_NDARRAY_BINARY(div, DivElewise)
+#undef HT_NDARRAY_BINARY
+
+#define HT_NDARRAY_CONST(fn, Kernel)                                                                        \
+  NDArray out = output.is_defined() ? output : NDArray::empty_like(input, stream_id);                       \
+  Stream stream(input->device(), stream_id);                                                                \
+  HT_DISPATCH_KERNEL_CPU_AND_CUDA(input->device().type(), __FUNCTION__, hetu::impl::Kernel, input, scalar,  \
+                                  out, stream);                                                             \
+  return out
+
+NDArray NDArray::add(const NDArray& input, double scalar, StreamIndex stream_id, NDArray& output) {
+  HT_NDARRAY_CONST(add, AddConst);
+}
+NDArray NDArray::sub(const NDArray& input, double scalar, StreamIndex stream_id, NDArray& output) {
+  return NDArray::add(input, -scalar, stream_id, output);
+}
+NDArray NDArray::sub(double scalar, const NDArray& input, StreamIndex stream_id, NDArray& output) {
+  HT_NDARRAY_CONST(sub, SubConst);
+}
+NDArray NDArray::mul(const NDArray& input, double scalar, StreamIndex stream_id, NDArray& output) {
+  HT_NDARRAY_CONST(mul, MulConst);
+}
+NDArray NDArray::div(const NDArray& input, double scalar, StreamIndex stream_id, NDArray& output) {
+  return NDArray::mul(input, 1.0 / scalar, stream_id, output);
+}
+NDArray NDArray::div(double scalar, const NDArray& input, StreamIndex stream_id, NDArray& output) {
+  HT_NDARRAY_CONST(div, DivConst);
+}
+#undef HT_NDARRAY_CONST
+
+#define HT_NDARRAY_UNARY(fn, Kernel)                                                                        \
+  NDArray NDArray::fn(const NDArray& input, StreamIndex stream_id, NDArray& output) {                       \
+    NDArray out = output.is_defined() ? output : NDArray::empty_like(input, stream_id);                     \
+    Stream stream(input->device(), stream_id);                                                              \
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(input->device().type(), __FUNCTION__, hetu::impl::Kernel, input, out,   \
+                                    stream);                                                                \
+    return out;                                                                                             \
+  }
+HT_NDARRAY_UNARY(neg, Opposite)
+HT_NDARRAY_UNARY(sqrt, Sqrt)
+HT_NDARRAY_UNARY(exp, Exp)
+HT_NDARRAY_UNARY(log, Log)
+#undef HT_NDARRAY_UNARY
+
 NDArray NDArray::softmax(const NDArray& input, int64_t dim, StreamIndex stream_id, NDArray& output) {
   NDArray out = output.is_defined() ? output : NDArray::empty_like(input, stream_id);
   Stream stream(input->device(), stream_id);

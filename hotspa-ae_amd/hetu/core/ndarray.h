@@ -153,6 +153,33 @@ class NDArray {
                                      const HTShape& normalized_shape, double eps = 0.01,
                                      StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY,
                                      NDArray& save_mean = EMPTY, NDArray& save_var = EMPTY);
+  // element-wise arithmetic with broadcasting (hetu/core/ndarray.cc:186-303, 388-404 of the reference);
+  // `output` may be one of the operands of the result's shape (in place)
+  static NDArray add(const NDArray& x, const NDArray& y, StreamIndex stream_id = DEFAULT_STREAM,
+                     NDArray& output = EMPTY);
+  static NDArray add(const NDArray& input, double scalar, StreamIndex stream_id = DEFAULT_STREAM,
+                     NDArray& output = EMPTY);
+  static NDArray sub(const NDArray& x, const NDArray& y, StreamIndex stream_id = DEFAULT_STREAM,
+                     NDArray& output = EMPTY);
+  static NDArray sub(const NDArray& input, double scalar, StreamIndex stream_id = DEFAULT_STREAM,
+                     NDArray& output = EMPTY);
+  static NDArray sub(double scalar, const NDArray& input, StreamIndex stream_id = DEFAULT_STREAM,
+                     NDArray& output = EMPTY);
+  static NDArray neg(const NDArray& input, StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY);
+  static NDArray mul(const NDArray& x, const NDArray& y, StreamIndex stream_id = DEFAULT_STREAM,
+                     NDArray& output = EMPTY);
+  static NDArray mul(const NDArray& input, double scalar, StreamIndex stream_id = DEFAULT_STREAM,
+                     NDArray& output = EMPTY);
+  static NDArray div(const NDArray& x, const NDArray& y, StreamIndex stream_id = DEFAULT_STREAM,
+                     NDArray& output = EMPTY);
+  static NDArray div(const NDArray& input, double scalar, StreamIndex stream_id = DEFAULT_STREAM,
+                     NDArray& output = EMPTY);
+  static NDArray div(double scalar, const NDArray& input, StreamIndex stream_id = DEFAULT_STREAM,
+                     NDArray& output = EMPTY);
+  static NDArray sqrt(const NDArray& input, StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY);
+  static NDArray exp(const NDArray& input, StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY);
+  static NDArray log(const NDArray& input, StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY);
+
   static NDArray softmax(const NDArray& input, int64_t dim, StreamIndex stream_id = DEFAULT_STREAM,
                          NDArray& output = EMPTY);
   static NDArray sceloss(const NDArray& preds, const NDArray& labels, ReductionType reduction = kMEAN,

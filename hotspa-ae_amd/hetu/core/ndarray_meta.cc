@@ -43,6 +43,19 @@ HTShape NDArrayMeta::Reduce(const HTShape& shape, const HTAxes& axes, bool keepd
   return out;
 }
 
+HTShape NDArrayMeta::Broadcast(const HTShape& shape_a, const HTShape& shape_b) {
+  const size_t na = shape_a.size(), nb = shape_b.size(), n = std::max(na, nb);
+  HTShape out(n);
+  for (size_t k = 0; k < n; ++k) {           // k counts from the last dimension
+    const int64_t a = k < na ? shape_a[na - 1 - k] : 1;
+    const int64_t b = k < nb ? shape_b[nb - 1 - k] : 1;
+    if (a != b && a != 1 && b != 1) return HTShape();
+    out[n - 1 - k] = std::max(a, b);
+    if ((a == 0 || b == 0)) out[n - 1 - k] = 0;   // an empty extent stays empty
+  }
+  return out;
+}
+
 std::ostream& operator<<(std::ostream& os, const NDArrayMeta& meta) {
   return os << "{dtype=" << meta.dtype << ", device=" << meta.device << ", shape=" << meta.shape
             << ", stride=" << meta.stride << "}";

@@ -76,6 +76,9 @@ class NDArrayMeta {
   static int64_t ParseAxis(int64_t axis, int64_t num_dim);
   static HTAxes ParseAxes(const HTAxes axes, int64_t num_dim);
   static HTShape Reduce(const HTShape& shape, const HTAxes& axes, bool keepdims);
+  // shape two operands broadcast to (trailing dimensions aligned, extent 1 repeats); empty when they cannot
+  // (hetu/core/ndarray_meta.cc:99-117 of the reference)
+  static HTShape Broadcast(const HTShape& shape_a, const HTShape& shape_b);
 
   DataType dtype{kUndeterminedDataType};
   Device device;

@@ -71,6 +71,26 @@ DECLARE_KERNEL_CPU_AND_CUDA(ReduceSum, const NDArray&, NDArray&, const int64_t*,
 DECLARE_KERNEL_CPU_AND_CUDA(ReduceMax, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(ReduceMin, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(ReduceProd, const NDArray&, NDArray&, const int64_t*, int64_t, const Stream&);
+// element-wise family (kernel_links.h:29-32, 117-120, 158, 214, 235-238, 250, 309-313 of the reference)
+DECLARE_KERNEL_CPU_AND_CUDA(AddConst, const NDArray&, double, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(SubConst, const NDArray&, double, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(MulConst, const NDArray&, double, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(DivConst, const NDArray&, double, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(AddElewise, const NDArray&, const NDArray&, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(SubElewise, const NDArray&, const NDArray&, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(MulElewise, const NDArray&, const NDArray&, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(DivElewise, const NDArray&, const NDArray&, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(Exp, const NDArray&, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(Log, const NDArray&, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(Opposite, const NDArray&, NDArray&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(Sqrt, const NDArray&, NDArray&, const Stream&);
+// vocab_parallel_logits, labels, vocab_start_index, vocab_end_index, ignored_index, predicted_logits_partial,
+// log_sum_exp_logits
+DECLARE_KERNEL_CUDA(VocabParallelCrossEntropy, const NDArray&, const NDArray&, const int64_t, const int64_t,
+                    const int64_t, NDArray&, NDArray&, const Stream&);
+// softmax, labels, vocab_start_index, vocab_end_index, ignored_index, grad_loss, output
+DECLARE_KERNEL_CUDA(VocabParallelCrossEntropyGradient, const NDArray&, const NDArray&, const int64_t, const int64_t,
+                    const int64_t, const NDArray&, NDArray&, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(Softmax, const NDArray&, NDArray&, int64_t, const Stream&);
 // y, dy, dx, dim
 DECLARE_KERNEL_CPU_AND_CUDA(SoftmaxGradient, const NDArray&, const NDArray&, NDArray&, int64_t, const Stream&);

@@ -184,6 +184,46 @@ def dropout_add_ln_parallel_residual_bwd(dz0, dz1, dx, x, dmask0, dmask1, mu, rs
           ctypes.c_int(int(has_residual)), ctypes.c_int(int(is_rms_norm)), ctypes.c_int(stream))
 
 
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+UNARY_OPS = {"exp": 0, "log": 1, "neg": 2, "sqrt": 3}
+
+
+def binary(op, a, b, out, stream=DEFAULT_STREAM):
+    _call("ht_binary", ctypes.c_int(BINARY_OPS[op]), desc(a), desc(b), desc(out), ctypes.c_int(stream))
+
+
+def binary_const(op, x, value, out, stream=DEFAULT_STREAM):
+    """AddConst / SubConst (value - x) / MulConst / DivConst (value / x)."""
+    _call("ht_binary_const", ctypes.c_int(BINARY_OPS[op]), desc(x), ctypes.c_double(value), desc(out),
+          ctypes.c_int(stream))
+
+
+def unary(op, x, out, stream=DEFAULT_STREAM):
+    _call("ht_unary", ctypes.c_int(UNARY_OPS[op]), desc(x), desc(out), ctypes.c_int(stream))
+
+
+def ndarray_binary(op, a, b, out=None, in_place=False, stream=DEFAULT_STREAM):
+    _call("ht_ndarray_binary", ctypes.c_int(BINARY_OPS[op]), desc(a), desc(b), desc(out),
+          ctypes.c_int(int(in_place)), ctypes.c_int(stream))
+
+
+def ndarray_unary(op, x, out=None, in_place=False, stream=DEFAULT_STREAM):
+    _call("ht_ndarray_unary", ctypes.c_int(UNARY_OPS[op]), desc(x), desc(out), ctypes.c_int(int(in_place)),
+          ctypes.c_int(stream))
+
+
+def vocab_parallel_cross_entropy(logits, labels, vocab_start, vocab_end, ignored_index, picked, lse,
+                                 stream=DEFAULT_STREAM):
+    _call("ht_vocab_parallel_cross_entropy", desc(logits), desc(labels), _i64(vocab_start), _i64(vocab_end),
+          _i64(ignored_index), desc(picked), desc(lse), ctypes.c_int(stream))
+
+
+def vocab_parallel_cross_entropy_gradient(softmax, labels, vocab_start, vocab_end, ignored_index, grad_loss, out,
+                                          stream=DEFAULT_STREAM):
+    _call("ht_vocab_parallel_cross_entropy_gradient", desc(softmax), desc(labels), _i64(vocab_start),
+          _i64(vocab_end), _i64(ignored_index), desc(grad_loss), desc(out), ctypes.c_int(stream))
+
+
 def set_random_seed(seed):
     _call("ht_set_random_seed", ctypes.c_uint64(seed))
 

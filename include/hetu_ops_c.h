@@ -114,6 +114,29 @@ HT_API int ht_reduce(const HtArray* in, HtArray* out, const int64_t* axes, int n
 
 /* ---- NDArray statics: device dispatch + output allocation from the pool ----
  * `out` (and mean / var) describe caller memory the result is written to. */
+/* Element-wise family.  op: 0 add, 1 sub, 2 mul, 3 div (binary); 0 exp, 1 log, 2 negate, 3 sqrt (unary).
+ * ht_binary      -> AddElewiseCuda / SubElewiseCuda / MulElewiseCuda / DivElewiseCuda (BinaryElewise.cu)
+ * ht_binary_const -> AddConstCuda / SubConstCuda (value - x) / MulConstCuda / DivConstCuda (value / x) (BinaryConst.cu)
+ * ht_unary       -> ExpCuda / LogCuda / OppositeCuda / SqrtCuda
+ * ht_ndarray_binary / _unary: NDArray::add / sub / mul / div / exp / log / neg / sqrt, which allocate their result
+ * from the pool (copied into `out`); with in_place != 0 the first operand is passed as the output, as the
+ * reference's loss op does (VocabParallelCrossEntropyLoss.cc:77-81). */
+HT_API int ht_binary(int op, const HtArray* a, const HtArray* b, HtArray* out, int stream_index);
+HT_API int ht_binary_const(int op, const HtArray* in, double value, HtArray* out, int stream_index);
+HT_API int ht_unary(int op, const HtArray* in, HtArray* out, int stream_index);
+HT_API int ht_ndarray_binary(int op, const HtArray* a, const HtArray* b, HtArray* out, int in_place,
+                             int stream_index);
+HT_API int ht_ndarray_unary(int op, const HtArray* in, HtArray* out, int in_place, int stream_index);
+/* VocabParallelCrossEntropyCuda / VocabParallelCrossEntropyGradientCuda
+ * (hetu/impl/kernel/VocabParallelCrossEntropyLoss.cu:38-64, 94-119) */
+HT_API int ht_vocab_parallel_cross_entropy(const HtArray* vocab_parallel_logits, const HtArray* labels,
+                                           int64_t vocab_start_index, int64_t vocab_end_index,
+                                           int64_t ignored_index, HtArray* predicted_logits_partial,
+                                           HtArray* log_sum_exp_logits, int stream_index);
+HT_API int ht_vocab_parallel_cross_entropy_gradient(const HtArray* softmax, const HtArray* labels,
+                                                    int64_t vocab_start_index, int64_t vocab_end_index,
+                                                    int64_t ignored_index, const HtArray* grad_loss,
+                                                    HtArray* output, int stream_index);
 HT_API int ht_ndarray_reduce(const HtArray* in, int red_type, const int64_t* axes, int naxes, int keepdims,
                              HtArray* out, int stream_index);
 HT_API int ht_ndarray_softmax(const HtArray* in, int64_t dim, HtArray* out, int stream_index);

@@ -163,6 +163,69 @@ int main() {
     for (int64_t r = 0; r < rows; r += 5) CHECK(pr[r] == 0.f);
   });
 
+  run("vocabulary-parallel cross-entropy over two column shards, written as the loss op writes it", [&] {
+    // the steps of VocabParallelCrossEntropyOpImpl::DoCompute (VocabParallelCrossEntropyLoss.cc:51-108 of the
+    // reference); what it all-reduces across devices is combined here from the two shards this device holds
+    NDArray d = NDArray::cuda(host_f32({rows, cols}, x));
+    NDArray lab = NDArray::empty({rows}, Device(kCPU), kInt64);
+    std::vector<double> want(rows, 0.0);
+    for (int64_t r = 0; r < rows; ++r) {
+      const int64_t l = (r % 7 == 0) ? -100 : (r * 131) % cols;
+      lab->data_ptr<int64_t>()[r] = l;
+      if (l < 0) continue;
+      double m = -1e300, sum = 0;
+      for (int64_t c = 0; c < cols; ++c) m = std::max<double>(m, x[r * cols + c]);
+      for (int64_t c = 0; c < cols; ++c) sum += std::exp(x[r * cols + c] - m);
+      want[r] = std::log(sum) + m - x[r * cols + l];
+    }
+    NDArray labels = NDArray::cuda(lab);
+    const int64_t half = cols / 2;
+    NDArray shard[2] = {NDArray::slice(d, {0, 0}, {rows, half}), NDArray::slice(d, {0, half}, {rows, half})};
+    NDArray part_max[2], shifted[2], exps[2], part_sum[2], picked[2];
+    for (int k = 0; k < 2; ++k) part_max[k] = NDArray::reduce(shard[k], kMAX, {-1}, true);
+    std::vector<float> m0 = fetch_f32(part_max[0]), m1 = fetch_f32(part_max[1]), mm(rows);
+    for (int64_t r = 0; r < rows; ++r) mm[r] = std::max(m0[r], m1[r]);
+    NDArray row_max = NDArray::cuda(host_f32({rows, 1}, mm));             // all-reduce(max)
+    for (int k = 0; k < 2; ++k) {
+      shifted[k] = NDArray::sub(shard[k], row_max);                       // logits - max, [rows, half] - [rows, 1]
+      exps[k] = NDArray::exp(shifted[k]);
+      part_sum[k] = NDArray::reduce(exps[k], kSUM, {-1}, true);
+    }
+    NDArray row_sum = NDArray::add(part_sum[0], part_sum[1]);             // all-reduce(sum)
+    NDArray softmax0 = NDArray::div(exps[0], row_sum, NDArray::DEFAULT_STREAM, exps[0]);   // in place
+    CHECK(softmax0->raw_data_ptr() == exps[0]->raw_data_ptr());
+    NDArray lse = NDArray::log(row_sum);
+    Stream stream(gpu, NDArray::DEFAULT_STREAM);
+    for (int k = 0; k < 2; ++k) {
+      picked[k] = NDArray::empty({rows, 1}, gpu, kFloat32);
+      hetu::impl::VocabParallelCrossEntropyCuda(shifted[k], labels, k * half, (k + 1) * half, -100, picked[k], lse,
+                                                stream);
+    }
+    NDArray picked_all = NDArray::add(picked[0], picked[1]);              // all-reduce(sum)
+    NDArray loss = NDArray::sub(lse, picked_all, NDArray::DEFAULT_STREAM, lse);              // in place
+    CHECK((loss->shape() == HTShape{rows, 1}));
+    CHECK(max_rel(fetch_f32(loss), want) < 1e-5);
+    // softmax of shard 0 sums, with shard 1's, to one in every row
+    std::vector<float> s0 = fetch_f32(NDArray::reduce(softmax0, kSUM, {-1}, false));
+    std::vector<float> s1 = fetch_f32(NDArray::reduce(NDArray::div(exps[1], row_sum), kSUM, {-1}, false));
+    for (int64_t r = 0; r < rows; ++r) CHECK(std::fabs(s0[r] + s1[r] - 1.0) < 1e-5);
+    // gradient of shard 0: (softmax - onehot) * grad, ignored rows through a zero loss gradient
+    std::vector<float> gl(rows);
+    for (int64_t r = 0; r < rows; ++r) gl[r] = (r % 7 == 0) ? 0.f : 1.f / rows;
+    NDArray grad = NDArray::empty({rows, half}, gpu, kFloat32);
+    std::vector<float> sm = fetch_f32(softmax0);
+    hetu::impl::VocabParallelCrossEntropyGradientCuda(softmax0, labels, 0, half, -100,
+                                                      NDArray::cuda(host_f32({rows, 1}, gl)), grad, stream);
+    std::vector<float> got = fetch_f32(grad);
+    std::vector<double> wantg(rows * half);
+    for (int64_t r = 0; r < rows; ++r) {
+      const int64_t l = lab->data_ptr<int64_t>()[r];
+      for (int64_t c = 0; c < half; ++c) wantg[r * half + c] = (double(sm[r * half + c]) - (c == l ? 1.0 : 0.0)) * gl[r];
+    }
+    CHECK(max_rel(got, wantg) < 1e-5);
+    CHECK(throws<assertion_error>([&] { NDArray::add(shard[0], NDArray::slice(d, {0, 0}, {rows, half - 1})); }));
+  });
+
   run("reductions: sum / mean / max with keepdims, all dims", [&] {
     NDArray d = NDArray::cuda(host_f32({rows, cols}, x));
     NDArray s0 = NDArray::sum(d, {0});

@@ -714,3 +714,98 @@ def test_instance_norm_and_gradient(ops, cuda, dtype, shape):
     assert ops.pool_stats()["alloc_cnt"] == before          # no column sums, so no scratch
     with pytest.raises(ops.AssertionError_, match="N, C, H, W"):
         ops.instance_norm(tx.reshape(n * c, h, w), tmean, tvar, ty.reshape(n * c, h, w), eps)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+def test_elementwise_entry_points(ops, cuda, dtype):
+    """AddElewiseCuda ... DivElewiseCuda with a per-row operand, the ...ConstCuda entries (constant on the left),
+    ExpCuda / LogCuda / OppositeCuda / SqrtCuda."""
+    import torch
+    rows, cols = 50, 768
+    a = oracle.round_to(np.abs(helpers.draw(1, (rows, cols))) + np.float32(0.5), dtype)
+    b = oracle.round_to(np.abs(helpers.draw(2, (rows, 1))) + np.float32(0.5), dtype)
+    ta, tb = _dev((a, b), dtype, cuda)
+    out = torch.empty_like(ta)
+    npf = {"add": np.add, "sub": np.subtract, "mul": np.multiply, "div": np.divide}
+    ad, bd = a.astype(np.float64), b.astype(np.float64)
+    _sync_in()
+    for op, f in npf.items():
+        ops.binary(op, ta, tb, out)
+        ops.stream_sync()
+        helpers.assert_close(out, f(ad, bd), dtype, op)
+        ops.binary(op, tb, ta, out)                       # the broadcast operand on the left
+        ops.stream_sync()
+        helpers.assert_close(out, f(bd, ad), dtype, op + " swapped")
+    c = 1.5
+    for op, f in npf.items():                             # the constant is the left operand
+        ops.binary_const(op, ta, c, out)
+        ops.stream_sync()
+        helpers.assert_close(out, f(c, ad), dtype, op + " const")
+    for op, f in {"exp": np.exp, "log": np.log, "neg": np.negative, "sqrt": np.sqrt}.items():
+        ops.unary(op, ta, out)
+        ops.stream_sync()
+        helpers.assert_close(out, f(ad), dtype, op)
+    with pytest.raises(ops.AssertionError_, match="Divided by 0"):
+        ops.binary_const("div", ta, 0.0, out)
+    with pytest.raises(ops.AssertionError_, match="broadcast"):
+        ops.binary("add", ta, ta[:, :cols - 1], out)
+    with pytest.raises(ops.NotImplemented_):
+        ops.unary("exp", ta.long(), out.long())
+
+
+def test_ndarray_elementwise_statics(ops, cuda):
+    """NDArray::add / sub / mul / div / exp / log / neg / sqrt: results from the pool, and in place."""
+    import torch
+    a = torch.rand(33, 1000, device=cuda) + 0.5
+    b = torch.rand(33, 1, device=cuda) + 0.5
+    out = torch.empty_like(a)
+    _sync_in()
+    for op, f in {"add": torch.add, "sub": torch.sub, "mul": torch.mul, "div": torch.div}.items():
+        ops.ndarray_binary(op, a, b, out)
+        assert torch.allclose(out, f(a, b), rtol=1e-6, atol=0)
+    for op, f in {"exp": torch.exp, "log": torch.log, "neg": torch.neg, "sqrt": torch.sqrt}.items():
+        ops.ndarray_unary(op, a, out)
+        assert torch.allclose(out, f(a), rtol=1e-6, atol=1e-7)
+    want = a / b
+    ops.ndarray_binary("div", a, b, in_place=True)
+    ops.stream_sync()
+    assert torch.allclose(a, want, rtol=1e-6, atol=0)
+    want = torch.log(a)
+    ops.ndarray_unary("log", a, in_place=True)
+    ops.stream_sync()
+    assert torch.allclose(a, want, rtol=1e-6, atol=1e-7)
+    t3 = torch.rand(4, 5, 6, device=cuda)
+    out3 = torch.empty(4, 5, 6, device=cuda)
+    ops.ndarray_binary("mul", t3, torch.rand(5, 1, device=cuda).add_(1.0), out3)
+    with pytest.raises(ops.AssertionError_, match="cannot be broadcast"):
+        ops.ndarray_binary("add", t3, torch.rand(4, 5, device=cuda), out3)
+
+
+def test_vocab_parallel_cross_entropy_entry_points(ops, cuda):
+    import torch
+    rows, cols, start, ignored = 64, 2048, 4096, -100
+    g = helpers.rng(3)
+    logits = helpers.draw(4, (rows, cols), dtype="bf16")
+    labels = g.integers(start - cols, start + 2 * cols, rows).astype(np.int64); labels[5] = ignored
+    tl = helpers.to_torch(logits, "bf16", cuda); tlab = torch.from_numpy(labels).to(cuda)
+    picked = torch.full((rows, 1), 9.0, dtype=torch.bfloat16, device=cuda)
+    lse = torch.full((rows, 1), 3.0, dtype=torch.bfloat16, device=cuda)
+    _sync_in()
+    ops.vocab_parallel_cross_entropy(tl, tlab, start, start + cols, ignored, picked, lse)
+    ops.stream_sync()
+    inside = (labels >= start) & (labels < start + cols)
+    want = np.where(inside, logits[np.arange(rows), np.clip(labels - start, 0, cols - 1)], 0.0)
+    assert np.array_equal(helpers.to_numpy(picked).reshape(rows), want)
+    assert np.array_equal(helpers.to_numpy(lse).reshape(rows), np.where(labels == ignored, 0.0, 3.0))
+    sm = torch.softmax(tl.float(), dim=1).bfloat16()
+    gl = torch.rand(rows, 1, device=cuda).bfloat16()
+    out = torch.empty_like(sm)
+    _sync_in()
+    ops.vocab_parallel_cross_entropy_gradient(sm, tlab, start, start + cols, ignored, gl, out)
+    ops.stream_sync()
+    onehot = np.zeros((rows, cols)); onehot[np.flatnonzero(inside), (labels - start)[inside]] = 1.0
+    helpers.assert_close(out, (helpers.to_numpy(sm).astype(np.float64) - onehot) * helpers.to_numpy(gl), "bf16", "grad")
+    with pytest.raises(ops.AssertionError_, match="does not match"):
+        ops.vocab_parallel_cross_entropy(tl, tlab, start, start + cols - 1, ignored, picked, lse)
+    with pytest.raises(ops.AssertionError_, match="int64"):
+        ops.vocab_parallel_cross_entropy(tl, tlab.int(), start, start + cols, ignored, picked, lse)

@@ -220,6 +220,27 @@ def case_dropout_ln(hk, torch, nsets, which):
     return bwd, n * (2 + 2 + 2 + 1 + 2 + 2) + rows * 4 + cols * 6, rows
 
 
+def case_elementwise(hk, torch, nsets, which):
+    """Steps of the vocabulary-parallel loss on one shard of [16384 x 32000] bf16 logits: logits - row maximum
+    (per-row operand), exp in place, softmax = exp / row sum in place, and the gradient kernel."""
+    rows, cols = 16384, 32000
+    bf = torch.bfloat16
+    n = rows * cols
+    xs = [_randn(torch, (rows, cols), bf, 2.0, 801 + i) for i in range(2)]
+    outs = [torch.empty((rows, cols), dtype=bf, device="cuda") for _ in range(2)]
+    per_row = _uniform(torch, (rows, 1), bf, 1.0, 2.0, 811)
+    if which == "sub":
+        return (lambda i: hk.binary("sub", xs[i % 2], per_row, outs[i % 2])), 2 * n * 2 + rows * 2, rows
+    if which == "exp":
+        return (lambda i: hk.unary("exp", xs[i % 2], outs[i % 2])), 2 * n * 2, rows
+    if which == "div":
+        return (lambda i: hk.binary("div", xs[i % 2], per_row, xs[i % 2])), 2 * n * 2 + rows * 2, rows
+    g = torch.Generator(device="cuda").manual_seed(812)
+    labels = torch.randint(0, 4 * cols, (rows,), generator=g, device="cuda", dtype=torch.int64)
+    gl = torch.full((rows,), 1.0 / rows, dtype=bf, device="cuda")
+    return (lambda i: hk.vocab_parallel_ce_bwd(xs[i % 2], labels, gl, outs[i % 2], cols)), 2 * n * 2 + rows * 10, rows
+
+
 def case_reduce(hk, torch, nsets, axes, op, three_d=False):
     rows, cols = 32768, 4096
     bf = torch.bfloat16
@@ -284,6 +305,10 @@ CASES = [
     ("next: instance norm fwd bf16 [256,256,32,32]", lambda hk, t, n: case_instance_norm(hk, t, n)),
     ("next: dropout(0.1)+residual+rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_dropout_ln(hk, t, 2, "fwd")),
     ("next: dropout(0.1)+residual+rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_dropout_ln(hk, t, 2, "bwd")),
+    ("next: logits - row max bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "sub")),
+    ("next: exp bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "exp")),
+    ("next: exp / row sum in place bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "div")),
+    ("next: vocab-parallel CE bwd bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "vce")),
     ("C4 rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "fwd")),
     ("C4 rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "bwd")),
     ("C5 sce fwd bf16 [16384x32000]", lambda hk, t, n: case_sce(hk, t, 2, "fwd")),

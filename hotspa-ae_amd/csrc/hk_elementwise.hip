@@ -95,37 +95,53 @@ __global__ __launch_bounds__(256) void ew_const_scalar_kernel(const T* in, doubl
 // How an operand maps onto the [rows, cols] output of the two-dimensional kernel.
 enum { EW_FULL = 0, EW_PER_ROW = 1, EW_PER_COL = 2, EW_SINGLE = 3 };
 
-template <typename T>
-__device__ __forceinline__ void ew_fetch(const T* p, int mode, int64_t v, int64_t r, int64_t c, float* f) {
-  constexpr int VEC = VecIO<T>::N;
-  if (mode == EW_FULL) {
-    VecIO<T>::unpack(ld16(p + v * VEC), f);
-  } else if (mode == EW_PER_COL) {
-    VecIO<T>::unpack(ld16_keep(p + c * VEC), f);
-  } else {
-    const float s = Cvt<T>::load(p + (mode == EW_PER_ROW ? r : 0));
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) f[j] = s;
+// An operand's 16 bytes (or its single value) as loaded, before any unpacking: both operands' loads are issued
+// back to back and waited for once.
+template <typename T, int MODE>
+struct EwRaw {
+  u32x4 vec;
+  float one;
+  __device__ __forceinline__ void load(const T* p, int64_t v, int64_t r, int64_t c) {
+    constexpr int VEC = VecIO<T>::N;
+    if constexpr (MODE == EW_FULL) vec = ld16(p + v * VEC);
+    else if constexpr (MODE == EW_PER_COL) vec = ld16_keep(p + c * VEC);
+    else if constexpr (MODE == EW_PER_ROW) one = Cvt<T>::load(p + r);
+    else one = Cvt<T>::load(p);
   }
-}
+  __device__ __forceinline__ void unpack(float* f) const {
+    constexpr int VEC = VecIO<T>::N;
+    if constexpr (MODE == EW_FULL || MODE == EW_PER_COL) {
+      VecIO<T>::unpack(vec, f);
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) f[j] = one;
+    }
+  }
+};
 
-// out[r, c] = a[..] op b[..]; cols_vec = vectors per output row.  IDX: uint32_t when the vector count fits,
-// which keeps the row / column split a 32-bit division.
-template <typename T, int OP, typename IDX>
-__global__ __launch_bounds__(256) void ew_binary_2d_vec_kernel(const T* a, const T* b,
-                                                               T* out, int64_t nvec, int64_t cols_vec,
-                                                               int amode, int bmode) {
+// out[r, c] = a[..] op b[..] over a [rows, cols] output; cols_vec = vectors per output row; AM / BM say how
+// each operand maps onto the output.
+template <typename T, int OP, int AM, int BM>
+__global__ __launch_bounds__(256) void ew_binary_2d_vec_kernel(const T* a, const T* b, T* out, uint32_t nvec,
+                                                               uint32_t cols_vec) {
   constexpr int VEC = VecIO<T>::N;
-  const int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
   if (v >= nvec) return;
-  const IDX r = IDX(v) / IDX(cols_vec);
-  const IDX c = IDX(v) - r * IDX(cols_vec);
+  uint32_t r = 0, c = v;
+  if constexpr (AM != EW_FULL || BM != EW_FULL) {
+    r = v / cols_vec;
+    c = v - r * cols_vec;
+  }
+  EwRaw<T, AM> ra;
+  EwRaw<T, BM> rb;
+  ra.load(a, v, r, c);
+  rb.load(b, v, r, c);
   float fa[VEC], fb[VEC];
-  ew_fetch<T>(a, amode, v, int64_t(r), int64_t(c), fa);
-  ew_fetch<T>(b, bmode, v, int64_t(r), int64_t(c), fb);
+  ra.unpack(fa);
+  rb.unpack(fb);
 #pragma unroll
   for (int j = 0; j < VEC; ++j) fa[j] = ew_bin<OP, float>(fa[j], fb[j]);
-  st16_stream(out + v * VEC, VecIO<T>::pack(fa));
+  st16_stream(out + size_t(v) * VEC, VecIO<T>::pack(fa));
 }
 
 struct EwDims {
@@ -267,14 +283,28 @@ static int binary_launch(const void* a, const void* b, void* out, const EwDims& 
       auto vec_ok = [&](const void* p, int mode) {
         return mode == EW_PER_ROW || mode == EW_SINGLE || aligned16(p);
       };
-      if (am >= 0 && bm >= 0 && cols % VEC == 0 && aligned16(out) && vec_ok(a, am) && vec_ok(b, bm)) {
-        const int64_t nvec = n / VEC, cols_vec = cols / VEC;
-        if (nvec < 0x7fffffffLL)
-          hipLaunchKernelGGL((ew_binary_2d_vec_kernel<T, OP, uint32_t>), dim3(blocks_for(nvec)), dim3(256), 0, s, pa,
-                             pb, po, nvec, cols_vec, am, bm);
-        else
-          hipLaunchKernelGGL((ew_binary_2d_vec_kernel<T, OP, int64_t>), dim3(blocks_for(nvec)), dim3(256), 0, s, pa,
-                             pb, po, nvec, cols_vec, am, bm);
+      // one full operand, the other in any of the four modes; two broadcast operands take the generic kernel
+      if (am >= 0 && bm >= 0 && (am == EW_FULL || bm == EW_FULL) && cols % VEC == 0 && aligned16(out) &&
+          vec_ok(a, am) && vec_ok(b, bm) && n / VEC < 0x7fffffffLL) {
+        const uint32_t nvec = uint32_t(n / VEC), cols_vec = uint32_t(cols / VEC);
+        const dim3 grid(blocks_for(nvec)), block(256);
+#define HK_EW_2D(AM, BM) \
+  hipLaunchKernelGGL((ew_binary_2d_vec_kernel<T, OP, AM, BM>), grid, block, 0, s, pa, pb, po, nvec, cols_vec)
+        if (am == EW_FULL) {
+          switch (bm) {
+            case EW_FULL: HK_EW_2D(EW_FULL, EW_FULL); break;
+            case EW_PER_ROW: HK_EW_2D(EW_FULL, EW_PER_ROW); break;
+            case EW_PER_COL: HK_EW_2D(EW_FULL, EW_PER_COL); break;
+            default: HK_EW_2D(EW_FULL, EW_SINGLE); break;
+          }
+        } else {
+          switch (am) {
+            case EW_PER_ROW: HK_EW_2D(EW_PER_ROW, EW_FULL); break;
+            case EW_PER_COL: HK_EW_2D(EW_PER_COL, EW_FULL); break;
+            default: HK_EW_2D(EW_SINGLE, EW_FULL); break;
+          }
+        }
+#undef HK_EW_2D
         profile_after(s);
         return launch_check("ew_binary_2d_vec_kernel");
       }

@@ -237,3 +237,46 @@ def test_vocab_parallel_loss_over_two_shards_equals_the_fused_loss(hk, cuda, dty
     helpers.assert_close(loss.view(rows), loss_ref, dtype, "loss", rtol=2e-2 if dtype == "bf16" else 1e-5)
     helpers.assert_close(torch.cat(grads, dim=1), grad_ref, dtype, "gradient",
                          rtol=1e-1 if dtype == "bf16" else 1e-5)
+
+
+def test_division_by_a_per_row_value_is_correctly_rounded(hk, cuda):
+    """The per-row divisor path forms one reciprocal per row and corrects each quotient twice; the result must
+    be the correctly rounded fp32 quotient, bit for bit, over the whole exponent range, zeros, infinities, NaN
+    and denormals included (torch's fp32 division is IEEE and serves as the reference)."""
+    import torch
+    rows, cols = 4096, 4096
+    g = torch.Generator(device="cuda").manual_seed(1)
+    mant = torch.rand(rows, cols, generator=g, device=cuda) + 1.0
+    expo = torch.randint(-60, 60, (rows, cols), generator=g, device=cuda)
+    a = torch.ldexp(mant, expo) * torch.where(torch.rand(rows, cols, generator=g, device=cuda) < 0.5, -1.0, 1.0)
+    b = torch.ldexp(torch.rand(rows, 1, generator=g, device=cuda) + 1.0,
+                    torch.randint(-126, 127, (rows, 1), generator=g, device=cuda))
+    special = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), float("nan"), 1e-45, -3e-39, 3e38, 1.0, 3.0],
+                           device=cuda)
+    a[:, :10] = special
+    b[:10, 0] = special
+    out = torch.empty_like(a)
+    hk.binary("div", a, b, out)
+    torch.cuda.synchronize()
+    want = a / b
+    same = (out.view(torch.int32) == want.view(torch.int32)) | (torch.isnan(out) & torch.isnan(want))
+    assert bool(same.all()), "%d of %d quotients differ from the correctly rounded ones" % (int((~same).sum()), same.numel())
+
+
+def test_bf16_division_rounds_like_the_exact_quotient(hk, cuda):
+    """bf16 quotients are formed with the hardware reciprocal; every bf16 bit pattern as dividend against 4096
+    divisors (random, plus zeros, infinities, NaN, denormals, extremes), full and per-row operand modes: bit
+    for bit the bf16 rounding of the IEEE fp32 quotient."""
+    import torch
+    a = torch.arange(65536, device=cuda, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)   # all patterns
+    g = torch.Generator(device="cuda").manual_seed(2)
+    b = torch.randint(0, 65536, (4096,), generator=g, device=cuda, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    b[:8] = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), float("nan"), 1e-40, 3e38, 1.0], device=cuda).bfloat16()
+    A = a.view(1, 65536).expand(4096, 65536).contiguous()
+    out = torch.empty_like(A)
+    for bb in (b.view(4096, 1), b.view(4096, 1).expand(4096, 65536).contiguous()):
+        hk.binary("div", A, bb, out)
+        torch.cuda.synchronize()
+        want = (A.float() / bb.float()).bfloat16()
+        same = (out.view(torch.int16) == want.view(torch.int16)) | (torch.isnan(out) & torch.isnan(want))
+        assert bool(same.all()), "%d of %d bf16 quotients differ" % (int((~same).sum()), same.numel())

@@ -238,7 +238,15 @@ def case_elementwise(hk, torch, nsets, which):
     g = torch.Generator(device="cuda").manual_seed(812)
     labels = torch.randint(0, 4 * cols, (rows,), generator=g, device="cuda", dtype=torch.int64)
     gl = torch.full((rows,), 1.0 / rows, dtype=bf, device="cuda")
-    return (lambda i: hk.vocab_parallel_ce_bwd(xs[i % 2], labels, gl, outs[i % 2], cols)), 2 * n * 2 + rows * 10, rows
+    if which == "vce":
+        return (lambda i: hk.vocab_parallel_ce_bwd(xs[i % 2], labels, gl, outs[i % 2], cols)), 2 * n * 2 + rows * 10, rows
+    # the fused form: shard 1 of 4 (columns [32000, 64000))
+    stats = torch.empty(3, rows, device="cuda")
+    if which == "stats":
+        return (lambda i: hk.vocab_parallel_ce_stats(xs[i % 2], labels, stats, cols, IGNORE)), n * 2 + rows * 20, rows
+    lse = torch.full((rows,), 12.0, device="cuda")
+    return (lambda i: hk.vocab_parallel_ce_bwd_fused(xs[i % 2], labels, lse, gl, outs[i % 2], cols, IGNORE)), \
+        2 * n * 2 + rows * 14, rows
 
 
 def case_reduce(hk, torch, nsets, axes, op, three_d=False):
@@ -309,6 +317,8 @@ CASES = [
     ("next: exp bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "exp")),
     ("next: exp / row sum in place bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "div")),
     ("next: vocab-parallel CE bwd bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "vce")),
+    ("next: vocab-parallel CE fused stats bf16 [16384x32000] (read only)", lambda hk, t, n: case_elementwise(hk, t, n, "stats")),
+    ("next: vocab-parallel CE fused bwd bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "fused")),
     ("C4 rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "fwd")),
     ("C4 rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "bwd")),
     ("C5 sce fwd bf16 [16384x32000]", lambda hk, t, n: case_sce(hk, t, 2, "fwd")),

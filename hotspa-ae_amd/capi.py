@@ -299,6 +299,31 @@ def vocab_parallel_ce_bwd(softmax, labels, grad_loss, out, vocab_start, stream=N
                                          stream if stream is not None else current_stream()))
 
 
+def vocab_parallel_ce_stats(logits, labels, stats, vocab_start, ignored_index, stream=None):
+    """stats: fp32 [3, rows] (row maximum, sum of exp(x - maximum), picked logit) of this column shard."""
+    rows, cols = logits.shape
+    check(lib().hk_vocab_parallel_ce_stats(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(stats), _i64(rows),
+                                           _i64(cols), _i64(vocab_start), _i64(ignored_index),
+                                           stream if stream is not None else current_stream()))
+
+
+def vocab_parallel_ce_combine(stats, labels, ignored_index, loss, lse, stream=None):
+    """stats: fp32 [nshards, 3, rows]; loss (any float dtype) and lse (fp32) are [rows]; either may be None."""
+    nshards, _, rows = stats.shape
+    code = dtype_code(loss) if loss is not None else HK_FLOAT32
+    check(lib().hk_vocab_parallel_ce_combine(code, _ptr(stats), ctypes.c_int(nshards), _ptr(labels),
+                                             _i64(ignored_index), _ptr(loss), _ptr(lse), _i64(rows),
+                                             stream if stream is not None else current_stream()))
+
+
+def vocab_parallel_ce_bwd_fused(logits, labels, lse, grad_loss, out, vocab_start, ignored_index, stream=None):
+    rows, cols = logits.shape
+    check(lib().hk_vocab_parallel_ce_bwd_fused(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(lse),
+                                               _ptr(grad_loss), _ptr(out), _i64(rows), _i64(cols),
+                                               _i64(vocab_start), _i64(ignored_index),
+                                               stream if stream is not None else current_stream()))
+
+
 def _odi(shape, dim):
     dim = dim % len(shape)
     outer = 1

@@ -176,6 +176,47 @@ void dal_fwd_kernel(DalFwdArgs a) {
   const bool load_x0 = row_x0 > 0;
   const bool dropout = a.dropout != 0;
 
+  // Every load of the row is issued before the first one is waited for (the optional operands sit behind
+  // uniform branches; unpacking inside those branches would serialise the loads).  A thread past the row's
+  // end shadows chunk 0 and contributes nothing.
+  constexpr int NI = kChunk / VecIO<IT>::N;
+  constexpr int NR = kChunk / VecIO<RT>::N;
+  u32x4 raw0[NC][NI], raw1[NC][NI], rawr[NC][NR];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+#pragma unroll
+    for (int k = 0; k < NI; ++k) { raw0[i][k] = u32x4{0, 0, 0, 0}; raw1[i][k] = u32x4{0, 0, 0, 0}; }
+#pragma unroll
+    for (int k = 0; k < NR; ++k) rawr[i][k] = u32x4{0, 0, 0, 0};
+  }
+  if (load_x0) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int c = i * tpr + t;
+      const IT* p = static_cast<const IT*>(a.x0) + (row_x0 - 1) * int64_t(a.cols) + (c < a.nchunks ? c : 0) * kChunk;
+#pragma unroll
+      for (int k = 0; k < NI; ++k) raw0[i][k] = ld16(p + k * VecIO<IT>::N);
+    }
+  }
+  if (a.x1) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int c = i * tpr + t;
+      const IT* p = static_cast<const IT*>(a.x1) + row * int64_t(a.cols) + (c < a.nchunks ? c : 0) * kChunk;
+#pragma unroll
+      for (int k = 0; k < NI; ++k) raw1[i][k] = ld16(p + k * VecIO<IT>::N);
+    }
+  }
+  if (a.residual) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int c = i * tpr + t;
+      const RT* p = static_cast<const RT*>(a.residual) + row * int64_t(a.cols) + (c < a.nchunks ? c : 0) * kChunk;
+#pragma unroll
+      for (int k = 0; k < NR; ++k) rawr[i][k] = ld16(p + k * VecIO<RT>::N);
+    }
+  }
+
   float xf[NC * kChunk];
   int cnt = 0;
 #pragma unroll
@@ -189,12 +230,13 @@ void dal_fwd_kernel(DalFwdArgs a) {
       const int col = c * kChunk;
       if (load_x0) {
         const int64_t e0 = (row_x0 - 1) * int64_t(a.cols) + col;
-        load8<IT>(static_cast<const IT*>(a.x0) + e0, v);
         uint32_t keep = 0xffu;
         if (dropout) {
           keep = keep_bits8(e0, 0, a.drop);
           if (row_ok) store_mask8(a.dmask + e0, keep);
         }
+#pragma unroll
+        for (int k = 0; k < NI; ++k) VecIO<IT>::unpack(raw0[i][k], v + k * VecIO<IT>::N);
 #pragma unroll
         for (int j = 0; j < kChunk; ++j) {
           float xv = v[j] * rowscale_val;
@@ -211,12 +253,13 @@ void dal_fwd_kernel(DalFwdArgs a) {
       const int64_t e = row * int64_t(a.cols) + col;
       if (a.x1) {
         float w[kChunk];
-        load8<IT>(static_cast<const IT*>(a.x1) + e, w);
         uint32_t keep = 0xffu;
         if (dropout) {
           keep = keep_bits8(e, 1, a.drop);
           if (row_ok) store_mask8(a.dmask1 + e, keep);
         }
+#pragma unroll
+        for (int k = 0; k < NI; ++k) VecIO<IT>::unpack(raw1[i][k], w + k * VecIO<IT>::N);
 #pragma unroll
         for (int j = 0; j < kChunk; ++j) {
           float xv = w[j];
@@ -226,7 +269,8 @@ void dal_fwd_kernel(DalFwdArgs a) {
       }
       if (a.residual) {
         float w[kChunk];
-        load8<RT>(static_cast<const RT*>(a.residual) + e, w);
+#pragma unroll
+        for (int k = 0; k < NR; ++k) VecIO<RT>::unpack(rawr[i][k], w + k * VecIO<RT>::N);
 #pragma unroll
         for (int j = 0; j < kChunk; ++j) v[j] += w[j];
       }

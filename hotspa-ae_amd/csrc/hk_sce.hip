@@ -28,6 +28,11 @@ struct SceArgs {
   int nvec;
   int64_t ignored_index;
   int stream_store;
+  // sparse forward on a column shard [vocab_start, vocab_start + cols) of a wider row: instead of a loss,
+  // stats[0..rows) = the shard's row maximum, stats[rows..2 rows) = sum of exp(x - that maximum),
+  // stats[2 rows..3 rows) = the logit at the label when the label falls into the shard, else 0
+  float* stats;
+  int64_t vocab_start;
 };
 
 template <bool WAVE_ROW>
@@ -52,7 +57,15 @@ void sce_sparse_fwd_kernel(SceArgs a) {
   T* loss = static_cast<T*>(a.out);
   const int64_t label = a.labels[row];
   if (label == a.ignored_index) {          // uniform over the row's threads
-    if (t == 0) Cvt<T>::store(loss + row, 0.f);
+    if (t == 0) {
+      if (a.stats) {
+        a.stats[row] = kNegInf;
+        a.stats[a.rows + row] = 0.f;
+        a.stats[2 * a.rows + row] = 0.f;
+      } else {
+        Cvt<T>::store(loss + row, 0.f);
+      }
+    }
     return;
   }
   const T* xr = static_cast<const T*>(a.logits) + row * int64_t(a.cols);
@@ -88,7 +101,14 @@ void sce_sparse_fwd_kernel(SceArgs a) {
   MaxSumMaxTuple p;
   p.v[0] = (m == kNegInf) ? kNegInf : ml; p.v[1] = s; p.v[2] = m;
   p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);
-  if (t == 0) {
+  if (t == 0 && a.stats) {
+    const float M = p.v[2];
+    // sum exp(x - M) = S * 2^(ML - M * log2e)
+    a.stats[row] = M;
+    a.stats[a.rows + row] = (M == kNegInf) ? 0.f : p.v[1] * __builtin_amdgcn_exp2f(-fmaf(M, kLog2e, -p.v[0]));
+    const int64_t local = label - a.vocab_start;
+    a.stats[2 * a.rows + row] = (local >= 0 && local < a.cols) ? Cvt<T>::load(xr + local) : 0.f;
+  } else if (t == 0) {
     float r;
     if (label >= 0 && label < a.cols) {
       const float xl = Cvt<T>::load(xr + label);
@@ -306,7 +326,15 @@ void sce_generic_kernel(SceArgs a) {
     label = a.labels[row];
     if (label == a.ignored_index) {
       if (MODE == 0) {
-        if (threadIdx.x == 0) SceIO<T, CT>::st(static_cast<T*>(a.out) + row, CT(0));
+        if (threadIdx.x == 0) {
+          if (a.stats) {
+            a.stats[row] = kNegInf;
+            a.stats[a.rows + row] = 0.f;
+            a.stats[2 * a.rows + row] = 0.f;
+          } else {
+            SceIO<T, CT>::st(static_cast<T*>(a.out) + row, CT(0));
+          }
+        }
       } else {
         T* dxr = static_cast<T*>(a.out) + row * cols;
         for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) SceIO<T, CT>::st(dxr + c, CT(0));
@@ -323,7 +351,14 @@ void sce_generic_kernel(SceArgs a) {
   CT s = 0;
   for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) s += sce_exp<CT>(SceIO<T, CT>::ld(xr + c) - m);
   s = sce_block_reduce<CT>(s, lds, false);
-  if (MODE == 0) {
+  if (MODE == 0 && a.stats) {
+    if (threadIdx.x == 0) {
+      const int64_t local = label - a.vocab_start;
+      a.stats[row] = float(m);
+      a.stats[a.rows + row] = float(s);
+      a.stats[2 * a.rows + row] = (local >= 0 && local < cols) ? float(SceIO<T, CT>::ld(xr + local)) : 0.f;
+    }
+  } else if (MODE == 0) {
     if (threadIdx.x == 0) {
       CT r;
       if (label >= 0 && label < cols) r = (sce_log<CT>(s) + m) - SceIO<T, CT>::ld(xr + label);
@@ -475,6 +510,16 @@ int hk_sce_sparse_fwd(int dtype, const void* logits, const int64_t* labels, void
   a.logits = logits; a.labels = labels; a.out = loss; a.rows = rows; a.cols = int(cols);
   a.ignored_index = ignored_index;
   return sce_dispatch<0>(dtype, a, as_hip(stream), "hk_sce_sparse_fwd");
+}
+
+int hk_vocab_parallel_ce_stats(int dtype, const void* logits, const int64_t* labels, float* stats, int64_t rows,
+                               int64_t cols, int64_t vocab_start, int64_t ignored_index, hkStream_t stream) {
+  HK_REQUIRE(cols <= 0x3fffffff, HK_ERR_INVALID, "hk_vocab_parallel_ce_stats: cols too large");
+  HK_REQUIRE(rows == 0 || stats != nullptr, HK_ERR_INVALID, "hk_vocab_parallel_ce_stats: null output");
+  SceArgs a{};
+  a.logits = logits; a.labels = labels; a.out = stats; a.rows = rows; a.cols = int(cols);
+  a.ignored_index = ignored_index; a.stats = stats; a.vocab_start = vocab_start;
+  return sce_dispatch<0>(dtype, a, as_hip(stream), "hk_vocab_parallel_ce_stats");
 }
 
 int hk_sce_sparse_bwd(int dtype, const void* logits, const int64_t* labels, const void* grad_loss,

@@ -40,12 +40,15 @@ void vocab_ce_bwd_vec_kernel(const T* softmax, const int64_t* __restrict__ label
   if (v >= nvec) return;
   const int64_t r = v / cols_vec;
   const int64_t c0 = (v - r * cols_vec) * VEC;
-  const uint64_t hit = uint64_t(labels[r]) - uint64_t(vocab_start);
+  const u32x4 raw = ld16(softmax + v * VEC);
+  // position of the label inside this vector, or a value no j reaches (labels outside the shard, negative ones)
+  const uint64_t rel = uint64_t(labels[r]) - uint64_t(vocab_start) - uint64_t(c0);
+  const uint32_t hit = rel < uint64_t(VEC) ? uint32_t(rel) : 0xffffffffu;
   const float g = Cvt<T>::load(grad_loss + r);
   float f[VEC];
-  VecIO<T>::unpack(ld16(softmax + v * VEC), f);
+  VecIO<T>::unpack(raw, f);
 #pragma unroll
-  for (int j = 0; j < VEC; ++j) f[j] = (uint64_t(c0 + j) == hit ? f[j] - 1.0f : f[j]) * g;
+  for (int j = 0; j < VEC; ++j) f[j] = (uint32_t(j) == hit ? f[j] - 1.0f : f[j]) * g;
   st16_stream(out + v * VEC, VecIO<T>::pack(f));
 }
 
@@ -61,6 +64,119 @@ void vocab_ce_bwd_scalar_kernel(const T* softmax, const int64_t* __restrict__ la
   const uint64_t hit = uint64_t(labels[r]) - uint64_t(vocab_start);
   const CT s = CT(Cvt<T>::load(softmax + i)), g = CT(Cvt<T>::load(grad_loss + r));
   Cvt<T>::store(out + i, (c == hit ? s - CT(1) : s) * g);
+}
+
+// ---------------------------------------------------------------------------
+// The fused form: one read of the shard in the forward (hk_vocab_parallel_ce_stats, in the cross-entropy
+// source), a per-row combination of the shards' statistics, and a backward that rebuilds softmax from the
+// logits and the global log-sum-exp instead of reading a stored softmax.
+// ---------------------------------------------------------------------------
+// stats: [nshards, 3, rows] (maximum, sum of exp(x - maximum), picked logit) as an all-gather leaves them.
+// lse[r] = log sum_k exp over the whole row; loss[r] = lse - picked logit, 0 for an ignored row.
+template <typename T>
+__global__ __launch_bounds__(256)
+void vocab_ce_combine_kernel(const float* __restrict__ stats, int nshards, const int64_t* __restrict__ labels,
+                             int64_t ignored_index, T* __restrict__ loss, float* __restrict__ lse, int64_t rows) {
+  const int64_t r = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (r >= rows) return;
+  float gmax = -__builtin_huge_valf();
+  for (int k = 0; k < nshards; ++k) gmax = fmaxf(gmax, stats[(int64_t(k) * 3 + 0) * rows + r]);
+  float gsum = 0.f, picked = 0.f;
+  for (int k = 0; k < nshards; ++k) {
+    const float m = stats[(int64_t(k) * 3 + 0) * rows + r];
+    const float s = stats[(int64_t(k) * 3 + 1) * rows + r];
+    if (s > 0.f) gsum += s * expf(m - gmax);
+    picked += stats[(int64_t(k) * 3 + 2) * rows + r];
+  }
+  const bool ignored = labels[r] == ignored_index;
+  const float l = ignored ? 0.f : logf(gsum) + gmax;
+  if (lse) lse[r] = l;
+  if (loss) {
+    using CT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
+    Cvt<T>::store(loss + r, CT(ignored ? 0.f : l - picked));
+  }
+}
+
+// out[r, c] = (exp(x[r, c] - lse[r]) - [c == labels[r] - vocab_start]) * grad_loss[r]; zeros for an ignored row
+template <typename T>
+__global__ __launch_bounds__(256)
+void vocab_ce_bwd_fused_kernel(const T* x, const int64_t* __restrict__ labels, const float* __restrict__ lse,
+                               const T* __restrict__ grad_loss, T* out, uint32_t nvec, uint32_t cols_vec,
+                               int64_t vocab_start, int64_t ignored_index, int stream_store) {
+  constexpr int VEC = VecIO<T>::N;
+  constexpr float kLog2e = 1.4426950408889634f;
+  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+  if (v >= nvec) return;
+  const uint32_t r = v / cols_vec;
+  const uint32_t c0 = (v - r * cols_vec) * VEC;
+  // all four loads are issued before any is waited for; an ignored row is read like the others (a branch on
+  // the label around the vector load would put the two loads in series) and its result replaced by zeros
+  const u32x4 raw = ld16(x + size_t(v) * VEC);
+  const int64_t label = labels[r];
+  const float l2 = lse[r] * kLog2e;
+  float g = Cvt<T>::load(grad_loss + r);
+  const bool ignored = label == ignored_index;
+  g = ignored ? 0.f : g;
+  float f[VEC];
+  VecIO<T>::unpack(raw, f);
+  // position of the label inside this vector, or a value no j reaches (labels outside the shard, negative ones)
+  const uint64_t rel = uint64_t(label) - uint64_t(vocab_start) - uint64_t(c0);
+  const uint32_t hit = rel < uint64_t(VEC) ? uint32_t(rel) : 0xffffffffu;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const float p = __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, -l2));
+    const float o = (uint32_t(j) == hit) ? fmaf(p, g, -g) : p * g;
+    f[j] = ignored ? 0.f : o;              // also when exp overflowed to inf or the logit was NaN
+  }
+  if (stream_store) st16_stream(out + size_t(v) * VEC, VecIO<T>::pack(f));
+  else st16(out + size_t(v) * VEC, VecIO<T>::pack(f));
+}
+
+template <typename T, typename CT>
+__global__ __launch_bounds__(256)
+void vocab_ce_bwd_fused_scalar_kernel(const T* x, const int64_t* __restrict__ labels, const float* __restrict__ lse,
+                                      const T* __restrict__ grad_loss, T* out, int64_t total, int64_t cols,
+                                      int64_t vocab_start, int64_t ignored_index) {
+  const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t r = i / cols;
+  const int64_t label = labels[r];
+  CT o = CT(0);
+  if (label != ignored_index) {
+    const uint64_t hit = uint64_t(label) - uint64_t(vocab_start);
+    const CT g = CT(Cvt<T>::load(grad_loss + r));
+    const CT p = CT(exp(double(Cvt<T>::load(x + i)) - double(lse[r])));
+    o = (uint64_t(i - r * cols) == hit) ? p * g - g : p * g;
+  }
+  Cvt<T>::store(out + i, o);
+}
+
+template <typename T>
+static int vocab_bwd_fused_typed(const void* x, const int64_t* labels, const float* lse, const void* grad_loss,
+                                 void* out, int64_t rows, int64_t cols, int64_t vocab_start, int64_t ignored_index,
+                                 hipStream_t s) {
+  const int64_t total = rows * cols;
+  if constexpr (!std::is_same<T, double>::value) {
+    constexpr int VEC = VecIO<T>::N;
+    if (cols % VEC == 0 && aligned16(x) && aligned16(out) && total / VEC < 0x7fffffffLL) {
+      const uint32_t nvec = uint32_t(total / VEC);
+      profile_before(s);
+      hipLaunchKernelGGL((vocab_ce_bwd_fused_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
+                         static_cast<const T*>(x), labels, lse, static_cast<const T*>(grad_loss), static_cast<T*>(out),
+                         nvec, uint32_t(cols / VEC), vocab_start, ignored_index,
+                         tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1);
+      profile_after(s);
+      return launch_check("vocab_ce_bwd_fused_kernel");
+    }
+  }
+  HK_REQUIRE((total + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_vocab_parallel_ce_bwd_fused: output too large");
+  using CT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
+  profile_before(s);
+  hipLaunchKernelGGL((vocab_ce_bwd_fused_scalar_kernel<T, CT>), dim3(unsigned((total + 255) / 256)), dim3(256), 0, s,
+                     static_cast<const T*>(x), labels, lse, static_cast<const T*>(grad_loss), static_cast<T*>(out),
+                     total, cols, vocab_start, ignored_index);
+  profile_after(s);
+  return launch_check("vocab_ce_bwd_fused_scalar_kernel");
 }
 
 template <typename T>
@@ -121,6 +237,51 @@ int hk_vocab_parallel_ce_gather(int dtype, const void* logits, const int64_t* la
   }
 #undef HK_VCE_GATHER
   return launch_check("vocab_ce_gather_kernel");
+}
+
+int hk_vocab_parallel_ce_combine(int loss_dtype, const float* stats, int nshards, const int64_t* labels,
+                                 int64_t ignored_index, void* loss, float* lse, int64_t rows, hkStream_t stream) {
+  HK_REQUIRE(rows >= 0 && nshards >= 1, HK_ERR_INVALID, "hk_vocab_parallel_ce_combine: bad shape");
+  if (rows == 0) return HK_OK;
+  HK_REQUIRE(stats && labels && (loss || lse), HK_ERR_INVALID, "hk_vocab_parallel_ce_combine: null input/output");
+  hipStream_t s = as_hip(stream);
+  const dim3 grid(unsigned((rows + 255) / 256)), block(256);
+#define HK_VCE_COMBINE(T)                                                                                       \
+  hipLaunchKernelGGL((vocab_ce_combine_kernel<T>), grid, block, 0, s, stats, nshards, labels, ignored_index,    \
+                     static_cast<T*>(loss), lse, rows)
+  switch (loss_dtype) {
+    case HK_FLOAT32: HK_VCE_COMBINE(float); break;
+    case HK_BFLOAT16: HK_VCE_COMBINE(bf16); break;
+    case HK_FLOAT16: HK_VCE_COMBINE(fp16); break;
+    case HK_FLOAT64: HK_VCE_COMBINE(double); break;
+    default:
+      set_last_error("hk_vocab_parallel_ce_combine: not implemented for dtype %d", loss_dtype);
+      return HK_ERR_UNSUPPORTED;
+  }
+#undef HK_VCE_COMBINE
+  return launch_check("vocab_ce_combine_kernel");
+}
+
+int hk_vocab_parallel_ce_bwd_fused(int dtype, const void* logits, const int64_t* labels, const float* lse,
+                                   const void* grad_loss, void* out, int64_t rows, int64_t cols,
+                                   int64_t vocab_start, int64_t ignored_index, hkStream_t stream) {
+  HK_REQUIRE(rows >= 0 && cols >= 0, HK_ERR_INVALID, "hk_vocab_parallel_ce_bwd_fused: negative shape");
+  if (rows == 0 || cols == 0) return HK_OK;
+  HK_REQUIRE(logits && labels && lse && grad_loss && out, HK_ERR_INVALID,
+             "hk_vocab_parallel_ce_bwd_fused: null input/output");
+  hipStream_t s = as_hip(stream);
+#define HK_VCE_BWD(T) \
+  return vocab_bwd_fused_typed<T>(logits, labels, lse, grad_loss, out, rows, cols, vocab_start, ignored_index, s)
+  switch (dtype) {
+    case HK_FLOAT32: HK_VCE_BWD(float);
+    case HK_BFLOAT16: HK_VCE_BWD(bf16);
+    case HK_FLOAT16: HK_VCE_BWD(fp16);
+    case HK_FLOAT64: HK_VCE_BWD(double);
+    default:
+      set_last_error("hk_vocab_parallel_ce_bwd_fused: not implemented for dtype %d", dtype);
+      return HK_ERR_UNSUPPORTED;
+  }
+#undef HK_VCE_BWD
 }
 
 int hk_vocab_parallel_ce_bwd(int dtype, const void* softmax, const int64_t* labels, const void* grad_loss,

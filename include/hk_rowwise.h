@@ -365,6 +365,29 @@ HK_API int hk_vocab_parallel_ce_bwd(int dtype, const void* softmax, const int64_
                                     const void* grad_loss, void* out, int64_t rows, int64_t cols,
                                     int64_t vocab_start, hkStream_t stream);
 
+/* The same loss in its fused form: the shard is read once in the forward and once in the backward, and no
+ * softmax array is kept.  No counterpart in the reference, which composes the loss from eight launches
+ * (hetu/graph/ops/VocabParallelCrossEntropyLoss.cc:51-108: max, subtract, exp, sum, divide, log, gather,
+ * subtract) and stores softmax for the backward.
+ *   stats:   per row of the shard, in ONE pass: stats[0][r] = max_c x, stats[1][r] = sum_c exp(x - max),
+ *            stats[2][r] = x[r, labels[r] - vocab_start] when the label lies in the shard, else 0
+ *            (fp32, [3, rows]); an ignored row is not read and gets (-inf, 0, 0).
+ *   combine: stats of all shards, [nshards, 3, rows] as an all-gather leaves them ->
+ *            lse[r] = log sum over the whole row (fp32), loss[r] = lse - picked (0 for an ignored row).
+ *            Either output may be NULL.
+ *   bwd_fused: out[r, c] = (exp(x[r, c] - lse[r]) - [c == labels[r] - vocab_start]) * grad_loss[r];
+ *            an ignored row is written as zeros.  out may alias logits. */
+HK_API int hk_vocab_parallel_ce_stats(int dtype, const void* logits, const int64_t* labels, float* stats,
+                                      int64_t rows, int64_t cols, int64_t vocab_start,
+                                      int64_t ignored_index, hkStream_t stream);
+HK_API int hk_vocab_parallel_ce_combine(int loss_dtype, const float* stats, int nshards,
+                                        const int64_t* labels, int64_t ignored_index, void* loss,
+                                        float* lse, int64_t rows, hkStream_t stream);
+HK_API int hk_vocab_parallel_ce_bwd_fused(int dtype, const void* logits, const int64_t* labels,
+                                          const float* lse, const void* grad_loss, void* out,
+                                          int64_t rows, int64_t cols, int64_t vocab_start,
+                                          int64_t ignored_index, hkStream_t stream);
+
 /* ======================================================================== *
  * Element-wise operators on dense arrays of fp32 / bf16 / fp16 / fp64 (16-bit
  * types compute in fp32 and round once).  out may alias an input of its shape.

@@ -280,3 +280,86 @@ def test_bf16_division_rounds_like_the_exact_quotient(hk, cuda):
         want = (A.float() / bb.float()).bfloat16()
         same = (out.view(torch.int16) == want.view(torch.int16)) | (torch.isnan(out) & torch.isnan(want))
         assert bool(same.all()), "%d of %d bf16 quotients differ" % (int((~same).sum()), same.numel())
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16", "fp64"])
+@pytest.mark.parametrize("rows,cols,nshards", [(96, 4096, 2), (33, 32000, 4), (50, 1000, 5), (7, 24, 3)])
+def test_vocab_parallel_fused_form_equals_the_whole_row_loss(hk, cuda, dtype, rows, cols, nshards):
+    """One read per shard (row maximum, sum of exponentials, picked logit), a per-row combination of the shards'
+    statistics, and a backward that rebuilds softmax from logits and log-sum-exp: loss and gradient must equal
+    the cross-entropy of the unsplit matrix; ignored rows give loss 0 and a zero gradient; the label gather is
+    exact."""
+    import torch
+    ignored = -100
+    g = helpers.rng(rows + cols)
+    logits = _draw(61 + cols, (rows, cols), dtype) * 3
+    if dtype != "fp64":
+        logits = oracle.round_to(logits.astype(np.float32), dtype)
+    labels = g.integers(0, cols, rows).astype(np.int64); labels[::6] = ignored
+    loss_ref = oracle.sce_sparse_fwd(logits, labels, ignored) if dtype != "fp64" else None
+    if dtype == "fp64":
+        m = logits.max(axis=1, keepdims=True)
+        lse64 = (np.log(np.exp(logits - m).sum(axis=1)) + m[:, 0])
+        loss_ref = np.where(labels == ignored, 0.0, lse64 - logits[np.arange(rows), np.clip(labels, 0, cols - 1)])
+    gl = _draw(62, (rows,), dtype)
+    sm = np.exp(logits.astype(np.float64) - logits.astype(np.float64).max(axis=1, keepdims=True))
+    sm /= sm.sum(axis=1, keepdims=True)
+    onehot = np.zeros((rows, cols)); keep = labels != ignored
+    onehot[np.flatnonzero(keep), labels[keep]] = 1.0
+    grad_ref = np.where(keep[:, None], (sm - onehot) * gl.astype(np.float64)[:, None], 0.0)
+
+    full = helpers.to_torch(logits, dtype, cuda); tlab = torch.from_numpy(labels).to(cuda)
+    width = cols // nshards
+    bounds = [(k * width, cols if k == nshards - 1 else (k + 1) * width) for k in range(nshards)]
+    shards = [full[:, lo:hi].contiguous() for lo, hi in bounds]
+    stats = torch.empty(nshards, 3, rows, dtype=torch.float32, device=cuda)
+    for k, (lo, hi) in enumerate(bounds):
+        hk.vocab_parallel_ce_stats(shards[k], tlab, stats[k], lo, ignored)
+    torch.cuda.synchronize()
+    # the gather is exact, and falls into exactly one shard per row
+    picked = stats[:, 2, :].sum(dim=0).cpu().numpy().astype(np.float64)
+    want_picked = np.where(keep, logits[np.arange(rows), np.clip(labels, 0, cols - 1)], 0.0).astype(np.float64)
+    if dtype != "fp64":
+        assert np.array_equal(picked, want_picked)
+    loss = torch.empty(rows, dtype=full.dtype, device=cuda)
+    lse = torch.empty(rows, dtype=torch.float32, device=cuda)
+    hk.vocab_parallel_ce_combine(stats, tlab, ignored, loss, lse)     # stats as an all-gather would leave them
+    tgl = helpers.to_torch(gl, dtype, cuda)
+    grads = []
+    for k, (lo, hi) in enumerate(bounds):
+        out = torch.empty_like(shards[k])
+        hk.vocab_parallel_ce_bwd_fused(shards[k], tlab, lse, tgl, out, lo, ignored)
+        grads.append(out)
+    torch.cuda.synchronize()
+    tol = {"fp64": 1e-5}.get(dtype)      # statistics and log-sum-exp are fp32 whatever the logits' type
+    helpers.assert_close(loss, loss_ref, dtype, "loss", rtol=tol)
+    assert (helpers.to_numpy(loss)[~keep] == 0).all()
+    got = torch.cat(grads, dim=1)
+    helpers.assert_close(got, grad_ref, dtype, "gradient", rtol=tol)
+    assert (helpers.to_numpy(got)[~keep] == 0).all()
+    # in place on the logits, as a caller short of memory would run it
+    hk.vocab_parallel_ce_bwd_fused(shards[0], tlab, lse, tgl, shards[0], bounds[0][0], ignored)
+    torch.cuda.synchronize()
+    assert torch.equal(shards[0], grads[0])
+
+
+def test_vocab_parallel_stats_of_one_shard_match_their_definition(hk, cuda):
+    import torch
+    rows, cols, start = 40, 5120, 10240
+    x = torch.randn(rows, cols, device=cuda) * 4
+    x[3] = -float("inf")                                  # a shard with no finite logit
+    x[4, :100] = float("inf")
+    labels = torch.randint(start, start + cols, (rows,), device=cuda); labels[5] = start - 7; labels[6] = -100
+    stats = torch.empty(3, rows, device=cuda)
+    hk.vocab_parallel_ce_stats(x, labels, stats, start, -100)
+    torch.cuda.synchronize()
+    m = x.max(dim=1).values
+    keep = torch.ones(rows, dtype=torch.bool, device=cuda); keep[6] = False
+    assert torch.equal(stats[0][keep], m[keep]) and stats[0][6] == -float("inf")
+    s = torch.exp(x - m[:, None]).sum(dim=1)
+    fin = torch.isfinite(m) & keep
+    assert torch.allclose(stats[1][fin], s[fin], rtol=1e-5)
+    assert stats[1][3] == 0 and stats[1][6] == 0
+    local = (labels - start).clamp(0, cols - 1)
+    want = torch.where((labels >= start) & (labels < start + cols) & keep, x[torch.arange(rows), local], torch.zeros(()).to(x))
+    assert torch.equal(stats[2], want)

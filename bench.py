@@ -332,9 +332,9 @@ CASES = [
 
 
 # HBM bytes one launch of the RMSNorm backward kernel moves at the headline shape: rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE read 262985.9 and 270336.0 KiB per dispatch; a 256 MiB copy kernel calibrates the counters at
+# --pmc WRITE_SIZE read 262985.0 and 270336.0 KiB per dispatch; a 256 MiB copy kernel calibrates the counters at
 # x2.000 (FETCH_SIZE reads 131086 KiB for 262144 KiB fetched) and x1.000 (WRITE_SIZE).
-NORM_BWD_TRAFFIC_BYTES = int((262985.9 * 2.0 + 270336.0 * 1.0) * 1024)
+NORM_BWD_TRAFFIC_BYTES = int((262985.0 * 2.0 + 270336.0 * 1.0) * 1024)
 
 
 def time_case(hk, torch, launch, steps, warmup, profile_main=True):

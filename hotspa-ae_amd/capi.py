@@ -324,6 +324,26 @@ def vocab_parallel_ce_bwd_fused(logits, labels, lse, grad_loss, out, vocab_start
                                                stream if stream is not None else current_stream()))
 
 
+def norm(x, out, dim, p, workspace=None, stream=None):
+    """hk_norm: p-norm of x (any strided view) over `dim` (already wrapped); out is dense."""
+    shape, strides = list(x.shape), list(x.stride())
+    if workspace is None:
+        workspace = _workspace(reduce_workspace_bytes(dtype_code(x), shape, strides, [dim]), x.device)
+    wsb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(lib().hk_norm(dtype_code(x), _ptr(x), _ptr(out), ctypes.c_int(len(shape)), _arr(shape), _arr(strides),
+                        _i64(dim), _i64(p), _ptr(workspace), ctypes.c_size_t(wsb),
+                        stream if stream is not None else current_stream()))
+    return workspace
+
+
+def norm_bwd(x, norm_out, grad, out, dim, p, stream=None):
+    """hk_norm_bwd on dense tensors; x viewed as [before, x.shape[dim], after]."""
+    before, _, after = _odi(list(x.shape), dim)
+    check(lib().hk_norm_bwd(dtype_code(x), _ptr(x), _ptr(norm_out), _ptr(grad), _ptr(out), _i64(before),
+                            _i64(x.shape[dim]), _i64(after), _i64(p),
+                            stream if stream is not None else current_stream()))
+
+
 def _odi(shape, dim):
     dim = dim % len(shape)
     outer = 1

@@ -56,15 +56,47 @@ template <typename A> __device__ __forceinline__ bool is_nan(A v) {
   if constexpr (std::is_floating_point<A>::value) return v != v;
   else return false;
 }
-struct RSum {
+// Every reduction also names what happens to an element as it is loaded (pre) and to the finished value as it
+// is stored (post); `factor` is the reduction's one parameter (1 / count for the mean, the exponent p for a
+// p-norm).  The plain reductions load unchanged and store through project().
+struct RNoTransform {
+  template <typename A> static __device__ __forceinline__ A pre(A v, float) { return v; }
+  template <typename A> static __device__ __forceinline__ A post(A v, float factor, int is_mean) {
+    return project<A>(v, factor, is_mean);
+  }
+};
+struct RSum : RNoTransform {
   template <typename A> static __device__ __forceinline__ A identity() { return A(0); }
   template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return a + b; }
 };
-struct RProd {
+// p-norms: sum |x|^p, stored as its p-th root (Norm1.cu:17-56); p = 1 and p = 2 without a pow()
+template <typename A> __device__ __forceinline__ A abs_of(A v) { return v < A(0) ? -v : v; }
+struct RNorm1 : RSum {
+  template <typename A> static __device__ __forceinline__ A pre(A v, float) { return abs_of(v); }
+  template <typename A> static __device__ __forceinline__ A post(A v, float, int) { return v; }
+};
+struct RNorm2 : RSum {
+  template <typename A> static __device__ __forceinline__ A pre(A v, float) { return v * v; }
+  template <typename A> static __device__ __forceinline__ A post(A v, float, int) {
+    if constexpr (std::is_same<A, double>::value) return sqrt(v);
+    else return A(sqrtf(float(v)));
+  }
+};
+struct RNormP : RSum {
+  template <typename A> static __device__ __forceinline__ A pre(A v, float p) {
+    if constexpr (std::is_same<A, double>::value) return pow(abs_of(v), double(p));
+    else return A(powf(float(abs_of(v)), p));
+  }
+  template <typename A> static __device__ __forceinline__ A post(A v, float p, int) {
+    if constexpr (std::is_same<A, double>::value) return pow(v, 1.0 / double(p));
+    else return A(powf(float(v), 1.0f / p));
+  }
+};
+struct RProd : RNoTransform {
   template <typename A> static __device__ __forceinline__ A identity() { return A(1); }
   template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return a * b; }
 };
-struct RMax {
+struct RMax : RNoTransform {
   template <typename A> static __device__ __forceinline__ A identity() {
     if constexpr (std::is_floating_point<A>::value) return -std::numeric_limits<A>::infinity();
     else return std::numeric_limits<A>::lowest();
@@ -73,7 +105,7 @@ struct RMax {
     return (is_nan(a) || a > b) ? a : (is_nan(b) ? b : (a > b ? a : b));
   }
 };
-struct RMin {
+struct RMin : RNoTransform {
   template <typename A> static __device__ __forceinline__ A identity() {
     if constexpr (std::is_floating_point<A>::value) return std::numeric_limits<A>::infinity();
     else return std::numeric_limits<A>::max();
@@ -149,18 +181,18 @@ void reduce_inner_vec_kernel(InnerArgs a) {
       float f[VEC];
       VecIO<T>::unpack(r[u], f);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[u] = R::apply(acc[u], f[j]);
+      for (int j = 0; j < VEC; ++j) acc[u] = R::apply(acc[u], R::pre(f[j], a.factor));
     }
   }
   for (; v < nvec; v += tpr) {
     float f[VEC];
     VecIO<T>::unpack(ld16(p + v * VEC), f);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[0] = R::apply(acc[0], f[j]);
+    for (int j = 0; j < VEC; ++j) acc[0] = R::apply(acc[0], R::pre(f[j], a.factor));
   }
   // scalar tail of the last split
   for (int64_t c = c0 + nvec * VEC + t; c < c1; c += tpr)
-    acc[1] = R::apply(acc[1], Cvt<T>::load(static_cast<const T*>(a.in) + row * a.row_stride + c));
+    acc[1] = R::apply(acc[1], R::pre(Cvt<T>::load(static_cast<const T*>(a.in) + row * a.row_stride + c), a.factor));
   float s = R::apply(R::apply(R::apply(acc[0], acc[1]), R::apply(acc[2], acc[3])),
                      R::apply(R::apply(acc[4], acc[5]), R::apply(acc[6], acc[7])));
   if constexpr (WAVE_ROW) {
@@ -169,7 +201,7 @@ void reduce_inner_vec_kernel(InnerArgs a) {
     s = block_allreduce<AsFloatOp<R>>(s, red, int(blockDim.x >> 6));
   }
   if (t == 0) {
-    if (a.nsplit == 1) st_acc<OUT_T, float>(static_cast<OUT_T*>(a.out) + row, project<float>(s, a.factor, a.is_mean));
+    if (a.nsplit == 1) st_acc<OUT_T, float>(static_cast<OUT_T*>(a.out) + row, R::template post<float>(s, a.factor, a.is_mean));
     else static_cast<float*>(a.out)[row * a.nsplit + split] = s;
   }
 }
@@ -183,9 +215,9 @@ void reduce_inner_scalar_kernel(const T* in, OUT_T* out, int64_t rows, int64_t r
   const int64_t row = blockIdx.x;
   const T* p = in + row * row_stride;
   ACC acc = R::template identity<ACC>();
-  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) acc = R::template apply<ACC>(acc, ld_acc<T, ACC>(p + c));
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) acc = R::template apply<ACC>(acc, R::template pre<ACC>(ld_acc<T, ACC>(p + c), factor));
   acc = block_reduce_lds<R, ACC>(acc, lds);
-  if (threadIdx.x == 0) st_acc<OUT_T, ACC>(out + row, project<ACC>(acc, factor, is_mean));
+  if (threadIdx.x == 0) st_acc<OUT_T, ACC>(out + row, R::template post<ACC>(acc, factor, is_mean));
 }
 
 // ---------------------------------------------------------------------------
@@ -235,14 +267,14 @@ void reduce_outer_vec_kernel(OuterArgs a) {
         float f[VEC];
         VecIO<T>::unpack(v[u], f);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] = R::apply(acc[j], f[j]);
+        for (int j = 0; j < VEC; ++j) acc[j] = R::apply(acc[j], R::pre(f[j], a.factor));
       }
     }
     for (; r < r1; r += wy) {
       float f[VEC];
       VecIO<T>::unpack(ld16(p + r * a.r_stride), f);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] = R::apply(acc[j], f[j]);
+      for (int j = 0; j < VEC; ++j) acc[j] = R::apply(acc[j], R::pre(f[j], a.factor));
     }
   }
   // fold the waves of the block: lane-major layout keeps LDS accesses conflict-free
@@ -255,7 +287,7 @@ void reduce_outer_vec_kernel(OuterArgs a) {
     for (int k = 0; k < wy; ++k) s = R::apply(s, lds[(k * VEC + j) * kWave + lane]);
     if (col_ok) {
       if (a.rsplit == 1)
-        st_acc<OUT_T, float>(static_cast<OUT_T*>(a.out) + b * a.C + c + j, project<float>(s, a.factor, a.is_mean));
+        st_acc<OUT_T, float>(static_cast<OUT_T*>(a.out) + b * a.C + c + j, R::template post<float>(s, a.factor, a.is_mean));
       else
         static_cast<float*>(a.out)[(int64_t(split) * a.B + b) * a.C + c + j] = s;
     }
@@ -289,7 +321,7 @@ void reduce_fold_partials_kernel(const float* part, OUT_T* out, int nparts, int6
   __syncthreads();
   if (w == 0 && i < n) {
     const float s = R::apply(R::apply(lds[0][lane], lds[1][lane]), R::apply(lds[2][lane], lds[3][lane]));
-    st_acc<OUT_T, float>(out + i, project<float>(s, factor, is_mean));
+    st_acc<OUT_T, float>(out + i, R::template post<float>(s, factor, is_mean));
   }
 }
 
@@ -303,8 +335,8 @@ void reduce_outer_scalar_kernel(const T* in, OUT_T* out, int64_t B, int64_t NR, 
   const int64_t b = i / C, c = i - b * C;
   const T* p = in + b * b_stride + c;
   ACC acc = R::template identity<ACC>();
-  for (int64_t r = 0; r < NR; ++r) acc = R::template apply<ACC>(acc, ld_acc<T, ACC>(p + r * r_stride));
-  st_acc<OUT_T, ACC>(out + i, project<ACC>(acc, factor, is_mean));
+  for (int64_t r = 0; r < NR; ++r) acc = R::template apply<ACC>(acc, R::template pre<ACC>(ld_acc<T, ACC>(p + r * r_stride), factor));
+  st_acc<OUT_T, ACC>(out + i, R::template post<ACC>(acc, factor, is_mean));
 }
 
 // ---------------------------------------------------------------------------
@@ -337,9 +369,9 @@ void reduce_generic_kernel(const T* in, OUT_T* out, GenericMeta m, float factor,
       off += (r - q * m.red_size[d]) * m.red_stride[d];
       r = q;
     }
-    acc = R::template apply<ACC>(acc, ld_acc<T, ACC>(in + off));
+    acc = R::template apply<ACC>(acc, R::template pre<ACC>(ld_acc<T, ACC>(in + off), factor));
   }
-  st_acc<OUT_T, ACC>(out + i, project<ACC>(acc, factor, is_mean));
+  st_acc<OUT_T, ACC>(out + i, R::template post<ACC>(acc, factor, is_mean));
 }
 
 // ---------------------------------------------------------------------------
@@ -634,11 +666,144 @@ static int reduce_typed(const ReducePlan& q, int in_dtype, int out_dtype, const 
 #undef HK_RED_SLOW
 }
 
+// p-norm over one dimension: floating types only
+template <typename R>
+static int norm_typed(const ReducePlan& q, int dtype, const void* in, void* out, float p, void* workspace,
+                      size_t workspace_bytes, hipStream_t st) {
+  switch (dtype) {
+    case HK_FLOAT32: return reduce_float_like<float, float, R>(q, in, out, p, 0, workspace, workspace_bytes, st);
+    case HK_BFLOAT16: return reduce_float_like<bf16, bf16, R>(q, in, out, p, 0, workspace, workspace_bytes, st);
+    case HK_FLOAT16: return reduce_float_like<fp16, fp16, R>(q, in, out, p, 0, workspace, workspace_bytes, st);
+    case HK_FLOAT64: return reduce_slow<double, double, double, R>(q, in, out, p, 0, st);
+    default:
+      set_last_error("hk_norm: not implemented for dtype %d", dtype);
+      return HK_ERR_UNSUPPORTED;
+  }
+}
+
+// Gradient of the p-norm over the middle dimension of a dense [before, reduce, after] array
+// (norm_gradient_kernel, Norm1.cu:59-97): with n = the norm and g = its gradient of the slice,
+//   p = 1: sign(x) * g;   p = 2: g * x / n;   p > 2: x * |x|^(p-2) * g / n^(p-1);   0 where n == 0.
+template <typename T, typename CT>
+__global__ __launch_bounds__(256)
+void norm_grad_kernel(const T* __restrict__ x, const T* __restrict__ norm, const T* __restrict__ grad, T* out,
+                      int64_t total, int64_t reduce_size, int64_t after, int64_t p) {
+  const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t b = i / (reduce_size * after);
+  const int64_t a = i % after;
+  const int64_t y = b * after + a;
+  const CT xv = CT(Cvt<T>::load(x + i)), g = CT(Cvt<T>::load(grad + y));
+  CT o;
+  if (p == 1) {
+    o = (xv == CT(0) ? CT(0) : (xv < CT(0) ? CT(-1) : CT(1))) * g;
+  } else {
+    const CT n = CT(Cvt<T>::load(norm + y));
+    if (n == CT(0)) o = CT(0);
+    else if (p == 2) o = g * xv / n;
+    else o = xv * CT(pow(double(abs_of(xv)), double(p - 2))) * g / CT(pow(double(n), double(p - 1)));
+  }
+  Cvt<T>::store(out + i, o);
+}
+
+// the same for a norm over the last dimension (after == 1), one 16-byte vector per thread
+template <typename T>
+__global__ __launch_bounds__(256)
+void norm_grad_rows_vec_kernel(const T* __restrict__ x, const T* __restrict__ norm, const T* __restrict__ grad,
+                               T* out, uint32_t nvec, uint32_t cols_vec, int64_t p) {
+  constexpr int VEC = VecIO<T>::N;
+  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+  if (v >= nvec) return;
+  const uint32_t r = v / cols_vec;
+  const u32x4 raw = ld16(x + size_t(v) * VEC);
+  const float g = Cvt<T>::load(grad + r);
+  const float n = Cvt<T>::load(norm + r);
+  float f[VEC];
+  VecIO<T>::unpack(raw, f);
+  if (p == 1) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) f[j] = (f[j] == 0.f ? 0.f : (f[j] < 0.f ? -1.f : 1.f)) * g;
+  } else if (n == 0.f) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) f[j] = 0.f;
+  } else if (p == 2) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) f[j] = g * f[j] / n;
+  } else {
+    const float scale = g / powf(n, float(p - 1));
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) f[j] = f[j] * powf(fabsf(f[j]), float(p - 2)) * scale;
+  }
+  st16_stream(out + size_t(v) * VEC, VecIO<T>::pack(f));
+}
+
+template <typename T>
+static int norm_grad_typed(const void* x, const void* norm, const void* grad, void* out, int64_t before,
+                           int64_t reduce_size, int64_t after, int64_t p, hipStream_t s) {
+  const int64_t total = before * reduce_size * after;
+  using CT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
+  if constexpr (!std::is_same<T, double>::value) {
+    constexpr int VEC = VecIO<T>::N;
+    if (after == 1 && reduce_size % VEC == 0 && aligned16(x) && aligned16(out) && total / VEC < 0x7fffffffLL) {
+      const uint32_t nvec = uint32_t(total / VEC);
+      profile_before(s);
+      hipLaunchKernelGGL((norm_grad_rows_vec_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
+                         static_cast<const T*>(x), static_cast<const T*>(norm), static_cast<const T*>(grad),
+                         static_cast<T*>(out), nvec, uint32_t(reduce_size / VEC), p);
+      profile_after(s);
+      return launch_check("norm_grad_rows_vec_kernel");
+    }
+  }
+  HK_REQUIRE((total + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_norm_bwd: array too large");
+  profile_before(s);
+  hipLaunchKernelGGL((norm_grad_kernel<T, CT>), dim3(unsigned((total + 255) / 256)), dim3(256), 0, s,
+                     static_cast<const T*>(x), static_cast<const T*>(norm), static_cast<const T*>(grad),
+                     static_cast<T*>(out), total, reduce_size, after, p);
+  profile_after(s);
+  return launch_check("norm_grad_kernel");
+}
+
 } // namespace hk
 
 using namespace hk;
 
 extern "C" {
+
+int hk_norm(int dtype, const void* in, void* out, int ndim, const int64_t* shape, const int64_t* strides,
+            int64_t dim, int64_t p, void* workspace, size_t workspace_bytes, hkStream_t stream) {
+  HK_REQUIRE(p >= 1, HK_ERR_INVALID, "hk_norm: p must be at least 1, got %lld", (long long) p);
+  HK_REQUIRE(dim >= 0 && dim < ndim, HK_ERR_INVALID, "hk_norm: dim %lld outside [0, %d)", (long long) dim, ndim);
+  ReducePlan q;
+  int rc = make_plan(ndim, shape, strides, 1, &dim, &q, "hk_norm");
+  if (rc != HK_OK) return rc;
+  if (q.kind == PLAN_EMPTY) return HK_OK;
+  HK_REQUIRE(out, HK_ERR_INVALID, "hk_norm: null output");
+  HK_REQUIRE(in || q.n_red == 0, HK_ERR_INVALID, "hk_norm: null input");
+  HK_REQUIRE((q.n_out + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_norm: output too large");
+  if (q.kind == PLAN_COPYLIKE || q.n_red == 0) q.kind = PLAN_GENERIC;   // extent 0 or 1: one thread per output
+  hipStream_t st = as_hip(stream);
+  if (p == 1) return norm_typed<RNorm1>(q, dtype, in, out, 1.f, workspace, workspace_bytes, st);
+  if (p == 2) return norm_typed<RNorm2>(q, dtype, in, out, 2.f, workspace, workspace_bytes, st);
+  return norm_typed<RNormP>(q, dtype, in, out, float(p), workspace, workspace_bytes, st);
+}
+
+int hk_norm_bwd(int dtype, const void* in, const void* norm, const void* grad, void* out, int64_t before,
+                int64_t reduce_size, int64_t after, int64_t p, hkStream_t stream) {
+  HK_REQUIRE(p >= 1, HK_ERR_INVALID, "hk_norm_bwd: p must be at least 1, got %lld", (long long) p);
+  HK_REQUIRE(before >= 0 && reduce_size >= 0 && after >= 0, HK_ERR_INVALID, "hk_norm_bwd: negative shape");
+  if (before == 0 || reduce_size == 0 || after == 0) return HK_OK;
+  HK_REQUIRE(in && grad && out && (norm || p == 1), HK_ERR_INVALID, "hk_norm_bwd: null input/output");
+  hipStream_t s = as_hip(stream);
+  switch (dtype) {
+    case HK_FLOAT32: return norm_grad_typed<float>(in, norm, grad, out, before, reduce_size, after, p, s);
+    case HK_BFLOAT16: return norm_grad_typed<bf16>(in, norm, grad, out, before, reduce_size, after, p, s);
+    case HK_FLOAT16: return norm_grad_typed<fp16>(in, norm, grad, out, before, reduce_size, after, p, s);
+    case HK_FLOAT64: return norm_grad_typed<double>(in, norm, grad, out, before, reduce_size, after, p, s);
+    default:
+      set_last_error("hk_norm_bwd: not implemented for dtype %d", dtype);
+      return HK_ERR_UNSUPPORTED;
+  }
+}
 
 int hk_reduce_workspace_bytes(int in_dtype, int ndim, const int64_t* shape, const int64_t* strides,
                               int naxes, const int64_t* axes, size_t* bytes) {

@@ -352,6 +352,29 @@ int ht_ndarray_unary(int op, const HtArray* in, HtArray* out, int in_place, int 
   });
 }
 
+int ht_norm(const HtArray* input, HtArray* output, int64_t dim, int64_t p, int stream_index) {
+  return guarded([&] {
+    NDArray o = wrap(output);
+    hetu::impl::NormCuda(wrap(input), o, dim, p, stream_of(input, stream_index));
+  });
+}
+
+int ht_norm_gradient(const HtArray* input, const HtArray* output, const HtArray* output_grad, HtArray* input_grad,
+                     int64_t dim, int64_t p, int stream_index) {
+  return guarded([&] {
+    NDArray g = wrap(input_grad);
+    hetu::impl::NormGradientCuda(wrap(input), wrap(output), wrap(output_grad), g, dim, p,
+                                 stream_of(input, stream_index));
+  });
+}
+
+int ht_ndarray_norm(const HtArray* input, int64_t p, int64_t dim, int keepdim, HtArray* out, int stream_index) {
+  return guarded([&] {
+    NDArray r = NDArray::norm(wrap(input), p, dim, keepdim != 0, stream_index);
+    copy_out(r, out, stream_of(input, stream_index));
+  });
+}
+
 int ht_vocab_parallel_cross_entropy(const HtArray* vocab_parallel_logits, const HtArray* labels,
                                     int64_t vocab_start_index, int64_t vocab_end_index, int64_t ignored_index,
                                     HtArray* predicted_logits_partial, HtArray* log_sum_exp_logits,

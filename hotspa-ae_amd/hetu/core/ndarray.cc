@@ -293,6 +293,23 @@ HT_NDARRAY_UNARY(exp, Exp)
 HT_NDARRAY_UNARY(log, Log)
 #undef HT_NDARRAY_UNARY
 
+NDArray NDArray::norm(const NDArray& input, int64_t p, int64_t dim, bool keepdim, StreamIndex stream_id,
+                      NDArray& output) {
+  NDArray out;
+  if (output.is_defined()) {
+    out = output;
+  } else {
+    HTShape outshape = input->shape();
+    const int64_t axi = NDArrayMeta::ParseAxis(dim, int64_t(outshape.size()));
+    if (keepdim) outshape[axi] = 1;
+    else outshape.erase(outshape.begin() + axi);
+    out = NDArray::empty(outshape, input->device(), input->dtype(), stream_id);
+  }
+  Stream stream(input->device(), stream_id);
+  HT_DISPATCH_KERNEL_CPU_AND_CUDA(input->device().type(), __FUNCTION__, hetu::impl::Norm, input, out, dim, p, stream);
+  return out;
+}
+
 NDArray NDArray::softmax(const NDArray& input, int64_t dim, StreamIndex stream_id, NDArray& output) {
   NDArray out = output.is_defined() ? output : NDArray::empty_like(input, stream_id);
   Stream stream(input->device(), stream_id);

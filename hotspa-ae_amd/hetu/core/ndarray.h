@@ -180,6 +180,10 @@ class NDArray {
   static NDArray exp(const NDArray& input, StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY);
   static NDArray log(const NDArray& input, StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY);
 
+  // p-norm over one dimension (hetu/core/ndarray.cc:1259-1279 of the reference)
+  static NDArray norm(const NDArray& input, int64_t p = 1, int64_t dim = 0, bool keepdim = false,
+                      StreamIndex stream_id = DEFAULT_STREAM, NDArray& output = EMPTY);
+
   static NDArray softmax(const NDArray& input, int64_t dim, StreamIndex stream_id = DEFAULT_STREAM,
                          NDArray& output = EMPTY);
   static NDArray sceloss(const NDArray& preds, const NDArray& labels, ReductionType reduction = kMEAN,

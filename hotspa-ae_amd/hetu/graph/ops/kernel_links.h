@@ -84,6 +84,10 @@ DECLARE_KERNEL_CPU_AND_CUDA(Exp, const NDArray&, NDArray&, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(Log, const NDArray&, NDArray&, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(Opposite, const NDArray&, NDArray&, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(Sqrt, const NDArray&, NDArray&, const Stream&);
+// input, output, dim, p  /  input, output (the norm), output_grad, input_grad, dim, p   (kernel_links.h:244-247)
+DECLARE_KERNEL_CPU_AND_CUDA(Norm, const NDArray&, NDArray&, int64_t, int64_t, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(NormGradient, const NDArray&, const NDArray&, const NDArray&, NDArray&, int64_t, int64_t,
+                            const Stream&);
 // vocab_parallel_logits, labels, vocab_start_index, vocab_end_index, ignored_index, predicted_logits_partial,
 // log_sum_exp_logits
 DECLARE_KERNEL_CUDA(VocabParallelCrossEntropy, const NDArray&, const NDArray&, const int64_t, const int64_t,

@@ -224,6 +224,18 @@ def vocab_parallel_cross_entropy_gradient(softmax, labels, vocab_start, vocab_en
           _i64(vocab_end), _i64(ignored_index), desc(grad_loss), desc(out), ctypes.c_int(stream))
 
 
+def norm(x, out, dim, p, stream=DEFAULT_STREAM):
+    _call("ht_norm", desc(x), desc(out), _i64(dim), _i64(p), ctypes.c_int(stream))
+
+
+def norm_gradient(x, norm_out, grad, dx, dim, p, stream=DEFAULT_STREAM):
+    _call("ht_norm_gradient", desc(x), desc(norm_out), desc(grad), desc(dx), _i64(dim), _i64(p), ctypes.c_int(stream))
+
+
+def ndarray_norm(x, p, dim, keepdim, out, stream=DEFAULT_STREAM):
+    _call("ht_ndarray_norm", desc(x), _i64(p), _i64(dim), ctypes.c_int(int(keepdim)), desc(out), ctypes.c_int(stream))
+
+
 def set_random_seed(seed):
     _call("ht_set_random_seed", ctypes.c_uint64(seed))
 

@@ -127,6 +127,12 @@ HT_API int ht_unary(int op, const HtArray* in, HtArray* out, int stream_index);
 HT_API int ht_ndarray_binary(int op, const HtArray* a, const HtArray* b, HtArray* out, int in_place,
                              int stream_index);
 HT_API int ht_ndarray_unary(int op, const HtArray* in, HtArray* out, int in_place, int stream_index);
+/* NormCuda / NormGradientCuda (hetu/impl/kernel/Norm1.cu:99-186) and NDArray::norm (result copied into `out`) */
+HT_API int ht_norm(const HtArray* input, HtArray* output, int64_t dim, int64_t p, int stream_index);
+HT_API int ht_norm_gradient(const HtArray* input, const HtArray* output, const HtArray* output_grad,
+                            HtArray* input_grad, int64_t dim, int64_t p, int stream_index);
+HT_API int ht_ndarray_norm(const HtArray* input, int64_t p, int64_t dim, int keepdim, HtArray* out,
+                           int stream_index);
 /* VocabParallelCrossEntropyCuda / VocabParallelCrossEntropyGradientCuda
  * (hetu/impl/kernel/VocabParallelCrossEntropyLoss.cu:38-64, 94-119) */
 HT_API int ht_vocab_parallel_cross_entropy(const HtArray* vocab_parallel_logits, const HtArray* labels,

@@ -442,6 +442,20 @@ HK_API int hk_reduce(int in_dtype, int out_dtype, const void* in, void* out, int
                      const int64_t* axes, int op, void* workspace, size_t workspace_bytes,
                      hkStream_t stream);
 
+/* p-norm over one dimension, out = (sum_k |x|^p)^(1/p), p >= 1 an integer, floating types; the reduction
+ * runs on hk_reduce's planner and kernels (same shape / strides / workspace rules, workspace from
+ * hk_reduce_workspace_bytes with that one axis), accumulating in fp32 for the 16-bit types.
+ * Replaces NormCuda (hetu/impl/kernel/Norm1.cu:99-133).
+ * Gradient over the middle dimension of a dense [before, reduce_size, after] array; norm and grad are dense
+ * [before, after]: p = 1: sign(x) g;  p = 2: g x / norm;  p > 2: x |x|^(p-2) g / norm^(p-1);  0 where norm == 0.
+ * Replaces NormGradientCuda (Norm1.cu:135-186). */
+HK_API int hk_norm(int dtype, const void* in, void* out, int ndim, const int64_t* shape,
+                   const int64_t* strides, int64_t dim, int64_t p, void* workspace,
+                   size_t workspace_bytes, hkStream_t stream);
+HK_API int hk_norm_bwd(int dtype, const void* in, const void* norm, const void* grad, void* out,
+                       int64_t before, int64_t reduce_size, int64_t after, int64_t p,
+                       hkStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

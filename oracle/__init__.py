@@ -249,3 +249,25 @@ def nll_loss_bwd(labels, grad_loss, cols):
     ok = (lab >= 0) & (lab < cols)
     out[np.arange(rows)[ok], lab[ok]] = -g[ok] * cols
     return out
+
+
+def norm_p_fwd(x, dim, p):
+    """(sum_k |x|^p)^(1/p) over `dim` (norm_kernel, hetu/impl/kernel/Norm1.cu:17-56), float64."""
+    x = np.asarray(x, dtype=np.float64)
+    return (np.abs(x) ** p).sum(axis=dim) ** (1.0 / p)
+
+
+def norm_p_bwd(x, norm, grad, dim, p):
+    """norm_gradient_kernel (Norm1.cu:59-97): p = 1: sign(x) g; p = 2: g x / n; p > 2: x |x|^(p-2) g / n^(p-1);
+    0 where the norm is 0 (p >= 2)."""
+    x = np.asarray(x, dtype=np.float64)
+    n = np.expand_dims(np.asarray(norm, dtype=np.float64), dim)
+    g = np.expand_dims(np.asarray(grad, dtype=np.float64), dim)
+    if p == 1:
+        return np.sign(x) * g
+    safe = np.where(n == 0, 1.0, n)
+    if p == 2:
+        out = g * x / safe
+    else:
+        out = x * np.abs(x) ** (p - 2) * g / safe ** (p - 1)
+    return np.where(n == 0, 0.0, out)

@@ -809,3 +809,38 @@ def test_vocab_parallel_cross_entropy_entry_points(ops, cuda):
         ops.vocab_parallel_cross_entropy(tl, tlab, start, start + cols - 1, ignored, picked, lse)
     with pytest.raises(ops.AssertionError_, match="int64"):
         ops.vocab_parallel_cross_entropy(tl, tlab.int(), start, start + cols, ignored, picked, lse)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("p", [1, 2, 3])
+def test_norm_and_gradient_entry_points(ops, cuda, dtype, p):
+    import torch
+    shape, dim = (6, 40, 64), -2
+    x = helpers.draw(70 + p, shape, dtype=dtype)
+    want = oracle.norm_p_fwd(x, 1, p)
+    tx = helpers.to_torch(x, dtype, cuda)
+    out = torch.empty(6, 64, dtype=tx.dtype, device=cuda)
+    _sync_in()
+    ops.norm(tx, out, dim, p)
+    ops.stream_sync()
+    helpers.assert_close(out, want, dtype, "norm")
+    keep = torch.empty(6, 1, 64, dtype=tx.dtype, device=cuda)
+    ops.ndarray_norm(tx, p, dim, True, keep)              # NDArray::norm with keepdim
+    assert torch.equal(keep.view(6, 64), out)
+    grad = helpers.draw(80, (6, 64), dtype=dtype)
+    want_g = oracle.norm_p_bwd(x, helpers.to_numpy(out).astype(np.float64), grad, 1, p)
+    dx = torch.empty_like(tx)
+    _sync_in()
+    ops.norm_gradient(tx, out, helpers.to_torch(grad, dtype, cuda), dx, dim, p)
+    ops.stream_sync()
+    helpers.assert_close(dx, want_g, dtype, "gradient")
+    # a permuted view as input: the forward plans on strides, the gradient makes its operands dense
+    tv = tx.permute(2, 0, 1)
+    out2 = torch.empty(64, 6, dtype=tx.dtype, device=cuda)
+    ops.norm(tv, out2, 2, p)
+    ops.stream_sync()
+    helpers.assert_close(out2, want.T, dtype, "norm of a view")
+    with pytest.raises(ops.ValueError_, match="at least 1"):
+        ops.norm(tx, out, dim, 0)
+    with pytest.raises(ops.AssertionError_, match="does not hold"):
+        ops.norm(tx, out[:, :63].contiguous(), dim, p)

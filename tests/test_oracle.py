@@ -366,3 +366,26 @@ def test_refcpu_ports_match_oracle():
     out1 = np.empty(rows, np.float32); out0 = np.empty(cols, np.float32)
     lib.refcpu_reduce_sum_axis1_f32(P(x), R, C, P(out1)); lib.refcpu_reduce_sum_axis0_f32(P(x), R, C, P(out0))
     assert np.allclose(out1, x.astype(np.float64).sum(1), atol=1e-3) and np.allclose(out0, x.astype(np.float64).sum(0), atol=1e-3)
+
+
+@pytest.mark.parametrize("p", [1, 2, 3, 4])
+@pytest.mark.parametrize("dim", [0, 1, 2])
+def test_p_norm_against_torch_autograd(p, dim):
+    """oracle.norm_p_fwd / norm_p_bwd against torch.linalg.vector_norm and its float64 autograd (an independent
+    implementation); the zero slice by the definition (gradient 0, sign(0) = 0)."""
+    import torch
+    g = np.random.default_rng(10 * p + dim)
+    x = g.standard_normal((4, 5, 6))
+    x[1, 2, 3] = 0.0                      # an exact zero inside a non-zero slice
+    grad = g.standard_normal(tuple(s for i, s in enumerate(x.shape) if i != dim))
+    n = oracle.norm_p_fwd(x, dim, p)
+    tx = torch.tensor(x, requires_grad=True)
+    tn = torch.linalg.vector_norm(tx, ord=p, dim=dim)
+    np.testing.assert_allclose(n, tn.detach().numpy(), rtol=1e-13)
+    (tn * torch.tensor(grad)).sum().backward()
+    np.testing.assert_allclose(oracle.norm_p_bwd(x, n, grad, dim, p), tx.grad.numpy(), rtol=1e-11, atol=1e-13)
+    z = np.zeros((2, 3, 4))
+    nz = oracle.norm_p_fwd(z, dim, p)
+    assert (nz == 0).all()
+    gz = np.ones(nz.shape)
+    assert (oracle.norm_p_bwd(z, nz, gz, dim, p) == 0).all()

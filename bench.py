@@ -249,6 +249,26 @@ def case_elementwise(hk, torch, nsets, which):
         2 * n * 2 + rows * 14, rows
 
 
+def case_batch_norm(hk, torch, nsets, which):
+    """Spatial batch norm in training mode, bf16 [256, 256, 56, 56]: statistics pass + element-wise pass
+    (forward: x read twice, y written once; backward: dy and x read twice, dx written once)."""
+    shape = (256, 256, 56, 56)
+    bf = torch.bfloat16
+    n = 256 * 256 * 56 * 56
+    xs = [_randn(torch, shape, bf, 1.5, 821 + i) for i in range(2)]
+    ys = [torch.empty(shape, dtype=bf, device="cuda") for _ in range(2)]
+    scale = _uniform(torch, (256,), torch.float32, 0.5, 1.5, 822)
+    bias = _randn(torch, (256,), torch.float32, 1.0, 823)
+    rm, rv = torch.zeros(256, device="cuda"), torch.ones(256, device="cuda")
+    sm, si = torch.empty(256, device="cuda"), torch.empty(256, device="cuda")
+    hk.batch_norm_fwd(xs[0], scale, bias, ys[0], 0.1, 1e-5, rm, rv, sm, si)
+    if which == "fwd":
+        return (lambda i: hk.batch_norm_fwd(xs[i % 2], scale, bias, ys[i % 2], 0.1, 1e-5, rm, rv, sm, si)), 3 * n * 2, 256
+    dys = [_randn(torch, shape, bf, 1.0, 825 + i) for i in range(2)]
+    ds, db = torch.empty(256, device="cuda"), torch.empty(256, device="cuda")
+    return (lambda i: hk.batch_norm_bwd(dys[i % 2], xs[i % 2], scale, ys[i % 2], ds, db, sm, si)), 5 * n * 2, 256
+
+
 def case_reduce(hk, torch, nsets, axes, op, three_d=False):
     rows, cols = 32768, 4096
     bf = torch.bfloat16
@@ -319,6 +339,8 @@ CASES = [
     ("next: vocab-parallel CE bwd bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "vce")),
     ("next: vocab-parallel CE fused stats bf16 [16384x32000] (read only)", lambda hk, t, n: case_elementwise(hk, t, n, "stats")),
     ("next: vocab-parallel CE fused bwd bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "fused")),
+    ("next: batch norm fwd bf16 [256,256,56,56] (2R+1W, 3 launches)", lambda hk, t, n: case_batch_norm(hk, t, n, "fwd")),
+    ("next: batch norm bwd bf16 [256,256,56,56] (4R+1W, 3 launches)", lambda hk, t, n: case_batch_norm(hk, t, n, "bwd")),
     ("C4 rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "fwd")),
     ("C4 rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "bwd")),
     ("C5 sce fwd bf16 [16384x32000]", lambda hk, t, n: case_sce(hk, t, 2, "fwd")),

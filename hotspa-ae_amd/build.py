@@ -20,7 +20,7 @@ OBJ = os.path.join(HERE, "build")
 INCLUDE = os.path.join(ROOT, "include")
 
 HIP_SOURCES = ["hk_device.hip", "hk_norm.hip", "hk_softmax.hip", "hk_sce.hip", "hk_reduce.hip", "hk_nll.hip",
-               "hk_dropout_ln.hip", "hk_elementwise.hip", "hk_vocab_ce.hip"]
+               "hk_dropout_ln.hip", "hk_elementwise.hip", "hk_vocab_ce.hip", "hk_batchnorm.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fvisibility=hidden",

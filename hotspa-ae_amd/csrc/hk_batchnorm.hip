@@ -1,0 +1,411 @@
+// Spatial batch normalisation of an NCHW array in training mode, forward and
+// backward, with the semantics of cuDNN's cudnnBatchNormalizationForwardTraining /
+// cudnnBatchNormalizationBackward in CUDNN_BATCHNORM_SPATIAL mode (what the
+// reference calls): per channel over N, H, W.
+//
+// A channel's data is N runs of H*W contiguous elements, C*H*W apart.  Three
+// launches each way: (1) per-channel partial statistics from several workgroups
+// per channel, (2) a one-thread-per-channel merge that also writes the saved /
+// running statistics and the per-channel coefficients, (3) an element-wise pass,
+// one 16-byte vector per thread.  The input is read twice and the output written
+// once in the forward; the backward reads dy and x twice and writes dx once.
+#include "hk_common.cuh"
+
+#include <algorithm>
+#include <type_traits>
+
+namespace hk {
+
+template <typename T> struct BnCT { using type = float; };
+template <> struct BnCT<double> { using type = double; };
+
+// V elements starting at p as compute-type values (V == 1: any alignment)
+template <typename T, int V, typename CT>
+__device__ __forceinline__ void bn_load(const T* p, CT* f) {
+  if constexpr (V == 1) {
+    f[0] = CT(Cvt<T>::load(p));
+  } else {
+    float t[V];
+    VecIO<T>::unpack(ld16(p), t);
+#pragma unroll
+    for (int j = 0; j < V; ++j) f[j] = t[j];
+  }
+}
+template <typename T, int V, typename CT>
+__device__ __forceinline__ void bn_store(T* p, const CT* f) {
+  if constexpr (V == 1) {
+    Cvt<T>::store(p, f[0]);
+  } else {
+    float t[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) t[j] = f[j];
+    st16_stream(p, VecIO<T>::pack(t));
+  }
+}
+
+struct BnShape {
+  int64_t N, C, HW;
+  int64_t hw_vec;         // HW / V
+  int64_t per_channel;    // N * hw_vec: loads of V elements per channel
+  int splits;
+};
+
+// address of load `v` (0 <= v < per_channel) of channel c
+__device__ __forceinline__ int64_t bn_offset(const BnShape& s, int64_t c, int64_t v, int V) {
+  const int64_t n = v / s.hw_vec;
+  const int64_t off = v - n * s.hw_vec;
+  return (n * s.C + c) * s.HW + off * V;
+}
+
+template <typename CT>
+__device__ __forceinline__ CT block_sum(CT v, CT* lds) {
+  const int tid = threadIdx.x;
+  lds[tid] = v;
+  __syncthreads();
+  for (int s = blockDim.x >> 1; s > 0; s >>= 1) {
+    if (tid < s) lds[tid] += lds[tid + s];
+    __syncthreads();
+  }
+  const CT r = lds[0];
+  __syncthreads();
+  return r;
+}
+
+// (count, mean, M2) of a slice of one channel -> part[(c * splits + split) * 3 ..]
+template <typename T, int V, typename CT>
+__global__ __launch_bounds__(256)
+void bn_stats_kernel(const T* __restrict__ x, BnShape s, CT* __restrict__ part) {
+  __shared__ CT lds[256];
+  const int64_t c = blockIdx.x;
+  const int split = blockIdx.y;
+  // per-thread Welford over whole loads: each load's V values are folded in as one group (Chan's update)
+  CT cnt = 0, mean = 0, m2 = 0;
+  for (int64_t v = int64_t(split) * 256 + threadIdx.x; v < s.per_channel; v += int64_t(s.splits) * 256) {
+    CT f[V];
+    bn_load<T, V, CT>(x + bn_offset(s, c, v, V), f);
+    CT gs = 0;
+#pragma unroll
+    for (int j = 0; j < V; ++j) gs += f[j];
+    const CT gm = gs / CT(V);
+    CT g2 = 0;
+#pragma unroll
+    for (int j = 0; j < V; ++j) { const CT d = f[j] - gm; g2 += d * d; }
+    const CT n = cnt + CT(V);
+    const CT delta = gm - mean;
+    mean += delta * (CT(V) / n);
+    m2 += g2 + delta * delta * (cnt * CT(V) / n);
+    cnt = n;
+  }
+  // block merge: total count and mean first, then M2 about the block mean
+  const CT bcnt = block_sum<CT>(cnt, lds);
+  const CT bsum = block_sum<CT>(mean * cnt, lds);
+  const CT bmean = bcnt > 0 ? bsum / bcnt : CT(0);
+  const CT d = mean - bmean;
+  const CT bm2 = block_sum<CT>(m2 + d * d * cnt, lds);
+  if (threadIdx.x == 0) {
+    CT* o = part + (c * s.splits + split) * 3;
+    o[0] = bcnt; o[1] = bmean; o[2] = bm2;
+  }
+}
+
+// One thread per channel: merge the slices; write the saved mean / inverse standard deviation, update the
+// running statistics (the running variance takes the unbiased estimate, as cuDNN does), and leave
+// coef[c] = scale * invstd, coef[C + c] = mean, coef[2 C + c] = bias for the element-wise pass.
+template <typename PT, typename CT>
+__global__ __launch_bounds__(256)
+void bn_finalize_kernel(const CT* __restrict__ part, int64_t C, int splits, const PT* __restrict__ scale,
+                        const PT* __restrict__ bias, double momentum, double eps, PT* running_mean,
+                        PT* running_var, PT* save_mean, PT* save_invstd, CT* __restrict__ coef) {
+  const int64_t c = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (c >= C) return;
+  CT cnt = 0, mean = 0, m2 = 0;
+  for (int k = 0; k < splits; ++k) {
+    const CT* p = part + (c * splits + k) * 3;
+    const CT nb = p[0];
+    if (nb <= 0) continue;
+    const CT n = cnt + nb;
+    const CT delta = p[1] - mean;
+    mean += delta * (nb / n);
+    m2 += p[2] + delta * delta * (cnt * nb / n);
+    cnt = n;
+  }
+  const CT var = cnt > 0 ? m2 / cnt : CT(0);
+  CT invstd;
+  if constexpr (std::is_same<CT, double>::value) invstd = 1.0 / sqrt(var + eps);
+  else invstd = 1.0f / sqrtf(var + float(eps));
+  if (save_mean) save_mean[c] = PT(mean);
+  if (save_invstd) save_invstd[c] = PT(invstd);
+  if (running_mean) running_mean[c] = PT((1.0 - momentum) * double(running_mean[c]) + momentum * double(mean));
+  if (running_var) {
+    const double unbiased = cnt > 1 ? double(m2) / (double(cnt) - 1.0) : double(var);
+    running_var[c] = PT((1.0 - momentum) * double(running_var[c]) + momentum * unbiased);
+  }
+  coef[c] = CT(scale[c]) * invstd;
+  coef[C + c] = mean;
+  coef[2 * C + c] = CT(bias[c]);
+}
+
+// y = (x - mean) * (scale * invstd) + bias; the mean is subtracted first: folding it into the constant term
+// would cancel badly for a channel whose mean is large against its spread
+template <typename T, int V, typename CT>
+__global__ __launch_bounds__(256)
+void bn_apply_kernel(const T* x, T* y, const CT* __restrict__ coef, int64_t total_loads, int64_t hw_vec, int64_t C) {
+  const int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (v >= total_loads) return;
+  const int64_t c = (v / hw_vec) % C;
+  const CT a = coef[c], mean = coef[C + c], b = coef[2 * C + c];
+  CT f[V];
+  bn_load<T, V, CT>(x + v * V, f);
+#pragma unroll
+  for (int j = 0; j < V; ++j) f[j] = (f[j] - mean) * a + b;
+  bn_store<T, V, CT>(y + v * V, f);
+}
+
+// per-channel partial sums of dy and dy * (x - mean) * invstd -> part[(c * splits + split) * 2 ..]
+template <typename T, int V, typename PT, typename CT>
+__global__ __launch_bounds__(256)
+void bn_bwd_stats_kernel(const T* __restrict__ dy, const T* __restrict__ x, BnShape s,
+                         const PT* __restrict__ save_mean, const PT* __restrict__ save_invstd,
+                         CT* __restrict__ part) {
+  __shared__ CT lds[256];
+  const int64_t c = blockIdx.x;
+  const int split = blockIdx.y;
+  const CT mean = CT(save_mean[c]), invstd = CT(save_invstd[c]);
+  CT sdy = 0, sdyx = 0;
+  for (int64_t v = int64_t(split) * 256 + threadIdx.x; v < s.per_channel; v += int64_t(s.splits) * 256) {
+    const int64_t off = bn_offset(s, c, v, V);
+    CT g[V], f[V];
+    bn_load<T, V, CT>(dy + off, g);
+    bn_load<T, V, CT>(x + off, f);
+#pragma unroll
+    for (int j = 0; j < V; ++j) { sdy += g[j]; sdyx += g[j] * ((f[j] - mean) * invstd); }
+  }
+  sdy = block_sum<CT>(sdy, lds);
+  sdyx = block_sum<CT>(sdyx, lds);
+  if (threadIdx.x == 0) {
+    CT* o = part + (c * s.splits + split) * 2;
+    o[0] = sdy; o[1] = sdyx;
+  }
+}
+
+// dscale = sum dy * xhat, dbias = sum dy; coefficients of dx = k0 * dy + k1 * (x - mean) + k2 with
+//   dx = scale * invstd * (dy - dbias / m - xhat * dscale / m),  xhat = (x - mean) * invstd
+template <typename PT, typename CT>
+__global__ __launch_bounds__(256)
+void bn_bwd_finalize_kernel(const CT* __restrict__ part, int64_t C, int splits, CT count,
+                            const PT* __restrict__ scale, const PT* __restrict__ save_mean,
+                            const PT* __restrict__ save_invstd, PT* dscale, PT* dbias, CT* __restrict__ coef) {
+  const int64_t c = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (c >= C) return;
+  CT sdy = 0, sdyx = 0;
+  for (int k = 0; k < splits; ++k) {
+    sdy += part[(c * splits + k) * 2];
+    sdyx += part[(c * splits + k) * 2 + 1];
+  }
+  if (dscale) dscale[c] = PT(sdyx);
+  if (dbias) dbias[c] = PT(sdy);
+  const CT mean = CT(save_mean[c]), invstd = CT(save_invstd[c]);
+  const CT a = CT(scale[c]) * invstd;
+  coef[c] = a;
+  coef[C + c] = -a * invstd * sdyx / count;
+  coef[2 * C + c] = -a * sdy / count;
+  coef[3 * C + c] = mean;
+}
+
+template <typename T, int V, typename CT>
+__global__ __launch_bounds__(256)
+void bn_bwd_apply_kernel(const T* dy, const T* x, T* dx, const CT* __restrict__ coef, int64_t total_loads,
+                         int64_t hw_vec, int64_t C) {
+  const int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (v >= total_loads) return;
+  const int64_t c = (v / hw_vec) % C;
+  const CT k0 = coef[c], k1 = coef[C + c], k2 = coef[2 * C + c], mean = coef[3 * C + c];
+  CT g[V], f[V];
+  bn_load<T, V, CT>(dy + v * V, g);
+  bn_load<T, V, CT>(x + v * V, f);
+#pragma unroll
+  for (int j = 0; j < V; ++j) g[j] = k0 * g[j] + (k1 * (f[j] - mean) + k2);
+  bn_store<T, V, CT>(dx + v * V, g);
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+static int bn_splits(int64_t C, int64_t per_channel) {
+  // enough workgroups to fill the chip (about 8 per compute unit), each with at least 8 loads per thread
+  const int64_t want = (int64_t(device_cu_count()) * 8 + C - 1) / C;
+  const int64_t most = std::max<int64_t>(1, per_channel / (256 * 8));
+  return int(std::max<int64_t>(1, std::min<int64_t>(std::min(want, most), 1024)));
+}
+
+template <int V>
+static BnShape bn_shape(int64_t N, int64_t C, int64_t HW) {
+  BnShape s{};
+  s.N = N; s.C = C; s.HW = HW;
+  s.hw_vec = HW / V;
+  s.per_channel = N * s.hw_vec;
+  s.splits = bn_splits(C, s.per_channel);
+  return s;
+}
+
+static size_t bn_ws_bytes(int64_t N, int64_t C, int64_t HW, size_t ct_size) {
+  // partials for the scalar decomposition (the larger one) + four coefficient rows
+  const BnShape s = bn_shape<1>(N, C, HW);
+  return (size_t(C) * size_t(s.splits) * 3 + size_t(C) * 4) * ct_size;
+}
+
+template <typename T, typename PT>
+static int bn_fwd_typed(const void* x, const void* scale, const void* bias, void* y, double momentum, double eps,
+                        void* running_mean, void* running_var, void* save_mean, void* save_invstd, int64_t N,
+                        int64_t C, int64_t HW, void* ws, hipStream_t st) {
+  using CT = typename BnCT<T>::type;
+  CT* part = static_cast<CT*>(ws);
+  const T* xp = static_cast<const T*>(x);
+  T* yp = static_cast<T*>(y);
+  bool vec = false;
+  if constexpr (!std::is_same<T, double>::value) {
+    vec = HW % VecIO<T>::N == 0 && aligned16(x) && aligned16(y);
+  }
+  auto run = [&](auto vtag) -> int {
+    constexpr int V = decltype(vtag)::value;
+    const BnShape s = bn_shape<V>(N, C, HW);
+    CT* coef = part + size_t(C) * size_t(s.splits) * 3;
+    HK_REQUIRE(C <= 0x7fffffffLL && (N * C * s.hw_vec + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID,
+               "hk_batch_norm_fwd: array too large");
+    hipLaunchKernelGGL((bn_stats_kernel<T, V, CT>), dim3(unsigned(C), unsigned(s.splits)), dim3(256), 0, st, xp, s, part);
+    int rc = launch_check("bn_stats_kernel");
+    if (rc != HK_OK) return rc;
+    hipLaunchKernelGGL((bn_finalize_kernel<PT, CT>), dim3(unsigned((C + 255) / 256)), dim3(256), 0, st, part, C,
+                       s.splits, static_cast<const PT*>(scale), static_cast<const PT*>(bias), momentum, eps,
+                       static_cast<PT*>(running_mean), static_cast<PT*>(running_var), static_cast<PT*>(save_mean),
+                       static_cast<PT*>(save_invstd), coef);
+    rc = launch_check("bn_finalize_kernel");
+    if (rc != HK_OK) return rc;
+    const int64_t loads = N * C * s.hw_vec;
+    profile_before(st);
+    hipLaunchKernelGGL((bn_apply_kernel<T, V, CT>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st, xp, yp,
+                       coef, loads, s.hw_vec, C);
+    profile_after(st);
+    return launch_check("bn_apply_kernel");
+  };
+  if constexpr (!std::is_same<T, double>::value) {
+    if (vec) return run(std::integral_constant<int, VecIO<T>::N>{});
+  }
+  return run(std::integral_constant<int, 1>{});
+}
+
+template <typename T, typename PT>
+static int bn_bwd_typed(const void* dy, const void* x, const void* scale, void* dx, void* dscale, void* dbias,
+                        const void* save_mean, const void* save_invstd, int64_t N, int64_t C, int64_t HW, void* ws,
+                        hipStream_t st) {
+  using CT = typename BnCT<T>::type;
+  CT* part = static_cast<CT*>(ws);
+  bool vec = false;
+  if constexpr (!std::is_same<T, double>::value) {
+    vec = HW % VecIO<T>::N == 0 && aligned16(x) && aligned16(dy) && aligned16(dx);
+  }
+  auto run = [&](auto vtag) -> int {
+    constexpr int V = decltype(vtag)::value;
+    const BnShape s = bn_shape<V>(N, C, HW);
+    CT* coef = part + size_t(C) * size_t(s.splits) * 3;
+    HK_REQUIRE(C <= 0x7fffffffLL && (N * C * s.hw_vec + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID,
+               "hk_batch_norm_bwd: array too large");
+    hipLaunchKernelGGL((bn_bwd_stats_kernel<T, V, PT, CT>), dim3(unsigned(C), unsigned(s.splits)), dim3(256), 0, st,
+                       static_cast<const T*>(dy), static_cast<const T*>(x), s, static_cast<const PT*>(save_mean),
+                       static_cast<const PT*>(save_invstd), part);
+    int rc = launch_check("bn_bwd_stats_kernel");
+    if (rc != HK_OK) return rc;
+    hipLaunchKernelGGL((bn_bwd_finalize_kernel<PT, CT>), dim3(unsigned((C + 255) / 256)), dim3(256), 0, st, part, C,
+                       s.splits, CT(N * HW), static_cast<const PT*>(scale), static_cast<const PT*>(save_mean),
+                       static_cast<const PT*>(save_invstd), static_cast<PT*>(dscale), static_cast<PT*>(dbias), coef);
+    rc = launch_check("bn_bwd_finalize_kernel");
+    if (rc != HK_OK) return rc;
+    const int64_t loads = N * C * s.hw_vec;
+    profile_before(st);
+    hipLaunchKernelGGL((bn_bwd_apply_kernel<T, V, CT>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st,
+                       static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<T*>(dx), coef, loads,
+                       s.hw_vec, C);
+    profile_after(st);
+    return launch_check("bn_bwd_apply_kernel");
+  };
+  if constexpr (!std::is_same<T, double>::value) {
+    if (vec) return run(std::integral_constant<int, VecIO<T>::N>{});
+  }
+  return run(std::integral_constant<int, 1>{});
+}
+
+static int bn_check(const char* who, int dtype, int64_t N, int64_t C, int64_t HW, const void* ws, size_t ws_bytes,
+                    size_t* need) {
+  HK_REQUIRE(N >= 0 && C >= 0 && HW >= 0, HK_ERR_INVALID, "%s: negative shape", who);
+  HK_REQUIRE(dtype == HK_FLOAT32 || dtype == HK_BFLOAT16 || dtype == HK_FLOAT16 || dtype == HK_FLOAT64,
+             HK_ERR_UNSUPPORTED, "%s: not implemented for dtype %d", who, dtype);
+  *need = bn_ws_bytes(N, C, HW, dtype == HK_FLOAT64 ? 8 : 4);
+  if (N * C * HW == 0) return HK_OK;
+  HK_REQUIRE(ws != nullptr && ws_bytes >= *need, HK_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given",
+             who, *need, ws_bytes);
+  HK_REQUIRE(aligned16(ws), HK_ERR_INVALID, "%s: workspace must be 16-byte aligned", who);
+  return HK_OK;
+}
+
+} // namespace hk
+
+using namespace hk;
+
+extern "C" {
+
+int hk_batch_norm_workspace_bytes(int dtype, int64_t N, int64_t C, int64_t HW, size_t* bytes) {
+  HK_REQUIRE(bytes, HK_ERR_INVALID, "hk_batch_norm_workspace_bytes: null output");
+  HK_REQUIRE(N >= 0 && C >= 0 && HW >= 0, HK_ERR_INVALID, "hk_batch_norm_workspace_bytes: negative shape");
+  *bytes = (N * C * HW == 0) ? 0 : bn_ws_bytes(N, C, HW, dtype == HK_FLOAT64 ? 8 : 4);
+  return HK_OK;
+}
+
+int hk_batch_norm_fwd(int dtype, const void* x, const void* scale, const void* bias, void* y, double momentum,
+                      double eps, void* running_mean, void* running_var, void* save_mean, void* save_invstd,
+                      int64_t N, int64_t C, int64_t HW, void* workspace, size_t workspace_bytes,
+                      hkStream_t stream) {
+  size_t need = 0;
+  int rc = bn_check("hk_batch_norm_fwd", dtype, N, C, HW, workspace, workspace_bytes, &need);
+  if (rc != HK_OK) return rc;
+  if (N * C * HW == 0) return HK_OK;
+  HK_REQUIRE(x && scale && bias && y, HK_ERR_INVALID, "hk_batch_norm_fwd: null input/output");
+  hipStream_t st = as_hip(stream);
+  switch (dtype) {
+    case HK_FLOAT32:
+      return bn_fwd_typed<float, float>(x, scale, bias, y, momentum, eps, running_mean, running_var, save_mean,
+                                        save_invstd, N, C, HW, workspace, st);
+    case HK_BFLOAT16:
+      return bn_fwd_typed<bf16, float>(x, scale, bias, y, momentum, eps, running_mean, running_var, save_mean,
+                                       save_invstd, N, C, HW, workspace, st);
+    case HK_FLOAT16:
+      return bn_fwd_typed<fp16, float>(x, scale, bias, y, momentum, eps, running_mean, running_var, save_mean,
+                                       save_invstd, N, C, HW, workspace, st);
+    default:
+      return bn_fwd_typed<double, double>(x, scale, bias, y, momentum, eps, running_mean, running_var, save_mean,
+                                          save_invstd, N, C, HW, workspace, st);
+  }
+}
+
+int hk_batch_norm_bwd(int dtype, const void* dy, const void* x, const void* scale, void* dx, void* dscale,
+                      void* dbias, const void* save_mean, const void* save_invstd, int64_t N, int64_t C,
+                      int64_t HW, void* workspace, size_t workspace_bytes, hkStream_t stream) {
+  size_t need = 0;
+  int rc = bn_check("hk_batch_norm_bwd", dtype, N, C, HW, workspace, workspace_bytes, &need);
+  if (rc != HK_OK) return rc;
+  if (N * C * HW == 0) return HK_OK;
+  HK_REQUIRE(dy && x && scale && dx && save_mean && save_invstd, HK_ERR_INVALID,
+             "hk_batch_norm_bwd: null input/output");
+  hipStream_t st = as_hip(stream);
+  switch (dtype) {
+    case HK_FLOAT32:
+      return bn_bwd_typed<float, float>(dy, x, scale, dx, dscale, dbias, save_mean, save_invstd, N, C, HW, workspace, st);
+    case HK_BFLOAT16:
+      return bn_bwd_typed<bf16, float>(dy, x, scale, dx, dscale, dbias, save_mean, save_invstd, N, C, HW, workspace, st);
+    case HK_FLOAT16:
+      return bn_bwd_typed<fp16, float>(dy, x, scale, dx, dscale, dbias, save_mean, save_invstd, N, C, HW, workspace, st);
+    default:
+      return bn_bwd_typed<double, double>(dy, x, scale, dx, dscale, dbias, save_mean, save_invstd, N, C, HW, workspace, st);
+  }
+}
+
+} // extern "C"

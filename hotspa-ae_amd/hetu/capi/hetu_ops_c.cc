@@ -352,6 +352,28 @@ int ht_ndarray_unary(int op, const HtArray* in, HtArray* out, int in_place, int 
   });
 }
 
+int ht_batch_norm(const HtArray* input_X, const HtArray* bn_scale, const HtArray* bn_bias, HtArray* output_Y,
+                  double momentum, double eps, HtArray* running_mean, HtArray* running_var, HtArray* save_mean,
+                  HtArray* save_var, int stream_index) {
+  return guarded([&] {
+    NDArray y = wrap(output_Y), rm = wrap(running_mean), rv = wrap(running_var), sm = wrap(save_mean),
+            sv = wrap(save_var);
+    hetu::impl::BatchNormCuda(wrap(input_X), wrap(bn_scale), wrap(bn_bias), y, momentum, eps, rm, rv, sm, sv,
+                              stream_of(input_X, stream_index));
+  });
+}
+
+int ht_batch_norm_gradient(const HtArray* gradient_Y, const HtArray* input_X, const HtArray* bn_scale,
+                           HtArray* gradient_X, HtArray* gradient_bn_scale, HtArray* gradient_bn_bias, double eps,
+                           HtArray* save_mean, HtArray* save_var, int stream_index) {
+  return guarded([&] {
+    NDArray dx = wrap(gradient_X), ds = wrap(gradient_bn_scale), db = wrap(gradient_bn_bias), sm = wrap(save_mean),
+            sv = wrap(save_var);
+    hetu::impl::BatchNormGradientCuda(wrap(gradient_Y), wrap(input_X), wrap(bn_scale), dx, ds, db, eps, sm, sv,
+                                      stream_of(input_X, stream_index));
+  });
+}
+
 int ht_norm(const HtArray* input, HtArray* output, int64_t dim, int64_t p, int stream_index) {
   return guarded([&] {
     NDArray o = wrap(output);

@@ -84,6 +84,12 @@ DECLARE_KERNEL_CPU_AND_CUDA(Exp, const NDArray&, NDArray&, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(Log, const NDArray&, NDArray&, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(Opposite, const NDArray&, NDArray&, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(Sqrt, const NDArray&, NDArray&, const Stream&);
+// input_X, bn_scale, bn_bias, output_Y, momentum, eps, running_mean, running_var, save_mean, save_var
+DECLARE_KERNEL_CPU_AND_CUDA(BatchNorm, const NDArray&, const NDArray&, const NDArray&, NDArray&, double, double,
+                            NDArray&, NDArray&, NDArray&, NDArray&, const Stream&);
+// gradient_Y, input_X, bn_scale, gradient_X, gradient_bn_scale, gradient_bn_bias, eps, save_mean, save_var
+DECLARE_KERNEL_CPU_AND_CUDA(BatchNormGradient, const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&,
+                            NDArray&, double, NDArray&, NDArray&, const Stream&);
 // input, output, dim, p  /  input, output (the norm), output_grad, input_grad, dim, p   (kernel_links.h:244-247)
 DECLARE_KERNEL_CPU_AND_CUDA(Norm, const NDArray&, NDArray&, int64_t, int64_t, const Stream&);
 DECLARE_KERNEL_CPU_AND_CUDA(NormGradient, const NDArray&, const NDArray&, const NDArray&, NDArray&, int64_t, int64_t,

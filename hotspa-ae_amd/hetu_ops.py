@@ -236,6 +236,17 @@ def ndarray_norm(x, p, dim, keepdim, out, stream=DEFAULT_STREAM):
     _call("ht_ndarray_norm", desc(x), _i64(p), _i64(dim), ctypes.c_int(int(keepdim)), desc(out), ctypes.c_int(stream))
 
 
+def batch_norm(x, scale, bias, y, momentum, eps, running_mean, running_var, save_mean, save_var,
+               stream=DEFAULT_STREAM):
+    _call("ht_batch_norm", desc(x), desc(scale), desc(bias), desc(y), ctypes.c_double(momentum), ctypes.c_double(eps),
+          desc(running_mean), desc(running_var), desc(save_mean), desc(save_var), ctypes.c_int(stream))
+
+
+def batch_norm_gradient(dy, x, scale, dx, dscale, dbias, eps, save_mean, save_var, stream=DEFAULT_STREAM):
+    _call("ht_batch_norm_gradient", desc(dy), desc(x), desc(scale), desc(dx), desc(dscale), desc(dbias),
+          ctypes.c_double(eps), desc(save_mean), desc(save_var), ctypes.c_int(stream))
+
+
 def set_random_seed(seed):
     _call("ht_set_random_seed", ctypes.c_uint64(seed))
 

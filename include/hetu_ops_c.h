@@ -127,6 +127,13 @@ HT_API int ht_unary(int op, const HtArray* in, HtArray* out, int stream_index);
 HT_API int ht_ndarray_binary(int op, const HtArray* a, const HtArray* b, HtArray* out, int in_place,
                              int stream_index);
 HT_API int ht_ndarray_unary(int op, const HtArray* in, HtArray* out, int in_place, int stream_index);
+/* BatchNormCuda / BatchNormGradientCuda (hetu/impl/kernel/BatchNorm.cu:8-83, 84-165) */
+HT_API int ht_batch_norm(const HtArray* input_X, const HtArray* bn_scale, const HtArray* bn_bias, HtArray* output_Y,
+                         double momentum, double eps, HtArray* running_mean, HtArray* running_var,
+                         HtArray* save_mean, HtArray* save_var, int stream_index);
+HT_API int ht_batch_norm_gradient(const HtArray* gradient_Y, const HtArray* input_X, const HtArray* bn_scale,
+                                  HtArray* gradient_X, HtArray* gradient_bn_scale, HtArray* gradient_bn_bias,
+                                  double eps, HtArray* save_mean, HtArray* save_var, int stream_index);
 /* NormCuda / NormGradientCuda (hetu/impl/kernel/Norm1.cu:99-186) and NDArray::norm (result copied into `out`) */
 HT_API int ht_norm(const HtArray* input, HtArray* output, int64_t dim, int64_t p, int stream_index);
 HT_API int ht_norm_gradient(const HtArray* input, const HtArray* output, const HtArray* output_grad,

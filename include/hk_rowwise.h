@@ -292,6 +292,30 @@ HK_API int hk_dropout_add_ln_bwd_ex_workspace_bytes(const hkDropoutAddLnBwdParam
 HK_API int hk_dropout_add_ln_bwd_ex(const hkDropoutAddLnBwdParams* params, hkStream_t stream);
 
 /* ======================================================================== *
+ * Spatial batch normalisation of a dense NCHW array (x viewed as [N, C, HW]) in
+ * training mode.  The reference calls cuDNN (>= 7) for this
+ * (hetu/impl/kernel/BatchNorm.cu:8-83, 84-165: cudnnBatchNormalizationForwardTraining /
+ * cudnnBatchNormalizationBackward, CUDNN_BATCHNORM_SPATIAL); cuDNN is not part of
+ * the reference's sources, so the arithmetic here restates its documented one:
+ *   mean_c, var_c over N, H, W (biased);  y = scale (x - mean) / sqrt(var + eps) + bias;
+ *   running_mean = (1 - momentum) running_mean + momentum mean;
+ *   running_var  = (1 - momentum) running_var  + momentum var * m / (m - 1)   (m = N*HW);
+ *   save_mean = mean,  save_invstd = 1 / sqrt(var + eps)   (the reference names this output save_var);
+ *   dscale = sum dy xhat,  dbias = sum dy,  dx = scale invstd (dy - dbias / m - xhat dscale / m).
+ * scale, bias, running_*, save_*, dscale, dbias are fp32 for fp16 / bf16 data and of the data type otherwise
+ * (BatchNorm.cu:55-70).  running_* and save_* may be NULL in the forward, dscale / dbias in the backward.
+ * ======================================================================== */
+HK_API int hk_batch_norm_workspace_bytes(int dtype, int64_t N, int64_t C, int64_t HW, size_t* bytes);
+HK_API int hk_batch_norm_fwd(int dtype, const void* x, const void* scale, const void* bias, void* y,
+                             double momentum, double eps, void* running_mean, void* running_var,
+                             void* save_mean, void* save_invstd, int64_t N, int64_t C, int64_t HW,
+                             void* workspace, size_t workspace_bytes, hkStream_t stream);
+HK_API int hk_batch_norm_bwd(int dtype, const void* dy, const void* x, const void* scale, void* dx,
+                             void* dscale, void* dbias, const void* save_mean, const void* save_invstd,
+                             int64_t N, int64_t C, int64_t HW, void* workspace, size_t workspace_bytes,
+                             hkStream_t stream);
+
+/* ======================================================================== *
  * Softmax along one dimension of a dense array viewed as [outer, dim, inner].
  * Replaces SoftmaxCuda (hetu/impl/kernel/Softmax.cu:250-310) and
  * SoftmaxGradientCuda (Softmax.cu:364-404): dx = dy*y - y*sum(dy*y).

@@ -271,3 +271,41 @@ def norm_p_bwd(x, norm, grad, dim, p):
     else:
         out = x * np.abs(x) ** (p - 2) * g / safe ** (p - 1)
     return np.where(n == 0, 0.0, out)
+
+
+def batch_norm_fwd(x, scale, bias, running_mean, running_var, momentum, eps):
+    """Spatial batch normalisation in training mode as cuDNN documents it for
+    cudnnBatchNormalizationForwardTraining(CUDNN_BATCHNORM_SPATIAL) (called at
+    hetu/impl/kernel/BatchNorm.cu:55-70; cuDNN itself is not among the reference's sources): statistics per
+    channel over every other dimension, biased variance in y, unbiased variance into the running average,
+    inverse standard deviation saved.  Returns y, new running mean, new running var, save_mean, save_invstd."""
+    x = np.asarray(x, dtype=np.float64)
+    axes = tuple(i for i in range(x.ndim) if i != 1)
+    m = x.size // x.shape[1]
+    mean = x.mean(axis=axes)
+    var = x.var(axis=axes)
+    shape = [1, -1] + [1] * (x.ndim - 2)
+    invstd = 1.0 / np.sqrt(var + eps)
+    y = (x - mean.reshape(shape)) * (invstd * np.asarray(scale, np.float64)).reshape(shape) \
+        + np.asarray(bias, np.float64).reshape(shape)
+    unbiased = var * m / (m - 1) if m > 1 else var
+    rm = (1 - momentum) * np.asarray(running_mean, np.float64) + momentum * mean
+    rv = (1 - momentum) * np.asarray(running_var, np.float64) + momentum * unbiased
+    return y, rm, rv, mean, invstd
+
+
+def batch_norm_bwd(dy, x, scale, save_mean, save_invstd):
+    """cudnnBatchNormalizationBackward (BatchNorm.cu:139-153): dscale = sum dy xhat, dbias = sum dy,
+    dx = scale invstd (dy - dbias / m - xhat dscale / m)."""
+    dy = np.asarray(dy, dtype=np.float64); x = np.asarray(x, dtype=np.float64)
+    axes = tuple(i for i in range(x.ndim) if i != 1)
+    m = x.size // x.shape[1]
+    shape = [1, -1] + [1] * (x.ndim - 2)
+    mean = np.asarray(save_mean, np.float64).reshape(shape)
+    invstd = np.asarray(save_invstd, np.float64).reshape(shape)
+    xhat = (x - mean) * invstd
+    dscale = (dy * xhat).sum(axis=axes)
+    dbias = dy.sum(axis=axes)
+    dx = np.asarray(scale, np.float64).reshape(shape) * invstd * (dy - dbias.reshape(shape) / m
+                                                                    - xhat * dscale.reshape(shape) / m)
+    return dx, dscale, dbias

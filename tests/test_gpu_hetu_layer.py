@@ -844,3 +844,38 @@ def test_norm_and_gradient_entry_points(ops, cuda, dtype, p):
         ops.norm(tx, out, dim, 0)
     with pytest.raises(ops.AssertionError_, match="does not hold"):
         ops.norm(tx, out[:, :63].contiguous(), dim, p)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_batch_norm_entry_points(ops, cuda, dtype):
+    import torch
+    shape = (6, 12, 10, 10)
+    g = helpers.rng(91)
+    x = oracle.round_to((g.standard_normal(shape) * 2 + 1).astype(np.float32), dtype)
+    scale = g.uniform(0.5, 1.5, 12).astype(np.float32); bias = g.standard_normal(12).astype(np.float32)
+    rm = g.standard_normal(12).astype(np.float32); rv = g.uniform(0.5, 2, 12).astype(np.float32)
+    dy = oracle.round_to(g.standard_normal(shape).astype(np.float32), dtype)
+    ey, erm, erv, emean, einv = oracle.batch_norm_fwd(x, scale, bias, rm, rv, 0.1, 1e-5)
+    tx = helpers.to_torch(x, dtype, cuda)
+    ts, tb, trm, trv = _dev((scale, bias, rm, rv), "fp32", cuda)
+    ty = torch.empty_like(tx); sm = torch.empty_like(ts); sv = torch.empty_like(ts)
+    _sync_in()
+    ops.batch_norm(tx, ts, tb, ty, 0.1, 1e-5, trm, trv, sm, sv)
+    ops.stream_sync()
+    helpers.assert_close(ty, ey, dtype, "y")
+    helpers.assert_close(trm, erm, "fp32", "running_mean", scale=1.0)
+    helpers.assert_close(trv, erv, "fp32", "running_var", rtol=1e-4)
+    helpers.assert_close(sv, einv, "fp32", "save_var (inverse standard deviation)", rtol=1e-4)
+    edx, eds, edb = oracle.batch_norm_bwd(dy, x, scale, helpers.to_numpy(sm), helpers.to_numpy(sv))
+    dx = torch.empty_like(tx); ds = torch.empty_like(ts); db = torch.empty_like(ts)
+    _sync_in()
+    ops.batch_norm_gradient(helpers.to_torch(dy, dtype, cuda), tx, ts, dx, ds, db, 1e-5, sm, sv)
+    ops.stream_sync()
+    helpers.assert_close(dx, edx, dtype, "dx", rtol=2e-2 if dtype == "bf16" else 1e-4)
+    helpers.assert_close(ds, eds, "fp32", "dscale", rtol=1e-4)
+    helpers.assert_close(db, edb, "fp32", "dbias", rtol=1e-4)
+    if dtype == "bf16":
+        with pytest.raises(ops.AssertionError_, match="bn_scale must have dtype"):
+            ops.batch_norm(tx, ts.bfloat16(), tb, ty, 0.1, 1e-5, trm, trv, sm, sv)
+    with pytest.raises(ops.AssertionError_, match="one value per channel"):
+        ops.batch_norm(tx, ts[:11].contiguous(), tb, ty, 0.1, 1e-5, trm, trv, sm, sv)

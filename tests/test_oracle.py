@@ -389,3 +389,29 @@ def test_p_norm_against_torch_autograd(p, dim):
     assert (nz == 0).all()
     gz = np.ones(nz.shape)
     assert (oracle.norm_p_bwd(z, nz, gz, dim, p) == 0).all()
+
+
+def test_batch_norm_against_torch():
+    """oracle.batch_norm_fwd / _bwd against torch.nn.functional.batch_norm in training mode (float64; its
+    running-variance update also takes the unbiased estimate) and torch autograd."""
+    import torch
+    g = np.random.default_rng(5)
+    x = g.standard_normal((6, 5, 4, 3)) * 2 + 1
+    scale = g.uniform(0.5, 1.5, 5); bias = g.standard_normal(5)
+    rm = g.standard_normal(5); rv = g.uniform(0.5, 2.0, 5)
+    dy = g.standard_normal(x.shape)
+    y, nrm, nrv, smean, sinv = oracle.batch_norm_fwd(x, scale, bias, rm, rv, 0.1, 1e-5)
+    tx = torch.tensor(x, requires_grad=True); ts = torch.tensor(scale, requires_grad=True)
+    tb = torch.tensor(bias, requires_grad=True)
+    trm, trv = torch.tensor(rm), torch.tensor(rv)
+    ty = torch.nn.functional.batch_norm(tx, trm, trv, ts, tb, training=True, momentum=0.1, eps=1e-5)
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(nrm, trm.numpy(), rtol=1e-13)
+    np.testing.assert_allclose(nrv, trv.numpy(), rtol=1e-13)
+    np.testing.assert_allclose(smean, x.mean(axis=(0, 2, 3)), rtol=1e-13)
+    np.testing.assert_allclose(sinv, 1 / np.sqrt(x.var(axis=(0, 2, 3)) + 1e-5), rtol=1e-13)
+    (ty * torch.tensor(dy)).sum().backward()
+    dx, dscale, dbias = oracle.batch_norm_bwd(dy, x, scale, smean, sinv)
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(dscale, ts.grad.numpy(), rtol=1e-11)
+    np.testing.assert_allclose(dbias, tb.grad.numpy(), rtol=1e-11)

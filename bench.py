@@ -283,6 +283,34 @@ def case_reduce(hk, torch, nsets, axes, op, three_d=False):
         (rows if 1 in axes and not three_d else cols)
 
 
+def case_p_norm(hk, torch, nsets, which):
+    """2-norm of every row of a bf16 [32768 x 4096] array (read only), and its gradient (2 reads, 1 write)."""
+    rows, cols = 32768, 4096
+    bf = torch.bfloat16
+    sets = [_randn(torch, (rows, cols), bf, 1.0, 901 + 10 * i) for i in range(nsets)]
+    out = torch.empty(rows, dtype=bf, device="cuda")
+    if which == "fwd":
+        ws = torch.empty(max(1, hk.reduce_workspace_bytes(8, [rows, cols], [cols, 1], [1]) // 4), device="cuda")
+        return (lambda i: hk.norm(sets[i % nsets], out, 1, 2, workspace=ws)), rows * cols * 2 + rows * 2, rows
+    hk.norm(sets[0], out, 1, 2)
+    grad = _randn(torch, (rows,), bf, 1.0, 977)
+    dx = [torch.empty_like(t) for t in sets]
+    return (lambda i: hk.norm_bwd(sets[i % nsets], out, grad, dx[i % nsets], 1, 2)), \
+        2 * rows * cols * 2 + 2 * rows * 2, rows
+
+
+def case_reduce_gradient(hk, torch, nsets, axis):
+    """Gradient of a mean over `axis` of a bf16 [32768 x 4096] array: the output's gradient laid back over the
+    input, times 1/n (write only but for one small vector)."""
+    rows, cols = 32768, 4096
+    bf = torch.bfloat16
+    nin = cols if axis == 0 else rows
+    grad = _randn(torch, (1, cols) if axis == 0 else (rows, 1), bf, 1.0, 951)
+    outs = [torch.empty(rows, cols, dtype=bf, device="cuda") for _ in range(nsets)]
+    scale = 1.0 / (rows if axis == 0 else cols)
+    return (lambda i: hk.broadcast(grad, outs[i % nsets], scalar=scale)), rows * cols * 2 + nin * 2, rows
+
+
 def case_copy(hk, torch, nsets):
     n = 1 << 28
     src = [torch.empty(n, dtype=torch.uint8, device="cuda").zero_() for _ in range(nsets)]
@@ -339,6 +367,10 @@ CASES = [
     ("next: vocab-parallel CE bwd bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "vce")),
     ("next: vocab-parallel CE fused stats bf16 [16384x32000] (read only)", lambda hk, t, n: case_elementwise(hk, t, n, "stats")),
     ("next: vocab-parallel CE fused bwd bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "fused")),
+    ("next: 2-norm of rows bf16 [32768x4096] (read only)", lambda hk, t, n: case_p_norm(hk, t, n, "fwd")),
+    ("next: 2-norm of rows, gradient bf16 [32768x4096]", lambda hk, t, n: case_p_norm(hk, t, n, "bwd")),
+    ("next: gradient of mean axis0 bf16 [32768x4096] (write only)", lambda hk, t, n: case_reduce_gradient(hk, t, n, 0)),
+    ("next: gradient of mean axis1 bf16 [32768x4096] (write only)", lambda hk, t, n: case_reduce_gradient(hk, t, n, 1)),
     ("next: batch norm fwd bf16 [256,256,56,56] (2R+1W, 3 launches)", lambda hk, t, n: case_batch_norm(hk, t, n, "fwd")),
     ("next: batch norm bwd bf16 [256,256,56,56] (4R+1W, 3 launches)", lambda hk, t, n: case_batch_norm(hk, t, n, "bwd")),
     ("C4 rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "fwd")),

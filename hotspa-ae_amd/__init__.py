@@ -18,7 +18,7 @@ from .capi import (  # noqa: F401
     HkError, lib, lib_path, check, DTYPES, dtype_code, torch_dtype,
     layer_norm_fwd, layer_norm_bwd, norm_bwd_workspace_bytes,
     dropout_add_ln_fwd, dropout_add_ln_bwd, dropout_add_ln_fwd_ex, dropout_add_ln_bwd_ex,
-    unary, binary_const, binary, vocab_parallel_ce_gather, vocab_parallel_ce_bwd,
+    unary, binary_const, binary, broadcast, sce_sparse_bwd_reduced, sce_dense_bwd_reduced, vocab_parallel_ce_gather, vocab_parallel_ce_bwd,
     vocab_parallel_ce_stats, vocab_parallel_ce_combine, vocab_parallel_ce_bwd_fused, UNARY_OPS, BINARY_OPS,
     softmax_fwd, softmax_bwd,
     sce_sparse_fwd, sce_sparse_bwd, sce_dense_fwd, sce_dense_bwd, nll_loss_fwd, nll_loss_bwd,

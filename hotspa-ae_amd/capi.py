@@ -285,6 +285,16 @@ def binary(op, a, b, out, stream=None):
                           _arr(shape), _arr(sa), _arr(sb), stream if stream is not None else current_stream()))
 
 
+def broadcast(x, out, scalar=None, stream=None):
+    """hk_broadcast: out (dense) = x broadcast to out's shape (x.expand(out.shape) must be legal; any strides),
+    times `scalar` when given."""
+    shape = list(out.shape)
+    sx = list(x.expand(shape).stride())
+    check(lib().hk_broadcast(dtype_code(out), _ptr(x), ctypes.c_int(int(scalar is not None)),
+                             ctypes.c_double(0.0 if scalar is None else scalar), _ptr(out), ctypes.c_int(len(shape)),
+                             _arr(shape), _arr(sx), stream if stream is not None else current_stream()))
+
+
 def vocab_parallel_ce_gather(logits, labels, vocab_start, vocab_end, ignored_index, picked, lse, stream=None):
     rows, cols = logits.shape
     check(lib().hk_vocab_parallel_ce_gather(dtype_code(logits), _ptr(logits), _ptr(labels), _i64(rows), _i64(cols),
@@ -407,6 +417,22 @@ def sce_sparse_bwd(logits, labels, grad_loss, dlogits, ignored_index, stream=Non
     check(lib().hk_sce_sparse_bwd(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(grad_loss), _ptr(dlogits),
                                   _i64(rows), _i64(cols), _i64(ignored_index),
                                   stream if stream is not None else current_stream()))
+
+
+def sce_sparse_bwd_reduced(logits, labels, grad_output, scale, dlogits, ignored_index, stream=None):
+    cols = logits.shape[-1]
+    rows = logits.numel() // cols if logits.numel() else 0
+    check(lib().hk_sce_sparse_bwd_reduced(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(grad_output),
+                                          ctypes.c_double(scale), _ptr(dlogits), _i64(rows), _i64(cols),
+                                          _i64(ignored_index), stream if stream is not None else current_stream()))
+
+
+def sce_dense_bwd_reduced(logits, labels, grad_output, scale, dlogits, stream=None):
+    cols = logits.shape[-1]
+    rows = logits.numel() // cols if logits.numel() else 0
+    check(lib().hk_sce_dense_bwd_reduced(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(grad_output),
+                                         ctypes.c_double(scale), _ptr(dlogits), _i64(rows), _i64(cols),
+                                         stream if stream is not None else current_stream()))
 
 
 def sce_dense_fwd(logits, labels, loss, stream=None):

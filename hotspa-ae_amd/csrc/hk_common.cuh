@@ -403,6 +403,30 @@ void set_last_error(const char* fmt, ...);
     }                                                                          \
   } while (0)
 
+// The constant enters the arithmetic rounded to the array's type, as static_cast<spec_t>(value) does.
+template <typename T> inline double round_const(double c) { return c; }
+template <> inline double round_const<float>(double c) { return double(float(c)); }
+template <> inline double round_const<fp16>(double c) { return double(float(_Float16(float(c)))); }
+template <> inline double round_const<bf16>(double c) {
+  const float f = float(c);
+  uint32_t u;
+  __builtin_memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return c;          // NaN stays NaN
+  u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;     // round to nearest even
+  float r;
+  __builtin_memcpy(&r, &u, 4);
+  return double(r);
+}
+
+inline double round_to_dtype(int dtype, double c) {
+  switch (dtype) {
+    case HK_FLOAT32: return round_const<float>(c);
+    case HK_BFLOAT16: return round_const<bf16>(c);
+    case HK_FLOAT16: return round_const<fp16>(c);
+    default: return c;
+  }
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline hipStream_t as_hip(hkStream_t s) { return reinterpret_cast<hipStream_t>(s); }

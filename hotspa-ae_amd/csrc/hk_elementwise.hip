@@ -169,6 +169,46 @@ __global__ __launch_bounds__(256) void ew_binary_generic_kernel(const T* a, cons
   Cvt<T>::store(out + i, ew_bin<OP, CT>(ew_load(a + oa), ew_load(b + ob)));
 }
 
+// out = broadcast(a) [* c]: a dense output filled from an operand that maps onto it in one of the four modes.
+// What a reduction's backward does with the gradient of its output.
+template <typename T, int AM, bool MUL>
+__global__ __launch_bounds__(256) void ew_broadcast_2d_vec_kernel(const T* a, float c, T* out, uint32_t nvec,
+                                                                  uint32_t cols_vec) {
+  constexpr int VEC = VecIO<T>::N;
+  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+  if (v >= nvec) return;
+  uint32_t r = 0, col = v;
+  if constexpr (AM != EW_FULL) {
+    r = v / cols_vec;
+    col = v - r * cols_vec;
+  }
+  EwRaw<T, AM> ra;
+  ra.load(a, v, r, col);
+  float f[VEC];
+  ra.unpack(f);
+  if constexpr (MUL) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) f[j] *= c;
+  }
+  st16_stream(out + size_t(v) * VEC, VecIO<T>::pack(f));
+}
+
+template <typename T, bool MUL>
+__global__ __launch_bounds__(256) void ew_broadcast_generic_kernel(const T* a, double c, T* out, EwDims d,
+                                                                   int64_t n) {
+  using CT = typename EwCT<T>::type;
+  const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n) return;
+  int64_t rem = i, oa = 0;
+  for (int k = d.ndim - 1; k >= 0; --k) {
+    const int64_t q = rem / d.shape[k];
+    oa += (rem - q * d.shape[k]) * d.astride[k];
+    rem = q;
+  }
+  const CT x = ew_load(a + oa);
+  Cvt<T>::store(out + i, MUL ? x * CT(c) : x);
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -191,21 +231,6 @@ static int unary_launch(const void* in, void* out, int64_t n, hipStream_t s) {
                      static_cast<const T*>(in), static_cast<T*>(out), n);
   profile_after(s);
   return launch_check("ew_unary_scalar_kernel");
-}
-
-// The constant enters the arithmetic rounded to the array's type, as static_cast<spec_t>(value) does.
-template <typename T> static double round_const(double c) { return c; }
-template <> double round_const<float>(double c) { return double(float(c)); }
-template <> double round_const<fp16>(double c) { return double(float(_Float16(float(c)))); }
-template <> double round_const<bf16>(double c) {
-  const float f = float(c);
-  uint32_t u;
-  __builtin_memcpy(&u, &f, 4);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return c;          // NaN stays NaN
-  u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;     // round to nearest even
-  float r;
-  __builtin_memcpy(&r, &u, 4);
-  return double(r);
 }
 
 template <typename T, int OP, bool REV>
@@ -315,6 +340,43 @@ static int binary_launch(const void* a, const void* b, void* out, const EwDims& 
   return launch_check("ew_binary_generic_kernel");
 }
 
+template <typename T, bool MUL>
+static int broadcast_launch(const void* a, double c, void* out, const EwDims& d, int64_t n, hipStream_t s) {
+  HK_REQUIRE((n + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_broadcast: array too large");
+  const T* pa = static_cast<const T*>(a);
+  T* po = static_cast<T*>(out);
+  c = round_const<T>(c);
+  profile_before(s);
+  if constexpr (!std::is_same<T, double>::value) {
+    constexpr int VEC = VecIO<T>::N;
+    if (d.ndim <= 2) {
+      const int64_t rows = d.ndim == 2 ? d.shape[0] : 1;
+      const int64_t cols = d.ndim == 2 ? d.shape[1] : d.shape[0];
+      const int64_t a0 = d.ndim == 2 ? d.astride[0] : 0, a1 = d.ndim == 2 ? d.astride[1] : d.astride[0];
+      const int am = operand_mode(rows, cols, a0, a1);
+      const bool a_ok = am == EW_PER_ROW || am == EW_SINGLE || aligned16(a);
+      if (am >= 0 && cols % VEC == 0 && aligned16(out) && a_ok && n / VEC < 0x7fffffffLL) {
+        const uint32_t nvec = uint32_t(n / VEC), cols_vec = uint32_t(cols / VEC);
+        const dim3 grid(blocks_for(nvec)), block(256);
+#define HK_EW_BC(AM) \
+  hipLaunchKernelGGL((ew_broadcast_2d_vec_kernel<T, AM, MUL>), grid, block, 0, s, pa, float(c), po, nvec, cols_vec)
+        switch (am) {
+          case EW_FULL: HK_EW_BC(EW_FULL); break;
+          case EW_PER_ROW: HK_EW_BC(EW_PER_ROW); break;
+          case EW_PER_COL: HK_EW_BC(EW_PER_COL); break;
+          default: HK_EW_BC(EW_SINGLE); break;
+        }
+#undef HK_EW_BC
+        profile_after(s);
+        return launch_check("ew_broadcast_2d_vec_kernel");
+      }
+    }
+  }
+  hipLaunchKernelGGL((ew_broadcast_generic_kernel<T, MUL>), dim3(blocks_for(n)), dim3(256), 0, s, pa, c, po, d, n);
+  profile_after(s);
+  return launch_check("ew_broadcast_generic_kernel");
+}
+
 #define HK_EW_TYPES(dtype, who, CALL)                                    \
   switch (dtype) {                                                       \
     case HK_FLOAT32: { using T = float; return CALL; }                   \
@@ -338,6 +400,12 @@ template <int OP>
 static int binary_typed(int dtype, const void* a, const void* b, void* out, const EwDims& d, int64_t n,
                         hipStream_t s) {
   HK_EW_TYPES(dtype, "hk_binary", (binary_launch<T, OP>(a, b, out, d, n, s)));
+}
+
+template <bool MUL>
+static int broadcast_typed(int dtype, const void* a, double c, void* out, const EwDims& d, int64_t n,
+                           hipStream_t s) {
+  HK_EW_TYPES(dtype, "hk_broadcast", (broadcast_launch<T, MUL>(a, c, out, d, n, s)));
 }
 
 } // namespace hk
@@ -401,6 +469,24 @@ int hk_binary(int op, int dtype, const void* a, const void* b, void* out, int nd
     case HK_BINARY_DIV: return binary_typed<EW_DIV>(dtype, a, b, out, d, n, s);
     default: set_last_error("hk_binary: unknown op %d", op); return HK_ERR_INVALID;
   }
+}
+
+int hk_broadcast(int dtype, const void* in, int multiply, double scalar, void* out, int ndim,
+                 const int64_t* out_shape, const int64_t* in_strides, hkStream_t stream) {
+  HK_REQUIRE(ndim >= 0 && ndim <= 8, HK_ERR_INVALID, "hk_broadcast: ndim %d outside [0, 8]", ndim);
+  HK_REQUIRE(ndim == 0 || (out_shape && in_strides), HK_ERR_INVALID, "hk_broadcast: null shape/strides");
+  int64_t n = 1;
+  for (int i = 0; i < ndim; ++i) {
+    HK_REQUIRE(out_shape[i] >= 0, HK_ERR_INVALID, "hk_broadcast: negative extent");
+    HK_REQUIRE(in_strides[i] >= 0, HK_ERR_INVALID, "hk_broadcast: negative stride");
+    n *= out_shape[i];
+  }
+  if (n == 0) return HK_OK;
+  HK_REQUIRE(in && out, HK_ERR_INVALID, "hk_broadcast: null input/output");
+  const EwDims d = merge_dims(ndim, out_shape, in_strides, in_strides);
+  hipStream_t s = as_hip(stream);
+  return multiply ? broadcast_typed<true>(dtype, in, scalar, out, d, n, s)
+                  : broadcast_typed<false>(dtype, in, scalar, out, d, n, s);
 }
 
 } // extern "C"

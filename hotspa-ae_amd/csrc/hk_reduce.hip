@@ -706,8 +706,10 @@ void norm_grad_kernel(const T* __restrict__ x, const T* __restrict__ norm, const
   Cvt<T>::store(out + i, o);
 }
 
-// the same for a norm over the last dimension (after == 1), one 16-byte vector per thread
-template <typename T>
+// the same for a norm over the last dimension (after == 1), one 16-byte vector per thread.  PK names the
+// exponent at compile time (1, 2, or 0 for any other) so that nothing but the arithmetic sits between the loads
+// and the store; the per-row factor is formed once per thread.
+template <typename T, int PK>
 __global__ __launch_bounds__(256)
 void norm_grad_rows_vec_kernel(const T* __restrict__ x, const T* __restrict__ norm, const T* __restrict__ grad,
                                T* out, uint32_t nvec, uint32_t cols_vec, int64_t p) {
@@ -717,22 +719,20 @@ void norm_grad_rows_vec_kernel(const T* __restrict__ x, const T* __restrict__ no
   const uint32_t r = v / cols_vec;
   const u32x4 raw = ld16(x + size_t(v) * VEC);
   const float g = Cvt<T>::load(grad + r);
-  const float n = Cvt<T>::load(norm + r);
+  const float n = PK == 1 ? 1.f : Cvt<T>::load(norm + r);
   float f[VEC];
   VecIO<T>::unpack(raw, f);
-  if (p == 1) {
+  if constexpr (PK == 1) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) f[j] = (f[j] == 0.f ? 0.f : (f[j] < 0.f ? -1.f : 1.f)) * g;
-  } else if (n == 0.f) {
+  } else if constexpr (PK == 2) {
+    const float scale = n == 0.f ? 0.f : g / n;
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) f[j] = 0.f;
-  } else if (p == 2) {
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) f[j] = g * f[j] / n;
+    for (int j = 0; j < VEC; ++j) f[j] = n == 0.f ? 0.f : f[j] * scale;
   } else {
-    const float scale = g / powf(n, float(p - 1));
+    const float scale = n == 0.f ? 0.f : g / powf(n, float(p - 1));
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) f[j] = f[j] * powf(fabsf(f[j]), float(p - 2)) * scale;
+    for (int j = 0; j < VEC; ++j) f[j] = n == 0.f ? 0.f : f[j] * powf(fabsf(f[j]), float(p - 2)) * scale;
   }
   st16_stream(out + size_t(v) * VEC, VecIO<T>::pack(f));
 }
@@ -746,8 +746,10 @@ static int norm_grad_typed(const void* x, const void* norm, const void* grad, vo
     constexpr int VEC = VecIO<T>::N;
     if (after == 1 && reduce_size % VEC == 0 && aligned16(x) && aligned16(out) && total / VEC < 0x7fffffffLL) {
       const uint32_t nvec = uint32_t(total / VEC);
+      auto kernel = p == 1 ? norm_grad_rows_vec_kernel<T, 1>
+                  : p == 2 ? norm_grad_rows_vec_kernel<T, 2> : norm_grad_rows_vec_kernel<T, 0>;
       profile_before(s);
-      hipLaunchKernelGGL((norm_grad_rows_vec_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
+      hipLaunchKernelGGL(kernel, dim3((nvec + 255) / 256), dim3(256), 0, s,
                          static_cast<const T*>(x), static_cast<const T*>(norm), static_cast<const T*>(grad),
                          static_cast<T*>(out), nvec, uint32_t(reduce_size / VEC), p);
       profile_after(s);

@@ -33,7 +33,21 @@ struct SceArgs {
   // stats[2 rows..3 rows) = the logit at the label when the label falls into the shard, else 0
   float* stats;
   int64_t vocab_start;
+  // backward of a reduced loss: grad_loss holds ONE value (the gradient of the mean / sum) and every row uses
+  // round_T(that value * grad_scale), which is what broadcasting it times 1/rows into a [rows] array of the
+  // storage type first would have handed to this kernel
+  int grad_scalar;
+  double grad_scale;
 };
+
+template <typename T, typename CT>
+__device__ __forceinline__ CT sce_row_grad(const SceArgs& a, int64_t row) {
+  const T* gp = static_cast<const T*>(a.grad_loss);
+  if (!a.grad_scalar) return CT(Cvt<T>::load(gp + row));
+  T rounded;
+  Cvt<T>::store(&rounded, CT(Cvt<T>::load(gp)) * CT(a.grad_scale));
+  return CT(Cvt<T>::load(&rounded));
+}
 
 template <bool WAVE_ROW>
 __device__ __forceinline__ void row_coords(int& tpr, int& t, int64_t& row, int& nwaves) {
@@ -156,7 +170,7 @@ void sce_sparse_bwd_kernel(SceArgs a) {
     raw[i] = u32x4{0, 0, 0, 0};
     if (v < a.nvec) raw[i] = ld16(xr + v * VEC);
   }
-  const float g = Cvt<T>::load(static_cast<const T*>(a.grad_loss) + row);
+  const float g = sce_row_grad<T, float>(a, row);
   float e[NV * VEC];
   float m = kNegInf;
 #pragma unroll
@@ -262,7 +276,7 @@ void sce_dense_kernel(SceArgs a) {
       Cvt<T>::store(static_cast<T*>(a.out) + row, lse * ls.v[0] - ls.v[1]);
     }
   } else {
-    const float g = Cvt<T>::load(static_cast<const T*>(a.grad_loss) + row);
+    const float g = sce_row_grad<T, float>(a, row);
     const float ML = (p.v[0] == kNegInf) ? 0.f : p.v[0];
     const float inv = 1.0f / p.v[1];
     T* dxr = static_cast<T*>(a.out) + row * int64_t(a.cols);
@@ -378,7 +392,7 @@ void sce_generic_kernel(SceArgs a) {
     if (threadIdx.x == 0)
       SceIO<T, CT>::st(static_cast<T*>(a.out) + row, (sce_log<CT>(s) + m) * sl - slx);
   } else {
-    const CT g = SceIO<T, CT>::ld(static_cast<const T*>(a.grad_loss) + row);
+    const CT g = sce_row_grad<T, CT>(a, row);
     const CT inv = CT(1) / s;
     T* dxr = static_cast<T*>(a.out) + row * cols;
     const T* lr = MODE == 3 ? static_cast<const T*>(a.dlabels) + row * cols : nullptr;
@@ -530,6 +544,29 @@ int hk_sce_sparse_bwd(int dtype, const void* logits, const int64_t* labels, cons
   a.logits = logits; a.labels = labels; a.grad_loss = grad_loss; a.out = dlogits; a.rows = rows;
   a.cols = int(cols); a.ignored_index = ignored_index;
   return sce_dispatch<1>(dtype, a, as_hip(stream), "hk_sce_sparse_bwd");
+}
+
+int hk_sce_sparse_bwd_reduced(int dtype, const void* logits, const int64_t* labels, const void* grad_output,
+                              double scale, void* dlogits, int64_t rows, int64_t cols, int64_t ignored_index,
+                              hkStream_t stream) {
+  HK_REQUIRE(cols <= 0x3fffffff, HK_ERR_INVALID, "hk_sce_sparse_bwd_reduced: cols too large");
+  SceArgs a{};
+  a.logits = logits; a.labels = labels; a.grad_loss = grad_output; a.out = dlogits; a.rows = rows;
+  a.cols = int(cols); a.ignored_index = ignored_index;
+  a.grad_scalar = 1;
+  a.grad_scale = round_to_dtype(dtype, scale);
+  return sce_dispatch<1>(dtype, a, as_hip(stream), "hk_sce_sparse_bwd_reduced");
+}
+
+int hk_sce_dense_bwd_reduced(int dtype, const void* logits, const void* labels, const void* grad_output,
+                             double scale, void* dlogits, int64_t rows, int64_t cols, hkStream_t stream) {
+  HK_REQUIRE(cols <= 0x3fffffff, HK_ERR_INVALID, "hk_sce_dense_bwd_reduced: cols too large");
+  SceArgs a{};
+  a.logits = logits; a.dlabels = labels; a.grad_loss = grad_output; a.out = dlogits; a.rows = rows;
+  a.cols = int(cols);
+  a.grad_scalar = 1;
+  a.grad_scale = round_to_dtype(dtype, scale);
+  return sce_dispatch<3>(dtype, a, as_hip(stream), "hk_sce_dense_bwd_reduced");
 }
 
 int hk_sce_dense_fwd(int dtype, const void* logits, const void* labels, void* loss, int64_t rows,

@@ -3,6 +3,7 @@
 
 #include <string>
 
+#include "hetu/graph/ops/gradient_compute.h"
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/random/CPURandomState.h"
 #include "hetu/impl/memory/CachingMemoryPool.h"
@@ -459,6 +460,43 @@ int ht_ndarray_sceloss(const HtArray* preds, const HtArray* labels, int sparse, 
     NDArray r = sparse ? NDArray::sceloss(wrap(preds), wrap(labels), ignored_index, red, stream_index)
                        : NDArray::sceloss(wrap(preds), wrap(labels), red, stream_index);
     copy_out(r, out, stream_of(preds, stream_index));
+  });
+}
+
+int ht_broadcast_shape(const HtArray* input, int multiply, double const_value, HtArray* output,
+                       const int64_t* add_axes, int n_add_axes, int stream_index) {
+  return guarded([&] {
+    NDArray out = wrap(output);
+    HTShape axes(add_axes, add_axes + (add_axes ? n_add_axes : 0));
+    if (multiply)
+      hetu::impl::BroadcastShapeMulCuda(wrap(input), const_value, out, axes, stream_of(input, stream_index));
+    else
+      hetu::impl::BroadcastShapeCuda(wrap(input), out, axes, stream_of(input, stream_index));
+  });
+}
+
+int ht_reduce_gradient(const HtArray* grad_output, int reduction, const int64_t* axes, int naxes,
+                       const int* keepdims, int n_keepdims, HtArray* output, int stream_index) {
+  return guarded([&] {
+    NDArray out = wrap(output);
+    HTAxes ax(axes, axes + (axes ? naxes : 0));
+    hetu::graph::HTKeepDims keep;
+    for (int i = 0; i < n_keepdims; ++i) keep.push_back(keepdims[i] != 0);
+    hetu::graph::ReduceGradientCompute(wrap(grad_output), out->shape(), static_cast<ReductionType>(reduction), ax,
+                                       keep, stream_index, out);
+  });
+}
+
+int ht_sceloss_gradient(const HtArray* preds, const HtArray* labels, const HtArray* grad_output, int sparse,
+                        int64_t ignored_index, int reduction, int fused, HtArray* output, int stream_index) {
+  return guarded([&] {
+    NDArray out = wrap(output);
+    const auto red = static_cast<ReductionType>(reduction);
+    if (sparse)
+      hetu::graph::SCESGradCompute(wrap(preds), wrap(labels), wrap(grad_output), ignored_index, red, stream_index,
+                                   out, fused != 0);
+    else
+      hetu::graph::SCEGradCompute(wrap(preds), wrap(labels), wrap(grad_output), red, stream_index, out, fused != 0);
   });
 }
 

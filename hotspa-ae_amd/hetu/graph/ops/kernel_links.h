@@ -143,5 +143,15 @@ DECLARE_KERNEL_CPU_AND_CUDA(SoftmaxCrossEntropySparseGradient, const NDArray&, c
 #define HT_DISPATCH_KERNEL_CUDA_ONLY(DEVICE_TYPE, OP_TYPE, KERNEL, ...)                             \
   HT_DISPATCH_KERNEL_SWITCH(DEVICE_TYPE, OP_TYPE, HT_DISPATCH_KERNEL_CASE_CUDA(KERNEL, __VA_ARGS__))
 
+// input, output, add_axes  /  input, const_value, output, add_axes   (hetu/graph/ops/kernel_links.h:64-67)
+DECLARE_KERNEL_CPU_AND_CUDA(BroadcastShape, const NDArray&, NDArray&, const HTShape&, const Stream&);
+DECLARE_KERNEL_CPU_AND_CUDA(BroadcastShapeMul, const NDArray&, double, NDArray&, const HTShape&, const Stream&);
+// The cross-entropy gradients fed the ONE gradient value of a reduced loss and its scale instead of a
+// per-row array (no counterpart in the reference): pred, label, grad_output, scale, output, [ignored_index]
+DECLARE_KERNEL_CUDA(SoftmaxCrossEntropySparseGradientReduced, const NDArray&, const NDArray&, const NDArray&, double,
+                    NDArray&, const int64_t, const Stream&);
+DECLARE_KERNEL_CUDA(SoftmaxCrossEntropyGradientReduced, const NDArray&, const NDArray&, const NDArray&, double,
+                    NDArray&, const Stream&);
+
 } // namespace impl
 } // namespace hetu

@@ -33,15 +33,18 @@ void SoftmaxCrossEntropyCuda(const NDArray& input, const NDArray& label, NDArray
   NDArray::MarkUsedBy({x, l, output}, stream);
 }
 
-void SoftmaxCrossEntropyGradientCuda(const NDArray& input_y, const NDArray& label, const NDArray& grad,
-                                     NDArray& output, const Stream& stream) {
+namespace {
+// scale == nullptr: grad holds one value per row; else it holds ONE value, used as
+// round(grad[0] * round(*scale)) by every row
+void DenseGradient(const NDArray& input_y, const NDArray& label, const NDArray& grad, const double* scale,
+                   NDArray& output, const Stream& stream) {
   HT_ASSERT_CUDA_DEVICE(input_y);
   HT_ASSERT_SAME_DEVICE(input_y, label);
   HT_ASSERT_SAME_DEVICE(input_y, grad);
   HT_ASSERT_SAME_DEVICE(input_y, output);
   const size_t indim = input_y->ndim();
   HT_ASSERT(indim >= 1 && indim == label->ndim() && indim == output->ndim() &&
-            (indim == grad->ndim() + 1 || (indim == 1 && grad->ndim() == 1)))
+            (scale || indim == grad->ndim() + 1 || (indim == 1 && grad->ndim() == 1)))
     << "Indim is " << indim << ", Label dim is " << label->ndim() << ", Output dim is " << output->ndim();
   HT_ASSERT_SAME_SHAPE(input_y, label);
   HT_ASSERT_SAME_SHAPE(input_y, output);
@@ -52,15 +55,37 @@ void SoftmaxCrossEntropyGradientCuda(const NDArray& input_y, const NDArray& labe
   int64_t rows = 1;
   for (size_t i = 0; i + 1 < indim; ++i) rows *= input_y->shape(i);
   const int64_t cols = input_y->shape(indim - 1);
-  HT_ASSERT(int64_t(grad->numel()) == rows) << "grad " << grad->shape() << " must hold one value per row";
+  if (scale) {
+    HT_ASSERT(grad->numel() == 1) << "the gradient of a reduced loss is one value, got " << grad->shape();
+  } else {
+    HT_ASSERT(int64_t(grad->numel()) == rows) << "grad " << grad->shape() << " must hold one value per row";
+  }
   if (rows * cols == 0) return;
 
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
   NDArray x = Dense(input_y, stream), l = Dense(label, stream), g = Dense(grad, stream);
-  HK_CALL(hk_sce_dense_bwd(int(input_y->dtype()), x->raw_data_ptr(), l->raw_data_ptr(), g->raw_data_ptr(),
-                           output->raw_data_ptr(), rows, cols, hip_stream));
+  if (scale) {
+    HK_CALL(hk_sce_dense_bwd_reduced(int(input_y->dtype()), x->raw_data_ptr(), l->raw_data_ptr(), g->raw_data_ptr(),
+                                     *scale, output->raw_data_ptr(), rows, cols, hip_stream));
+  } else {
+    HK_CALL(hk_sce_dense_bwd(int(input_y->dtype()), x->raw_data_ptr(), l->raw_data_ptr(), g->raw_data_ptr(),
+                             output->raw_data_ptr(), rows, cols, hip_stream));
+  }
   NDArray::MarkUsedBy({x, l, g, output}, stream);
+}
+} // namespace
+
+void SoftmaxCrossEntropyGradientCuda(const NDArray& input_y, const NDArray& label, const NDArray& grad,
+                                     NDArray& output, const Stream& stream) {
+  DenseGradient(input_y, label, grad, nullptr, output, stream);
+}
+
+// No counterpart in the reference, whose gradient op first broadcasts the one gradient value times `scale`
+// into a [rows] array (hetu/graph/ops/SoftmaxCrossEntropy.cc:59-80) and then calls the kernel above.
+void SoftmaxCrossEntropyGradientReducedCuda(const NDArray& input_y, const NDArray& label, const NDArray& grad_output,
+                                            double scale, NDArray& output, const Stream& stream) {
+  DenseGradient(input_y, label, grad_output, &scale, output, stream);
 }
 
 void SoftmaxCrossEntropyCpu(const NDArray&, const NDArray&, NDArray&, const Stream&) {

@@ -41,8 +41,11 @@ void SoftmaxCrossEntropySparseCuda(const NDArray& pred, const NDArray& label, ND
   NDArray::MarkUsedBy({p, l, loss}, stream);
 }
 
-void SoftmaxCrossEntropySparseGradientCuda(const NDArray& pred, const NDArray& label, const NDArray& grad_loss,
-                                           NDArray& output, const int64_t ignored_index, const Stream& stream) {
+namespace {
+// scale == nullptr: grad_loss holds one value per row; else it holds ONE value, used as
+// round(grad_loss[0] * round(*scale)) by every row
+void SparseGradient(const NDArray& pred, const NDArray& label, const NDArray& grad_loss, const double* scale,
+                    NDArray& output, const int64_t ignored_index, const Stream& stream) {
   HT_ASSERT_CUDA_DEVICE(pred);
   HT_ASSERT_SAME_DEVICE(pred, label);
   HT_ASSERT_SAME_DEVICE(pred, grad_loss);
@@ -54,17 +57,43 @@ void SoftmaxCrossEntropySparseGradientCuda(const NDArray& pred, const NDArray& l
   HT_ASSERT_CONTIGUOUS(output);
   int64_t rows, cols;
   RowsCols(pred, rows, cols);
-  HT_ASSERT(int64_t(label->numel()) == rows && int64_t(grad_loss->numel()) == rows)
-    << "labels " << label->shape() << " / grad_loss " << grad_loss->shape() << " must hold one value per row of "
-    << pred->shape();
+  HT_ASSERT(int64_t(label->numel()) == rows) << "labels " << label->shape() << " must hold one value per row of "
+                                             << pred->shape();
+  if (scale) {
+    HT_ASSERT(grad_loss->numel() == 1) << "the gradient of a reduced loss is one value, got " << grad_loss->shape();
+  } else {
+    HT_ASSERT(int64_t(grad_loss->numel()) == rows)
+      << "labels " << label->shape() << " / grad_loss " << grad_loss->shape() << " must hold one value per row of "
+      << pred->shape();
+  }
   if (rows == 0 || cols == 0) return;
 
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
   NDArray p = Dense(pred, stream), l = Dense(label, stream), g = Dense(grad_loss, stream);
-  HK_CALL(hk_sce_sparse_bwd(int(pred->dtype()), p->raw_data_ptr(), l->data_ptr<int64_t>(), g->raw_data_ptr(),
-                            output->raw_data_ptr(), rows, cols, ignored_index, hip_stream));
+  if (scale) {
+    HK_CALL(hk_sce_sparse_bwd_reduced(int(pred->dtype()), p->raw_data_ptr(), l->data_ptr<int64_t>(),
+                                      g->raw_data_ptr(), *scale, output->raw_data_ptr(), rows, cols, ignored_index,
+                                      hip_stream));
+  } else {
+    HK_CALL(hk_sce_sparse_bwd(int(pred->dtype()), p->raw_data_ptr(), l->data_ptr<int64_t>(), g->raw_data_ptr(),
+                              output->raw_data_ptr(), rows, cols, ignored_index, hip_stream));
+  }
   NDArray::MarkUsedBy({p, l, g, output}, stream);
+}
+} // namespace
+
+void SoftmaxCrossEntropySparseGradientCuda(const NDArray& pred, const NDArray& label, const NDArray& grad_loss,
+                                           NDArray& output, const int64_t ignored_index, const Stream& stream) {
+  SparseGradient(pred, label, grad_loss, nullptr, output, ignored_index, stream);
+}
+
+// No counterpart in the reference, whose gradient op first broadcasts the one gradient value times `scale`
+// into a [rows] array (hetu/graph/ops/SoftmaxCrossEntropySparse.cc:64-85) and then calls the kernel above.
+void SoftmaxCrossEntropySparseGradientReducedCuda(const NDArray& pred, const NDArray& label,
+                                                  const NDArray& grad_output, double scale, NDArray& output,
+                                                  const int64_t ignored_index, const Stream& stream) {
+  SparseGradient(pred, label, grad_output, &scale, output, ignored_index, stream);
 }
 
 void SoftmaxCrossEntropySparseCpu(const NDArray&, const NDArray&, NDArray&, const int64_t, const Stream&) {

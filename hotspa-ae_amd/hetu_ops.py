@@ -323,6 +323,30 @@ def ndarray_sceloss(preds, labels, out, reduction="mean", ignored_index=None, st
           _i64(ignored_index if sparse else 0), ctypes.c_int(RED[reduction]), desc(out), ctypes.c_int(stream))
 
 
+# ---- gradients of the reductions and of the reduced losses ----------------
+def broadcast_shape(x, out, add_axes=(), const_value=None, stream=DEFAULT_STREAM):
+    """BroadcastShapeCuda, or BroadcastShapeMulCuda when const_value is given."""
+    ax, n = _axes(list(add_axes))
+    _call("ht_broadcast_shape", desc(x), ctypes.c_int(int(const_value is not None)),
+          ctypes.c_double(0.0 if const_value is None else const_value), desc(out), ax, n, ctypes.c_int(stream))
+
+
+def reduce_gradient(grad_output, out, reduction, axes, keepdims, stream=DEFAULT_STREAM):
+    ax, n = _axes(list(axes))
+    keep = [keepdims] if isinstance(keepdims, bool) else list(keepdims)
+    karr = (ctypes.c_int * max(len(keep), 1))(*[int(k) for k in keep])
+    _call("ht_reduce_gradient", desc(grad_output), ctypes.c_int(RED[reduction]), ax, n, karr,
+          ctypes.c_int(len(keep)), desc(out), ctypes.c_int(stream))
+
+
+def sceloss_gradient(preds, labels, grad_output, out, reduction="mean", ignored_index=None, fused=True,
+                     stream=DEFAULT_STREAM):
+    sparse = ignored_index is not None
+    _call("ht_sceloss_gradient", desc(preds), desc(labels), desc(grad_output), ctypes.c_int(int(sparse)),
+          _i64(ignored_index if sparse else 0), ctypes.c_int(RED[reduction]), ctypes.c_int(int(fused)), desc(out),
+          ctypes.c_int(stream))
+
+
 # ---- device memory pool ---------------------------------------------------
 class PoolBlock:
     def __init__(self, ptr, ident, size, device):

@@ -160,6 +160,22 @@ HT_API int ht_ndarray_layernorm(const HtArray* in, const HtArray* scale, const H
 HT_API int ht_ndarray_sceloss(const HtArray* preds, const HtArray* labels, int sparse, int64_t ignored_index,
                               int reduction, HtArray* out, int stream_index);
 
+/* ---- gradients of the reductions and of the reduced losses ---- */
+/* BroadcastShapeCuda / BroadcastShapeMulCuda (hetu/impl/kernel/BroadcastShape.cu:30-99, 119-186);
+ * multiply = 0 ignores const_value. */
+HT_API int ht_broadcast_shape(const HtArray* input, int multiply, double const_value, HtArray* output,
+                              const int64_t* add_axes, int n_add_axes, int stream_index);
+/* ReduceGradientOpImpl::DoCompute (hetu/graph/ops/Reduce.cc:153-165): output has the reduced input's shape;
+ * keepdims holds n_keepdims (= naxes, or 1 for all) flags. */
+HT_API int ht_reduce_gradient(const HtArray* grad_output, int reduction, const int64_t* axes, int naxes,
+                              const int* keepdims, int n_keepdims, HtArray* output, int stream_index);
+/* SCESGradOpImpl / SCEGradOpImpl::DoCompute (hetu/graph/ops/SoftmaxCrossEntropySparse.cc:64-85,
+ * SoftmaxCrossEntropy.cc:59-80).  sparse as in ht_ndarray_sceloss; fused = 0 runs the reference's two steps
+ * (broadcast, then the gradient kernel), 1 the single kernel that takes the one gradient value. */
+HT_API int ht_sceloss_gradient(const HtArray* preds, const HtArray* labels, const HtArray* grad_output, int sparse,
+                               int64_t ignored_index, int reduction, int fused, HtArray* output,
+                               int stream_index);
+
 /* ---- streams and the device memory pool ---- */
 HT_API int ht_stream_sync(int device_index, int stream_index);
 HT_API int ht_synchronize_all(void);

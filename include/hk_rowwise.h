@@ -344,6 +344,15 @@ HK_API int hk_sce_sparse_bwd(int dtype, const void* logits, const int64_t* label
                              const void* grad_loss, void* dlogits, int64_t rows, int64_t cols,
                              int64_t ignored_index, hkStream_t stream);
 
+/* The same with the gradient of a REDUCED loss: grad_output holds one value and every row uses
+ * round_dtype(grad_output[0] * round_dtype(scale)) -- what BroadcastShapeMul(grad, 1/rows) into a [rows]
+ * array followed by the call above computes, without that array (SCESGradOpImpl::DoCompute,
+ * hetu/graph/ops/SoftmaxCrossEntropySparse.cc:64-85; scale 1 for reduction "sum"). */
+HK_API int hk_sce_sparse_bwd_reduced(int dtype, const void* logits, const int64_t* labels,
+                                     const void* grad_output, double scale, void* dlogits,
+                                     int64_t rows, int64_t cols, int64_t ignored_index,
+                                     hkStream_t stream);
+
 /* Dense (soft / one-hot) labels of the logits' shape:
  *   loss[r] = -sum_c labels[r,c] * log_softmax(x[r,:])[c]
  *   dlogits = (softmax(x) - labels) * grad_loss[r]
@@ -354,6 +363,12 @@ HK_API int hk_sce_dense_fwd(int dtype, const void* logits, const void* labels, v
 HK_API int hk_sce_dense_bwd(int dtype, const void* logits, const void* labels,
                             const void* grad_loss, void* dlogits, int64_t rows, int64_t cols,
                             hkStream_t stream);
+
+/* Dense labels, gradient of a reduced loss (SoftmaxCrossEntropyGradientOpImpl::DoCompute,
+ * hetu/graph/ops/SoftmaxCrossEntropy.cc:59-80); see hk_sce_sparse_bwd_reduced. */
+HK_API int hk_sce_dense_bwd_reduced(int dtype, const void* logits, const void* labels,
+                                    const void* grad_output, double scale, void* dlogits,
+                                    int64_t rows, int64_t cols, hkStream_t stream);
 
 /* ======================================================================== *
  * Negative log-likelihood loss on log-probabilities, int64 class labels.
@@ -437,6 +452,15 @@ HK_API int hk_binary_const(int op, int dtype, const void* in, double scalar, int
 HK_API int hk_binary(int op, int dtype, const void* a, const void* b, void* out, int ndim,
                      const int64_t* out_shape, const int64_t* a_strides, const int64_t* b_strides,
                      hkStream_t stream);
+
+/* out = in broadcast to out_shape (dense), optionally times `scalar` (rounded to `dtype` first, as
+ * static_cast<spec_t>(const_value) does).  in_strides holds, per output dimension, the input's stride in
+ * elements, 0 where the input is broadcast along that dimension; a strided input view is read in place.
+ * The backward of Reduce sum / mean and of every reduced loss.
+ * Replaces broadcast_shape_kernel / broadcast_shape_mul_kernel and their launchers BroadcastShapeCuda /
+ * BroadcastShapeMulCuda (hetu/impl/kernel/BroadcastShape.cu:11-28, 30-99, 101-117, 119-186). */
+HK_API int hk_broadcast(int dtype, const void* in, int multiply, double scalar, void* out, int ndim,
+                        const int64_t* out_shape, const int64_t* in_strides, hkStream_t stream);
 
 /* ======================================================================== *
  * Reduce sum / mean / max / min / product over a set of axes of a (possibly

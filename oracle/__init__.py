@@ -273,6 +273,39 @@ def norm_p_bwd(x, norm, grad, dim, p):
     return np.where(n == 0, 0.0, out)
 
 
+def broadcast_shape(x, out_shape, add_axes=(), const_value=None):
+    """broadcast_shape_kernel / broadcast_shape_mul_kernel with the host set-up of BroadcastShapeCuda
+    (hetu/impl/kernel/BroadcastShape.cu:11-28, 44-68, 101-117): per output dimension an input extent in_dims[i]
+    (1 where the input is laid over a dimension it lacks or broadcasts), and for every output element the flat
+    input index  i_ind = sum over dimensions of (in_dims[i] > 1) * coordinate, in row-major order of in_dims.
+    Index arithmetic as the kernel does it, one output element at a time; float64 product."""
+    x = np.asarray(x)
+    out_nd, diff = len(out_shape), len(out_shape) - x.ndim
+    if not add_axes:
+        in_dims = [1 if i < diff else x.shape[i - diff] for i in range(out_nd)]
+    else:
+        in_dims = [0] * out_nd
+        for i in range(diff):
+            in_dims[add_axes[i]] = 1
+        o_ind = 0
+        for i in range(x.ndim):
+            while in_dims[o_ind] == 1:
+                o_ind += 1
+            in_dims[o_ind] = x.shape[i]
+            o_ind += 1
+    out_strides = [int(np.prod(out_shape[i + 1:], dtype=np.int64)) for i in range(out_nd)]
+    flat = x.reshape(-1)
+    size = int(np.prod(out_shape, dtype=np.int64))
+    out = np.empty(size, dtype=np.float64)
+    for idx in range(size):
+        i_ind, temp = 0, idx
+        for i in range(out_nd):
+            i_ind = i_ind * in_dims[i] + (temp // out_strides[i] if in_dims[i] > 1 else 0)
+            temp %= out_strides[i]
+        out[idx] = float(flat[i_ind]) * (1.0 if const_value is None else float(const_value))
+    return out.reshape(out_shape)
+
+
 def batch_norm_fwd(x, scale, bias, running_mean, running_var, momentum, eps):
     """Spatial batch normalisation in training mode as cuDNN documents it for
     cudnnBatchNormalizationForwardTraining(CUDNN_BATCHNORM_SPATIAL) (called at

@@ -1,0 +1,217 @@
+"""GPU parity of the gradient side of the reductions and of the reduced losses: hk_broadcast (BroadcastShape /
+BroadcastShapeMul), the cross-entropy gradients that take the one gradient value of a reduced loss, and the
+operator-level functions built from them (ReduceGradient, the loss gradients)."""
+import importlib
+
+import numpy as np
+import pytest
+
+import helpers
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["fp32", "bf16", "fp16", "fp64"]
+# (input shape, output shape): every operand mode of the two-dimensional kernel, the generic kernel
+# (middle-dimension broadcast, ragged columns) and a plain copy
+BROADCASTS = [((1,), (4096,)), ((1,), (33, 7)), ((64, 1), (64, 512)), ((512,), (64, 512)), ((64, 512), (64, 512)),
+              ((3, 1, 40), (3, 5, 40)), ((6, 1), (6, 37)), ((2, 1, 1, 8), (2, 3, 4, 8)), ((1, 1), (1, 1))]
+
+
+@pytest.fixture(scope="module")
+def ops(hk):
+    return importlib.import_module("hotspa-ae_amd.hetu_ops")
+
+
+def _draw(seed, shape, dtype):
+    x = helpers.rng(seed).standard_normal(shape).astype(np.float32)      # the oracle takes float32 operands
+    return x.astype(np.float64) if dtype == "fp64" else oracle.round_to(x, dtype)
+
+
+def _rounded(v, dtype):
+    v = np.asarray(v, np.float32)
+    return v.astype(np.float64) if dtype == "fp64" else oracle.round_to(v, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shapes", BROADCASTS, ids=str)
+def test_broadcast_bit_exact(hk, cuda, dtype, shapes):
+    """A copy moves bits; the product of two values of a 16-bit type is exact in fp32, so rounding it once to the
+    storage type is the correctly rounded product, which numpy forms from the same operands in float64."""
+    import torch
+    sin, sout = shapes
+    x = _draw(11 + len(sout), sin, dtype)
+    tx = helpers.to_torch(x, dtype, cuda)
+    out = torch.empty(sout, dtype=tx.dtype, device=cuda)
+    hk.broadcast(tx, out)
+    torch.cuda.synchronize()
+    want = oracle.broadcast_shape(x, sout)
+    assert np.array_equal(helpers.to_numpy(out).astype(np.float64), want)
+    c = 1.0 / 3.0
+    cr = c if dtype == "fp64" else float(_rounded([c], dtype)[0])
+    hk.broadcast(tx, out, scalar=c)
+    torch.cuda.synchronize()
+    if dtype == "fp32":
+        want = (np.broadcast_to(x, sout).astype(np.float32) * np.float32(cr)).astype(np.float64)
+    else:
+        want = oracle.broadcast_shape(x, sout, const_value=cr)
+        want = want if dtype == "fp64" else oracle.round_to(want.astype(np.float32), dtype).astype(np.float64)
+    assert np.array_equal(helpers.to_numpy(out).astype(np.float64), want)
+
+
+def test_broadcast_strided_input_and_refusals(hk, cuda):
+    import torch
+    base = torch.randn(40, 6, device=cuda)
+    out = torch.empty(6, 40, device=cuda)
+    hk.broadcast(base.t(), out)                              # transposed view, read in place
+    torch.cuda.synchronize()
+    assert torch.equal(out, base.t())
+    col = base[:, 2:3]                                       # [40, 1] with row stride 6
+    wide = torch.empty(40, 128, device=cuda)
+    hk.broadcast(col, wide, scalar=2.0)
+    torch.cuda.synchronize()
+    assert torch.equal(wide, (col * 2.0).expand(40, 128))
+    e = torch.empty(0, 8, device=cuda)
+    hk.broadcast(torch.ones(1, device=cuda), e)              # empty output: nothing to do
+    with pytest.raises(hk.HkError) as err:
+        hk.broadcast(base.t().long(), out.long())
+    assert err.value.code == -2
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(64, 1000), (33, 4096), (5, 37), (16, 32000)])
+def test_reduced_loss_gradient_equals_two_step_form(hk, cuda, dtype, rows, cols):
+    """The kernel fed (one gradient value, 1/rows) against the reference's sequence on the same inputs (broadcast
+    the value times 1/rows into a [rows] array, then the per-row gradient kernel): the same bits, sparse and dense."""
+    import torch
+    g = helpers.rng(rows + cols)
+    x = _draw(rows * 3 + cols, (rows, cols), dtype) * 3
+    x = _rounded(x, dtype)
+    labels = g.integers(0, cols, rows)
+    labels[::5] = -100
+    tx = helpers.to_torch(x, dtype, cuda)
+    tl = torch.tensor(labels, device=cuda)
+    grad = helpers.to_torch(_rounded([0.7], dtype), dtype, cuda)
+    scale = float(np.float32(1.0) / np.float32(rows))
+    per_row = torch.empty(rows, dtype=tx.dtype, device=cuda)
+    hk.broadcast(grad, per_row, scalar=scale)
+    two_step, fused = torch.empty_like(tx), torch.empty_like(tx)
+    hk.sce_sparse_bwd(tx, tl, per_row, two_step, -100)
+    hk.sce_sparse_bwd_reduced(tx, tl, grad, scale, fused, -100)
+    torch.cuda.synchronize()
+    assert torch.equal(two_step.view(torch.uint8), fused.view(torch.uint8))
+    assert (fused[::5] == 0).all()
+    # against the oracle with the per-row value as stored
+    gr = helpers.to_numpy(per_row).astype(np.float64)
+    # the oracle takes float32 gradients; it is linear in them, so scale its unit-gradient answer instead
+    ones = np.ones(rows)
+    helpers.assert_close(fused, oracle.sce_sparse_bwd(x, labels, ones, -100) * gr[:, None], dtype, "sparse gradient")
+    soft = np.abs(g.standard_normal((rows, cols))) + 0.01
+    soft = _rounded(soft / soft.sum(1, keepdims=True), dtype)
+    ts = helpers.to_torch(soft, dtype, cuda)
+    hk.sce_dense_bwd(tx, ts, per_row, two_step)
+    hk.sce_dense_bwd_reduced(tx, ts, grad, scale, fused)
+    torch.cuda.synchronize()
+    assert torch.equal(two_step.view(torch.uint8), fused.view(torch.uint8))
+    helpers.assert_close(fused, oracle.sce_dense_bwd(x, soft, ones) * gr[:, None], dtype, "dense gradient")
+
+
+# ---- operator layer ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("case", [((4, 5), (3, 4, 5), ()), ((3, 5), (3, 4, 5), (1,)), ((4,), (3, 4, 5), (0, 2)),
+                                  ((3, 1, 5), (3, 4, 5), (1,)), ((1,), (2, 3), ())], ids=str)
+def test_broadcast_shape_entry_points(ops, cuda, dtype, case):
+    import torch
+    sin, sout, add_axes = case
+    x = _draw(5, sin, dtype)
+    tx = helpers.to_torch(x, dtype, cuda)
+    out = torch.empty(sout, dtype=tx.dtype, device=cuda)
+    torch.cuda.synchronize()
+    ops.broadcast_shape(tx, out, add_axes)
+    ops.stream_sync()
+    assert np.array_equal(helpers.to_numpy(out).astype(np.float64), oracle.broadcast_shape(x, sout, add_axes))
+    ops.broadcast_shape(tx, out, add_axes, const_value=0.5)
+    ops.stream_sync()
+    assert np.array_equal(helpers.to_numpy(out).astype(np.float64), oracle.broadcast_shape(x, sout, add_axes, 0.5))
+
+
+def test_broadcast_shape_refusals(ops, cuda):
+    import torch
+    out = torch.empty(3, 4, 5, device=cuda)
+    with pytest.raises(ops.AssertionError_, match="does not broadcast"):
+        ops.broadcast_shape(torch.ones(3, 4, device=cuda), out, (1,))      # [3,4] laid over dims 0 and 2
+    with pytest.raises(ops.AssertionError_, match="more dimensions"):
+        ops.broadcast_shape(torch.ones(1, 3, 4, 5, device=cuda), out)
+    with pytest.raises(ops.AssertionError_, match="outside the output"):
+        ops.broadcast_shape(torch.ones(4, 5, device=cuda), out, (3,))
+
+
+@pytest.mark.parametrize("reduction", ["sum", "mean"])
+@pytest.mark.parametrize("axes,keepdims", [((0,), False), ((1,), False), ((2,), True), ((0, 2), False),
+                                           ((0, 1, 2), False), ((), False), ((1, 2), True), ((-1,), False)], ids=str)
+def test_reduce_gradient_is_autograd_of_the_reduction(ops, cuda, reduction, axes, keepdims):
+    import torch
+    shape = (6, 5, 8)
+    dims = tuple(axes) if axes else (0, 1, 2)
+    t = torch.randn(shape, dtype=torch.float64, requires_grad=True)
+    red = (t.sum if reduction == "sum" else t.mean)(dim=dims, keepdim=keepdims)
+    grad = torch.randn(red.shape, dtype=torch.float64)
+    (red * grad).sum().backward()
+    g_dev = grad.to(torch.float32).to(cuda)
+    if g_dev.ndim == 0:
+        g_dev = g_dev.reshape(1)                                 # a full reduction's output is [1]
+    out = torch.empty(shape, device=cuda)
+    torch.cuda.synchronize()
+    ops.reduce_gradient(g_dev, out, reduction, axes, keepdims)
+    ops.stream_sync()
+    helpers.assert_close(out, t.grad.numpy(), "fp32", "reduce gradient")
+    with pytest.raises(ops.AssertionError_, match="only the sum and the mean"):
+        ops.reduce_gradient(g_dev, out, "max", axes, keepdims)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
+@pytest.mark.parametrize("sparse", [True, False])
+def test_loss_gradient_ops(ops, cuda, dtype, reduction, sparse):
+    """Gradient of NDArray::sceloss through the operator-level function: the two-step and the single-kernel form
+    agree bit for bit, and both are the oracle's gradient for the per-row value 1/rows (mean), 1 (sum) or the
+    given rows (none), times the incoming gradient."""
+    import torch
+    lead, cols = (4, 9), 515
+    rows = lead[0] * lead[1]
+    g = helpers.rng(77)
+    x = _rounded(_draw(3, lead + (cols,), dtype) * 2, dtype)
+    tx = helpers.to_torch(x, dtype, cuda)
+    if sparse:
+        labels = g.integers(0, cols, lead)
+        labels[0, ::4] = -1
+        tl = torch.tensor(labels, device=cuda)
+    else:
+        soft = np.abs(g.standard_normal(lead + (cols,))) + 0.01
+        labels = _rounded(soft / soft.sum(-1, keepdims=True), dtype)
+        tl = helpers.to_torch(labels, dtype, cuda)
+    if reduction == "none":
+        go = _rounded(g.standard_normal(lead), dtype)
+        per_row = go.astype(np.float64).reshape(-1)
+    else:
+        go = _rounded([1.25], dtype)
+        factor = float(_rounded([np.float32(1.0) / np.float32(rows)], dtype)[0]) if reduction == "mean" else 1.0
+        per_row = np.full(rows, float(_rounded([float(go[0]) * factor], dtype)[0]))
+    tg = helpers.to_torch(go, dtype, cuda)
+    outs = []
+    for fused in (False, True):
+        out = torch.empty_like(tx)
+        torch.cuda.synchronize()
+        ops.sceloss_gradient(tx, tl, tg, out, reduction, ignored_index=-1 if sparse else None, fused=fused)
+        ops.stream_sync()
+        outs.append(out)
+    assert torch.equal(outs[0].view(torch.uint8), outs[1].view(torch.uint8))
+    x2 = x.reshape(rows, cols)
+    ones = np.ones(rows)
+    want = (oracle.sce_sparse_bwd(x2, labels.reshape(-1), ones, -1) if sparse
+            else oracle.sce_dense_bwd(x2, labels.reshape(rows, cols), ones)) * per_row[:, None]
+    helpers.assert_close(outs[1].reshape(rows, cols), want, dtype, "loss gradient")
+    if reduction != "none":
+        with pytest.raises(ops.AssertionError_, match="one value"):
+            ops.sceloss_gradient(tx, tl, torch.ones(2, dtype=tx.dtype, device=cuda), outs[0], reduction,
+                                 ignored_index=-1 if sparse else None, fused=True)

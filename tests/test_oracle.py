@@ -415,3 +415,28 @@ def test_batch_norm_against_torch():
     np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-10, atol=1e-12)
     np.testing.assert_allclose(dscale, ts.grad.numpy(), rtol=1e-11)
     np.testing.assert_allclose(dbias, tb.grad.numpy(), rtol=1e-11)
+
+
+@pytest.mark.parametrize("case", [
+    ((4, 5), (3, 4, 5), ()), ((1, 5), (3, 4, 5), ()), ((1,), (2, 3), ()), ((4, 1), (3, 4, 5), ()),
+    ((3, 5), (3, 4, 5), (1,)), ((4,), (3, 4, 5), (0, 2)), ((3,), (3, 4, 5), (1, 2)), ((5,), (3, 4, 5), (0, 1)),
+    ((3, 1, 5), (3, 4, 5), (1,)),     # keepdims: no dimension to add, the axis list is not consulted
+], ids=str)
+def test_broadcast_shape_is_numpy_broadcasting(case):
+    """oracle.broadcast_shape's index arithmetic against numpy's own broadcasting, with the dropped dimensions put
+    back by expand_dims (an independent statement of the same layout), and against torch autograd of sum / mean,
+    whose gradient is this broadcast (times 1/n for the mean)."""
+    import torch
+    in_shape, out_shape, add_axes = case
+    g = np.random.default_rng(len(in_shape) * 7 + len(add_axes))
+    x = g.standard_normal(in_shape)
+    diff = len(out_shape) - len(in_shape)
+    want = np.broadcast_to(np.expand_dims(x, tuple(add_axes[:diff])) if add_axes else x, out_shape)
+    np.testing.assert_array_equal(oracle.broadcast_shape(x, out_shape, add_axes), want)
+    np.testing.assert_allclose(oracle.broadcast_shape(x, out_shape, add_axes, 0.25), want * 0.25, rtol=0)
+    if add_axes and diff == len(add_axes):
+        t = torch.zeros(out_shape, dtype=torch.float64, requires_grad=True)
+        (t.mean(dim=tuple(add_axes)) * torch.tensor(x)).sum().backward()
+        n = np.prod([out_shape[a] for a in add_axes])
+        np.testing.assert_allclose(oracle.broadcast_shape(x, out_shape, add_axes, 1.0 / n), t.grad.numpy(),
+                                   rtol=1e-15)

@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "hetu/core/ndarray.h"
+#include "hetu/graph/ops/gradient_compute.h"
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/memory/CachingMemoryPool.h"
 #include "hetu/impl/stream/HIPStream.h"
@@ -224,6 +225,45 @@ int main() {
     }
     CHECK(max_rel(got, wantg) < 1e-5);
     CHECK(throws<assertion_error>([&] { NDArray::add(shard[0], NDArray::slice(d, {0, 0}, {rows, half - 1})); }));
+  });
+
+  run("gradient of the mean cross-entropy: the loss op's two steps and the single kernel agree", [&] {
+    NDArray d = NDArray::cuda(host_f32({rows, cols}, x));
+    NDArray lab = NDArray::empty({rows}, Device(kCPU), kInt64);
+    for (int64_t r = 0; r < rows; ++r) lab->data_ptr<int64_t>()[r] = (r % 5 == 0) ? -100 : (r * 131) % cols;
+    NDArray labels = NDArray::cuda(lab);
+    NDArray grad_output = NDArray::cuda(host_f32({1}, std::vector<float>{1.5f}));
+    NDArray none;
+    NDArray two_step = hetu::graph::SCESGradCompute(d, labels, grad_output, -100, kMEAN, NDArray::DEFAULT_STREAM,
+                                                    none, /*fused=*/false);
+    NDArray fused = hetu::graph::SCESGradCompute(d, labels, grad_output, -100, kMEAN, NDArray::DEFAULT_STREAM, none,
+                                                 /*fused=*/true);
+    std::vector<float> a = fetch_f32(two_step), b = fetch_f32(fused);
+    CHECK(a == b);
+    const float per_row = 1.5f * (1.0f / float(rows));
+    std::vector<double> want(rows * cols);
+    for (int64_t r = 0; r < rows; ++r) {
+      const int64_t l = lab->data_ptr<int64_t>()[r];
+      double m = -1e300, sum = 0;
+      for (int64_t c = 0; c < cols; ++c) m = std::max<double>(m, x[r * cols + c]);
+      for (int64_t c = 0; c < cols; ++c) sum += std::exp(x[r * cols + c] - m);
+      for (int64_t c = 0; c < cols; ++c)
+        want[r * cols + c] = l < 0 ? 0.0 : (std::exp(x[r * cols + c] - m) / sum - (c == l ? 1.0 : 0.0)) * per_row;
+    }
+    CHECK(max_rel(b, want) < 1e-5);
+    // gradient of a mean over the columns: every element of a row gets grad[r] / cols
+    std::vector<float> gr(rows);
+    for (int64_t r = 0; r < rows; ++r) gr[r] = float(r + 1);
+    NDArray back = hetu::graph::ReduceGradientCompute(NDArray::cuda(host_f32({rows}, gr)), {rows, cols}, kMEAN, {-1},
+                                                      {false}, NDArray::DEFAULT_STREAM, none);
+    std::vector<float> got = fetch_f32(back);
+    for (int64_t r = 0; r < rows; ++r)
+      for (int64_t c = 0; c < cols; c += 97) CHECK(std::fabs(got[r * cols + c] - gr[r] / cols) <= 1e-6 * gr[r] / cols);
+    CHECK(throws<assertion_error>([&] {
+      NDArray out = NDArray::empty({rows, cols}, gpu, kFloat32);
+      hetu::impl::BroadcastShapeCuda(NDArray::cuda(host_f32({rows - 1}, std::vector<float>(rows - 1, 0.f))), out,
+                                     {1}, Stream(gpu, NDArray::DEFAULT_STREAM));
+    }));
   });
 
   run("reductions: sum / mean / max with keepdims, all dims", [&] {

@@ -50,12 +50,33 @@ struct BnShape {
   int splits;
 };
 
-// address of load `v` (0 <= v < per_channel) of channel c
-__device__ __forceinline__ int64_t bn_offset(const BnShape& s, int64_t c, int64_t v, int V) {
-  const int64_t n = v / s.hw_vec;
-  const int64_t off = v - n * s.hw_vec;
-  return (n * s.C + c) * s.HW + off * V;
-}
+// A thread's walk over the loads v0, v0 + stride, v0 + 2 stride, ... (< per_channel) of channel c: the element
+// offset of the current load, kept up by additions (one division per thread at the start, none per load).
+struct BnWalk {
+  int64_t off;        // element offset of the current load
+  int64_t in_plane;   // its load index inside its H*W plane
+  int64_t left;       // loads still to do, the current one included
+  int64_t step_off, step_in_plane, wrap_off, hw_vec;
+  __device__ __forceinline__ BnWalk(const BnShape& s, int64_t c, int64_t v0, int64_t stride, int V) {
+    const int64_t n = v0 / s.hw_vec;
+    in_plane = v0 - n * s.hw_vec;
+    off = (n * s.C + c) * s.HW + in_plane * V;
+    left = v0 < s.per_channel ? (s.per_channel - v0 + stride - 1) / stride : 0;
+    const int64_t q = stride / s.hw_vec;                 // whole planes per step
+    step_in_plane = stride - q * s.hw_vec;
+    step_off = q * s.C * s.HW + step_in_plane * V;
+    wrap_off = (s.C - 1) * s.HW;                         // from the end of a plane to the same channel of the next image
+    hw_vec = s.hw_vec;
+  }
+  __device__ __forceinline__ void next() {
+    in_plane += step_in_plane;
+    off += step_off;
+    const bool wrap = in_plane >= hw_vec;
+    in_plane -= wrap ? hw_vec : 0;
+    off += wrap ? wrap_off : 0;
+    --left;
+  }
+};
 
 template <typename CT>
 __device__ __forceinline__ CT block_sum(CT v, CT* lds) {
@@ -78,23 +99,30 @@ void bn_stats_kernel(const T* __restrict__ x, BnShape s, CT* __restrict__ part) 
   __shared__ CT lds[256];
   const int64_t c = blockIdx.x;
   const int split = blockIdx.y;
-  // per-thread Welford over whole loads: each load's V values are folded in as one group (Chan's update)
+  // per thread: sums of (x - K) and (x - K)^2 about a pivot K taken from the thread's first load, so that a
+  // large common offset of the channel never enters a sum; no division inside the loop
+  BnWalk w(s, c, int64_t(split) * 256 + threadIdx.x, int64_t(s.splits) * 256, V);
   CT cnt = 0, mean = 0, m2 = 0;
-  for (int64_t v = int64_t(split) * 256 + threadIdx.x; v < s.per_channel; v += int64_t(s.splits) * 256) {
+  if (w.left > 0) {
     CT f[V];
-    bn_load<T, V, CT>(x + bn_offset(s, c, v, V), f);
-    CT gs = 0;
+    bn_load<T, V, CT>(x + w.off, f);
+    CT K = 0;
 #pragma unroll
-    for (int j = 0; j < V; ++j) gs += f[j];
-    const CT gm = gs / CT(V);
-    CT g2 = 0;
+    for (int j = 0; j < V; ++j) K += f[j];
+    K /= CT(V);
+    CT s1 = 0, s2 = 0;
 #pragma unroll
-    for (int j = 0; j < V; ++j) { const CT d = f[j] - gm; g2 += d * d; }
-    const CT n = cnt + CT(V);
-    const CT delta = gm - mean;
-    mean += delta * (CT(V) / n);
-    m2 += g2 + delta * delta * (cnt * CT(V) / n);
-    cnt = n;
+    for (int j = 0; j < V; ++j) { const CT d = f[j] - K; s1 += d; s2 += d * d; }
+    cnt = CT(V);
+    for (w.next(); w.left > 0; w.next()) {
+      bn_load<T, V, CT>(x + w.off, f);
+#pragma unroll
+      for (int j = 0; j < V; ++j) { const CT d = f[j] - K; s1 += d; s2 += d * d; }
+      cnt += CT(V);
+    }
+    mean = K + s1 / cnt;
+    m2 = s2 - s1 * (s1 / cnt);
+    m2 = m2 > 0 ? m2 : CT(0);
   }
   // block merge: total count and mean first, then M2 about the block mean
   const CT bcnt = block_sum<CT>(cnt, lds);
@@ -145,20 +173,63 @@ void bn_finalize_kernel(const CT* __restrict__ part, int64_t C, int splits, cons
   coef[2 * C + c] = CT(bias[c]);
 }
 
+// One load of V elements as it comes from memory; unpacked only after every load of the thread is issued.
+template <typename T, int V>
+struct BnRaw {
+  u32x4 vec;
+  T one;
+  __device__ __forceinline__ void load(const T* p) {
+    if constexpr (V == 1) one = *p;
+    else vec = ld16(p);
+  }
+  template <typename CT>
+  __device__ __forceinline__ void unpack(CT* f) const {
+    if constexpr (V == 1) {
+      f[0] = CT(Cvt<T>::load(&one));
+    } else {
+      float t[V];
+      VecIO<T>::unpack(vec, t);
+#pragma unroll
+      for (int j = 0; j < V; ++j) f[j] = t[j];
+    }
+  }
+};
+
+// Channel of load v of a dense [N, C, H*W] array, and whether the whole wavefront shares it (it does unless the
+// wavefront crosses from one plane into the next): then the channel's coefficients are fetched once per
+// wavefront through the scalar unit instead of once per lane.
+template <typename IT>
+__device__ __forceinline__ IT bn_channel(IT v, IT hw_vec, IT C, bool& uniform) {
+  const IT plane = v / hw_vec;
+  const IT plane0 = IT(__builtin_amdgcn_readfirstlane(uint32_t(plane)));
+  uniform = __builtin_amdgcn_ballot_w64(plane != plane0) == 0;
+  return uniform ? plane0 % C : plane % C;
+}
+
 // y = (x - mean) * (scale * invstd) + bias; the mean is subtracted first: folding it into the constant term
-// would cancel badly for a channel whose mean is large against its spread
-template <typename T, int V, typename CT>
+// would cancel badly for a channel whose mean is large against its spread.  IT: index type (32-bit when the
+// array allows it: the per-lane division is then a few instructions).
+template <typename T, int V, typename CT, typename IT>
 __global__ __launch_bounds__(256)
-void bn_apply_kernel(const T* x, T* y, const CT* __restrict__ coef, int64_t total_loads, int64_t hw_vec, int64_t C) {
-  const int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+void bn_apply_kernel(const T* x, T* y, const CT* __restrict__ coef, IT total_loads, IT hw_vec, IT C) {
+  const IT v = IT(blockIdx.x) * 256 + threadIdx.x;
   if (v >= total_loads) return;
-  const int64_t c = (v / hw_vec) % C;
-  const CT a = coef[c], mean = coef[C + c], b = coef[2 * C + c];
+  BnRaw<T, V> rx;
+  rx.load(x + size_t(v) * V);
+  bool uniform;
+  const IT c = bn_channel<IT>(v, hw_vec, C, uniform);
+  CT a, mean, b;
+  if (uniform) {
+    const IT c0 = IT(__builtin_amdgcn_readfirstlane(uint32_t(c)));
+    a = coef[c0]; mean = coef[size_t(C) + c0]; b = coef[2 * size_t(C) + c0];
+  } else {
+    a = coef[c]; mean = coef[size_t(C) + c]; b = coef[2 * size_t(C) + c];
+  }
   CT f[V];
-  bn_load<T, V, CT>(x + v * V, f);
+  rx.unpack(f);
 #pragma unroll
   for (int j = 0; j < V; ++j) f[j] = (f[j] - mean) * a + b;
-  bn_store<T, V, CT>(y + v * V, f);
+  bn_store<T, V, CT>(y + size_t(v) * V, f);
 }
 
 // per-channel partial sums of dy and dy * (x - mean) * invstd -> part[(c * splits + split) * 2 ..]
@@ -172,11 +243,10 @@ void bn_bwd_stats_kernel(const T* __restrict__ dy, const T* __restrict__ x, BnSh
   const int split = blockIdx.y;
   const CT mean = CT(save_mean[c]), invstd = CT(save_invstd[c]);
   CT sdy = 0, sdyx = 0;
-  for (int64_t v = int64_t(split) * 256 + threadIdx.x; v < s.per_channel; v += int64_t(s.splits) * 256) {
-    const int64_t off = bn_offset(s, c, v, V);
+  for (BnWalk w(s, c, int64_t(split) * 256 + threadIdx.x, int64_t(s.splits) * 256, V); w.left > 0; w.next()) {
     CT g[V], f[V];
-    bn_load<T, V, CT>(dy + off, g);
-    bn_load<T, V, CT>(x + off, f);
+    bn_load<T, V, CT>(dy + w.off, g);
+    bn_load<T, V, CT>(x + w.off, f);
 #pragma unroll
     for (int j = 0; j < V; ++j) { sdy += g[j]; sdyx += g[j] * ((f[j] - mean) * invstd); }
   }
@@ -212,20 +282,30 @@ void bn_bwd_finalize_kernel(const CT* __restrict__ part, int64_t C, int splits, 
   coef[3 * C + c] = mean;
 }
 
-template <typename T, int V, typename CT>
+template <typename T, int V, typename CT, typename IT>
 __global__ __launch_bounds__(256)
-void bn_bwd_apply_kernel(const T* dy, const T* x, T* dx, const CT* __restrict__ coef, int64_t total_loads,
-                         int64_t hw_vec, int64_t C) {
-  const int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+void bn_bwd_apply_kernel(const T* dy, const T* x, T* dx, const CT* __restrict__ coef, IT total_loads, IT hw_vec,
+                         IT C) {
+  const IT v = IT(blockIdx.x) * 256 + threadIdx.x;
   if (v >= total_loads) return;
-  const int64_t c = (v / hw_vec) % C;
-  const CT k0 = coef[c], k1 = coef[C + c], k2 = coef[2 * C + c], mean = coef[3 * C + c];
+  BnRaw<T, V> rg, rx;
+  rg.load(dy + size_t(v) * V);
+  rx.load(x + size_t(v) * V);
+  bool uniform;
+  const IT c = bn_channel<IT>(v, hw_vec, C, uniform);
+  CT k0, k1, k2, mean;
+  if (uniform) {
+    const IT c0 = IT(__builtin_amdgcn_readfirstlane(uint32_t(c)));
+    k0 = coef[c0]; k1 = coef[size_t(C) + c0]; k2 = coef[2 * size_t(C) + c0]; mean = coef[3 * size_t(C) + c0];
+  } else {
+    k0 = coef[c]; k1 = coef[size_t(C) + c]; k2 = coef[2 * size_t(C) + c]; mean = coef[3 * size_t(C) + c];
+  }
   CT g[V], f[V];
-  bn_load<T, V, CT>(dy + v * V, g);
-  bn_load<T, V, CT>(x + v * V, f);
+  rg.unpack(g);
+  rx.unpack(f);
 #pragma unroll
   for (int j = 0; j < V; ++j) g[j] = k0 * g[j] + (k1 * (f[j] - mean) + k2);
-  bn_store<T, V, CT>(dx + v * V, g);
+  bn_store<T, V, CT>(dx + size_t(v) * V, g);
 }
 
 // ---------------------------------------------------------------------------
@@ -283,8 +363,13 @@ static int bn_fwd_typed(const void* x, const void* scale, const void* bias, void
     if (rc != HK_OK) return rc;
     const int64_t loads = N * C * s.hw_vec;
     profile_before(st);
-    hipLaunchKernelGGL((bn_apply_kernel<T, V, CT>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st, xp, yp,
-                       coef, loads, s.hw_vec, C);
+    if (loads < 0x7fffffffLL) {
+      hipLaunchKernelGGL((bn_apply_kernel<T, V, CT, uint32_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st,
+                         xp, yp, coef, uint32_t(loads), uint32_t(s.hw_vec), uint32_t(C));
+    } else {
+      hipLaunchKernelGGL((bn_apply_kernel<T, V, CT, int64_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st,
+                         xp, yp, coef, loads, s.hw_vec, C);
+    }
     profile_after(st);
     return launch_check("bn_apply_kernel");
   };
@@ -322,9 +407,15 @@ static int bn_bwd_typed(const void* dy, const void* x, const void* scale, void* 
     if (rc != HK_OK) return rc;
     const int64_t loads = N * C * s.hw_vec;
     profile_before(st);
-    hipLaunchKernelGGL((bn_bwd_apply_kernel<T, V, CT>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st,
-                       static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<T*>(dx), coef, loads,
-                       s.hw_vec, C);
+    if (loads < 0x7fffffffLL) {
+      hipLaunchKernelGGL((bn_bwd_apply_kernel<T, V, CT, uint32_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0,
+                         st, static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<T*>(dx), coef,
+                         uint32_t(loads), uint32_t(s.hw_vec), uint32_t(C));
+    } else {
+      hipLaunchKernelGGL((bn_bwd_apply_kernel<T, V, CT, int64_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0,
+                         st, static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<T*>(dx), coef, loads,
+                         s.hw_vec, C);
+    }
     profile_after(st);
     return launch_check("bn_bwd_apply_kernel");
   };

@@ -34,22 +34,23 @@ void vocab_ce_gather_kernel(const T* __restrict__ logits, const int64_t* __restr
 template <typename T>
 __global__ __launch_bounds__(256)
 void vocab_ce_bwd_vec_kernel(const T* softmax, const int64_t* __restrict__ labels, const T* __restrict__ grad_loss,
-                             T* out, int64_t nvec, int64_t cols_vec, int64_t vocab_start) {
+                             T* out, uint32_t nvec, uint32_t cols_vec, int64_t vocab_start) {
   constexpr int VEC = VecIO<T>::N;
-  const int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
   if (v >= nvec) return;
-  const int64_t r = v / cols_vec;
-  const int64_t c0 = (v - r * cols_vec) * VEC;
-  const u32x4 raw = ld16(softmax + v * VEC);
-  // position of the label inside this vector, or a value no j reaches (labels outside the shard, negative ones)
-  const uint64_t rel = uint64_t(labels[r]) - uint64_t(vocab_start) - uint64_t(c0);
-  const uint32_t hit = rel < uint64_t(VEC) ? uint32_t(rel) : 0xffffffffu;
+  const uint32_t r = v / cols_vec;
+  const uint32_t c0 = (v - r * cols_vec) * VEC;
+  const u32x4 raw = ld16(softmax + size_t(v) * VEC);
+  const int64_t label = labels[r];
   const float g = Cvt<T>::load(grad_loss + r);
+  // position of the label inside this vector, or a value no j reaches (labels outside the shard, negative ones)
+  const uint64_t rel = uint64_t(label) - uint64_t(vocab_start) - uint64_t(c0);
+  const uint32_t hit = rel < uint64_t(VEC) ? uint32_t(rel) : 0xffffffffu;
   float f[VEC];
   VecIO<T>::unpack(raw, f);
 #pragma unroll
   for (int j = 0; j < VEC; ++j) f[j] = (uint32_t(j) == hit ? f[j] - 1.0f : f[j]) * g;
-  st16_stream(out + v * VEC, VecIO<T>::pack(f));
+  st16_stream(out + size_t(v) * VEC, VecIO<T>::pack(f));
 }
 
 template <typename T, typename CT>
@@ -112,9 +113,20 @@ void vocab_ce_bwd_fused_kernel(const T* x, const int64_t* __restrict__ labels, c
   // all four loads are issued before any is waited for; an ignored row is read like the others (a branch on
   // the label around the vector load would put the two loads in series) and its result replaced by zeros
   const u32x4 raw = ld16(x + size_t(v) * VEC);
-  const int64_t label = labels[r];
-  const float l2 = lse[r] * kLog2e;
-  float g = Cvt<T>::load(grad_loss + r);
+  // a wavefront almost always lies inside one row: then the row's three values come through the scalar unit,
+  // one load per wavefront instead of one per lane
+  const uint32_t r0 = __builtin_amdgcn_readfirstlane(r);
+  int64_t label;
+  float l2, g;
+  if (__builtin_amdgcn_ballot_w64(r != r0) == 0) {
+    label = labels[r0];
+    l2 = lse[r0] * kLog2e;
+    g = Cvt<T>::load(grad_loss + r0);
+  } else {
+    label = labels[r];
+    l2 = lse[r] * kLog2e;
+    g = Cvt<T>::load(grad_loss + r);
+  }
   const bool ignored = label == ignored_index;
   g = ignored ? 0.f : g;
   float f[VEC];
@@ -185,13 +197,12 @@ static int vocab_bwd_typed(const void* softmax, const int64_t* labels, const voi
   const int64_t total = rows * cols;
   if constexpr (!std::is_same<T, double>::value) {
     constexpr int VEC = VecIO<T>::N;
-    if (cols % VEC == 0 && aligned16(softmax) && aligned16(out)) {
-      const int64_t nvec = total / VEC;
-      HK_REQUIRE((nvec + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_vocab_parallel_ce_bwd: output too large");
+    if (cols % VEC == 0 && aligned16(softmax) && aligned16(out) && total / VEC < 0x7fffffffLL) {
+      const uint32_t nvec = uint32_t(total / VEC);
       profile_before(s);
-      hipLaunchKernelGGL((vocab_ce_bwd_vec_kernel<T>), dim3(unsigned((nvec + 255) / 256)), dim3(256), 0, s,
+      hipLaunchKernelGGL((vocab_ce_bwd_vec_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
                          static_cast<const T*>(softmax), labels, static_cast<const T*>(grad_loss),
-                         static_cast<T*>(out), nvec, cols / VEC, vocab_start);
+                         static_cast<T*>(out), nvec, uint32_t(cols / VEC), vocab_start);
       profile_after(s);
       return launch_check("vocab_ce_bwd_vec_kernel");
     }

@@ -261,12 +261,15 @@ def case_batch_norm(hk, torch, nsets, which):
     bias = _randn(torch, (256,), torch.float32, 1.0, 823)
     rm, rv = torch.zeros(256, device="cuda"), torch.ones(256, device="cuda")
     sm, si = torch.empty(256, device="cuda"), torch.empty(256, device="cuda")
-    hk.batch_norm_fwd(xs[0], scale, bias, ys[0], 0.1, 1e-5, rm, rv, sm, si)
+    ws = torch.empty(hk.batch_norm_workspace_bytes(xs[0]) // 4 + 4, device="cuda")
+    hk.batch_norm_fwd(xs[0], scale, bias, ys[0], 0.1, 1e-5, rm, rv, sm, si, workspace=ws)
     if which == "fwd":
-        return (lambda i: hk.batch_norm_fwd(xs[i % 2], scale, bias, ys[i % 2], 0.1, 1e-5, rm, rv, sm, si)), 3 * n * 2, 256
+        return (lambda i: hk.batch_norm_fwd(xs[i % 2], scale, bias, ys[i % 2], 0.1, 1e-5, rm, rv, sm, si,
+                                            workspace=ws)), 3 * n * 2, 256
     dys = [_randn(torch, shape, bf, 1.0, 825 + i) for i in range(2)]
     ds, db = torch.empty(256, device="cuda"), torch.empty(256, device="cuda")
-    return (lambda i: hk.batch_norm_bwd(dys[i % 2], xs[i % 2], scale, ys[i % 2], ds, db, sm, si)), 5 * n * 2, 256
+    return (lambda i: hk.batch_norm_bwd(dys[i % 2], xs[i % 2], scale, ys[i % 2], ds, db, sm, si,
+                                        workspace=ws)), 5 * n * 2, 256
 
 
 def case_reduce(hk, torch, nsets, axes, op, three_d=False):

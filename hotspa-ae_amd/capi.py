@@ -354,18 +354,26 @@ def norm_bwd(x, norm_out, grad, out, dim, p, stream=None):
                             stream if stream is not None else current_stream()))
 
 
-def _bn_workspace(x):
+def batch_norm_workspace_bytes(x):
     n, c = x.shape[0], x.shape[1]
     hw = x.numel() // max(n * c, 1)
     need = ctypes.c_size_t(0)
     check(lib().hk_batch_norm_workspace_bytes(dtype_code(x), _i64(n), _i64(c), _i64(hw), ctypes.byref(need)))
-    return n, c, hw, _workspace(need.value, x.device)
+    return need.value
+
+
+def _bn_workspace(x, workspace):
+    n, c = x.shape[0], x.shape[1]
+    hw = x.numel() // max(n * c, 1)
+    if workspace is None:
+        workspace = _workspace(batch_norm_workspace_bytes(x), x.device)
+    return n, c, hw, workspace
 
 
 def batch_norm_fwd(x, scale, bias, y, momentum, eps, running_mean, running_var, save_mean, save_invstd,
-                   stream=None):
-    """hk_batch_norm_fwd on a dense [N, C, ...] tensor."""
-    n, c, hw, ws = _bn_workspace(x)
+                   workspace=None, stream=None):
+    """hk_batch_norm_fwd on a dense [N, C, ...] tensor; allocates the workspace when none is passed."""
+    n, c, hw, ws = _bn_workspace(x, workspace)
     wsb = 0 if ws is None else ws.numel() * ws.element_size()
     check(lib().hk_batch_norm_fwd(dtype_code(x), _ptr(x), _ptr(scale), _ptr(bias), _ptr(y), ctypes.c_double(momentum),
                                   ctypes.c_double(eps), _ptr(running_mean), _ptr(running_var), _ptr(save_mean),
@@ -373,8 +381,8 @@ def batch_norm_fwd(x, scale, bias, y, momentum, eps, running_mean, running_var, 
                                   stream if stream is not None else current_stream()))
 
 
-def batch_norm_bwd(dy, x, scale, dx, dscale, dbias, save_mean, save_invstd, stream=None):
-    n, c, hw, ws = _bn_workspace(x)
+def batch_norm_bwd(dy, x, scale, dx, dscale, dbias, save_mean, save_invstd, workspace=None, stream=None):
+    n, c, hw, ws = _bn_workspace(x, workspace)
     wsb = 0 if ws is None else ws.numel() * ws.element_size()
     check(lib().hk_batch_norm_bwd(dtype_code(x), _ptr(dy), _ptr(x), _ptr(scale), _ptr(dx), _ptr(dscale), _ptr(dbias),
                                   _ptr(save_mean), _ptr(save_invstd), _i64(n), _i64(c), _i64(hw), _ptr(ws),

@@ -179,21 +179,39 @@ void norm_fwd_kernel(NormFwdArgs a) {
   const float shift = a.is_rms ? 0.f : mu;
   T* yr = static_cast<T*>(a.y) + row * int64_t(a.cols);
   // gamma / beta are fetched here, after the reduction: holding them in registers across it was measured
-  // slower (fewer resident waves) than these cache hits
+  // slower (fewer resident waves) than these cache hits.  All of them are issued before the first is
+  // unpacked: a load inside the per-vector branch on the pointer would wait for the one before it.
   const T* gp = static_cast<const T*>(a.gamma);
   const T* bp = static_cast<const T*>(a.beta);
+  u32x4 rawg[NV], rawb[NV];
+  if (gp) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = i * tpr + t;
+      rawg[i] = u32x4{0, 0, 0, 0};
+      if (v < a.nvec) rawg[i] = ld16_keep(gp + v * VEC);
+    }
+  }
+  if (bp) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = i * tpr + t;
+      rawb[i] = u32x4{0, 0, 0, 0};
+      if (v < a.nvec) rawb[i] = ld16_keep(bp + v * VEC);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int v = i * tpr + t;
     if (v < a.nvec) {
       float f[VEC], g[VEC], b[VEC];
       get(i, f);
-      if (gp) VecIO<T>::unpack(ld16_keep(gp + v * VEC), g);
+      if (gp) VecIO<T>::unpack(rawg[i], g);
       else {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) g[j] = 1.f;
       }
-      if (bp) VecIO<T>::unpack(ld16_keep(bp + v * VEC), b);
+      if (bp) VecIO<T>::unpack(rawb[i], b);
       else {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) b[j] = 0.f;

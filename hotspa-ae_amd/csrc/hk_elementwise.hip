@@ -36,12 +36,23 @@ __device__ __forceinline__ CT ew_un(CT a) {
   }
 }
 
-template <typename T> struct EwCT { using type = float; };
+// arithmetic type: fp32 for the 16-bit floats, the type itself for fp64 and the integers (which wrap as the
+// type does: the result of the promoted operation is converted back on the store)
+template <typename T> struct EwCT { using type = typename std::conditional<std::is_integral<T>::value, T, float>::type; };
 template <> struct EwCT<double> { using type = double; };
 
 template <typename T>
 __device__ __forceinline__ typename EwCT<T>::type ew_load(const T* p) {
-  return typename EwCT<T>::type(Cvt<T>::load(p));
+  if constexpr (std::is_integral<T>::value) return *p;
+  else return typename EwCT<T>::type(Cvt<T>::load(p));
+}
+template <typename T>
+__device__ __forceinline__ void ew_store(T* p, typename EwCT<T>::type v) {
+  if constexpr (std::is_integral<T>::value) *p = v;
+  else Cvt<T>::store(p, v);
+}
+template <typename T> constexpr bool ew_vectorised() {
+  return !std::is_same<T, double>::value && !std::is_integral<T>::value;
 }
 
 // ---------------------------------------------------------------------------
@@ -63,7 +74,7 @@ template <typename T, int OP>
 __global__ __launch_bounds__(256) void ew_unary_scalar_kernel(const T* in, T* out, int64_t n) {
   using CT = typename EwCT<T>::type;
   const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
-  if (i < n) Cvt<T>::store(out + i, ew_un<OP, CT>(ew_load(in + i)));
+  if (i < n) ew_store(out + i, CT(ew_un<OP, CT>(ew_load(in + i))));
 }
 
 template <typename T, int OP, bool REV>
@@ -86,7 +97,7 @@ __global__ __launch_bounds__(256) void ew_const_scalar_kernel(const T* in, doubl
   const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
   if (i >= n) return;
   const CT x = ew_load(in + i), k = CT(c);
-  Cvt<T>::store(out + i, REV ? ew_bin<OP, CT>(k, x) : ew_bin<OP, CT>(x, k));
+  ew_store(out + i, CT(REV ? ew_bin<OP, CT>(k, x) : ew_bin<OP, CT>(x, k)));
 }
 
 // ---------------------------------------------------------------------------
@@ -166,7 +177,7 @@ __global__ __launch_bounds__(256) void ew_binary_generic_kernel(const T* a, cons
     oa += idx * d.astride[k];
     ob += idx * d.bstride[k];
   }
-  Cvt<T>::store(out + i, ew_bin<OP, CT>(ew_load(a + oa), ew_load(b + ob)));
+  ew_store(out + i, CT(ew_bin<OP, CT>(ew_load(a + oa), ew_load(b + ob))));
 }
 
 // out = broadcast(a) [* c]: a dense output filled from an operand that maps onto it in one of the four modes.
@@ -206,7 +217,7 @@ __global__ __launch_bounds__(256) void ew_broadcast_generic_kernel(const T* a, d
     rem = q;
   }
   const CT x = ew_load(a + oa);
-  Cvt<T>::store(out + i, MUL ? x * CT(c) : x);
+  ew_store(out + i, MUL ? CT(x * CT(c)) : x);
 }
 
 // ---------------------------------------------------------------------------
@@ -218,7 +229,7 @@ template <typename T, int OP>
 static int unary_launch(const void* in, void* out, int64_t n, hipStream_t s) {
   HK_REQUIRE((n + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_unary: array too large");
   profile_before(s);
-  if constexpr (!std::is_same<T, double>::value) {
+  if constexpr (ew_vectorised<T>()) {
     constexpr int VEC = VecIO<T>::N;
     if (n % VEC == 0 && aligned16(in) && aligned16(out)) {
       hipLaunchKernelGGL((ew_unary_vec_kernel<T, OP>), dim3(blocks_for(n / VEC)), dim3(256), 0, s,
@@ -238,7 +249,7 @@ static int const_launch(const void* in, double c, void* out, int64_t n, hipStrea
   HK_REQUIRE((n + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_binary_const: array too large");
   c = round_const<T>(c);
   profile_before(s);
-  if constexpr (!std::is_same<T, double>::value) {
+  if constexpr (ew_vectorised<T>()) {
     constexpr int VEC = VecIO<T>::N;
     if (n % VEC == 0 && aligned16(in) && aligned16(out)) {
       hipLaunchKernelGGL((ew_const_vec_kernel<T, OP, REV>), dim3(blocks_for(n / VEC)), dim3(256), 0, s,
@@ -297,7 +308,7 @@ static int binary_launch(const void* a, const void* b, void* out, const EwDims& 
   const T* pb = static_cast<const T*>(b);
   T* po = static_cast<T*>(out);
   profile_before(s);
-  if constexpr (!std::is_same<T, double>::value) {
+  if constexpr (ew_vectorised<T>()) {
     constexpr int VEC = VecIO<T>::N;
     if (d.ndim <= 2) {
       const int64_t rows = d.ndim == 2 ? d.shape[0] : 1;
@@ -347,7 +358,7 @@ static int broadcast_launch(const void* a, double c, void* out, const EwDims& d,
   T* po = static_cast<T*>(out);
   c = round_const<T>(c);
   profile_before(s);
-  if constexpr (!std::is_same<T, double>::value) {
+  if constexpr (ew_vectorised<T>()) {
     constexpr int VEC = VecIO<T>::N;
     if (d.ndim <= 2) {
       const int64_t rows = d.ndim == 2 ? d.shape[0] : 1;
@@ -377,35 +388,49 @@ static int broadcast_launch(const void* a, double c, void* out, const EwDims& d,
   return launch_check("ew_broadcast_generic_kernel");
 }
 
-#define HK_EW_TYPES(dtype, who, CALL)                                    \
-  switch (dtype) {                                                       \
+#define HK_EW_FLOAT_CASES(CALL)                                          \
     case HK_FLOAT32: { using T = float; return CALL; }                   \
     case HK_BFLOAT16: { using T = bf16; return CALL; }                   \
     case HK_FLOAT16: { using T = fp16; return CALL; }                    \
-    case HK_FLOAT64: { using T = double; return CALL; }                  \
+    case HK_FLOAT64: { using T = double; return CALL; }
+#define HK_EW_INT_CASES(CALL)                                            \
+    case HK_UINT8: { using T = uint8_t; return CALL; }                   \
+    case HK_INT8: { using T = int8_t; return CALL; }                     \
+    case HK_INT16: { using T = int16_t; return CALL; }                   \
+    case HK_INT32: { using T = int32_t; return CALL; }                   \
+    case HK_INT64: { using T = int64_t; return CALL; }
+#define HK_EW_UNSUPPORTED(dtype, who)                                    \
     default:                                                             \
       set_last_error("%s: not implemented for dtype %d", who, dtype);    \
-      return HK_ERR_UNSUPPORTED;                                         \
-  }
+      return HK_ERR_UNSUPPORTED;
+// floating types only (exp, log, sqrt), or the integers as well (the arithmetic, negation, broadcast)
+#define HK_EW_TYPES(dtype, who, CALL) \
+  switch (dtype) { HK_EW_FLOAT_CASES(CALL) HK_EW_UNSUPPORTED(dtype, who) }
+#define HK_EW_ALL_TYPES(dtype, who, CALL) \
+  switch (dtype) { HK_EW_FLOAT_CASES(CALL) HK_EW_INT_CASES(CALL) HK_EW_UNSUPPORTED(dtype, who) }
 
 template <int OP>
 static int unary_typed(int dtype, const void* in, void* out, int64_t n, hipStream_t s) {
-  HK_EW_TYPES(dtype, "hk_unary", (unary_launch<T, OP>(in, out, n, s)));
+  if constexpr (OP == EW_NEG) {
+    HK_EW_ALL_TYPES(dtype, "hk_unary", (unary_launch<T, OP>(in, out, n, s)));
+  } else {
+    HK_EW_TYPES(dtype, "hk_unary", (unary_launch<T, OP>(in, out, n, s)));
+  }
 }
 template <int OP, bool REV>
 static int const_typed(int dtype, const void* in, double c, void* out, int64_t n, hipStream_t s) {
-  HK_EW_TYPES(dtype, "hk_binary_const", (const_launch<T, OP, REV>(in, c, out, n, s)));
+  HK_EW_ALL_TYPES(dtype, "hk_binary_const", (const_launch<T, OP, REV>(in, c, out, n, s)));
 }
 template <int OP>
 static int binary_typed(int dtype, const void* a, const void* b, void* out, const EwDims& d, int64_t n,
                         hipStream_t s) {
-  HK_EW_TYPES(dtype, "hk_binary", (binary_launch<T, OP>(a, b, out, d, n, s)));
+  HK_EW_ALL_TYPES(dtype, "hk_binary", (binary_launch<T, OP>(a, b, out, d, n, s)));
 }
 
 template <bool MUL>
 static int broadcast_typed(int dtype, const void* a, double c, void* out, const EwDims& d, int64_t n,
                            hipStream_t s) {
-  HK_EW_TYPES(dtype, "hk_broadcast", (broadcast_launch<T, MUL>(a, c, out, d, n, s)));
+  HK_EW_ALL_TYPES(dtype, "hk_broadcast", (broadcast_launch<T, MUL>(a, c, out, d, n, s)));
 }
 
 } // namespace hk

@@ -429,7 +429,7 @@ HK_API int hk_vocab_parallel_ce_bwd_fused(int dtype, const void* logits, const i
 
 /* ======================================================================== *
  * Element-wise operators on dense arrays of fp32 / bf16 / fp16 / fp64 (16-bit
- * types compute in fp32 and round once).  out may alias an input of its shape.
+ * floats compute in fp32 and round once).  out may alias an input of its shape.
  *   hk_unary: exp, log, negate, sqrt.  Replaces ExpCuda, LogCuda, OppositeCuda,
  *     SqrtCuda (hetu/impl/kernel/Exp.cu:12-29, Log.cu, Opposite.cu, Sqrt.cu).
  *   hk_binary_const: x op c, or c op x when scalar_first != 0 (sub, div); the
@@ -442,7 +442,11 @@ HK_API int hk_vocab_parallel_ce_bwd_fused(int dtype, const void* logits, const i
  *     Replaces AddElewiseCuda, SubElewiseCuda, MulElewiseCuda, DivElewiseCuda
  *     (hetu/impl/kernel/BinaryElewise.cu) and the launch_loop_kernel /
  *     vectorize_broadcast_loop_kernel family they run on (Vectorized.cuh).
- * Integer arrays are not implemented (HK_ERR_UNSUPPORTED).
+ * The arithmetic (hk_binary, hk_binary_const), negation and hk_broadcast also take the integer
+ * types uint8 / int8 / int16 / int32 / int64, as the reference dispatches them
+ * (HT_DISPATCH_INTEGER_AND_FLOATING_TYPES, BinaryElewise.cu:332, BinaryConst.cu:16,
+ * Opposite.cu:19): results wrap in the type, division truncates; exp / log / sqrt are
+ * floating only (HK_ERR_UNSUPPORTED otherwise, as for bool).
  * ======================================================================== */
 enum { HK_UNARY_EXP = 0, HK_UNARY_LOG = 1, HK_UNARY_NEG = 2, HK_UNARY_SQRT = 3 };
 enum { HK_BINARY_ADD = 0, HK_BINARY_SUB = 1, HK_BINARY_MUL = 2, HK_BINARY_DIV = 3 };

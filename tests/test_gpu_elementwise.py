@@ -134,8 +134,54 @@ def test_binary_strided_operands_and_in_place(hk, cuda):
     e = torch.empty(0, 16, device=cuda)
     hk.binary("add", e, e, e)                             # empty: nothing to do
     with pytest.raises(hk.HkError) as err:
-        hk.binary("add", a.long(), a.long(), a.long())
+        hk.binary("add", a > 0, a > 0, a > 0)             # bool is not an arithmetic type here
     assert err.value.code == -2
+    with pytest.raises(hk.HkError) as err:
+        hk.unary("exp", a.long(), a.long())               # exp / log / sqrt: floating types only
+    assert err.value.code == -2
+
+
+INT_TYPES = ["uint8", "int8", "int16", "int32", "int64"]
+
+
+@pytest.mark.parametrize("tname", INT_TYPES)
+def test_integer_types(hk, cuda, tname):
+    """The reference dispatches add / sub / mul / div, their constant forms, negation and the broadcast kernels for
+    the integer types too; integers are exact, so torch's own integer arithmetic is the expectation (wrapping in the
+    type, division truncating toward zero)."""
+    import torch
+    td = getattr(torch, tname)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    lo, hi = (0, 200) if tname == "uint8" else (-100, 100)
+    a = torch.randint(lo, hi, (37, 129), generator=g, device=cuda).to(td)
+    b = torch.randint(1, 9, (37, 129), generator=g, device=cuda).to(td)
+    row = torch.randint(1, 9, (37, 1), generator=g, device=cuda).to(td)
+    col = torch.randint(1, 9, (129,), generator=g, device=cuda).to(td)
+    out = torch.empty_like(a)
+    for name, fn in (("add", torch.add), ("sub", torch.sub), ("mul", torch.mul)):
+        for other in (b, row, col):
+            hk.binary(name, a, other, out)
+            torch.cuda.synchronize()
+            assert torch.equal(out, fn(a, other)), name
+    hk.binary("div", a, b, out)
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.div(a, b, rounding_mode="trunc"))
+    hk.binary_const("mul", a, 3, out)
+    torch.cuda.synchronize()
+    assert torch.equal(out, a * 3)
+    hk.binary_const("sub", a, 7, out, scalar_first=True)
+    torch.cuda.synchronize()
+    assert torch.equal(out, 7 - a)
+    hk.unary("neg", a, out)
+    torch.cuda.synchronize()
+    assert torch.equal(out, -a if tname != "uint8" else (256 - a.to(torch.int32)).remainder(256).to(td))
+    wide = torch.empty(5, 37, 129, dtype=td, device=cuda)
+    hk.broadcast(a, wide)
+    torch.cuda.synchronize()
+    assert torch.equal(wide, a.expand(5, 37, 129))
+    hk.broadcast(row, out, scalar=2)
+    torch.cuda.synchronize()
+    assert torch.equal(out, (row * 2).expand(37, 129))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

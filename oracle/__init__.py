@@ -5,6 +5,12 @@ cpu_baseline leg.  Nothing in the product package may import this module.
 
 Every ``oracle_*`` wrapper takes numpy arrays holding values already rounded
 to the storage type (as float32) and returns float64 arrays.
+
+The functions written here in numpy (p-norm, batch normalisation, the broadcast
+of a reduction's gradient, ...) restate the reference lines their docstrings
+cite; each is pinned in tests/test_oracle.py against an independent
+implementation (torch float64 and its autograd, numpy broadcasting) and by
+closed forms.  No function of this package is left unpinned.
 """
 import ctypes
 import os

@@ -333,6 +333,65 @@ def case_fill(hk, torch, nsets):
     return launch, n, 1
 
 
+def case_torch_op(hk, torch, nsets, which):
+    """PyTorch-ROCm's own operators at the benchmark shapes on the same GPU (its kernels for these ops are the
+    CUDA sources compiled for AMD): yardsticks, not product paths.  Wall time per call, PyTorch's dispatch and
+    autograd bookkeeping included; bytes counted as for this library's kernels."""
+    F = torch.nn.functional
+    bf = torch.bfloat16
+    if which in ("rms_fwd", "rms_fwd_bwd"):
+        rows, cols = 32768, 4096
+        xs = [_randn(torch, (rows, cols), bf, 1.0, 401 + i).requires_grad_(True) for i in range(nsets)]
+        dz = _randn(torch, (rows, cols), bf, 1.0, 499)
+        w = _uniform(torch, (cols,), bf, 0.8, 1.2, 403).requires_grad_(True)
+        if which == "rms_fwd":
+            def launch(i):
+                with torch.no_grad():
+                    F.rms_norm(xs[i % nsets], (cols,), w, 1e-6)
+            nbytes = rows * (2 * cols * 2 + 4) + cols * 2
+        else:
+            def launch(i):
+                z = F.rms_norm(xs[i % nsets], (cols,), w, 1e-6)
+                torch.autograd.grad(z, (xs[i % nsets], w), dz)
+            nbytes = rows * (5 * cols * 2 + 12)
+        units = rows
+    elif which in ("softmax_fwd", "softmax_bwd"):
+        shape = (4, 32, 2048, 2048)
+        n = 4 * 32 * 2048 * 2048
+        xs = [_randn(torch, shape, bf, 1.0, 201 + i) for i in range(2)]
+        if which == "softmax_fwd":
+            def launch(i):
+                torch.softmax(xs[i % 2], -1)
+            nbytes = 2 * n * 2
+        else:
+            ys = [torch.softmax(x, -1) for x in xs]
+            dy = _randn(torch, shape, bf, 1.0, 299)
+
+            def launch(i):
+                torch._softmax_backward_data(dy, ys[i % 2], -1, bf)
+            nbytes = 3 * n * 2
+        units = n // 2048
+    else:
+        rows, cols = 16384, 32000
+        xs = [_randn(torch, (rows, cols), bf, 2.0, 501 + i).requires_grad_(True) for i in range(2)]
+        g = torch.Generator(device="cuda").manual_seed(77)
+        labels = torch.randint(0, cols, (rows,), generator=g, device="cuda")
+        labels[::20] = -100
+        if which == "ce_fwd":
+            def launch(i):
+                with torch.no_grad():
+                    F.cross_entropy(xs[i % 2], labels, ignore_index=-100)
+            nbytes = rows * (cols * 2 + 8 + 2)
+        else:
+            def launch(i):
+                loss = F.cross_entropy(xs[i % 2], labels, ignore_index=-100)
+                torch.autograd.grad(loss, xs[i % 2])
+            nbytes = rows * (3 * cols * 2 + 2 * (8 + 2))
+        units = rows
+    launch.no_hook = True
+    return launch, nbytes, units
+
+
 def case_torch_add(hk, torch, nsets):
     """torch's own elementwise add (two reads, one write per element): an independent yardstick for what
     a plain streaming kernel with this read/write mix reaches on the same GPU."""
@@ -385,6 +444,12 @@ CASES = [
     ("copy kernel 256 MiB (calibration)", lambda hk, t, n: case_copy(hk, t, n)),
     ("fill kernel 256 MiB (write-only calibration)", lambda hk, t, n: case_fill(hk, t, n)),
     ("torch.add bf16 [32768x4096] (2R:1W yardstick)", lambda hk, t, n: case_torch_add(hk, t, n)),
+    ("torch F.rms_norm fwd bf16 [32768x4096] (yardstick for C4 fwd)", lambda hk, t, n: case_torch_op(hk, t, n, "rms_fwd")),
+    ("torch F.rms_norm fwd+bwd bf16 [32768x4096] (yardstick for the headline)", lambda hk, t, n: case_torch_op(hk, t, n, "rms_fwd_bwd")),
+    ("torch softmax fwd bf16 [4,32,2048,2048] (yardstick for C2 fwd)", lambda hk, t, n: case_torch_op(hk, t, n, "softmax_fwd")),
+    ("torch softmax bwd bf16 [4,32,2048,2048] (yardstick for C2 bwd)", lambda hk, t, n: case_torch_op(hk, t, n, "softmax_bwd")),
+    ("torch F.cross_entropy fwd bf16 [16384x32000] (yardstick for C5 fwd)", lambda hk, t, n: case_torch_op(hk, t, n, "ce_fwd")),
+    ("torch F.cross_entropy fwd+bwd bf16 [16384x32000] (yardstick for C5 fwd+bwd)", lambda hk, t, n: case_torch_op(hk, t, n, "ce_fwd_bwd")),
 ]
 
 

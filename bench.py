@@ -371,6 +371,37 @@ def case_torch_op(hk, torch, nsets, which):
                 torch._softmax_backward_data(dy, ys[i % 2], -1, bf)
             nbytes = 3 * n * 2
         units = n // 2048
+    elif which in ("ln_fwd_c1", "ln_fwd_bwd_c5"):
+        if which == "ln_fwd_c1":
+            rows, cols, dt = 8192, 4096, torch.float32
+        else:
+            rows, cols, dt = 16384, 5120, bf
+        es = 4 if dt == torch.float32 else 2
+        xs = [_randn(torch, (rows, cols), dt, 1.0, 101 + i).requires_grad_(True) for i in range(nsets)]
+        w = _uniform(torch, (cols,), dt, 0.5, 1.5, 103).requires_grad_(True)
+        b = _randn(torch, (cols,), dt, 0.1, 104).requires_grad_(True)
+        if which == "ln_fwd_c1":
+            def launch(i):
+                with torch.no_grad():
+                    F.layer_norm(xs[i % nsets], (cols,), w, b, 1e-5)
+            nbytes = rows * (2 * cols * es + 8) + 2 * cols * es
+        else:
+            dz = _randn(torch, (rows, cols), dt, 1.0, 199)
+
+            def launch(i):
+                z = F.layer_norm(xs[i % nsets], (cols,), w, b, 1e-5)
+                torch.autograd.grad(z, (xs[i % nsets], w, b), dz)
+            nbytes = rows * (5 * cols * es + 16)
+        units = rows
+    elif which in ("sum_axis0", "sum_axis1"):
+        rows, cols = 32768, 4096
+        xs = [_randn(torch, (rows, cols), bf, 1.0, 301 + 10 * i) for i in range(nsets)]
+        axis = 0 if which == "sum_axis0" else 1
+
+        def launch(i):
+            torch.sum(xs[i % nsets], dim=axis)
+        nbytes = rows * cols * 2 + (cols if axis == 0 else rows) * 2
+        units = rows
     else:
         rows, cols = 16384, 32000
         xs = [_randn(torch, (rows, cols), bf, 2.0, 501 + i).requires_grad_(True) for i in range(2)]
@@ -446,6 +477,10 @@ CASES = [
     ("torch.add bf16 [32768x4096] (2R:1W yardstick)", lambda hk, t, n: case_torch_add(hk, t, n)),
     ("torch F.rms_norm fwd bf16 [32768x4096] (yardstick for C4 fwd)", lambda hk, t, n: case_torch_op(hk, t, n, "rms_fwd")),
     ("torch F.rms_norm fwd+bwd bf16 [32768x4096] (yardstick for the headline)", lambda hk, t, n: case_torch_op(hk, t, n, "rms_fwd_bwd")),
+    ("torch F.layer_norm fwd fp32 [8192x4096] (yardstick for C1)", lambda hk, t, n: case_torch_op(hk, t, n, "ln_fwd_c1")),
+    ("torch F.layer_norm fwd+bwd bf16 [16384x5120] (yardstick for C5 LN fwd+bwd)", lambda hk, t, n: case_torch_op(hk, t, n, "ln_fwd_bwd_c5")),
+    ("torch.sum axis0 bf16 [32768x4096] (yardstick for C3)", lambda hk, t, n: case_torch_op(hk, t, n, "sum_axis0")),
+    ("torch.sum axis1 bf16 [32768x4096] (yardstick for C3)", lambda hk, t, n: case_torch_op(hk, t, n, "sum_axis1")),
     ("torch softmax fwd bf16 [4,32,2048,2048] (yardstick for C2 fwd)", lambda hk, t, n: case_torch_op(hk, t, n, "softmax_fwd")),
     ("torch softmax bwd bf16 [4,32,2048,2048] (yardstick for C2 bwd)", lambda hk, t, n: case_torch_op(hk, t, n, "softmax_bwd")),
     ("torch F.cross_entropy fwd bf16 [16384x32000] (yardstick for C5 fwd)", lambda hk, t, n: case_torch_op(hk, t, n, "ce_fwd")),

@@ -29,8 +29,10 @@ IGNORE = -100
 
 
 def _load():
+    import __graft_entry__
+    __graft_entry__.ensure_built()      # a fresh checkout: compile once; built libraries are used as they are
     hk = importlib.import_module("hotspa-ae_amd")
-    hk.lib()  # fails loudly when the HIP library has not been built
+    hk.lib()  # fails loudly when the HIP library is missing
     return hk
 
 

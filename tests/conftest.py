@@ -14,6 +14,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """A fresh checkout has no native libraries: compile them once (hipcc cross-compiles without a GPU).
+    Libraries that are there are used as they are."""
+    import __graft_entry__
+    __graft_entry__.ensure_built()
+
+
 @pytest.fixture(scope="session")
 def hk():
     """The product package (ctypes harness over libhk_rowwise.so)."""

@@ -215,3 +215,26 @@ def test_loss_gradient_ops(ops, cuda, dtype, reduction, sparse):
         with pytest.raises(ops.AssertionError_, match="one value"):
             ops.sceloss_gradient(tx, tl, torch.ones(2, dtype=tx.dtype, device=cuda), outs[0], reduction,
                                  ignored_index=-1 if sparse else None, fused=True)
+
+
+def test_reduced_gradient_edge_cases(hk, cuda):
+    import torch
+    bf = torch.bfloat16
+    grad = torch.ones(1, dtype=bf, device=cuda)
+    empty = torch.empty(0, 128, dtype=bf, device=cuda)
+    hk.sce_sparse_bwd_reduced(empty, torch.empty(0, dtype=torch.int64, device=cuda), grad, 1.0, empty, -100)   # no rows
+    # every row ignored: a zero gradient whatever the incoming value, also a non-finite one
+    x = torch.randn(9, 256, device=cuda).to(bf)
+    labels = torch.full((9,), -100, dtype=torch.int64, device=cuda)
+    out = torch.full_like(x, 7.0)
+    hk.sce_sparse_bwd_reduced(x, labels, torch.full((1,), float("inf"), dtype=bf, device=cuda), 0.5, out, -100)
+    torch.cuda.synchronize()
+    assert (out == 0).all()
+    # one row, one class: softmax is 1, the gradient (1 - 1) * g is an exact zero
+    one = torch.randn(1, 1, device=cuda)
+    o1 = torch.empty_like(one)
+    hk.sce_sparse_bwd_reduced(one, torch.zeros(1, dtype=torch.int64, device=cuda), torch.ones(1, device=cuda), 1.0, o1, -100)
+    torch.cuda.synchronize()
+    assert o1.item() == 0.0
+    with pytest.raises(hk.HkError):
+        hk.sce_sparse_bwd_reduced(x, labels, None, 1.0, out, -100)          # the gradient value is required

@@ -17,7 +17,7 @@ The directory name contains a hyphen, so import it with
 from .capi import (  # noqa: F401
     HkError, lib, lib_path, check, DTYPES, dtype_code, torch_dtype,
     layer_norm_fwd, layer_norm_bwd, norm_bwd_workspace_bytes,
-    dropout_add_ln_fwd, dropout_add_ln_bwd, dropout_add_ln_fwd_ex, dropout_add_ln_bwd_ex,
+    dropout_add_ln_fwd, dropout_add_ln_bwd, dropout_add_ln_bwd_static, dropout_add_ln_fwd_ex, dropout_add_ln_bwd_ex,
     unary, binary_const, binary, broadcast, sce_sparse_bwd_reduced, sce_dense_bwd_reduced, vocab_parallel_ce_gather, vocab_parallel_ce_bwd,
     vocab_parallel_ce_stats, vocab_parallel_ce_combine, vocab_parallel_ce_bwd_fused, UNARY_OPS, BINARY_OPS,
     softmax_fwd, softmax_bwd,

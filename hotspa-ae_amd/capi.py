@@ -173,6 +173,17 @@ def dropout_add_ln_bwd(dz, dx_in, x, mu, rsigma, gamma, dx0, dresidual, dgamma, 
     return workspace
 
 
+def dropout_add_ln_bwd_static(dz, dx_in, x, mu, rsigma, gamma, dx0, dresidual, dgamma, dbeta, is_rms, stream=None):
+    """hk_dropout_add_ln_bwd_static: the same backward with its partials in the library's own static array;
+    nothing is allocated, here or inside."""
+    rows, cols = x.shape
+    check(lib().hk_dropout_add_ln_bwd_static(dtype_code(dz), dtype_code(x), dtype_code(gamma), _ptr(dz),
+                                             _ptr(dx_in), _ptr(x), _ptr(mu), _ptr(rsigma), _ptr(gamma), _ptr(dx0),
+                                             _ptr(dresidual), _ptr(dgamma), _ptr(dbeta), _i64(rows), _i64(cols),
+                                             ctypes.c_int(int(is_rms)),
+                                             stream if stream is not None else current_stream()))
+
+
 class DropoutAddLnFwdParams(ctypes.Structure):
     """hkDropoutAddLnFwdParams of include/hk_rowwise.h"""
     _fields_ = [("itype", ctypes.c_int), ("rtype", ctypes.c_int), ("wtype", ctypes.c_int),

@@ -13,6 +13,7 @@
 #include "hk_common.cuh"
 
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 namespace hk {
@@ -1054,6 +1055,36 @@ static int norm_bwd_dispatch(int dtype, NormBwdArgs& a, int mode, void* dgamma, 
   }
 }
 
+// ---------------------------------------------------------------------------
+// Scratch memory owned by the library, for the entry point that must not
+// allocate.  The array lives in the code object's global segment, so every
+// device the library is loaded on holds its own copy at its own address; host
+// code only ever uses the address looked up below, never the array's name.
+// ---------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = size_t(16) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_scratch(void** out) {
+  int dev = -1;
+  HK_CHECK_HIP(hipGetDevice(&dev));
+  HK_REQUIRE(dev >= 0 && dev < kMaxDevices, HK_ERR_UNSUPPORTED,
+             "static scratch: device index %d is beyond the %d devices this table holds", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    HK_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    HK_REQUIRE(p != nullptr, HK_ERR_HIP, "static scratch: symbol address is null on device %d", dev);
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return HK_OK;
+}
+
 } // namespace hk
 
 using namespace hk;
@@ -1159,6 +1190,26 @@ int hk_dropout_add_ln_bwd(int itype, int rtype, int wtype, const void* dz, const
   a.stat_kind = HK_STAT_RSTD; a.stats_f32 = 1; a.clamp_gamma = 0;
   return norm_bwd_dispatch(itype, a, is_rms_norm ? BWD_RMS : BWD_LN, dgamma, dbeta, workspace,
                            workspace_bytes, as_hip(stream), "hk_dropout_add_ln_bwd");
+}
+
+int hk_dropout_add_ln_bwd_static(int itype, int rtype, int wtype, const void* dz, const void* dx_in,
+                                 const void* x, const void* mu, const void* rsigma, const void* gamma,
+                                 void* dx0, void* dresidual, void* dgamma, void* dbeta, int64_t rows,
+                                 int64_t cols, int is_rms_norm, hkStream_t stream) {
+  size_t need = 0;
+  int rc = hk_norm_bwd_workspace_bytes(itype, rows, cols, &need);
+  if (rc != HK_OK) return rc;
+  HK_REQUIRE(need <= kStaticScratchBytes, HK_ERR_WORKSPACE,
+             "hk_dropout_add_ln_bwd_static: a [%lld, %lld] backward needs %zu bytes of column-sum partials, "
+             "the library's static scratch holds %zu; use hk_dropout_add_ln_bwd with a caller workspace",
+             (long long)rows, (long long)cols, need, kStaticScratchBytes);
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc != HK_OK) return rc;
+  // every partial row the fold kernel reads is written by this call's main kernel first: nothing in the
+  // scratch has to start at zero
+  return hk_dropout_add_ln_bwd(itype, rtype, wtype, dz, dx_in, x, mu, rsigma, gamma, dx0, dresidual, dgamma,
+                               dbeta, rows, cols, is_rms_norm, ws, kStaticScratchBytes, stream);
 }
 
 } // extern "C"

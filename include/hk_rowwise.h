@@ -187,6 +187,22 @@ HK_API int hk_dropout_add_ln_bwd(int itype, int rtype, int wtype, const void* dz
                                  int64_t cols, int is_rms_norm, void* workspace,
                                  size_t workspace_bytes, hkStream_t stream);
 
+/* hk_dropout_add_ln_bwd for callers that cannot allocate device memory and so have no workspace to
+ * pass: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose launcher allocates its partials itself, RMSNorm.cu:429-431).
+ * Same arguments and results, bit for bit, as hk_dropout_add_ln_bwd; the column-sum partials go to a
+ * 16 MiB array that is part of the library's code object (one copy per device the library is loaded
+ * on, held until the process ends).  The call allocates and frees nothing.  16 MiB is what the widest
+ * row the register kernel takes (8192 columns) needs on 256 persistent workgroups; a plan that needs
+ * more (hk_norm_bwd_workspace_bytes > 16 MiB: a device with more compute units, or a raised
+ * "norm_bwd_blocks") is refused with HK_ERR_WORKSPACE.  All calls on one device share the array: calls that overlap on one
+ * device (different streams, or threads) race and must be ordered by the caller. */
+HK_API int hk_dropout_add_ln_bwd_static(int itype, int rtype, int wtype, const void* dz,
+                                        const void* dx_in, const void* x, const void* mu,
+                                        const void* rsigma, const void* gamma, void* dx0,
+                                        void* dresidual, void* dgamma, void* dbeta, int64_t rows,
+                                        int64_t cols, int is_rms_norm, hkStream_t stream);
+
 /* ------------------------------------------------------------------------ *
  * The same interface with every feature of the flash-attention layer_norm
  * kernels the reference vendors: dropout, per-row and per-column scaling, row

@@ -297,6 +297,8 @@ static int operand_mode(int64_t rows, int64_t cols, int64_t s0, int64_t s1) {
   if (row_fixed && col_fixed) return EW_SINGLE;
   if (col_fixed) return (s0 == 1) ? EW_PER_ROW : -1;
   if (s1 != 1) return -1;
+  // a single row walked with unit stride is the whole array (two dense arrays of one shape merge to this)
+  if (rows == 1) return EW_FULL;
   if (row_fixed) return EW_PER_COL;
   return s0 == cols ? EW_FULL : -1;
 }

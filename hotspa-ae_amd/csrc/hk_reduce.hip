@@ -114,6 +114,10 @@ struct RMin : RNoTransform {
     return (is_nan(a) || a < b) ? a : (is_nan(b) ? b : (a < b ? a : b));
   }
 };
+// R without its load transform: what folds partial results, which went through pre() when they were formed
+template <typename R> struct Folded : R {
+  template <typename A> static __device__ __forceinline__ A pre(A v, float) { return v; }
+};
 // the float face the wave / block reduction helpers expect
 template <typename R> struct AsFloatOp {
   static __device__ __forceinline__ float identity() { return R::template identity<float>(); }
@@ -570,8 +574,9 @@ static int reduce_fast(const ReducePlan& p, const void* in, void* out, float fac
     profile_after(st);
     int rc = launch_check("reduce_inner_vec_kernel");
     if (rc != HK_OK || s.nsplit == 1) return rc;
-    // second pass over the fp32 partials [rows, nsplit]
-    hipLaunchKernelGGL((reduce_inner_scalar_kernel<float, float, OUT_T, R>), dim3(unsigned(p.rows)), dim3(256), 0, st,
+    // second pass over the fp32 partials [rows, nsplit]: combine and store only, the elements' own
+    // transform (|x|, x^2, |x|^p of the p-norms) was applied when the partials were formed
+    hipLaunchKernelGGL((reduce_inner_scalar_kernel<float, float, OUT_T, Folded<R>>), dim3(unsigned(p.rows)), dim3(256), 0, st,
                        static_cast<const float*>(ws), static_cast<OUT_T*>(out), p.rows, int64_t(s.nsplit),
                        int64_t(s.nsplit), factor, is_mean);
     return launch_check("reduce_inner_scalar_kernel");

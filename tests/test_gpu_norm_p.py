@@ -39,6 +39,27 @@ def test_norm_and_gradient(hk, cuda, dtype, shape, dim, p):
     helpers.assert_close(dx, want_g, dtype, "gradient")
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("p", [1, 2, 3])
+def test_norm_of_few_long_rows_is_split_over_workgroups(hk, cuda, dtype, p):
+    """Few rows of 2^20 elements (a global gradient norm): the row is split over workgroups and the fp32
+    partial sums of |x|^p are folded by a second launch, which must add them up as they are."""
+    import torch
+    shape = (4, 1 << 20)
+    assert hk.reduce_workspace_bytes(hk.DTYPES[dtype], list(shape), [shape[1], 1], [1]) > 0   # the split path
+    x = oracle.round_to(helpers.rng(77 + p).standard_normal(shape).astype(np.float32), dtype)
+    want = oracle.norm_p_fwd(x, 1, p)
+    tx = helpers.to_torch(x, dtype, cuda)
+    out = torch.empty(4, dtype=tx.dtype, device=cuda)
+    hk.norm(tx, out, 1, p)
+    torch.cuda.synchronize()
+    helpers.assert_close(out, want, dtype, "norm of split rows")
+    ones = torch.ones(1, 1 << 20, dtype=tx.dtype, device=cuda)     # exact: (2^20)^(1/p)
+    hk.norm(ones, out[:1], 1, 2)
+    torch.cuda.synchronize()
+    assert float(out[0]) == 1024.0
+
+
 def test_norm_edge_cases(hk, cuda):
     import torch
     z = torch.zeros(5, 512, device=cuda)

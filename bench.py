@@ -10,8 +10,16 @@ of the step (the backward row kernel), timed with HIP events recorded around
 that kernel on its stream; `cpu_baseline` is the oracle's fp32 CPU port timed
 on a bounded sample of the same rows.
 
-`--all` additionally times every kernel of every BASELINE configuration and
-adds the table as `kernels` (also printed to stderr).
+Every run starts each measured case with an untimed pre-roll (PREROLL_* below) whatever
+`--warmup` says: after idle the GPU's clocks take a few hundred launches to settle, and a
+timed region that falls into the ramp reads 15 % slow.  The count is reported as
+`preroll_steps`.
+
+The line also carries `kernels`: every forward / backward kernel of every BASELINE
+configuration (C1..C5) with its own microseconds, GB/s and fraction of the HBM peak over
+KERNEL_STEPS launches, and `cpu_baselines`: the CPU ports of the reference's CPU kernels
+for the same configurations on bounded samples.  `--all` adds the kernels beyond the
+configurations, the streaming yardsticks and PyTorch-ROCm's own operators.
 """
 import argparse
 import importlib
@@ -26,6 +34,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 IGNORE = -100
+# untimed launches before any timed region of a case: at least this many and at least this long
+PREROLL_MIN_STEPS = 300
+PREROLL_MIN_SECONDS = 0.3
+# timed launches per entry of the `kernels` table
+KERNEL_STEPS = 200
 
 
 def _load():
@@ -440,6 +453,11 @@ def case_torch_add(hk, torch, nsets):
     return launch, 3 * rows * cols * 2, rows
 
 
+def is_config_case(name):
+    """The kernels of the BASELINE configurations: always measured, also by the default run."""
+    return name[:2] in ("C1", "C2", "C3", "C4", "C5")
+
+
 CASES = [
     ("C1 layernorm fwd fp32 [8192x4096]", lambda hk, t, n: case_layernorm(hk, t, n, "fwd", "C1")),
     ("C2 softmax fwd bf16 [4,32,2048,2048]", lambda hk, t, n: case_softmax(hk, t, 2, "fwd")),
@@ -496,9 +514,21 @@ CASES = [
 NORM_BWD_TRAFFIC_BYTES = int((262985.0 * 2.0 + 270336.0 * 1.0) * 1024)
 
 
+def preroll(torch, launch, min_steps=PREROLL_MIN_STEPS, min_seconds=PREROLL_MIN_SECONDS):
+    """Untimed launches of the case until the clocks have settled; returns how many were made."""
+    done, t0 = 0, time.perf_counter()
+    while done < min_steps or time.perf_counter() - t0 < min_seconds:
+        for _ in range(50):
+            launch(done)
+            done += 1
+        torch.cuda.synchronize()
+    return done
+
+
 def time_case(hk, torch, launch, steps, warmup, profile_main=True):
     """Returns (ms per step over a plain timed region, mean us of the main kernel measured in a
-    second region with HIP events recorded around that kernel on its stream)."""
+    second region with HIP events recorded around that kernel on its stream, pre-roll launches made)."""
+    pre = preroll(torch, launch)
     for i in range(warmup):
         launch(i)
     torch.cuda.synchronize()
@@ -516,17 +546,21 @@ def time_case(hk, torch, launch, steps, warmup, profile_main=True):
         torch.cuda.synchronize()
         hk.lib().hk_profile_next_kernel(None, None)
         main_us = sum(b.elapsed_ns_since(a) for a, b in pairs) / 1000.0 / steps
-    return (t1 - t0) * 1000.0 / steps, main_us
+    return (t1 - t0) * 1000.0 / steps, main_us, pre
 
 
-def cpu_baseline(rows=32768, cols=4096, budget_s=12.0):
-    """fp32 CPU port of the step (oracle's refcpu_rmsnorm_*) on all host threads: the full workload, repeated
-    for about `budget_s` seconds of CPU work; the mean over the repetitions is reported."""
+def _cpu_cores():
+    return min(int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1), 64)
+
+
+def cpu_baseline(rows=32768, cols=4096, budget_s=3.0):
+    """fp32 CPU port of the headline step (oracle's refcpu_rmsnorm_*) on all host threads: the full workload,
+    repeated for about `budget_s` seconds of CPU work; the mean over the repetitions is reported."""
     import ctypes
     import numpy as np
     import oracle
     lib = oracle.lib()
-    cores = min(int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1), 64)
+    cores = _cpu_cores()
     lib.refcpu_set_num_threads(ctypes.c_int(cores))
     g = np.random.default_rng(402)
     # a 1024-row random block repeated down the array: the values do not change the timing
@@ -545,7 +579,7 @@ def cpu_baseline(rows=32768, cols=4096, budget_s=12.0):
 
     step()  # page in the outputs
     reps, t0 = 0, time.perf_counter()
-    while reps < 3 or time.perf_counter() - t0 < budget_s:
+    while reps < 2 or time.perf_counter() - t0 < budget_s:
         step()
         reps += 1
     dt = (time.perf_counter() - t0) / reps
@@ -556,69 +590,100 @@ def cpu_baseline(rows=32768, cols=4096, budget_s=12.0):
                       "formula" % (rows, reps, reps * dt)}
 
 
-def cpu_kernels(budget_s=1.5):
-    """fp32 CPU ports of the reference's CPU kernels (oracle's refcpu_*: the pass structure of
-    LayerNormCpu, the softmax / cross-entropy loops, the reductions), timed on all host threads and,
-    for the serial loops of the reference, on one; bytes counted in the ports' own fp32 storage."""
+def cpu_baselines(budget_s=1.2):
+    """One entry per BASELINE configuration kernel: the fp32 CPU ports of the reference's CPU kernels (the pass
+    structure of LayerNormCpu / LayerNormGradientCpu, the softmax and cross-entropy loops, the reductions) timed on
+    all host threads on a bounded sample of the configuration's rows, and on one thread where the reference's own
+    loop is serial.  `value` counts the same algorithmic bytes per row as the GPU entry of that configuration
+    (storage type of the configuration), so the two columns compare like with like."""
     import ctypes
     import numpy as np
     import oracle
     lib = oracle.lib()
-    cores = min(int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1), 64)
+    cores = _cpu_cores()
     g = np.random.default_rng(7)
     fp = ctypes.POINTER(ctypes.c_float)
     P = lambda a: a.ctypes.data_as(fp)
     I = ctypes.c_int64
+    F = ctypes.c_float
 
     def block(rows, cols):
         b = g.standard_normal((min(rows, 512), cols), dtype=np.float32)
         return np.tile(b, ((rows + b.shape[0] - 1) // b.shape[0], 1))[:rows].copy()
 
-    def timed(fn, nbytes, threads):
+    def timed(fn, threads):
         lib.refcpu_set_num_threads(ctypes.c_int(threads))
         fn()
         reps, t0 = 0, time.perf_counter()
         while reps < 2 or time.perf_counter() - t0 < budget_s:
             fn()
             reps += 1
-        dt = (time.perf_counter() - t0) / reps
-        return round(dt * 1e6, 1), round(nbytes / dt / 1e9, 2), reps
+        return (time.perf_counter() - t0) / reps, reps
 
     out = []
 
-    def add(name, fn, nbytes, sample, serial_too=False):
-        us, gbs, reps = timed(fn, nbytes, cores)
-        rec = {"case": name, "us": us, "GBps": gbs, "cores": cores, "sample": sample, "reps": reps}
+    def add(config, case, fn, algo_bytes, sample_rows, full_rows, serial_too=False):
+        dt, reps = timed(fn, cores)
+        rec = {"config": config, "case": case, "value": round(algo_bytes / dt / 1e9, 3), "unit": "GB/s",
+               "us": round(dt * 1e6, 1), "cores": cores, "kind": "port",
+               "sample": "%d of %d rows, fp32 arithmetic, %d repetitions, mean" % (sample_rows, full_rows, reps)}
         if serial_too:
-            us1, gbs1, _ = timed(fn, nbytes, 1)
-            rec["us_1_thread"], rec["GBps_1_thread"] = us1, gbs1
+            dt1, _ = timed(fn, 1)
+            rec["value_1_thread"], rec["us_1_thread"] = round(algo_bytes / dt1 / 1e9, 3), round(dt1 * 1e6, 1)
         out.append(rec)
 
+    # C1: the whole configuration (LayerNormCpu: two mean reductions + two element-wise passes, fp32)
     rows, cols = 8192, 4096
     x = block(rows, cols); y = np.empty_like(x)
     gm = np.ones(cols, np.float32); bt = np.zeros(cols, np.float32)
     mean = np.empty(rows, np.float32); var = np.empty(rows, np.float32)
-    add("C1 layernorm fwd fp32 [8192x4096] (LayerNormCpu pass structure)",
-        lambda: lib.refcpu_layernorm_fwd_f32(P(x), P(gm), P(bt), I(rows), I(cols), ctypes.c_float(1e-5), P(y), P(mean), P(var)),
-        2 * rows * cols * 4, "full size", serial_too=True)
+    add("C1", "layernorm fwd fp32 [8192x4096] (LayerNormCpu pass structure)",
+        lambda: lib.refcpu_layernorm_fwd_f32(P(x), P(gm), P(bt), I(rows), I(cols), F(1e-5), P(y), P(mean), P(var)),
+        rows * (2 * cols * 4 + 8), rows, rows, serial_too=True)
+    # C5 layer norm at 5120 columns, forward and gradient, 1/4 of the rows; bf16 storage accounting
+    rows, cols = 4096, 5120
+    x = block(rows, cols); y = np.empty_like(x); dy = block(rows, cols); dx = np.empty_like(x)
+    gm = np.ones(cols, np.float32); bt = np.zeros(cols, np.float32)
+    mean = np.empty(rows, np.float32); var = np.empty(rows, np.float32)
+    dgm = np.empty(cols, np.float32); dbt = np.empty(cols, np.float32)
+    add("C5", "layernorm fwd [16384x5120]",
+        lambda: lib.refcpu_layernorm_fwd_f32(P(x), P(gm), P(bt), I(rows), I(cols), F(1e-5), P(y), P(mean), P(var)),
+        rows * (2 * cols * 2 + 8), rows, 16384)
+    add("C5", "layernorm bwd [16384x5120] (LayerNormGradientCpu pass structure)",
+        lambda: lib.refcpu_layernorm_bwd_f32(P(dy), P(x), P(gm), P(mean), P(var), I(rows), I(cols), F(1e-5), P(dx),
+                                             P(dgm), P(dbt)),
+        rows * (3 * cols * 2 + 8), rows, 16384)
+    # C2: 1/16 of the rows
     rows, cols = 16384, 2048
     x = block(rows, cols); y = np.empty_like(x); dx = np.empty_like(x)
-    add("C2 softmax fwd fp32 [16384 of 262144 rows x 2048]",
-        lambda: lib.refcpu_softmax_fwd_f32(P(x), I(rows), I(cols), P(y)), 2 * rows * cols * 4, "1/16 of the rows")
-    add("C2 softmax bwd fp32 [16384 of 262144 rows x 2048]",
-        lambda: lib.refcpu_softmax_bwd_f32(P(y), P(x), I(rows), I(cols), P(dx)), 3 * rows * cols * 4, "1/16 of the rows")
+    add("C2", "softmax fwd [4,32,2048,2048]",
+        lambda: lib.refcpu_softmax_fwd_f32(P(x), I(rows), I(cols), P(y)), 2 * rows * cols * 2, rows, 262144)
+    add("C2", "softmax bwd [4,32,2048,2048]",
+        lambda: lib.refcpu_softmax_bwd_f32(P(y), P(x), I(rows), I(cols), P(dx)), 3 * rows * cols * 2, rows, 262144)
+    # C3: 1/4 of the rows
     rows, cols = 8192, 4096
     x = block(rows, cols); o0 = np.empty(cols, np.float32); o1 = np.empty(rows, np.float32)
-    add("C3 reduce sum axis1 fp32 [8192 of 32768 rows x 4096]",
-        lambda: lib.refcpu_reduce_sum_axis1_f32(P(x), I(rows), I(cols), P(o1)), rows * cols * 4, "1/4 of the rows")
-    add("C3 reduce sum axis0 fp32 [8192 of 32768 rows x 4096] (serial loop)",
-        lambda: lib.refcpu_reduce_sum_axis0_f32(P(x), I(rows), I(cols), P(o0)), rows * cols * 4, "1/4 of the rows")
+    add("C3", "reduce sum axis 1 [32768x4096]",
+        lambda: lib.refcpu_reduce_sum_axis1_f32(P(x), I(rows), I(cols), P(o1)), rows * cols * 2, rows, 32768)
+    add("C3", "reduce mean axis 1 [32768x4096]",
+        lambda: lib.refcpu_reduce_mean_axis1_f32(P(x), I(rows), I(cols), P(o1)), rows * cols * 2, rows, 32768)
+    add("C3", "reduce sum axis 0 [32768x4096] (also the merged axes (0,1) of [64x512x4096])",
+        lambda: lib.refcpu_reduce_sum_axis0_f32(P(x), I(rows), I(cols), P(o0)), rows * cols * 2, rows, 32768)
+    add("C3", "reduce mean axis 0 [32768x4096]",
+        lambda: lib.refcpu_reduce_mean_axis0_f32(P(x), I(rows), I(cols), P(o0)), rows * cols * 2, rows, 32768)
+    # C5 cross-entropy: 1/16 of the rows
     rows, cols = 1024, 32000
-    x = block(rows, cols); loss = np.empty(rows, np.float32)
+    x = block(rows, cols); loss = np.empty(rows, np.float32); dx = np.empty_like(x)
+    gl = np.full(rows, 1.0 / 16384, np.float32)
     lab = (np.arange(rows, dtype=np.int64) * 31) % cols
-    add("C5 sce fwd fp32 [1024 of 16384 rows x 32000]",
-        lambda: lib.refcpu_sce_sparse_fwd_f32(P(x), lab.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)), I(rows), I(cols),
-                                              I(-100), P(loss)), rows * cols * 4, "1/16 of the rows")
+    lab[::20] = IGNORE
+    L = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_int64))
+    add("C5", "cross-entropy fwd [16384x32000]",
+        lambda: lib.refcpu_sce_sparse_fwd_f32(P(x), L(lab), I(rows), I(cols), I(IGNORE), P(loss)),
+        rows * (cols * 2 + 10), rows, 16384)
+    add("C5", "cross-entropy bwd [16384x32000]",
+        lambda: lib.refcpu_sce_sparse_bwd_f32(P(x), L(lab), P(gl), I(rows), I(cols), I(IGNORE), P(dx)),
+        rows * (2 * cols * 2 + 10), rows, 16384)
     lib.refcpu_set_num_threads(ctypes.c_int(cores))
     return out
 
@@ -627,11 +692,14 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
-    ap.add_argument("--warmup", type=int, default=300,
-                    help="untimed steps; a few hundred let the clocks settle after idle")
-    ap.add_argument("--all", action="store_true", help="also time every kernel of every configuration")
-    ap.add_argument("--only", default="", help="substring filter for --all (comma-separated: any of them)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--warmup", type=int, default=100,
+                    help="untimed steps after the fixed pre-roll that every case gets")
+    ap.add_argument("--all", action="store_true",
+                    help="also time the kernels beyond the configurations, the yardsticks and torch's operators")
+    ap.add_argument("--only", default="", help="substring filter for the kernels table (comma-separated: any of them)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table (headline only)")
+    ap.add_argument("--kernel-steps", type=int, default=KERNEL_STEPS, help="timed launches per kernels-table entry")
     ap.add_argument("--nsets", type=int, default=3, help="rotating buffer sets (working set > cache)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -644,38 +712,42 @@ def main():
     hk = _load()
     torch.cuda.set_device(0)
 
-    kernels = []
-    if args.all:
-        for name, make in CASES:
-            if args.only and not any(part in name for part in args.only.split(",")):
-                continue
-            launch, nbytes, rows = make(hk, torch, args.nsets)
-            ms, main_us = time_case(hk, torch, launch, args.steps, args.warmup,
-                                    profile_main=not getattr(launch, "no_hook", False))
-            if main_us is None:
-                main_us = ms * 1000
-            rec = {"case": name, "us": round(ms * 1000, 2), "main_kernel_us": round(main_us, 2),
-                   "GBps": round(nbytes / ms / 1e6, 1), "frac_of_8TBps": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
-                   "main_kernel_frac": round(nbytes / main_us / 1e3 / HBM_PEAK_GBS, 4),
-                   "rows_per_s": round(rows / ms * 1e3), "bytes": nbytes}
-            kernels.append(rec)
-            print("%-46s %9.2f us (main %8.2f us) %8.1f GB/s  %5.1f%% (main %5.1f%%)" % (
-                name, rec["us"], rec["main_kernel_us"], rec["GBps"], 100 * rec["frac_of_8TBps"],
-                100 * rec["main_kernel_frac"]), file=sys.stderr, flush=True)
-            del launch
-            torch.cuda.empty_cache()
-
-    # headline: fwd + bwd at the Llama-7B token shape
+    # headline: fwd + bwd at the Llama-7B token shape, exactly --steps steps after pre-roll and --warmup
     step, step_bytes, rows = case_rmsnorm(hk, torch, args.nsets, "both")
-    ms, _ = time_case(hk, torch, step, args.steps, args.warmup, profile_main=False)
+    ms, _, pre = time_case(hk, torch, step, args.steps, args.warmup, profile_main=False)
     bwd, bwd_bytes, _ = case_rmsnorm(hk, torch, args.nsets, "bwd")
-    _, bwd_us = time_case(hk, torch, bwd, args.steps, args.warmup, profile_main=True)
+    _, bwd_us, _ = time_case(hk, torch, bwd, max(args.steps, KERNEL_STEPS), args.warmup, profile_main=True)
+    del step, bwd
+    torch.cuda.empty_cache()
+
+    kernels = []
+    for name, make in CASES:
+        if args.no_kernels or not (args.all or is_config_case(name)):
+            continue
+        if args.only and not any(part in name for part in args.only.split(",")):
+            continue
+        launch, nbytes, nrows = make(hk, torch, args.nsets)
+        kms, main_us, _ = time_case(hk, torch, launch, args.kernel_steps, 0,
+                                    profile_main=not getattr(launch, "no_hook", False))
+        if main_us is None:
+            main_us = kms * 1000
+        rec = {"case": name, "us": round(kms * 1000, 2), "main_kernel_us": round(main_us, 2),
+               "GBps": round(nbytes / kms / 1e6, 1), "frac": round(nbytes / kms / 1e6 / HBM_PEAK_GBS, 4),
+               "main_kernel_frac": round(nbytes / main_us / 1e3 / HBM_PEAK_GBS, 4),
+               "rows_per_s": round(nrows / kms * 1e3), "bytes": nbytes}
+        kernels.append(rec)
+        print("%-46s %9.2f us (main %8.2f us) %8.1f GB/s  %5.1f%% (main %5.1f%%)" % (
+            name, rec["us"], rec["main_kernel_us"], rec["GBps"], 100 * rec["frac"],
+            100 * rec["main_kernel_frac"]), file=sys.stderr, flush=True)
+        del launch
+        torch.cuda.empty_cache()
+
     achieved = bwd_bytes / bwd_us / 1e3
     out = {
         "metric": "HBM GB/s, RMSNorm fwd+bwd at Llama-7B token shape (algorithmic bytes / step time)",
         "value": round(step_bytes / ms / 1e6, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "warmup": args.warmup, "preroll_steps": pre, "ms_per_step": round(ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "C4 RMSNorm fwd+bwd bf16 [32768 packed tokens x 4096], eps 1e-6, weight U(0.8,1.2)",
                    "rows": rows, "hidden": 4096, "storage": "bf16", "accumulate": "fp32", "us_fwd_plus_bwd": round(ms * 1000, 2),
                    "rows_per_s": round(rows / ms * 1e3), "frac_of_hbm_peak": round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)},
@@ -687,12 +759,13 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     if kernels:
+        out["kernel_steps"] = args.kernel_steps
         out["kernels"] = kernels
-        if not args.no_cpu:
-            out["cpu_kernels"] = cpu_kernels()
-            for rec in out["cpu_kernels"]:
-                print("cpu  %-66s %10.1f us %8.2f GB/s (%d threads)" % (rec["case"], rec["us"], rec["GBps"], rec["cores"]),
-                      file=sys.stderr, flush=True)
+    if not args.no_cpu and not args.no_kernels:
+        out["cpu_baselines"] = cpu_baselines()
+        for rec in out["cpu_baselines"]:
+            print("cpu  %-3s %-66s %10.1f us %8.2f GB/s (%d threads)" % (rec["config"], rec["case"], rec["us"], rec["value"],
+                                                                        rec["cores"]), file=sys.stderr, flush=True)
     print(json.dumps(out), flush=True)
 
 

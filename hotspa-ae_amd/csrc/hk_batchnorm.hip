@@ -313,6 +313,7 @@ void bn_bwd_apply_kernel(const T* dy, const T* x, T* dx, const CT* __restrict__ 
 // ---------------------------------------------------------------------------
 static int bn_splits(int64_t C, int64_t per_channel) {
   // enough workgroups to fill the chip (about 8 per compute unit), each with at least 8 loads per thread
+  if (C <= 0) return 1;   // an empty array: callers return before launching anything
   const int64_t want = (int64_t(device_cu_count()) * 8 + C - 1) / C;
   const int64_t most = std::max<int64_t>(1, per_channel / (256 * 8));
   return int(std::max<int64_t>(1, std::min<int64_t>(std::min(want, most), 1024)));

@@ -178,7 +178,15 @@ int hk_malloc(void** ptr, size_t bytes) {
   HK_REQUIRE(ptr, HK_ERR_INVALID, "hk_malloc: null output");
   *ptr = nullptr;
   if (bytes == 0) return HK_OK;
-  HK_CHECK_HIP(hipMalloc(ptr, bytes));
+  const hipError_t e = hipMalloc(ptr, bytes);
+  if (e != hipSuccess) {
+    // the runtime keeps a failed call as its "last error": take it out, or the launch check of the next
+    // kernel (after a caller has freed memory and retried) would report this failure as its own
+    (void)hipGetLastError();
+    *ptr = nullptr;
+    set_last_error("hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+    return HK_ERR_HIP;
+  }
   return HK_OK;
 }
 int hk_free(void* ptr) {
@@ -189,7 +197,13 @@ int hk_host_malloc(void** ptr, size_t bytes) {
   HK_REQUIRE(ptr, HK_ERR_INVALID, "hk_host_malloc: null output");
   *ptr = nullptr;
   if (bytes == 0) return HK_OK;
-  HK_CHECK_HIP(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+  const hipError_t e = hipHostMalloc(ptr, bytes, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    *ptr = nullptr;
+    set_last_error("hipHostMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+    return HK_ERR_HIP;
+  }
   return HK_OK;
 }
 int hk_host_free(void* ptr) {

@@ -451,6 +451,62 @@ ORACLE_API void refcpu_layernorm_fwd_f32(const float* x, const float* gamma, con
   }
 }
 
+/* LayerNormGradientCpu pass structure, hetu/impl/kernel/LayerNorm.cc:177-364: reduction_sum(dy) over rows ->
+ * dbias; calculate_gscale (:145-157) writes dy * x_hat into a full-size temporary; reduction_sum -> dscale;
+ * reduction_sum(dy) over columns -> db; binary_mul dy * x into a second full-size temporary; reduction_sum ->
+ * ds; calculate_grad_kernel (:159-174) writes dx.  The reference's CPU kernel leaves gamma out of db / ds / dx
+ * (its GPU kernel does not, LayerNorm.cu:198-201); gamma is applied here, as in the GPU formula:
+ *   db = sum_c gamma dy,  ds = sum_c gamma dy x,
+ *   dx = gamma dy / sd + ((db mean - ds)(x - mean) / (var + eps) - db) / cols / sd,   sd = sqrt(var + eps). */
+ORACLE_API void refcpu_layernorm_bwd_f32(const float* dy, const float* x, const float* gamma,
+                                         const float* mean, const float* var, int64_t rows,
+                                         int64_t cols, float eps, float* dx, float* dgamma,
+                                         float* dbeta) {
+  float* t1 = (float*)malloc(sizeof(float) * (size_t)(rows * cols));
+  float* t2 = (float*)malloc(sizeof(float) * (size_t)(rows * cols));
+  float* ds = (float*)malloc(sizeof(float) * (size_t)rows);
+  float* db = (float*)malloc(sizeof(float) * (size_t)rows);
+  /* dbias: column sums of dy (the reduction walks rows for a block of columns) */
+#pragma omp parallel for schedule(static)
+  for (int64_t c = 0; c < cols; ++c) {
+    float s = 0.f;
+    for (int64_t r = 0; r < rows; ++r) s += dy[r * cols + c];
+    dbeta[c] = s;
+  }
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < rows * cols; ++i) {
+    const int64_t r = i / cols;
+    t1[i] = dy[i] * ((x[i] - mean[r]) / sqrtf(var[r] + eps));
+  }
+#pragma omp parallel for schedule(static)
+  for (int64_t c = 0; c < cols; ++c) {
+    float s = 0.f;
+    for (int64_t r = 0; r < rows; ++r) s += t1[r * cols + c];
+    dgamma[c] = s;
+  }
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < rows * cols; ++i) {
+    const float gd = gamma[i % cols] * dy[i];
+    t1[i] = gd;
+    t2[i] = gd * x[i];
+  }
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    float s1 = 0.f, s2 = 0.f;
+    for (int64_t c = 0; c < cols; ++c) { s1 += t1[r * cols + c]; s2 += t2[r * cols + c]; }
+    db[r] = s1;
+    ds[r] = s2;
+  }
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < rows * cols; ++i) {
+    const int64_t r = i / cols;
+    const float sd = sqrtf(var[r] + eps);
+    const float tmp = (db[r] * mean[r] - ds[r]) * (x[i] - mean[r]) / (var[r] + eps);
+    dx[i] = t1[i] / sd + ((tmp - db[r]) / (float)cols) / sd;
+  }
+  free(t1); free(t2); free(ds); free(db);
+}
+
 /* RMSNorm has no CPU kernel in the reference (HT_DISPATCH_KERNEL_CUDA_ONLY,
  * hetu/graph/ops/RMSNorm.cc:42): this is the oracle formula in fp32. */
 ORACLE_API void refcpu_rmsnorm_fwd_f32(const float* x, const float* gamma, int64_t rows,
@@ -535,7 +591,26 @@ ORACLE_API void refcpu_sce_sparse_fwd_f32(const float* x, const int64_t* labels,
   }
 }
 
-/* ReduceCpu -> oneDNN reduction_sum (hetu/impl/kernel/Reduce.cc:41-68). */
+/* softmax_cross_entropy_sparse_gradient_cpu, hetu/impl/kernel/SoftmaxCrossEntropySparse.cc:41-75: an ignored row
+ * is written as zeros (:49-55), every other row as (softmax - onehot) * grad_loss[row] after a max pass and a
+ * sum-of-exponentials pass. */
+ORACLE_API void refcpu_sce_sparse_bwd_f32(const float* x, const int64_t* labels, const float* grad_loss,
+                                          int64_t rows, int64_t cols, int64_t ignored, float* dx) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    float* dr = dx + r * cols;
+    if (labels[r] == ignored) { memset(dr, 0, sizeof(float) * (size_t)cols); continue; }
+    const float* xr = x + r * cols;
+    float m = xr[0];
+    for (int64_t c = 1; c < cols; ++c) m = xr[c] > m ? xr[c] : m;
+    float s = 0.f;
+    for (int64_t c = 0; c < cols; ++c) s += expf(xr[c] - m);
+    const float g = grad_loss[r];
+    for (int64_t c = 0; c < cols; ++c) dr[c] = (expf(xr[c] - m) / s - (c == labels[r] ? 1.f : 0.f)) * g;
+  }
+}
+
+/* ReduceCpu -> oneDNN reduction_sum / reduction_mean (hetu/impl/kernel/Reduce.cc:41-68). */
 ORACLE_API void refcpu_reduce_sum_axis1_f32(const float* x, int64_t rows, int64_t cols, float* out) {
 #pragma omp parallel for schedule(static)
   for (int64_t r = 0; r < rows; ++r) {
@@ -549,6 +624,22 @@ ORACLE_API void refcpu_reduce_sum_axis0_f32(const float* x, int64_t rows, int64_
   memset(out, 0, sizeof(float) * (size_t)cols);
   for (int64_t r = 0; r < rows; ++r)
     for (int64_t c = 0; c < cols; ++c) out[c] += x[r * cols + c];
+}
+
+ORACLE_API void refcpu_reduce_mean_axis1_f32(const float* x, int64_t rows, int64_t cols, float* out) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    float s = 0.f;
+    for (int64_t c = 0; c < cols; ++c) s += x[r * cols + c];
+    out[r] = s / (float)cols;
+  }
+}
+
+ORACLE_API void refcpu_reduce_mean_axis0_f32(const float* x, int64_t rows, int64_t cols, float* out) {
+  memset(out, 0, sizeof(float) * (size_t)cols);
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t c = 0; c < cols; ++c) out[c] += x[r * cols + c];
+  for (int64_t c = 0; c < cols; ++c) out[c] /= (float)rows;
 }
 
 ORACLE_API int refcpu_num_threads(void) {

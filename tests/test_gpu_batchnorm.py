@@ -87,6 +87,9 @@ def test_refused_and_empty(hk, cuda):
     assert rc == -4                                       # no workspace
     e0 = torch.empty(0, 3, 4, 4, device=cuda)
     hk.batch_norm_fwd(e0, p, p, e0.clone(), 0.1, 1e-5, None, None, None, None)
+    c0 = torch.empty(2, 0, 4, 4, device=cuda)             # no channel at all: nothing to do, forward and backward
+    hk.batch_norm_fwd(c0, p[:0], p[:0], c0.clone(), 0.1, 1e-5, None, None, None, None)
+    hk.batch_norm_bwd(c0, c0, p[:0], c0.clone(), p[:0].clone(), p[:0].clone(), p[:0], p[:0])
     # a constant channel: variance 0, output = bias, finite statistics
     c = torch.full((4, 2, 8, 8), 3.0, device=cuda)
     y = torch.empty_like(c); sm = torch.empty(2, device=cuda); si = torch.empty(2, device=cuda)

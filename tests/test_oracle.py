@@ -366,6 +366,23 @@ def test_refcpu_ports_match_oracle():
     out1 = np.empty(rows, np.float32); out0 = np.empty(cols, np.float32)
     lib.refcpu_reduce_sum_axis1_f32(P(x), R, C, P(out1)); lib.refcpu_reduce_sum_axis0_f32(P(x), R, C, P(out0))
     assert np.allclose(out1, x.astype(np.float64).sum(1), atol=1e-3) and np.allclose(out0, x.astype(np.float64).sum(0), atol=1e-3)
+    lib.refcpu_reduce_mean_axis1_f32(P(x), R, C, P(out1)); lib.refcpu_reduce_mean_axis0_f32(P(x), R, C, P(out0))
+    assert np.allclose(out1, x.astype(np.float64).mean(1), atol=1e-5) and np.allclose(out0, x.astype(np.float64).mean(0), atol=1e-5)
+    # LayerNorm gradient in the reference's pass structure (statistics: mean and variance) against the float64 oracle
+    dy = g.standard_normal((rows, cols)).astype(np.float32)
+    _, em, ev, erstd = oracle.layernorm_fwd(x, gamma, beta, 1e-5)
+    mean32, var32 = em.astype(np.float32), ev.astype(np.float32)
+    dxl = np.empty_like(x); dgl = np.empty(cols, np.float32); dbl = np.empty(cols, np.float32)
+    lib.refcpu_layernorm_bwd_f32(P(dy), P(x), P(gamma), P(mean32), P(var32), R, C, ctypes.c_float(1e-5), P(dxl), P(dgl), P(dbl))
+    edx, edg, edb = oracle.layernorm_bwd(dy, x, gamma, em, erstd)
+    assert np.allclose(dxl, edx, rtol=1e-3, atol=1e-4) and np.allclose(dgl, edg, rtol=1e-3, atol=1e-3)
+    assert np.allclose(dbl, edb, rtol=1e-4, atol=1e-4)
+    # sparse cross-entropy gradient: ignored row all zeros, the rest against the float64 oracle
+    gl = g.standard_normal(rows).astype(np.float32)
+    dxc = np.empty_like(x)
+    lib.refcpu_sce_sparse_bwd_f32(P(x), lab.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)), P(gl), R, C, ctypes.c_int64(-100), P(dxc))
+    assert not dxc[3].any()
+    assert np.allclose(dxc, oracle.sce_sparse_bwd(x, lab, gl, -100), rtol=1e-4, atol=1e-6)
 
 
 @pytest.mark.parametrize("p", [1, 2, 3, 4])

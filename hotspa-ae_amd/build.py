@@ -19,7 +19,8 @@ LIB = os.path.join(HERE, "lib")
 OBJ = os.path.join(HERE, "build")
 INCLUDE = os.path.join(ROOT, "include")
 
-HIP_SOURCES = ["hk_device.hip", "hk_norm.hip", "hk_softmax.hip", "hk_sce.hip", "hk_reduce.hip", "hk_nll.hip",
+HIP_SOURCES = ["hk_norm_bwd_bf16.hip", "hk_norm_bwd_f32.hip", "hk_norm_bwd_f16.hip", "hk_norm_fwd_bf16.hip",
+               "hk_norm_fwd_f32.hip", "hk_norm_fwd_f16.hip", "hk_device.hip", "hk_norm.hip", "hk_softmax.hip", "hk_sce.hip", "hk_reduce.hip", "hk_nll.hip",
                "hk_dropout_ln.hip", "hk_elementwise.hip", "hk_vocab_ce.hip", "hk_batchnorm.hip"]
 
 HIPCC_FLAGS = [
@@ -51,7 +52,9 @@ def _stale(src, obj):
     if not os.path.exists(obj):
         return True
     own = os.path.getmtime(os.path.join(CSRC, src))
-    common = os.path.getmtime(os.path.join(CSRC, "hk_common.cuh"))
+    # hk_common.h is included by every source; the norm headers only by the norm sources
+    shared = [f for f in os.listdir(CSRC) if f.endswith(".h") and (f == "hk_common.h" or src.startswith("hk_norm"))]
+    common = max(os.path.getmtime(os.path.join(CSRC, f)) for f in shared)
     header = max(os.path.getmtime(os.path.join(INCLUDE, f)) for f in os.listdir(INCLUDE))
     return os.path.getmtime(obj) < max(own, common, header)
 

@@ -9,7 +9,7 @@
 // running statistics and the per-channel coefficients, (3) an element-wise pass,
 // one 16-byte vector per thread.  The input is read twice and the output written
 // once in the forward; the backward reads dy and x twice and writes dx once.
-#include "hk_common.cuh"
+#include "hk_common.h"
 
 #include <algorithm>
 #include <type_traits>

@@ -278,6 +278,10 @@ __device__ __forceinline__ P group_allreduce_tuple(P a, float* scratch, int firs
   return group_combine_tuple<P>(a, scratch, first_wave, nwaves);
 }
 
+// Every thread walks the group's waves in order.  The reads are wave-uniform LDS broadcasts which the
+// compiler keeps in flight together; a butterfly over per-lane reads (one LDS round trip, then DPP merges on
+// every lane) was measured slower at every group width (5120-column LayerNorm backward, ten waves: 96.5
+// against 91.0 us).
 template <typename P>
 __device__ __forceinline__ P group_combine_tuple(P a, float* scratch, int first_wave, int nwaves) {
   if (nwaves == 1) return a;
@@ -315,6 +319,12 @@ template <int KK>
 struct SumTuple {
   static constexpr int K = KK;
   float v[KK];
+  static __device__ __forceinline__ SumTuple identity() {
+    SumTuple r;
+#pragma unroll
+    for (int k = 0; k < KK; ++k) r.v[k] = 0.f;
+    return r;
+  }
   static __device__ __forceinline__ SumTuple merge(SumTuple a, const SumTuple& b) {
 #pragma unroll
     for (int k = 0; k < KK; ++k) a.v[k] += b.v[k];
@@ -326,6 +336,7 @@ struct SumTuple {
 struct MomentTuple {
   static constexpr int K = 3;
   float v[3];
+  static __device__ __forceinline__ MomentTuple identity() { return MomentTuple{{0.f, 0.f, 0.f}}; }
   static __device__ __forceinline__ MomentTuple merge(const MomentTuple& a, const MomentTuple& b) {
     MomentTuple r;
     const float n = a.v[0] + b.v[0];
@@ -365,6 +376,13 @@ template <int KK>
 struct OnlineSoftmaxTuple {
   static constexpr int K = KK;
   float v[KK];
+  static __device__ __forceinline__ OnlineSoftmaxTuple identity() {
+    OnlineSoftmaxTuple r;
+    r.v[0] = -__builtin_huge_valf();
+    r.v[1] = 0.f;
+    if constexpr (KK == 3) r.v[2] = -__builtin_huge_valf();
+    return r;
+  }
   static __device__ __forceinline__ OnlineSoftmaxTuple merge(const OnlineSoftmaxTuple& a,
                                                               const OnlineSoftmaxTuple& b) {
     OnlineSoftmaxTuple r;

@@ -1,6 +1,6 @@
 // Device / memory / stream / event entry points of the C-ABI, plus the small
 // utility kernels (fill, streaming copy, strided gather) and the tuning table.
-#include "hk_common.cuh"
+#include "hk_common.h"
 
 #include <cstdarg>
 #include <cstdio>

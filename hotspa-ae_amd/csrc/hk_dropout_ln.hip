@@ -13,7 +13,7 @@
 // Dropout mask: element e of the input draws word e % 4 of Philox4x32-10 (key =
 // seed, counter = (2 * (e / 4) + input number, offset)), so the mask does not
 // depend on the launch shape.
-#include "hk_common.cuh"
+#include "hk_common.h"
 
 #include <algorithm>
 #include <type_traits>

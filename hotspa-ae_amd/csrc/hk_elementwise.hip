@@ -6,7 +6,7 @@
 // the 16-bit types (one rounding at the store), fp64 for fp64.  Outputs may
 // alias an input of the same shape (every thread reads its elements before it
 // writes them).
-#include "hk_common.cuh"
+#include "hk_common.h"
 
 #include <type_traits>
 

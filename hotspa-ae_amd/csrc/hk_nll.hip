@@ -4,7 +4,7 @@
 // The forward is a gather of one element per row.  The backward writes every element of the output
 // exactly once: the zero fill and the scatter are one pass of 128-bit stores, where the reference clears
 // the array and then scatters in a second kernel (hetu/impl/kernel/NLLLoss.cu:8-41, :88-128).
-#include "hk_common.cuh"
+#include "hk_common.h"
 
 namespace hk {
 

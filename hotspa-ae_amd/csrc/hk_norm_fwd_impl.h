@@ -1,0 +1,350 @@
+// LayerNorm / RMSNorm forward kernels and their launch logic, included by the per-type instantiation files.
+//
+// A row lives in registers as packed 128-bit vectors (one HBM read), statistics are Welford moments merged with
+// Chan's update across lanes (DPP, equal-count form when the row fills every lane) and waves (LDS), output is
+// written with 128-bit stores.  One wavefront per row for short rows, one workgroup per row for long rows.
+#pragma once
+
+#include "hk_norm.h"
+
+namespace hk {
+
+// T: element type; NV: 16-byte vectors per thread; WAVE_ROW: one wavefront per
+// row (4 rows per 256-thread block) instead of one workgroup per row;
+// HAS_RES: x = x0 + residual is formed in fp32 and optionally written back.
+template <typename T, int NV, bool WAVE_ROW, bool HAS_RES>
+__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
+void norm_fwd_kernel(NormFwdArgs a) {
+  constexpr int VEC = VecIO<T>::N;
+  __shared__ float red[kMaxWaves * 3];
+
+  const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
+  const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
+  const int64_t row = WAVE_ROW
+      ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index()
+      : int64_t(blockIdx.x);
+  if (WAVE_ROW && row >= a.rows) return;  // wave-uniform; no block barrier in this mode
+  const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
+
+  const T* xr = static_cast<const T*>(a.x) + row * a.x_pitch;
+  u32x4 raw[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) raw[i] = u32x4{0, 0, 0, 0};
+  [[maybe_unused]] float xf[HAS_RES ? NV * VEC : 1];
+
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * tpr + t;
+    if (v < a.nvec) raw[i] = ld16(xr + v * VEC);
+  }
+  if constexpr (HAS_RES) {
+    const T* rr = static_cast<const T*>(a.residual) + row * a.res_pitch;
+    T* xo = a.x_out ? static_cast<T*>(a.x_out) + row * a.xout_pitch : nullptr;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = i * tpr + t;
+      if (v < a.nvec) {
+        float f0[VEC], f1[VEC];
+        VecIO<T>::unpack(raw[i], f0);
+        VecIO<T>::unpack(ld16(rr + v * VEC), f1);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) xf[i * VEC + j] = f0[j] + f1[j];
+        if (xo) st16(xo + v * VEC, VecIO<T>::pack(&xf[i * VEC]));
+      }
+    }
+  }
+
+  auto get = [&](int i, float* f) {
+    if constexpr (HAS_RES) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) f[j] = xf[i * VEC + j];
+    } else {
+      VecIO<T>::unpack(raw[i], f);
+    }
+  };
+
+  float mu, rs, var;
+  if (a.is_rms) {
+    SumTuple<2> s;
+    s.v[0] = 0.f; s.v[1] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      if (i * tpr + t < a.nvec) {
+        float f[VEC];
+        get(i, f);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) { s.v[0] += f[j]; s.v[1] = fmaf(f[j], f[j], s.v[1]); }
+      }
+    }
+    s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red, 0, nwaves);
+    mu = s.v[0] * a.inv_cols;
+    const float ms = s.v[1] * a.inv_cols;  // mean(x^2) = var + mu^2
+    var = fmaxf(ms - mu * mu, 0.f);
+    rs = 1.0f / sqrtf(ms + a.eps);
+  } else {
+    // Welford statistics, merged with Chan's parallel update: each thread forms (count, mean, M2) of the
+    // elements it holds in registers, lanes merge through a DPP butterfly, waves through LDS.  When every
+    // thread holds the same count (the row fills all vector slots: a uniform test) each butterfly step
+    // merges equal-sized halves and needs no reciprocal; a ragged row takes the general update.
+    float s = 0.f;
+    int cnt = 0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      if (i * tpr + t < a.nvec) {
+        float f[VEC];
+        get(i, f);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) s += f[j];
+        cnt += VEC;
+      }
+    }
+    const bool even = a.nvec == NV * tpr;                    // uniform
+    const float mean_t = even ? s * (1.0f / float(NV * VEC)) : (cnt > 0 ? s / float(cnt) : 0.f);
+    float m2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      if (i * tpr + t < a.nvec) {
+        float f[VEC];
+        get(i, f);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) { const float d = f[j] - mean_t; m2 = fmaf(d, d, m2); }
+      }
+    }
+    MomentTuple m;
+    m.v[0] = float(cnt); m.v[1] = mean_t; m.v[2] = m2;
+    if (even) {
+      EqualMomentTuple e;
+      e.v[0] = m.v[0]; e.v[1] = m.v[1]; e.v[2] = m.v[2];
+      e = wave_allreduce_tuple(e);
+      m.v[0] = e.v[0]; m.v[1] = e.v[1]; m.v[2] = e.v[2];
+    } else {
+      m = wave_allreduce_tuple(m);
+    }
+    // waves are merged one after the other (growing count on one side): the general update
+    if (!WAVE_ROW) m = group_combine_tuple(m, red, 0, nwaves);
+    mu = m.v[1];
+    var = m.v[2] * a.inv_cols;
+    rs = 1.0f / sqrtf(var + a.eps);
+  }
+
+  if (t == 0) {
+    store_stat<T>(a.mean, row, mu, a.stats_f32);
+    store_stat<T>(a.stat, row, a.stat_kind == HK_STAT_VAR ? var : rs, a.stats_f32);
+  }
+
+  const float shift = a.is_rms ? 0.f : mu;
+  T* yr = static_cast<T*>(a.y) + row * a.y_pitch;
+  // gamma / beta are fetched here, after the reduction, and one vector ahead of the arithmetic: holding all of
+  // them in registers (across the reduction, or merely across this loop) costs resident waves, which is what
+  // hides the row's own load latency.  The scheduling fences keep the compiler from hoisting every fetch to the
+  // top of the unrolled loop again.  The four cases of missing parameters are separate straight-line copies, so
+  // that no fetch sits inside a branch.
+  const T* gp = static_cast<const T*>(a.gamma);
+  const T* bp = static_cast<const T*>(a.beta);
+  auto epilogue = [&](auto has_g, auto has_b) {
+    constexpr bool HG = decltype(has_g)::value, HB = decltype(has_b)::value;
+    [[maybe_unused]] u32x4 gn, bn;
+    auto fetch = [&](int i) {
+      int v = i * tpr + t;
+      v = v < a.nvec ? v : 0;                 // a lane past the row's end reads the first vector; never used
+      if constexpr (HG) gn = ld16_keep(gp + v * VEC);
+      if constexpr (HB) bn = ld16_keep(bp + v * VEC);
+    };
+    fetch(0);
+    static_for<NV>([&](auto idx) {
+      constexpr int i = decltype(idx)::value;
+      [[maybe_unused]] const u32x4 gc = gn, bc = bn;
+      if constexpr (i + 1 < NV) fetch(i + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      const int v = i * tpr + t;
+      if (v < a.nvec) {
+        float f[VEC], g[VEC], b[VEC];
+        get(i, f);
+        if constexpr (HG) VecIO<T>::unpack(gc, g);
+        if constexpr (HB) VecIO<T>::unpack(bc, b);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float n = rs * (f[j] - shift);
+          f[j] = HG ? (HB ? fmaf(g[j], n, b[j]) : g[j] * n) : (HB ? n + b[j] : n);
+        }
+        const u32x4 o = VecIO<T>::pack(f);
+        if (a.stream_store) st16_stream(yr + v * VEC, o);
+        else st16(yr + v * VEC, o);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  if (gp && bp) epilogue(std::true_type{}, std::true_type{});
+  else if (gp) epilogue(std::true_type{}, std::false_type{});
+  else if (bp) epilogue(std::false_type{}, std::true_type{});
+  else epilogue(std::false_type{}, std::false_type{});
+}
+
+// Fallback for rows that are not a whole number of 16-byte vectors, are not
+// 16-byte aligned, or do not fit the register file: one workgroup per row,
+// three strided passes (the re-reads hit L2).  CT is the arithmetic type.
+template <typename T, typename CT>
+__global__ __launch_bounds__(256)
+void norm_fwd_generic_kernel(NormFwdArgs a) {
+  __shared__ CT lds[256];
+  const int64_t row = blockIdx.x;
+  const T* xr = static_cast<const T*>(a.x) + row * a.x_pitch;
+  const T* rr = a.residual ? static_cast<const T*>(a.residual) + row * a.res_pitch : nullptr;
+  T* xo = a.x_out ? static_cast<T*>(a.x_out) + row * a.xout_pitch : nullptr;
+  auto ldx = [&](int c) -> CT {
+    CT v = GenericIO<T, CT>::ld(xr + c);
+    if (rr) v += GenericIO<T, CT>::ld(rr + c);
+    return v;
+  };
+  CT s = 0, ss = 0;
+  for (int c = threadIdx.x; c < a.cols; c += blockDim.x) {
+    const CT v = ldx(c);
+    if (xo) GenericIO<T, CT>::st(xo + c, v);
+    s += v;
+    ss += v * v;
+  }
+  s = block_sum_generic<CT>(s, lds);
+  const CT inv = CT(1) / CT(a.cols);
+  const CT mu = s * inv;
+  CT var, rs;
+  if (a.is_rms) {
+    ss = block_sum_generic<CT>(ss, lds);
+    const CT ms = ss * inv;
+    var = ms - mu * mu;
+    if (var < CT(0)) var = CT(0);
+    rs = CT(1) / sqrt(ms + CT(a.eps));
+  } else {
+    CT m2 = 0;
+    for (int c = threadIdx.x; c < a.cols; c += blockDim.x) {
+      const CT d = ldx(c) - mu;
+      m2 += d * d;
+    }
+    m2 = block_sum_generic<CT>(m2, lds);
+    var = m2 * inv;
+    rs = CT(1) / sqrt(var + CT(a.eps));
+  }
+  if (threadIdx.x == 0) {
+    const CT st = a.stat_kind == HK_STAT_VAR ? var : rs;
+    if (a.mean) {
+      if (a.stats_f32) static_cast<float*>(a.mean)[row] = float(mu);
+      else GenericIO<T, CT>::st(static_cast<T*>(a.mean) + row, mu);
+    }
+    if (a.stat) {
+      if (a.stats_f32) static_cast<float*>(a.stat)[row] = float(st);
+      else GenericIO<T, CT>::st(static_cast<T*>(a.stat) + row, st);
+    }
+  }
+  const CT shift = a.is_rms ? CT(0) : mu;
+  T* yr = static_cast<T*>(a.y) + row * a.y_pitch;
+  const T* gp = static_cast<const T*>(a.gamma);
+  const T* bp = static_cast<const T*>(a.beta);
+  for (int c = threadIdx.x; c < a.cols; c += blockDim.x) {
+    const CT g = gp ? GenericIO<T, CT>::ld(gp + c) : CT(1);
+    const CT b = bp ? GenericIO<T, CT>::ld(bp + c) : CT(0);
+    GenericIO<T, CT>::st(yr + c, g * (rs * (ldx(c) - shift)) + b);
+  }
+}
+
+template <typename T, bool WAVE_ROW, bool HAS_RES>
+static int launch_norm_fwd_nv(const NormFwdArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
+  profile_before(s);
+  switch (nv) {
+    case 1: hipLaunchKernelGGL((norm_fwd_kernel<T, 1, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 2: hipLaunchKernelGGL((norm_fwd_kernel<T, 2, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 3: hipLaunchKernelGGL((norm_fwd_kernel<T, 3, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 4: hipLaunchKernelGGL((norm_fwd_kernel<T, 4, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 5: hipLaunchKernelGGL((norm_fwd_kernel<T, 5, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 6: hipLaunchKernelGGL((norm_fwd_kernel<T, 6, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 8: hipLaunchKernelGGL((norm_fwd_kernel<T, 8, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 16: hipLaunchKernelGGL((norm_fwd_kernel<T, 16, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    default:
+      set_last_error("norm_fwd: no kernel for %d vectors per thread", nv);
+      return HK_ERR_UNSUPPORTED;
+  }
+  profile_after(s);
+  return launch_check("norm_fwd_kernel");
+}
+
+// Picks threads-per-row and vectors-per-thread for a row of `nvec` 16-byte
+// vectors.  Returns false when the row does not fit the register kernels.
+static bool pick_row_shape(int nvec, int forced_threads, int max_nv, int wave_row_max_nv,
+                           int* threads, int* nv) {
+  if (forced_threads > 0) {
+    int t = std::min(1024, std::max(64, (forced_threads + 63) / 64 * 64));
+    int n = pow2_ceil((nvec + t - 1) / t);
+    if (n > max_nv) return false;
+    *threads = t;
+    *nv = n;
+    return true;
+  }
+  // short rows: one wavefront per row
+  if (nvec <= 64 * wave_row_max_nv && nvec <= 256) {
+    *threads = 64;
+    *nv = pow2_ceil((nvec + 63) / 64);
+    return true;
+  }
+  // medium rows (measured on MI355X: 4096 / 5120 bf16 columns, 4096 fp32
+  // columns): small workgroups of 128..256 threads per row stream fastest.
+  // First choice: the fewest vectors per thread that fill every lane exactly
+  // (5120 bf16 columns = 640 vectors = 128 threads x 5): no idle lanes, and the
+  // statistics merge takes its equal-count form.
+  static const int kCounts[] = {2, 3, 4, 5, 6, 8};
+  for (int n : kCounts) {
+    if (n > max_nv) break;
+    int t = ((nvec + n - 1) / n + 63) / 64 * 64;
+    if (t <= 256 && n * t == nvec) {
+      *threads = t;
+      *nv = n;
+      return true;
+    }
+  }
+  for (int n = 2; n <= max_nv; n <<= 1) {
+    int t = ((nvec + n - 1) / n + 63) / 64 * 64;
+    if (t <= 256) {
+      *threads = t;
+      *nv = n;
+      return true;
+    }
+  }
+  // long rows: one workgroup per row, smallest power-of-two vector count that
+  // keeps the block within 1024 threads
+  for (int n = 4; n <= max_nv; n <<= 1) {
+    int t = ((nvec + n - 1) / n + 63) / 64 * 64;
+    if (t <= 1024) {
+      *threads = t;
+      *nv = n;
+      return true;
+    }
+  }
+  return false;
+}
+
+template <typename T>
+int norm_fwd_typed(NormFwdArgs a, hipStream_t s) {
+  constexpr int VEC = VecIO<T>::N;
+  auto pitch_ok = [](int64_t p) { return p % VEC == 0; };
+  const bool vec_ok = (a.cols % VEC == 0) && aligned16(a.x) && aligned16(a.y) &&
+                      aligned16(a.gamma) && aligned16(a.beta) && aligned16(a.residual) &&
+                      aligned16(a.x_out) && pitch_ok(a.x_pitch) && pitch_ok(a.y_pitch) &&
+                      (!a.residual || pitch_ok(a.res_pitch)) && (!a.x_out || pitch_ok(a.xout_pitch));
+  int threads = 0, nv = 0;
+  a.nvec = a.cols / VEC;
+  const bool has_res = a.residual != nullptr;
+  // with a residual the summed row is kept unpacked: halve the budget
+  const int max_nv = has_res ? (VEC == 4 ? 16 : 8) : 16;
+  const int wave_nv = has_res ? (VEC == 4 ? 8 : 4) : (VEC == 4 ? 16 : 8);
+  if (vec_ok && pick_row_shape(a.nvec, tune_get(TUNE_NORM_FWD_THREADS), max_nv, wave_nv, &threads, &nv)) {
+    if (threads == 64) {
+      dim3 grid(unsigned((a.rows + 3) / 4)), block(256);
+      return has_res ? launch_norm_fwd_nv<T, true, true>(a, nv, grid, block, s)
+                     : launch_norm_fwd_nv<T, true, false>(a, nv, grid, block, s);
+    }
+    dim3 grid{unsigned(a.rows)}, block{unsigned(threads)};
+    return has_res ? launch_norm_fwd_nv<T, false, true>(a, nv, grid, block, s)
+                   : launch_norm_fwd_nv<T, false, false>(a, nv, grid, block, s);
+  }
+  hipLaunchKernelGGL((norm_fwd_generic_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
+  return launch_check("norm_fwd_generic_kernel");
+}
+
+} // namespace hk

@@ -13,7 +13,7 @@
 // bf16 / fp16 accumulate in fp32; mean multiplies the final sum by
 // float(1 / reduce_num).  Every kernel takes the reduction (identity + combine)
 // as a type, so all five share the same planning and memory access.
-#include "hk_common.cuh"
+#include "hk_common.h"
 
 #include <algorithm>
 #include <limits>

@@ -7,7 +7,7 @@
 // rescales the stored exponentials into (softmax - onehot) * grad_loss and
 // writes the row once.  Rows whose label equals the ignored index are not read
 // at all: loss 0 / a zero gradient row is written.
-#include "hk_common.cuh"
+#include "hk_common.h"
 
 #include <algorithm>
 

@@ -5,7 +5,7 @@
 // merged online across lanes (DPP) and waves (LDS), and the stored exponentials
 // are rescaled on the way out, so exp is evaluated once per element.
 // One wavefront per row for short rows, one workgroup per row for long rows.
-#include "hk_common.cuh"
+#include "hk_common.h"
 
 #include <algorithm>
 

@@ -2,7 +2,7 @@
 // columns [vocab_start, vocab_end) of the logits; what crosses devices (the row
 // maximum, the sum of exponentials, the picked logit) is reduced by the caller
 // between these kernels.
-#include "hk_common.cuh"
+#include "hk_common.h"
 
 #include <type_traits>
 

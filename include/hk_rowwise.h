@@ -139,6 +139,18 @@ HK_API int hk_layer_norm_fwd(int dtype, const void* x, const void* gamma, const 
                              void* y, void* mean, void* stat, int stats_dtype, int stat_kind,
                              int64_t rows, int64_t cols, float eps, hkStream_t stream);
 
+/* The same on rows that lie a fixed pitch apart: row r of x starts x_pitch ELEMENTS after row r - 1, likewise
+ * y (x_pitch, y_pitch >= cols; pitch == cols is the dense call above).  This is the view a column slice
+ * x[:, a:b] of a wider array, or a row-padded buffer, presents; the last dimension must have unit stride.
+ * A pitch that is a whole number of 16-byte vectors keeps the 128-bit kernels; any other pitch is taken by
+ * the element-wise fallback.  Replaces, for such views, the per-element StridedOffsetCalculator of the
+ * reference (hetu/impl/utils/offset_calculator.cuh:16-68), which its LayerNorm operators run on because they
+ * accept non-contiguous inputs (hetu/graph/ops/LayerNorm.h:78-80). */
+HK_API int hk_layer_norm_fwd_pitched(int dtype, const void* x, int64_t x_pitch, const void* gamma,
+                                     const void* beta, void* y, int64_t y_pitch, void* mean, void* stat,
+                                     int stats_dtype, int stat_kind, int64_t rows, int64_t cols,
+                                     float eps, hkStream_t stream);
+
 /* Bytes of scratch hk_layer_norm_bwd / hk_dropout_add_ln_bwd need for the
  * column-sum partials of dgamma / dbeta. */
 HK_API int hk_norm_bwd_workspace_bytes(int dtype, int64_t rows, int64_t cols, size_t* bytes);
@@ -158,6 +170,14 @@ HK_API int hk_layer_norm_bwd(int dtype, const void* dy, const void* x_or_y, cons
                              void* dbeta, int64_t rows, int64_t cols, float eps,
                              int memory_efficient, int clamp_gamma, void* workspace,
                              size_t workspace_bytes, hkStream_t stream);
+
+/* hk_layer_norm_bwd on row-pitched dy, x_or_y and dx (see hk_layer_norm_fwd_pitched). */
+HK_API int hk_layer_norm_bwd_pitched(int dtype, const void* dy, int64_t dy_pitch, const void* x_or_y,
+                                     int64_t x_pitch, const void* gamma, const void* beta,
+                                     const void* mean, const void* stat, int stats_dtype, int stat_kind,
+                                     void* dx, int64_t dx_pitch, void* dgamma, void* dbeta, int64_t rows,
+                                     int64_t cols, float eps, int memory_efficient, int clamp_gamma,
+                                     void* workspace, size_t workspace_bytes, hkStream_t stream);
 
 /* ======================================================================== *
  * Dropout-add-LayerNorm / RMSNorm (flash-attention layer_norm path).
@@ -186,6 +206,21 @@ HK_API int hk_dropout_add_ln_bwd(int itype, int rtype, int wtype, const void* dz
                                  void* dresidual, void* dgamma, void* dbeta, int64_t rows,
                                  int64_t cols, int is_rms_norm, void* workspace,
                                  size_t workspace_bytes, hkStream_t stream);
+
+/* The two calls above on row-pitched arrays (see hk_layer_norm_fwd_pitched): every [rows, cols] operand
+ * carries its own pitch in elements; the pitch of an absent optional operand is ignored. */
+HK_API int hk_dropout_add_ln_fwd_pitched(int itype, int rtype, int wtype, const void* x0, int64_t x0_pitch,
+                                         const void* residual, int64_t residual_pitch, const void* gamma,
+                                         const void* beta, void* z, int64_t z_pitch, void* x_out,
+                                         int64_t x_out_pitch, void* mu, void* rsigma, int64_t rows,
+                                         int64_t cols, float eps, int is_rms_norm, hkStream_t stream);
+HK_API int hk_dropout_add_ln_bwd_pitched(int itype, int rtype, int wtype, const void* dz, int64_t dz_pitch,
+                                         const void* dx_in, int64_t dx_in_pitch, const void* x,
+                                         int64_t x_pitch, const void* mu, const void* rsigma,
+                                         const void* gamma, void* dx0, int64_t dx0_pitch, void* dresidual,
+                                         int64_t dresidual_pitch, void* dgamma, void* dbeta, int64_t rows,
+                                         int64_t cols, int is_rms_norm, void* workspace,
+                                         size_t workspace_bytes, hkStream_t stream);
 
 /* hk_dropout_add_ln_bwd for callers that cannot allocate device memory and so have no workspace to
  * pass: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no

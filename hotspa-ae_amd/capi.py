@@ -110,15 +110,28 @@ class Event:
 
 
 # ---------------------------------------------------------------------------
-# operators: tensors are torch CUDA tensors, dense, already allocated
+# operators: tensors are torch CUDA tensors, already allocated; dense, or 2-D views whose rows lie a constant
+# pitch apart (a column slice of a wider tensor), which go to the *_pitched entry points as they are
 # ---------------------------------------------------------------------------
+def _pitch(t, cols):
+    """Row pitch, in elements, of a [rows, cols] operand: its row stride when it is a 2-D view with a unit-stride
+    last dimension, cols when it is dense (any number of leading dimensions) or absent."""
+    if t is None or t.is_contiguous():
+        return cols
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise HkError(-1, "operand must be dense or a 2-D view with a unit-stride last dimension, got shape %s "
+                          "strides %s" % (tuple(t.shape), tuple(t.stride())))
+    return t.stride(0) if t.shape[0] > 1 else cols
+
+
 def layer_norm_fwd(x, gamma, beta, y, mean, stat, eps, stat_kind=HK_STAT_RSTD, stream=None):
     rows = x.numel() // x.shape[-1] if x.numel() else 0
     cols = x.shape[-1]
-    check(lib().hk_layer_norm_fwd(dtype_code(x), _ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _ptr(mean), _ptr(stat),
-                                  dtype_code(mean if mean is not None else stat), ctypes.c_int(stat_kind),
-                                  _i64(rows), _i64(cols), ctypes.c_float(eps),
-                                  stream if stream is not None else current_stream()))
+    check(lib().hk_layer_norm_fwd_pitched(dtype_code(x), _ptr(x), _i64(_pitch(x, cols)), _ptr(gamma), _ptr(beta),
+                                          _ptr(y), _i64(_pitch(y, cols)), _ptr(mean), _ptr(stat),
+                                          dtype_code(mean if mean is not None else stat), ctypes.c_int(stat_kind),
+                                          _i64(rows), _i64(cols), ctypes.c_float(eps),
+                                          stream if stream is not None else current_stream()))
 
 
 def norm_bwd_workspace_bytes(dtype, rows, cols):
@@ -141,22 +154,25 @@ def layer_norm_bwd(dy, x_or_y, gamma, beta, mean, stat, dx, dgamma, dbeta, eps, 
     if workspace is None:
         workspace = _workspace(norm_bwd_workspace_bytes(dtype_code(dy), rows, cols), dy.device)
     wsb = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    check(lib().hk_layer_norm_bwd(dtype_code(dy), _ptr(dy), _ptr(x_or_y), _ptr(gamma), _ptr(beta), _ptr(mean),
-                                  _ptr(stat), dtype_code(stat), ctypes.c_int(stat_kind), _ptr(dx), _ptr(dgamma),
-                                  _ptr(dbeta), _i64(rows), _i64(cols), ctypes.c_float(eps),
-                                  ctypes.c_int(int(memory_efficient)), ctypes.c_int(int(clamp_gamma)),
-                                  _ptr(workspace), ctypes.c_size_t(wsb),
-                                  stream if stream is not None else current_stream()))
+    check(lib().hk_layer_norm_bwd_pitched(dtype_code(dy), _ptr(dy), _i64(_pitch(dy, cols)), _ptr(x_or_y),
+                                          _i64(_pitch(x_or_y, cols)), _ptr(gamma), _ptr(beta), _ptr(mean),
+                                          _ptr(stat), dtype_code(stat), ctypes.c_int(stat_kind), _ptr(dx),
+                                          _i64(_pitch(dx, cols)), _ptr(dgamma), _ptr(dbeta), _i64(rows), _i64(cols),
+                                          ctypes.c_float(eps), ctypes.c_int(int(memory_efficient)),
+                                          ctypes.c_int(int(clamp_gamma)), _ptr(workspace), ctypes.c_size_t(wsb),
+                                          stream if stream is not None else current_stream()))
     return workspace
 
 
 def dropout_add_ln_fwd(x0, residual, gamma, beta, z, x_out, mu, rsigma, eps, is_rms, stream=None):
     rows, cols = x0.shape
     rtype = dtype_code(residual) if residual is not None else dtype_code(x0)
-    check(lib().hk_dropout_add_ln_fwd(dtype_code(x0), rtype, dtype_code(gamma), _ptr(x0), _ptr(residual),
-                                      _ptr(gamma), _ptr(beta), _ptr(z), _ptr(x_out), _ptr(mu), _ptr(rsigma),
-                                      _i64(rows), _i64(cols), ctypes.c_float(eps), ctypes.c_int(int(is_rms)),
-                                      stream if stream is not None else current_stream()))
+    check(lib().hk_dropout_add_ln_fwd_pitched(dtype_code(x0), rtype, dtype_code(gamma), _ptr(x0),
+                                              _i64(_pitch(x0, cols)), _ptr(residual), _i64(_pitch(residual, cols)),
+                                              _ptr(gamma), _ptr(beta), _ptr(z), _i64(_pitch(z, cols)), _ptr(x_out),
+                                              _i64(_pitch(x_out, cols)), _ptr(mu), _ptr(rsigma), _i64(rows),
+                                              _i64(cols), ctypes.c_float(eps), ctypes.c_int(int(is_rms)),
+                                              stream if stream is not None else current_stream()))
 
 
 def dropout_add_ln_bwd(dz, dx_in, x, mu, rsigma, gamma, dx0, dresidual, dgamma, dbeta, is_rms,
@@ -165,11 +181,14 @@ def dropout_add_ln_bwd(dz, dx_in, x, mu, rsigma, gamma, dx0, dresidual, dgamma, 
     if workspace is None:
         workspace = _workspace(norm_bwd_workspace_bytes(dtype_code(dz), rows, cols), dz.device)
     wsb = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    check(lib().hk_dropout_add_ln_bwd(dtype_code(dz), dtype_code(x), dtype_code(gamma), _ptr(dz), _ptr(dx_in),
-                                      _ptr(x), _ptr(mu), _ptr(rsigma), _ptr(gamma), _ptr(dx0), _ptr(dresidual),
-                                      _ptr(dgamma), _ptr(dbeta), _i64(rows), _i64(cols), ctypes.c_int(int(is_rms)),
-                                      _ptr(workspace), ctypes.c_size_t(wsb),
-                                      stream if stream is not None else current_stream()))
+    check(lib().hk_dropout_add_ln_bwd_pitched(dtype_code(dz), dtype_code(x), dtype_code(gamma), _ptr(dz),
+                                              _i64(_pitch(dz, cols)), _ptr(dx_in), _i64(_pitch(dx_in, cols)),
+                                              _ptr(x), _i64(_pitch(x, cols)), _ptr(mu), _ptr(rsigma), _ptr(gamma),
+                                              _ptr(dx0), _i64(_pitch(dx0, cols)), _ptr(dresidual),
+                                              _i64(_pitch(dresidual, cols)), _ptr(dgamma), _ptr(dbeta), _i64(rows),
+                                              _i64(cols), ctypes.c_int(int(is_rms)), _ptr(workspace),
+                                              ctypes.c_size_t(wsb),
+                                              stream if stream is not None else current_stream()))
     return workspace
 
 
@@ -412,12 +431,24 @@ def _odi(shape, dim):
 
 
 def softmax_fwd(x, y, dim=-1, stream=None):
+    if x.dim() == 2 and dim in (-1, 1) and not (x.is_contiguous() and y.is_contiguous()):
+        rows, cols = x.shape
+        check(lib().hk_softmax_fwd_pitched(dtype_code(x), _ptr(x), _i64(_pitch(x, cols)), _ptr(y),
+                                           _i64(_pitch(y, cols)), _i64(rows), _i64(cols),
+                                           stream if stream is not None else current_stream()))
+        return
     o, d, i = _odi(list(x.shape), dim)
     check(lib().hk_softmax_fwd(dtype_code(x), _ptr(x), _ptr(y), _i64(o), _i64(d), _i64(i),
                                stream if stream is not None else current_stream()))
 
 
 def softmax_bwd(y, dy, dx, dim=-1, stream=None):
+    if y.dim() == 2 and dim in (-1, 1) and not (y.is_contiguous() and dy.is_contiguous() and dx.is_contiguous()):
+        rows, cols = y.shape
+        check(lib().hk_softmax_bwd_pitched(dtype_code(y), _ptr(y), _i64(_pitch(y, cols)), _ptr(dy),
+                                           _i64(_pitch(dy, cols)), _ptr(dx), _i64(_pitch(dx, cols)), _i64(rows),
+                                           _i64(cols), stream if stream is not None else current_stream()))
+        return
     o, d, i = _odi(list(y.shape), dim)
     check(lib().hk_softmax_bwd(dtype_code(y), _ptr(y), _ptr(dy), _ptr(dx), _i64(o), _i64(d), _i64(i),
                                stream if stream is not None else current_stream()))
@@ -426,16 +457,18 @@ def softmax_bwd(y, dy, dx, dim=-1, stream=None):
 def sce_sparse_fwd(logits, labels, loss, ignored_index, stream=None):
     cols = logits.shape[-1]
     rows = logits.numel() // cols if logits.numel() else 0
-    check(lib().hk_sce_sparse_fwd(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(loss), _i64(rows), _i64(cols),
-                                  _i64(ignored_index), stream if stream is not None else current_stream()))
+    check(lib().hk_sce_sparse_fwd_pitched(dtype_code(logits), _ptr(logits), _i64(_pitch(logits, cols)), _ptr(labels),
+                                          _ptr(loss), _i64(rows), _i64(cols), _i64(ignored_index),
+                                          stream if stream is not None else current_stream()))
 
 
 def sce_sparse_bwd(logits, labels, grad_loss, dlogits, ignored_index, stream=None):
     cols = logits.shape[-1]
     rows = logits.numel() // cols if logits.numel() else 0
-    check(lib().hk_sce_sparse_bwd(dtype_code(logits), _ptr(logits), _ptr(labels), _ptr(grad_loss), _ptr(dlogits),
-                                  _i64(rows), _i64(cols), _i64(ignored_index),
-                                  stream if stream is not None else current_stream()))
+    check(lib().hk_sce_sparse_bwd_pitched(dtype_code(logits), _ptr(logits), _i64(_pitch(logits, cols)), _ptr(labels),
+                                          _ptr(grad_loss), _ptr(dlogits), _i64(_pitch(dlogits, cols)), _i64(rows),
+                                          _i64(cols), _i64(ignored_index),
+                                          stream if stream is not None else current_stream()))
 
 
 def sce_sparse_bwd_reduced(logits, labels, grad_output, scale, dlogits, ignored_index, stream=None):

@@ -24,6 +24,8 @@ struct SceArgs {
   const void* grad_loss;   // backward
   void* out;               // forward: loss [rows]; backward: dlogits
   int64_t rows;
+  // elements between the starts of consecutive rows of logits / dense labels / dlogits (0 = dense: cols)
+  int64_t x_pitch, lab_pitch, out_pitch;
   int cols;
   int nvec;
   int64_t ignored_index;
@@ -82,7 +84,7 @@ void sce_sparse_fwd_kernel(SceArgs a) {
     }
     return;
   }
-  const T* xr = static_cast<const T*>(a.logits) + row * int64_t(a.cols);
+  const T* xr = static_cast<const T*>(a.logits) + row * a.x_pitch;
   // slots past the row's end hold -inf: they change neither the maximum nor the sum
   float f[NV * VEC];
   {
@@ -148,7 +150,7 @@ void sce_sparse_bwd_kernel(SceArgs a) {
   row_coords<WAVE_ROW>(tpr, t, row, nwaves);
   if (WAVE_ROW && row >= a.rows) return;
 
-  T* dxr = static_cast<T*>(a.out) + row * int64_t(a.cols);
+  T* dxr = static_cast<T*>(a.out) + row * a.out_pitch;
   const int64_t label = a.labels[row];
   if (label == a.ignored_index) {
     const u32x4 z = {0, 0, 0, 0};
@@ -162,7 +164,7 @@ void sce_sparse_bwd_kernel(SceArgs a) {
     }
     return;
   }
-  const T* xr = static_cast<const T*>(a.logits) + row * int64_t(a.cols);
+  const T* xr = static_cast<const T*>(a.logits) + row * a.x_pitch;
   u32x4 raw[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -227,8 +229,8 @@ void sce_dense_kernel(SceArgs a) {
   row_coords<WAVE_ROW>(tpr, t, row, nwaves);
   if (WAVE_ROW && row >= a.rows) return;
 
-  const T* xr = static_cast<const T*>(a.logits) + row * int64_t(a.cols);
-  const T* lr = static_cast<const T*>(a.dlabels) + row * int64_t(a.cols);
+  const T* xr = static_cast<const T*>(a.logits) + row * a.x_pitch;
+  const T* lr = static_cast<const T*>(a.dlabels) + row * a.lab_pitch;
   u32x4 rx[NV], rl[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -279,7 +281,7 @@ void sce_dense_kernel(SceArgs a) {
     const float g = sce_row_grad<T, float>(a, row);
     const float ML = (p.v[0] == kNegInf) ? 0.f : p.v[0];
     const float inv = 1.0f / p.v[1];
-    T* dxr = static_cast<T*>(a.out) + row * int64_t(a.cols);
+    T* dxr = static_cast<T*>(a.out) + row * a.out_pitch;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = i * tpr + t;
@@ -334,7 +336,7 @@ void sce_generic_kernel(SceArgs a) {
   __shared__ CT lds[256];
   const int64_t row = blockIdx.x;
   const int64_t cols = a.cols;
-  const T* xr = static_cast<const T*>(a.logits) + row * cols;
+  const T* xr = static_cast<const T*>(a.logits) + row * a.x_pitch;
   int64_t label = 0;
   if (MODE < 2) {
     label = a.labels[row];
@@ -350,7 +352,7 @@ void sce_generic_kernel(SceArgs a) {
           }
         }
       } else {
-        T* dxr = static_cast<T*>(a.out) + row * cols;
+        T* dxr = static_cast<T*>(a.out) + row * a.out_pitch;
         for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) SceIO<T, CT>::st(dxr + c, CT(0));
       }
       return;
@@ -380,7 +382,7 @@ void sce_generic_kernel(SceArgs a) {
       SceIO<T, CT>::st(static_cast<T*>(a.out) + row, r);
     }
   } else if (MODE == 2) {
-    const T* lr = static_cast<const T*>(a.dlabels) + row * cols;
+    const T* lr = static_cast<const T*>(a.dlabels) + row * a.lab_pitch;
     CT sl = 0, slx = 0;
     for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
       const CT l = SceIO<T, CT>::ld(lr + c);
@@ -394,8 +396,8 @@ void sce_generic_kernel(SceArgs a) {
   } else {
     const CT g = sce_row_grad<T, CT>(a, row);
     const CT inv = CT(1) / s;
-    T* dxr = static_cast<T*>(a.out) + row * cols;
-    const T* lr = MODE == 3 ? static_cast<const T*>(a.dlabels) + row * cols : nullptr;
+    T* dxr = static_cast<T*>(a.out) + row * a.out_pitch;
+    const T* lr = MODE == 3 ? static_cast<const T*>(a.dlabels) + row * a.lab_pitch : nullptr;
     for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
       CT pr = sce_exp<CT>(SceIO<T, CT>::ld(xr + c) - m) * inv;
       if (MODE == 1) pr = (c == label) ? (pr * g - g) : pr * g;
@@ -469,7 +471,8 @@ template <typename T, int MODE>
 static int sce_typed(SceArgs a, hipStream_t s) {
   constexpr int VEC = VecIO<T>::N;
   const bool vec_ok = a.cols % VEC == 0 && aligned16(a.logits) && aligned16(a.dlabels) &&
-                      (MODE == 0 || MODE == 2 || aligned16(a.out));
+                      (MODE == 0 || MODE == 2 || (aligned16(a.out) && a.out_pitch % VEC == 0)) &&
+                      a.x_pitch % VEC == 0 && (MODE < 2 || a.lab_pitch % VEC == 0);
   a.nvec = a.cols / VEC;
   // sparse forward only keeps the packed row; the others keep 32 floats or two rows
   const int max_nv = (MODE == 0) ? 8 : 32 / VEC;
@@ -497,6 +500,11 @@ static int sce_dispatch(int dtype, SceArgs& a, hipStream_t s, const char* who) {
   HK_REQUIRE(MODE >= 2 || a.labels, HK_ERR_INVALID, "%s: null labels", who);
   HK_REQUIRE(MODE < 2 || a.dlabels, HK_ERR_INVALID, "%s: null labels", who);
   HK_REQUIRE((MODE & 1) == 0 || a.grad_loss, HK_ERR_INVALID, "%s: null grad_loss", who);
+  if (a.x_pitch == 0) a.x_pitch = a.cols;
+  if (a.lab_pitch == 0) a.lab_pitch = a.cols;
+  if (a.out_pitch == 0) a.out_pitch = a.cols;
+  HK_REQUIRE(a.x_pitch >= a.cols && a.lab_pitch >= a.cols && a.out_pitch >= a.cols, HK_ERR_INVALID,
+             "%s: a row pitch is smaller than the %d columns of a row", who, a.cols);
   a.stream_store = tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1;
   switch (dtype) {
     case HK_FLOAT32: return sce_typed<float, MODE>(a, s);
@@ -524,6 +532,28 @@ int hk_sce_sparse_fwd(int dtype, const void* logits, const int64_t* labels, void
   a.logits = logits; a.labels = labels; a.out = loss; a.rows = rows; a.cols = int(cols);
   a.ignored_index = ignored_index;
   return sce_dispatch<0>(dtype, a, as_hip(stream), "hk_sce_sparse_fwd");
+}
+
+int hk_sce_sparse_fwd_pitched(int dtype, const void* logits, int64_t logits_pitch, const int64_t* labels,
+                              void* loss, int64_t rows, int64_t cols, int64_t ignored_index, hkStream_t stream) {
+  HK_REQUIRE(cols <= 0x3fffffff, HK_ERR_INVALID, "hk_sce_sparse_fwd_pitched: cols too large");
+  HK_REQUIRE(logits_pitch > 0, HK_ERR_INVALID, "hk_sce_sparse_fwd_pitched: a row pitch must be positive");
+  SceArgs a{};
+  a.logits = logits; a.labels = labels; a.out = loss; a.rows = rows; a.cols = int(cols);
+  a.x_pitch = logits_pitch; a.ignored_index = ignored_index;
+  return sce_dispatch<0>(dtype, a, as_hip(stream), "hk_sce_sparse_fwd_pitched");
+}
+
+int hk_sce_sparse_bwd_pitched(int dtype, const void* logits, int64_t logits_pitch, const int64_t* labels,
+                              const void* grad_loss, void* dlogits, int64_t dlogits_pitch, int64_t rows,
+                              int64_t cols, int64_t ignored_index, hkStream_t stream) {
+  HK_REQUIRE(cols <= 0x3fffffff, HK_ERR_INVALID, "hk_sce_sparse_bwd_pitched: cols too large");
+  HK_REQUIRE(logits_pitch > 0 && dlogits_pitch > 0, HK_ERR_INVALID,
+             "hk_sce_sparse_bwd_pitched: a row pitch must be positive");
+  SceArgs a{};
+  a.logits = logits; a.labels = labels; a.grad_loss = grad_loss; a.out = dlogits; a.rows = rows;
+  a.cols = int(cols); a.x_pitch = logits_pitch; a.out_pitch = dlogits_pitch; a.ignored_index = ignored_index;
+  return sce_dispatch<1>(dtype, a, as_hip(stream), "hk_sce_sparse_bwd_pitched");
 }
 
 int hk_vocab_parallel_ce_stats(int dtype, const void* logits, const int64_t* labels, float* stats, int64_t rows,

@@ -19,6 +19,7 @@ struct SoftmaxArgs {
   const void* dy;   // backward only
   void* out;        // forward: y;      backward: dx
   int64_t rows;
+  int64_t x_pitch, dy_pitch, out_pitch;   // elements between row starts (== cols for a dense array)
   int cols;
   int nvec;
   int stream_store;
@@ -37,7 +38,7 @@ void softmax_fwd_kernel(SoftmaxArgs a) {
   if (WAVE_ROW && row >= a.rows) return;
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
 
-  const T* xr = static_cast<const T*>(a.x) + row * int64_t(a.cols);
+  const T* xr = static_cast<const T*>(a.x) + row * a.x_pitch;
   u32x4 raw[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -71,7 +72,7 @@ void softmax_fwd_kernel(SoftmaxArgs a) {
   const float ML = (p.v[0] == kNegInf) ? 0.f : p.v[0];
   const float scale = __builtin_amdgcn_exp2f(ml - ML) / p.v[1];
 
-  T* yr = static_cast<T*>(a.out) + row * int64_t(a.cols);
+  T* yr = static_cast<T*>(a.out) + row * a.out_pitch;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int v = i * tpr + t;
@@ -98,8 +99,8 @@ void softmax_bwd_kernel(SoftmaxArgs a) {
   if (WAVE_ROW && row >= a.rows) return;
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
 
-  const T* yr = static_cast<const T*>(a.x) + row * int64_t(a.cols);
-  const T* dyr = static_cast<const T*>(a.dy) + row * int64_t(a.cols);
+  const T* yr = static_cast<const T*>(a.x) + row * a.x_pitch;
+  const T* dyr = static_cast<const T*>(a.dy) + row * a.dy_pitch;
   u32x4 ry[NV], rdy[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -120,7 +121,7 @@ void softmax_bwd_kernel(SoftmaxArgs a) {
   }
   s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red, 0, nwaves);
   const float dot = s.v[0];
-  T* dxr = static_cast<T*>(a.out) + row * int64_t(a.cols);
+  T* dxr = static_cast<T*>(a.out) + row * a.out_pitch;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int v = i * tpr + t;
@@ -204,10 +205,10 @@ __device__ __forceinline__ CT block_reduce_generic(CT v, CT* lds, bool is_max) {
 
 template <typename T, typename CT>
 __global__ __launch_bounds__(256)
-void softmax_fwd_longrow_kernel(const T* x, T* y, int64_t cols) {
+void softmax_fwd_longrow_kernel(const T* x, T* y, int64_t cols, int64_t x_pitch, int64_t y_pitch) {
   __shared__ CT lds[256];
-  const T* xr = x + int64_t(blockIdx.x) * cols;
-  T* yr = y + int64_t(blockIdx.x) * cols;
+  const T* xr = x + int64_t(blockIdx.x) * x_pitch;
+  T* yr = y + int64_t(blockIdx.x) * y_pitch;
   CT m = -__builtin_huge_val();
   for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
     const CT v = SmIO<T, CT>::ld(xr + c);
@@ -224,16 +225,19 @@ void softmax_fwd_longrow_kernel(const T* x, T* y, int64_t cols) {
 
 template <typename T, typename CT>
 __global__ __launch_bounds__(256)
-void softmax_bwd_longrow_kernel(const T* y, const T* dy, T* dx, int64_t cols) {
+void softmax_bwd_longrow_kernel(const T* y, const T* dy, T* dx, int64_t cols, int64_t y_pitch,
+                                int64_t dy_pitch, int64_t dx_pitch) {
   __shared__ CT lds[256];
-  const int64_t base = int64_t(blockIdx.x) * cols;
+  const T* yr = y + int64_t(blockIdx.x) * y_pitch;
+  const T* dyr = dy + int64_t(blockIdx.x) * dy_pitch;
+  T* dxr = dx + int64_t(blockIdx.x) * dx_pitch;
   CT dot = 0;
   for (int64_t c = threadIdx.x; c < cols; c += blockDim.x)
-    dot += SmIO<T, CT>::ld(y + base + c) * SmIO<T, CT>::ld(dy + base + c);
+    dot += SmIO<T, CT>::ld(yr + c) * SmIO<T, CT>::ld(dyr + c);
   dot = block_reduce_generic<CT>(dot, lds, false);
   for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
-    const CT yv = SmIO<T, CT>::ld(y + base + c);
-    SmIO<T, CT>::st(dx + base + c, yv * (SmIO<T, CT>::ld(dy + base + c) - dot));
+    const CT yv = SmIO<T, CT>::ld(yr + c);
+    SmIO<T, CT>::st(dxr + c, yv * (SmIO<T, CT>::ld(dyr + c) - dot));
   }
 }
 
@@ -296,7 +300,8 @@ static int launch_softmax_nv(const SoftmaxArgs& a, int nv, dim3 grid, dim3 block
 template <typename T, bool BWD>
 static int softmax_lastdim_typed(SoftmaxArgs a, hipStream_t s) {
   constexpr int VEC = VecIO<T>::N;
-  const bool vec_ok = a.cols % VEC == 0 && aligned16(a.x) && aligned16(a.dy) && aligned16(a.out);
+  const bool vec_ok = a.cols % VEC == 0 && aligned16(a.x) && aligned16(a.dy) && aligned16(a.out) &&
+                      a.x_pitch % VEC == 0 && a.out_pitch % VEC == 0 && (!BWD || a.dy_pitch % VEC == 0);
   a.nvec = a.cols / VEC;
   // forward keeps NV*VEC exponentials per thread: at most 64 floats
   // backward holds y and dy: at most 4 vectors of each per thread
@@ -314,25 +319,27 @@ static int softmax_lastdim_typed(SoftmaxArgs a, hipStream_t s) {
   if constexpr (BWD) {
     hipLaunchKernelGGL((softmax_bwd_longrow_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s,
                        static_cast<const T*>(a.x), static_cast<const T*>(a.dy), static_cast<T*>(a.out),
-                       int64_t(a.cols));
+                       int64_t(a.cols), a.x_pitch, a.dy_pitch, a.out_pitch);
     return launch_check("softmax_bwd_longrow_kernel");
   } else {
     hipLaunchKernelGGL((softmax_fwd_longrow_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s,
-                       static_cast<const T*>(a.x), static_cast<T*>(a.out), int64_t(a.cols));
+                       static_cast<const T*>(a.x), static_cast<T*>(a.out), int64_t(a.cols), a.x_pitch, a.out_pitch);
     return launch_check("softmax_fwd_longrow_kernel");
   }
 }
 
 template <typename T, typename CT, bool BWD>
 static int softmax_strided_typed(const void* x, const void* dy, void* out, int64_t outer, int64_t dim,
-                                 int64_t inner, hipStream_t s) {
+                                 int64_t inner, int64_t x_pitch, int64_t dy_pitch, int64_t out_pitch,
+                                 hipStream_t s) {
   if (inner == 1) {
     if constexpr (BWD) {
       hipLaunchKernelGGL((softmax_bwd_longrow_kernel<T, CT>), dim3(unsigned(outer)), dim3(256), 0, s,
-                         static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<T*>(out), dim);
+                         static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<T*>(out), dim, x_pitch,
+                         dy_pitch, out_pitch);
     } else {
       hipLaunchKernelGGL((softmax_fwd_longrow_kernel<T, CT>), dim3(unsigned(outer)), dim3(256), 0, s,
-                         static_cast<const T*>(x), static_cast<T*>(out), dim);
+                         static_cast<const T*>(x), static_cast<T*>(out), dim, x_pitch, out_pitch);
     }
     return launch_check("softmax_longrow_kernel");
   }
@@ -349,17 +356,28 @@ static int softmax_strided_typed(const void* x, const void* dy, void* out, int64
   return launch_check("softmax_strided_kernel");
 }
 
+// x_pitch / dy_pitch / out_pitch: elements between the starts of consecutive rows when inner == 1 (0: dense, the
+// row's own length); a dimension other than the last (inner > 1) only exists for dense arrays.
 template <bool BWD>
 static int softmax_dispatch(int dtype, const void* x, const void* dy, void* out, int64_t outer,
-                            int64_t dim, int64_t inner, hipStream_t s, const char* who) {
+                            int64_t dim, int64_t inner, int64_t x_pitch, int64_t dy_pitch, int64_t out_pitch,
+                            hipStream_t s, const char* who) {
   HK_REQUIRE(outer >= 0 && dim >= 0 && inner >= 0, HK_ERR_INVALID, "%s: negative extent", who);
   if (outer == 0 || dim == 0 || inner == 0) return HK_OK;
   HK_REQUIRE(x && out && (!BWD || dy), HK_ERR_INVALID, "%s: null input/output", who);
+  if (x_pitch == 0) x_pitch = dim;
+  if (dy_pitch == 0) dy_pitch = dim;
+  if (out_pitch == 0) out_pitch = dim;
+  HK_REQUIRE(x_pitch >= dim && out_pitch >= dim && dy_pitch >= dim, HK_ERR_INVALID,
+             "%s: a row pitch is smaller than the %lld columns of a row", who, (long long)dim);
+  HK_REQUIRE(inner == 1 || (x_pitch == dim && dy_pitch == dim && out_pitch == dim), HK_ERR_INVALID,
+             "%s: row pitches only apply to the last dimension", who);
   HK_REQUIRE(outer <= 0x7fffffffLL && (outer * inner + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID,
              "%s: too many rows", who);
   if (inner == 1 && dim <= 0x3fffffff && dtype != HK_FLOAT64) {
     SoftmaxArgs a{};
     a.x = x; a.dy = dy; a.out = out; a.rows = outer; a.cols = int(dim);
+    a.x_pitch = x_pitch; a.dy_pitch = dy_pitch; a.out_pitch = out_pitch;
     a.stream_store = tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1;
     switch (dtype) {
       case HK_FLOAT32: return softmax_lastdim_typed<float, BWD>(a, s);
@@ -369,10 +387,10 @@ static int softmax_dispatch(int dtype, const void* x, const void* dy, void* out,
     }
   }
   switch (dtype) {
-    case HK_FLOAT32: return softmax_strided_typed<float, float, BWD>(x, dy, out, outer, dim, inner, s);
-    case HK_BFLOAT16: return softmax_strided_typed<bf16, float, BWD>(x, dy, out, outer, dim, inner, s);
-    case HK_FLOAT16: return softmax_strided_typed<fp16, float, BWD>(x, dy, out, outer, dim, inner, s);
-    case HK_FLOAT64: return softmax_strided_typed<double, double, BWD>(x, dy, out, outer, dim, inner, s);
+    case HK_FLOAT32: return softmax_strided_typed<float, float, BWD>(x, dy, out, outer, dim, inner, x_pitch, dy_pitch, out_pitch, s);
+    case HK_BFLOAT16: return softmax_strided_typed<bf16, float, BWD>(x, dy, out, outer, dim, inner, x_pitch, dy_pitch, out_pitch, s);
+    case HK_FLOAT16: return softmax_strided_typed<fp16, float, BWD>(x, dy, out, outer, dim, inner, x_pitch, dy_pitch, out_pitch, s);
+    case HK_FLOAT64: return softmax_strided_typed<double, double, BWD>(x, dy, out, outer, dim, inner, x_pitch, dy_pitch, out_pitch, s);
     default:
       set_last_error("%s: not implemented for dtype %d", who, dtype);
       return HK_ERR_UNSUPPORTED;
@@ -387,12 +405,27 @@ extern "C" {
 
 int hk_softmax_fwd(int dtype, const void* x, void* y, int64_t outer, int64_t dim, int64_t inner,
                    hkStream_t stream) {
-  return softmax_dispatch<false>(dtype, x, nullptr, y, outer, dim, inner, as_hip(stream), "hk_softmax_fwd");
+  return softmax_dispatch<false>(dtype, x, nullptr, y, outer, dim, inner, 0, 0, 0, as_hip(stream), "hk_softmax_fwd");
+}
+
+int hk_softmax_fwd_pitched(int dtype, const void* x, int64_t x_pitch, void* y, int64_t y_pitch, int64_t rows,
+                           int64_t cols, hkStream_t stream) {
+  HK_REQUIRE(x_pitch > 0 && y_pitch > 0, HK_ERR_INVALID, "hk_softmax_fwd_pitched: a row pitch must be positive");
+  return softmax_dispatch<false>(dtype, x, nullptr, y, rows, cols, 1, x_pitch, x_pitch, y_pitch, as_hip(stream),
+                                 "hk_softmax_fwd_pitched");
 }
 
 int hk_softmax_bwd(int dtype, const void* y, const void* dy, void* dx, int64_t outer, int64_t dim,
                    int64_t inner, hkStream_t stream) {
-  return softmax_dispatch<true>(dtype, y, dy, dx, outer, dim, inner, as_hip(stream), "hk_softmax_bwd");
+  return softmax_dispatch<true>(dtype, y, dy, dx, outer, dim, inner, 0, 0, 0, as_hip(stream), "hk_softmax_bwd");
+}
+
+int hk_softmax_bwd_pitched(int dtype, const void* y, int64_t y_pitch, const void* dy, int64_t dy_pitch, void* dx,
+                           int64_t dx_pitch, int64_t rows, int64_t cols, hkStream_t stream) {
+  HK_REQUIRE(y_pitch > 0 && dy_pitch > 0 && dx_pitch > 0, HK_ERR_INVALID,
+             "hk_softmax_bwd_pitched: a row pitch must be positive");
+  return softmax_dispatch<true>(dtype, y, dy, dx, rows, cols, 1, y_pitch, dy_pitch, dx_pitch, as_hip(stream),
+                                "hk_softmax_bwd_pitched");
 }
 
 } // extern "C"

@@ -23,12 +23,13 @@ void FusedLayerNormCuda(const NDArray& in_arr, const NDArray& ln_scale, const ND
   HT_ASSERT(mean_arr->dtype() == kFloat32 && var_arr->dtype() == kFloat32)
     << "the fused layer norm keeps its statistics in float32, got " << mean_arr->dtype() << " / "
     << var_arr->dtype();
-  HT_ASSERT_CONTIGUOUS(out_arr);
   HT_ASSERT_CONTIGUOUS(mean_arr);
   HT_ASSERT_CONTIGUOUS(var_arr);
 
   int64_t rows, cols;
   SplitRows(in_arr, reduce_dims, rows, cols);
+  int64_t x_pitch = cols, y_pitch = cols;
+  HT_ASSERT_ROW_PITCHED(out_arr, reduce_dims, &y_pitch);
   HT_ASSERT(int64_t(ln_scale->numel()) == cols && int64_t(ln_bias->numel()) == cols)
     << "scale " << ln_scale->shape() << " / bias " << ln_bias->shape() << " do not match " << cols << " columns";
   HT_ASSERT(int64_t(mean_arr->numel()) == rows && int64_t(var_arr->numel()) == rows)
@@ -37,10 +38,12 @@ void FusedLayerNormCuda(const NDArray& in_arr, const NDArray& ln_scale, const ND
 
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
-  NDArray x = Dense(in_arr, stream), g = Dense(ln_scale, stream), b = Dense(ln_bias, stream);
-  HK_CALL(hk_layer_norm_fwd(int(in_arr->dtype()), x->raw_data_ptr(), g->raw_data_ptr(), b->raw_data_ptr(),
-                            out_arr->raw_data_ptr(), mean_arr->raw_data_ptr(), var_arr->raw_data_ptr(), HK_FLOAT32,
-                            HK_STAT_RSTD, rows, cols, eps, hip_stream));
+  NDArray x = RowOperand(in_arr, reduce_dims, stream, &x_pitch);
+  NDArray g = Dense(ln_scale, stream), b = Dense(ln_bias, stream);
+  HK_CALL(hk_layer_norm_fwd_pitched(int(in_arr->dtype()), x->raw_data_ptr(), x_pitch, g->raw_data_ptr(),
+                                    b->raw_data_ptr(), out_arr->raw_data_ptr(), y_pitch, mean_arr->raw_data_ptr(),
+                                    var_arr->raw_data_ptr(), HK_FLOAT32, HK_STAT_RSTD, rows, cols, eps,
+                                    hip_stream));
   NDArray::MarkUsedBy({x, g, b, mean_arr, var_arr, out_arr}, stream);
 }
 
@@ -66,12 +69,13 @@ void FusedLayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr,
   HT_ASSERT(mean_arr->dtype() == kFloat32 && var_arr->dtype() == kFloat32)
     << "the fused layer norm keeps its statistics in float32";
   HT_ASSERT(!inplace || ln_bias.is_defined()) << "the memory-efficient backward needs the bias to undo it";
-  HT_ASSERT_CONTIGUOUS(grad_arr);
   HT_ASSERT_CONTIGUOUS(grad_scale);
   HT_ASSERT_CONTIGUOUS(grad_bias);
 
   int64_t rows, cols;
   SplitRows(in_arr, reduce_dims, rows, cols);
+  int64_t dy_pitch = cols, x_pitch = cols, dx_pitch = cols;
+  HT_ASSERT_ROW_PITCHED(grad_arr, reduce_dims, &dx_pitch);
   HT_ASSERT(int64_t(ln_scale->numel()) == cols && int64_t(grad_scale->numel()) == cols &&
             int64_t(grad_bias->numel()) == cols)
     << "scale / grad_scale / grad_bias must hold " << cols << " values";
@@ -90,17 +94,19 @@ void FusedLayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr,
     }
     return;
   }
-  NDArray dy = Dense(out_grads, stream), xy = Dense(in_arr, stream), g = Dense(ln_scale, stream);
+  NDArray dy = RowOperand(out_grads, reduce_dims, stream, &dy_pitch);
+  NDArray xy = RowOperand(in_arr, reduce_dims, stream, &x_pitch), g = Dense(ln_scale, stream);
   NDArray b = Dense(ln_bias, stream), mean = Dense(mean_arr, stream), rstd = Dense(var_arr, stream);
   size_t ws_bytes = 0;
   HK_CALL(hk_norm_bwd_workspace_bytes(dt, rows, cols, &ws_bytes));
   NDArray ws = Scratch(ws_bytes, in_arr->device(), stream);
   // gamma enters dx through clamp_by_magnitude(gamma, eps) in both modes
   // (FusedLayerNorm.cu:911-938)
-  HK_CALL(hk_layer_norm_bwd(dt, dy->raw_data_ptr(), xy->raw_data_ptr(), g->raw_data_ptr(), PtrOrNull(b),
-                            mean->raw_data_ptr(), rstd->raw_data_ptr(), HK_FLOAT32, HK_STAT_RSTD,
-                            grad_arr->raw_data_ptr(), grad_scale->raw_data_ptr(), grad_bias->raw_data_ptr(), rows,
-                            cols, eps, inplace ? 1 : 0, /*clamp_gamma=*/1, MutPtrOrNull(ws), ws_bytes, hip_stream));
+  HK_CALL(hk_layer_norm_bwd_pitched(dt, dy->raw_data_ptr(), dy_pitch, xy->raw_data_ptr(), x_pitch, g->raw_data_ptr(),
+                                    PtrOrNull(b), mean->raw_data_ptr(), rstd->raw_data_ptr(), HK_FLOAT32,
+                                    HK_STAT_RSTD, grad_arr->raw_data_ptr(), dx_pitch, grad_scale->raw_data_ptr(),
+                                    grad_bias->raw_data_ptr(), rows, cols, eps, inplace ? 1 : 0, /*clamp_gamma=*/1,
+                                    MutPtrOrNull(ws), ws_bytes, hip_stream));
   NDArray::MarkUsedBy({dy, xy, g, b, mean, rstd, grad_arr, grad_scale, grad_bias, ws}, stream);
 }
 

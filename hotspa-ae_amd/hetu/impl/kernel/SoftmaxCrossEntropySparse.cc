@@ -35,9 +35,10 @@ void SoftmaxCrossEntropySparseCuda(const NDArray& pred, const NDArray& label, ND
 
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
-  NDArray p = Dense(pred, stream), l = Dense(label, stream);
-  HK_CALL(hk_sce_sparse_fwd(int(pred->dtype()), p->raw_data_ptr(), l->data_ptr<int64_t>(), loss->raw_data_ptr(), rows,
-                            cols, ignored_index, hip_stream));
+  int64_t p_pitch = cols;
+  NDArray p = RowOperand(pred, 1, stream, &p_pitch), l = Dense(label, stream);
+  HK_CALL(hk_sce_sparse_fwd_pitched(int(pred->dtype()), p->raw_data_ptr(), p_pitch, l->data_ptr<int64_t>(),
+                                    loss->raw_data_ptr(), rows, cols, ignored_index, hip_stream));
   NDArray::MarkUsedBy({p, l, loss}, stream);
 }
 
@@ -54,9 +55,14 @@ void SparseGradient(const NDArray& pred, const NDArray& label, const NDArray& gr
   HT_ASSERT_SAME_DTYPE(pred, output);
   HT_ASSERT_SAME_DTYPE(pred, grad_loss);
   HT_ASSERT(label->dtype() == kInt64) << "labels must be int64 class ids, got " << label->dtype();
-  HT_ASSERT_CONTIGUOUS(output);
   int64_t rows, cols;
   RowsCols(pred, rows, cols);
+  int64_t p_pitch = cols, out_pitch = cols;
+  if (scale) {
+    HT_ASSERT_CONTIGUOUS(output);
+  } else {
+    HT_ASSERT_ROW_PITCHED(output, 1, &out_pitch);
+  }
   HT_ASSERT(int64_t(label->numel()) == rows) << "labels " << label->shape() << " must hold one value per row of "
                                              << pred->shape();
   if (scale) {
@@ -70,14 +76,16 @@ void SparseGradient(const NDArray& pred, const NDArray& label, const NDArray& gr
 
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
-  NDArray p = Dense(pred, stream), l = Dense(label, stream), g = Dense(grad_loss, stream);
+  NDArray p = scale ? Dense(pred, stream) : RowOperand(pred, 1, stream, &p_pitch);
+  NDArray l = Dense(label, stream), g = Dense(grad_loss, stream);
   if (scale) {
     HK_CALL(hk_sce_sparse_bwd_reduced(int(pred->dtype()), p->raw_data_ptr(), l->data_ptr<int64_t>(),
                                       g->raw_data_ptr(), *scale, output->raw_data_ptr(), rows, cols, ignored_index,
                                       hip_stream));
   } else {
-    HK_CALL(hk_sce_sparse_bwd(int(pred->dtype()), p->raw_data_ptr(), l->data_ptr<int64_t>(), g->raw_data_ptr(),
-                              output->raw_data_ptr(), rows, cols, ignored_index, hip_stream));
+    HK_CALL(hk_sce_sparse_bwd_pitched(int(pred->dtype()), p->raw_data_ptr(), p_pitch, l->data_ptr<int64_t>(),
+                                      g->raw_data_ptr(), output->raw_data_ptr(), out_pitch, rows, cols,
+                                      ignored_index, hip_stream));
   }
   NDArray::MarkUsedBy({p, l, g, output}, stream);
 }

@@ -16,6 +16,49 @@ inline NDArray Dense(const NDArray& a, const Stream& stream) {
   return NDArray::contiguous(a, stream.stream_index());
 }
 
+// The [rows, cols] view the row kernels take: the last `inner_dims` dimensions hold `cols` consecutive elements
+// and the leading ones step by one constant pitch (a dense array, a slice x[..., a:b] of a wider one, a
+// row-padded buffer).  Sets the pitch in elements; false for any other layout (transposed, strided columns).
+inline bool RowPitch(const NDArray& a, int64_t inner_dims, int64_t* pitch) {
+  const int64_t nd = int64_t(a->ndim());
+  const int64_t split = nd - inner_dims;
+  int64_t expect = 1;
+  for (int64_t i = nd - 1; i >= split; --i) {
+    if (a->shape(i) != 1 && a->stride(i) != expect) return false;
+    expect *= a->shape(i);
+  }
+  const int64_t cols = expect;
+  *pitch = cols;
+  bool seen = false;
+  for (int64_t i = split - 1; i >= 0; --i) {
+    if (a->shape(i) == 1) continue;
+    if (!seen) {
+      *pitch = a->stride(i);
+      seen = true;
+    } else if (a->stride(i) != expect) {
+      return false;
+    }
+    expect = a->stride(i) * a->shape(i);
+  }
+  return *pitch >= cols;
+}
+
+// An input of a row kernel: the array itself when it is row-pitched (no copy is made), else a dense copy on
+// `stream`.  This is what stands in for the reference's per-element OffsetCalculator
+// (hetu/impl/utils/offset_calculator.cuh:16-68) on the operators that accept non-contiguous inputs.
+inline NDArray RowOperand(const NDArray& a, int64_t inner_dims, const Stream& stream, int64_t* pitch) {
+  if (a.is_defined() && RowPitch(a, inner_dims, pitch)) return a;
+  NDArray dense = Dense(a, stream);
+  if (dense.is_defined()) RowPitch(dense, inner_dims, pitch);
+  return dense;
+}
+
+// An output of a row kernel must be row-pitched; anything else has no 128-bit store pattern and is refused.
+#define HT_ASSERT_ROW_PITCHED(x, inner_dims, pitch_ptr)                                                   \
+  HT_ASSERT(::hetu::impl::RowPitch(x, inner_dims, pitch_ptr))                                              \
+    << "Output " << #x << " must be dense or a row-pitched view (unit-stride trailing dimensions, one "   \
+    << "constant row pitch). Shape: " << x->shape() << ". Strides: " << x->stride() << "."
+
 inline const void* PtrOrNull(const NDArray& a) {
   return a.is_defined() ? a->raw_data_ptr() : nullptr;
 }

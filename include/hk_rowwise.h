@@ -376,6 +376,15 @@ HK_API int hk_softmax_fwd(int dtype, const void* x, void* y, int64_t outer, int6
 HK_API int hk_softmax_bwd(int dtype, const void* y, const void* dy, void* dx, int64_t outer,
                           int64_t dim, int64_t inner, hkStream_t stream);
 
+/* Last-dimension softmax of [rows, cols] arrays whose rows lie a pitch (in elements, >= cols) apart: column
+ * slices of wider buffers, row-padded arrays.  A pitch that is a whole number of 16-byte vectors keeps the
+ * 128-bit kernels.  SoftmaxOp accepts non-contiguous inputs (hetu/graph/ops/Softmax.h:52-54) and the
+ * reference resolves them per element (hetu/impl/utils/offset_calculator.cuh:16-68). */
+HK_API int hk_softmax_fwd_pitched(int dtype, const void* x, int64_t x_pitch, void* y, int64_t y_pitch,
+                                  int64_t rows, int64_t cols, hkStream_t stream);
+HK_API int hk_softmax_bwd_pitched(int dtype, const void* y, int64_t y_pitch, const void* dy, int64_t dy_pitch,
+                                  void* dx, int64_t dx_pitch, int64_t rows, int64_t cols, hkStream_t stream);
+
 /* ======================================================================== *
  * Fused softmax cross-entropy, sparse int64 labels.
  * logits: [rows, cols]; labels: [rows] int64; loss: [rows] `dtype`.
@@ -394,6 +403,16 @@ HK_API int hk_sce_sparse_fwd(int dtype, const void* logits, const int64_t* label
 HK_API int hk_sce_sparse_bwd(int dtype, const void* logits, const int64_t* labels,
                              const void* grad_loss, void* dlogits, int64_t rows, int64_t cols,
                              int64_t ignored_index, hkStream_t stream);
+
+/* The two calls above on logits / dlogits whose rows lie a pitch (in elements, >= cols) apart, e.g. the
+ * un-padded columns of a vocabulary padded to a multiple of the tensor-parallel degree. */
+HK_API int hk_sce_sparse_fwd_pitched(int dtype, const void* logits, int64_t logits_pitch,
+                                     const int64_t* labels, void* loss, int64_t rows, int64_t cols,
+                                     int64_t ignored_index, hkStream_t stream);
+HK_API int hk_sce_sparse_bwd_pitched(int dtype, const void* logits, int64_t logits_pitch,
+                                     const int64_t* labels, const void* grad_loss, void* dlogits,
+                                     int64_t dlogits_pitch, int64_t rows, int64_t cols,
+                                     int64_t ignored_index, hkStream_t stream);
 
 /* The same with the gradient of a REDUCED loss: grad_output holds one value and every row uses
  * round_dtype(grad_output[0] * round_dtype(scale)) -- what BroadcastShapeMul(grad, 1/rows) into a [rows]

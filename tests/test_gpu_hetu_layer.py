@@ -352,7 +352,8 @@ def test_softmax_and_gradient(ops, cuda, dtype, shape, dim):
 
 
 def test_softmax_of_a_permuted_view(ops, cuda):
-    """Inputs of any stride are accepted (made dense inside); outputs must be dense."""
+    """Inputs of any stride are accepted (row-pitched ones as they are, others made dense inside); outputs must
+    be dense or row-pitched."""
     import torch
     x = helpers.draw(61, (12, 40, 24), "normal", 0.0, 2.0, "fp32")
     tx = helpers.to_torch(x, "fp32", cuda).permute(2, 0, 1)       # [24, 12, 40], not dense
@@ -362,10 +363,92 @@ def test_softmax_of_a_permuted_view(ops, cuda):
     ops.softmax(tx, ty, -1)
     ops.stream_sync()
     helpers.assert_close(ty, ey, "fp32", "y")
-    with pytest.raises(ops.AssertionError_, match="not contiguous"):
+    with pytest.raises(ops.AssertionError_, match="row-pitched"):
         ops.softmax(tx, torch.empty((12, 40, 24), device=cuda).permute(2, 0, 1), -1)
     with pytest.raises(ops.AssertionError_, match="Invalid dimension"):
         ops.softmax(tx, ty, 3)
+
+
+def test_row_pitched_views_reach_the_kernels_without_a_copy(ops, cuda):
+    """Column slices of wider arrays (3-D here: [batch, seq, hidden] cut along hidden) as inputs AND outputs of the
+    LayerNorm, Softmax and cross-entropy operators: results match the oracle, nothing outside the output slices is
+    written, and the pool hands out no block for a dense copy (its allocation count only moves by the backward's
+    scratch)."""
+    import torch
+    B, S, H, W, off = 3, 21, 512, 768, 128
+    dt = "bf16"
+    x = helpers.draw(81, (B, S, H), dtype=dt)
+    dy = helpers.draw(82, (B, S, H), dtype=dt)
+    g = helpers.draw(83, (H,), "uniform", 0.5, 1.5, dt)
+    b = helpers.draw(84, (H,), "normal", 0.0, 0.1, dt)
+    sent = 12288.0
+
+    def wide(values=None):
+        w = torch.full((B, S, W), sent, dtype=torch.bfloat16, device=cuda)
+        if values is not None:
+            w[:, :, off:off + H] = helpers.to_torch(values, dt, cuda)
+        return w, w[:, :, off:off + H]
+
+    def untouched(w):
+        keep = torch.ones(W, dtype=torch.bool, device=cuda)
+        keep[off:off + H] = False
+        return bool((w[:, :, keep].float() == sent).all())
+
+    _, sx = wide(x)
+    _, sdy = wide(dy)
+    wy, sy = wide()
+    tg, tb = helpers.to_torch(g, dt, cuda), helpers.to_torch(b, dt, cuda)
+    mean = torch.empty(B, S, 1, device=cuda)
+    rstd = torch.empty(B, S, 1, device=cuda)
+    _sync_in()
+    before = ops.pool_stats()
+    ops.fused_layer_norm(sx, tg, tb, mean, rstd, sy, 1, 1e-5)
+    wp, sp = wide()
+    ops.softmax(sx, sp, -1)
+    ops.stream_sync()
+    assert ops.pool_stats()["alloc_cnt"] == before["alloc_cnt"]          # no dense copy, no scratch
+    x2, g64, b64 = x.reshape(-1, H), g, b
+    ey, _, _, ers = oracle.layernorm_fwd(x2, g64, b64, 1e-5)
+    helpers.assert_close(sy, ey.reshape(B, S, H), dt, "y")
+    helpers.assert_close(rstd.reshape(-1), ers, "fp32", "rstd")
+    helpers.assert_close(sp, oracle.softmax_fwd(x2).reshape(B, S, H), dt, "softmax")
+    assert untouched(wy) and untouched(wp)
+    wdx, sdx = wide()
+    dg, db = torch.empty_like(tg), torch.empty_like(tb)
+    mid = ops.pool_stats()
+    ops.fused_layer_norm_gradient(sdy, sx, tg, tb, sdx, dg, db, mean, rstd, 1, 1e-5, False)
+    wsm, ssm = wide()
+    ops.softmax_gradient(sp, sdy, ssm, -1)
+    ops.stream_sync()
+    assert ops.pool_stats()["alloc_cnt"] - mid["alloc_cnt"] <= 1          # the backward's column-sum scratch only
+    edx, edg, edb = oracle.layernorm_bwd(dy.reshape(-1, H), x2, g, helpers.to_numpy(mean).reshape(-1),
+                                         helpers.to_numpy(rstd).reshape(-1), eps=1e-5, clamp_gamma=True)
+    helpers.assert_close(sdx, edx.reshape(B, S, H), dt, "dx")
+    helpers.assert_close(dg, edg, dt, "dgamma", scale=float(np.sqrt(B * S)))
+    helpers.assert_close(ssm, oracle.softmax_bwd(helpers.to_numpy(sp).reshape(-1, H), dy.reshape(-1, H)).reshape(B, S, H),
+                         dt, "softmax gradient")
+    assert untouched(wdx) and untouched(wsm)
+    # cross-entropy on logits padded along the class dimension, gradient written into a padded array
+    lab = helpers.rng(85).integers(0, H, (B, S)).astype(np.int64)
+    lab.reshape(-1)[::4] = -100
+    tl = torch.from_numpy(lab).to(cuda)
+    loss = torch.empty(B, S, dtype=torch.bfloat16, device=cuda)
+    gl = helpers.draw(86, (B, S), "uniform", 0.5, 1.5, dt)
+    wdl, sdl = wide()
+    mid = ops.pool_stats()
+    ops.softmax_cross_entropy_sparse(sx, tl, loss, -100)
+    ops.softmax_cross_entropy_sparse_gradient(sx, tl, helpers.to_torch(gl, dt, cuda), sdl, -100)
+    ops.stream_sync()
+    assert ops.pool_stats()["alloc_cnt"] == mid["alloc_cnt"]
+    helpers.assert_close(loss.reshape(-1), oracle.sce_sparse_fwd(x2, lab.reshape(-1), -100), dt, "loss")
+    edl = oracle.sce_sparse_bwd(x2, lab.reshape(-1), gl.reshape(-1), -100)
+    helpers.assert_close(sdl, edl.reshape(B, S, H), dt, "dlogits", scale=float(np.abs(edl).max()) * 1e-2)
+    assert untouched(wdl)
+    # a view that is not row-pitched (every other column) still works as an input, through a dense copy
+    half = torch.empty(B, S, H // 2, dtype=torch.bfloat16, device=cuda)
+    ops.softmax(sx[:, :, ::2], half, -1)
+    ops.stream_sync()
+    helpers.assert_close(half, oracle.softmax_fwd(x2[:, ::2]).reshape(B, S, H // 2), dt, "softmax of strided columns")
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])

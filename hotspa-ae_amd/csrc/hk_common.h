@@ -172,6 +172,26 @@ __device__ __forceinline__ void st16(void* p, const u32x4& v) {
 __device__ __forceinline__ void st16_stream(void* p, const u32x4& v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
+// Buffer addressing: a 128-bit resource descriptor (base address + byte count) held in scalar registers, plus a
+// per-lane byte offset.  The hardware checks every lane's offset against the byte count: a load past the end
+// returns zeros and a store past the end is dropped, so a kernel that walks a row in whole vectors needs no branch
+// around its memory instructions for a ragged last step.  One descriptor addresses at most 4 GiB.
+typedef __amdgpu_buffer_rsrc_t BufferRsrc;
+constexpr int kBufKeep = 0;     // default cache policy (reused data: gamma, beta)
+constexpr int kBufStream = 2;   // "nt": data touched once (rows in, rows out)
+__device__ __forceinline__ BufferRsrc make_rsrc(const void* base, uint32_t bytes) {
+  // word 3 = 0x00020000: raw buffer, 32-bit data format, no swizzle (the gfx9 / CDNA encoding)
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, int(bytes), 0x00020000);
+}
+template <int POLICY>
+__device__ __forceinline__ u32x4 buf_ld16(BufferRsrc r, uint32_t byte_offset) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, int(byte_offset), 0, POLICY);
+}
+template <int POLICY>
+__device__ __forceinline__ void buf_st16(BufferRsrc r, uint32_t byte_offset, const u32x4& v) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, int(byte_offset), 0, POLICY);
+}
+
 __device__ __forceinline__ u32x4 ld16_stream(const void* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }

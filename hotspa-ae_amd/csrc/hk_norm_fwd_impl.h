@@ -12,6 +12,10 @@ namespace hk {
 // T: element type; NV: 16-byte vectors per thread; WAVE_ROW: one wavefront per
 // row (4 rows per 256-thread block) instead of one workgroup per row;
 // HAS_RES: x = x0 + residual is formed in fp32 and optionally written back.
+//
+// Every row operand is addressed through a buffer descriptor of exactly one row (base = the row's first byte,
+// size = cols * sizeof(T)): the hardware returns zeros for a lane past the row's end and drops its stores, so no
+// memory instruction sits inside a branch and all of a thread's loads are issued back to back.
 template <typename T, int NV, bool WAVE_ROW, bool HAS_RES>
 __global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
 void norm_fwd_kernel(NormFwdArgs a) {
@@ -25,35 +29,44 @@ void norm_fwd_kernel(NormFwdArgs a) {
       : int64_t(blockIdx.x);
   if (WAVE_ROW && row >= a.rows) return;  // wave-uniform; no block barrier in this mode
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
+  const uint32_t row_bytes = uint32_t(a.nvec) * 16u;
+  auto off = [&](int i) { return uint32_t(i * tpr + t) * 16u; };   // vector i of thread t, in bytes from the row's start
 
-  const T* xr = static_cast<const T*>(a.x) + row * a.x_pitch;
+  const BufferRsrc xr = make_rsrc(static_cast<const T*>(a.x) + row * a.x_pitch, row_bytes);
   u32x4 raw[NV];
 #pragma unroll
-  for (int i = 0; i < NV; ++i) raw[i] = u32x4{0, 0, 0, 0};
+  for (int i = 0; i < NV; ++i) raw[i] = buf_ld16<kBufStream>(xr, off(i));
   [[maybe_unused]] float xf[HAS_RES ? NV * VEC : 1];
-
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int v = i * tpr + t;
-    if (v < a.nvec) raw[i] = ld16(xr + v * VEC);
-  }
   if constexpr (HAS_RES) {
-    const T* rr = static_cast<const T*>(a.residual) + row * a.res_pitch;
-    T* xo = a.x_out ? static_cast<T*>(a.x_out) + row * a.xout_pitch : nullptr;
+    const BufferRsrc rr = make_rsrc(static_cast<const T*>(a.residual) + row * a.res_pitch, row_bytes);
+    u32x4 res[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) res[i] = buf_ld16<kBufStream>(rr, off(i));
+    // an absent x_out becomes an empty buffer: its stores are dropped by the bounds check
+    const BufferRsrc xo = make_rsrc(a.x_out ? static_cast<T*>(a.x_out) + row * a.xout_pitch : static_cast<T*>(a.y),
+                                    a.x_out ? row_bytes : 0u);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int v = i * tpr + t;
-      if (v < a.nvec) {
-        float f0[VEC], f1[VEC];
-        VecIO<T>::unpack(raw[i], f0);
-        VecIO<T>::unpack(ld16(rr + v * VEC), f1);
+      float f0[VEC], f1[VEC];
+      VecIO<T>::unpack(raw[i], f0);
+      VecIO<T>::unpack(res[i], f1);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) xf[i * VEC + j] = f0[j] + f1[j];
-        if (xo) st16(xo + v * VEC, VecIO<T>::pack(&xf[i * VEC]));
-      }
+      for (int j = 0; j < VEC; ++j) xf[i * VEC + j] = f0[j] + f1[j];
+      buf_st16<kBufStream>(xo, off(i), VecIO<T>::pack(&xf[i * VEC]));
     }
   }
 
+  // The row stays packed between the passes over it (4 registers per vector, not one per element): the empty
+  // statement makes the packed words opaque, so the next pass unpacks them again instead of keeping the floats
+  // of the previous one alive.
+  auto repack = [&]() {
+    if constexpr (!HAS_RES && VEC > 4) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) asm volatile("" : "+v"(raw[i]));
+    }
+  };
+  // long rows: stops the scheduler from unpacking every vector of a pass before the first one is consumed
+  auto fence = [] { if constexpr (NV >= 8) __builtin_amdgcn_sched_barrier(0); };
   auto get = [&](int i, float* f) {
     if constexpr (HAS_RES) {
 #pragma unroll
@@ -65,16 +78,16 @@ void norm_fwd_kernel(NormFwdArgs a) {
 
   float mu, rs, var;
   if (a.is_rms) {
+    // lanes past the row's end hold zeros, which add nothing to either sum
     SumTuple<2> s;
     s.v[0] = 0.f; s.v[1] = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      if (i * tpr + t < a.nvec) {
-        float f[VEC];
-        get(i, f);
+      float f[VEC];
+      fence();
+      get(i, f);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) { s.v[0] += f[j]; s.v[1] = fmaf(f[j], f[j], s.v[1]); }
-      }
+      for (int j = 0; j < VEC; ++j) { s.v[0] += f[j]; s.v[1] = fmaf(f[j], f[j], s.v[1]); }
     }
     s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red, 0, nwaves);
     mu = s.v[0] * a.inv_cols;
@@ -90,25 +103,26 @@ void norm_fwd_kernel(NormFwdArgs a) {
     int cnt = 0;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      if (i * tpr + t < a.nvec) {
-        float f[VEC];
-        get(i, f);
+      float f[VEC];
+      fence();
+      get(i, f);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) s += f[j];
-        cnt += VEC;
-      }
+      for (int j = 0; j < VEC; ++j) s += f[j];            // zeros past the end
+      cnt += (i * tpr + t < a.nvec) ? VEC : 0;
     }
+    repack();
     const bool even = a.nvec == NV * tpr;                    // uniform
     const float mean_t = even ? s * (1.0f / float(NV * VEC)) : (cnt > 0 ? s / float(cnt) : 0.f);
     float m2 = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      if (i * tpr + t < a.nvec) {
-        float f[VEC];
-        get(i, f);
+      float f[VEC];
+      fence();
+      get(i, f);
+      float q = 0.f;
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) { const float d = f[j] - mean_t; m2 = fmaf(d, d, m2); }
-      }
+      for (int j = 0; j < VEC; ++j) { const float d = f[j] - mean_t; q = fmaf(d, d, q); }
+      m2 += (even || i * tpr + t < a.nvec) ? q : 0.f;
     }
     MomentTuple m;
     m.v[0] = float(cnt); m.v[1] = mean_t; m.v[2] = m2;
@@ -132,51 +146,39 @@ void norm_fwd_kernel(NormFwdArgs a) {
     store_stat<T>(a.stat, row, a.stat_kind == HK_STAT_VAR ? var : rs, a.stats_f32);
   }
 
+  repack();
   const float shift = a.is_rms ? 0.f : mu;
-  T* yr = static_cast<T*>(a.y) + row * a.y_pitch;
-  // gamma / beta are fetched here, after the reduction, and one vector ahead of the arithmetic: holding all of
-  // them in registers (across the reduction, or merely across this loop) costs resident waves, which is what
-  // hides the row's own load latency.  The scheduling fences keep the compiler from hoisting every fetch to the
-  // top of the unrolled loop again.  The four cases of missing parameters are separate straight-line copies, so
-  // that no fetch sits inside a branch.
-  const T* gp = static_cast<const T*>(a.gamma);
-  const T* bp = static_cast<const T*>(a.beta);
+  const BufferRsrc yr = make_rsrc(static_cast<T*>(a.y) + row * a.y_pitch, row_bytes);
+  // gamma / beta are fetched after the reduction: every fetch is a miss in the compute unit's own cache (the
+  // rows stream through it) and holds one of its outstanding-request slots until the data is back; issued
+  // before the row has arrived they would hold those slots for the whole HBM latency instead of the L2's.
+  // The four cases of missing parameters are separate straight-line copies, so that no fetch sits inside a
+  // branch; the compiler is free to issue all of a thread's fetches together.
   auto epilogue = [&](auto has_g, auto has_b) {
     constexpr bool HG = decltype(has_g)::value, HB = decltype(has_b)::value;
-    [[maybe_unused]] u32x4 gn, bn;
-    auto fetch = [&](int i) {
-      int v = i * tpr + t;
-      v = v < a.nvec ? v : 0;                 // a lane past the row's end reads the first vector; never used
-      if constexpr (HG) gn = ld16_keep(gp + v * VEC);
-      if constexpr (HB) bn = ld16_keep(bp + v * VEC);
-    };
-    fetch(0);
-    static_for<NV>([&](auto idx) {
-      constexpr int i = decltype(idx)::value;
-      [[maybe_unused]] const u32x4 gc = gn, bc = bn;
-      if constexpr (i + 1 < NV) fetch(i + 1);
-      __builtin_amdgcn_sched_barrier(0);
-      const int v = i * tpr + t;
-      if (v < a.nvec) {
-        float f[VEC], g[VEC], b[VEC];
-        get(i, f);
-        if constexpr (HG) VecIO<T>::unpack(gc, g);
-        if constexpr (HB) VecIO<T>::unpack(bc, b);
+    const BufferRsrc gr = make_rsrc(HG ? a.gamma : a.y, row_bytes);   // an absent parameter is not fetched at all
+    const BufferRsrc br = make_rsrc(HB ? a.beta : a.y, row_bytes);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const float n = rs * (f[j] - shift);
-          f[j] = HG ? (HB ? fmaf(g[j], n, b[j]) : g[j] * n) : (HB ? n + b[j] : n);
-        }
-        const u32x4 o = VecIO<T>::pack(f);
-        if (a.stream_store) st16_stream(yr + v * VEC, o);
-        else st16(yr + v * VEC, o);
+    for (int i = 0; i < NV; ++i) {
+      float f[VEC];
+      [[maybe_unused]] float g[VEC], b[VEC];
+      get(i, f);
+      if constexpr (HG) VecIO<T>::unpack(buf_ld16<kBufKeep>(gr, off(i)), g);
+      if constexpr (HB) VecIO<T>::unpack(buf_ld16<kBufKeep>(br, off(i)), b);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float n = rs * (f[j] - shift);
+        f[j] = HG ? (HB ? fmaf(g[j], n, b[j]) : g[j] * n) : (HB ? n + b[j] : n);
       }
-      __builtin_amdgcn_sched_barrier(0);
-    });
+      buf_st16<kBufStream>(yr, off(i), VecIO<T>::pack(f));
+      // long rows: keep the compiler from hoisting every parameter fetch above the first store, which would
+      // hold 2 * NV more vectors in registers than the row itself
+      if constexpr (NV >= 8) __builtin_amdgcn_sched_barrier(0);
+    }
   };
-  if (gp && bp) epilogue(std::true_type{}, std::true_type{});
-  else if (gp) epilogue(std::true_type{}, std::false_type{});
-  else if (bp) epilogue(std::false_type{}, std::true_type{});
+  if (a.gamma && a.beta) epilogue(std::true_type{}, std::true_type{});
+  else if (a.gamma) epilogue(std::true_type{}, std::false_type{});
+  else if (a.beta) epilogue(std::false_type{}, std::true_type{});
   else epilogue(std::false_type{}, std::false_type{});
 }
 
@@ -256,7 +258,13 @@ static int launch_norm_fwd_nv(const NormFwdArgs& a, int nv, dim3 grid, dim3 bloc
     case 5: hipLaunchKernelGGL((norm_fwd_kernel<T, 5, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
     case 6: hipLaunchKernelGGL((norm_fwd_kernel<T, 6, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
     case 8: hipLaunchKernelGGL((norm_fwd_kernel<T, 8, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
-    case 16: hipLaunchKernelGGL((norm_fwd_kernel<T, 16, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 16:
+      // only the fp32 row without a residual fits sixteen vectors into a 1024-thread workgroup's registers
+      if constexpr (sizeof(T) == 4 && !HAS_RES && !WAVE_ROW) {
+        hipLaunchKernelGGL((norm_fwd_kernel<T, 16, WAVE_ROW, HAS_RES>), grid, block, 0, s, a);
+        break;
+      }
+      [[fallthrough]];
     default:
       set_last_error("norm_fwd: no kernel for %d vectors per thread", nv);
       return HK_ERR_UNSUPPORTED;
@@ -288,11 +296,13 @@ static bool pick_row_shape(int nvec, int forced_threads, int max_nv, int wave_ro
   // First choice: the fewest vectors per thread that fill every lane exactly
   // (5120 bf16 columns = 640 vectors = 128 threads x 5): no idle lanes, and the
   // statistics merge takes its equal-count form.
+  // A 512-thread workgroup (two wavefronts on each of the four SIMDs) is as good when it gets by with two vectors
+  // (4096 fp32 columns: 46 us against 49 us for 256 x 4); widths that load the SIMDs unevenly (320, 384) are not.
   static const int kCounts[] = {2, 3, 4, 5, 6, 8};
   for (int n : kCounts) {
     if (n > max_nv) break;
     int t = ((nvec + n - 1) / n + 63) / 64 * 64;
-    if (t <= 256 && n * t == nvec) {
+    if ((t <= 256 || (t == 512 && n == 2)) && n * t == nvec) {
       *threads = t;
       *nv = n;
       return true;
@@ -330,8 +340,9 @@ int norm_fwd_typed(NormFwdArgs a, hipStream_t s) {
   int threads = 0, nv = 0;
   a.nvec = a.cols / VEC;
   const bool has_res = a.residual != nullptr;
-  // with a residual the summed row is kept unpacked: halve the budget
-  const int max_nv = has_res ? (VEC == 4 ? 16 : 8) : 16;
+  // with a residual the summed row is kept unpacked: halve the budget; sixteen vectors of a 16-bit type (one
+  // 1024-thread workgroup on more than 65536 columns) do not fit the 128 registers such a workgroup leaves a thread
+  const int max_nv = has_res ? 8 : (VEC == 4 ? 16 : 8);
   const int wave_nv = has_res ? (VEC == 4 ? 8 : 4) : (VEC == 4 ? 16 : 8);
   if (vec_ok && pick_row_shape(a.nvec, tune_get(TUNE_NORM_FWD_THREADS), max_nv, wave_nv, &threads, &nv)) {
     if (threads == 64) {

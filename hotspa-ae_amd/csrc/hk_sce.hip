@@ -140,8 +140,16 @@ void sce_sparse_fwd_kernel(SceArgs a) {
 }
 
 // ------------------------------- sparse backward ---------------------------
+// A 1024-thread workgroup is four wavefronts on every SIMD: two such workgroups fit a compute unit only at the
+// full eight wavefronts per SIMD, i.e. at 64 registers or fewer.  The second launch bound asks the compiler for
+// that; without it the kernel came out at 68 registers and ran with one workgroup per compute unit (448 us
+// instead of 345 us at 16384 x 32000 bf16).  Eight fp32 vectors per thread do not fit 64 registers and keep the
+// looser bound.
+template <typename T, int NV>
+constexpr int sce_min_waves(bool wave_row) { return wave_row ? 1 : (sizeof(T) == 4 && NV == 8 ? 4 : 8); }
+
 template <typename T, int NV, bool WAVE_ROW>
-__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
+__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024, (sce_min_waves<T, NV>(WAVE_ROW)))
 void sce_sparse_bwd_kernel(SceArgs a) {
   constexpr int VEC = VecIO<T>::N;
   __shared__ float red[kMaxWaves * 2];
@@ -219,7 +227,7 @@ void sce_sparse_bwd_kernel(SceArgs a) {
 // ------------------------------- dense labels ------------------------------
 // loss = (M + log S) * sum(l) - sum(l * x);  dx = (softmax - l) * g
 template <typename T, int NV, bool WAVE_ROW, bool BWD>
-__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
+__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024, (sce_min_waves<T, NV>(WAVE_ROW)))
 void sce_dense_kernel(SceArgs a) {
   constexpr int VEC = VecIO<T>::N;
   __shared__ float red[kMaxWaves * 3];

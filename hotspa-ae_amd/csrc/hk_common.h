@@ -479,7 +479,6 @@ enum TuneKey {
   TUNE_SCE_THREADS,
   TUNE_REDUCE_INNER_THREADS,
   TUNE_REDUCE_OUTER_ROW_BLOCKS,
-  TUNE_STREAM_STORES,
   TUNE_NORM_BWD_ROWS_PER_BLOCK,
   TUNE_NORM_BWD_PREFETCH,
   TUNE_NUM_KEYS

@@ -50,7 +50,6 @@ static const char* const kTuneNames[] = {
   "sce_threads",
   "reduce_inner_threads",
   "reduce_outer_row_blocks",
-  "stream_stores",      // 1: non-temporal stores for write-once outputs, 2: plain stores
   "norm_bwd_rows_per_block",
   "norm_bwd_prefetch",  // rows loaded ahead by the backward kernel (1..3)
 };

@@ -99,9 +99,11 @@ __device__ __forceinline__ void load8_keep(const T* p, float* f) {
   VecIO<T>::unpack(ld16_keep(p), f);
   if constexpr (VecIO<T>::N == 4) VecIO<T>::unpack(ld16_keep(p + 4), f + 4);
 }
-template <typename T>
-__device__ __forceinline__ void store8(T* p, const float* f, bool stream) {
-  if (stream) {
+// STREAM is a template argument on purpose: with the choice as a run-time flag the compiler merges the two
+// branches into one plain store and the non-temporal hint is lost.
+template <typename T, bool STREAM>
+__device__ __forceinline__ void store8(T* p, const float* f) {
+  if constexpr (STREAM) {
     st16_stream(p, VecIO<T>::pack(f));
     if constexpr (VecIO<T>::N == 4) st16_stream(p + 4, VecIO<T>::pack(f + 4));
   } else {
@@ -143,7 +145,7 @@ struct DalFwdArgs {
   int64_t rows, x0_numrows, z_numrows;
   int cols, nchunks, tpr;
   float eps, inv_cols, scale, rowscale_const;
-  int is_rms, dropout, stream_store;
+  int is_rms, dropout;
   DropArgs drop;
 };
 
@@ -274,7 +276,7 @@ void dal_fwd_kernel(DalFwdArgs a) {
 #pragma unroll
         for (int j = 0; j < kChunk; ++j) v[j] += w[j];
       }
-      if (a.x && row_ok) store8<RT>(static_cast<RT*>(a.x) + e, v, false);
+      if (a.x && row_ok) store8<RT, false>(static_cast<RT*>(a.x) + e, v);
     }
   }
 
@@ -328,7 +330,7 @@ void dal_fwd_kernel(DalFwdArgs a) {
       if (a.beta) load8_keep<WT>(static_cast<const WT*>(a.beta) + col, b);
 #pragma unroll
       for (int j = 0; j < kChunk; ++j) o[j] = fmaf(g[j], y[j], b[j]);
-      store8<IT>(static_cast<IT*>(a.z) + zbase + col, o, a.stream_store != 0);
+      store8<IT, true>(static_cast<IT*>(a.z) + zbase + col, o);
       if (a.gamma1) {
 #pragma unroll
         for (int j = 0; j < kChunk; ++j) b[j] = 0.f;
@@ -336,7 +338,7 @@ void dal_fwd_kernel(DalFwdArgs a) {
         if (a.beta1) load8_keep<WT>(static_cast<const WT*>(a.beta1) + col, b);
 #pragma unroll
         for (int j = 0; j < kChunk; ++j) o[j] = fmaf(g[j], y[j], b[j]);
-        store8<IT>(static_cast<IT*>(a.z1) + zbase + col, o, a.stream_store != 0);
+        store8<IT, true>(static_cast<IT*>(a.z1) + zbase + col, o);
       }
     }
   }
@@ -370,7 +372,7 @@ struct DalBwdArgs {
   int64_t rows, x0_numrows, z_numrows;
   int cols, nchunks, tpr;
   float inv_cols, scale, rowscale_const;
-  int is_rms, dropout, stream_store;
+  int is_rms, dropout;
 };
 
 // One chunk of 8 columns per thread.  COLSCALE: per-column scaling (and its gradient); G1: a second
@@ -474,7 +476,7 @@ void dal_bwd_kernel(DalBwdArgs a) {
 #pragma unroll
       for (int j = 0; j < kChunk; ++j) dxr[j] += u[j];
     }
-    if (a.dresidual) store8<RT>(static_cast<RT*>(a.dresidual) + e, dxr, false);
+    if (a.dresidual) store8<RT, false>(static_cast<RT*>(a.dresidual) + e, dxr);
     if (save_dx0) {
       const int64_t e0 = (row_x0 - 1) * int64_t(a.cols) + col;
       uint32_t keep = 0xffu;
@@ -498,7 +500,7 @@ void dal_bwd_kernel(DalBwdArgs a) {
       }
 #pragma unroll
       for (int j = 0; j < kChunk; ++j) o[j] = ((keep >> j) & 1u) ? o[j] : 0.f;
-      store8<IT>(static_cast<IT*>(a.dx0) + e0, o, a.stream_store != 0);
+      store8<IT, true>(static_cast<IT*>(a.dx0) + e0, o);
     }
     if (a.dx1) {
       float o[kChunk];
@@ -509,7 +511,7 @@ void dal_bwd_kernel(DalBwdArgs a) {
         const float v = dropout ? dxr[j] * a.scale : dxr[j];
         o[j] = ((keep >> j) & 1u) ? v : 0.f;
       }
-      store8<IT>(static_cast<IT*>(a.dx1) + e, o, a.stream_store != 0);
+      store8<IT, true>(static_cast<IT*>(a.dx1) + e, o);
     }
   }
 
@@ -620,8 +622,8 @@ void dal_bwd_stream_kernel(DalBwdArgs a) {
         o[j] = byte ? u[j] * a.scale : 0.f;
       }
       const int64_t e = row * int64_t(a.cols) + col;
-      store8<RT>(static_cast<RT*>(a.dresidual) + e, u, false);
-      store8<IT>(static_cast<IT*>(a.dx0) + e, o, true);
+      store8<RT, false>(static_cast<RT*>(a.dresidual) + e, u);
+      store8<IT, true>(static_cast<IT*>(a.dx0) + e, o);
     }
   };
   int64_t base = int64_t(blockIdx.x) * rpb;
@@ -813,7 +815,6 @@ int hk_dropout_add_ln_fwd_ex(const hkDropoutAddLnFwdParams* pp, hkStream_t strea
   a.eps = p.epsilon; a.inv_cols = 1.0f / float(p.cols);
   a.scale = 1.0f / (1.0f - p.dropout_p); a.rowscale_const = p.rowscale_const;
   a.is_rms = p.is_rms_norm ? 1 : 0; a.dropout = dropout ? 1 : 0;
-  a.stream_store = tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1;
   a.drop.seed_lo = uint32_t(p.seed); a.drop.seed_hi = uint32_t(p.seed >> 32);
   a.drop.off_lo = uint32_t(p.offset); a.drop.off_hi = uint32_t(p.offset >> 32);
   a.drop.keep_p = 1.0f - p.dropout_p;
@@ -945,7 +946,6 @@ int hk_dropout_add_ln_bwd_ex(const hkDropoutAddLnBwdParams* pp, hkStream_t strea
   a.cols = int(p.cols); a.nchunks = int(p.cols) / kChunk; a.tpr = sh.tpr;
   a.inv_cols = 1.0f / float(p.cols); a.scale = 1.0f / (1.0f - p.dropout_p); a.rowscale_const = p.rowscale_const;
   a.is_rms = p.is_rms_norm ? 1 : 0; a.dropout = dropout ? 1 : 0;
-  a.stream_store = tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1;
 
   DalFoldArgs f{};
   for (int k = 0; k < kMaxParts; ++k) { f.part[k] = a.part[k]; f.out[k] = outs[k]; }

@@ -31,7 +31,6 @@ struct NormFwdArgs {
   int is_rms;
   int stat_kind;
   int stats_f32;
-  int stream_store;
 };
 
 enum NormBwdMode { BWD_LN = 0, BWD_RMS = 1, BWD_LN_MEMEFF = 2 };
@@ -58,7 +57,6 @@ struct NormBwdArgs {
   int stat_kind;
   int stats_f32;
   int clamp_gamma;
-  int stream_store;
 };
 
 struct BwdPlan {

@@ -16,8 +16,6 @@ static int norm_fwd_dispatch(int dtype, NormFwdArgs& a, hipStream_t s, const cha
              (!a.x_out || a.xout_pitch >= a.cols), HK_ERR_INVALID,
              "%s: a row pitch is smaller than the %d columns of a row", who, a.cols);
   a.inv_cols = 1.0f / float(a.cols);
-  const int st = tune_get(TUNE_STREAM_STORES);
-  a.stream_store = (st == 2) ? 0 : 1;
   switch (dtype) {
     case HK_FLOAT32: return norm_fwd_typed<float>(a, s);
     case HK_BFLOAT16: return norm_fwd_typed<bf16>(a, s);
@@ -41,7 +39,6 @@ static int norm_bwd_dispatch(int dtype, NormBwdArgs& a, int mode, void* dgamma, 
              (!a.dx_in || a.dxin_pitch >= a.cols) && (!a.dres || a.dres_pitch >= a.cols), HK_ERR_INVALID,
              "%s: a row pitch is smaller than the %d columns of a row", who, a.cols);
   a.inv_cols = 1.0f / float(a.cols);
-  a.stream_store = tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1;
   switch (dtype) {
     case HK_FLOAT32: return norm_bwd_typed<float>(a, mode, dgamma, dbeta, ws, ws_bytes, s);
     case HK_BFLOAT16: return norm_bwd_typed<bf16>(a, mode, dgamma, dbeta, ws, ws_bytes, s);

@@ -212,8 +212,7 @@ void norm_bwd_kernel(NormBwdArgs a) {
             }
           }
           const u32x4 pk = VecIO<T>::pack(o);
-          if (a.stream_store) st16_stream(dxr + v * VEC, pk);
-          else st16(dxr + v * VEC, pk);
+          st16_stream(dxr + v * VEC, pk);
           if constexpr (EXTRA) {
             if (drr) st16(drr + v * VEC, pk);
           }

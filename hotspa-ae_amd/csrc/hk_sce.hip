@@ -29,7 +29,6 @@ struct SceArgs {
   int cols;
   int nvec;
   int64_t ignored_index;
-  int stream_store;
   // sparse forward on a column shard [vocab_start, vocab_start + cols) of a wider row: instead of a loss,
   // stats[0..rows) = the shard's row maximum, stats[rows..2 rows) = sum of exp(x - that maximum),
   // stats[2 rows..3 rows) = the logit at the label when the label falls into the shard, else 0
@@ -166,8 +165,7 @@ void sce_sparse_bwd_kernel(SceArgs a) {
     for (int i = 0; i < NV; ++i) {
       const int v = i * tpr + t;
       if (v < a.nvec) {
-        if (a.stream_store) st16_stream(dxr + v * VEC, z);
-        else st16(dxr + v * VEC, z);
+        st16_stream(dxr + v * VEC, z);
       }
     }
     return;
@@ -218,8 +216,7 @@ void sce_sparse_bwd_kernel(SceArgs a) {
           if (j == lsub) e[i * VEC + j] -= g;
       }
       const u32x4 o = VecIO<T>::pack(&e[i * VEC]);
-      if (a.stream_store) st16_stream(dxr + v * VEC, o);
-      else st16(dxr + v * VEC, o);
+      st16_stream(dxr + v * VEC, o);
     }
   }
 }
@@ -301,8 +298,7 @@ void sce_dense_kernel(SceArgs a) {
         for (int j = 0; j < VEC; ++j)
           f[j] = (__builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, -ML)) * inv - l[j]) * g;
         const u32x4 o = VecIO<T>::pack(f);
-        if (a.stream_store) st16_stream(dxr + v * VEC, o);
-        else st16(dxr + v * VEC, o);
+        st16_stream(dxr + v * VEC, o);
       }
     }
   }
@@ -513,7 +509,6 @@ static int sce_dispatch(int dtype, SceArgs& a, hipStream_t s, const char* who) {
   if (a.out_pitch == 0) a.out_pitch = a.cols;
   HK_REQUIRE(a.x_pitch >= a.cols && a.lab_pitch >= a.cols && a.out_pitch >= a.cols, HK_ERR_INVALID,
              "%s: a row pitch is smaller than the %d columns of a row", who, a.cols);
-  a.stream_store = tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1;
   switch (dtype) {
     case HK_FLOAT32: return sce_typed<float, MODE>(a, s);
     case HK_BFLOAT16: return sce_typed<bf16, MODE>(a, s);

@@ -22,7 +22,6 @@ struct SoftmaxArgs {
   int64_t x_pitch, dy_pitch, out_pitch;   // elements between row starts (== cols for a dense array)
   int cols;
   int nvec;
-  int stream_store;
 };
 
 template <typename T, int NV, bool WAVE_ROW>
@@ -80,8 +79,7 @@ void softmax_fwd_kernel(SoftmaxArgs a) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) e[i * VEC + j] *= scale;
       const u32x4 o = VecIO<T>::pack(&e[i * VEC]);
-      if (a.stream_store) st16_stream(yr + v * VEC, o);
-      else st16(yr + v * VEC, o);
+      st16_stream(yr + v * VEC, o);
     }
   }
 }
@@ -132,8 +130,7 @@ void softmax_bwd_kernel(SoftmaxArgs a) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) d[j] = y[j] * (d[j] - dot);
       const u32x4 o = VecIO<T>::pack(d);
-      if (a.stream_store) st16_stream(dxr + v * VEC, o);
-      else st16(dxr + v * VEC, o);
+      st16_stream(dxr + v * VEC, o);
     }
   }
 }
@@ -378,7 +375,6 @@ static int softmax_dispatch(int dtype, const void* x, const void* dy, void* out,
     SoftmaxArgs a{};
     a.x = x; a.dy = dy; a.out = out; a.rows = outer; a.cols = int(dim);
     a.x_pitch = x_pitch; a.dy_pitch = dy_pitch; a.out_pitch = out_pitch;
-    a.stream_store = tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1;
     switch (dtype) {
       case HK_FLOAT32: return softmax_lastdim_typed<float, BWD>(a, s);
       case HK_BFLOAT16: return softmax_lastdim_typed<bf16, BWD>(a, s);

@@ -103,7 +103,7 @@ template <typename T>
 __global__ __launch_bounds__(256)
 void vocab_ce_bwd_fused_kernel(const T* x, const int64_t* __restrict__ labels, const float* __restrict__ lse,
                                const T* __restrict__ grad_loss, T* out, uint32_t nvec, uint32_t cols_vec,
-                               int64_t vocab_start, int64_t ignored_index, int stream_store) {
+                               int64_t vocab_start, int64_t ignored_index) {
   constexpr int VEC = VecIO<T>::N;
   constexpr float kLog2e = 1.4426950408889634f;
   const uint32_t v = blockIdx.x * 256u + threadIdx.x;
@@ -140,8 +140,7 @@ void vocab_ce_bwd_fused_kernel(const T* x, const int64_t* __restrict__ labels, c
     const float o = (uint32_t(j) == hit) ? fmaf(p, g, -g) : p * g;
     f[j] = ignored ? 0.f : o;              // also when exp overflowed to inf or the logit was NaN
   }
-  if (stream_store) st16_stream(out + size_t(v) * VEC, VecIO<T>::pack(f));
-  else st16(out + size_t(v) * VEC, VecIO<T>::pack(f));
+  st16_stream(out + size_t(v) * VEC, VecIO<T>::pack(f));
 }
 
 template <typename T, typename CT>
@@ -175,8 +174,7 @@ static int vocab_bwd_fused_typed(const void* x, const int64_t* labels, const flo
       profile_before(s);
       hipLaunchKernelGGL((vocab_ce_bwd_fused_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
                          static_cast<const T*>(x), labels, lse, static_cast<const T*>(grad_loss), static_cast<T*>(out),
-                         nvec, uint32_t(cols / VEC), vocab_start, ignored_index,
-                         tune_get(TUNE_STREAM_STORES) == 2 ? 0 : 1);
+                         nvec, uint32_t(cols / VEC), vocab_start, ignored_index);
       profile_after(s);
       return launch_check("vocab_ce_bwd_fused_kernel");
     }

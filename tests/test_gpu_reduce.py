@@ -202,3 +202,50 @@ def test_prod_parity_and_widened_output(hk, cuda, dtype):
     # max / min have no widened output
     with pytest.raises(hk.HkError):
         _run(hk, cuda, helpers.to_torch(xi, "bf16", cuda), (1,), "max", out_dtype=torch.float32)
+
+
+def test_split_column_reduction_on_many_streams(hk, cuda):
+    """A column reduction whose rows are split over workgroups gives the same bits eagerly and as a graph replay, on
+    every one of 40 streams whose calls overlap, call after call, with calls of other shapes in between."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(77)
+    shapes = [(4096, 4096), (2048, 512), (3000, 1032), (4, 1024, 2048)]
+    xs = [torch.randn(*s, generator=g, device=cuda).to(torch.bfloat16) for s in shapes]
+    axes = [[0], [0], [0], [1]]
+    # reference: a graph replay
+    want = []
+    for x, ax in zip(xs, axes):
+        kept = [d for i, d in enumerate(x.shape) if i not in ax]
+        out = torch.empty(kept, dtype=torch.bfloat16, device=cuda)
+        ws = torch.empty(max(1, hk.reduce_workspace_bytes(8, list(x.shape), list(x.stride()), ax) // 4 + 4), device=cuda)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            hk.reduce(x, out, ax, "sum", workspace=ws)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            hk.reduce(x, out, ax, "sum", workspace=ws)
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        want.append(out.clone())
+        # against float64 sums as well
+        ref = x.double().sum(dim=ax[0])
+        assert float(((out.double() - ref).abs() / (ref.abs() + ref.abs().mean())).max()) < 1e-2
+    streams = [torch.cuda.Stream() for _ in range(40)]
+    outs = [[torch.empty_like(w) for w in want] for _ in streams]
+    wss = [[torch.empty(max(1, hk.reduce_workspace_bytes(8, list(x.shape), list(x.stride()), ax) // 4 + 4), device=cuda)
+            for x, ax in zip(xs, axes)] for _ in streams]
+    for rep in range(3):
+        for si, st in enumerate(streams):
+            st.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(st):
+                for k, (x, ax) in enumerate(zip(xs, axes)):
+                    outs[si][k].fill_(float("nan"))
+                    hk.reduce(x, outs[si][k], ax, "sum", workspace=wss[si][k])
+        torch.cuda.synchronize()
+        for si in range(len(streams)):
+            for k in range(len(xs)):
+                assert torch.equal(outs[si][k].view(torch.int16), want[k].view(torch.int16)), (rep, si, k)

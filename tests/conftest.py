@@ -34,3 +34,17 @@ def cuda():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda:0")
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The strictly element-relative error of every comparison against the oracle, worst case per test file and
+    quantity (helpers.assert_close)."""
+    import helpers
+    if not helpers.STRICT_LOG:
+        return
+    tr = terminalreporter
+    tr.section("strict relative error |a - e| / |e| over elements with |e| >= %.0e rms(e)" % helpers.STRICT_FLOOR)
+    tr.write_line("%-34s %-22s %-5s %11s %9s %11s %6s" % ("test file", "quantity", "dtype", "strict", "bound",
+                                                          "gate", "calls"))
+    for (f, what, dt), (strict, bound, gate, n) in sorted(helpers.STRICT_LOG.items()):
+        tr.write_line("%-34s %-22s %-5s %11.3e %9.1e %11.3e %6d" % (f, what[:22], dt, strict, bound, gate, n))

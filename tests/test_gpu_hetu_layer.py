@@ -442,7 +442,7 @@ def test_row_pitched_views_reach_the_kernels_without_a_copy(ops, cuda):
     assert ops.pool_stats()["alloc_cnt"] == mid["alloc_cnt"]
     helpers.assert_close(loss.reshape(-1), oracle.sce_sparse_fwd(x2, lab.reshape(-1), -100), dt, "loss")
     edl = oracle.sce_sparse_bwd(x2, lab.reshape(-1), gl.reshape(-1), -100)
-    helpers.assert_close(sdl, edl.reshape(B, S, H), dt, "dlogits", scale=float(np.abs(edl).max()) * 1e-2)
+    helpers.assert_close(sdl, edl.reshape(B, S, H), dt, "dlogits")
     assert untouched(wdl)
     # a view that is not row-pitched (every other column) still works as an input, through a dense copy
     half = torch.empty(B, S, H // 2, dtype=torch.bfloat16, device=cuda)

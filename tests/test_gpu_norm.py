@@ -281,4 +281,7 @@ def test_layer_norm_statistics_conditioning(hk, cuda, dtype, cols):
     assert np.all(got_rstd[16:18] == np.float32(1.0 / np.sqrt(np.float32(eps))))
     # a mean near 300 is only known to half an fp32 ulp (1.5e-5) in fp32 arithmetic, and x - mean inherits
     # that: the fp32 bound for y is loosened accordingly in this stress case
-    helpers.assert_close(ty, ey, dtype, "y", rtol=1e-4 if dtype == "fp32" else None)
+    # The strict figure is left out of the bound here on purpose: in the outlier rows the regular elements come out
+    # as |y| ~ 1e-3 (the outlier owns the variance) from x - mean with mean ~ 0.6..300, so the half ulp of the mean
+    # alone is percents of such an element, in any fp32 arithmetic.  It is still printed with the others.
+    helpers.assert_close(ty, ey, dtype, "y", rtol=1e-4 if dtype == "fp32" else None, strict_rtol=1e-1)

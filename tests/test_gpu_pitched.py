@@ -167,7 +167,7 @@ def test_cross_entropy_on_a_padded_vocabulary(hk, cuda, dt, layout):
     hk.sce_sparse_bwd(sx, tl, tgl, sdx, -100)
     torch.cuda.synchronize()
     edx = oracle.sce_sparse_bwd(x, lab, gl, -100)
-    helpers.assert_close(sdx, edx, dt, "dlogits", scale=float(np.abs(edx).max()) * 1e-2)
+    helpers.assert_close(sdx, edx, dt, "dlogits")
     assert not sdx[::5].float().any()            # ignored rows are zero rows inside the slice ...
     assert _untouched(wdx, off, cols)            # ... and nothing is written outside it
 

@@ -43,7 +43,7 @@ def test_sce_sparse(hk, cuda, dtype, shape):
     tdx = torch.full_like(tx, 3.0)
     hk.sce_sparse_bwd(tx, tl, tg, tdx, IGN)
     torch.cuda.synchronize()
-    helpers.assert_close(tdx, edx, dtype, "dlogits", scale=float(np.abs(edx).max()) * 1e-2)
+    helpers.assert_close(tdx, edx, dtype, "dlogits")
     if ign.any():
         assert torch.count_nonzero(tdx[torch.from_numpy(ign).to(cuda)]) == 0   # zero rows, bit exact
     # valid rows sum to ~0 (softmax sums to one)
@@ -104,7 +104,7 @@ def test_sce_dense(hk, cuda, dtype, shape):
     tdx = torch.empty_like(tx)
     hk.sce_dense_bwd(tx, tl, tg, tdx)
     torch.cuda.synchronize()
-    helpers.assert_close(tdx, edx, dtype, "dlogits", scale=float(np.abs(edx).max()) * 1e-2)
+    helpers.assert_close(tdx, edx, dtype, "dlogits")
 
 
 def test_sce_full_size_bf16(hk, cuda):
@@ -128,8 +128,7 @@ def test_sce_full_size_bf16(hk, cuda):
     eloss = oracle.sce_sparse_fwd(xs, lab[sel], IGN)
     helpers.assert_close(tloss[torch.from_numpy(sel).to(cuda)], eloss, "bf16", "loss")
     edx = oracle.sce_sparse_bwd(xs, lab[sel], np.full(len(sel), helpers.to_numpy(tg[:1])[0]), IGN)
-    helpers.assert_close(tdx[torch.from_numpy(sel).to(cuda)], edx, "bf16", "dlogits",
-                         scale=float(np.abs(edx).max()) * 1e-2)
+    helpers.assert_close(tdx[torch.from_numpy(sel).to(cuda)], edx, "bf16", "dlogits")
     ign = torch.from_numpy(lab == IGN).to(cuda)
     assert torch.count_nonzero(tloss[ign]) == 0
     assert torch.count_nonzero(tdx[ign]) == 0
@@ -154,4 +153,4 @@ def test_large_common_offset(hk, cuda):
         torch.cuda.synchronize()
         helpers.assert_close(tloss, oracle.sce_sparse_fwd(x, lab, IGN), "fp32", "loss")
         edx = oracle.sce_sparse_bwd(x, lab, g, IGN)
-        helpers.assert_close(tdx, edx, "fp32", "dlogits", scale=float(np.abs(edx).max()) * 1e-2)
+        helpers.assert_close(tdx, edx, "fp32", "dlogits")

@@ -20,7 +20,7 @@ def test_softmax_fwd_bwd(hk, cuda, dtype, shape, dim):
     ty = torch.empty_like(tx)
     hk.softmax_fwd(tx, ty, dim)
     torch.cuda.synchronize()
-    helpers.assert_close(ty, ey, dtype, "y", scale=float(ey.max()) * 1e-2)
+    helpers.assert_close(ty, ey, dtype, "y")
     sums = ty.float().sum(dim % len(shape)).cpu().numpy()
     assert np.max(np.abs(sums - 1.0)) <= (2e-2 if dtype != "fp32" else 1e-5)
 
@@ -70,7 +70,7 @@ def test_softmax_full_size_bf16(hk, cuda):
     sel = torch.from_numpy(np.sort(helpers.rng(3).choice(rows, 64, replace=False))).to(cuda)
     x2, y2, dy2, dx2 = (t.view(rows, 2048)[sel] for t in (tx, ty, tdy, tdx))
     ey = oracle.softmax_fwd(helpers.to_numpy(x2))
-    helpers.assert_close(y2, ey, "bf16", "y", scale=float(ey.max()) * 1e-2)
+    helpers.assert_close(y2, ey, "bf16", "y")
     edx = oracle.softmax_bwd(helpers.to_numpy(y2), helpers.to_numpy(dy2))
     helpers.assert_close(dx2, edx, "bf16", "dx")
     # size-independent properties on the whole tensor

@@ -591,28 +591,26 @@ def cpu_baseline(rows=32768, cols=4096, budget_s=3.0):
 
 
 def cpu_baselines(budget_s=1.2):
-    """One entry per BASELINE configuration kernel: the fp32 CPU ports of the reference's CPU kernels (the pass
-    structure of LayerNormCpu / LayerNormGradientCpu, the softmax and cross-entropy loops, the reductions) timed on
-    all host threads on a bounded sample of the configuration's rows, and on one thread where the reference's own
-    loop is serial.  `value` counts the same algorithmic bytes per row as the GPU entry of that configuration
-    (storage type of the configuration), so the two columns compare like with like."""
-    import ctypes
-    import numpy as np
-    import oracle
-    lib = oracle.lib()
+    """One entry per BASELINE configuration kernel: the host twins of the kernels (LayerNormCpu /
+    LayerNormGradientCpu, SoftmaxCpu / SoftmaxGradientCpu, SoftmaxCrossEntropySparseCpu / ...GradientCpu, ReduceCpu:
+    the reference's CPU pass structure as fp32 loops, OpenMP over rows), called through the same operator entry
+    points and device dispatch as the accelerator kernels, on a bounded sample of the configuration's rows in the
+    configuration's storage type.  `value` counts the same algorithmic bytes per row as the GPU entry of that
+    configuration, so the two columns compare like with like."""
+    import importlib
+    import torch
+    importlib.import_module("hotspa-ae_amd")
+    ops = importlib.import_module("hotspa-ae_amd.hetu_ops")
     cores = _cpu_cores()
-    g = np.random.default_rng(7)
-    fp = ctypes.POINTER(ctypes.c_float)
-    P = lambda a: a.ctypes.data_as(fp)
-    I = ctypes.c_int64
-    F = ctypes.c_float
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(7)
+    bf = torch.bfloat16
 
-    def block(rows, cols):
-        b = g.standard_normal((min(rows, 512), cols), dtype=np.float32)
-        return np.tile(b, ((rows + b.shape[0] - 1) // b.shape[0], 1))[:rows].copy()
+    def block(rows, cols, dt):
+        b = torch.randn(min(rows, 512), cols, generator=g)
+        return b.repeat((rows + b.shape[0] - 1) // b.shape[0], 1)[:rows].to(dt).contiguous()
 
-    def timed(fn, threads):
-        lib.refcpu_set_num_threads(ctypes.c_int(threads))
+    def timed(fn):
         fn()
         reps, t0 = 0, time.perf_counter()
         while reps < 2 or time.perf_counter() - t0 < budget_s:
@@ -622,69 +620,56 @@ def cpu_baselines(budget_s=1.2):
 
     out = []
 
-    def add(config, case, fn, algo_bytes, sample_rows, full_rows, serial_too=False):
-        dt, reps = timed(fn, cores)
-        rec = {"config": config, "case": case, "value": round(algo_bytes / dt / 1e9, 3), "unit": "GB/s",
-               "us": round(dt * 1e6, 1), "cores": cores, "kind": "port",
-               "sample": "%d of %d rows, fp32 arithmetic, %d repetitions, mean" % (sample_rows, full_rows, reps)}
-        if serial_too:
-            dt1, _ = timed(fn, 1)
-            rec["value_1_thread"], rec["us_1_thread"] = round(algo_bytes / dt1 / 1e9, 3), round(dt1 * 1e6, 1)
-        out.append(rec)
+    def add(config, case, fn, algo_bytes, sample_rows, full_rows, arith="fp32"):
+        dt, reps = timed(fn)
+        out.append({"config": config, "case": case, "value": round(algo_bytes / dt / 1e9, 3), "unit": "GB/s",
+                    "us": round(dt * 1e6, 1), "cores": cores, "kind": "port",
+                    "sample": "%d of %d rows, %s arithmetic, %d repetitions, mean" % (sample_rows, full_rows, arith, reps)})
 
-    # C1: the whole configuration (LayerNormCpu: two mean reductions + two element-wise passes, fp32)
+    # C1: the whole configuration, fp32 storage
     rows, cols = 8192, 4096
-    x = block(rows, cols); y = np.empty_like(x)
-    gm = np.ones(cols, np.float32); bt = np.zeros(cols, np.float32)
-    mean = np.empty(rows, np.float32); var = np.empty(rows, np.float32)
-    add("C1", "layernorm fwd fp32 [8192x4096] (LayerNormCpu pass structure)",
-        lambda: lib.refcpu_layernorm_fwd_f32(P(x), P(gm), P(bt), I(rows), I(cols), F(1e-5), P(y), P(mean), P(var)),
-        rows * (2 * cols * 4 + 8), rows, rows, serial_too=True)
-    # C5 layer norm at 5120 columns, forward and gradient, 1/4 of the rows; bf16 storage accounting
+    x = block(rows, cols, torch.float32); y = torch.empty_like(x)
+    gm, bt = torch.ones(cols), torch.zeros(cols)
+    mean, var = torch.empty(rows, 1), torch.empty(rows, 1)
+    add("C1", "layernorm fwd fp32 [8192x4096] (LayerNormCpu)",
+        lambda: ops.layer_norm(x, gm, bt, mean, var, y, 1, 1e-5), rows * (2 * cols * 4 + 8), rows, rows)
+    # C5 layer norm at 5120 columns, forward and gradient, 1/4 of the rows, bf16 storage
     rows, cols = 4096, 5120
-    x = block(rows, cols); y = np.empty_like(x); dy = block(rows, cols); dx = np.empty_like(x)
-    gm = np.ones(cols, np.float32); bt = np.zeros(cols, np.float32)
-    mean = np.empty(rows, np.float32); var = np.empty(rows, np.float32)
-    dgm = np.empty(cols, np.float32); dbt = np.empty(cols, np.float32)
-    add("C5", "layernorm fwd [16384x5120]",
-        lambda: lib.refcpu_layernorm_fwd_f32(P(x), P(gm), P(bt), I(rows), I(cols), F(1e-5), P(y), P(mean), P(var)),
-        rows * (2 * cols * 2 + 8), rows, 16384)
-    add("C5", "layernorm bwd [16384x5120] (LayerNormGradientCpu pass structure)",
-        lambda: lib.refcpu_layernorm_bwd_f32(P(dy), P(x), P(gm), P(mean), P(var), I(rows), I(cols), F(1e-5), P(dx),
-                                             P(dgm), P(dbt)),
+    x = block(rows, cols, bf); y = torch.empty_like(x); dy = block(rows, cols, bf); dx = torch.empty_like(x)
+    gm, bt = torch.ones(cols, dtype=bf), torch.zeros(cols, dtype=bf)
+    mean, var = torch.empty(rows, 1, dtype=bf), torch.empty(rows, 1, dtype=bf)
+    dgm, dbt = torch.empty(cols, dtype=bf), torch.empty(cols, dtype=bf)
+    add("C5", "layernorm fwd bf16 [16384x5120] (LayerNormCpu)",
+        lambda: ops.layer_norm(x, gm, bt, mean, var, y, 1, 1e-5), rows * (2 * cols * 2 + 8), rows, 16384)
+    add("C5", "layernorm bwd bf16 [16384x5120] (LayerNormGradientCpu)",
+        lambda: ops.layer_norm_gradient(dy, x, gm, dx, dgm, dbt, mean, var, 1, 1e-5),
         rows * (3 * cols * 2 + 8), rows, 16384)
     # C2: 1/16 of the rows
     rows, cols = 16384, 2048
-    x = block(rows, cols); y = np.empty_like(x); dx = np.empty_like(x)
-    add("C2", "softmax fwd [4,32,2048,2048]",
-        lambda: lib.refcpu_softmax_fwd_f32(P(x), I(rows), I(cols), P(y)), 2 * rows * cols * 2, rows, 262144)
-    add("C2", "softmax bwd [4,32,2048,2048]",
-        lambda: lib.refcpu_softmax_bwd_f32(P(y), P(x), I(rows), I(cols), P(dx)), 3 * rows * cols * 2, rows, 262144)
+    x = block(rows, cols, bf); y = torch.empty_like(x); dx = torch.empty_like(x)
+    add("C2", "softmax fwd bf16 [4,32,2048,2048] (SoftmaxCpu)", lambda: ops.softmax(x, y, 1),
+        2 * rows * cols * 2, rows, 262144)
+    add("C2", "softmax bwd bf16 [4,32,2048,2048] (SoftmaxGradientCpu)", lambda: ops.softmax_gradient(y, x, dx, 1),
+        3 * rows * cols * 2, rows, 262144)
     # C3: 1/4 of the rows
     rows, cols = 8192, 4096
-    x = block(rows, cols); o0 = np.empty(cols, np.float32); o1 = np.empty(rows, np.float32)
-    add("C3", "reduce sum axis 1 [32768x4096]",
-        lambda: lib.refcpu_reduce_sum_axis1_f32(P(x), I(rows), I(cols), P(o1)), rows * cols * 2, rows, 32768)
-    add("C3", "reduce mean axis 1 [32768x4096]",
-        lambda: lib.refcpu_reduce_mean_axis1_f32(P(x), I(rows), I(cols), P(o1)), rows * cols * 2, rows, 32768)
-    add("C3", "reduce sum axis 0 [32768x4096] (also the merged axes (0,1) of [64x512x4096])",
-        lambda: lib.refcpu_reduce_sum_axis0_f32(P(x), I(rows), I(cols), P(o0)), rows * cols * 2, rows, 32768)
-    add("C3", "reduce mean axis 0 [32768x4096]",
-        lambda: lib.refcpu_reduce_mean_axis0_f32(P(x), I(rows), I(cols), P(o0)), rows * cols * 2, rows, 32768)
+    x = block(rows, cols, bf); o0 = torch.empty(cols, dtype=bf); o1 = torch.empty(rows, dtype=bf)
+    for name, axes, o in (("axis 1", [1], o1), ("axis 0", [0], o0)):
+        for red in ("sum", "mean"):
+            add("C3", "reduce %s %s bf16 [32768x4096] (ReduceCpu)%s" % (
+                red, name, "; also the merged axes (0,1) of [64x512x4096]" if (axes == [0] and red == "sum") else ""),
+                (lambda axes=axes, o=o, red=red: ops.reduce(x, o, axes, red)), rows * cols * 2, rows, 32768)
     # C5 cross-entropy: 1/16 of the rows
     rows, cols = 1024, 32000
-    x = block(rows, cols); loss = np.empty(rows, np.float32); dx = np.empty_like(x)
-    gl = np.full(rows, 1.0 / 16384, np.float32)
-    lab = (np.arange(rows, dtype=np.int64) * 31) % cols
+    x = block(rows, cols, bf); loss = torch.empty(rows, dtype=bf); dx = torch.empty_like(x)
+    gl = torch.full((rows,), 1.0 / 16384, dtype=bf)
+    lab = (torch.arange(rows, dtype=torch.int64) * 31) % cols
     lab[::20] = IGNORE
-    L = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_int64))
-    add("C5", "cross-entropy fwd [16384x32000]",
-        lambda: lib.refcpu_sce_sparse_fwd_f32(P(x), L(lab), I(rows), I(cols), I(IGNORE), P(loss)),
-        rows * (cols * 2 + 10), rows, 16384)
-    add("C5", "cross-entropy bwd [16384x32000]",
-        lambda: lib.refcpu_sce_sparse_bwd_f32(P(x), L(lab), P(gl), I(rows), I(cols), I(IGNORE), P(dx)),
+    add("C5", "cross-entropy fwd bf16 [16384x32000] (SoftmaxCrossEntropySparseCpu)",
+        lambda: ops.softmax_cross_entropy_sparse(x, lab, loss, IGNORE), rows * (cols * 2 + 10), rows, 16384)
+    add("C5", "cross-entropy bwd bf16 [16384x32000] (SoftmaxCrossEntropySparseGradientCpu)",
+        lambda: ops.softmax_cross_entropy_sparse_gradient(x, lab, gl, dx, IGNORE),
         rows * (2 * cols * 2 + 10), rows, 16384)
-    lib.refcpu_set_num_threads(ctypes.c_int(cores))
     return out
 
 

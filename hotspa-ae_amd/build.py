@@ -97,7 +97,8 @@ def build_host(verbose=True):
     os.makedirs(LIB, exist_ok=True)
     objdir = os.path.join(OBJ, "host")
     os.makedirs(objdir, exist_ok=True)
-    cxx = ["g++", "-O2", "-std=c++17", "-fPIC", "-pthread", "-I" + INCLUDE, "-I" + HERE]
+    # OpenMP: the host twins of the kernels share their rows out over the cores
+    cxx = ["g++", "-O3", "-std=c++17", "-fPIC", "-pthread", "-fopenmp", "-I" + INCLUDE, "-I" + HERE]
     srcs = sorted(srcs)
     objs = [os.path.join(objdir, os.path.relpath(s, HOST).replace(os.sep, "_")[:-3] + ".o") for s in srcs]
 
@@ -111,7 +112,7 @@ def build_host(verbose=True):
             if verbose:
                 print("[build] compiled", os.path.relpath(src, ROOT), flush=True)
     out = os.path.join(LIB, "libhetu_rowwise.so")
-    _run(["g++", "-shared", "-pthread", "-o", out] + objs +
+    _run(["g++", "-shared", "-pthread", "-fopenmp", "-o", out] + objs +
          ["-L" + LIB, "-lhk_rowwise", "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("[build] linked", out, flush=True)

@@ -1,6 +1,8 @@
 // extern "C" face of the operator layer (declared in hetu_ops_c.h).
 #include "hetu_ops_c.h"
 
+#include <cstring>
+
 #include <string>
 
 #include "hetu/graph/ops/gradient_compute.h"
@@ -66,6 +68,10 @@ void copy_out(const NDArray& result, HtArray* out, const Stream& stream) {
     << "result " << result->meta() << " does not fit the buffer " << dst->meta();
   if (result->numel() == 0) return;
   NDArray src = NDArray::contiguous(result, stream.stream_index());
+  if (stream.device().is_cpu()) {   // host result (the host twins ran in this thread): a plain copy
+    std::memcpy(dst->raw_data_ptr(), src->raw_data_ptr(), src->numel() * DataType2Size(src->dtype()));
+    return;
+  }
   hetu::impl::HIPStream hs(stream);
   hetu::hip::DeviceGuard guard(hs.device_id());
   HK_CALL(hk_memcpy_d2d(dst->raw_data_ptr(), src->raw_data_ptr(), src->numel() * DataType2Size(src->dtype()), hs));
@@ -90,8 +96,9 @@ int ht_layer_norm(const HtArray* in, const HtArray* scale, const HtArray* bias, 
                   HtArray* out, int64_t reduce_dims, float eps, int stream_index) {
   return guarded([&] {
     NDArray m = wrap(mean), v = wrap(var), o = wrap(out);
-    hetu::impl::LayerNormCuda(wrap(in), wrap(scale), wrap(bias), m, v, o, reduce_dims, eps,
-                              stream_of(in, stream_index));
+    const Stream st = stream_of(in, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_layer_norm", hetu::impl::LayerNorm, wrap(in), wrap(scale),
+                                    wrap(bias), m, v, o, reduce_dims, eps, st);
   });
 }
 
@@ -100,8 +107,10 @@ int ht_layer_norm_gradient(const HtArray* out_grads, const HtArray* in, const Ht
                            int64_t reduce_dims, float eps, int stream_index) {
   return guarded([&] {
     NDArray gi = wrap(grad_in), gs = wrap(grad_scale), gb = wrap(grad_bias);
-    hetu::impl::LayerNormGradientCuda(wrap(out_grads), wrap(in), wrap(scale), gi, gs, gb, wrap(mean), wrap(var),
-                                      reduce_dims, eps, stream_of(in, stream_index));
+    const Stream st = stream_of(in, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_layer_norm_gradient", hetu::impl::LayerNormGradient,
+                                    wrap(out_grads), wrap(in), wrap(scale), gi, gs, gb, wrap(mean), wrap(var),
+                                    reduce_dims, eps, st);
   });
 }
 
@@ -213,14 +222,17 @@ int ht_instance_norm_gradient(const HtArray* out_grads, const HtArray* in, HtArr
 int ht_softmax(const HtArray* in, HtArray* out, int64_t dim, int stream_index) {
   return guarded([&] {
     NDArray o = wrap(out);
-    hetu::impl::SoftmaxCuda(wrap(in), o, dim, stream_of(in, stream_index));
+    const Stream st = stream_of(in, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_softmax", hetu::impl::Softmax, wrap(in), o, dim, st);
   });
 }
 
 int ht_softmax_gradient(const HtArray* y, const HtArray* dy, HtArray* dx, int64_t dim, int stream_index) {
   return guarded([&] {
     NDArray o = wrap(dx);
-    hetu::impl::SoftmaxGradientCuda(wrap(y), wrap(dy), o, dim, stream_of(y, stream_index));
+    const Stream st = stream_of(y, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_softmax_gradient", hetu::impl::SoftmaxGradient, wrap(y),
+                                    wrap(dy), o, dim, st);
   });
 }
 
@@ -244,8 +256,10 @@ int ht_softmax_cross_entropy_sparse(const HtArray* pred, const HtArray* label, H
                                     int64_t ignored_index, int stream_index) {
   return guarded([&] {
     NDArray o = wrap(loss);
-    hetu::impl::SoftmaxCrossEntropySparseCuda(wrap(pred), wrap(label), o, ignored_index,
-                                              stream_of(pred, stream_index));
+    const Stream st = stream_of(pred, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_softmax_cross_entropy_sparse",
+                                    hetu::impl::SoftmaxCrossEntropySparse, wrap(pred), wrap(label), o,
+                                    ignored_index, st);
   });
 }
 
@@ -253,8 +267,10 @@ int ht_softmax_cross_entropy_sparse_gradient(const HtArray* pred, const HtArray*
                                              HtArray* out, int64_t ignored_index, int stream_index) {
   return guarded([&] {
     NDArray o = wrap(out);
-    hetu::impl::SoftmaxCrossEntropySparseGradientCuda(wrap(pred), wrap(label), wrap(grad_loss), o, ignored_index,
-                                                      stream_of(pred, stream_index));
+    const Stream st = stream_of(pred, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_softmax_cross_entropy_sparse_gradient",
+                                    hetu::impl::SoftmaxCrossEntropySparseGradient, wrap(pred), wrap(label),
+                                    wrap(grad_loss), o, ignored_index, st);
   });
 }
 
@@ -277,7 +293,9 @@ int ht_reduce(const HtArray* in, HtArray* out, const int64_t* axes, int naxes, i
   return guarded([&] {
     NDArray o = wrap(out);
     HTAxes ax(axes, axes + naxes);
-    hetu::impl::ReduceCuda(wrap(in), o, ax, static_cast<ReductionType>(red_type), stream_of(in, stream_index));
+    const Stream st = stream_of(in, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_reduce", hetu::impl::Reduce, wrap(in), o, ax,
+                                    static_cast<ReductionType>(red_type), st);
   });
 }
 

@@ -6,6 +6,10 @@
 // the kernels as they are, any other input layout through a dense copy.
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
+#include "hetu/impl/utils/cpu_utils.h"
+#include "hetu/impl/utils/dispatch.h"
+
+#include <algorithm>
 
 namespace hetu {
 namespace impl {
@@ -108,15 +112,153 @@ void LayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr, cons
   NDArray::MarkUsedBy({dy, x, g, mean, var, grad_arr, grad_scale, grad_bias, ws}, stream);
 }
 
-void LayerNormCpu(const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&, NDArray&, int64_t, float,
-                  const Stream&) {
-  HT_NOT_IMPLEMENTED << "LayerNorm has no host kernel in this build (the reference's is a oneDNN primitive); "
-                        "move the arrays to the accelerator";
+// ---------------------------------------------------------------------------------------------------------
+// Host twins (hetu/impl/kernel/LayerNorm.cc:34-142 and :177-364 of the reference): the same three passes over a
+// row as the reference makes over the array (mean; mean of (x - mean)^2; the output), and for the gradient the
+// column sums first (grad_bias = sum dy, grad_scale = sum dy * x_hat) and then dx from the two row sums.  The
+// reference's host dx leaves the scale out of the row terms (calculate_grad_kernel, LayerNorm.cc:160-175, never
+// reads ln_scale); this twin computes what the accelerator kernel computes,
+//   t = dy * scale,  dx = rstd * (t - mean(t) - x_hat * mean(t * x_hat)).
+// The work runs in the calling thread (and its OpenMP team) before the call returns.
+// ---------------------------------------------------------------------------------------------------------
+void LayerNormCpu(const NDArray& in_arr, const NDArray& ln_scale, const NDArray& ln_bias, NDArray& mean_arr,
+                  NDArray& var_arr, NDArray& out_arr, int64_t reduce_dims, float eps, const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(in_arr);
+  HT_ASSERT_SAME_DEVICE(in_arr, ln_scale);
+  HT_ASSERT_SAME_DEVICE(in_arr, ln_bias);
+  HT_ASSERT_SAME_DEVICE(in_arr, mean_arr);
+  HT_ASSERT_SAME_DEVICE(in_arr, var_arr);
+  HT_ASSERT_SAME_DEVICE(in_arr, out_arr);
+  HT_ASSERT_SAME_SHAPE(in_arr, out_arr);
+  HT_ASSERT_SAME_DTYPE(in_arr, out_arr);
+  HT_ASSERT_SAME_DTYPE(in_arr, ln_scale);
+  HT_ASSERT_SAME_DTYPE(in_arr, ln_bias);
+  HT_ASSERT_SAME_DTYPE(in_arr, mean_arr);
+  HT_ASSERT_SAME_DTYPE(in_arr, var_arr);
+  HT_ASSERT_CONTIGUOUS(out_arr);
+  HT_ASSERT_CONTIGUOUS(mean_arr);
+  HT_ASSERT_CONTIGUOUS(var_arr);
+  int64_t rows, cols;
+  SplitRows(in_arr, reduce_dims, rows, cols);
+  HT_ASSERT(int64_t(ln_scale->numel()) == cols && int64_t(ln_bias->numel()) == cols)
+    << "scale / bias must hold " << cols << " values";
+  HT_ASSERT(int64_t(mean_arr->numel()) == rows && int64_t(var_arr->numel()) == rows)
+    << "statistics must hold one value per row (" << rows << ")";
+  if (in_arr->numel() == 0) return;
+  NDArray x = Dense(in_arr, stream), g = Dense(ln_scale, stream), b = Dense(ln_bias, stream);
+  HT_DISPATCH_FLOATING_TYPES(in_arr->dtype(), spec_t, "LayerNormCpu", [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* xp = x->data_ptr<spec_t>();
+    const spec_t* gp = g->data_ptr<spec_t>();
+    const spec_t* bp = b->data_ptr<spec_t>();
+    spec_t* mp = mean_arr->data_ptr<spec_t>();
+    spec_t* vp = var_arr->data_ptr<spec_t>();
+    spec_t* yp = out_arr->data_ptr<spec_t>();
+    const A inv = A(1) / A(cols);
+    cpu::parallel_rows(rows, cols, [&](int64_t r) {
+      const spec_t* xr = xp + r * cols;
+      const A mean = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); }) * inv;
+      const A var = cpu::blocked_sum<A>(cols, [&](int64_t i) {
+        const A d = cpu::ld<spec_t, A>(xr + i) - mean;
+        return d * d;
+      }) * inv;
+      cpu::st<spec_t, A>(mp + r, mean);
+      cpu::st<spec_t, A>(vp + r, var);
+      const A rstd = A(1) / std::sqrt(var + A(eps));
+      spec_t* yr = yp + r * cols;
+      for (int64_t i = 0; i < cols; ++i)
+        cpu::st<spec_t, A>(yr + i, (cpu::ld<spec_t, A>(xr + i) - mean) * rstd * cpu::ld<spec_t, A>(gp + i) +
+                                     cpu::ld<spec_t, A>(bp + i));
+    });
+  });
 }
 
-void LayerNormGradientCpu(const NDArray&, const NDArray&, const NDArray&, NDArray&, NDArray&, NDArray&,
-                          const NDArray&, const NDArray&, int64_t, float, const Stream&) {
-  HT_NOT_IMPLEMENTED << "LayerNormGradient has no host kernel in this build; move the arrays to the accelerator";
+void LayerNormGradientCpu(const NDArray& out_grads, const NDArray& in_arr, const NDArray& ln_scale,
+                          NDArray& grad_arr, NDArray& grad_scale, NDArray& grad_bias, const NDArray& mean_arr,
+                          const NDArray& var_arr, int64_t reduce_dims, float eps, const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(out_grads);
+  HT_ASSERT_SAME_DEVICE(out_grads, ln_scale);
+  HT_ASSERT_SAME_DEVICE(out_grads, in_arr);
+  HT_ASSERT_SAME_DEVICE(out_grads, mean_arr);
+  HT_ASSERT_SAME_DEVICE(out_grads, var_arr);
+  HT_ASSERT_SAME_DEVICE(out_grads, grad_scale);
+  HT_ASSERT_SAME_DEVICE(out_grads, grad_arr);
+  HT_ASSERT_SAME_DEVICE(out_grads, grad_bias);
+  HT_ASSERT_SAME_SHAPE(out_grads, in_arr);
+  HT_ASSERT_SAME_SHAPE(out_grads, grad_arr);
+  HT_ASSERT_SAME_DTYPE(out_grads, in_arr);
+  HT_ASSERT_SAME_DTYPE(out_grads, grad_arr);
+  HT_ASSERT_SAME_DTYPE(out_grads, ln_scale);
+  HT_ASSERT_SAME_DTYPE(out_grads, grad_scale);
+  HT_ASSERT_SAME_DTYPE(out_grads, grad_bias);
+  HT_ASSERT_SAME_DTYPE(out_grads, mean_arr);
+  HT_ASSERT_SAME_DTYPE(out_grads, var_arr);
+  HT_ASSERT_CONTIGUOUS(grad_arr);
+  HT_ASSERT_CONTIGUOUS(grad_scale);
+  HT_ASSERT_CONTIGUOUS(grad_bias);
+  int64_t rows, cols;
+  SplitRows(in_arr, reduce_dims, rows, cols);
+  HT_ASSERT(int64_t(ln_scale->numel()) == cols && int64_t(grad_scale->numel()) == cols &&
+            int64_t(grad_bias->numel()) == cols)
+    << "scale / grad_scale / grad_bias must hold " << cols << " values";
+  HT_ASSERT(int64_t(mean_arr->numel()) == rows && int64_t(var_arr->numel()) == rows)
+    << "statistics must hold one value per row (" << rows << ")";
+  NDArray dy = Dense(out_grads, stream), x = Dense(in_arr, stream), g = Dense(ln_scale, stream);
+  NDArray mean = Dense(mean_arr, stream), var = Dense(var_arr, stream);
+  HT_DISPATCH_FLOATING_TYPES(in_arr->dtype(), spec_t, "LayerNormGradientCpu", [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* dyp = dy->data_ptr<spec_t>();
+    const spec_t* xp = x->data_ptr<spec_t>();
+    const spec_t* gp = g->data_ptr<spec_t>();
+    const spec_t* mp = mean->data_ptr<spec_t>();
+    const spec_t* vp = var->data_ptr<spec_t>();
+    spec_t* dxp = grad_arr->data_ptr<spec_t>();
+    spec_t* dgp = grad_scale->data_ptr<spec_t>();
+    spec_t* dbp = grad_bias->data_ptr<spec_t>();
+    // column sums, a band of columns per thread: every thread walks all rows of its band
+    constexpr int64_t kBand = 64;
+    const int64_t bands = (cols + kBand - 1) / kBand;
+    cpu::parallel_rows(bands, rows * kBand, [&](int64_t band) {
+      const int64_t c0 = band * kBand, c1 = std::min(cols, c0 + kBand);
+      A sg[kBand], sb[kBand];
+      for (int64_t c = 0; c < kBand; ++c) sg[c] = sb[c] = A(0);
+      for (int64_t r = 0; r < rows; ++r) {
+        const A m = cpu::ld<spec_t, A>(mp + r);
+        const A rstd = A(1) / std::sqrt(cpu::ld<spec_t, A>(vp + r) + A(eps));
+        const spec_t* dyr = dyp + r * cols;
+        const spec_t* xr = xp + r * cols;
+        for (int64_t c = c0; c < c1; ++c) {
+          const A d = cpu::ld<spec_t, A>(dyr + c);
+          sb[c - c0] += d;
+          sg[c - c0] += d * (cpu::ld<spec_t, A>(xr + c) - m) * rstd;
+        }
+      }
+      for (int64_t c = c0; c < c1; ++c) {
+        cpu::st<spec_t, A>(dgp + c, sg[c - c0]);
+        cpu::st<spec_t, A>(dbp + c, sb[c - c0]);
+      }
+    });
+    if (in_arr->numel() == 0) return;
+    const A inv = A(1) / A(cols);
+    cpu::parallel_rows(rows, cols, [&](int64_t r) {
+      const A m = cpu::ld<spec_t, A>(mp + r);
+      const A rstd = A(1) / std::sqrt(cpu::ld<spec_t, A>(vp + r) + A(eps));
+      const spec_t* dyr = dyp + r * cols;
+      const spec_t* xr = xp + r * cols;
+      const A s1 = cpu::blocked_sum<A>(cols, [&](int64_t i) {
+        return cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i);
+      }) * inv;
+      const A s2 = cpu::blocked_sum<A>(cols, [&](int64_t i) {
+        return cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i) * (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
+      }) * inv;
+      spec_t* dxr = dxp + r * cols;
+      for (int64_t i = 0; i < cols; ++i) {
+        const A xh = (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
+        const A t = cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i);
+        cpu::st<spec_t, A>(dxr + i, rstd * (t - s1 - xh * s2));
+      }
+    });
+  });
 }
 
 } // namespace impl

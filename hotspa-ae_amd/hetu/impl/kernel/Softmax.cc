@@ -6,6 +6,8 @@
 // dense first, and a softmax over another dimension needs a dense output.
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
+#include "hetu/impl/utils/cpu_utils.h"
+#include "hetu/impl/utils/dispatch.h"
 
 namespace hetu {
 namespace impl {
@@ -80,13 +82,72 @@ void SoftmaxGradientCuda(const NDArray& input_Y, const NDArray& output_grad, NDA
   NDArray::MarkUsedBy({y, dy, input_grad}, stream);
 }
 
-void SoftmaxCpu(const NDArray&, NDArray&, int64_t, const Stream&) {
-  HT_NOT_IMPLEMENTED << "Softmax has no host kernel in this build (the reference's is a oneDNN primitive); "
-                        "move the arrays to the accelerator";
+// ---------------------------------------------------------------------------------------------------------
+// Host twins (hetu/impl/kernel/Softmax.cc:11-97 of the reference, oneDNN's softmax_accurate there): per line
+// along `dim` the maximum, the sum of exp(x - max), then exp(x - max) / sum; for the gradient
+// dx = y * (dy - sum(dy * y)).  Lines are independent and shared out over the OpenMP team.
+// ---------------------------------------------------------------------------------------------------------
+void SoftmaxCpu(const NDArray& input, NDArray& output, int64_t dim, const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(input);
+  HT_ASSERT_SAME_DEVICE(input, output);
+  HT_ASSERT_SAME_SHAPE(input, output);
+  HT_ASSERT_SAME_DTYPE(input, output);
+  HT_ASSERT_CONTIGUOUS(output);
+  int64_t outer, extent, inner;
+  SplitAtDim(input, dim, outer, extent, inner);
+  if (input->numel() == 0) return;
+  NDArray x = Dense(input, stream);
+  HT_DISPATCH_FLOATING_TYPES(input->dtype(), spec_t, "SoftmaxCpu", [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* xp = x->data_ptr<spec_t>();
+    spec_t* yp = output->data_ptr<spec_t>();
+    cpu::parallel_rows(outer * inner, extent, [&](int64_t line) {
+      const int64_t o = line / inner, i = line - o * inner;
+      const spec_t* xl = xp + o * extent * inner + i;
+      spec_t* yl = yp + o * extent * inner + i;
+      const A m = cpu::blocked_max<A>(extent, [&](int64_t k) { return cpu::ld<spec_t, A>(xl + k * inner); });
+      // a line of -inf only: exp(-inf - -inf) is NaN, as on the accelerator
+      const A sum = cpu::blocked_sum<A>(extent, [&](int64_t k) {
+        return std::exp(cpu::ld<spec_t, A>(xl + k * inner) - m);
+      });
+      const A inv = A(1) / sum;
+      for (int64_t k = 0; k < extent; ++k)
+        cpu::st<spec_t, A>(yl + k * inner, std::exp(cpu::ld<spec_t, A>(xl + k * inner) - m) * inv);
+    });
+  });
 }
 
-void SoftmaxGradientCpu(const NDArray&, const NDArray&, NDArray&, int64_t, const Stream&) {
-  HT_NOT_IMPLEMENTED << "SoftmaxGradient has no host kernel in this build; move the arrays to the accelerator";
+void SoftmaxGradientCpu(const NDArray& input_Y, const NDArray& output_grad, NDArray& input_grad, int64_t dim,
+                        const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(input_Y);
+  HT_ASSERT_SAME_DEVICE(input_Y, output_grad);
+  HT_ASSERT_SAME_DEVICE(input_Y, input_grad);
+  HT_ASSERT_SAME_SHAPE(input_Y, output_grad);
+  HT_ASSERT_SAME_SHAPE(input_Y, input_grad);
+  HT_ASSERT_SAME_DTYPE(input_Y, output_grad);
+  HT_ASSERT_SAME_DTYPE(input_Y, input_grad);
+  HT_ASSERT_CONTIGUOUS(input_grad);
+  int64_t outer, extent, inner;
+  SplitAtDim(input_Y, dim, outer, extent, inner);
+  if (input_Y->numel() == 0) return;
+  NDArray y = Dense(input_Y, stream), dy = Dense(output_grad, stream);
+  HT_DISPATCH_FLOATING_TYPES(input_Y->dtype(), spec_t, "SoftmaxGradientCpu", [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* yp = y->data_ptr<spec_t>();
+    const spec_t* dyp = dy->data_ptr<spec_t>();
+    spec_t* dxp = input_grad->data_ptr<spec_t>();
+    cpu::parallel_rows(outer * inner, extent, [&](int64_t line) {
+      const int64_t o = line / inner, i = line - o * inner;
+      const int64_t base = o * extent * inner + i;
+      const A dot = cpu::blocked_sum<A>(extent, [&](int64_t k) {
+        return cpu::ld<spec_t, A>(yp + base + k * inner) * cpu::ld<spec_t, A>(dyp + base + k * inner);
+      });
+      for (int64_t k = 0; k < extent; ++k) {
+        const int64_t e = base + k * inner;
+        cpu::st<spec_t, A>(dxp + e, cpu::ld<spec_t, A>(yp + e) * (cpu::ld<spec_t, A>(dyp + e) - dot));
+      }
+    });
+  });
 }
 
 } // namespace impl

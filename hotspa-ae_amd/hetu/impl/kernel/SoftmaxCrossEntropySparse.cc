@@ -4,6 +4,8 @@
 // `ignored_index` has loss 0 and a zero gradient row.
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
+#include "hetu/impl/utils/cpu_utils.h"
+#include "hetu/impl/utils/dispatch.h"
 
 namespace hetu {
 namespace impl {
@@ -104,14 +106,92 @@ void SoftmaxCrossEntropySparseGradientReducedCuda(const NDArray& pred, const NDA
   SparseGradient(pred, label, grad_output, &scale, output, ignored_index, stream);
 }
 
-void SoftmaxCrossEntropySparseCpu(const NDArray&, const NDArray&, NDArray&, const int64_t, const Stream&) {
-  HT_NOT_IMPLEMENTED << "SoftmaxCrossEntropySparse has no host kernel in this build; move the arrays to the accelerator";
+// ---------------------------------------------------------------------------------------------------------
+// Host twins (hetu/impl/kernel/SoftmaxCrossEntropySparse.cc:11-126 of the reference): per row the maximum, the sum
+// of exp(x - max), then loss = log(sum) - (x[label] - max), or the gradient (softmax - onehot) * grad_loss.  A row
+// whose label is `ignored_index` gets loss 0 / a zero gradient row and the other rows are still computed (the
+// reference's loops leave the whole parallel chunk at the first such row, SoftmaxCrossEntropySparse.cc:21-24,
+// 47-53); a label outside [0, cols) gives NaN, as on the accelerator.
+// ---------------------------------------------------------------------------------------------------------
+void SoftmaxCrossEntropySparseCpu(const NDArray& pred, const NDArray& label, NDArray& loss,
+                                  const int64_t ignored_index, const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(pred);
+  HT_ASSERT_SAME_DEVICE(pred, label);
+  HT_ASSERT_SAME_DEVICE(pred, loss);
+  HT_ASSERT_SAME_DTYPE(pred, loss);
+  HT_ASSERT(label->dtype() == kInt64) << "labels must be int64 class ids, got " << label->dtype();
+  HT_ASSERT_CONTIGUOUS(loss);
+  int64_t rows, cols;
+  RowsCols(pred, rows, cols);
+  HT_ASSERT(int64_t(label->numel()) == rows && int64_t(loss->numel()) == rows)
+    << "labels " << label->shape() << " / loss " << loss->shape() << " must hold one value per row of "
+    << pred->shape();
+  if (rows == 0) return;
+  HT_VALUE_ERROR_IF(cols == 0) << "cross entropy over zero classes";
+  NDArray p = Dense(pred, stream), l = Dense(label, stream);
+  HT_DISPATCH_FLOATING_TYPES(pred->dtype(), spec_t, "SoftmaxCrossEntropySparseCpu", [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* pp = p->data_ptr<spec_t>();
+    const int64_t* lp = l->data_ptr<int64_t>();
+    spec_t* out = loss->data_ptr<spec_t>();
+    cpu::parallel_rows(rows, cols, [&](int64_t r) {
+      const int64_t lab = lp[r];
+      if (lab == ignored_index) { cpu::st<spec_t, A>(out + r, A(0)); return; }
+      if (lab < 0 || lab >= cols) { cpu::st<spec_t, A>(out + r, std::numeric_limits<A>::quiet_NaN()); return; }
+      const spec_t* xr = pp + r * cols;
+      const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
+      const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+      cpu::st<spec_t, A>(out + r, std::log(sum) - (cpu::ld<spec_t, A>(xr + lab) - m));
+    });
+  });
 }
 
-void SoftmaxCrossEntropySparseGradientCpu(const NDArray&, const NDArray&, const NDArray&, NDArray&, const int64_t,
-                                          const Stream&) {
-  HT_NOT_IMPLEMENTED << "SoftmaxCrossEntropySparseGradient has no host kernel in this build; move the arrays to the "
-                        "accelerator";
+void SoftmaxCrossEntropySparseGradientCpu(const NDArray& pred, const NDArray& label, const NDArray& grad_loss,
+                                          NDArray& output, const int64_t ignored_index, const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(pred);
+  HT_ASSERT_SAME_DEVICE(pred, label);
+  HT_ASSERT_SAME_DEVICE(pred, grad_loss);
+  HT_ASSERT_SAME_DEVICE(pred, output);
+  HT_ASSERT_SAME_SHAPE(pred, output);
+  HT_ASSERT_SAME_DTYPE(pred, output);
+  HT_ASSERT_SAME_DTYPE(pred, grad_loss);
+  HT_ASSERT(label->dtype() == kInt64) << "labels must be int64 class ids, got " << label->dtype();
+  HT_ASSERT_CONTIGUOUS(output);
+  int64_t rows, cols;
+  RowsCols(pred, rows, cols);
+  HT_ASSERT(int64_t(label->numel()) == rows && int64_t(grad_loss->numel()) == rows)
+    << "labels " << label->shape() << " / grad_loss " << grad_loss->shape()
+    << " must hold one value per row of " << pred->shape();
+  if (pred->numel() == 0) return;
+  NDArray p = Dense(pred, stream), l = Dense(label, stream), gl = Dense(grad_loss, stream);
+  HT_DISPATCH_FLOATING_TYPES(pred->dtype(), spec_t, "SoftmaxCrossEntropySparseGradientCpu", [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* pp = p->data_ptr<spec_t>();
+    const int64_t* lp = l->data_ptr<int64_t>();
+    const spec_t* gp = gl->data_ptr<spec_t>();
+    spec_t* out = output->data_ptr<spec_t>();
+    cpu::parallel_rows(rows, cols, [&](int64_t r) {
+      const int64_t lab = lp[r];
+      spec_t* dr = out + r * cols;
+      if (lab == ignored_index) {
+        for (int64_t i = 0; i < cols; ++i) cpu::st<spec_t, A>(dr + i, A(0));
+        return;
+      }
+      if (lab < 0 || lab >= cols) {
+        for (int64_t i = 0; i < cols; ++i) cpu::st<spec_t, A>(dr + i, std::numeric_limits<A>::quiet_NaN());
+        return;
+      }
+      const spec_t* xr = pp + r * cols;
+      const A g = cpu::ld<spec_t, A>(gp + r);
+      const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
+      const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+      const A scale = g / sum;
+      for (int64_t i = 0; i < cols; ++i) {
+        const A pr = std::exp(cpu::ld<spec_t, A>(xr + i) - m) * scale;
+        cpu::st<spec_t, A>(dr + i, i == lab ? pr - g : pr);
+      }
+    });
+  });
 }
 
 } // namespace impl

@@ -262,16 +262,28 @@ int main() {
     CHECK(throws<assertion_error>([&] { NDArray::as_strided(a, {2, 3, 4}, {12, 4, 1}, 9); }));
   });
 
-  run("device switch: host arrays have no kernels on this path", [] {
+  run("device switch: host arrays run the host twins, accelerator-only kernels refuse them", [] {
     NDArray a = NDArray::zeros({4, 8}, Device(kCPU), kFloat32);
     NDArray g = NDArray::zeros({8}, Device(kCPU), kFloat32);
-    CHECK(throws<not_implemented>([&] { NDArray::softmax(a, 1); }));
-    CHECK(throws<not_implemented>([&] { NDArray::sum(a, {0}); }));
-    CHECK(throws<not_implemented>([&] { NDArray::layernorm(a, g, g, {8}); }));
+    for (int i = 0; i < 32; ++i) a->data_ptr<float>()[i] = float(i % 8);
+    for (int i = 0; i < 8; ++i) g->data_ptr<float>()[i] = 1.f;
+    NDArray sm = NDArray::softmax(a, 1);
+    for (int r = 0; r < 4; ++r) {
+      float s = 0.f;
+      for (int c = 0; c < 8; ++c) s += sm->data_ptr<float>()[r * 8 + c];
+      CHECK(std::fabs(s - 1.f) < 1e-6f);
+    }
+    NDArray cs = NDArray::sum(a, {0});
+    for (int c = 0; c < 8; ++c) CHECK(cs->data_ptr<float>()[c] == 4.f * float(c));
+    NDArrayList ln = NDArray::layernorm(a, g, NDArray::zeros({8}, Device(kCPU), kFloat32), {8});
+    CHECK(std::fabs(ln[1]->data_ptr<float>()[0] - 3.5f) < 1e-6f);     // mean of 0..7
+    CHECK(std::fabs(ln[2]->data_ptr<float>()[0] - 5.25f) < 1e-5f);    // variance of 0..7
     // the fused variant exists for the accelerator only: the switch itself refuses
     CHECK(throws<not_implemented>([&] { NDArray::fused_layernorm(a, g, g, {8}); }, "cpu"));
     NDArray lab = NDArray::zeros({4}, Device(kCPU), kInt64);
-    CHECK(throws<not_implemented>([&] { NDArray::sceloss(a, lab, int64_t(-1)); }));
+    lab->data_ptr<int64_t>()[1] = -1;   // ignored
+    NDArray loss = NDArray::sceloss(a, lab, int64_t(-1), kNONE);
+    CHECK(loss->data_ptr<float>()[1] == 0.f && loss->data_ptr<float>()[0] > 7.f);
     // an accelerator kernel handed host arrays fails its device assertion
     NDArray out = NDArray::empty_like(a);
     CHECK(throws<assertion_error>([&] { hetu::impl::SoftmaxCuda(a, out, 1, Stream(Device(kCUDA, 0), 1)); }));

@@ -52,14 +52,20 @@ def test_errors_map_to_exception_kinds_without_a_gpu():
     ops = _ops()
     x = torch.zeros(4, 8)
     out = torch.empty(4, 8)
-    # host arrays handed to an accelerator kernel: the device assertion fires before any GPU call
+    # host arrays handed to an accelerator-only kernel: the device assertion fires before any GPU call
     with pytest.raises(ops.AssertionError_, match="not on an accelerator"):
-        ops.softmax(x, out, 1)
-    # the NDArray static dispatches on the device type; the host has no kernel here
+        ops.fused_layer_norm(x, torch.ones(8), torch.zeros(8), torch.empty(4), torch.empty(4), out, 1, 1e-5)
+    # kernels with a host twin dispatch on the device type and run on the host
+    ops.softmax(x, out, 1)
+    assert torch.allclose(out, torch.full((4, 8), 0.125))
+    ops.ndarray_softmax(x, 1, out)
+    assert torch.allclose(out, torch.full((4, 8), 0.125))
+    red = torch.empty(8)
+    ops.ndarray_reduce(x + 1, "sum", [0], False, red)
+    assert torch.equal(red, torch.full((8,), 4.0))
+    # a kernel without a host twin reached through the NDArray static: the switch itself refuses the host
     with pytest.raises(ops.NotImplemented_):
-        ops.ndarray_softmax(x, 1, out)
-    with pytest.raises(ops.NotImplemented_):
-        ops.ndarray_reduce(x, "sum", [0], False, torch.empty(8))
+        ops.ndarray_layernorm(x, torch.ones(8), torch.zeros(8), 1, 1e-5, True, out)
 
 
 def test_missing_operator_library_fails_loudly(monkeypatch, tmp_path):

@@ -673,6 +673,58 @@ def cpu_baselines(budget_s=1.2):
     return out
 
 
+def stream_sweep(hk, torch, steps=40):
+    """The streaming roof of every read : write mix the kernels have: hipMemcpyAsync device to device, then a kernel
+    that only moves 256 MiB arrays in every launch shape (workgroup size, vectors in flight per thread, non-temporal
+    hints, one-shot grid or a fixed number of workgroups per compute unit).  Prints the table and returns the best
+    shape per mix."""
+    n = 256 << 20
+    bufs = [torch.empty(n, dtype=torch.uint8, device="cuda").fill_(i + 1) for i in range(8)]
+
+    def timed(fn):
+        for i in range(10):
+            fn(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            fn(i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    preroll(torch, lambda i: hk.memcpy_d2d(bufs[(2 * i) % 8], bufs[(2 * i + 1) % 8]))
+    d = timed(lambda i: hk.memcpy_d2d(bufs[(2 * i) % 8], bufs[(2 * i + 1) % 8]))
+    res = {"hipMemcpyAsync device-to-device 256 MiB": {"us": round(d * 1e6, 2), "GBps": round(2 * n / d / 1e9, 1),
+                                                      "frac": round(2 * n / d / 1e9 / HBM_PEAK_GBS, 4)}}
+    print("stream %-8s %-58s %8.2f us %7.1f GB/s %5.1f%%" % ("1R:1W", "hipMemcpyAsync device-to-device", d * 1e6,
+                                                           2 * n / d / 1e9, 2 * n / d / 1e9 / HBM_PEAK_GBS * 100), file=sys.stderr, flush=True)
+    shapes = [(bs, u, ntl, nts, 0) for bs in (64, 128, 256, 512, 1024) for u in (1, 2, 4)
+              for ntl in (0, 1) for nts in (0, 1)]
+    shapes += [(bs, u, 1, 1, w) for bs in (256, 512, 1024) for u in (1, 2, 4) for w in (1, 2, 4, 8)]
+    for nr, nw in ((1, 1), (2, 1), (1, 2), (1, 0), (0, 1)):
+        best = None
+        for bs, u, ntl, nts, w in shapes:
+            if (nr == 0 and ntl) or (nw == 0 and nts):
+                continue
+
+            def fn(i, bs=bs, u=u, ntl=ntl, nts=nts, w=w):
+                o = (4 * i) % 8
+                hk.stream_probe([bufs[(o + 2 + k) % 8] for k in range(nw)], [bufs[(o + k) % 8] for k in range(nr)],
+                                bs, u, bool(ntl), bool(nts), w)
+            d = timed(fn)
+            gbs = (nr + nw) * n / d / 1e9
+            name = "%4d threads x %d vectors, nt loads %d stores %d, %s" % (
+                bs, u, ntl, nts, "one-shot grid" if w == 0 else "%d workgroups per CU" % w)
+            print("stream %-8s %-58s %8.2f us %7.1f GB/s %5.1f%%" % ("%dR:%dW" % (nr, nw), name, d * 1e6, gbs,
+                                                                   gbs / HBM_PEAK_GBS * 100), file=sys.stderr, flush=True)
+            if best is None or gbs > best[0]:
+                best = (gbs, name, d)
+        res["%dR:%dW" % (nr, nw)] = {"best_shape": best[1], "us": round(best[2] * 1e6, 2), "GBps": round(best[0], 1),
+                                     "frac": round(best[0] / HBM_PEAK_GBS, 4)}
+    del bufs
+    torch.cuda.empty_cache()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -741,6 +793,8 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": NORM_BWD_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_us": round(bwd_us, 2)},
     }
+    if args.all and not args.only:
+        out["stream_roof"] = stream_sweep(hk, torch)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     if kernels:

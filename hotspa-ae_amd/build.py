@@ -21,7 +21,7 @@ INCLUDE = os.path.join(ROOT, "include")
 
 HIP_SOURCES = ["hk_norm_bwd_bf16.hip", "hk_norm_bwd_f32.hip", "hk_norm_bwd_f16.hip", "hk_norm_fwd_bf16.hip",
                "hk_norm_fwd_f32.hip", "hk_norm_fwd_f16.hip", "hk_device.hip", "hk_norm.hip", "hk_softmax.hip", "hk_sce.hip", "hk_reduce.hip", "hk_nll.hip",
-               "hk_dropout_ln.hip", "hk_elementwise.hip", "hk_vocab_ce.hip", "hk_batchnorm.hip"]
+               "hk_dropout_ln.hip", "hk_elementwise.hip", "hk_vocab_ce.hip", "hk_batchnorm.hip", "hk_stream_probe.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fvisibility=hidden",

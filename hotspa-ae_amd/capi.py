@@ -540,6 +540,25 @@ def copy_kernel(dst, src, stream=None):
                                stream if stream is not None else current_stream()))
 
 
+def stream_probe(dsts, srcs, block_threads=256, vectors_per_thread=1, nt_loads=True, nt_stores=True,
+                 workgroups_per_cu=0, stream=None):
+    """Streaming yardstick: len(srcs) arrays read, len(dsts) arrays written, all of the first array's size."""
+    ref = (list(srcs) + list(dsts))[0]
+    nbytes = ref.numel() * ref.element_size()
+    d = list(dsts) + [None, None]
+    r = list(srcs) + [None, None]
+    check(lib().hk_stream_probe(_ptr(d[0]), _ptr(d[1]), _ptr(r[0]), _ptr(r[1]), ctypes.c_int(len(srcs)),
+                                ctypes.c_int(len(dsts)), ctypes.c_size_t(nbytes), ctypes.c_int(block_threads),
+                                ctypes.c_int(vectors_per_thread), ctypes.c_int(int(nt_loads)),
+                                ctypes.c_int(int(nt_stores)), ctypes.c_int(workgroups_per_cu),
+                                stream if stream is not None else current_stream()))
+
+
+def memcpy_d2d(dst, src, stream=None):
+    check(lib().hk_memcpy_d2d(_ptr(dst), _ptr(src), ctypes.c_size_t(src.numel() * src.element_size()),
+                              stream if stream is not None else current_stream()))
+
+
 def strided_copy(src, dst, stream=None):
     check(lib().hk_strided_copy(dtype_code(src), _ptr(src), _ptr(dst), ctypes.c_int(src.dim()), _arr(src.shape),
                                 _arr(src.stride()), stream if stream is not None else current_stream()))

@@ -1,0 +1,142 @@
+// Streaming yardstick: a kernel that only moves bytes, NR arrays read and NW arrays written per launch, in every
+// launch shape a row kernel could take (workgroup size, 16-byte vectors in flight per thread, one-shot grid or a
+// fixed number of workgroups per compute unit walking the array, non-temporal hint on the loads and / or the
+// stores).  What the best shape of a mix reaches is the roof the operator kernels with that mix are held against.
+// The hints are template arguments: as run-time flags the compiler merges the two branches into a plain access.
+#include "hk_common.h"
+
+namespace hk {
+
+struct ProbeArgs {
+  const u32x4* src[2];
+  u32x4* dst[2];
+  size_t nvec;
+  uint32_t* sink;
+};
+
+template <int BS, int U, int NR, int NW, bool NTL, bool NTS>
+__global__ __launch_bounds__(BS)
+void stream_probe_kernel(ProbeArgs a) {
+  const size_t tile = size_t(BS) * U;
+  uint32_t acc = 0;
+  // grid-stride over tiles of BS * U vectors; a one-shot launch has one tile per workgroup
+  for (size_t t0 = size_t(blockIdx.x) * tile; t0 < a.nvec; t0 += size_t(gridDim.x) * tile) {
+    const size_t base = t0 + threadIdx.x;
+    u32x4 v[U];
+#pragma unroll
+    for (int i = 0; i < U; ++i) v[i] = u32x4{1u, 2u, 3u, uint32_t(threadIdx.x)};
+    if constexpr (NR >= 1) {
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        const size_t idx = base + size_t(i) * BS;
+        if (idx < a.nvec) v[i] = NTL ? __builtin_nontemporal_load(a.src[0] + idx) : a.src[0][idx];
+      }
+    }
+    if constexpr (NR >= 2) {
+      u32x4 w[U];
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        const size_t idx = base + size_t(i) * BS;
+        w[i] = u32x4{0, 0, 0, 0};
+        if (idx < a.nvec) w[i] = NTL ? __builtin_nontemporal_load(a.src[1] + idx) : a.src[1][idx];
+      }
+#pragma unroll
+      for (int i = 0; i < U; ++i) v[i] ^= w[i];
+    }
+#pragma unroll
+    for (int o = 0; o < NW; ++o) {
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        const size_t idx = base + size_t(i) * BS;
+        if (idx < a.nvec) {
+          if constexpr (NTS) __builtin_nontemporal_store(v[i], a.dst[o] + idx);
+          else a.dst[o][idx] = v[i];
+        }
+      }
+    }
+    if constexpr (NW == 0) {
+#pragma unroll
+      for (int i = 0; i < U; ++i) acc += v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    }
+  }
+  if (NW == 0 && acc == 0x12345678u && a.sink) a.sink[0] = acc;   // keeps the loads of a read-only run alive
+}
+
+template <int BS, int U, int NR, int NW>
+static int probe_nt(const ProbeArgs& a, int ntl, int nts, unsigned grid, hipStream_t s) {
+  if (NR == 0) ntl = 0;
+  if (NW == 0) nts = 0;
+  profile_before(s);
+  if (ntl && nts) hipLaunchKernelGGL((stream_probe_kernel<BS, U, NR, NW, NR != 0, NW != 0>), dim3(grid), dim3(BS), 0, s, a);
+  else if (ntl) hipLaunchKernelGGL((stream_probe_kernel<BS, U, NR, NW, NR != 0, false>), dim3(grid), dim3(BS), 0, s, a);
+  else if (nts) hipLaunchKernelGGL((stream_probe_kernel<BS, U, NR, NW, false, NW != 0>), dim3(grid), dim3(BS), 0, s, a);
+  else hipLaunchKernelGGL((stream_probe_kernel<BS, U, NR, NW, false, false>), dim3(grid), dim3(BS), 0, s, a);
+  profile_after(s);
+  return launch_check("stream_probe_kernel");
+}
+
+template <int BS, int U>
+static int probe_mix(const ProbeArgs& a, int nr, int nw, int ntl, int nts, unsigned grid, hipStream_t s) {
+  if (nr == 1 && nw == 1) return probe_nt<BS, U, 1, 1>(a, ntl, nts, grid, s);
+  if (nr == 2 && nw == 1) return probe_nt<BS, U, 2, 1>(a, ntl, nts, grid, s);
+  if (nr == 1 && nw == 2) return probe_nt<BS, U, 1, 2>(a, ntl, nts, grid, s);
+  if (nr == 1 && nw == 0) return probe_nt<BS, U, 1, 0>(a, ntl, nts, grid, s);
+  if (nr == 0 && nw == 1) return probe_nt<BS, U, 0, 1>(a, ntl, nts, grid, s);
+  set_last_error("hk_stream_probe: no kernel for %d reads : %d writes", nr, nw);
+  return HK_ERR_UNSUPPORTED;
+}
+
+template <int BS>
+static int probe_unroll(const ProbeArgs& a, int unroll, int nr, int nw, int ntl, int nts, unsigned grid, hipStream_t s) {
+  switch (unroll) {
+    case 1: return probe_mix<BS, 1>(a, nr, nw, ntl, nts, grid, s);
+    case 2: return probe_mix<BS, 2>(a, nr, nw, ntl, nts, grid, s);
+    case 4: return probe_mix<BS, 4>(a, nr, nw, ntl, nts, grid, s);
+    default:
+      set_last_error("hk_stream_probe: 1, 2 or 4 vectors per thread, got %d", unroll);
+      return HK_ERR_UNSUPPORTED;
+  }
+}
+
+} // namespace hk
+
+using namespace hk;
+
+extern "C" {
+
+int hk_stream_probe(void* dst0, void* dst1, const void* src0, const void* src1, int reads, int writes, size_t bytes,
+                    int block_threads, int vectors_per_thread, int nt_loads, int nt_stores, int workgroups_per_cu,
+                    hkStream_t stream) {
+  HK_REQUIRE(bytes % 16 == 0 && bytes > 0, HK_ERR_INVALID, "hk_stream_probe: size must be a positive multiple of 16");
+  HK_REQUIRE(reads >= 0 && reads <= 2 && writes >= 0 && writes <= 2 && reads + writes > 0, HK_ERR_INVALID,
+             "hk_stream_probe: 0..2 reads and 0..2 writes, not both 0");
+  HK_REQUIRE((reads < 1 || src0) && (reads < 2 || src1) && (writes < 1 || dst0) && (writes < 2 || dst1),
+             HK_ERR_INVALID, "hk_stream_probe: null array");
+  HK_REQUIRE(aligned16(src0) && aligned16(src1) && aligned16(dst0) && aligned16(dst1), HK_ERR_INVALID,
+             "hk_stream_probe: arrays must be 16-byte aligned");
+  HK_REQUIRE(workgroups_per_cu >= 0 && workgroups_per_cu <= 64, HK_ERR_INVALID,
+             "hk_stream_probe: 0 (one-shot grid) to 64 workgroups per compute unit");
+  ProbeArgs a{};
+  a.src[0] = static_cast<const u32x4*>(src0); a.src[1] = static_cast<const u32x4*>(src1);
+  a.dst[0] = static_cast<u32x4*>(dst0); a.dst[1] = static_cast<u32x4*>(dst1);
+  a.nvec = bytes / 16;
+  a.sink = nullptr;
+  const size_t tile = size_t(block_threads) * size_t(vectors_per_thread > 0 ? vectors_per_thread : 1);
+  const size_t tiles = (a.nvec + tile - 1) / tile;
+  HK_REQUIRE(tiles <= 0x7fffffffu, HK_ERR_INVALID, "hk_stream_probe: size too large");
+  const unsigned grid = workgroups_per_cu == 0 ? unsigned(tiles)
+                                               : unsigned(std::min<size_t>(tiles, size_t(device_cu_count()) * workgroups_per_cu));
+  hipStream_t s = as_hip(stream);
+  switch (block_threads) {
+    case 64: return probe_unroll<64>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
+    case 128: return probe_unroll<128>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
+    case 256: return probe_unroll<256>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
+    case 512: return probe_unroll<512>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
+    case 1024: return probe_unroll<1024>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
+    default:
+      set_last_error("hk_stream_probe: workgroups of 64, 128, 256, 512 or 1024 threads, got %d", block_threads);
+      return HK_ERR_UNSUPPORTED;
+  }
+}
+
+} // extern "C"

@@ -118,6 +118,15 @@ HK_API int hk_profile_next_kernel(hkEvent_t before, hkEvent_t after);
  * calibration reference for bandwidth counters and timings. */
 HK_API int hk_copy_kernel(void* dst, const void* src, size_t bytes, hkStream_t stream);
 
+/* Streaming yardstick (no counterpart in the reference): moves `bytes` per array, `reads` arrays in (0..2) and
+ * `writes` arrays out (0..2), with workgroups of `block_threads` (64 .. 1024), `vectors_per_thread` 16-byte vectors
+ * in flight per thread (1, 2, 4), the non-temporal hint on loads / stores, and either a one-shot grid
+ * (`workgroups_per_cu` 0) or that many workgroups per compute unit walking the arrays.  The best shape of a
+ * read : write mix is the roof the operator kernels with that mix are measured against (bench.py --all). */
+HK_API int hk_stream_probe(void* dst0, void* dst1, const void* src0, const void* src1, int reads, int writes,
+                           size_t bytes, int block_threads, int vectors_per_thread, int nt_loads, int nt_stores,
+                           int workgroups_per_cu, hkStream_t stream);
+
 /* Gathers a strided view into a dense row-major array (what the reference's
  * OffsetCalculator does per element, hetu/impl/utils/offset_calculator.cuh:16-68).
  * shape/strides in elements, ndim <= 8. */

@@ -481,6 +481,8 @@ enum TuneKey {
   TUNE_REDUCE_OUTER_ROW_BLOCKS,
   TUNE_NORM_BWD_ROWS_PER_BLOCK,
   TUNE_NORM_BWD_PREFETCH,
+  TUNE_REDUCE_OUTER_WAVES_ACROSS,
+  TUNE_REDUCE_OUTER_WAVES,
   TUNE_NUM_KEYS
 };
 int tune_get(int key);

@@ -52,6 +52,8 @@ static const char* const kTuneNames[] = {
   "reduce_outer_row_blocks",
   "norm_bwd_rows_per_block",
   "norm_bwd_prefetch",  // rows loaded ahead by the backward kernel (1..3)
+  "reduce_outer_waves_across",  // wavefronts of a column-reduction workgroup side by side across columns
+  "reduce_outer_waves",         // wavefronts of a column-reduction workgroup in all
 };
 constexpr int kNumTune = sizeof(kTuneNames) / sizeof(kTuneNames[0]);
 static_assert(kNumTune == TUNE_NUM_KEYS, "tune name table out of sync with TuneKey");

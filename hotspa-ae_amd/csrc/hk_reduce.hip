@@ -239,6 +239,7 @@ struct OuterArgs {
   int64_t b_stride, r_stride;   // elements
   int64_t rows_per_split;
   int rsplit;
+  int wx;               // wavefronts of a workgroup side by side across columns (the others stack over rows)
   float factor;
   int is_mean;
 };
@@ -248,11 +249,14 @@ __global__ __launch_bounds__(512)
 void reduce_outer_vec_kernel(OuterArgs a) {
   constexpr int VEC = VecIO<T>::N;
   constexpr int U = 8;
-  extern __shared__ float lds[];   // [WY][64 * VEC]
+  extern __shared__ float lds[];   // [WY][WX][VEC][64]
   const int lane = threadIdx.x & 63;
-  const int w = threadIdx.x >> 6;
-  const int wy = blockDim.x >> 6;
-  const int64_t cv = int64_t(blockIdx.x) * kWave + lane;   // column vector index
+  const int wave = wave_index();
+  const int wx = a.wx;
+  const int wc = wave % wx;        // this wavefront's place across columns ...
+  const int w = wave / wx;         // ... and over rows
+  const int wy = int(blockDim.x >> 6) / wx;
+  const int64_t cv = (int64_t(blockIdx.x) * wx + wc) * kWave + lane;   // column vector index
   const int64_t c = cv * VEC;
   const bool col_ok = c < a.C;                              // C is a multiple of VEC here
   const int split = blockIdx.y;
@@ -290,12 +294,12 @@ void reduce_outer_vec_kernel(OuterArgs a) {
   }
   // fold the waves of the block: lane-major layout keeps LDS accesses conflict-free
 #pragma unroll
-  for (int j = 0; j < VEC; ++j) lds[(w * VEC + j) * kWave + lane] = acc[j];
+  for (int j = 0; j < VEC; ++j) lds[((w * wx + wc) * VEC + j) * kWave + lane] = acc[j];
   __syncthreads();
   // thread (w, lane) finishes element j = w, w + wy, ... of its lane's vector
   for (int j = w; j < VEC; j += wy) {
     float s = R::template identity<float>();
-    for (int k = 0; k < wy; ++k) s = R::apply(s, lds[(k * VEC + j) * kWave + lane]);
+    for (int k = 0; k < wy; ++k) s = R::apply(s, lds[((k * wx + wc) * VEC + j) * kWave + lane]);
     if (col_ok) {
       if (a.rsplit == 1)
         st_acc<OUT_T, float>(static_cast<OUT_T*>(a.out) + b * a.C + c + j, R::template post<float>(s, a.factor, a.is_mean));
@@ -466,7 +470,7 @@ static int make_plan(int ndim, const int64_t* shape, const int64_t* strides, int
 }
 
 struct InnerShape { int tpr; int nsplit; int64_t chunk; bool vec; };
-struct OuterShape { int wy; int rsplit; int64_t rows_per_split; bool vec; };
+struct OuterShape { int wy; int wx; int rsplit; int64_t rows_per_split; bool vec; };
 
 template <typename T>
 static InnerShape shape_inner(const ReducePlan& p, const void* in) {
@@ -504,14 +508,21 @@ static OuterShape shape_outer(const ReducePlan& p, const void* in) {
   constexpr int VEC = 16 / sizeof(T);
   OuterShape s{};
   s.vec = aligned16(in) && p.C % VEC == 0 && p.r_stride % VEC == 0 && (p.B == 1 || p.b_stride % VEC == 0);
-  s.wy = 1; s.rsplit = 1; s.rows_per_split = p.R;
+  s.wy = 1; s.wx = 1; s.rsplit = 1; s.rows_per_split = p.R;
   if (!s.vec) return s;
-  const int64_t col_tiles = std::max<int64_t>(1, (p.C / VEC + 63) / 64);
-  // waves per block: enough rows per wave to keep 8 loads in flight; eight wavefronts (512 threads) on one
-  // workgroup per compute unit measured fastest (40.7 us against 42.3 us for sixteen at 32768 x 4096 bf16)
-  int wy = 8;
+  int64_t col_tiles = std::max<int64_t>(1, (p.C / VEC + 63) / 64);
+  // waves per block: enough rows per wave to keep 8 loads in flight
+  // Measured at 32768 x 4096 bf16 (whole call, one workgroup per compute unit): 4 wavefronts 42.5 us, 8 wavefronts
+  // 43.4 us, 16 wavefronts 44.3 us; putting 2, 4 or 8 of them side by side across columns (a workgroup then reads
+  // 2 KiB or more of consecutive bytes per row) changed nothing (43.2 .. 43.5 us), so the default keeps one.
+  int waves = tune_get(TUNE_REDUCE_OUTER_WAVES) > 0 ? std::min(8, tune_get(TUNE_REDUCE_OUTER_WAVES)) : 4;
+  int wx = tune_get(TUNE_REDUCE_OUTER_WAVES_ACROSS) > 0 ? tune_get(TUNE_REDUCE_OUTER_WAVES_ACROSS) : 1;
+  while (wx > 1 && (wx > waves || col_tiles % wx != 0)) wx >>= 1;
+  int wy = waves / wx;
   while (wy > 1 && p.R < int64_t(wy) * 8) wy >>= 1;
   s.wy = wy;
+  s.wx = wx;
+  col_tiles /= wx;
   int rsplit = tune_get(TUNE_REDUCE_OUTER_ROW_BLOCKS);
   if (rsplit <= 0) {
     const int64_t want_blocks = int64_t(device_cu_count());   // one workgroup per CU measured fastest
@@ -596,7 +607,7 @@ static int reduce_fast(const ReducePlan& p, const void* in, void* out, float fac
     constexpr int VEC = 16 / sizeof(T);
     OuterArgs a{};
     a.in = in; a.B = p.B; a.R = p.R; a.C = p.C; a.b_stride = p.b_stride; a.r_stride = p.r_stride;
-    a.rows_per_split = s.rows_per_split; a.rsplit = s.rsplit; a.factor = factor; a.is_mean = is_mean;
+    a.rows_per_split = s.rows_per_split; a.rsplit = s.rsplit; a.wx = s.wx; a.factor = factor; a.is_mean = is_mean;
     if (s.rsplit > 1) {
       const size_t need = size_t(s.rsplit) * p.B * p.C * sizeof(float);
       HK_REQUIRE(ws && ws_bytes >= need, HK_ERR_WORKSPACE, "hk_reduce: workspace of %zu bytes needed, %zu given", need, ws_bytes);
@@ -605,9 +616,9 @@ static int reduce_fast(const ReducePlan& p, const void* in, void* out, float fac
       a.out = out;
     }
     HK_REQUIRE(p.B <= 65535, HK_ERR_UNSUPPORTED, "hk_reduce: batch extent %lld too large for the column kernel", (long long)p.B);
-    const int64_t col_tiles = (p.C / VEC + 63) / 64;
-    dim3 grid(unsigned(col_tiles), unsigned(s.rsplit), unsigned(p.B)), block{unsigned(64 * s.wy)};
-    const size_t lds = size_t(s.wy) * 64 * VEC * sizeof(float);
+    const int64_t col_tiles = ((p.C / VEC + 63) / 64 + s.wx - 1) / s.wx;
+    dim3 grid(unsigned(col_tiles), unsigned(s.rsplit), unsigned(p.B)), block{unsigned(64 * s.wy * s.wx)};
+    const size_t lds = size_t(s.wy) * s.wx * 64 * VEC * sizeof(float);
     profile_before(st);
     hipLaunchKernelGGL((reduce_outer_vec_kernel<T, OUT_T, R>), grid, block, lds, st, a);
     profile_after(st);

@@ -9,17 +9,23 @@
 
 namespace hk {
 
-// T: element type; NV: 16-byte vectors per thread; WAVE_ROW: one wavefront per
-// row (4 rows per 256-thread block) instead of one workgroup per row;
-// HAS_RES: x = x0 + residual is formed in fp32 and optionally written back.
+// T: element type; NV: 16-byte vectors per thread; WAVE_ROW: one wavefront per row (4 rows per 256-thread block)
+// instead of one workgroup per row; HAS_RES: x = x0 + residual is formed in fp32 and optionally written back;
+// IS_RMS: RMSNorm (no centring, no bias term in the statistics).
 //
 // Every row operand is addressed through a buffer descriptor of exactly one row (base = the row's first byte,
 // size = cols * sizeof(T)): the hardware returns zeros for a lane past the row's end and drops its stores, so no
 // memory instruction sits inside a branch and all of a thread's loads are issued back to back.
-template <typename T, int NV, bool WAVE_ROW, bool HAS_RES>
+//
+// The row is unpacked to fp32 registers once (at most 64 per thread) and, for LayerNorm, centred in place by the
+// second statistics pass, so the normalisation costs one multiply and one multiply-add per element.  Which values
+// stay in registers across the reductions is written out here rather than left to the compiler: with the row kept
+// packed and unpacked again per pass, unrelated edits moved the 5120-column bf16 kernel between 57.7 and 61 us.
+template <typename T, int NV, bool WAVE_ROW, bool HAS_RES, bool IS_RMS>
 __global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
 void norm_fwd_kernel(NormFwdArgs a) {
   constexpr int VEC = VecIO<T>::N;
+  constexpr int NE = NV * VEC;
   __shared__ float red[kMaxWaves * 3];
 
   const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
@@ -31,113 +37,88 @@ void norm_fwd_kernel(NormFwdArgs a) {
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
   const uint32_t row_bytes = uint32_t(a.nvec) * 16u;
   auto off = [&](int i) { return uint32_t(i * tpr + t) * 16u; };   // vector i of thread t, in bytes from the row's start
+  // long rows: stops the scheduler from unpacking every vector of a pass before the first one is consumed
+  auto fence = [] { if constexpr (NV >= 8) __builtin_amdgcn_sched_barrier(0); };
 
-  const BufferRsrc xr = make_rsrc(static_cast<const T*>(a.x) + row * a.x_pitch, row_bytes);
-  u32x4 raw[NV];
+  float v[NE];
+  {
+    const BufferRsrc xr = make_rsrc(static_cast<const T*>(a.x) + row * a.x_pitch, row_bytes);
+    u32x4 raw[NV];
 #pragma unroll
-  for (int i = 0; i < NV; ++i) raw[i] = buf_ld16<kBufStream>(xr, off(i));
-  [[maybe_unused]] float xf[HAS_RES ? NV * VEC : 1];
-  if constexpr (HAS_RES) {
-    const BufferRsrc rr = make_rsrc(static_cast<const T*>(a.residual) + row * a.res_pitch, row_bytes);
-    u32x4 res[NV];
+    for (int i = 0; i < NV; ++i) raw[i] = buf_ld16<kBufStream>(xr, off(i));
+    if constexpr (HAS_RES) {
+      const BufferRsrc rr = make_rsrc(static_cast<const T*>(a.residual) + row * a.res_pitch, row_bytes);
+      u32x4 res[NV];
 #pragma unroll
-    for (int i = 0; i < NV; ++i) res[i] = buf_ld16<kBufStream>(rr, off(i));
-    // an absent x_out becomes an empty buffer: its stores are dropped by the bounds check
-    const BufferRsrc xo = make_rsrc(a.x_out ? static_cast<T*>(a.x_out) + row * a.xout_pitch : static_cast<T*>(a.y),
-                                    a.x_out ? row_bytes : 0u);
+      for (int i = 0; i < NV; ++i) res[i] = buf_ld16<kBufStream>(rr, off(i));
+      // an absent x_out becomes an empty buffer: its stores are dropped by the bounds check
+      const BufferRsrc xo = make_rsrc(a.x_out ? static_cast<T*>(a.x_out) + row * a.xout_pitch : static_cast<T*>(a.y),
+                                      a.x_out ? row_bytes : 0u);
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      float f0[VEC], f1[VEC];
-      VecIO<T>::unpack(raw[i], f0);
-      VecIO<T>::unpack(res[i], f1);
+      for (int i = 0; i < NV; ++i) {
+        float f1[VEC];
+        VecIO<T>::unpack(raw[i], &v[i * VEC]);
+        VecIO<T>::unpack(res[i], f1);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) xf[i * VEC + j] = f0[j] + f1[j];
-      buf_st16<kBufStream>(xo, off(i), VecIO<T>::pack(&xf[i * VEC]));
+        for (int j = 0; j < VEC; ++j) v[i * VEC + j] += f1[j];
+        buf_st16<kBufStream>(xo, off(i), VecIO<T>::pack(&v[i * VEC]));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) { fence(); VecIO<T>::unpack(raw[i], &v[i * VEC]); }
     }
   }
 
-  // The row stays packed between the passes over it (4 registers per vector, not one per element): the empty
-  // statement makes the packed words opaque, so the next pass unpacks them again instead of keeping the floats
-  // of the previous one alive.
-  auto repack = [&]() {
-    if constexpr (!HAS_RES && VEC > 4) {
-#pragma unroll
-      for (int i = 0; i < NV; ++i) asm volatile("" : "+v"(raw[i]));
-    }
-  };
-  // long rows: stops the scheduler from unpacking every vector of a pass before the first one is consumed
-  auto fence = [] { if constexpr (NV >= 8) __builtin_amdgcn_sched_barrier(0); };
-  auto get = [&](int i, float* f) {
-    if constexpr (HAS_RES) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) f[j] = xf[i * VEC + j];
-    } else {
-      VecIO<T>::unpack(raw[i], f);
-    }
+  // sums over the group of threads that holds the row; the two reductions of a kernel use separate LDS slots,
+  // so no barrier is needed between them
+  auto allred = [&](float x, int slot) -> float {
+    SumTuple<1> s;
+    s.v[0] = x;
+    s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red + slot * kMaxWaves, 0, nwaves);
+    return s.v[0];
   };
 
   float mu, rs, var;
-  if (a.is_rms) {
+  if constexpr (IS_RMS) {
     // lanes past the row's end hold zeros, which add nothing to either sum
-    SumTuple<2> s;
-    s.v[0] = 0.f; s.v[1] = 0.f;
+    float s0 = 0.f, ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      float f[VEC];
-      fence();
-      get(i, f);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) { s.v[0] += f[j]; s.v[1] = fmaf(f[j], f[j], s.v[1]); }
-    }
-    s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red, 0, nwaves);
-    mu = s.v[0] * a.inv_cols;
-    const float ms = s.v[1] * a.inv_cols;  // mean(x^2) = var + mu^2
+    for (int e = 0; e < NE; ++e) { s0 += v[e]; ss = fmaf(v[e], v[e], ss); }
+    const float ms = allred(ss, 0) * a.inv_cols;   // mean(x^2) = var + mu^2
+    mu = allred(s0, 1) * a.inv_cols;
     var = fmaxf(ms - mu * mu, 0.f);
     rs = 1.0f / sqrtf(ms + a.eps);
   } else {
-    // Welford statistics, merged with Chan's parallel update: each thread forms (count, mean, M2) of the
-    // elements it holds in registers, lanes merge through a DPP butterfly, waves through LDS.  When every
-    // thread holds the same count (the row fills all vector slots: a uniform test) each butterfly step
-    // merges equal-sized halves and needs no reciprocal; a ragged row takes the general update.
+    // Two passes over the registers: the mean first, then the sum of squares about it, each reduced over the
+    // group.  Centring on the row's own mean keeps fp32 accuracy for rows with an outlier, a large common offset
+    // or no variance at all.  The centred values replace the row in the registers.
     float s = 0.f;
-    int cnt = 0;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      float f[VEC];
-      fence();
-      get(i, f);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) s += f[j];            // zeros past the end
-      cnt += (i * tpr + t < a.nvec) ? VEC : 0;
-    }
-    repack();
-    const bool even = a.nvec == NV * tpr;                    // uniform
-    const float mean_t = even ? s * (1.0f / float(NV * VEC)) : (cnt > 0 ? s / float(cnt) : 0.f);
+    for (int e = 0; e < NE; ++e) s += v[e];            // zeros past the end
+    mu = allred(s, 0) * a.inv_cols;
     float m2 = 0.f;
+    if (a.nvec == NV * tpr) {                            // uniform: the row fills every lane's every vector
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      float f[VEC];
-      fence();
-      get(i, f);
-      float q = 0.f;
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) { const float d = f[j] - mean_t; q = fmaf(d, d, q); }
-      m2 += (even || i * tpr + t < a.nvec) ? q : 0.f;
-    }
-    MomentTuple m;
-    m.v[0] = float(cnt); m.v[1] = mean_t; m.v[2] = m2;
-    if (even) {
-      EqualMomentTuple e;
-      e.v[0] = m.v[0]; e.v[1] = m.v[1]; e.v[2] = m.v[2];
-      e = wave_allreduce_tuple(e);
-      m.v[0] = e.v[0]; m.v[1] = e.v[1]; m.v[2] = e.v[2];
+      for (int e = 0; e < NE; ++e) {
+        v[e] -= mu;
+        m2 = fmaf(v[e], v[e], m2);
+      }
     } else {
-      m = wave_allreduce_tuple(m);
+      // a lane past the row's end holds -mu, not data: its vectors are left out.  Kept apart from the full-row
+      // case, whose straight-line code the per-vector selects would break up (57.8 against 61 us at 5120 bf16
+      // columns).
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        float q = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          v[i * VEC + j] -= mu;
+          q = fmaf(v[i * VEC + j], v[i * VEC + j], q);
+        }
+        m2 += (i * tpr + t < a.nvec) ? q : 0.f;
+      }
     }
-    // waves are merged one after the other (growing count on one side): the general update
-    if (!WAVE_ROW) m = group_combine_tuple(m, red, 0, nwaves);
-    mu = m.v[1];
-    var = m.v[2] * a.inv_cols;
+    var = allred(m2, 1) * a.inv_cols;
     rs = 1.0f / sqrtf(var + a.eps);
   }
 
@@ -146,14 +127,11 @@ void norm_fwd_kernel(NormFwdArgs a) {
     store_stat<T>(a.stat, row, a.stat_kind == HK_STAT_VAR ? var : rs, a.stats_f32);
   }
 
-  repack();
-  const float shift = a.is_rms ? 0.f : mu;
   const BufferRsrc yr = make_rsrc(static_cast<T*>(a.y) + row * a.y_pitch, row_bytes);
   // gamma / beta are fetched after the reduction: every fetch is a miss in the compute unit's own cache (the
   // rows stream through it) and holds one of its outstanding-request slots until the data is back; issued
   // before the row has arrived they would hold those slots for the whole HBM latency instead of the L2's.
-  // The four cases of missing parameters are separate straight-line copies, so that no fetch sits inside a
-  // branch; the compiler is free to issue all of a thread's fetches together.
+  // The four cases of missing parameters are separate straight-line copies, so that no fetch sits inside a branch.
   auto epilogue = [&](auto has_g, auto has_b) {
     constexpr bool HG = decltype(has_g)::value, HB = decltype(has_b)::value;
     const BufferRsrc gr = make_rsrc(HG ? a.gamma : a.y, row_bytes);   // an absent parameter is not fetched at all
@@ -162,18 +140,17 @@ void norm_fwd_kernel(NormFwdArgs a) {
     for (int i = 0; i < NV; ++i) {
       float f[VEC];
       [[maybe_unused]] float g[VEC], b[VEC];
-      get(i, f);
       if constexpr (HG) VecIO<T>::unpack(buf_ld16<kBufKeep>(gr, off(i)), g);
       if constexpr (HB) VecIO<T>::unpack(buf_ld16<kBufKeep>(br, off(i)), b);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        const float n = rs * (f[j] - shift);
+        const float n = rs * v[i * VEC + j];
         f[j] = HG ? (HB ? fmaf(g[j], n, b[j]) : g[j] * n) : (HB ? n + b[j] : n);
       }
       buf_st16<kBufStream>(yr, off(i), VecIO<T>::pack(f));
       // long rows: keep the compiler from hoisting every parameter fetch above the first store, which would
       // hold 2 * NV more vectors in registers than the row itself
-      if constexpr (NV >= 8) __builtin_amdgcn_sched_barrier(0);
+      fence();
     }
   };
   if (a.gamma && a.beta) epilogue(std::true_type{}, std::true_type{});
@@ -247,21 +224,22 @@ void norm_fwd_generic_kernel(NormFwdArgs a) {
   }
 }
 
-template <typename T, bool WAVE_ROW, bool HAS_RES>
-static int launch_norm_fwd_nv(const NormFwdArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
+template <typename T, bool WAVE_ROW, bool HAS_RES, bool IS_RMS>
+static int launch_norm_fwd_rms(const NormFwdArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
   profile_before(s);
   switch (nv) {
-    case 1: hipLaunchKernelGGL((norm_fwd_kernel<T, 1, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
-    case 2: hipLaunchKernelGGL((norm_fwd_kernel<T, 2, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
-    case 3: hipLaunchKernelGGL((norm_fwd_kernel<T, 3, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
-    case 4: hipLaunchKernelGGL((norm_fwd_kernel<T, 4, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
-    case 5: hipLaunchKernelGGL((norm_fwd_kernel<T, 5, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
-    case 6: hipLaunchKernelGGL((norm_fwd_kernel<T, 6, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
-    case 8: hipLaunchKernelGGL((norm_fwd_kernel<T, 8, WAVE_ROW, HAS_RES>), grid, block, 0, s, a); break;
+    case 1: hipLaunchKernelGGL((norm_fwd_kernel<T, 1, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 2: hipLaunchKernelGGL((norm_fwd_kernel<T, 2, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 3: hipLaunchKernelGGL((norm_fwd_kernel<T, 3, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 4: hipLaunchKernelGGL((norm_fwd_kernel<T, 4, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 5: hipLaunchKernelGGL((norm_fwd_kernel<T, 5, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 6: hipLaunchKernelGGL((norm_fwd_kernel<T, 6, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 8: hipLaunchKernelGGL((norm_fwd_kernel<T, 8, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
     case 16:
-      // only the fp32 row without a residual fits sixteen vectors into a 1024-thread workgroup's registers
-      if constexpr (sizeof(T) == 4 && !HAS_RES && !WAVE_ROW) {
-        hipLaunchKernelGGL((norm_fwd_kernel<T, 16, WAVE_ROW, HAS_RES>), grid, block, 0, s, a);
+      // sixteen vectors are 64 fp32 registers only for fp32 data; with a residual two packed rows of that length
+      // are in flight on top
+      if constexpr (sizeof(T) == 4 && !WAVE_ROW && !HAS_RES) {
+        hipLaunchKernelGGL((norm_fwd_kernel<T, 16, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a);
         break;
       }
       [[fallthrough]];
@@ -271,6 +249,12 @@ static int launch_norm_fwd_nv(const NormFwdArgs& a, int nv, dim3 grid, dim3 bloc
   }
   profile_after(s);
   return launch_check("norm_fwd_kernel");
+}
+
+template <typename T, bool WAVE_ROW, bool HAS_RES>
+static int launch_norm_fwd_nv(const NormFwdArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
+  return a.is_rms ? launch_norm_fwd_rms<T, WAVE_ROW, HAS_RES, true>(a, nv, grid, block, s)
+                  : launch_norm_fwd_rms<T, WAVE_ROW, HAS_RES, false>(a, nv, grid, block, s);
 }
 
 // Picks threads-per-row and vectors-per-thread for a row of `nvec` 16-byte
@@ -340,9 +324,9 @@ int norm_fwd_typed(NormFwdArgs a, hipStream_t s) {
   int threads = 0, nv = 0;
   a.nvec = a.cols / VEC;
   const bool has_res = a.residual != nullptr;
-  // with a residual the summed row is kept unpacked: halve the budget; sixteen vectors of a 16-bit type (one
-  // 1024-thread workgroup on more than 65536 columns) do not fit the 128 registers such a workgroup leaves a thread
-  const int max_nv = has_res ? 8 : (VEC == 4 ? 16 : 8);
+  // the row is held as at most 64 fp32 registers per thread (and at most 8 vectors when a residual row is in
+  // flight next to it)
+  const int max_nv = has_res ? std::min(8, 64 / VEC) : 64 / VEC;
   const int wave_nv = has_res ? (VEC == 4 ? 8 : 4) : (VEC == 4 ? 16 : 8);
   if (vec_ok && pick_row_shape(a.nvec, tune_get(TUNE_NORM_FWD_THREADS), max_nv, wave_nv, &threads, &nv)) {
     if (threads == 64) {

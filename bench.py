@@ -103,6 +103,34 @@ def case_rmsnorm(hk, torch, nsets, which):
     return (lambda i: (fwd(i), bwd(i))), fwd_bytes + bwd_bytes, rows
 
 
+def case_rmsnorm_pitched(hk, torch, nsets, which):
+    """The headline shape as a column slice of a wider buffer: rows of 4096 bf16 columns lying 4608 apart, inputs and
+    outputs alike.  The kernels take the pitch; nothing is copied."""
+    rows, cols, wide, eps = 32768, 4096, 4608, 1e-6
+    bf = torch.bfloat16
+    sets = []
+    for i in range(nsets):
+        big = {k: torch.empty((rows, wide), dtype=bf, device="cuda") for k in ("x", "dz", "z", "dx")}
+        big["x"][:, :cols] = _randn(torch, (rows, cols), bf, 1.0, 402 + 10 * i)
+        big["dz"][:, :cols] = _randn(torch, (rows, cols), bf, 1.0, 404 + 10 * i)
+        s = {k: v[:, 256:256 + cols] if k in ("z", "dx") else v[:, :cols] for k, v in big.items()}
+        s["mu"], s["rs"] = torch.empty(rows, device="cuda"), torch.empty(rows, device="cuda")
+        sets.append(s)
+    w = _uniform(torch, (cols,), bf, 0.8, 1.2, 403)
+    dg, db = torch.empty_like(w), torch.empty_like(w)
+    ws = torch.empty(max(1, hk.norm_bwd_workspace_bytes(8, rows, cols) // 4), device="cuda")
+    for s in sets:
+        hk.dropout_add_ln_fwd(s["x"], None, w, None, s["z"], None, s["mu"], s["rs"], eps, True)
+    if which == "fwd":
+        return (lambda i: hk.dropout_add_ln_fwd(sets[i % nsets]["x"], None, w, None, sets[i % nsets]["z"], None,
+                                                sets[i % nsets]["mu"], sets[i % nsets]["rs"], eps, True)), \
+            2 * rows * cols * 2 + cols * 2 + rows * 8, rows
+    return (lambda i: hk.dropout_add_ln_bwd(sets[i % nsets]["dz"], None, sets[i % nsets]["x"], sets[i % nsets]["mu"],
+                                            sets[i % nsets]["rs"], w, sets[i % nsets]["dx"], None, dg, db, True,
+                                            workspace=ws)), \
+        3 * rows * cols * 2 + rows * 4 + cols * 2 + 2 * cols * 2, rows
+
+
 def case_layernorm(hk, torch, nsets, which, cfg):
     if cfg == "C1":
         rows, cols, dt, eps = 8192, 4096, torch.float32, 1e-5
@@ -279,12 +307,17 @@ def case_batch_norm(hk, torch, nsets, which):
     ws = torch.empty(hk.batch_norm_workspace_bytes(xs[0]) // 4 + 4, device="cuda")
     hk.batch_norm_fwd(xs[0], scale, bias, ys[0], 0.1, 1e-5, rm, rv, sm, si, workspace=ws)
     if which == "fwd":
-        return (lambda i: hk.batch_norm_fwd(xs[i % 2], scale, bias, ys[i % 2], 0.1, 1e-5, rm, rv, sm, si,
-                                            workspace=ws)), 3 * n * 2, 256
+        def launch(i):
+            hk.batch_norm_fwd(xs[i % 2], scale, bias, ys[i % 2], 0.1, 1e-5, rm, rv, sm, si, workspace=ws)
+        launch.main_bytes = 2 * n * 2      # the element-wise pass alone: x read, y written
+        return launch, 3 * n * 2, 256
     dys = [_randn(torch, shape, bf, 1.0, 825 + i) for i in range(2)]
     ds, db = torch.empty(256, device="cuda"), torch.empty(256, device="cuda")
-    return (lambda i: hk.batch_norm_bwd(dys[i % 2], xs[i % 2], scale, ys[i % 2], ds, db, sm, si,
-                                        workspace=ws)), 5 * n * 2, 256
+
+    def launch(i):
+        hk.batch_norm_bwd(dys[i % 2], xs[i % 2], scale, ys[i % 2], ds, db, sm, si, workspace=ws)
+    launch.main_bytes = 3 * n * 2          # the element-wise pass alone: dy and x read, dx written
+    return launch, 5 * n * 2, 256
 
 
 def case_reduce(hk, torch, nsets, axes, op, three_d=False):
@@ -467,6 +500,10 @@ CASES = [
     ("C3 reduce sum axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "sum")),
     ("C3 reduce mean axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "mean")),
     ("C3 reduce sum axes(0,1) bf16 [64x512x4096]", lambda hk, t, n: case_reduce(hk, t, n, (0, 1), "sum", True)),
+    ("next: rmsnorm fwd bf16 on a [32768x4096] slice of [32768x4608] (row-pitched in and out)",
+     lambda hk, t, n: case_rmsnorm_pitched(hk, t, n, "fwd")),
+    ("next: rmsnorm bwd bf16 on a [32768x4096] slice of [32768x4608] (row-pitched in and out)",
+     lambda hk, t, n: case_rmsnorm_pitched(hk, t, n, "bwd")),
     ("next: reduce max axis0 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (0,), "max")),
     ("next: reduce max axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "max")),
     ("next: reduce prod axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "prod")),
@@ -770,7 +807,7 @@ def main():
             main_us = kms * 1000
         rec = {"case": name, "us": round(kms * 1000, 2), "main_kernel_us": round(main_us, 2),
                "GBps": round(nbytes / kms / 1e6, 1), "frac": round(nbytes / kms / 1e6 / HBM_PEAK_GBS, 4),
-               "main_kernel_frac": round(nbytes / main_us / 1e3 / HBM_PEAK_GBS, 4),
+               "main_kernel_frac": round(getattr(launch, "main_bytes", nbytes) / main_us / 1e3 / HBM_PEAK_GBS, 4),
                "rows_per_s": round(nrows / kms * 1e3), "bytes": nbytes}
         kernels.append(rec)
         print("%-46s %9.2f us (main %8.2f us) %8.1f GB/s  %5.1f%% (main %5.1f%%)" % (

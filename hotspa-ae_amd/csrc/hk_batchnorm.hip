@@ -431,8 +431,9 @@ static int bn_check(const char* who, int dtype, int64_t N, int64_t C, int64_t HW
   HK_REQUIRE(N >= 0 && C >= 0 && HW >= 0, HK_ERR_INVALID, "%s: negative shape", who);
   HK_REQUIRE(dtype == HK_FLOAT32 || dtype == HK_BFLOAT16 || dtype == HK_FLOAT16 || dtype == HK_FLOAT64,
              HK_ERR_UNSUPPORTED, "%s: not implemented for dtype %d", who, dtype);
+  *need = 0;
+  if (N * C * HW == 0) return HK_OK;   // before the split plan, which divides by C
   *need = bn_ws_bytes(N, C, HW, dtype == HK_FLOAT64 ? 8 : 4);
-  if (N * C * HW == 0) return HK_OK;
   HK_REQUIRE(ws != nullptr && ws_bytes >= *need, HK_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given",
              who, *need, ws_bytes);
   HK_REQUIRE(aligned16(ws), HK_ERR_INVALID, "%s: workspace must be 16-byte aligned", who);

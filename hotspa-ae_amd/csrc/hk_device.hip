@@ -2,6 +2,8 @@
 // utility kernels (fill, streaming copy, strided gather) and the tuning table.
 #include "hk_common.h"
 
+#include <atomic>
+
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -57,9 +59,10 @@ static const char* const kTuneNames[] = {
 };
 constexpr int kNumTune = sizeof(kTuneNames) / sizeof(kTuneNames[0]);
 static_assert(kNumTune == TUNE_NUM_KEYS, "tune name table out of sync with TuneKey");
-static int g_tune[kNumTune] = {0};
+// process-wide; written by hk_tune_set from any thread, read by every launch plan: relaxed atomics
+static std::atomic<int> g_tune[kNumTune];
 
-int tune_get(int key) { return (key >= 0 && key < kNumTune) ? g_tune[key] : 0; }
+int tune_get(int key) { return (key >= 0 && key < kNumTune) ? g_tune[key].load(std::memory_order_relaxed) : 0; }
 
 // Compute-unit count of the current device, cached per device index.
 int device_cu_count() {
@@ -310,7 +313,7 @@ int hk_tune_set(const char* key, int value) {
   HK_REQUIRE(key, HK_ERR_INVALID, "hk_tune_set: null key");
   for (int i = 0; i < kNumTune; ++i) {
     if (std::strcmp(key, kTuneNames[i]) == 0) {
-      g_tune[i] = value;
+      g_tune[i].store(value, std::memory_order_relaxed);
       return HK_OK;
     }
   }

@@ -103,8 +103,10 @@ HK_API int hk_event_query(hkEvent_t event, int* done);
 /* nanoseconds from `start` to `stop` (CUDAEvent::TimeSince, CUDAStream.h:96-109) */
 HK_API int hk_event_elapsed_ns(hkEvent_t start, hkEvent_t stop, int64_t* ns);
 
-/* Launch-shape overrides for tuning sweeps; key names are listed in
- * hk_tune_keys().  value 0 restores the automatic choice. */
+/* Debugging / tuning hook, not part of the operator interface: launch-shape overrides for sweeps (bench.py,
+ * profiling).  The values are process-wide (every device, every stream, every thread sees them; they are read
+ * atomically) and change performance only, never results.  Key names are listed in hk_tune_keys(); value 0
+ * restores the automatic choice.  A deployment leaves them alone. */
 HK_API int hk_tune_set(const char* key, int value);
 HK_API const char* hk_tune_keys(void);
 

@@ -353,10 +353,10 @@ static int bn_fwd_typed(const void* x, const void* scale, const void* bias, void
     CT* coef = part + size_t(C) * size_t(s.splits) * 3;
     HK_REQUIRE(C <= 0x7fffffffLL && (N * C * s.hw_vec + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID,
                "hk_batch_norm_fwd: array too large");
-    hipLaunchKernelGGL((bn_stats_kernel<T, V, CT>), dim3(unsigned(C), unsigned(s.splits)), dim3(256), 0, st, xp, s, part);
+    HK_LAUNCH((bn_stats_kernel<T, V, CT>), dim3(unsigned(C), unsigned(s.splits)), dim3(256), 0, st, xp, s, part);
     int rc = launch_check("bn_stats_kernel");
     if (rc != HK_OK) return rc;
-    hipLaunchKernelGGL((bn_finalize_kernel<PT, CT>), dim3(unsigned((C + 255) / 256)), dim3(256), 0, st, part, C,
+    HK_LAUNCH((bn_finalize_kernel<PT, CT>), dim3(unsigned((C + 255) / 256)), dim3(256), 0, st, part, C,
                        s.splits, static_cast<const PT*>(scale), static_cast<const PT*>(bias), momentum, eps,
                        static_cast<PT*>(running_mean), static_cast<PT*>(running_var), static_cast<PT*>(save_mean),
                        static_cast<PT*>(save_invstd), coef);
@@ -365,10 +365,10 @@ static int bn_fwd_typed(const void* x, const void* scale, const void* bias, void
     const int64_t loads = N * C * s.hw_vec;
     profile_before(st);
     if (loads < 0x7fffffffLL) {
-      hipLaunchKernelGGL((bn_apply_kernel<T, V, CT, uint32_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st,
+      HK_LAUNCH((bn_apply_kernel<T, V, CT, uint32_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st,
                          xp, yp, coef, uint32_t(loads), uint32_t(s.hw_vec), uint32_t(C));
     } else {
-      hipLaunchKernelGGL((bn_apply_kernel<T, V, CT, int64_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st,
+      HK_LAUNCH((bn_apply_kernel<T, V, CT, int64_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st,
                          xp, yp, coef, loads, s.hw_vec, C);
     }
     profile_after(st);
@@ -396,12 +396,12 @@ static int bn_bwd_typed(const void* dy, const void* x, const void* scale, void* 
     CT* coef = part + size_t(C) * size_t(s.splits) * 3;
     HK_REQUIRE(C <= 0x7fffffffLL && (N * C * s.hw_vec + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID,
                "hk_batch_norm_bwd: array too large");
-    hipLaunchKernelGGL((bn_bwd_stats_kernel<T, V, PT, CT>), dim3(unsigned(C), unsigned(s.splits)), dim3(256), 0, st,
+    HK_LAUNCH((bn_bwd_stats_kernel<T, V, PT, CT>), dim3(unsigned(C), unsigned(s.splits)), dim3(256), 0, st,
                        static_cast<const T*>(dy), static_cast<const T*>(x), s, static_cast<const PT*>(save_mean),
                        static_cast<const PT*>(save_invstd), part);
     int rc = launch_check("bn_bwd_stats_kernel");
     if (rc != HK_OK) return rc;
-    hipLaunchKernelGGL((bn_bwd_finalize_kernel<PT, CT>), dim3(unsigned((C + 255) / 256)), dim3(256), 0, st, part, C,
+    HK_LAUNCH((bn_bwd_finalize_kernel<PT, CT>), dim3(unsigned((C + 255) / 256)), dim3(256), 0, st, part, C,
                        s.splits, CT(N * HW), static_cast<const PT*>(scale), static_cast<const PT*>(save_mean),
                        static_cast<const PT*>(save_invstd), static_cast<PT*>(dscale), static_cast<PT*>(dbias), coef);
     rc = launch_check("bn_bwd_finalize_kernel");
@@ -409,11 +409,11 @@ static int bn_bwd_typed(const void* dy, const void* x, const void* scale, void* 
     const int64_t loads = N * C * s.hw_vec;
     profile_before(st);
     if (loads < 0x7fffffffLL) {
-      hipLaunchKernelGGL((bn_bwd_apply_kernel<T, V, CT, uint32_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0,
+      HK_LAUNCH((bn_bwd_apply_kernel<T, V, CT, uint32_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0,
                          st, static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<T*>(dx), coef,
                          uint32_t(loads), uint32_t(s.hw_vec), uint32_t(C));
     } else {
-      hipLaunchKernelGGL((bn_bwd_apply_kernel<T, V, CT, int64_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0,
+      HK_LAUNCH((bn_bwd_apply_kernel<T, V, CT, int64_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0,
                          st, static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<T*>(dx), coef, loads,
                          s.hw_vec, C);
     }

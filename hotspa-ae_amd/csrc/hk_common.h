@@ -7,6 +7,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <type_traits>
 #include <utility>
 #include <stdint.h>
@@ -500,9 +501,22 @@ inline size_t dtype_size(int dtype) {
 
 int launch_check(const char* what);
 
-// Brackets the main kernel of an operator with the events armed through
-// hk_profile_next_kernel(); no-ops when nothing is armed.
+// Timing of an operator's main kernel with the events armed through hk_profile_next_kernel().  profile_before()
+// hands the armed pair to the next HK_LAUNCH made by this thread, which binds both events to that very dispatch
+// (hipExtLaunchKernelGGL): their difference is the kernel's own begin-to-end time, as a kernel trace reports it,
+// without the few microseconds between an event marker on the stream and the kernel's start.  profile_after()
+// drops a pair that no launch took (an early error return).  All three are no-ops when nothing is armed.
 void profile_before(hipStream_t s);
 void profile_after(hipStream_t s);
+bool profile_claim(hipEvent_t* before, hipEvent_t* after);
+
+#define HK_LAUNCH(kernel, grid, block, lds_bytes, stream, ...)                                                  \
+  do {                                                                                                          \
+    hipEvent_t hk_ev_before_, hk_ev_after_;                                                                     \
+    if (::hk::profile_claim(&hk_ev_before_, &hk_ev_after_))                                                     \
+      hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, hk_ev_before_, hk_ev_after_, 0, __VA_ARGS__); \
+    else                                                                                                        \
+      hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, __VA_ARGS__);                                  \
+  } while (0)
 
 } // namespace hk

@@ -31,14 +31,25 @@ int launch_check(const char* what) {
   return HK_OK;
 }
 
-static thread_local hipEvent_t g_prof_before = nullptr;
+static thread_local hipEvent_t g_prof_before = nullptr;   // armed by hk_profile_next_kernel()
 static thread_local hipEvent_t g_prof_after = nullptr;
+static thread_local hipEvent_t g_pend_before = nullptr;   // handed to the next HK_LAUNCH by profile_before()
+static thread_local hipEvent_t g_pend_after = nullptr;
 
-void profile_before(hipStream_t s) {
-  if (g_prof_before) { (void)hipEventRecord(g_prof_before, s); g_prof_before = nullptr; }
+void profile_before(hipStream_t) {
+  g_pend_before = g_prof_before;
+  g_pend_after = g_prof_after;
+  g_prof_before = g_prof_after = nullptr;
 }
-void profile_after(hipStream_t s) {
-  if (g_prof_after) { (void)hipEventRecord(g_prof_after, s); g_prof_after = nullptr; }
+void profile_after(hipStream_t) {
+  g_pend_before = g_pend_after = nullptr;
+}
+bool profile_claim(hipEvent_t* before, hipEvent_t* after) {
+  if (!g_pend_before || !g_pend_after) return false;
+  *before = g_pend_before;
+  *after = g_pend_after;
+  g_pend_before = g_pend_after = nullptr;
+  return true;
 }
 
 // ---------------------------------------------------------------------------
@@ -238,7 +249,7 @@ int hk_memset(void* dst, int value, size_t bytes, hkStream_t stream) {
   size_t blocks = (nvec + 255) / 256;
   HK_REQUIRE(blocks <= 0x7fffffffu, HK_ERR_INVALID, "hk_memset: size too large");
   profile_before(as_hip(stream));
-  hipLaunchKernelGGL(fill_bytes_kernel, dim3(unsigned(blocks)), dim3(256), 0, as_hip(stream),
+  HK_LAUNCH(fill_bytes_kernel, dim3(unsigned(blocks)), dim3(256), 0, as_hip(stream),
                      static_cast<uint8_t*>(dst), word, bytes);
   profile_after(as_hip(stream));
   return launch_check("fill_bytes_kernel");
@@ -343,7 +354,7 @@ int hk_copy_kernel(void* dst, const void* src, size_t bytes, hkStream_t stream) 
   size_t blocks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
   HK_REQUIRE(blocks <= 0x7fffffffu, HK_ERR_INVALID, "hk_copy_kernel: size too large");
   profile_before(as_hip(stream));
-  hipLaunchKernelGGL(copy16_kernel<UNROLL>, dim3(unsigned(blocks)), dim3(256), 0, as_hip(stream),
+  HK_LAUNCH(copy16_kernel<UNROLL>, dim3(unsigned(blocks)), dim3(256), 0, as_hip(stream),
                      static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), nvec);
   profile_after(as_hip(stream));
   return launch_check("copy16_kernel");
@@ -371,10 +382,10 @@ int hk_strided_copy(int dtype, const void* src, void* dst, int ndim, const int64
   dim3 g{unsigned(blocks)}, b{256};
   hipStream_t s = as_hip(stream);
   switch (es) {
-    case 1: hipLaunchKernelGGL(strided_copy_kernel<uint8_t>, g, b, 0, s, (const uint8_t*)src, (uint8_t*)dst, m, numel); break;
-    case 2: hipLaunchKernelGGL(strided_copy_kernel<uint16_t>, g, b, 0, s, (const uint16_t*)src, (uint16_t*)dst, m, numel); break;
-    case 4: hipLaunchKernelGGL(strided_copy_kernel<uint32_t>, g, b, 0, s, (const uint32_t*)src, (uint32_t*)dst, m, numel); break;
-    default: hipLaunchKernelGGL(strided_copy_kernel<uint64_t>, g, b, 0, s, (const uint64_t*)src, (uint64_t*)dst, m, numel); break;
+    case 1: HK_LAUNCH(strided_copy_kernel<uint8_t>, g, b, 0, s, (const uint8_t*)src, (uint8_t*)dst, m, numel); break;
+    case 2: HK_LAUNCH(strided_copy_kernel<uint16_t>, g, b, 0, s, (const uint16_t*)src, (uint16_t*)dst, m, numel); break;
+    case 4: HK_LAUNCH(strided_copy_kernel<uint32_t>, g, b, 0, s, (const uint32_t*)src, (uint32_t*)dst, m, numel); break;
+    default: HK_LAUNCH(strided_copy_kernel<uint64_t>, g, b, 0, s, (const uint64_t*)src, (uint64_t*)dst, m, numel); break;
   }
   return launch_check("strided_copy_kernel");
 }

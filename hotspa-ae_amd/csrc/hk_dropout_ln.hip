@@ -831,9 +831,9 @@ int hk_dropout_add_ln_fwd_ex(const hkDropoutAddLnFwdParams* pp, hkStream_t strea
     using WT = typename decltype(wt)::type;
     profile_before(s);
     switch (nc) {
-      case 1: hipLaunchKernelGGL((dal_fwd_kernel<IT, RT, WT, 1>), grid, block, 0, s, a); break;
-      case 2: hipLaunchKernelGGL((dal_fwd_kernel<IT, RT, WT, 2>), grid, block, 0, s, a); break;
-      default: hipLaunchKernelGGL((dal_fwd_kernel<IT, RT, WT, 4>), grid, block, 0, s, a); break;
+      case 1: HK_LAUNCH((dal_fwd_kernel<IT, RT, WT, 1>), grid, block, 0, s, a); break;
+      case 2: HK_LAUNCH((dal_fwd_kernel<IT, RT, WT, 2>), grid, block, 0, s, a); break;
+      default: HK_LAUNCH((dal_fwd_kernel<IT, RT, WT, 4>), grid, block, 0, s, a); break;
     }
     profile_after(s);
     return launch_check("dal_fwd_kernel");
@@ -959,14 +959,14 @@ int hk_dropout_add_ln_bwd_ex(const hkDropoutAddLnBwdParams* pp, hkStream_t strea
     profile_before(s);
     // two rows in flight where the ring fits the registers (a 16-bit residual stream), else one
     constexpr int PF = sizeof(RT) == 2 ? 2 : 1;
-    if (stream_form) hipLaunchKernelGGL((dal_bwd_stream_kernel<IT, RT, WT, PF>), grid, block, 0, s, a);
-    else if (g1) hipLaunchKernelGGL((dal_bwd_kernel<IT, RT, WT, false, true>), grid, block, 0, s, a);
-    else if (colscale) hipLaunchKernelGGL((dal_bwd_kernel<IT, RT, WT, true, false>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((dal_bwd_kernel<IT, RT, WT, false, false>), grid, block, 0, s, a);
+    if (stream_form) HK_LAUNCH((dal_bwd_stream_kernel<IT, RT, WT, PF>), grid, block, 0, s, a);
+    else if (g1) HK_LAUNCH((dal_bwd_kernel<IT, RT, WT, false, true>), grid, block, 0, s, a);
+    else if (colscale) HK_LAUNCH((dal_bwd_kernel<IT, RT, WT, true, false>), grid, block, 0, s, a);
+    else HK_LAUNCH((dal_bwd_kernel<IT, RT, WT, false, false>), grid, block, 0, s, a);
     profile_after(s);
     int r = launch_check("dal_bwd_kernel");
     if (r != HK_OK || nslots == 0) return r;
-    hipLaunchKernelGGL((dal_fold_kernel<WT>), dim3(unsigned((p.cols + 127) / 128), kMaxParts), dim3(512), 0, s, f);
+    HK_LAUNCH((dal_fold_kernel<WT>), dim3(unsigned((p.cols + 127) / 128), kMaxParts), dim3(512), 0, s, f);
     return launch_check("dal_fold_kernel");
   });
 }

@@ -232,13 +232,13 @@ static int unary_launch(const void* in, void* out, int64_t n, hipStream_t s) {
   if constexpr (ew_vectorised<T>()) {
     constexpr int VEC = VecIO<T>::N;
     if (n % VEC == 0 && aligned16(in) && aligned16(out)) {
-      hipLaunchKernelGGL((ew_unary_vec_kernel<T, OP>), dim3(blocks_for(n / VEC)), dim3(256), 0, s,
+      HK_LAUNCH((ew_unary_vec_kernel<T, OP>), dim3(blocks_for(n / VEC)), dim3(256), 0, s,
                          static_cast<const T*>(in), static_cast<T*>(out), n / VEC);
       profile_after(s);
       return launch_check("ew_unary_vec_kernel");
     }
   }
-  hipLaunchKernelGGL((ew_unary_scalar_kernel<T, OP>), dim3(blocks_for(n)), dim3(256), 0, s,
+  HK_LAUNCH((ew_unary_scalar_kernel<T, OP>), dim3(blocks_for(n)), dim3(256), 0, s,
                      static_cast<const T*>(in), static_cast<T*>(out), n);
   profile_after(s);
   return launch_check("ew_unary_scalar_kernel");
@@ -252,13 +252,13 @@ static int const_launch(const void* in, double c, void* out, int64_t n, hipStrea
   if constexpr (ew_vectorised<T>()) {
     constexpr int VEC = VecIO<T>::N;
     if (n % VEC == 0 && aligned16(in) && aligned16(out)) {
-      hipLaunchKernelGGL((ew_const_vec_kernel<T, OP, REV>), dim3(blocks_for(n / VEC)), dim3(256), 0, s,
+      HK_LAUNCH((ew_const_vec_kernel<T, OP, REV>), dim3(blocks_for(n / VEC)), dim3(256), 0, s,
                          static_cast<const T*>(in), float(c), static_cast<T*>(out), n / VEC);
       profile_after(s);
       return launch_check("ew_const_vec_kernel");
     }
   }
-  hipLaunchKernelGGL((ew_const_scalar_kernel<T, OP, REV>), dim3(blocks_for(n)), dim3(256), 0, s,
+  HK_LAUNCH((ew_const_scalar_kernel<T, OP, REV>), dim3(blocks_for(n)), dim3(256), 0, s,
                      static_cast<const T*>(in), c, static_cast<T*>(out), n);
   profile_after(s);
   return launch_check("ew_const_scalar_kernel");
@@ -327,7 +327,7 @@ static int binary_launch(const void* a, const void* b, void* out, const EwDims& 
         const uint32_t nvec = uint32_t(n / VEC), cols_vec = uint32_t(cols / VEC);
         const dim3 grid(blocks_for(nvec)), block(256);
 #define HK_EW_2D(AM, BM) \
-  hipLaunchKernelGGL((ew_binary_2d_vec_kernel<T, OP, AM, BM>), grid, block, 0, s, pa, pb, po, nvec, cols_vec)
+  HK_LAUNCH((ew_binary_2d_vec_kernel<T, OP, AM, BM>), grid, block, 0, s, pa, pb, po, nvec, cols_vec)
         if (am == EW_FULL) {
           switch (bm) {
             case EW_FULL: HK_EW_2D(EW_FULL, EW_FULL); break;
@@ -348,7 +348,7 @@ static int binary_launch(const void* a, const void* b, void* out, const EwDims& 
       }
     }
   }
-  hipLaunchKernelGGL((ew_binary_generic_kernel<T, OP>), dim3(blocks_for(n)), dim3(256), 0, s, pa, pb, po, d, n);
+  HK_LAUNCH((ew_binary_generic_kernel<T, OP>), dim3(blocks_for(n)), dim3(256), 0, s, pa, pb, po, d, n);
   profile_after(s);
   return launch_check("ew_binary_generic_kernel");
 }
@@ -372,7 +372,7 @@ static int broadcast_launch(const void* a, double c, void* out, const EwDims& d,
         const uint32_t nvec = uint32_t(n / VEC), cols_vec = uint32_t(cols / VEC);
         const dim3 grid(blocks_for(nvec)), block(256);
 #define HK_EW_BC(AM) \
-  hipLaunchKernelGGL((ew_broadcast_2d_vec_kernel<T, AM, MUL>), grid, block, 0, s, pa, float(c), po, nvec, cols_vec)
+  HK_LAUNCH((ew_broadcast_2d_vec_kernel<T, AM, MUL>), grid, block, 0, s, pa, float(c), po, nvec, cols_vec)
         switch (am) {
           case EW_FULL: HK_EW_BC(EW_FULL); break;
           case EW_PER_ROW: HK_EW_BC(EW_PER_ROW); break;
@@ -385,7 +385,7 @@ static int broadcast_launch(const void* a, double c, void* out, const EwDims& d,
       }
     }
   }
-  hipLaunchKernelGGL((ew_broadcast_generic_kernel<T, MUL>), dim3(blocks_for(n)), dim3(256), 0, s, pa, c, po, d, n);
+  HK_LAUNCH((ew_broadcast_generic_kernel<T, MUL>), dim3(blocks_for(n)), dim3(256), 0, s, pa, c, po, d, n);
   profile_after(s);
   return launch_check("ew_broadcast_generic_kernel");
 }

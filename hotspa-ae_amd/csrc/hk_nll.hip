@@ -76,7 +76,7 @@ static int nll_bwd_typed(const int64_t* label, const void* grad_loss, void* out,
       const int64_t nvec = total / VEC;
       HK_REQUIRE((nvec + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_nll_loss_bwd: output too large");
       profile_before(s);
-      hipLaunchKernelGGL((nll_bwd_vec_kernel<T>), dim3(unsigned((nvec + 255) / 256)), dim3(256), 0, s, label,
+      HK_LAUNCH((nll_bwd_vec_kernel<T>), dim3(unsigned((nvec + 255) / 256)), dim3(256), 0, s, label,
                          static_cast<const T*>(grad_loss), static_cast<T*>(out), rows, cols, cols / VEC, float(cols));
       profile_after(s);
       return launch_check("nll_bwd_vec_kernel");
@@ -84,7 +84,7 @@ static int nll_bwd_typed(const int64_t* label, const void* grad_loss, void* out,
   }
   HK_REQUIRE((total + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_nll_loss_bwd: output too large");
   using CT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
-  hipLaunchKernelGGL((nll_bwd_scalar_kernel<T, CT>), dim3(unsigned((total + 255) / 256)), dim3(256), 0, s, label,
+  HK_LAUNCH((nll_bwd_scalar_kernel<T, CT>), dim3(unsigned((total + 255) / 256)), dim3(256), 0, s, label,
                      static_cast<const T*>(grad_loss), static_cast<T*>(out), rows, cols, CT(cols));
   return launch_check("nll_bwd_scalar_kernel");
 }
@@ -106,19 +106,19 @@ int hk_nll_loss_fwd(int dtype, const void* pred, const int64_t* labels, void* lo
   profile_before(s);
   switch (dtype) {
     case HK_FLOAT32:
-      hipLaunchKernelGGL((nll_fwd_kernel<float>), grid, block, 0, s, static_cast<const float*>(pred), labels,
+      HK_LAUNCH((nll_fwd_kernel<float>), grid, block, 0, s, static_cast<const float*>(pred), labels,
                          static_cast<float*>(loss), rows, cols);
       break;
     case HK_BFLOAT16:
-      hipLaunchKernelGGL((nll_fwd_kernel<bf16>), grid, block, 0, s, static_cast<const bf16*>(pred), labels,
+      HK_LAUNCH((nll_fwd_kernel<bf16>), grid, block, 0, s, static_cast<const bf16*>(pred), labels,
                          static_cast<bf16*>(loss), rows, cols);
       break;
     case HK_FLOAT16:
-      hipLaunchKernelGGL((nll_fwd_kernel<fp16>), grid, block, 0, s, static_cast<const fp16*>(pred), labels,
+      HK_LAUNCH((nll_fwd_kernel<fp16>), grid, block, 0, s, static_cast<const fp16*>(pred), labels,
                          static_cast<fp16*>(loss), rows, cols);
       break;
     case HK_FLOAT64:
-      hipLaunchKernelGGL((nll_fwd_kernel<double>), grid, block, 0, s, static_cast<const double*>(pred), labels,
+      HK_LAUNCH((nll_fwd_kernel<double>), grid, block, 0, s, static_cast<const double*>(pred), labels,
                          static_cast<double*>(loss), rows, cols);
       break;
     default:

@@ -489,7 +489,7 @@ static int launch_norm_bwd_inst(const NormBwdArgs& a, const BwdPlan& p, int pf, 
   // the deep ring exists for the plain case only: full rows, no optional operands
   if (!exact || extra) pf = 1;
 #define HK_BWD_LAUNCH(P, E, F, X) \
-  hipLaunchKernelGGL((norm_bwd_kernel<T, NV, MODE, P, E, F, X, MAXT>), grid, block, p.lds_bytes, s, a)
+  HK_LAUNCH((norm_bwd_kernel<T, NV, MODE, P, E, F, X, MAXT>), grid, block, p.lds_bytes, s, a)
 #define HK_BWD_F(F)                                                         \
   do {                                                                      \
     if (exact && !extra) { if (pf >= 2) HK_BWD_LAUNCH(2, true, F, false); else HK_BWD_LAUNCH(1, true, F, false); } \
@@ -549,11 +549,11 @@ int norm_bwd_typed(NormBwdArgs a, int mode, void* dgamma, void* dbeta, void* ws,
                        (!a.dx_in || pitch_ok(a.dxin_pitch)) && (!a.dres || pitch_ok(a.dres_pitch));
   BwdPlan p = plan_norm_bwd<T>(a.rows, a.cols, aligned);
   if (!p.reg_path) {
-    hipLaunchKernelGGL((norm_bwd_generic_dx_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s, a, mode);
+    HK_LAUNCH((norm_bwd_generic_dx_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s, a, mode);
     int rc = launch_check("norm_bwd_generic_dx_kernel");
     if (rc != HK_OK) return rc;
     if (dgamma || dbeta) {
-      hipLaunchKernelGGL((norm_bwd_generic_cols_kernel<T, float>), dim3(unsigned((a.cols + 63) / 64)),
+      HK_LAUNCH((norm_bwd_generic_cols_kernel<T, float>), dim3(unsigned((a.cols + 63) / 64)),
                          dim3(256), 0, s, a, mode, static_cast<T*>(dgamma), static_cast<T*>(dbeta));
       rc = launch_check("norm_bwd_generic_cols_kernel");
     }
@@ -579,7 +579,7 @@ int norm_bwd_typed(NormBwdArgs a, int mode, void* dgamma, void* dbeta, void* ws,
     default: rc = launch_norm_bwd_nv<T, BWD_LN_MEMEFF>(a, p, s); break;
   }
   if (rc != HK_OK || !want_cols) return rc;
-  hipLaunchKernelGGL((norm_bwd_finalize_kernel<T>), dim3(unsigned((a.cols + 127) / 128), 2), dim3(512), 0, s,
+  HK_LAUNCH((norm_bwd_finalize_kernel<T>), dim3(unsigned((a.cols + 127) / 128), 2), dim3(512), 0, s,
                      a.part_dgamma, a.part_dbeta, static_cast<T*>(dgamma), static_cast<T*>(dbeta),
                      p.grid, a.cols);
   return launch_check("norm_bwd_finalize_kernel");

@@ -228,18 +228,18 @@ template <typename T, bool WAVE_ROW, bool HAS_RES, bool IS_RMS>
 static int launch_norm_fwd_rms(const NormFwdArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
   profile_before(s);
   switch (nv) {
-    case 1: hipLaunchKernelGGL((norm_fwd_kernel<T, 1, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 2: hipLaunchKernelGGL((norm_fwd_kernel<T, 2, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 3: hipLaunchKernelGGL((norm_fwd_kernel<T, 3, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 4: hipLaunchKernelGGL((norm_fwd_kernel<T, 4, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 5: hipLaunchKernelGGL((norm_fwd_kernel<T, 5, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 6: hipLaunchKernelGGL((norm_fwd_kernel<T, 6, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 8: hipLaunchKernelGGL((norm_fwd_kernel<T, 8, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 1: HK_LAUNCH((norm_fwd_kernel<T, 1, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 2: HK_LAUNCH((norm_fwd_kernel<T, 2, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 3: HK_LAUNCH((norm_fwd_kernel<T, 3, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 4: HK_LAUNCH((norm_fwd_kernel<T, 4, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 5: HK_LAUNCH((norm_fwd_kernel<T, 5, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 6: HK_LAUNCH((norm_fwd_kernel<T, 6, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 8: HK_LAUNCH((norm_fwd_kernel<T, 8, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
     case 16:
       // sixteen vectors are 64 fp32 registers only for fp32 data; with a residual two packed rows of that length
       // are in flight on top
       if constexpr (sizeof(T) == 4 && !WAVE_ROW && !HAS_RES) {
-        hipLaunchKernelGGL((norm_fwd_kernel<T, 16, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a);
+        HK_LAUNCH((norm_fwd_kernel<T, 16, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a);
         break;
       }
       [[fallthrough]];
@@ -338,7 +338,7 @@ int norm_fwd_typed(NormFwdArgs a, hipStream_t s) {
     return has_res ? launch_norm_fwd_nv<T, false, true>(a, nv, grid, block, s)
                    : launch_norm_fwd_nv<T, false, false>(a, nv, grid, block, s);
   }
-  hipLaunchKernelGGL((norm_fwd_generic_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
+  HK_LAUNCH((norm_fwd_generic_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
   return launch_check("norm_fwd_generic_kernel");
 }
 

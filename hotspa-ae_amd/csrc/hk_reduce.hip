@@ -585,17 +585,17 @@ static int reduce_fast(const ReducePlan& p, const void* in, void* out, float fac
     profile_before(st);
     if (s.tpr == 64) {
       dim3 grid(unsigned((p.rows + 3) / 4), unsigned(s.nsplit)), block(256);
-      hipLaunchKernelGGL((reduce_inner_vec_kernel<T, OUT_T, true, R>), grid, block, 0, st, a);
+      HK_LAUNCH((reduce_inner_vec_kernel<T, OUT_T, true, R>), grid, block, 0, st, a);
     } else {
       dim3 grid(unsigned(p.rows), unsigned(s.nsplit)), block{unsigned(s.tpr)};
-      hipLaunchKernelGGL((reduce_inner_vec_kernel<T, OUT_T, false, R>), grid, block, 0, st, a);
+      HK_LAUNCH((reduce_inner_vec_kernel<T, OUT_T, false, R>), grid, block, 0, st, a);
     }
     profile_after(st);
     int rc = launch_check("reduce_inner_vec_kernel");
     if (rc != HK_OK || s.nsplit == 1) return rc;
     // second pass over the fp32 partials [rows, nsplit]: combine and store only, the elements' own
     // transform (|x|, x^2, |x|^p of the p-norms) was applied when the partials were formed
-    hipLaunchKernelGGL((reduce_inner_scalar_kernel<float, float, OUT_T, Folded<R>>), dim3(unsigned(p.rows)), dim3(256), 0, st,
+    HK_LAUNCH((reduce_inner_scalar_kernel<float, float, OUT_T, Folded<R>>), dim3(unsigned(p.rows)), dim3(256), 0, st,
                        static_cast<const float*>(ws), static_cast<OUT_T*>(out), p.rows, int64_t(s.nsplit),
                        int64_t(s.nsplit), factor, is_mean);
     return launch_check("reduce_inner_scalar_kernel");
@@ -620,12 +620,12 @@ static int reduce_fast(const ReducePlan& p, const void* in, void* out, float fac
     dim3 grid(unsigned(col_tiles), unsigned(s.rsplit), unsigned(p.B)), block{unsigned(64 * s.wy * s.wx)};
     const size_t lds = size_t(s.wy) * s.wx * 64 * VEC * sizeof(float);
     profile_before(st);
-    hipLaunchKernelGGL((reduce_outer_vec_kernel<T, OUT_T, R>), grid, block, lds, st, a);
+    HK_LAUNCH((reduce_outer_vec_kernel<T, OUT_T, R>), grid, block, lds, st, a);
     profile_after(st);
     int rc = launch_check("reduce_outer_vec_kernel");
     if (rc != HK_OK || s.rsplit == 1) return rc;
     const int64_t n = p.B * p.C;
-    hipLaunchKernelGGL((reduce_fold_partials_kernel<OUT_T, R>), dim3(unsigned((n + 63) / 64)), dim3(256), 0, st,
+    HK_LAUNCH((reduce_fold_partials_kernel<OUT_T, R>), dim3(unsigned((n + 63) / 64)), dim3(256), 0, st,
                        static_cast<const float*>(ws), static_cast<OUT_T*>(out), s.rsplit, n, factor, is_mean);
     return launch_check("reduce_fold_partials_kernel");
   }
@@ -639,18 +639,18 @@ static int reduce_slow(const ReducePlan& p, const void* in, void* out, float fac
   OUT_T* op = static_cast<OUT_T*>(out);
   if (p.kind == PLAN_INNER) {
     HK_REQUIRE(p.rows <= 0x7fffffffLL, HK_ERR_INVALID, "hk_reduce: too many rows");
-    hipLaunchKernelGGL((reduce_inner_scalar_kernel<T, ACC, OUT_T, R>), dim3(unsigned(p.rows)), dim3(256), 0, st, ip, op,
+    HK_LAUNCH((reduce_inner_scalar_kernel<T, ACC, OUT_T, R>), dim3(unsigned(p.rows)), dim3(256), 0, st, ip, op,
                        p.rows, p.row_stride, p.cols, factor, is_mean);
     return launch_check("reduce_inner_scalar_kernel");
   }
   if (p.kind == PLAN_OUTER) {
     const int64_t n = p.B * p.C;
-    hipLaunchKernelGGL((reduce_outer_scalar_kernel<T, ACC, OUT_T, R>), dim3(unsigned((n + 255) / 256)), dim3(256), 0, st,
+    HK_LAUNCH((reduce_outer_scalar_kernel<T, ACC, OUT_T, R>), dim3(unsigned((n + 255) / 256)), dim3(256), 0, st,
                        ip, op, p.B, p.R, p.C, p.b_stride, p.r_stride, factor, is_mean);
     return launch_check("reduce_outer_scalar_kernel");
   }
   GenericMeta m = generic_meta(p);
-  hipLaunchKernelGGL((reduce_generic_kernel<T, ACC, OUT_T, R>), dim3(unsigned((m.n_out + 255) / 256)), dim3(256), 0, st,
+  HK_LAUNCH((reduce_generic_kernel<T, ACC, OUT_T, R>), dim3(unsigned((m.n_out + 255) / 256)), dim3(256), 0, st,
                      ip, op, m, factor, is_mean);
   return launch_check("reduce_generic_kernel");
 }
@@ -773,7 +773,7 @@ static int norm_grad_typed(const void* x, const void* norm, const void* grad, vo
       auto kernel = p == 1 ? norm_grad_rows_vec_kernel<T, 1>
                   : p == 2 ? norm_grad_rows_vec_kernel<T, 2> : norm_grad_rows_vec_kernel<T, 0>;
       profile_before(s);
-      hipLaunchKernelGGL(kernel, dim3((nvec + 255) / 256), dim3(256), 0, s,
+      HK_LAUNCH(kernel, dim3((nvec + 255) / 256), dim3(256), 0, s,
                          static_cast<const T*>(x), static_cast<const T*>(norm), static_cast<const T*>(grad),
                          static_cast<T*>(out), nvec, uint32_t(reduce_size / VEC), p);
       profile_after(s);
@@ -782,7 +782,7 @@ static int norm_grad_typed(const void* x, const void* norm, const void* grad, vo
   }
   HK_REQUIRE((total + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_norm_bwd: array too large");
   profile_before(s);
-  hipLaunchKernelGGL((norm_grad_kernel<T, CT>), dim3(unsigned((total + 255) / 256)), dim3(256), 0, s,
+  HK_LAUNCH((norm_grad_kernel<T, CT>), dim3(unsigned((total + 255) / 256)), dim3(256), 0, s,
                      static_cast<const T*>(x), static_cast<const T*>(norm), static_cast<const T*>(grad),
                      static_cast<T*>(out), total, reduce_size, after, p);
   profile_after(s);

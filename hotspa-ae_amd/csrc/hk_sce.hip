@@ -449,10 +449,10 @@ template <typename T, int MODE, bool WAVE_ROW>
 static int launch_sce_nv(const SceArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
 #define HK_SCE_LAUNCH(N)                                                                         \
   do {                                                                                           \
-    if constexpr (MODE == 0) hipLaunchKernelGGL((sce_sparse_fwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a); \
-    else if constexpr (MODE == 1) hipLaunchKernelGGL((sce_sparse_bwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a); \
-    else if constexpr (MODE == 2) hipLaunchKernelGGL((sce_dense_kernel<T, N, WAVE_ROW, false>), grid, block, 0, s, a); \
-    else hipLaunchKernelGGL((sce_dense_kernel<T, N, WAVE_ROW, true>), grid, block, 0, s, a);       \
+    if constexpr (MODE == 0) HK_LAUNCH((sce_sparse_fwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a); \
+    else if constexpr (MODE == 1) HK_LAUNCH((sce_sparse_bwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a); \
+    else if constexpr (MODE == 2) HK_LAUNCH((sce_dense_kernel<T, N, WAVE_ROW, false>), grid, block, 0, s, a); \
+    else HK_LAUNCH((sce_dense_kernel<T, N, WAVE_ROW, true>), grid, block, 0, s, a);       \
   } while (0)
   profile_before(s);
   switch (nv) {
@@ -490,7 +490,7 @@ static int sce_typed(SceArgs a, hipStream_t s) {
     dim3 grid{unsigned(a.rows)}, block{unsigned(threads)};
     return launch_sce_nv<T, MODE, false>(a, nv, grid, block, s);
   }
-  hipLaunchKernelGGL((sce_generic_kernel<T, float, MODE>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
+  HK_LAUNCH((sce_generic_kernel<T, float, MODE>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
   return launch_check("sce_generic_kernel");
 }
 
@@ -514,7 +514,7 @@ static int sce_dispatch(int dtype, SceArgs& a, hipStream_t s, const char* who) {
     case HK_BFLOAT16: return sce_typed<bf16, MODE>(a, s);
     case HK_FLOAT16: return sce_typed<fp16, MODE>(a, s);
     case HK_FLOAT64:
-      hipLaunchKernelGGL((sce_generic_kernel<double, double, MODE>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
+      HK_LAUNCH((sce_generic_kernel<double, double, MODE>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
       return launch_check("sce_generic_kernel<double>");
     default:
       set_last_error("%s: not implemented for dtype %d", who, dtype);

@@ -273,15 +273,15 @@ template <typename T, bool BWD, bool WAVE_ROW>
 static int launch_softmax_nv(const SoftmaxArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
 #define HK_SM_CASE(N)                                                                      \
   case N:                                                                                  \
-    if constexpr (BWD) hipLaunchKernelGGL((softmax_bwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a); \
-    else hipLaunchKernelGGL((softmax_fwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a);   \
+    if constexpr (BWD) HK_LAUNCH((softmax_bwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a); \
+    else HK_LAUNCH((softmax_fwd_kernel<T, N, WAVE_ROW>), grid, block, 0, s, a);   \
     break;
   profile_before(s);
   switch (nv) {
     HK_SM_CASE(1) HK_SM_CASE(2) HK_SM_CASE(4) HK_SM_CASE(8)
     case 16:
       if constexpr (VecIO<T>::N == 4 && !BWD) {
-        hipLaunchKernelGGL((softmax_fwd_kernel<T, 16, WAVE_ROW>), grid, block, 0, s, a);
+        HK_LAUNCH((softmax_fwd_kernel<T, 16, WAVE_ROW>), grid, block, 0, s, a);
         break;
       }
       [[fallthrough]];
@@ -314,12 +314,12 @@ static int softmax_lastdim_typed(SoftmaxArgs a, hipStream_t s) {
     return launch_softmax_nv<T, BWD, false>(a, nv, grid, block, s);
   }
   if constexpr (BWD) {
-    hipLaunchKernelGGL((softmax_bwd_longrow_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s,
+    HK_LAUNCH((softmax_bwd_longrow_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s,
                        static_cast<const T*>(a.x), static_cast<const T*>(a.dy), static_cast<T*>(a.out),
                        int64_t(a.cols), a.x_pitch, a.dy_pitch, a.out_pitch);
     return launch_check("softmax_bwd_longrow_kernel");
   } else {
-    hipLaunchKernelGGL((softmax_fwd_longrow_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s,
+    HK_LAUNCH((softmax_fwd_longrow_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s,
                        static_cast<const T*>(a.x), static_cast<T*>(a.out), int64_t(a.cols), a.x_pitch, a.out_pitch);
     return launch_check("softmax_fwd_longrow_kernel");
   }
@@ -331,11 +331,11 @@ static int softmax_strided_typed(const void* x, const void* dy, void* out, int64
                                  hipStream_t s) {
   if (inner == 1) {
     if constexpr (BWD) {
-      hipLaunchKernelGGL((softmax_bwd_longrow_kernel<T, CT>), dim3(unsigned(outer)), dim3(256), 0, s,
+      HK_LAUNCH((softmax_bwd_longrow_kernel<T, CT>), dim3(unsigned(outer)), dim3(256), 0, s,
                          static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<T*>(out), dim, x_pitch,
                          dy_pitch, out_pitch);
     } else {
-      hipLaunchKernelGGL((softmax_fwd_longrow_kernel<T, CT>), dim3(unsigned(outer)), dim3(256), 0, s,
+      HK_LAUNCH((softmax_fwd_longrow_kernel<T, CT>), dim3(unsigned(outer)), dim3(256), 0, s,
                          static_cast<const T*>(x), static_cast<T*>(out), dim, x_pitch, out_pitch);
     }
     return launch_check("softmax_longrow_kernel");
@@ -343,11 +343,11 @@ static int softmax_strided_typed(const void* x, const void* dy, void* out, int64
   const int64_t npos = outer * inner;
   const int64_t blocks = (npos + 255) / 256;
   if constexpr (BWD) {
-    hipLaunchKernelGGL((softmax_bwd_strided_kernel<T, CT>), dim3(unsigned(blocks)), dim3(256), 0, s,
+    HK_LAUNCH((softmax_bwd_strided_kernel<T, CT>), dim3(unsigned(blocks)), dim3(256), 0, s,
                        static_cast<const T*>(x), static_cast<const T*>(dy), static_cast<T*>(out), outer,
                        dim, inner);
   } else {
-    hipLaunchKernelGGL((softmax_fwd_strided_kernel<T, CT>), dim3(unsigned(blocks)), dim3(256), 0, s,
+    HK_LAUNCH((softmax_fwd_strided_kernel<T, CT>), dim3(unsigned(blocks)), dim3(256), 0, s,
                        static_cast<const T*>(x), static_cast<T*>(out), outer, dim, inner);
   }
   return launch_check("softmax_strided_kernel");

@@ -67,10 +67,10 @@ static int probe_nt(const ProbeArgs& a, int ntl, int nts, unsigned grid, hipStre
   if (NR == 0) ntl = 0;
   if (NW == 0) nts = 0;
   profile_before(s);
-  if (ntl && nts) hipLaunchKernelGGL((stream_probe_kernel<BS, U, NR, NW, NR != 0, NW != 0>), dim3(grid), dim3(BS), 0, s, a);
-  else if (ntl) hipLaunchKernelGGL((stream_probe_kernel<BS, U, NR, NW, NR != 0, false>), dim3(grid), dim3(BS), 0, s, a);
-  else if (nts) hipLaunchKernelGGL((stream_probe_kernel<BS, U, NR, NW, false, NW != 0>), dim3(grid), dim3(BS), 0, s, a);
-  else hipLaunchKernelGGL((stream_probe_kernel<BS, U, NR, NW, false, false>), dim3(grid), dim3(BS), 0, s, a);
+  if (ntl && nts) HK_LAUNCH((stream_probe_kernel<BS, U, NR, NW, NR != 0, NW != 0>), dim3(grid), dim3(BS), 0, s, a);
+  else if (ntl) HK_LAUNCH((stream_probe_kernel<BS, U, NR, NW, NR != 0, false>), dim3(grid), dim3(BS), 0, s, a);
+  else if (nts) HK_LAUNCH((stream_probe_kernel<BS, U, NR, NW, false, NW != 0>), dim3(grid), dim3(BS), 0, s, a);
+  else HK_LAUNCH((stream_probe_kernel<BS, U, NR, NW, false, false>), dim3(grid), dim3(BS), 0, s, a);
   profile_after(s);
   return launch_check("stream_probe_kernel");
 }

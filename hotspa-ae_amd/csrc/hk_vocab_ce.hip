@@ -172,7 +172,7 @@ static int vocab_bwd_fused_typed(const void* x, const int64_t* labels, const flo
     if (cols % VEC == 0 && aligned16(x) && aligned16(out) && total / VEC < 0x7fffffffLL) {
       const uint32_t nvec = uint32_t(total / VEC);
       profile_before(s);
-      hipLaunchKernelGGL((vocab_ce_bwd_fused_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
+      HK_LAUNCH((vocab_ce_bwd_fused_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
                          static_cast<const T*>(x), labels, lse, static_cast<const T*>(grad_loss), static_cast<T*>(out),
                          nvec, uint32_t(cols / VEC), vocab_start, ignored_index);
       profile_after(s);
@@ -182,7 +182,7 @@ static int vocab_bwd_fused_typed(const void* x, const int64_t* labels, const flo
   HK_REQUIRE((total + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_vocab_parallel_ce_bwd_fused: output too large");
   using CT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
   profile_before(s);
-  hipLaunchKernelGGL((vocab_ce_bwd_fused_scalar_kernel<T, CT>), dim3(unsigned((total + 255) / 256)), dim3(256), 0, s,
+  HK_LAUNCH((vocab_ce_bwd_fused_scalar_kernel<T, CT>), dim3(unsigned((total + 255) / 256)), dim3(256), 0, s,
                      static_cast<const T*>(x), labels, lse, static_cast<const T*>(grad_loss), static_cast<T*>(out),
                      total, cols, vocab_start, ignored_index);
   profile_after(s);
@@ -198,7 +198,7 @@ static int vocab_bwd_typed(const void* softmax, const int64_t* labels, const voi
     if (cols % VEC == 0 && aligned16(softmax) && aligned16(out) && total / VEC < 0x7fffffffLL) {
       const uint32_t nvec = uint32_t(total / VEC);
       profile_before(s);
-      hipLaunchKernelGGL((vocab_ce_bwd_vec_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
+      HK_LAUNCH((vocab_ce_bwd_vec_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
                          static_cast<const T*>(softmax), labels, static_cast<const T*>(grad_loss),
                          static_cast<T*>(out), nvec, uint32_t(cols / VEC), vocab_start);
       profile_after(s);
@@ -208,7 +208,7 @@ static int vocab_bwd_typed(const void* softmax, const int64_t* labels, const voi
   HK_REQUIRE((total + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID, "hk_vocab_parallel_ce_bwd: output too large");
   using CT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
   profile_before(s);
-  hipLaunchKernelGGL((vocab_ce_bwd_scalar_kernel<T, CT>), dim3(unsigned((total + 255) / 256)), dim3(256), 0, s,
+  HK_LAUNCH((vocab_ce_bwd_scalar_kernel<T, CT>), dim3(unsigned((total + 255) / 256)), dim3(256), 0, s,
                      static_cast<const T*>(softmax), labels, static_cast<const T*>(grad_loss), static_cast<T*>(out),
                      total, cols, vocab_start);
   profile_after(s);
@@ -233,7 +233,7 @@ int hk_vocab_parallel_ce_gather(int dtype, const void* logits, const int64_t* la
   hipStream_t s = as_hip(stream);
   const dim3 grid(unsigned((rows + 255) / 256)), block(256);
 #define HK_VCE_GATHER(T)                                                                                         \
-  hipLaunchKernelGGL((vocab_ce_gather_kernel<T>), grid, block, 0, s, static_cast<const T*>(logits), labels, rows, \
+  HK_LAUNCH((vocab_ce_gather_kernel<T>), grid, block, 0, s, static_cast<const T*>(logits), labels, rows, \
                      cols, vocab_start, vocab_end, ignored_index, static_cast<T*>(picked), static_cast<T*>(lse))
   switch (dtype) {
     case HK_FLOAT32: HK_VCE_GATHER(float); break;
@@ -256,7 +256,7 @@ int hk_vocab_parallel_ce_combine(int loss_dtype, const float* stats, int nshards
   hipStream_t s = as_hip(stream);
   const dim3 grid(unsigned((rows + 255) / 256)), block(256);
 #define HK_VCE_COMBINE(T)                                                                                       \
-  hipLaunchKernelGGL((vocab_ce_combine_kernel<T>), grid, block, 0, s, stats, nshards, labels, ignored_index,    \
+  HK_LAUNCH((vocab_ce_combine_kernel<T>), grid, block, 0, s, stats, nshards, labels, ignored_index,    \
                      static_cast<T*>(loss), lse, rows)
   switch (loss_dtype) {
     case HK_FLOAT32: HK_VCE_COMBINE(float); break;

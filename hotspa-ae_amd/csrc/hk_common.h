@@ -207,6 +207,14 @@ __device__ __forceinline__ float dpp_f(float v, float old = 0.f) {
       int(f2u(old)), int(f2u(v)), CTRL, ROW_MASK, 0xf, false)));
 }
 
+// The four controls below permute the lanes of a row of 16 among themselves: every lane has a source, so the
+// "old" operand never shows.  Passing 0 with bound_ctrl set lets the compiler fold the move into the instruction
+// that consumes it (one v_add_f32 with a DPP operand instead of copy + v_mov_b32_dpp + add).
+template <int CTRL>
+__device__ __forceinline__ float dpp_perm(float v) {
+  return u2f(uint32_t(__builtin_amdgcn_update_dpp(0, int(f2u(v)), CTRL, 0xf, 0xf, true)));
+}
+
 constexpr int kDppXor1 = 0xB1;        // quad_perm:[1,0,3,2]
 constexpr int kDppXor2 = 0x4E;        // quad_perm:[2,3,0,1]
 constexpr int kDppHalfMirror = 0x141; // row_half_mirror
@@ -221,10 +229,10 @@ __device__ __forceinline__ float readlane_f(float v, int lane) {
 // Op: a struct with `static float identity()` and `static float apply(float, float)`.
 template <typename Op>
 __device__ __forceinline__ float wave_allreduce(float v) {
-  v = Op::apply(v, dpp_f<kDppXor1>(v, v));
-  v = Op::apply(v, dpp_f<kDppXor2>(v, v));
-  v = Op::apply(v, dpp_f<kDppHalfMirror>(v, v));
-  v = Op::apply(v, dpp_f<kDppMirror>(v, v));
+  v = Op::apply(v, dpp_perm<kDppXor1>(v));
+  v = Op::apply(v, dpp_perm<kDppXor2>(v));
+  v = Op::apply(v, dpp_perm<kDppHalfMirror>(v));
+  v = Op::apply(v, dpp_perm<kDppMirror>(v));
   // every lane of a 16-lane row now holds that row's result; fold the 4 rows
   float r0 = readlane_f(v, 0), r1 = readlane_f(v, 16);
   float r2 = readlane_f(v, 32), r3 = readlane_f(v, 48);
@@ -237,8 +245,8 @@ __device__ __forceinline__ float wave_allreduce(float v) {
 // tuples (Chan merge, online softmax) where the combine is not a plain op.
 template <int STRIDE>
 __device__ __forceinline__ float lane_xor(float v) {
-  if constexpr (STRIDE == 1) return dpp_f<kDppXor1>(v, v);
-  else if constexpr (STRIDE == 2) return dpp_f<kDppXor2>(v, v);
+  if constexpr (STRIDE == 1) return dpp_perm<kDppXor1>(v);
+  else if constexpr (STRIDE == 2) return dpp_perm<kDppXor2>(v);
   else return __shfl_xor(v, STRIDE, kWave);
 }
 
@@ -269,16 +277,16 @@ template <typename P>
 __device__ __forceinline__ P wave_allreduce_tuple(P a) {
   P b;
 #pragma unroll
-  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_f<kDppXor1>(a.v[k], a.v[k]);
+  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_perm<kDppXor1>(a.v[k]);
   a = P::merge(a, b);
 #pragma unroll
-  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_f<kDppXor2>(a.v[k], a.v[k]);
+  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_perm<kDppXor2>(a.v[k]);
   a = P::merge(a, b);
 #pragma unroll
-  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_f<kDppHalfMirror>(a.v[k], a.v[k]);
+  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_perm<kDppHalfMirror>(a.v[k]);
   a = P::merge(a, b);
 #pragma unroll
-  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_f<kDppMirror>(a.v[k], a.v[k]);
+  for (int k = 0; k < P::K; ++k) b.v[k] = dpp_perm<kDppMirror>(a.v[k]);
   a = P::merge(a, b);
   P r[4];
 #pragma unroll
@@ -319,6 +327,31 @@ __device__ __forceinline__ P group_combine_tuple(P a, float* scratch, int first_
     P o;
 #pragma unroll
     for (int k = 0; k < P::K; ++k) o.v[k] = scratch[(first_wave + i) * P::K + k];
+    r = P::merge(r, o);
+  }
+  return r;
+}
+
+// The same for a group that is the whole workgroup and whose number of wavefronts is a constant: no loop, the
+// NW partials are read with wide LDS loads at constant offsets.
+template <typename P, int NW>
+__device__ __forceinline__ P group_allreduce_tuple_fixed(P a, float* scratch) {
+  a = wave_allreduce_tuple<P>(a);
+  if constexpr (NW == 1) return a;
+  const int w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int k = 0; k < P::K; ++k) scratch[w * P::K + k] = a.v[k];
+  }
+  __syncthreads();
+  P r;
+#pragma unroll
+  for (int k = 0; k < P::K; ++k) r.v[k] = scratch[k];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) {
+    P o;
+#pragma unroll
+    for (int k = 0; k < P::K; ++k) o.v[k] = scratch[i * P::K + k];
     r = P::merge(r, o);
   }
   return r;

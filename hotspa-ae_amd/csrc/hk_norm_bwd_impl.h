@@ -36,7 +36,17 @@ __device__ __forceinline__ float clamp_by_magnitude(float g, float eps) {
 // really uses (a 640-thread block of the 5120-column LayerNorm may hold 170
 // registers per lane where a 1024-thread block may hold 128), which is what lets
 // the LayerNorm modes, with the mean in their ring as well, keep two rows in flight.
-template <typename T, int NV, int MODE, int PF, bool EXACT, bool STATS_F32, bool EXTRA, int MAXT>
+//
+// FIXED says that one group of exactly MAXT threads is the whole block: the group's
+// width, and with it the number of wavefront partials every thread adds up after the
+// barrier, is then a constant and the cross-wavefront step is straight-line code.
+// Whatever the hot case never has is decided at compile time there: EXTRA also stands
+// for "gamma clamped in dx on request" (a uniform branch between two copies of the
+// arithmetic otherwise, whose merge costs one register move per live value per row);
+// without EXTRA, CLAMP says at compile time whether gamma enters dx clamped (the fused
+// LayerNorm's backward does that in both of its modes, the plain one never).
+template <typename T, int NV, int MODE, int PF, bool EXACT, bool STATS_F32, bool EXTRA, int MAXT, bool FIXED,
+          bool CLAMP>
 __global__ __launch_bounds__(MAXT)
 void norm_bwd_kernel(NormBwdArgs a) {
   constexpr int VEC = VecIO<T>::N;
@@ -45,11 +55,11 @@ void norm_bwd_kernel(NormBwdArgs a) {
   using StatT = typename std::conditional<STATS_F32, float, T>::type;
   using RowSums = SumTuple<KS>;
   extern __shared__ float lds[];            // [rows_per_block, cols] column-sum staging
-  __shared__ float red[2][kMaxWaves * KS];  // double-buffered by step parity
+  __shared__ __align__(16) float red[2][kMaxWaves * KS];  // double-buffered by step parity
 
-  const int tpr = a.tpr;                   // multiple of 64: a wavefront never straddles two rows
-  const int rpb = int(blockDim.x) / tpr;
-  const int group = __builtin_amdgcn_readfirstlane(int(threadIdx.x) / tpr);
+  const int tpr = FIXED ? MAXT : a.tpr;    // multiple of 64: a wavefront never straddles two rows
+  const int rpb = FIXED ? 1 : int(blockDim.x) / tpr;
+  const int group = FIXED ? 0 : __builtin_amdgcn_readfirstlane(int(threadIdx.x) / tpr);
   const int t = int(threadIdx.x) - group * tpr;
   const int waves_per_group = tpr >> 6;
   const int first_wave = group * waves_per_group;
@@ -83,7 +93,7 @@ void norm_bwd_kernel(NormBwdArgs a) {
       }
     }
   }
-  const bool clamp = a.clamp_gamma != 0 || MODE == BWD_LN_MEMEFF;
+  [[maybe_unused]] const bool clamp = MODE == BWD_LN_MEMEFF || CLAMP || (EXTRA && a.clamp_gamma != 0);
 
   float dg[NE], db[NE];
 #pragma unroll
@@ -132,7 +142,8 @@ void norm_bwd_kernel(NormBwdArgs a) {
     [[maybe_unused]] float mu = 0.f;
     if constexpr (MODE == BWD_LN) mu = Cvt<StatT>::to_float(nmu[d]);
     const float sv = Cvt<StatT>::to_float(nsv[d]);
-    const float rs = a.stat_kind == HK_STAT_VAR ? 1.0f / sqrtf(sv + a.eps) : sv;
+    // RMSNorm keeps the inverse root mean square, never a variance
+    const float rs = (MODE != BWD_RMS && a.stat_kind == HK_STAT_VAR) ? 1.0f / sqrtf(sv + a.eps) : sv;
     // the slot is free again: refill it with the row PF steps ahead
     issue(slot, row + int64_t(PF) * stride);
 
@@ -169,10 +180,12 @@ void norm_bwd_kernel(NormBwdArgs a) {
         }
       }
     };
-    if (clamp) accumulate(std::true_type{});   // uniform
+    if constexpr (!EXTRA) accumulate(std::integral_constant<bool, MODE == BWD_LN_MEMEFF || CLAMP>{});
+    else if (clamp) accumulate(std::true_type{});   // uniform
     else accumulate(std::false_type{});
 
-    s = group_allreduce_tuple(s, red[parity], first_wave, waves_per_group);
+    if constexpr (FIXED) s = group_allreduce_tuple_fixed<RowSums, MAXT / 64>(s, red[parity]);
+    else s = group_allreduce_tuple(s, red[parity], first_wave, waves_per_group);
     parity ^= 1;
     if (valid) {
       // plain modes: s0 = rs * sum(dy g), s1 = rs * sum(dy g xc);  dx = q - s0/n - xc * rs^2 * s1/n
@@ -478,24 +491,40 @@ BwdPlan plan_norm_bwd(int64_t rows, int cols, bool aligned) {
 }
 
 // launch bound of the kernel instance that runs a block of `block` threads
-static inline int bound_for(int block) { return block <= 512 ? 512 : (block <= 768 ? 768 : 1024); }
+static inline int bound_for(int block) {
+  return block <= 512 ? 512 : (block <= 640 ? 640 : (block <= 768 ? 768 : 1024));
+}
 
 template <typename T, int MODE, int NV, int MAXT>
 static int launch_norm_bwd_inst(const NormBwdArgs& a, const BwdPlan& p, int pf, hipStream_t s) {
   dim3 grid{unsigned(p.grid)}, block{unsigned(p.block)};
   const bool exact = int64_t(p.nv) * p.tpr == a.nvec;
   const bool f32 = a.stats_f32 != 0;
-  const bool extra = a.dx_in != nullptr || a.dres != nullptr;
+  // the kernel's "extra" instance takes the optional operands behind uniform branches, and the clamp request in
+  // the modes that have no instance of their own for it
+  const bool want_clamp = a.clamp_gamma != 0 && MODE != BWD_LN_MEMEFF;   // the memory-efficient mode always clamps
+  const bool extra = a.dx_in != nullptr || a.dres != nullptr || (want_clamp && MODE != BWD_LN);
+  // one group that is the whole block, of exactly the bound's size: the instance with a constant group width
+  const bool fixed = p.rpb == 1 && p.block == MAXT;
   // the deep ring exists for the plain case only: full rows, no optional operands
   if (!exact || extra) pf = 1;
-#define HK_BWD_LAUNCH(P, E, F, X) \
-  HK_LAUNCH((norm_bwd_kernel<T, NV, MODE, P, E, F, X, MAXT>), grid, block, p.lds_bytes, s, a)
+#define HK_BWD_LAUNCH(P, E, F, X, FX, C) \
+  HK_LAUNCH((norm_bwd_kernel<T, NV, MODE, P, E, F, X, MAXT, FX, C>), grid, block, p.lds_bytes, s, a)
+#define HK_BWD_LEAN(P, F, FX)                                               \
+  do {                                                                      \
+    if constexpr (MODE == BWD_LN) {                                         \
+      if (want_clamp) HK_BWD_LAUNCH(P, true, F, false, FX, true); else HK_BWD_LAUNCH(P, true, F, false, FX, false); \
+    } else {                                                                \
+      HK_BWD_LAUNCH(P, true, F, false, FX, false);                          \
+    }                                                                       \
+  } while (0)
 #define HK_BWD_F(F)                                                         \
   do {                                                                      \
-    if (exact && !extra) { if (pf >= 2) HK_BWD_LAUNCH(2, true, F, false); else HK_BWD_LAUNCH(1, true, F, false); } \
-    else if (exact) HK_BWD_LAUNCH(1, true, F, true);                        \
-    else if (!extra) HK_BWD_LAUNCH(1, false, F, false);                     \
-    else HK_BWD_LAUNCH(1, false, F, true);                                  \
+    if (exact && !extra && fixed) { if (pf >= 2) HK_BWD_LEAN(2, F, true); else HK_BWD_LEAN(1, F, true); } \
+    else if (exact && !extra) { if (pf >= 2) HK_BWD_LEAN(2, F, false); else HK_BWD_LEAN(1, F, false); } \
+    else if (exact) HK_BWD_LAUNCH(1, true, F, true, false, false);          \
+    else if (!extra && !want_clamp) HK_BWD_LAUNCH(1, false, F, false, false, false); \
+    else HK_BWD_LAUNCH(1, false, F, true, false, false);                    \
   } while (0)
   if constexpr (MODE == BWD_LN && !std::is_same<T, float>::value) {
     if (f32) HK_BWD_F(true); else HK_BWD_F(false);
@@ -503,6 +532,7 @@ static int launch_norm_bwd_inst(const NormBwdArgs& a, const BwdPlan& p, int pf, 
     HK_BWD_F(true);   // for float data "statistics in the data type" and "in float" are the same kernel
   }
 #undef HK_BWD_F
+#undef HK_BWD_LEAN
 #undef HK_BWD_LAUNCH
   return HK_OK;
 }
@@ -523,6 +553,7 @@ static int launch_norm_bwd_nv(const NormBwdArgs& a, const BwdPlan& p, hipStream_
   int rc = HK_ERR_UNSUPPORTED;
   if (p.nv == 1) {
     if (bound == 512) rc = launch_norm_bwd_inst<T, MODE, 1, 512>(a, p, pf, s);
+    else if (bound == 640) rc = launch_norm_bwd_inst<T, MODE, 1, 640>(a, p, pf, s);
     else if (bound == 768) rc = launch_norm_bwd_inst<T, MODE, 1, 768>(a, p, pf, s);
     else rc = launch_norm_bwd_inst<T, MODE, 1, 1024>(a, p, pf, s);
   } else if (p.nv == 2) {

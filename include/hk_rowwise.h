@@ -112,8 +112,9 @@ HK_API const char* hk_tune_keys(void);
 
 /* Measurement hook: the next launch of an operator's main kernel (the one that
  * streams the rows; not the small fold / finalize launches) made by the calling
- * thread records `before` and `after` around that kernel on its stream, then the
- * hook clears itself.  Pass NULLs to cancel. */
+ * thread carries `before` and `after` on its own dispatch (hipExtLaunchKernelGGL),
+ * so that hk_event_elapsed_ns(before, after) is that kernel's begin-to-end time on
+ * its stream; then the hook clears itself.  Pass NULLs to cancel. */
 HK_API int hk_profile_next_kernel(hkEvent_t before, hkEvent_t after);
 
 /* Plain streaming copy kernel of `bytes` (multiple of 16, 16-byte aligned):

@@ -517,6 +517,7 @@ enum TuneKey {
   TUNE_NORM_BWD_PREFETCH,
   TUNE_REDUCE_OUTER_WAVES_ACROSS,
   TUNE_REDUCE_OUTER_WAVES,
+  TUNE_NORM_FWD_ROWS,
   TUNE_NUM_KEYS
 };
 int tune_get(int key);

@@ -67,6 +67,7 @@ static const char* const kTuneNames[] = {
   "norm_bwd_prefetch",  // rows loaded ahead by the backward kernel (1..3)
   "reduce_outer_waves_across",  // wavefronts of a column-reduction workgroup side by side across columns
   "reduce_outer_waves",         // wavefronts of a column-reduction workgroup in all
+  "norm_fwd_rows",              // rows a workgroup of the forward norm kernel takes (1 or 2)
 };
 constexpr int kNumTune = sizeof(kTuneNames) / sizeof(kTuneNames[0]);
 static_assert(kNumTune == TUNE_NUM_KEYS, "tune name table out of sync with TuneKey");

@@ -1,153 +1,223 @@
 // LayerNorm / RMSNorm forward kernels and their launch logic, included by the per-type instantiation files.
 //
-// A row lives in registers as packed 128-bit vectors (one HBM read), statistics are Welford moments merged with
-// Chan's update across lanes (DPP, equal-count form when the row fills every lane) and waves (LDS), output is
-// written with 128-bit stores.  One wavefront per row for short rows, one workgroup per row for long rows.
+// A row is read once with 128-bit loads and lives in fp32 registers; its sums are reduced across lanes (DPP) and
+// wavefronts (LDS), the output is written with 128-bit stores.  One wavefront per row for short rows, one
+// workgroup per row for long rows.
 #pragma once
 
 #include "hk_norm.h"
 
 namespace hk {
 
-// T: element type; NV: 16-byte vectors per thread; WAVE_ROW: one wavefront per row (4 rows per 256-thread block)
-// instead of one workgroup per row; HAS_RES: x = x0 + residual is formed in fp32 and optionally written back;
-// IS_RMS: RMSNorm (no centring, no bias term in the statistics).
+// T: element type; NV: 16-byte vectors per thread and row; WAVE_ROW: one wavefront per row (4 rows per 256-thread
+// block) instead of one workgroup per row; HAS_RES: x = x0 + residual is formed in fp32 and optionally written
+// back; IS_RMS: RMSNorm (no centring, no bias term in the statistics); R: rows a workgroup takes, 1 or 2.
+//
+// With R > 1 a thread holds its columns of R consecutive rows: all their loads are issued back to back, each
+// reduction carries every row's sums through one barrier, and gamma / beta are fetched once for the lot.  The
+// parameter fetches go through the compute unit's vector cache like the rows themselves and are as many bytes per
+// row as the row: with gamma and beta a one-row workgroup moves three rows' worth through that cache for every
+// row it reads, and the kernel pays for it (4096 bf16 columns, 32768 rows: 86 us with gamma alone, 92 us with
+// gamma and beta).
 //
 // Every row operand is addressed through a buffer descriptor of exactly one row (base = the row's first byte,
 // size = cols * sizeof(T)): the hardware returns zeros for a lane past the row's end and drops its stores, so no
-// memory instruction sits inside a branch and all of a thread's loads are issued back to back.
+// memory instruction sits inside a branch and all of a thread's loads are issued back to back.  The second row of
+// the last workgroup of an odd number of rows gets an empty descriptor in the same way.
 //
-// The row is unpacked to fp32 registers once (at most 64 per thread) and, for LayerNorm, centred in place by the
-// second statistics pass, so the normalisation costs one multiply and one multiply-add per element.  Which values
-// stay in registers across the reductions is written out here rather than left to the compiler: with the row kept
-// packed and unpacked again per pass, unrelated edits moved the 5120-column bf16 kernel between 57.7 and 61 us.
-template <typename T, int NV, bool WAVE_ROW, bool HAS_RES, bool IS_RMS>
-__global__ __launch_bounds__(WAVE_ROW ? 256 : 1024)
+// A row is unpacked to fp32 registers once and, for LayerNorm, centred in place by the second statistics pass, so
+// the normalisation costs one multiply and one multiply-add per element.  Which values stay in registers across
+// the reductions is written out here rather than left to the compiler: with the row kept packed and unpacked again
+// per pass, unrelated edits moved the 5120-column bf16 kernel between 57.7 and 61 us.
+template <typename T, int NV, bool WAVE_ROW, bool HAS_RES, bool IS_RMS, int R>
+__global__ __launch_bounds__(WAVE_ROW ? 256 : (R >= 2 ? 512 : 1024))   // several rows: at most 512 threads
 void norm_fwd_kernel(NormFwdArgs a) {
+  static_assert(R == 1 || !WAVE_ROW, "a wavefront takes one row");
   constexpr int VEC = VecIO<T>::N;
   constexpr int NE = NV * VEC;
-  __shared__ float red[kMaxWaves * 3];
+  __shared__ __align__(16) float red[2][kMaxWaves * 2 * R];   // one slot per reduction of the kernel
 
   const int tpr = WAVE_ROW ? kWave : int(blockDim.x);
   const int t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
-  const int64_t row = WAVE_ROW
+  const int64_t row0 = WAVE_ROW
       ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index()
-      : int64_t(blockIdx.x);
-  if (WAVE_ROW && row >= a.rows) return;  // wave-uniform; no block barrier in this mode
+      : int64_t(blockIdx.x) * R;
+  if (WAVE_ROW && row0 >= a.rows) return;  // wave-uniform; no block barrier in this mode
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
-  const uint32_t row_bytes = uint32_t(a.nvec) * 16u;
   auto off = [&](int i) { return uint32_t(i * tpr + t) * 16u; };   // vector i of thread t, in bytes from the row's start
   // long rows: stops the scheduler from unpacking every vector of a pass before the first one is consumed
-  auto fence = [] { if constexpr (NV >= 8) __builtin_amdgcn_sched_barrier(0); };
+  auto fence = [] { if constexpr (NV * R >= 8) __builtin_amdgcn_sched_barrier(0); };
 
-  float v[NE];
+  // row r of this workgroup; one past the end is addressed as the first row with a size of zero bytes
+  int64_t rowi[R];
+  uint32_t bytes[R];
+  bool live[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    live[r] = r == 0 || row0 + r < a.rows;
+    rowi[r] = live[r] ? row0 + r : row0;
+    bytes[r] = live[r] ? uint32_t(a.nvec) * 16u : 0u;
+  }
+
+  float v[R][NE];
   {
-    const BufferRsrc xr = make_rsrc(static_cast<const T*>(a.x) + row * a.x_pitch, row_bytes);
-    u32x4 raw[NV];
+    u32x4 raw[R][NV];
 #pragma unroll
-    for (int i = 0; i < NV; ++i) raw[i] = buf_ld16<kBufStream>(xr, off(i));
+    for (int r = 0; r < R; ++r) {
+      const BufferRsrc xr = make_rsrc(static_cast<const T*>(a.x) + rowi[r] * a.x_pitch, bytes[r]);
+#pragma unroll
+      for (int i = 0; i < NV; ++i) raw[r][i] = buf_ld16<kBufStream>(xr, off(i));
+    }
     if constexpr (HAS_RES) {
-      const BufferRsrc rr = make_rsrc(static_cast<const T*>(a.residual) + row * a.res_pitch, row_bytes);
-      u32x4 res[NV];
+      u32x4 res[R][NV];
 #pragma unroll
-      for (int i = 0; i < NV; ++i) res[i] = buf_ld16<kBufStream>(rr, off(i));
-      // an absent x_out becomes an empty buffer: its stores are dropped by the bounds check
-      const BufferRsrc xo = make_rsrc(a.x_out ? static_cast<T*>(a.x_out) + row * a.xout_pitch : static_cast<T*>(a.y),
-                                      a.x_out ? row_bytes : 0u);
+      for (int r = 0; r < R; ++r) {
+        const BufferRsrc rr = make_rsrc(static_cast<const T*>(a.residual) + rowi[r] * a.res_pitch, bytes[r]);
 #pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        float f1[VEC];
-        VecIO<T>::unpack(raw[i], &v[i * VEC]);
-        VecIO<T>::unpack(res[i], f1);
+        for (int i = 0; i < NV; ++i) res[r][i] = buf_ld16<kBufStream>(rr, off(i));
+      }
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) v[i * VEC + j] += f1[j];
-        buf_st16<kBufStream>(xo, off(i), VecIO<T>::pack(&v[i * VEC]));
+      for (int r = 0; r < R; ++r) {
+        // an absent x_out becomes an empty buffer: its stores are dropped by the bounds check
+        const BufferRsrc xo = make_rsrc(a.x_out ? static_cast<T*>(a.x_out) + rowi[r] * a.xout_pitch
+                                                : static_cast<T*>(a.y), a.x_out ? bytes[r] : 0u);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          float f1[VEC];
+          VecIO<T>::unpack(raw[r][i], &v[r][i * VEC]);
+          VecIO<T>::unpack(res[r][i], f1);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[r][i * VEC + j] += f1[j];
+          buf_st16<kBufStream>(xo, off(i), VecIO<T>::pack(&v[r][i * VEC]));
+        }
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < NV; ++i) { fence(); VecIO<T>::unpack(raw[i], &v[i * VEC]); }
+      for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) { fence(); VecIO<T>::unpack(raw[r][i], &v[r][i * VEC]); }
+      }
     }
   }
 
-  // sums over the group of threads that holds the row; the two reductions of a kernel use separate LDS slots,
+  // sums over the group of threads that holds the rows; the two reductions of a kernel use separate LDS slots,
   // so no barrier is needed between them
-  auto allred = [&](float x, int slot) -> float {
-    SumTuple<1> s;
-    s.v[0] = x;
-    s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red + slot * kMaxWaves, 0, nwaves);
-    return s.v[0];
+  auto allred = [&](auto s, int slot) {
+    if constexpr (WAVE_ROW) return wave_allreduce_tuple(s);
+    else return group_allreduce_tuple(s, red[slot], 0, nwaves);
   };
 
-  float mu, rs, var;
+  float mu[R], rs[R], var[R];
   if constexpr (IS_RMS) {
-    // lanes past the row's end hold zeros, which add nothing to either sum
-    float s0 = 0.f, ss = 0.f;
+    // lanes past the row's end hold zeros, which add nothing to either sum; one reduction carries both sums
+    SumTuple<2 * R> both;
 #pragma unroll
-    for (int e = 0; e < NE; ++e) { s0 += v[e]; ss = fmaf(v[e], v[e], ss); }
-    const float ms = allred(ss, 0) * a.inv_cols;   // mean(x^2) = var + mu^2
-    mu = allred(s0, 1) * a.inv_cols;
-    var = fmaxf(ms - mu * mu, 0.f);
-    rs = 1.0f / sqrtf(ms + a.eps);
+    for (int r = 0; r < R; ++r) {
+      float s0 = 0.f, ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < NE; ++e) { s0 += v[r][e]; ss = fmaf(v[r][e], v[r][e], ss); }
+      both.v[2 * r] = ss;
+      both.v[2 * r + 1] = s0;
+    }
+    both = allred(both, 0);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float ms = both.v[2 * r] * a.inv_cols;   // mean(x^2) = var + mu^2
+      mu[r] = both.v[2 * r + 1] * a.inv_cols;
+      var[r] = fmaxf(ms - mu[r] * mu[r], 0.f);
+      rs[r] = 1.0f / sqrtf(ms + a.eps);
+    }
   } else {
     // Two passes over the registers: the mean first, then the sum of squares about it, each reduced over the
     // group.  Centring on the row's own mean keeps fp32 accuracy for rows with an outlier, a large common offset
     // or no variance at all.  The centred values replace the row in the registers.
-    float s = 0.f;
+    SumTuple<R> s1, s2;
 #pragma unroll
-    for (int e = 0; e < NE; ++e) s += v[e];            // zeros past the end
-    mu = allred(s, 0) * a.inv_cols;
-    float m2 = 0.f;
-    if (a.nvec == NV * tpr) {                            // uniform: the row fills every lane's every vector
+    for (int r = 0; r < R; ++r) {
+      float s = 0.f;
 #pragma unroll
-      for (int e = 0; e < NE; ++e) {
-        v[e] -= mu;
-        m2 = fmaf(v[e], v[e], m2);
+      for (int e = 0; e < NE; ++e) s += v[r][e];         // zeros past the end
+      s1.v[r] = s;
+    }
+    s1 = allred(s1, 0);
+#pragma unroll
+    for (int r = 0; r < R; ++r) mu[r] = s1.v[r] * a.inv_cols;
+    if (a.nvec == NV * tpr) {                            // uniform: a row fills every lane's every vector
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float m2 = 0.f;
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+          v[r][e] -= mu[r];
+          m2 = fmaf(v[r][e], v[r][e], m2);
+        }
+        s2.v[r] = m2;
       }
     } else {
       // a lane past the row's end holds -mu, not data: its vectors are left out.  Kept apart from the full-row
       // case, whose straight-line code the per-vector selects would break up (57.8 against 61 us at 5120 bf16
       // columns).
 #pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        float q = 0.f;
+      for (int r = 0; r < R; ++r) {
+        float m2 = 0.f;
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          v[i * VEC + j] -= mu;
-          q = fmaf(v[i * VEC + j], v[i * VEC + j], q);
+        for (int i = 0; i < NV; ++i) {
+          float q = 0.f;
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            v[r][i * VEC + j] -= mu[r];
+            q = fmaf(v[r][i * VEC + j], v[r][i * VEC + j], q);
+          }
+          m2 += (i * tpr + t < a.nvec) ? q : 0.f;
         }
-        m2 += (i * tpr + t < a.nvec) ? q : 0.f;
+        s2.v[r] = m2;
       }
     }
-    var = allred(m2, 1) * a.inv_cols;
-    rs = 1.0f / sqrtf(var + a.eps);
+    s2 = allred(s2, 1);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      var[r] = s2.v[r] * a.inv_cols;
+      rs[r] = 1.0f / sqrtf(var[r] + a.eps);
+    }
   }
 
   if (t == 0) {
-    store_stat<T>(a.mean, row, mu, a.stats_f32);
-    store_stat<T>(a.stat, row, a.stat_kind == HK_STAT_VAR ? var : rs, a.stats_f32);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (live[r]) {
+        store_stat<T>(a.mean, rowi[r], mu[r], a.stats_f32);
+        store_stat<T>(a.stat, rowi[r], a.stat_kind == HK_STAT_VAR ? var[r] : rs[r], a.stats_f32);
+      }
+    }
   }
 
-  const BufferRsrc yr = make_rsrc(static_cast<T*>(a.y) + row * a.y_pitch, row_bytes);
-  // gamma / beta are fetched after the reduction: every fetch is a miss in the compute unit's own cache (the
-  // rows stream through it) and holds one of its outstanding-request slots until the data is back; issued
-  // before the row has arrived they would hold those slots for the whole HBM latency instead of the L2's.
-  // The four cases of missing parameters are separate straight-line copies, so that no fetch sits inside a branch.
+  BufferRsrc yr[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) yr[r] = make_rsrc(static_cast<T*>(a.y) + rowi[r] * a.y_pitch, bytes[r]);
+  const uint32_t row_bytes = uint32_t(a.nvec) * 16u;
+  // gamma / beta are fetched after the reduction: every fetch holds one of the compute unit's outstanding-request
+  // slots until the data is back; issued before the row has arrived they would hold those slots for the whole HBM
+  // latency instead of the L2's.  The four cases of missing parameters are separate straight-line copies, so that
+  // no fetch sits inside a branch.
   auto epilogue = [&](auto has_g, auto has_b) {
     constexpr bool HG = decltype(has_g)::value, HB = decltype(has_b)::value;
     const BufferRsrc gr = make_rsrc(HG ? a.gamma : a.y, row_bytes);   // an absent parameter is not fetched at all
     const BufferRsrc br = make_rsrc(HB ? a.beta : a.y, row_bytes);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      float f[VEC];
       [[maybe_unused]] float g[VEC], b[VEC];
       if constexpr (HG) VecIO<T>::unpack(buf_ld16<kBufKeep>(gr, off(i)), g);
       if constexpr (HB) VecIO<T>::unpack(buf_ld16<kBufKeep>(br, off(i)), b);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float n = rs * v[i * VEC + j];
-        f[j] = HG ? (HB ? fmaf(g[j], n, b[j]) : g[j] * n) : (HB ? n + b[j] : n);
+      for (int r = 0; r < R; ++r) {
+        float f[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float n = rs[r] * v[r][i * VEC + j];
+          f[j] = HG ? (HB ? fmaf(g[j], n, b[j]) : g[j] * n) : (HB ? n + b[j] : n);
+        }
+        buf_st16<kBufStream>(yr[r], off(i), VecIO<T>::pack(f));
       }
-      buf_st16<kBufStream>(yr, off(i), VecIO<T>::pack(f));
       // long rows: keep the compiler from hoisting every parameter fetch above the first store, which would
       // hold 2 * NV more vectors in registers than the row itself
       fence();
@@ -224,22 +294,43 @@ void norm_fwd_generic_kernel(NormFwdArgs a) {
   }
 }
 
+// the most rows a workgroup of the register kernel may take: two where both stay within 80 fp32 registers per
+// thread (64 with a residual row in flight next to each).  Four were measured too: 4096 bf16 columns 88.9 us
+// against 84.7 us for two and 86.2 us for one, 4096 fp32 columns 45.4 / 45.8 / 46.4 us.
+template <typename T>
+static constexpr int max_rows_per_block(int nv, bool has_res) {
+  const int floats = nv * VecIO<T>::N, budget = has_res ? 64 : 80;
+  return floats * 2 <= budget ? 2 : 1;
+}
+
+// rows_per_block: 1 or 2 (one-wavefront rows always 1)
+template <typename T, int NV, bool WAVE_ROW, bool HAS_RES, bool IS_RMS>
+static void launch_norm_fwd_width(const NormFwdArgs& a, int rows_per_block, dim3 grid, dim3 block, hipStream_t s) {
+  if constexpr (!WAVE_ROW && max_rows_per_block<T>(NV, HAS_RES) >= 2) {
+    if (rows_per_block == 2) {
+      HK_LAUNCH((norm_fwd_kernel<T, NV, false, HAS_RES, IS_RMS, 2>), grid, block, 0, s, a);
+      return;
+    }
+  }
+  HK_LAUNCH((norm_fwd_kernel<T, NV, WAVE_ROW, HAS_RES, IS_RMS, 1>), grid, block, 0, s, a);
+}
+
 template <typename T, bool WAVE_ROW, bool HAS_RES, bool IS_RMS>
-static int launch_norm_fwd_rms(const NormFwdArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
+static int launch_norm_fwd_rms(const NormFwdArgs& a, int nv, int rpb, dim3 grid, dim3 block, hipStream_t s) {
   profile_before(s);
   switch (nv) {
-    case 1: HK_LAUNCH((norm_fwd_kernel<T, 1, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 2: HK_LAUNCH((norm_fwd_kernel<T, 2, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 3: HK_LAUNCH((norm_fwd_kernel<T, 3, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 4: HK_LAUNCH((norm_fwd_kernel<T, 4, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 5: HK_LAUNCH((norm_fwd_kernel<T, 5, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 6: HK_LAUNCH((norm_fwd_kernel<T, 6, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
-    case 8: HK_LAUNCH((norm_fwd_kernel<T, 8, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a); break;
+    case 1: launch_norm_fwd_width<T, 1, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 2: launch_norm_fwd_width<T, 2, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 3: launch_norm_fwd_width<T, 3, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 4: launch_norm_fwd_width<T, 4, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 5: launch_norm_fwd_width<T, 5, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 6: launch_norm_fwd_width<T, 6, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 8: launch_norm_fwd_width<T, 8, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
     case 16:
       // sixteen vectors are 64 fp32 registers only for fp32 data; with a residual two packed rows of that length
       // are in flight on top
       if constexpr (sizeof(T) == 4 && !WAVE_ROW && !HAS_RES) {
-        HK_LAUNCH((norm_fwd_kernel<T, 16, WAVE_ROW, HAS_RES, IS_RMS>), grid, block, 0, s, a);
+        launch_norm_fwd_width<T, 16, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s);
         break;
       }
       [[fallthrough]];
@@ -252,9 +343,9 @@ static int launch_norm_fwd_rms(const NormFwdArgs& a, int nv, dim3 grid, dim3 blo
 }
 
 template <typename T, bool WAVE_ROW, bool HAS_RES>
-static int launch_norm_fwd_nv(const NormFwdArgs& a, int nv, dim3 grid, dim3 block, hipStream_t s) {
-  return a.is_rms ? launch_norm_fwd_rms<T, WAVE_ROW, HAS_RES, true>(a, nv, grid, block, s)
-                  : launch_norm_fwd_rms<T, WAVE_ROW, HAS_RES, false>(a, nv, grid, block, s);
+static int launch_norm_fwd_nv(const NormFwdArgs& a, int nv, int rpb, dim3 grid, dim3 block, hipStream_t s) {
+  return a.is_rms ? launch_norm_fwd_rms<T, WAVE_ROW, HAS_RES, true>(a, nv, rpb, grid, block, s)
+                  : launch_norm_fwd_rms<T, WAVE_ROW, HAS_RES, false>(a, nv, rpb, grid, block, s);
 }
 
 // Picks threads-per-row and vectors-per-thread for a row of `nvec` 16-byte
@@ -331,12 +422,22 @@ int norm_fwd_typed(NormFwdArgs a, hipStream_t s) {
   if (vec_ok && pick_row_shape(a.nvec, tune_get(TUNE_NORM_FWD_THREADS), max_nv, wave_nv, &threads, &nv)) {
     if (threads == 64) {
       dim3 grid(unsigned((a.rows + 3) / 4)), block(256);
-      return has_res ? launch_norm_fwd_nv<T, true, true>(a, nv, grid, block, s)
-                     : launch_norm_fwd_nv<T, true, false>(a, nv, grid, block, s);
+      return has_res ? launch_norm_fwd_nv<T, true, true>(a, nv, 1, grid, block, s)
+                     : launch_norm_fwd_nv<T, true, false>(a, nv, 1, grid, block, s);
     }
-    dim3 grid{unsigned(a.rows)}, block{unsigned(threads)};
-    return has_res ? launch_norm_fwd_nv<T, false, true>(a, nv, grid, block, s)
-                   : launch_norm_fwd_nv<T, false, false>(a, nv, grid, block, s);
+    // two rows per workgroup where both fit the registers (the same bound as in launch_norm_fwd_width) and the
+    // grid still fills the device many times over
+    int rpb = 1;
+    if (threads <= 512) {
+      const int most = max_rows_per_block<T>(nv, has_res);
+      const int want = tune_get(TUNE_NORM_FWD_ROWS);
+      if (want > 0) rpb = want >= 2 ? 2 : 1;
+      else rpb = a.rows >= 16 * int64_t(device_cu_count()) ? 2 : 1;
+      rpb = std::min(rpb, most);
+    }
+    dim3 grid{unsigned((a.rows + rpb - 1) / rpb)}, block{unsigned(threads)};
+    return has_res ? launch_norm_fwd_nv<T, false, true>(a, nv, rpb, grid, block, s)
+                   : launch_norm_fwd_nv<T, false, false>(a, nv, rpb, grid, block, s);
   }
   HK_LAUNCH((norm_fwd_generic_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
   return launch_check("norm_fwd_generic_kernel");

@@ -285,3 +285,65 @@ def test_layer_norm_statistics_conditioning(hk, cuda, dtype, cols):
     # as |y| ~ 1e-3 (the outlier owns the variance) from x - mean with mean ~ 0.6..300, so the half ulp of the mean
     # alone is percents of such an element, in any fp32 arithmetic.  It is still printed with the others.
     helpers.assert_close(ty, ey, dtype, "y", rtol=1e-4 if dtype == "fp32" else None, strict_rtol=1e-1)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(7, 4096), (9, 5120), (1, 4096), (5, 1000), (3, 2048 + 8), (6, 8192)])
+@pytest.mark.parametrize("is_rms", [True, False])
+@pytest.mark.parametrize("residual", [False, True])
+def test_forward_two_rows_per_workgroup(hk, cuda, dtype, shape, is_rms, residual):
+    """Large inputs give a workgroup two consecutive rows (one fetch of gamma / beta for the pair, the last
+    workgroup of an odd row count holding one row only).  Forced here on small inputs, next to the one-row launch:
+    both must match the oracle, and nothing past the last row may be written."""
+    import torch
+    rows, cols = shape
+    eps = 1e-6
+    x0, gamma, beta, _ = _inputs(rows, cols, dtype, 8100 + cols + rows)
+    res = helpers.draw(8200 + cols, (rows, cols), dtype=dtype) if residual else None
+    ez, exo, emu, ers = oracle.dropout_add_ln_fwd(x0, res, gamma, None if is_rms else beta, eps, is_rms)
+    tx0, tg, tb = (helpers.to_torch(v, dtype, cuda) for v in (x0, gamma, beta))
+    tres = helpers.to_torch(res, dtype, cuda) if residual else None
+    got = {}
+    try:
+        for rpb in (1, 2):
+            hk.tune_set("norm_fwd_rows", rpb)
+            tz = torch.full_like(tx0, float("nan"))
+            txo = torch.full_like(tx0, float("nan")) if residual else None
+            tmu = torch.full((rows,), float("nan"), dtype=torch.float32, device=cuda)
+            trs = torch.full((rows,), float("nan"), dtype=torch.float32, device=cuda)
+            hk.dropout_add_ln_fwd(tx0, tres, tg, None if is_rms else tb, tz, txo, tmu, trs, eps, is_rms)
+            torch.cuda.synchronize()
+            got[rpb] = (tz, txo, tmu, trs)
+    finally:
+        hk.tune_set("norm_fwd_rows", 0)
+    for rpb in (1, 2):
+        tz, txo, tmu, trs = got[rpb]
+        helpers.assert_close(tz, ez, dtype, "z")
+        helpers.assert_close(trs, ers, "fp32", "rsigma")
+        helpers.assert_close(tmu, emu, "fp32", "mu", scale=1.0)
+        if residual:
+            helpers.assert_close(txo, exo, dtype, "x")
+
+
+def test_forward_two_rows_per_workgroup_pitched(hk, cuda):
+    """The same on a column slice of a wider array, odd row count: nothing outside the slice is written."""
+    import torch
+    rows, cols, wide = 11, 4096, 4608
+    x = helpers.draw(8301, (rows, wide), dtype="bf16")
+    gamma = helpers.draw(8302, (cols,), "uniform", 0.5, 1.5, "bf16")
+    beta = helpers.draw(8303, (cols,), "normal", 0.0, 0.1, "bf16")
+    ey, emean, _, erstd = oracle.layernorm_fwd(x[:, :cols], gamma, beta, 1e-5)
+    tx = helpers.to_torch(x, "bf16", cuda)
+    tg, tb = helpers.to_torch(gamma, "bf16", cuda), helpers.to_torch(beta, "bf16", cuda)
+    ty = torch.full((rows, wide), 7.0, dtype=torch.bfloat16, device=cuda)
+    tmean = torch.empty(rows, dtype=torch.float32, device=cuda)
+    trstd = torch.empty(rows, dtype=torch.float32, device=cuda)
+    try:
+        hk.tune_set("norm_fwd_rows", 2)
+        hk.layer_norm_fwd(tx[:, :cols], tg, tb, ty[:, :cols], tmean, trstd, 1e-5, stat_kind=1)
+        torch.cuda.synchronize()
+    finally:
+        hk.tune_set("norm_fwd_rows", 0)
+    helpers.assert_close(ty[:, :cols], ey, "bf16", "y")
+    helpers.assert_close(trstd, erstd, "fp32", "rstd")
+    assert bool((ty[:, cols:] == 7.0).all())

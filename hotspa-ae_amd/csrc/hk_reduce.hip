@@ -106,7 +106,9 @@ struct RMax : RNoTransform {
     else return std::numeric_limits<A>::lowest();
   }
   template <typename A> static __device__ __forceinline__ A apply(A a, A b) {
-    return (is_nan(a) || a > b) ? a : (is_nan(b) ? b : (a > b ? a : b));
+    // fp32: the hardware's NaN-propagating maximum (one v_maximum3_f32)
+    if constexpr (std::is_same<A, float>::value) return __builtin_elementwise_maximum(a, b);
+    else return (is_nan(a) || a > b) ? a : (is_nan(b) ? b : (a > b ? a : b));
   }
 };
 struct RMin : RNoTransform {
@@ -115,7 +117,8 @@ struct RMin : RNoTransform {
     else return std::numeric_limits<A>::max();
   }
   template <typename A> static __device__ __forceinline__ A apply(A a, A b) {
-    return (is_nan(a) || a < b) ? a : (is_nan(b) ? b : (a < b ? a : b));
+    if constexpr (std::is_same<A, float>::value) return __builtin_elementwise_minimum(a, b);
+    else return (is_nan(a) || a < b) ? a : (is_nan(b) ? b : (a < b ? a : b));
   }
 };
 // R without its load transform: what folds partial results, which went through pre() when they were formed

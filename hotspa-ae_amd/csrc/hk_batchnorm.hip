@@ -212,7 +212,7 @@ __device__ __forceinline__ IT bn_channel(IT v, IT hw_vec, IT C, bool& uniform) {
 template <typename T, int V, typename CT, typename IT>
 __global__ __launch_bounds__(256)
 void bn_apply_kernel(const T* x, T* y, const CT* __restrict__ coef, IT total_loads, IT hw_vec, IT C) {
-  const IT v = IT(blockIdx.x) * 256 + threadIdx.x;
+  const IT v = IT(blockIdx.x) * kStreamThreads + threadIdx.x;
   if (v >= total_loads) return;
   BnRaw<T, V> rx;
   rx.load(x + size_t(v) * V);
@@ -286,7 +286,7 @@ template <typename T, int V, typename CT, typename IT>
 __global__ __launch_bounds__(256)
 void bn_bwd_apply_kernel(const T* dy, const T* x, T* dx, const CT* __restrict__ coef, IT total_loads, IT hw_vec,
                          IT C) {
-  const IT v = IT(blockIdx.x) * 256 + threadIdx.x;
+  const IT v = IT(blockIdx.x) * kStreamThreads + threadIdx.x;
   if (v >= total_loads) return;
   BnRaw<T, V> rg, rx;
   rg.load(dy + size_t(v) * V);
@@ -351,7 +351,7 @@ static int bn_fwd_typed(const void* x, const void* scale, const void* bias, void
     constexpr int V = decltype(vtag)::value;
     const BnShape s = bn_shape<V>(N, C, HW);
     CT* coef = part + size_t(C) * size_t(s.splits) * 3;
-    HK_REQUIRE(C <= 0x7fffffffLL && (N * C * s.hw_vec + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID,
+    HK_REQUIRE(C <= 0x7fffffffLL && (N * C * s.hw_vec + kStreamThreads - 1) / kStreamThreads <= 0x7fffffffLL, HK_ERR_INVALID,
                "hk_batch_norm_fwd: array too large");
     HK_LAUNCH((bn_stats_kernel<T, V, CT>), dim3(unsigned(C), unsigned(s.splits)), dim3(256), 0, st, xp, s, part);
     int rc = launch_check("bn_stats_kernel");
@@ -365,10 +365,10 @@ static int bn_fwd_typed(const void* x, const void* scale, const void* bias, void
     const int64_t loads = N * C * s.hw_vec;
     profile_before(st);
     if (loads < 0x7fffffffLL) {
-      HK_LAUNCH((bn_apply_kernel<T, V, CT, uint32_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st,
+      HK_LAUNCH((bn_apply_kernel<T, V, CT, uint32_t>), dim3(unsigned((loads + kStreamThreads - 1) / kStreamThreads)), dim3(kStreamThreads), 0, st,
                          xp, yp, coef, uint32_t(loads), uint32_t(s.hw_vec), uint32_t(C));
     } else {
-      HK_LAUNCH((bn_apply_kernel<T, V, CT, int64_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0, st,
+      HK_LAUNCH((bn_apply_kernel<T, V, CT, int64_t>), dim3(unsigned((loads + kStreamThreads - 1) / kStreamThreads)), dim3(kStreamThreads), 0, st,
                          xp, yp, coef, loads, s.hw_vec, C);
     }
     profile_after(st);
@@ -394,7 +394,7 @@ static int bn_bwd_typed(const void* dy, const void* x, const void* scale, void* 
     constexpr int V = decltype(vtag)::value;
     const BnShape s = bn_shape<V>(N, C, HW);
     CT* coef = part + size_t(C) * size_t(s.splits) * 3;
-    HK_REQUIRE(C <= 0x7fffffffLL && (N * C * s.hw_vec + 255) / 256 <= 0x7fffffffLL, HK_ERR_INVALID,
+    HK_REQUIRE(C <= 0x7fffffffLL && (N * C * s.hw_vec + kStreamThreads - 1) / kStreamThreads <= 0x7fffffffLL, HK_ERR_INVALID,
                "hk_batch_norm_bwd: array too large");
     HK_LAUNCH((bn_bwd_stats_kernel<T, V, PT, CT>), dim3(unsigned(C), unsigned(s.splits)), dim3(256), 0, st,
                        static_cast<const T*>(dy), static_cast<const T*>(x), s, static_cast<const PT*>(save_mean),
@@ -409,11 +409,11 @@ static int bn_bwd_typed(const void* dy, const void* x, const void* scale, void* 
     const int64_t loads = N * C * s.hw_vec;
     profile_before(st);
     if (loads < 0x7fffffffLL) {
-      HK_LAUNCH((bn_bwd_apply_kernel<T, V, CT, uint32_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0,
+      HK_LAUNCH((bn_bwd_apply_kernel<T, V, CT, uint32_t>), dim3(unsigned((loads + kStreamThreads - 1) / kStreamThreads)), dim3(kStreamThreads), 0,
                          st, static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<T*>(dx), coef,
                          uint32_t(loads), uint32_t(s.hw_vec), uint32_t(C));
     } else {
-      HK_LAUNCH((bn_bwd_apply_kernel<T, V, CT, int64_t>), dim3(unsigned((loads + 255) / 256)), dim3(256), 0,
+      HK_LAUNCH((bn_bwd_apply_kernel<T, V, CT, int64_t>), dim3(unsigned((loads + kStreamThreads - 1) / kStreamThreads)), dim3(kStreamThreads), 0,
                          st, static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<T*>(dx), coef, loads,
                          s.hw_vec, C);
     }

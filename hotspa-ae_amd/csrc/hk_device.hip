@@ -118,20 +118,21 @@ __global__ __launch_bounds__(256) void fill_bytes_kernel(uint8_t* dst, uint32_t 
   }
 }
 
+// the copy in the shape that streams fastest: one-wavefront workgroups, non-temporal loads and stores
 template <int UNROLL>
-__global__ __launch_bounds__(256) void copy16_kernel(u32x4* __restrict__ dst,
-                                                     const u32x4* __restrict__ src, size_t nvec) {
-  const size_t base = (size_t(blockIdx.x) * UNROLL) * 256 + threadIdx.x;
+__global__ __launch_bounds__(kStreamThreads) void copy16_kernel(u32x4* __restrict__ dst,
+                                                                const u32x4* __restrict__ src, size_t nvec) {
+  const size_t base = (size_t(blockIdx.x) * UNROLL) * kStreamThreads + threadIdx.x;
   u32x4 v[UNROLL];
 #pragma unroll
   for (int i = 0; i < UNROLL; ++i) {
-    size_t idx = base + size_t(i) * 256;
-    if (idx < nvec) v[i] = src[idx];
+    size_t idx = base + size_t(i) * kStreamThreads;
+    if (idx < nvec) v[i] = ld16(src + idx);
   }
 #pragma unroll
   for (int i = 0; i < UNROLL; ++i) {
-    size_t idx = base + size_t(i) * 256;
-    if (idx < nvec) dst[idx] = v[i];
+    size_t idx = base + size_t(i) * kStreamThreads;
+    if (idx < nvec) st16_stream(dst + idx, v[i]);
   }
 }
 
@@ -352,10 +353,10 @@ int hk_copy_kernel(void* dst, const void* src, size_t bytes, hkStream_t stream) 
              "hk_copy_kernel: needs 16-byte aligned pointers and size");
   constexpr int UNROLL = 1;
   size_t nvec = bytes / 16;
-  size_t blocks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
+  size_t blocks = (nvec + kStreamThreads * UNROLL - 1) / (kStreamThreads * UNROLL);
   HK_REQUIRE(blocks <= 0x7fffffffu, HK_ERR_INVALID, "hk_copy_kernel: size too large");
   profile_before(as_hip(stream));
-  HK_LAUNCH(copy16_kernel<UNROLL>, dim3(unsigned(blocks)), dim3(256), 0, as_hip(stream),
+  HK_LAUNCH(copy16_kernel<UNROLL>, dim3(unsigned(blocks)), dim3(kStreamThreads), 0, as_hip(stream),
                      static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), nvec);
   profile_after(as_hip(stream));
   return launch_check("copy16_kernel");

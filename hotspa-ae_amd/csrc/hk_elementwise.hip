@@ -59,9 +59,9 @@ template <typename T> constexpr bool ew_vectorised() {
 // unary, and binary with a constant (REV: constant op x instead of x op constant)
 // ---------------------------------------------------------------------------
 template <typename T, int OP>
-__global__ __launch_bounds__(256) void ew_unary_vec_kernel(const T* in, T* out, int64_t nvec) {
+__global__ __launch_bounds__(kStreamThreads) void ew_unary_vec_kernel(const T* in, T* out, int64_t nvec) {
   constexpr int VEC = VecIO<T>::N;
-  const int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t v = int64_t(blockIdx.x) * kStreamThreads + threadIdx.x;
   if (v >= nvec) return;
   float f[VEC];
   VecIO<T>::unpack(ld16(in + v * VEC), f);
@@ -78,10 +78,10 @@ __global__ __launch_bounds__(256) void ew_unary_scalar_kernel(const T* in, T* ou
 }
 
 template <typename T, int OP, bool REV>
-__global__ __launch_bounds__(256) void ew_const_vec_kernel(const T* in, float c, T* out,
-                                                           int64_t nvec) {
+__global__ __launch_bounds__(kStreamThreads) void ew_const_vec_kernel(const T* in, float c, T* out,
+                                                                      int64_t nvec) {
   constexpr int VEC = VecIO<T>::N;
-  const int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t v = int64_t(blockIdx.x) * kStreamThreads + threadIdx.x;
   if (v >= nvec) return;
   float f[VEC];
   VecIO<T>::unpack(ld16(in + v * VEC), f);
@@ -133,10 +133,10 @@ struct EwRaw {
 // out[r, c] = a[..] op b[..] over a [rows, cols] output; cols_vec = vectors per output row; AM / BM say how
 // each operand maps onto the output.
 template <typename T, int OP, int AM, int BM>
-__global__ __launch_bounds__(256) void ew_binary_2d_vec_kernel(const T* a, const T* b, T* out, uint32_t nvec,
+__global__ __launch_bounds__(kStreamThreads) void ew_binary_2d_vec_kernel(const T* a, const T* b, T* out, uint32_t nvec,
                                                                uint32_t cols_vec) {
   constexpr int VEC = VecIO<T>::N;
-  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t v = blockIdx.x * uint32_t(kStreamThreads) + threadIdx.x;
   if (v >= nvec) return;
   uint32_t r = 0, c = v;
   if constexpr (AM != EW_FULL || BM != EW_FULL) {
@@ -224,6 +224,7 @@ __global__ __launch_bounds__(256) void ew_broadcast_generic_kernel(const T* a, d
 // host side
 // ---------------------------------------------------------------------------
 static inline unsigned blocks_for(int64_t n) { return unsigned((n + 255) / 256); }
+static inline unsigned stream_blocks_for(int64_t nvec) { return unsigned((nvec + kStreamThreads - 1) / kStreamThreads); }
 
 template <typename T, int OP>
 static int unary_launch(const void* in, void* out, int64_t n, hipStream_t s) {
@@ -232,7 +233,7 @@ static int unary_launch(const void* in, void* out, int64_t n, hipStream_t s) {
   if constexpr (ew_vectorised<T>()) {
     constexpr int VEC = VecIO<T>::N;
     if (n % VEC == 0 && aligned16(in) && aligned16(out)) {
-      HK_LAUNCH((ew_unary_vec_kernel<T, OP>), dim3(blocks_for(n / VEC)), dim3(256), 0, s,
+      HK_LAUNCH((ew_unary_vec_kernel<T, OP>), dim3(stream_blocks_for(n / VEC)), dim3(kStreamThreads), 0, s,
                          static_cast<const T*>(in), static_cast<T*>(out), n / VEC);
       profile_after(s);
       return launch_check("ew_unary_vec_kernel");
@@ -252,7 +253,7 @@ static int const_launch(const void* in, double c, void* out, int64_t n, hipStrea
   if constexpr (ew_vectorised<T>()) {
     constexpr int VEC = VecIO<T>::N;
     if (n % VEC == 0 && aligned16(in) && aligned16(out)) {
-      HK_LAUNCH((ew_const_vec_kernel<T, OP, REV>), dim3(blocks_for(n / VEC)), dim3(256), 0, s,
+      HK_LAUNCH((ew_const_vec_kernel<T, OP, REV>), dim3(stream_blocks_for(n / VEC)), dim3(kStreamThreads), 0, s,
                          static_cast<const T*>(in), float(c), static_cast<T*>(out), n / VEC);
       profile_after(s);
       return launch_check("ew_const_vec_kernel");
@@ -325,7 +326,7 @@ static int binary_launch(const void* a, const void* b, void* out, const EwDims& 
       if (am >= 0 && bm >= 0 && (am == EW_FULL || bm == EW_FULL) && cols % VEC == 0 && aligned16(out) &&
           vec_ok(a, am) && vec_ok(b, bm) && n / VEC < 0x7fffffffLL) {
         const uint32_t nvec = uint32_t(n / VEC), cols_vec = uint32_t(cols / VEC);
-        const dim3 grid(blocks_for(nvec)), block(256);
+        const dim3 grid(stream_blocks_for(nvec)), block(kStreamThreads);
 #define HK_EW_2D(AM, BM) \
   HK_LAUNCH((ew_binary_2d_vec_kernel<T, OP, AM, BM>), grid, block, 0, s, pa, pb, po, nvec, cols_vec)
         if (am == EW_FULL) {

@@ -737,11 +737,11 @@ void norm_grad_kernel(const T* __restrict__ x, const T* __restrict__ norm, const
 // exponent at compile time (1, 2, or 0 for any other) so that nothing but the arithmetic sits between the loads
 // and the store; the per-row factor is formed once per thread.
 template <typename T, int PK>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(kStreamThreads)
 void norm_grad_rows_vec_kernel(const T* __restrict__ x, const T* __restrict__ norm, const T* __restrict__ grad,
                                T* out, uint32_t nvec, uint32_t cols_vec, int64_t p) {
   constexpr int VEC = VecIO<T>::N;
-  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t v = blockIdx.x * uint32_t(kStreamThreads) + threadIdx.x;
   if (v >= nvec) return;
   const uint32_t r = v / cols_vec;
   const u32x4 raw = ld16(x + size_t(v) * VEC);
@@ -776,7 +776,7 @@ static int norm_grad_typed(const void* x, const void* norm, const void* grad, vo
       auto kernel = p == 1 ? norm_grad_rows_vec_kernel<T, 1>
                   : p == 2 ? norm_grad_rows_vec_kernel<T, 2> : norm_grad_rows_vec_kernel<T, 0>;
       profile_before(s);
-      HK_LAUNCH(kernel, dim3((nvec + 255) / 256), dim3(256), 0, s,
+      HK_LAUNCH(kernel, dim3((nvec + kStreamThreads - 1) / kStreamThreads), dim3(kStreamThreads), 0, s,
                          static_cast<const T*>(x), static_cast<const T*>(norm), static_cast<const T*>(grad),
                          static_cast<T*>(out), nvec, uint32_t(reduce_size / VEC), p);
       profile_after(s);

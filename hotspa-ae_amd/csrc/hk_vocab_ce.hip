@@ -32,11 +32,11 @@ void vocab_ce_gather_kernel(const T* __restrict__ logits, const int64_t* __restr
 // out[r, c] = (softmax[r, c] - [c == labels[r] - vocab_start]) * grad_loss[r]; the comparison is made on
 // unsigned 64-bit values, so a label outside the shard (or a negative one) matches no column.
 template <typename T>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(kStreamThreads)
 void vocab_ce_bwd_vec_kernel(const T* softmax, const int64_t* __restrict__ labels, const T* __restrict__ grad_loss,
                              T* out, uint32_t nvec, uint32_t cols_vec, int64_t vocab_start) {
   constexpr int VEC = VecIO<T>::N;
-  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t v = blockIdx.x * uint32_t(kStreamThreads) + threadIdx.x;
   if (v >= nvec) return;
   const uint32_t r = v / cols_vec;
   const uint32_t c0 = (v - r * cols_vec) * VEC;
@@ -100,13 +100,13 @@ void vocab_ce_combine_kernel(const float* __restrict__ stats, int nshards, const
 
 // out[r, c] = (exp(x[r, c] - lse[r]) - [c == labels[r] - vocab_start]) * grad_loss[r]; zeros for an ignored row
 template <typename T>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(kStreamThreads)
 void vocab_ce_bwd_fused_kernel(const T* x, const int64_t* __restrict__ labels, const float* __restrict__ lse,
                                const T* __restrict__ grad_loss, T* out, uint32_t nvec, uint32_t cols_vec,
                                int64_t vocab_start, int64_t ignored_index) {
   constexpr int VEC = VecIO<T>::N;
   constexpr float kLog2e = 1.4426950408889634f;
-  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t v = blockIdx.x * uint32_t(kStreamThreads) + threadIdx.x;
   if (v >= nvec) return;
   const uint32_t r = v / cols_vec;
   const uint32_t c0 = (v - r * cols_vec) * VEC;
@@ -172,7 +172,7 @@ static int vocab_bwd_fused_typed(const void* x, const int64_t* labels, const flo
     if (cols % VEC == 0 && aligned16(x) && aligned16(out) && total / VEC < 0x7fffffffLL) {
       const uint32_t nvec = uint32_t(total / VEC);
       profile_before(s);
-      HK_LAUNCH((vocab_ce_bwd_fused_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
+      HK_LAUNCH((vocab_ce_bwd_fused_kernel<T>), dim3((nvec + kStreamThreads - 1) / kStreamThreads), dim3(kStreamThreads), 0, s,
                          static_cast<const T*>(x), labels, lse, static_cast<const T*>(grad_loss), static_cast<T*>(out),
                          nvec, uint32_t(cols / VEC), vocab_start, ignored_index);
       profile_after(s);
@@ -198,7 +198,7 @@ static int vocab_bwd_typed(const void* softmax, const int64_t* labels, const voi
     if (cols % VEC == 0 && aligned16(softmax) && aligned16(out) && total / VEC < 0x7fffffffLL) {
       const uint32_t nvec = uint32_t(total / VEC);
       profile_before(s);
-      HK_LAUNCH((vocab_ce_bwd_vec_kernel<T>), dim3((nvec + 255) / 256), dim3(256), 0, s,
+      HK_LAUNCH((vocab_ce_bwd_vec_kernel<T>), dim3((nvec + kStreamThreads - 1) / kStreamThreads), dim3(kStreamThreads), 0, s,
                          static_cast<const T*>(softmax), labels, static_cast<const T*>(grad_loss),
                          static_cast<T*>(out), nvec, uint32_t(cols / VEC), vocab_start);
       profile_after(s);

@@ -546,9 +546,9 @@ CASES = [
 
 
 # HBM bytes one launch of the RMSNorm backward kernel moves at the headline shape: rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE read 262985.0 and 270336.0 KiB per dispatch; a 256 MiB copy kernel calibrates the counters at
-# x2.000 (FETCH_SIZE reads 131086 KiB for 262144 KiB fetched) and x1.000 (WRITE_SIZE).
-NORM_BWD_TRAFFIC_BYTES = int((262985.0 * 2.0 + 270336.0 * 1.0) * 1024)
+# --pmc WRITE_SIZE read 262868.3 and 270336.0 KiB per dispatch; a 256 MiB copy kernel calibrates the counters at
+# x1.99986 (FETCH_SIZE reads 131081.5 KiB for 262144 KiB fetched) and x1.000 (WRITE_SIZE).
+NORM_BWD_TRAFFIC_BYTES = int((262868.3 * 1.99986 + 270336.0 * 1.0) * 1024)
 
 
 def preroll(torch, launch, min_steps=PREROLL_MIN_STEPS, min_seconds=PREROLL_MIN_SECONDS):
@@ -773,6 +773,8 @@ def main():
     ap.add_argument("--only", default="", help="substring filter for the kernels table (comma-separated: any of them)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table (headline only)")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="only the per-kernel table (with --only: only those cases run at all, e.g. under a counter pass)")
     ap.add_argument("--kernel-steps", type=int, default=KERNEL_STEPS, help="timed launches per kernels-table entry")
     ap.add_argument("--nsets", type=int, default=3, help="rotating buffer sets (working set > cache)")
     args = ap.parse_args()
@@ -786,13 +788,14 @@ def main():
     hk = _load()
     torch.cuda.set_device(0)
 
-    # headline: fwd + bwd at the Llama-7B token shape, exactly --steps steps after pre-roll and --warmup
-    step, step_bytes, rows = case_rmsnorm(hk, torch, args.nsets, "both")
-    ms, _, pre = time_case(hk, torch, step, args.steps, args.warmup, profile_main=False)
-    bwd, bwd_bytes, _ = case_rmsnorm(hk, torch, args.nsets, "bwd")
-    _, bwd_us, _ = time_case(hk, torch, bwd, max(args.steps, KERNEL_STEPS), args.warmup, profile_main=True)
-    del step, bwd
-    torch.cuda.empty_cache()
+    if not args.kernels_only:
+        # headline: fwd + bwd at the Llama-7B token shape, exactly --steps steps after pre-roll and --warmup
+        step, step_bytes, rows = case_rmsnorm(hk, torch, args.nsets, "both")
+        ms, _, pre = time_case(hk, torch, step, args.steps, args.warmup, profile_main=False)
+        bwd, bwd_bytes, _ = case_rmsnorm(hk, torch, args.nsets, "bwd")
+        _, bwd_us, _ = time_case(hk, torch, bwd, max(args.steps, KERNEL_STEPS), args.warmup, profile_main=True)
+        del step, bwd
+        torch.cuda.empty_cache()
 
     kernels = []
     for name, make in CASES:
@@ -816,6 +819,9 @@ def main():
         del launch
         torch.cuda.empty_cache()
 
+    if args.kernels_only:
+        print(json.dumps({"kernel_steps": args.kernel_steps, "kernels": kernels}), flush=True)
+        return
     achieved = bwd_bytes / bwd_us / 1e3
     out = {
         "metric": "HBM GB/s, RMSNorm fwd+bwd at Llama-7B token shape (algorithmic bytes / step time)",

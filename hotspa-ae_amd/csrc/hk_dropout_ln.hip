@@ -534,16 +534,18 @@ void dal_bwd_kernel(DalBwdArgs a) {
 // around a memory instruction, so the compiler counts outstanding loads exactly and PF rows stay in flight
 // per thread group (a ring of register slots refilled as soon as a slot has been unpacked); rows past the
 // end are clamped to the last row and their results dropped.
-template <typename IT, typename RT, typename WT, int PF>
-__global__ __launch_bounds__(1024)
+// TPR: the group width when the one group of a block is the whole block and its size is known at compile time
+// (512 threads = 4096 columns), else 0: the launch bound and the cross-wavefront step of the row sums follow it.
+template <typename IT, typename RT, typename WT, int PF, int TPR>
+__global__ __launch_bounds__(TPR ? TPR : 1024)
 void dal_bwd_stream_kernel(DalBwdArgs a) {
   constexpr int NI = kChunk / VecIO<IT>::N;   // 16-byte vectors per chunk of the input type
   constexpr int NR = kChunk / VecIO<RT>::N;   //                       ... of the residual type
-  __shared__ float red[2][kMaxWaves * 2];
-  const int tpr = a.tpr;
-  const int group = __builtin_amdgcn_readfirstlane(int(threadIdx.x) / tpr);
+  __shared__ __align__(16) float red[2][kMaxWaves * 2];
+  const int tpr = TPR ? TPR : a.tpr;
+  const int group = TPR ? 0 : __builtin_amdgcn_readfirstlane(int(threadIdx.x) / tpr);
   const int t = int(threadIdx.x) - group * tpr;
-  const int rpb = int(blockDim.x) / tpr;
+  const int rpb = TPR ? 1 : int(blockDim.x) / tpr;
   const int wpg = tpr >> 6;
   const int first_wave = group * wpg;
   const int col = t * kChunk;
@@ -609,7 +611,8 @@ void dal_bwd_stream_kernel(DalBwdArgs a) {
       s.v[0] += dy[j];
       s.v[1] = fmaf(dy[j], y[j], s.v[1]);
     }
-    s = group_allreduce_tuple(s, red[parity], first_wave, wpg);
+    if constexpr (TPR != 0) s = group_allreduce_tuple_fixed<SumTuple<2>, TPR / 64>(s, red[parity]);
+    else s = group_allreduce_tuple(s, red[parity], first_wave, wpg);
     parity ^= 1;
     if (valid) {
       const float mdy = a.is_rms ? 0.f : s.v[0] * a.inv_cols;
@@ -959,7 +962,8 @@ int hk_dropout_add_ln_bwd_ex(const hkDropoutAddLnBwdParams* pp, hkStream_t strea
     profile_before(s);
     // two rows in flight where the ring fits the registers (a 16-bit residual stream), else one
     constexpr int PF = sizeof(RT) == 2 ? 2 : 1;
-    if (stream_form) HK_LAUNCH((dal_bwd_stream_kernel<IT, RT, WT, PF>), grid, block, 0, s, a);
+    if (stream_form && sh.tpr == 512 && sh.block == 512) HK_LAUNCH((dal_bwd_stream_kernel<IT, RT, WT, PF, 512>), grid, block, 0, s, a);
+    else if (stream_form) HK_LAUNCH((dal_bwd_stream_kernel<IT, RT, WT, PF, 0>), grid, block, 0, s, a);
     else if (g1) HK_LAUNCH((dal_bwd_kernel<IT, RT, WT, false, true>), grid, block, 0, s, a);
     else if (colscale) HK_LAUNCH((dal_bwd_kernel<IT, RT, WT, true, false>), grid, block, 0, s, a);
     else HK_LAUNCH((dal_bwd_kernel<IT, RT, WT, false, false>), grid, block, 0, s, a);

@@ -41,8 +41,18 @@ void vocab_ce_bwd_vec_kernel(const T* softmax, const int64_t* __restrict__ label
   const uint32_t r = v / cols_vec;
   const uint32_t c0 = (v - r * cols_vec) * VEC;
   const u32x4 raw = ld16(softmax + size_t(v) * VEC);
-  const int64_t label = labels[r];
-  const float g = Cvt<T>::load(grad_loss + r);
+  // a wavefront almost always lies inside one row: then the row's label and gradient come through the scalar
+  // unit, one load per wavefront instead of one per lane
+  const uint32_t r0 = __builtin_amdgcn_readfirstlane(r);
+  int64_t label;
+  float g;
+  if (__builtin_amdgcn_ballot_w64(r != r0) == 0) {
+    label = labels[r0];
+    g = Cvt<T>::load(grad_loss + r0);
+  } else {
+    label = labels[r];
+    g = Cvt<T>::load(grad_loss + r);
+  }
   // position of the label inside this vector, or a value no j reaches (labels outside the shard, negative ones)
   const uint64_t rel = uint64_t(label) - uint64_t(vocab_start) - uint64_t(c0);
   const uint32_t hit = rel < uint64_t(VEC) ? uint32_t(rel) : 0xffffffffu;

@@ -276,6 +276,8 @@ def case_elementwise(hk, torch, nsets, which):
         return (lambda i: hk.binary("sub", xs[i % 2], per_row, outs[i % 2])), 2 * n * 2 + rows * 2, rows
     if which == "exp":
         return (lambda i: hk.unary("exp", xs[i % 2], outs[i % 2])), 2 * n * 2, rows
+    if which == "add":   # two dense operands of the same shape: the commonest element-wise call
+        return (lambda i: hk.binary("add", xs[i % 2], outs[(i + 1) % 2], outs[i % 2])), 3 * n * 2, rows
     if which == "div":
         return (lambda i: hk.binary("div", xs[i % 2], per_row, xs[i % 2])), 2 * n * 2 + rows * 2, rows
     g = torch.Generator(device="cuda").manual_seed(812)
@@ -512,6 +514,7 @@ CASES = [
     ("next: dropout(0.1)+residual+rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_dropout_ln(hk, t, 2, "fwd")),
     ("next: dropout(0.1)+residual+rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_dropout_ln(hk, t, 2, "bwd")),
     ("next: logits - row max bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "sub")),
+    ("next: dense + dense bf16 [16384x32000] (2R:1W)", lambda hk, t, n: case_elementwise(hk, t, n, "add")),
     ("next: exp bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "exp")),
     ("next: exp / row sum in place bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "div")),
     ("next: vocab-parallel CE bwd bf16 [16384x32000]", lambda hk, t, n: case_elementwise(hk, t, n, "vce")),

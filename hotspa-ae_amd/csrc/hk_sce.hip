@@ -171,26 +171,26 @@ void sce_sparse_bwd_kernel(SceArgs a) {
     return;
   }
   const T* xr = static_cast<const T*>(a.logits) + row * a.x_pitch;
+  // slots past the row's end hold -inf: they change neither the maximum nor the sum
   u32x4 raw[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int v = i * tpr + t;
-    raw[i] = u32x4{0, 0, 0, 0};
-    if (v < a.nvec) raw[i] = ld16(xr + v * VEC);
+    if ((i + 1) * tpr <= a.nvec) {       // uniform: every thread's slot i is inside the row
+      raw[i] = ld16(xr + v * VEC);
+    } else {
+      raw[i] = neg_inf_vec<T>();
+      if (v < a.nvec) raw[i] = ld16(xr + v * VEC);
+    }
   }
   const float g = sce_row_grad<T, float>(a, row);
   float e[NV * VEC];
-  float m = kNegInf;
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const bool ok = i * tpr + t < a.nvec;
-    VecIO<T>::unpack(raw[i], &e[i * VEC]);
+  for (int i = 0; i < NV; ++i) VecIO<T>::unpack(raw[i], &e[i * VEC]);
+  static_assert((NV * VEC) % 2 == 0, "pairs of elements per max3");
+  float m = fmaxf(e[0], e[1]);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      if (!ok) e[i * VEC + j] = kNegInf;
-      m = fmaxf(m, e[i * VEC + j]);
-    }
-  }
+  for (int k = 2; k < NV * VEC; k += 2) m = max3(m, e[k], e[k + 1]);
   const float ml = (m == kNegInf) ? 0.f : m * kLog2e;
   float s = 0.f;
 #pragma unroll

@@ -96,3 +96,22 @@ def test_refused_and_empty(hk, cuda):
     hk.batch_norm_fwd(c, torch.ones(2, device=cuda), torch.full((2,), 0.25, device=cuda), y, 0.1, 1e-5, None, None, sm, si)
     torch.cuda.synchronize()
     assert (y == 0.25).all() and (sm == 3.0).all() and torch.allclose(si, torch.full((2,), 1e-5 ** -0.5, device=cuda))
+
+
+@pytest.mark.parametrize("shape", [(0, 8, 4, 4), (4, 0, 4, 4), (4, 8, 0, 4)])
+def test_batch_norm_empty_shapes(hk, cuda, shape):
+    """An array without elements (no samples, no channels, no pixels) returns at once, forward and backward, and
+    needs no workspace; running statistics are left as they are."""
+    import torch
+    N, C = shape[0], shape[1]
+    x = torch.empty(shape, dtype=torch.float32, device=cuda)
+    y = torch.empty_like(x)
+    scale = torch.ones(C, device=cuda); bias = torch.zeros(C, device=cuda)
+    rm = torch.full((C,), 3.0, device=cuda); rv = torch.full((C,), 5.0, device=cuda)
+    sm = torch.empty(C, device=cuda); si = torch.empty(C, device=cuda)
+    assert hk.batch_norm_workspace_bytes(x) == 0
+    hk.batch_norm_fwd(x, scale, bias, y, 0.1, 1e-5, rm, rv, sm, si)
+    dx = torch.empty_like(x); ds = torch.empty(C, device=cuda); db = torch.empty(C, device=cuda)
+    hk.batch_norm_bwd(y, x, scale, dx, ds, db, sm, si)
+    torch.cuda.synchronize()
+    assert bool((rm == 3.0).all()) and bool((rv == 5.0).all())

@@ -142,7 +142,8 @@ struct StridedMeta {
   int64_t stride[8];
 };
 
-template <typename W>
+// SCATTER = false: dst (dense) <- src laid out by m; SCATTER = true: dst laid out by m <- src (dense)
+template <typename W, bool SCATTER>
 __global__ __launch_bounds__(256) void strided_copy_kernel(const W* __restrict__ src,
                                                            W* __restrict__ dst, StridedMeta m,
                                                            int64_t numel) {
@@ -155,13 +156,45 @@ __global__ __launch_bounds__(256) void strided_copy_kernel(const W* __restrict__
       off += (rem - q * m.shape[d]) * m.stride[d];
       rem = q;
     }
-    dst[i] = src[off];
+    if constexpr (SCATTER) dst[off] = src[i];
+    else dst[i] = src[off];
   }
 }
 
 } // namespace hk
 
 using namespace hk;
+
+template <bool SCATTER>
+static int strided_copy_any(const char* who, int dtype, const void* src, void* dst, int ndim, const int64_t* shape,
+                            const int64_t* strides, hkStream_t stream) {
+  HK_REQUIRE(ndim >= 0 && ndim <= 8, HK_ERR_INVALID, "%s: ndim %d not in [0, 8]", who, ndim);
+  HK_REQUIRE(ndim == 0 || (shape && strides), HK_ERR_INVALID, "%s: null meta", who);
+  size_t es = dtype_size(dtype);
+  HK_REQUIRE(es != 0, HK_ERR_UNSUPPORTED, "%s: unknown dtype %d", who, dtype);
+  StridedMeta m;
+  m.ndim = ndim;
+  int64_t numel = 1;
+  for (int d = 0; d < ndim; ++d) {
+    HK_REQUIRE(shape[d] >= 0, HK_ERR_INVALID, "%s: negative extent", who);
+    m.shape[d] = shape[d];
+    m.stride[d] = strides[d];
+    numel *= shape[d];
+  }
+  if (numel == 0) return HK_OK;
+  HK_REQUIRE(src && dst, HK_ERR_INVALID, "%s: null pointer", who);
+  int64_t blocks = (numel + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  dim3 g{unsigned(blocks)}, b{256};
+  hipStream_t s = as_hip(stream);
+  switch (es) {
+    case 1: HK_LAUNCH((strided_copy_kernel<uint8_t, SCATTER>), g, b, 0, s, (const uint8_t*)src, (uint8_t*)dst, m, numel); break;
+    case 2: HK_LAUNCH((strided_copy_kernel<uint16_t, SCATTER>), g, b, 0, s, (const uint16_t*)src, (uint16_t*)dst, m, numel); break;
+    case 4: HK_LAUNCH((strided_copy_kernel<uint32_t, SCATTER>), g, b, 0, s, (const uint32_t*)src, (uint32_t*)dst, m, numel); break;
+    default: HK_LAUNCH((strided_copy_kernel<uint64_t, SCATTER>), g, b, 0, s, (const uint64_t*)src, (uint64_t*)dst, m, numel); break;
+  }
+  return launch_check("strided_copy_kernel");
+}
 
 extern "C" {
 
@@ -364,32 +397,12 @@ int hk_copy_kernel(void* dst, const void* src, size_t bytes, hkStream_t stream) 
 
 int hk_strided_copy(int dtype, const void* src, void* dst, int ndim, const int64_t* shape,
                     const int64_t* src_strides, hkStream_t stream) {
-  HK_REQUIRE(ndim >= 0 && ndim <= 8, HK_ERR_INVALID, "hk_strided_copy: ndim %d not in [0, 8]", ndim);
-  HK_REQUIRE(ndim == 0 || (shape && src_strides), HK_ERR_INVALID, "hk_strided_copy: null meta");
-  size_t es = dtype_size(dtype);
-  HK_REQUIRE(es != 0, HK_ERR_UNSUPPORTED, "hk_strided_copy: unknown dtype %d", dtype);
-  StridedMeta m;
-  m.ndim = ndim;
-  int64_t numel = 1;
-  for (int d = 0; d < ndim; ++d) {
-    HK_REQUIRE(shape[d] >= 0, HK_ERR_INVALID, "hk_strided_copy: negative extent");
-    m.shape[d] = shape[d];
-    m.stride[d] = src_strides[d];
-    numel *= shape[d];
-  }
-  if (numel == 0) return HK_OK;
-  HK_REQUIRE(src && dst, HK_ERR_INVALID, "hk_strided_copy: null pointer");
-  int64_t blocks = (numel + 255) / 256;
-  if (blocks > 65536) blocks = 65536;
-  dim3 g{unsigned(blocks)}, b{256};
-  hipStream_t s = as_hip(stream);
-  switch (es) {
-    case 1: HK_LAUNCH(strided_copy_kernel<uint8_t>, g, b, 0, s, (const uint8_t*)src, (uint8_t*)dst, m, numel); break;
-    case 2: HK_LAUNCH(strided_copy_kernel<uint16_t>, g, b, 0, s, (const uint16_t*)src, (uint16_t*)dst, m, numel); break;
-    case 4: HK_LAUNCH(strided_copy_kernel<uint32_t>, g, b, 0, s, (const uint32_t*)src, (uint32_t*)dst, m, numel); break;
-    default: HK_LAUNCH(strided_copy_kernel<uint64_t>, g, b, 0, s, (const uint64_t*)src, (uint64_t*)dst, m, numel); break;
-  }
-  return launch_check("strided_copy_kernel");
+  return strided_copy_any<false>("hk_strided_copy", dtype, src, dst, ndim, shape, src_strides, stream);
+}
+
+int hk_strided_scatter(int dtype, const void* src, void* dst, int ndim, const int64_t* shape,
+                       const int64_t* dst_strides, hkStream_t stream) {
+  return strided_copy_any<true>("hk_strided_scatter", dtype, src, dst, ndim, shape, dst_strides, stream);
 }
 
 } // extern "C"

@@ -28,8 +28,7 @@ void FusedLayerNormCuda(const NDArray& in_arr, const NDArray& ln_scale, const ND
 
   int64_t rows, cols;
   SplitRows(in_arr, reduce_dims, rows, cols);
-  int64_t x_pitch = cols, y_pitch = cols;
-  HT_ASSERT_ROW_PITCHED(out_arr, reduce_dims, &y_pitch);
+  int64_t x_pitch = cols;
   HT_ASSERT(int64_t(ln_scale->numel()) == cols && int64_t(ln_bias->numel()) == cols)
     << "scale " << ln_scale->shape() << " / bias " << ln_bias->shape() << " do not match " << cols << " columns";
   HT_ASSERT(int64_t(mean_arr->numel()) == rows && int64_t(var_arr->numel()) == rows)
@@ -40,11 +39,13 @@ void FusedLayerNormCuda(const NDArray& in_arr, const NDArray& ln_scale, const ND
   hip::DeviceGuard guard(hip_stream.device_id());
   NDArray x = RowOperand(in_arr, reduce_dims, stream, &x_pitch);
   NDArray g = Dense(ln_scale, stream), b = Dense(ln_bias, stream);
+  RowOutput y(out_arr, reduce_dims, stream);
   HK_CALL(hk_layer_norm_fwd_pitched(int(in_arr->dtype()), x->raw_data_ptr(), x_pitch, g->raw_data_ptr(),
-                                    b->raw_data_ptr(), out_arr->raw_data_ptr(), y_pitch, mean_arr->raw_data_ptr(),
+                                    b->raw_data_ptr(), y.ptr(), y.pitch(), mean_arr->raw_data_ptr(),
                                     var_arr->raw_data_ptr(), HK_FLOAT32, HK_STAT_RSTD, rows, cols, eps,
                                     hip_stream));
-  NDArray::MarkUsedBy({x, g, b, mean_arr, var_arr, out_arr}, stream);
+  NDArray::MarkUsedBy({x, g, b, mean_arr, var_arr, y.array()}, stream);
+  y.Commit();
 }
 
 void FusedLayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr, const NDArray& ln_scale,
@@ -74,8 +75,7 @@ void FusedLayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr,
 
   int64_t rows, cols;
   SplitRows(in_arr, reduce_dims, rows, cols);
-  int64_t dy_pitch = cols, x_pitch = cols, dx_pitch = cols;
-  HT_ASSERT_ROW_PITCHED(grad_arr, reduce_dims, &dx_pitch);
+  int64_t dy_pitch = cols, x_pitch = cols;
   HT_ASSERT(int64_t(ln_scale->numel()) == cols && int64_t(grad_scale->numel()) == cols &&
             int64_t(grad_bias->numel()) == cols)
     << "scale / grad_scale / grad_bias must hold " << cols << " values";
@@ -100,14 +100,16 @@ void FusedLayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr,
   size_t ws_bytes = 0;
   HK_CALL(hk_norm_bwd_workspace_bytes(dt, rows, cols, &ws_bytes));
   NDArray ws = Scratch(ws_bytes, in_arr->device(), stream);
+  RowOutput dx(grad_arr, reduce_dims, stream);
   // gamma enters dx through clamp_by_magnitude(gamma, eps) in both modes
   // (FusedLayerNorm.cu:911-938)
   HK_CALL(hk_layer_norm_bwd_pitched(dt, dy->raw_data_ptr(), dy_pitch, xy->raw_data_ptr(), x_pitch, g->raw_data_ptr(),
                                     PtrOrNull(b), mean->raw_data_ptr(), rstd->raw_data_ptr(), HK_FLOAT32,
-                                    HK_STAT_RSTD, grad_arr->raw_data_ptr(), dx_pitch, grad_scale->raw_data_ptr(),
+                                    HK_STAT_RSTD, dx.ptr(), dx.pitch(), grad_scale->raw_data_ptr(),
                                     grad_bias->raw_data_ptr(), rows, cols, eps, inplace ? 1 : 0, /*clamp_gamma=*/1,
                                     MutPtrOrNull(ws), ws_bytes, hip_stream));
-  NDArray::MarkUsedBy({dy, xy, g, b, mean, rstd, grad_arr, grad_scale, grad_bias, ws}, stream);
+  NDArray::MarkUsedBy({dy, xy, g, b, mean, rstd, dx.array(), grad_scale, grad_bias, ws}, stream);
+  dx.Commit();
 }
 
 } // namespace impl

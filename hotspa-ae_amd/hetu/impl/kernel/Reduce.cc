@@ -21,7 +21,6 @@ void LaunchReduce(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, 
                   const Stream& stream) {
   HT_ASSERT_CUDA_DEVICE(in_arr);
   HT_ASSERT_SAME_DEVICE(in_arr, out_arr);
-  HT_ASSERT_CONTIGUOUS(out_arr);
   const int64_t nd = int64_t(in_arr->ndim());
   HT_NOT_IMPLEMENTED_IF(nd > 8) << "reductions of arrays with more than 8 dimensions";
   size_t kept = 1;
@@ -42,10 +41,12 @@ void LaunchReduce(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, 
   HK_CALL(hk_reduce_workspace_bytes(int(in_arr->dtype()), int(nd), in_arr->shape().data(), in_arr->stride().data(),
                                     int(num_ax), axes, &ws_bytes));
   NDArray ws = Scratch(ws_bytes, in_arr->device(), stream);
-  HK_CALL(hk_reduce(int(in_arr->dtype()), int(out_arr->dtype()), in_arr->raw_data_ptr(), out_arr->raw_data_ptr(),
+  RowOutput out(out_arr, -1, stream);   // the kept elements in row-major order, laid over the output's strides
+  HK_CALL(hk_reduce(int(in_arr->dtype()), int(out_arr->dtype()), in_arr->raw_data_ptr(), out.ptr(),
                     int(nd), in_arr->shape().data(), in_arr->stride().data(), int(num_ax), axes, op,
                     MutPtrOrNull(ws), ws_bytes, hip_stream));
-  NDArray::MarkUsedBy({in_arr, out_arr, ws}, stream);
+  NDArray::MarkUsedBy({in_arr, out.array(), ws}, stream);
+  out.Commit();
 }
 } // namespace
 

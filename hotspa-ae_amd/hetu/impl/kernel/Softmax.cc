@@ -3,7 +3,8 @@
 // is seen as [outer, dim, inner].  The operator takes non-contiguous arrays
 // (hetu/graph/ops/Softmax.h:52-54): for a softmax over the last dimension row-pitched
 // inputs and outputs go to the kernels as they are; any other input layout is made
-// dense first, and a softmax over another dimension needs a dense output.
+// dense first, any other output layout is written dense and laid over its strides
+// afterwards (RowOutput), as is the output of a softmax over another dimension.
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
 #include "hetu/impl/utils/cpu_utils.h"
@@ -36,19 +37,20 @@ void SoftmaxCuda(const NDArray& input, NDArray& output, int64_t dim, const Strea
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
   if (inner == 1) {
-    int64_t x_pitch = extent, y_pitch = extent;
-    HT_ASSERT_ROW_PITCHED(output, 1, &y_pitch);
+    int64_t x_pitch = extent;
     NDArray x = RowOperand(input, 1, stream, &x_pitch);
-    HK_CALL(hk_softmax_fwd_pitched(int(input->dtype()), x->raw_data_ptr(), x_pitch, output->raw_data_ptr(), y_pitch,
+    RowOutput y(output, 1, stream);
+    HK_CALL(hk_softmax_fwd_pitched(int(input->dtype()), x->raw_data_ptr(), x_pitch, y.ptr(), y.pitch(),
                                    outer, extent, hip_stream));
-    NDArray::MarkUsedBy({x, output}, stream);
+    NDArray::MarkUsedBy({x, y.array()}, stream);
+    y.Commit();
     return;
   }
-  HT_ASSERT_CONTIGUOUS(output);
   NDArray x = Dense(input, stream);
-  HK_CALL(hk_softmax_fwd(int(input->dtype()), x->raw_data_ptr(), output->raw_data_ptr(), outer, extent, inner,
-                         hip_stream));
-  NDArray::MarkUsedBy({x, output}, stream);
+  RowOutput y(output, -1, stream);
+  HK_CALL(hk_softmax_fwd(int(input->dtype()), x->raw_data_ptr(), y.ptr(), outer, extent, inner, hip_stream));
+  NDArray::MarkUsedBy({x, y.array()}, stream);
+  y.Commit();
 }
 
 void SoftmaxGradientCuda(const NDArray& input_Y, const NDArray& output_grad, NDArray& input_grad, int64_t dim,
@@ -67,19 +69,21 @@ void SoftmaxGradientCuda(const NDArray& input_Y, const NDArray& output_grad, NDA
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
   if (inner == 1) {
-    int64_t y_pitch = extent, dy_pitch = extent, dx_pitch = extent;
-    HT_ASSERT_ROW_PITCHED(input_grad, 1, &dx_pitch);
+    int64_t y_pitch = extent, dy_pitch = extent;
     NDArray y = RowOperand(input_Y, 1, stream, &y_pitch), dy = RowOperand(output_grad, 1, stream, &dy_pitch);
+    RowOutput dx(input_grad, 1, stream);
     HK_CALL(hk_softmax_bwd_pitched(int(input_Y->dtype()), y->raw_data_ptr(), y_pitch, dy->raw_data_ptr(), dy_pitch,
-                                   input_grad->raw_data_ptr(), dx_pitch, outer, extent, hip_stream));
-    NDArray::MarkUsedBy({y, dy, input_grad}, stream);
+                                   dx.ptr(), dx.pitch(), outer, extent, hip_stream));
+    NDArray::MarkUsedBy({y, dy, dx.array()}, stream);
+    dx.Commit();
     return;
   }
-  HT_ASSERT_CONTIGUOUS(input_grad);
   NDArray y = Dense(input_Y, stream), dy = Dense(output_grad, stream);
-  HK_CALL(hk_softmax_bwd(int(input_Y->dtype()), y->raw_data_ptr(), dy->raw_data_ptr(), input_grad->raw_data_ptr(),
-                         outer, extent, inner, hip_stream));
-  NDArray::MarkUsedBy({y, dy, input_grad}, stream);
+  RowOutput dx(input_grad, -1, stream);
+  HK_CALL(hk_softmax_bwd(int(input_Y->dtype()), y->raw_data_ptr(), dy->raw_data_ptr(), dx.ptr(), outer, extent, inner,
+                         hip_stream));
+  NDArray::MarkUsedBy({y, dy, dx.array()}, stream);
+  dx.Commit();
 }
 
 // ---------------------------------------------------------------------------------------------------------

@@ -51,7 +51,6 @@ void DenseGradient(const NDArray& input_y, const NDArray& label, const NDArray& 
   HT_ASSERT_SAME_DTYPE(input_y, label);
   HT_ASSERT_SAME_DTYPE(input_y, grad);
   HT_ASSERT_SAME_DTYPE(input_y, output);
-  HT_ASSERT_CONTIGUOUS(output);
   int64_t rows = 1;
   for (size_t i = 0; i + 1 < indim; ++i) rows *= input_y->shape(i);
   const int64_t cols = input_y->shape(indim - 1);
@@ -65,14 +64,16 @@ void DenseGradient(const NDArray& input_y, const NDArray& label, const NDArray& 
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
   NDArray x = Dense(input_y, stream), l = Dense(label, stream), g = Dense(grad, stream);
+  RowOutput out(output, -1, stream);
   if (scale) {
     HK_CALL(hk_sce_dense_bwd_reduced(int(input_y->dtype()), x->raw_data_ptr(), l->raw_data_ptr(), g->raw_data_ptr(),
-                                     *scale, output->raw_data_ptr(), rows, cols, hip_stream));
+                                     *scale, out.ptr(), rows, cols, hip_stream));
   } else {
     HK_CALL(hk_sce_dense_bwd(int(input_y->dtype()), x->raw_data_ptr(), l->raw_data_ptr(), g->raw_data_ptr(),
-                             output->raw_data_ptr(), rows, cols, hip_stream));
+                             out.ptr(), rows, cols, hip_stream));
   }
-  NDArray::MarkUsedBy({x, l, g, output}, stream);
+  NDArray::MarkUsedBy({x, l, g, out.array()}, stream);
+  out.Commit();
 }
 } // namespace
 

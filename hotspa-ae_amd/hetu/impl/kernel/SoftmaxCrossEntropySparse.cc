@@ -59,12 +59,7 @@ void SparseGradient(const NDArray& pred, const NDArray& label, const NDArray& gr
   HT_ASSERT(label->dtype() == kInt64) << "labels must be int64 class ids, got " << label->dtype();
   int64_t rows, cols;
   RowsCols(pred, rows, cols);
-  int64_t p_pitch = cols, out_pitch = cols;
-  if (scale) {
-    HT_ASSERT_CONTIGUOUS(output);
-  } else {
-    HT_ASSERT_ROW_PITCHED(output, 1, &out_pitch);
-  }
+  int64_t p_pitch = cols;
   HT_ASSERT(int64_t(label->numel()) == rows) << "labels " << label->shape() << " must hold one value per row of "
                                              << pred->shape();
   if (scale) {
@@ -80,16 +75,18 @@ void SparseGradient(const NDArray& pred, const NDArray& label, const NDArray& gr
   hip::DeviceGuard guard(hip_stream.device_id());
   NDArray p = scale ? Dense(pred, stream) : RowOperand(pred, 1, stream, &p_pitch);
   NDArray l = Dense(label, stream), g = Dense(grad_loss, stream);
+  RowOutput out(output, scale ? -1 : 1, stream);
   if (scale) {
     HK_CALL(hk_sce_sparse_bwd_reduced(int(pred->dtype()), p->raw_data_ptr(), l->data_ptr<int64_t>(),
-                                      g->raw_data_ptr(), *scale, output->raw_data_ptr(), rows, cols, ignored_index,
+                                      g->raw_data_ptr(), *scale, out.ptr(), rows, cols, ignored_index,
                                       hip_stream));
   } else {
     HK_CALL(hk_sce_sparse_bwd_pitched(int(pred->dtype()), p->raw_data_ptr(), p_pitch, l->data_ptr<int64_t>(),
-                                      g->raw_data_ptr(), output->raw_data_ptr(), out_pitch, rows, cols,
+                                      g->raw_data_ptr(), out.ptr(), out.pitch(), rows, cols,
                                       ignored_index, hip_stream));
   }
-  NDArray::MarkUsedBy({p, l, g, output}, stream);
+  NDArray::MarkUsedBy({p, l, g, out.array()}, stream);
+  out.Commit();
 }
 } // namespace
 

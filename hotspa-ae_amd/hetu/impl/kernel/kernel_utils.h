@@ -53,11 +53,44 @@ inline NDArray RowOperand(const NDArray& a, int64_t inner_dims, const Stream& st
   return dense;
 }
 
-// An output of a row kernel must be row-pitched; anything else has no 128-bit store pattern and is refused.
-#define HT_ASSERT_ROW_PITCHED(x, inner_dims, pitch_ptr)                                                   \
-  HT_ASSERT(::hetu::impl::RowPitch(x, inner_dims, pitch_ptr))                                              \
-    << "Output " << #x << " must be dense or a row-pitched view (unit-stride trailing dimensions, one "   \
-    << "constant row pitch). Shape: " << x->shape() << ". Strides: " << x->stride() << "."
+// An output of a row kernel.  A row-pitched array (dense, a column slice of a wider array, a row-padded buffer)
+// is written in place.  Any other layout (a transposed view, strided columns) has no 128-bit store pattern: the
+// kernel then writes a dense stand-in from the pool and Commit() lays it over the array's own strides.  The
+// reference's kernels write every element through an OffsetCalculator instead
+// (hetu/impl/utils/offset_calculator.cuh:16-68); here that costs one more pass, and only for such outputs.
+// inner_dims < 0 asks for a dense array outright (kernels that take no pitch).
+class RowOutput {
+ public:
+  RowOutput(NDArray& target, int64_t inner_dims, const Stream& stream) : target_(target), stream_(stream) {
+    const bool in_place = inner_dims < 0 ? target->is_contiguous() : RowPitch(target, inner_dims, &pitch_);
+    if (in_place) {
+      work_ = target;
+    } else {
+      work_ = NDArray::empty(target->shape(), target->device(), target->dtype(), stream.stream_index());
+      if (inner_dims >= 0) RowPitch(work_, inner_dims, &pitch_);
+    }
+  }
+  NDArray& array() { return work_; }
+  void* ptr() { return work_->raw_data_ptr(); }
+  int64_t pitch() const { return pitch_; }
+  bool staged() const { return work_->raw_data_ptr() != target_->raw_data_ptr(); }
+  // after the kernel call, on the same stream
+  void Commit() {
+    if (!staged()) return;
+    HIPStream hip_stream(stream_);
+    const HTShape& shape = target_->shape();
+    const HTStride& stride = target_->stride();
+    HK_CALL(hk_strided_scatter(int(target_->dtype()), work_->raw_data_ptr(), target_->raw_data_ptr(),
+                               int(shape.size()), shape.data(), stride.data(), hip_stream));
+    NDArray::MarkUsedBy({work_, target_}, stream_);
+  }
+
+ private:
+  NDArray& target_;
+  NDArray work_;
+  Stream stream_;
+  int64_t pitch_ = 0;
+};
 
 inline const void* PtrOrNull(const NDArray& a) {
   return a.is_defined() ? a->raw_data_ptr() : nullptr;

@@ -137,6 +137,13 @@ HK_API int hk_strided_copy(int dtype, const void* src, void* dst, int ndim,
                            const int64_t* shape, const int64_t* src_strides,
                            hkStream_t stream);
 
+/* The other direction: lays a dense row-major array over a strided view (the output side of the same
+ * OffsetCalculator, offset_calculator.cuh:16-68: the reference's kernels write every element through it).
+ * Used for an operator output that is neither dense nor row-pitched. */
+HK_API int hk_strided_scatter(int dtype, const void* src, void* dst, int ndim,
+                              const int64_t* shape, const int64_t* dst_strides,
+                              hkStream_t stream);
+
 /* ======================================================================== *
  * LayerNorm.
  * x, y: [rows, cols] dense, dtype `dtype` (fp32 / bf16 / fp16); gamma, beta:

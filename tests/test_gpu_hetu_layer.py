@@ -352,8 +352,8 @@ def test_softmax_and_gradient(ops, cuda, dtype, shape, dim):
 
 
 def test_softmax_of_a_permuted_view(ops, cuda):
-    """Inputs of any stride are accepted (row-pitched ones as they are, others made dense inside); outputs must
-    be dense or row-pitched."""
+    """Inputs and outputs of any stride are accepted: row-pitched ones go to the kernels as they are, any other
+    input is made dense inside, any other output is written dense and laid over its strides afterwards."""
     import torch
     x = helpers.draw(61, (12, 40, 24), "normal", 0.0, 2.0, "fp32")
     tx = helpers.to_torch(x, "fp32", cuda).permute(2, 0, 1)       # [24, 12, 40], not dense
@@ -363,10 +363,76 @@ def test_softmax_of_a_permuted_view(ops, cuda):
     ops.softmax(tx, ty, -1)
     ops.stream_sync()
     helpers.assert_close(ty, ey, "fp32", "y")
-    with pytest.raises(ops.AssertionError_, match="row-pitched"):
-        ops.softmax(tx, torch.empty((12, 40, 24), device=cuda).permute(2, 0, 1), -1)
+    # the same into a permuted output
+    base = torch.full((12, 40, 24), float("nan"), device=cuda)
+    _sync_in()
+    ops.softmax(tx, base.permute(2, 0, 1), -1)
+    ops.stream_sync()
+    helpers.assert_close(base.permute(2, 0, 1).contiguous(), ey, "fp32", "y")
     with pytest.raises(ops.AssertionError_, match="Invalid dimension"):
         ops.softmax(tx, ty, 3)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_outputs_of_any_layout(ops, cuda, dtype):
+    """A transposed view, and a view with a stride between columns, as the output of LayerNorm forward / backward,
+    softmax forward / backward (last and middle dimension), the cross-entropy gradients and a reduction: the
+    values that land in the view equal the dense result bit for bit, and nothing outside the view is written."""
+    import torch
+    R, C = 37, 96
+    x = helpers.draw(901, (R, C), dtype=dtype)
+    dy = helpers.draw(902, (R, C), dtype=dtype)
+    g = helpers.draw(903, (C,), "uniform", 0.5, 1.5, dtype)
+    b = helpers.draw(904, (C,), "normal", 0.0, 0.1, dtype)
+    tx, tdy, tg, tb = (helpers.to_torch(v, dtype, cuda) for v in (x, dy, g, b))
+    td = tx.dtype
+
+    def layouts():
+        # (name, view of shape [R, C], its backing array, mask of the elements the view covers)
+        t = torch.full((C, R), 7.0, dtype=td, device=cuda)
+        yield "transposed", t.t(), t, torch.ones((C, R), dtype=torch.bool, device=cuda)
+        w = torch.full((R, 2 * C), 7.0, dtype=td, device=cuda)
+        m = torch.zeros((R, 2 * C), dtype=torch.bool, device=cuda)
+        m[:, ::2] = True
+        yield "every other column", w[:, ::2], w, m
+
+    def check(run, what):
+        dense = torch.empty((R, C), dtype=td, device=cuda)
+        _sync_in()
+        run(dense)
+        ops.stream_sync()
+        for name, view, backing, covered in layouts():
+            assert not view.is_contiguous()
+            _sync_in()
+            run(view)
+            ops.stream_sync()
+            assert torch.equal(view.contiguous(), dense), "%s into a %s view" % (what, name)
+            assert bool((backing[~covered] == 7.0).all()), "%s wrote outside a %s view" % (what, name)
+
+    mean = torch.empty(R, dtype=torch.float32, device=cuda)
+    rstd = torch.empty(R, dtype=torch.float32, device=cuda)
+    check(lambda out: ops.fused_layer_norm(tx, tg, tb, mean, rstd, out, 1, 1e-5), "fused layer norm")
+    dg, db = torch.empty_like(tg), torch.empty_like(tg)
+    check(lambda out: ops.fused_layer_norm_gradient(tdy, tx, tg, tb, out, dg, db, mean, rstd, 1, 1e-5, False),
+          "fused layer norm gradient")
+    mean_t, var_t = torch.empty(R, dtype=td, device=cuda), torch.empty(R, dtype=td, device=cuda)
+    check(lambda out: ops.layer_norm(tx, tg, tb, mean_t, var_t, out, 1, 1e-5), "layer norm")
+    check(lambda out: ops.layer_norm_gradient(tdy, tx, tg, out, dg, db, mean_t, var_t, 1, 1e-5), "layer norm gradient")
+    check(lambda out: ops.softmax(tx, out, -1), "softmax")
+    check(lambda out: ops.softmax(tx, out, 0), "softmax over dimension 0")
+    ty = torch.empty_like(tx)
+    _sync_in()
+    ops.softmax(tx, ty, -1)
+    ops.stream_sync()
+    check(lambda out: ops.softmax_gradient(ty, tdy, out, -1), "softmax gradient")
+    labels = torch.randint(0, C, (R,), device=cuda, dtype=torch.int64)
+    labels[3] = -100
+    gl = helpers.to_torch(helpers.draw(905, (R,), dtype=dtype), dtype, cuda)
+    check(lambda out: ops.softmax_cross_entropy_sparse_gradient(tx, labels, gl, out, -100), "sparse CE gradient")
+    dense_labels = torch.softmax(tdy.float(), -1).to(td)
+    check(lambda out: ops.softmax_cross_entropy_gradient(tx, dense_labels, gl, out), "dense CE gradient")
+    x3 = helpers.to_torch(helpers.draw(906, (R, 5, C), dtype=dtype), dtype, cuda)
+    check(lambda out: ops.reduce(x3, out, [1], "sum"), "sum over the middle dimension")
 
 
 def test_row_pitched_views_reach_the_kernels_without_a_copy(ops, cuda):

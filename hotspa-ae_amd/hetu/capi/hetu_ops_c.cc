@@ -206,7 +206,9 @@ int ht_set_random_seed(uint64_t seed) {
 int ht_instance_norm(const HtArray* in, HtArray* mean, HtArray* var, HtArray* out, float eps, int stream_index) {
   return guarded([&] {
     NDArray m = wrap(mean), v = wrap(var), o = wrap(out);
-    hetu::impl::InstanceNormCuda(wrap(in), m, v, o, eps, stream_of(in, stream_index));
+    const Stream st = stream_of(in, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_instance_norm", hetu::impl::InstanceNorm, wrap(in), m, v, o,
+                                    eps, st);
   });
 }
 
@@ -214,8 +216,9 @@ int ht_instance_norm_gradient(const HtArray* out_grads, const HtArray* in, HtArr
                               const HtArray* var, float eps, int stream_index) {
   return guarded([&] {
     NDArray g = wrap(grad_in);
-    hetu::impl::InstanceNormGradientCuda(wrap(out_grads), wrap(in), g, wrap(mean), wrap(var), eps,
-                                         stream_of(in, stream_index));
+    const Stream st = stream_of(in, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_instance_norm_gradient", hetu::impl::InstanceNormGradient,
+                                    wrap(out_grads), wrap(in), g, wrap(mean), wrap(var), eps, st);
   });
 }
 
@@ -239,7 +242,9 @@ int ht_softmax_gradient(const HtArray* y, const HtArray* dy, HtArray* dx, int64_
 int ht_softmax_cross_entropy(const HtArray* pred, const HtArray* label, HtArray* loss, int stream_index) {
   return guarded([&] {
     NDArray o = wrap(loss);
-    hetu::impl::SoftmaxCrossEntropyCuda(wrap(pred), wrap(label), o, stream_of(pred, stream_index));
+    const Stream st = stream_of(pred, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_softmax_cross_entropy", hetu::impl::SoftmaxCrossEntropy,
+                                    wrap(pred), wrap(label), o, st);
   });
 }
 
@@ -247,8 +252,10 @@ int ht_softmax_cross_entropy_gradient(const HtArray* pred, const HtArray* label,
                                       HtArray* out, int stream_index) {
   return guarded([&] {
     NDArray o = wrap(out);
-    hetu::impl::SoftmaxCrossEntropyGradientCuda(wrap(pred), wrap(label), wrap(grad_loss), o,
-                                                stream_of(pred, stream_index));
+    const Stream st = stream_of(pred, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_softmax_cross_entropy_gradient",
+                                    hetu::impl::SoftmaxCrossEntropyGradient, wrap(pred), wrap(label), wrap(grad_loss),
+                                    o, st);
   });
 }
 
@@ -277,7 +284,9 @@ int ht_softmax_cross_entropy_sparse_gradient(const HtArray* pred, const HtArray*
 int ht_nll_loss(const HtArray* pred, const HtArray* label, HtArray* loss, int stream_index) {
   return guarded([&] {
     NDArray o = wrap(loss);
-    hetu::impl::NLLLossCuda(wrap(pred), wrap(label), o, stream_of(pred, stream_index));
+    const Stream st = stream_of(pred, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_nll_loss", hetu::impl::NLLLoss, wrap(pred), wrap(label), o,
+                                    st);
   });
 }
 
@@ -285,7 +294,9 @@ int ht_nll_loss_gradient(const HtArray* pred, const HtArray* label, const HtArra
                          int stream_index) {
   return guarded([&] {
     NDArray o = wrap(out);
-    hetu::impl::NLLLossGradientCuda(wrap(pred), wrap(label), wrap(grad_loss), o, stream_of(pred, stream_index));
+    const Stream st = stream_of(pred, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_nll_loss_gradient", hetu::impl::NLLLossGradient, wrap(pred),
+                                    wrap(label), wrap(grad_loss), o, st);
   });
 }
 
@@ -304,10 +315,18 @@ int ht_binary(int op, const HtArray* a, const HtArray* b, HtArray* out, int stre
     NDArray o = wrap(out);
     const Stream st = stream_of(a, stream_index);
     switch (op) {
-      case 0: hetu::impl::AddElewiseCuda(wrap(a), wrap(b), o, st); break;
-      case 1: hetu::impl::SubElewiseCuda(wrap(a), wrap(b), o, st); break;
-      case 2: hetu::impl::MulElewiseCuda(wrap(a), wrap(b), o, st); break;
-      case 3: hetu::impl::DivElewiseCuda(wrap(a), wrap(b), o, st); break;
+      case 0:
+        HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_binary", hetu::impl::AddElewise, wrap(a), wrap(b), o, st);
+        break;
+      case 1:
+        HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_binary", hetu::impl::SubElewise, wrap(a), wrap(b), o, st);
+        break;
+      case 2:
+        HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_binary", hetu::impl::MulElewise, wrap(a), wrap(b), o, st);
+        break;
+      case 3:
+        HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_binary", hetu::impl::DivElewise, wrap(a), wrap(b), o, st);
+        break;
       default: HT_VALUE_ERROR << "unknown binary op " << op;
     }
   });
@@ -318,10 +337,18 @@ int ht_binary_const(int op, const HtArray* in, double value, HtArray* out, int s
     NDArray o = wrap(out);
     const Stream st = stream_of(in, stream_index);
     switch (op) {
-      case 0: hetu::impl::AddConstCuda(wrap(in), value, o, st); break;
-      case 1: hetu::impl::SubConstCuda(wrap(in), value, o, st); break;
-      case 2: hetu::impl::MulConstCuda(wrap(in), value, o, st); break;
-      case 3: hetu::impl::DivConstCuda(wrap(in), value, o, st); break;
+      case 0:
+        HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_binary_const", hetu::impl::AddConst, wrap(in), value, o, st);
+        break;
+      case 1:
+        HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_binary_const", hetu::impl::SubConst, wrap(in), value, o, st);
+        break;
+      case 2:
+        HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_binary_const", hetu::impl::MulConst, wrap(in), value, o, st);
+        break;
+      case 3:
+        HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_binary_const", hetu::impl::DivConst, wrap(in), value, o, st);
+        break;
       default: HT_VALUE_ERROR << "unknown binary op " << op;
     }
   });
@@ -332,10 +359,10 @@ int ht_unary(int op, const HtArray* in, HtArray* out, int stream_index) {
     NDArray o = wrap(out);
     const Stream st = stream_of(in, stream_index);
     switch (op) {
-      case 0: hetu::impl::ExpCuda(wrap(in), o, st); break;
-      case 1: hetu::impl::LogCuda(wrap(in), o, st); break;
-      case 2: hetu::impl::OppositeCuda(wrap(in), o, st); break;
-      case 3: hetu::impl::SqrtCuda(wrap(in), o, st); break;
+      case 0: HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_unary", hetu::impl::Exp, wrap(in), o, st); break;
+      case 1: HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_unary", hetu::impl::Log, wrap(in), o, st); break;
+      case 2: HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_unary", hetu::impl::Opposite, wrap(in), o, st); break;
+      case 3: HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_unary", hetu::impl::Sqrt, wrap(in), o, st); break;
       default: HT_VALUE_ERROR << "unknown unary op " << op;
     }
   });
@@ -377,8 +404,9 @@ int ht_batch_norm(const HtArray* input_X, const HtArray* bn_scale, const HtArray
   return guarded([&] {
     NDArray y = wrap(output_Y), rm = wrap(running_mean), rv = wrap(running_var), sm = wrap(save_mean),
             sv = wrap(save_var);
-    hetu::impl::BatchNormCuda(wrap(input_X), wrap(bn_scale), wrap(bn_bias), y, momentum, eps, rm, rv, sm, sv,
-                              stream_of(input_X, stream_index));
+    const Stream st = stream_of(input_X, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_batch_norm", hetu::impl::BatchNorm, wrap(input_X),
+                                    wrap(bn_scale), wrap(bn_bias), y, momentum, eps, rm, rv, sm, sv, st);
   });
 }
 
@@ -388,15 +416,17 @@ int ht_batch_norm_gradient(const HtArray* gradient_Y, const HtArray* input_X, co
   return guarded([&] {
     NDArray dx = wrap(gradient_X), ds = wrap(gradient_bn_scale), db = wrap(gradient_bn_bias), sm = wrap(save_mean),
             sv = wrap(save_var);
-    hetu::impl::BatchNormGradientCuda(wrap(gradient_Y), wrap(input_X), wrap(bn_scale), dx, ds, db, eps, sm, sv,
-                                      stream_of(input_X, stream_index));
+    const Stream st = stream_of(input_X, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_batch_norm_gradient", hetu::impl::BatchNormGradient,
+                                    wrap(gradient_Y), wrap(input_X), wrap(bn_scale), dx, ds, db, eps, sm, sv, st);
   });
 }
 
 int ht_norm(const HtArray* input, HtArray* output, int64_t dim, int64_t p, int stream_index) {
   return guarded([&] {
     NDArray o = wrap(output);
-    hetu::impl::NormCuda(wrap(input), o, dim, p, stream_of(input, stream_index));
+    const Stream st = stream_of(input, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_norm", hetu::impl::Norm, wrap(input), o, dim, p, st);
   });
 }
 
@@ -404,8 +434,9 @@ int ht_norm_gradient(const HtArray* input, const HtArray* output, const HtArray*
                      int64_t dim, int64_t p, int stream_index) {
   return guarded([&] {
     NDArray g = wrap(input_grad);
-    hetu::impl::NormGradientCuda(wrap(input), wrap(output), wrap(output_grad), g, dim, p,
-                                 stream_of(input, stream_index));
+    const Stream st = stream_of(input, stream_index);
+    HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_norm_gradient", hetu::impl::NormGradient, wrap(input),
+                                    wrap(output), wrap(output_grad), g, dim, p, st);
   });
 }
 
@@ -486,10 +517,13 @@ int ht_broadcast_shape(const HtArray* input, int multiply, double const_value, H
   return guarded([&] {
     NDArray out = wrap(output);
     HTShape axes(add_axes, add_axes + (add_axes ? n_add_axes : 0));
+    const Stream st = stream_of(input, stream_index);
     if (multiply)
-      hetu::impl::BroadcastShapeMulCuda(wrap(input), const_value, out, axes, stream_of(input, stream_index));
+      HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_broadcast_shape", hetu::impl::BroadcastShapeMul,
+                                      wrap(input), const_value, out, axes, st);
     else
-      hetu::impl::BroadcastShapeCuda(wrap(input), out, axes, stream_of(input, stream_index));
+      HT_DISPATCH_KERNEL_CPU_AND_CUDA(st.device_type(), "ht_broadcast_shape", hetu::impl::BroadcastShape, wrap(input),
+                                      out, axes, st);
   });
 }
 

@@ -4,6 +4,8 @@
 // is rounded to the array's type before it is used.
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
+#include "hetu/impl/utils/cpu_utils.h"
+#include "hetu/impl/utils/dispatch.h"
 
 namespace hetu {
 namespace impl {
@@ -39,15 +41,42 @@ void DivConstCuda(const NDArray& input, double value, NDArray& output, const Str
   BinaryConst(HK_BINARY_DIV, input, value, output, stream);
 }
 
-#define HT_NO_CPU_CONST(name)                                                                        \
-  void name##Cpu(const NDArray&, double, NDArray&, const Stream&) {                                  \
-    HT_NOT_IMPLEMENTED << #name << " has no CPU kernel in this build (the product path is the GPU)"; \
-  }
-HT_NO_CPU_CONST(AddConst)
-HT_NO_CPU_CONST(SubConst)
-HT_NO_CPU_CONST(MulConst)
-HT_NO_CPU_CONST(DivConst)
-#undef HT_NO_CPU_CONST
+// Host twins (hetu/impl/kernel/BinaryConst.cc of the reference): value op x with the constant rounded to the
+// array's type first; arithmetic as in the element-wise twins (float / double, integers wrap, x = 0 under an
+// integer division gives 0).
+namespace {
+void BinaryConstHost(int op, const char* who, const NDArray& input, double value, NDArray& output,
+                     const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(input);
+  HT_ASSERT_SAME_DEVICE(input, output);
+  HT_ASSERT_SAME_SHAPE(input, output);
+  HT_ASSERT_SAME_DTYPE(input, output);
+  HT_ASSERT_CONTIGUOUS(output);
+  if (input->numel() == 0) return;
+  NDArray x = Dense(input, stream);
+  const int64_t n = int64_t(input->numel());
+  HT_DISPATCH_INTEGER_AND_FLOATING_TYPES(input->dtype(), spec_t, who, [&]() {
+    const spec_t* px = x->data_ptr<spec_t>();
+    spec_t* po = output->data_ptr<spec_t>();
+    const spec_t c = static_cast<spec_t>(value);   // the constant in the array's type, as the accelerator path
+    cpu::parallel_for(n, [&](int64_t i) { po[i] = cpu::binary_op<spec_t>(op, c, px[i]); });
+  });
+}
+} // namespace
+
+void AddConstCpu(const NDArray& input, double value, NDArray& output, const Stream& stream) {
+  BinaryConstHost(HK_BINARY_ADD, "AddConstCpu", input, value, output, stream);
+}
+void SubConstCpu(const NDArray& input, double value, NDArray& output, const Stream& stream) {
+  BinaryConstHost(HK_BINARY_SUB, "SubConstCpu", input, value, output, stream);
+}
+void MulConstCpu(const NDArray& input, double value, NDArray& output, const Stream& stream) {
+  BinaryConstHost(HK_BINARY_MUL, "MulConstCpu", input, value, output, stream);
+}
+void DivConstCpu(const NDArray& input, double value, NDArray& output, const Stream& stream) {
+  HT_ASSERT(value != 0) << "Divided by 0.";
+  BinaryConstHost(HK_BINARY_DIV, "DivConstCpu", input, value, output, stream);
+}
 
 } // namespace impl
 } // namespace hetu

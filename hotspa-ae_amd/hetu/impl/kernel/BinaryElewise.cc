@@ -4,6 +4,8 @@
 // repeats) and may have any strides; the output is dense.
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
+#include "hetu/impl/utils/cpu_utils.h"
+#include "hetu/impl/utils/dispatch.h"
 
 namespace hetu {
 namespace impl {
@@ -65,15 +67,55 @@ void DivElewiseCuda(const NDArray& inputA, const NDArray& inputB, NDArray& outpu
   BinaryElewise(HK_BINARY_DIV, inputA, inputB, output, stream);
 }
 
-#define HT_NO_CPU_BINARY(name)                                                                       \
-  void name##Cpu(const NDArray&, const NDArray&, NDArray&, const Stream&) {                          \
-    HT_NOT_IMPLEMENTED << #name << " has no CPU kernel in this build (the product path is the GPU)"; \
-  }
-HT_NO_CPU_BINARY(AddElewise)
-HT_NO_CPU_BINARY(SubElewise)
-HT_NO_CPU_BINARY(MulElewise)
-HT_NO_CPU_BINARY(DivElewise)
-#undef HT_NO_CPU_BINARY
+// ---------------------------------------------------------------------------------------------------------
+// Host twins (hetu/impl/kernel/BinaryElewise.cc of the reference, oneDNN binary primitives there): the same
+// broadcasting, one run along the last dimension at a time.  Floating-point types compute in float (double for
+// float64) and round once; the integer types wrap in their own width, a division by zero gives 0 instead of a trap.
+// ---------------------------------------------------------------------------------------------------------
+namespace {
+void BinaryElewiseHost(int op, const char* who, const NDArray& inputA, const NDArray& inputB, NDArray& output) {
+  HT_ASSERT_CPU_DEVICE(inputA);
+  HT_ASSERT_SAME_DEVICE(inputA, output);
+  HT_ASSERT_SAME_DEVICE(inputB, output);
+  HT_ASSERT_SAME_DTYPE(inputA, output);
+  HT_ASSERT_SAME_DTYPE(inputB, output);
+  HT_ASSERT_CONTIGUOUS(output);
+  HT_ASSERT(output->ndim() <= 8) << "At most 8 dimensions, got " << output->shape();
+  const HTShape expect = NDArrayMeta::Broadcast(inputA->shape(), inputB->shape());
+  HT_ASSERT(!expect.empty() || (inputA->ndim() == 0 && inputB->ndim() == 0))
+    << "Shapes cannot be broadcast together: " << inputA->shape() << " vs. " << inputB->shape();
+  HT_ASSERT(expect == output->shape())
+    << "Output " << output->shape() << " does not have the broadcast shape " << expect;
+  if (output->numel() == 0) return;
+  const std::vector<int64_t> sa = BroadcastStrides(inputA, output->shape());
+  const std::vector<int64_t> sb = BroadcastStrides(inputB, output->shape());
+  const std::vector<int64_t> shape(output->shape().begin(), output->shape().end());
+  const int nd = int(shape.size());
+  HT_DISPATCH_INTEGER_AND_FLOATING_TYPES(output->dtype(), spec_t, who, [&]() {
+    const spec_t* pa = inputA->data_ptr<spec_t>();
+    const spec_t* pb = inputB->data_ptr<spec_t>();
+    spec_t* po = output->data_ptr<spec_t>();
+    const int64_t n = nd ? shape[size_t(nd - 1)] : 1;
+    const int64_t ia = nd ? sa[size_t(nd - 1)] : 0, ib = nd ? sb[size_t(nd - 1)] : 0;
+    cpu::for_each_run(nd, shape.data(), sa.data(), sb.data(), [&](int64_t o, int64_t oa, int64_t ob) {
+      for (int64_t i = 0; i < n; ++i) po[o + i] = cpu::binary_op<spec_t>(op, pa[oa + i * ia], pb[ob + i * ib]);
+    });
+  });
+}
+} // namespace
+
+void AddElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream&) {
+  BinaryElewiseHost(HK_BINARY_ADD, "AddElewiseCpu", inputA, inputB, output);
+}
+void SubElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream&) {
+  BinaryElewiseHost(HK_BINARY_SUB, "SubElewiseCpu", inputA, inputB, output);
+}
+void MulElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream&) {
+  BinaryElewiseHost(HK_BINARY_MUL, "MulElewiseCpu", inputA, inputB, output);
+}
+void DivElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream&) {
+  BinaryElewiseHost(HK_BINARY_DIV, "DivElewiseCpu", inputA, inputB, output);
+}
 
 } // namespace impl
 } // namespace hetu

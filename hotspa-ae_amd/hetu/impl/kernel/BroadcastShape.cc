@@ -9,18 +9,20 @@
 // equals the output's (a mismatch reads out of place there); here it is checked.
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
+#include "hetu/impl/utils/cpu_utils.h"
+#include "hetu/impl/utils/dispatch.h"
 
 namespace hetu {
 namespace impl {
 
 namespace {
-void Broadcast(const char* who, const NDArray& input, bool multiply, double const_value, NDArray& output,
-               const HTShape& add_axes, const Stream& stream) {
-  HT_ASSERT_CUDA_DEVICE(input);
+// The input's strides per output dimension (0 where it broadcasts), checked; false when there is nothing to do.
+bool BroadcastLayout(const char* who, const NDArray& input, const NDArray& output, const HTShape& add_axes,
+                     int64_t out_shape[8], int64_t in_strides[8]) {
   HT_ASSERT_SAME_DEVICE(input, output);
   HT_ASSERT_SAME_DTYPE(input, output);
   HT_ASSERT_CONTIGUOUS(output);
-  if (output->numel() == 0 || input->numel() == 0) return;
+  if (output->numel() == 0 || input->numel() == 0) return false;
 
   const int in_nd = int(input->ndim()), out_nd = int(output->ndim());
   HT_ASSERT(in_nd <= out_nd) << who << ": input " << input->shape() << " has more dimensions than output "
@@ -45,7 +47,6 @@ void Broadcast(const char* who, const NDArray& input, bool multiply, double cons
     for (int i = 0; i < out_nd; ++i)
       if (!added[size_t(i)]) source[size_t(i)] = next++;
   }
-  int64_t out_shape[8], in_strides[8];
   for (int i = 0; i < out_nd; ++i) {
     out_shape[i] = output->shape(i);
     in_strides[i] = 0;
@@ -57,7 +58,15 @@ void Broadcast(const char* who, const NDArray& input, bool multiply, double cons
       << add_axes << "): extent " << extent << " meets " << out_shape[i] << " at output dimension " << i;
     if (extent > 1) in_strides[i] = input->stride(src);
   }
+  return true;
+}
 
+void Broadcast(const char* who, const NDArray& input, bool multiply, double const_value, NDArray& output,
+               const HTShape& add_axes, const Stream& stream) {
+  HT_ASSERT_CUDA_DEVICE(input);
+  int64_t out_shape[8], in_strides[8];
+  if (!BroadcastLayout(who, input, output, add_axes, out_shape, in_strides)) return;
+  const int out_nd = int(output->ndim());
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
   HK_CALL(hk_broadcast(int(input->dtype()), input->raw_data_ptr(), multiply ? 1 : 0, const_value,
@@ -75,11 +84,37 @@ void BroadcastShapeMulCuda(const NDArray& input, double const_value, NDArray& ou
   Broadcast("BroadcastShapeMul", input, true, const_value, output, add_axes, stream);
 }
 
-void BroadcastShapeCpu(const NDArray&, NDArray&, const HTShape&, const Stream&) {
-  HT_NOT_IMPLEMENTED << "BroadcastShape has no CPU kernel in this build (the product path is the GPU)";
+// Host twins (hetu/impl/kernel/BroadcastShape.cc of the reference): the same layout, copied (or multiplied by
+// the constant rounded to the array's type) one run along the last dimension at a time.
+namespace {
+void BroadcastHost(const char* who, const NDArray& input, bool multiply, double const_value, NDArray& output,
+                   const HTShape& add_axes) {
+  HT_ASSERT_CPU_DEVICE(input);
+  int64_t out_shape[8], in_strides[8], none[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (!BroadcastLayout(who, input, output, add_axes, out_shape, in_strides)) return;
+  const int nd = int(output->ndim());
+  HT_DISPATCH_INTEGER_AND_FLOATING_TYPES(output->dtype(), spec_t, who, [&]() {
+    const spec_t* pi = input->data_ptr<spec_t>();
+    spec_t* po = output->data_ptr<spec_t>();
+    const spec_t c = static_cast<spec_t>(const_value);
+    const int64_t n = nd ? out_shape[nd - 1] : 1, step = nd ? in_strides[nd - 1] : 0;
+    cpu::for_each_run(nd, out_shape, in_strides, none, [&](int64_t o, int64_t oi, int64_t) {
+      if (multiply) {
+        for (int64_t i = 0; i < n; ++i) po[o + i] = cpu::binary_op<spec_t>(2, pi[oi + i * step], c);
+      } else {
+        for (int64_t i = 0; i < n; ++i) po[o + i] = pi[oi + i * step];
+      }
+    });
+  });
 }
-void BroadcastShapeMulCpu(const NDArray&, double, NDArray&, const HTShape&, const Stream&) {
-  HT_NOT_IMPLEMENTED << "BroadcastShapeMul has no CPU kernel in this build (the product path is the GPU)";
+} // namespace
+
+void BroadcastShapeCpu(const NDArray& input, NDArray& output, const HTShape& add_axes, const Stream&) {
+  BroadcastHost("BroadcastShape", input, false, 1.0, output, add_axes);
+}
+void BroadcastShapeMulCpu(const NDArray& input, double const_value, NDArray& output, const HTShape& add_axes,
+                          const Stream&) {
+  BroadcastHost("BroadcastShapeMul", input, true, const_value, output, add_axes);
 }
 
 } // namespace impl

@@ -4,6 +4,10 @@
 // from the end.
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
+#include "hetu/impl/utils/cpu_utils.h"
+#include "hetu/impl/utils/dispatch.h"
+
+#include <cmath>
 
 namespace hetu {
 namespace impl {
@@ -68,11 +72,97 @@ void NormGradientCuda(const NDArray& input, const NDArray& output, const NDArray
   NDArray::MarkUsedBy({x, n, g, input_grad}, stream);
 }
 
-void NormCpu(const NDArray&, NDArray&, int64_t, int64_t, const Stream&) {
-  HT_NOT_IMPLEMENTED << "Norm has no CPU kernel in this build (the product path is the GPU)";
+// Host twins (hetu/impl/kernel/Norm.cc of the reference): the array is seen as [before, reduce, after]; each of
+// the before * after norms is a blocked sum of |x|^p in the arithmetic type, and the gradient follows the
+// accelerator's three cases (p = 1: sign(x) g; p = 2: g x / n; p > 2: x |x|^(p-2) g / n^(p-1); 0 where n = 0).
+namespace {
+template <typename A>
+inline A AbsPow(A v, int64_t p) {
+  const A a = std::fabs(v);
+  if (p == 1) return a;
+  if (p == 2) return a * a;
+  return std::pow(a, A(p));
 }
-void NormGradientCpu(const NDArray&, const NDArray&, const NDArray&, NDArray&, int64_t, int64_t, const Stream&) {
-  HT_NOT_IMPLEMENTED << "NormGradient has no CPU kernel in this build (the product path is the GPU)";
+} // namespace
+
+void NormCpu(const NDArray& input, NDArray& output, int64_t dim, int64_t p, const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(input);
+  HT_ASSERT_SAME_DEVICE(input, output);
+  HT_ASSERT_SAME_DTYPE(input, output);
+  HT_ASSERT_CONTIGUOUS(output);
+  HT_VALUE_ERROR_IF(p < 1) << "The norm's exponent must be at least 1, got " << p;
+  const int64_t nd = int64_t(input->ndim());
+  dim = NDArrayMeta::ParseAxis(dim, nd);
+  int64_t before = 1, after = 1;
+  for (int64_t i = 0; i < nd; ++i) {
+    if (i < dim) before *= input->shape(i);
+    else if (i > dim) after *= input->shape(i);
+  }
+  const int64_t reduce_size = input->shape(dim);
+  HT_ASSERT(int64_t(output->numel()) == before * after)
+    << "output " << output->shape() << " does not hold the " << before * after << " norms of " << input->shape()
+    << " over dimension " << dim;
+  if (before * after == 0) return;
+  NDArray x = Dense(input, stream);
+  HT_DISPATCH_FLOATING_TYPES(input->dtype(), spec_t, "NormCpu", [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* px = x->data_ptr<spec_t>();
+    spec_t* po = output->data_ptr<spec_t>();
+    cpu::parallel_rows(before * after, reduce_size, [&](int64_t o) {
+      const spec_t* base = px + (o / after) * reduce_size * after + (o % after);
+      const A sum = cpu::blocked_sum<A>(reduce_size, [&](int64_t k) {
+        return AbsPow<A>(cpu::ld<spec_t, A>(base + k * after), p);
+      });
+      cpu::st<spec_t, A>(po + o, p == 1 ? sum : p == 2 ? std::sqrt(sum) : std::pow(sum, A(1) / A(p)));
+    });
+  });
+}
+
+void NormGradientCpu(const NDArray& input, const NDArray& output, const NDArray& output_grad, NDArray& input_grad,
+                     int64_t dim, int64_t p, const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(input);
+  HT_ASSERT_SAME_DEVICE(input, output);
+  HT_ASSERT_SAME_DEVICE(input, output_grad);
+  HT_ASSERT_SAME_DEVICE(input, input_grad);
+  HT_ASSERT_SAME_SHAPE(input, input_grad);
+  HT_ASSERT_SAME_DTYPE(input, output);
+  HT_ASSERT_SAME_DTYPE(input, output_grad);
+  HT_ASSERT_SAME_DTYPE(input, input_grad);
+  HT_ASSERT_CONTIGUOUS(input_grad);
+  HT_VALUE_ERROR_IF(p < 1) << "The norm's exponent must be at least 1, got " << p;
+  const int64_t nd = int64_t(input->ndim());
+  dim = NDArrayMeta::ParseAxis(dim, nd);
+  int64_t before = 1, after = 1;
+  for (int64_t i = 0; i < nd; ++i) {
+    if (i < dim) before *= input->shape(i);
+    else if (i > dim) after *= input->shape(i);
+  }
+  const int64_t reduce_size = input->shape(dim);
+  HT_ASSERT(int64_t(output->numel()) == before * after && int64_t(output_grad->numel()) == before * after)
+    << "norm " << output->shape() << " and its gradient " << output_grad->shape() << " must hold " << before * after
+    << " values for " << input->shape() << " over dimension " << dim;
+  if (input->numel() == 0) return;
+  NDArray x = Dense(input, stream), n = Dense(output, stream), g = Dense(output_grad, stream);
+  HT_DISPATCH_FLOATING_TYPES(input->dtype(), spec_t, "NormGradientCpu", [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* px = x->data_ptr<spec_t>();
+    const spec_t* pn = n->data_ptr<spec_t>();
+    const spec_t* pg = g->data_ptr<spec_t>();
+    spec_t* pd = input_grad->data_ptr<spec_t>();
+    cpu::parallel_rows(before * reduce_size, after, [&](int64_t row) {
+      const int64_t b = row / reduce_size;
+      for (int64_t a = 0; a < after; ++a) {
+        const A v = cpu::ld<spec_t, A>(px + row * after + a);
+        const A nv = cpu::ld<spec_t, A>(pn + b * after + a), gv = cpu::ld<spec_t, A>(pg + b * after + a);
+        A r;
+        if (p == 1) r = (v > A(0) ? A(1) : v < A(0) ? A(-1) : A(0)) * gv;
+        else if (nv == A(0)) r = A(0);
+        else if (p == 2) r = gv * v / nv;
+        else r = v * std::pow(std::fabs(v), A(p - 2)) * gv / std::pow(nv, A(p - 1));
+        cpu::st<spec_t, A>(pd + row * after + a, r);
+      }
+    });
+  });
 }
 
 } // namespace impl

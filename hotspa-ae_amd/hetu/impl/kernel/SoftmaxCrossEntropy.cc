@@ -4,6 +4,11 @@
 // cuDNN softmax + elementwise + cuDNN reduce.
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
+#include "hetu/impl/utils/cpu_utils.h"
+#include "hetu/impl/utils/dispatch.h"
+
+#include <cmath>
+#include <limits>
 
 namespace hetu {
 namespace impl {
@@ -89,13 +94,81 @@ void SoftmaxCrossEntropyGradientReducedCuda(const NDArray& input_y, const NDArra
   DenseGradient(input_y, label, grad_output, &scale, output, stream);
 }
 
-void SoftmaxCrossEntropyCpu(const NDArray&, const NDArray&, NDArray&, const Stream&) {
-  HT_NOT_IMPLEMENTED << "SoftmaxCrossEntropy has no host kernel in this build; move the arrays to the accelerator";
+// Host twins (hetu/impl/kernel/SoftmaxCrossEntropy.cc:12-45 and :90-125 of the reference): per row the maximum and
+// the sum of exp(x - max); loss = -sum label * (x - max - log sum), gradient (softmax - label) * grad_loss.
+void SoftmaxCrossEntropyCpu(const NDArray& input, const NDArray& label, NDArray& output, const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(input);
+  HT_ASSERT_SAME_DEVICE(input, label);
+  HT_ASSERT_SAME_DEVICE(input, output);
+  const size_t indim = input->ndim();
+  HT_ASSERT(indim >= 1 && indim == label->ndim() && (indim == output->ndim() + 1 || (indim == 1 && output->ndim() == 1)))
+    << "Indim is " << indim << ", Label dim is " << label->ndim() << ", Output dim is " << output->ndim();
+  HT_ASSERT_SAME_SHAPE(input, label);
+  HT_ASSERT_SAME_DTYPE(input, label);
+  HT_ASSERT_SAME_DTYPE(input, output);
+  HT_ASSERT_CONTIGUOUS(output);
+  int64_t rows = 1;
+  for (size_t i = 0; i + 1 < indim; ++i) rows *= input->shape(i);
+  const int64_t cols = input->shape(indim - 1);
+  HT_ASSERT(int64_t(output->numel()) == rows) << "loss " << output->shape() << " must hold one value per row";
+  if (rows * cols == 0) return;
+  NDArray x = Dense(input, stream), l = Dense(label, stream);
+  HT_DISPATCH_FLOATING_TYPES(input->dtype(), spec_t, "SoftmaxCrossEntropyCpu", [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* xp = x->data_ptr<spec_t>();
+    const spec_t* lp = l->data_ptr<spec_t>();
+    spec_t* out = output->data_ptr<spec_t>();
+    cpu::parallel_rows(rows, cols, [&](int64_t r) {
+      const spec_t* xr = xp + r * cols;
+      const spec_t* lr = lp + r * cols;
+      const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
+      const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+      const A lse = m + std::log(sum);
+      const A acc = cpu::blocked_sum<A>(cols, [&](int64_t i) {
+        return cpu::ld<spec_t, A>(lr + i) * (lse - cpu::ld<spec_t, A>(xr + i));
+      });
+      cpu::st<spec_t, A>(out + r, acc);
+    });
+  });
 }
 
-void SoftmaxCrossEntropyGradientCpu(const NDArray&, const NDArray&, const NDArray&, NDArray&, const Stream&) {
-  HT_NOT_IMPLEMENTED << "SoftmaxCrossEntropyGradient has no host kernel in this build; move the arrays to the "
-                        "accelerator";
+void SoftmaxCrossEntropyGradientCpu(const NDArray& input_y, const NDArray& label, const NDArray& grad,
+                                    NDArray& output, const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(input_y);
+  HT_ASSERT_SAME_DEVICE(input_y, label);
+  HT_ASSERT_SAME_DEVICE(input_y, grad);
+  HT_ASSERT_SAME_DEVICE(input_y, output);
+  HT_ASSERT_SAME_SHAPE(input_y, label);
+  HT_ASSERT_SAME_SHAPE(input_y, output);
+  HT_ASSERT_SAME_DTYPE(input_y, label);
+  HT_ASSERT_SAME_DTYPE(input_y, grad);
+  HT_ASSERT_SAME_DTYPE(input_y, output);
+  HT_ASSERT_CONTIGUOUS(output);
+  const size_t indim = input_y->ndim();
+  HT_ASSERT(indim >= 1);
+  int64_t rows = 1;
+  for (size_t i = 0; i + 1 < indim; ++i) rows *= input_y->shape(i);
+  const int64_t cols = input_y->shape(indim - 1);
+  HT_ASSERT(int64_t(grad->numel()) == rows) << "grad " << grad->shape() << " must hold one value per row";
+  if (rows * cols == 0) return;
+  NDArray x = Dense(input_y, stream), l = Dense(label, stream), g = Dense(grad, stream);
+  HT_DISPATCH_FLOATING_TYPES(input_y->dtype(), spec_t, "SoftmaxCrossEntropyGradientCpu", [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* xp = x->data_ptr<spec_t>();
+    const spec_t* lp = l->data_ptr<spec_t>();
+    const spec_t* gp = g->data_ptr<spec_t>();
+    spec_t* out = output->data_ptr<spec_t>();
+    cpu::parallel_rows(rows, cols, [&](int64_t r) {
+      const spec_t* xr = xp + r * cols;
+      const spec_t* lr = lp + r * cols;
+      spec_t* dr = out + r * cols;
+      const A gr = cpu::ld<spec_t, A>(gp + r);
+      const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
+      const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+      for (int64_t i = 0; i < cols; ++i)
+        cpu::st<spec_t, A>(dr + i, (std::exp(cpu::ld<spec_t, A>(xr + i) - m) / sum - cpu::ld<spec_t, A>(lr + i)) * gr);
+    });
+  });
 }
 
 } // namespace impl

@@ -3,6 +3,10 @@
 // reference (one launch_loop_kernel each there, one hk_unary call here).
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
+#include "hetu/impl/utils/cpu_utils.h"
+#include "hetu/impl/utils/dispatch.h"
+
+#include <cmath>
 
 namespace hetu {
 namespace impl {
@@ -31,15 +35,44 @@ void OppositeCuda(const NDArray& input, NDArray& output, const Stream& stream) {
 }
 void SqrtCuda(const NDArray& input, NDArray& output, const Stream& stream) { Unary(HK_UNARY_SQRT, input, output, stream); }
 
-#define HT_NO_CPU_UNARY(name)                                                                        \
-  void name##Cpu(const NDArray&, NDArray&, const Stream&) {                                          \
-    HT_NOT_IMPLEMENTED << #name << " has no CPU kernel in this build (the product path is the GPU)"; \
+// Host twins (hetu/impl/kernel/Exp.cc, Log.cc, Opposite.cc, Sqrt.cc of the reference): one pass, float arithmetic
+// (double for float64) rounded once; the negation also takes the integer types and wraps.
+namespace {
+void UnaryHost(int op, const char* who, const NDArray& input, NDArray& output, const Stream& stream) {
+  HT_ASSERT_CPU_DEVICE(input);
+  HT_ASSERT_SAME_DEVICE(input, output);
+  HT_ASSERT_SAME_SHAPE(input, output);
+  HT_ASSERT_SAME_DTYPE(input, output);
+  HT_ASSERT_CONTIGUOUS(output);
+  if (input->numel() == 0) return;
+  NDArray x = Dense(input, stream);
+  const int64_t n = int64_t(input->numel());
+  if (op == HK_UNARY_NEG) {
+    HT_DISPATCH_INTEGER_AND_FLOATING_TYPES(input->dtype(), spec_t, who, [&]() {
+      const spec_t* px = x->data_ptr<spec_t>();
+      spec_t* po = output->data_ptr<spec_t>();
+      cpu::parallel_for(n, [&](int64_t i) { po[i] = cpu::negate<spec_t>(px[i]); });
+    });
+    return;
   }
-HT_NO_CPU_UNARY(Exp)
-HT_NO_CPU_UNARY(Log)
-HT_NO_CPU_UNARY(Opposite)
-HT_NO_CPU_UNARY(Sqrt)
-#undef HT_NO_CPU_UNARY
+  HT_DISPATCH_FLOATING_TYPES(input->dtype(), spec_t, who, [&]() {
+    using A = typename cpu::Arith<spec_t>::type;
+    const spec_t* px = x->data_ptr<spec_t>();
+    spec_t* po = output->data_ptr<spec_t>();
+    cpu::parallel_for(n, [&](int64_t i) {
+      const A v = cpu::ld<spec_t, A>(px + i);
+      cpu::st<spec_t, A>(po + i, op == HK_UNARY_EXP ? std::exp(v) : op == HK_UNARY_LOG ? std::log(v) : std::sqrt(v));
+    });
+  });
+}
+} // namespace
+
+void ExpCpu(const NDArray& input, NDArray& output, const Stream& stream) { UnaryHost(HK_UNARY_EXP, "ExpCpu", input, output, stream); }
+void LogCpu(const NDArray& input, NDArray& output, const Stream& stream) { UnaryHost(HK_UNARY_LOG, "LogCpu", input, output, stream); }
+void OppositeCpu(const NDArray& input, NDArray& output, const Stream& stream) {
+  UnaryHost(HK_UNARY_NEG, "OppositeCpu", input, output, stream);
+}
+void SqrtCpu(const NDArray& input, NDArray& output, const Stream& stream) { UnaryHost(HK_UNARY_SQRT, "SqrtCpu", input, output, stream); }
 
 } // namespace impl
 } // namespace hetu

@@ -14,6 +14,7 @@
 #include <cstdint>
 #include <limits>
 #include <type_traits>
+#include <vector>
 
 namespace hetu {
 namespace impl {
@@ -59,6 +60,79 @@ inline A blocked_max(int64_t n, F f) {
     m = v > m ? v : m;
   }
   return nan ? std::numeric_limits<A>::quiet_NaN() : m;
+}
+
+// x op y on one element of storage type T, op being 0 add, 1 subtract, 2 multiply, 3 divide (the values of the
+// HK_BINARY_* constants).  Floating-point types compute in their arithmetic type and round once; integers wrap in
+// their own width, and a division by zero gives 0 instead of a trap.
+template <typename T>
+inline T binary_op(int op, T x, T y) {
+  if constexpr (std::is_integral<T>::value) {
+    using U = typename std::make_unsigned<T>::type;
+    switch (op) {
+      case 0: return T(U(U(x) + U(y)));
+      case 1: return T(U(U(x) - U(y)));
+      case 2: return T(U(U(x) * U(y)));
+      default:
+        if (y == T(0)) return T(0);
+        if constexpr (std::is_signed<T>::value) {
+          if (y == T(-1)) return T(U(U(0) - U(x)));   // the one quotient that does not fit
+        }
+        return T(x / y);
+    }
+  } else {
+    using A = typename Arith<T>::type;
+    const A a = ld<T, A>(&x), b = ld<T, A>(&y);
+    const A r = op == 0 ? a + b : op == 1 ? a - b : op == 2 ? a * b : a / b;
+    T out;
+    st<T, A>(&out, r);
+    return out;
+  }
+}
+
+// the negation of one element; integers wrap
+template <typename T>
+inline T negate(T x) {
+  if constexpr (std::is_integral<T>::value) {
+    using U = typename std::make_unsigned<T>::type;
+    return T(U(U(0) - U(x)));
+  } else {
+    using A = typename Arith<T>::type;
+    T out;
+    st<T, A>(&out, -ld<T, A>(&x));
+    return out;
+  }
+}
+
+// f(i) for i in [0, n), shared out over the OpenMP team when there is enough of it
+template <typename F>
+inline void parallel_for(int64_t n, F f) {
+#pragma omp parallel for schedule(static) if (n >= (int64_t(1) << 16))
+  for (int64_t i = 0; i < n; ++i) f(i);
+}
+
+// Walks a dense row-major array of `nd` dimensions run by run along the last dimension: f(out_offset, a_offset,
+// b_offset) is called once per run with the element offsets of its first element in the output and in two operands
+// laid out by the strides sa / sb (0 where an operand repeats); the run has shape[nd - 1] elements, sa[nd - 1] /
+// sb[nd - 1] apart in the operands.  Runs are shared out over the OpenMP team.
+template <typename F>
+inline void for_each_run(int nd, const int64_t* shape, const int64_t* sa, const int64_t* sb, F f) {
+  if (nd == 0) { f(int64_t(0), int64_t(0), int64_t(0)); return; }
+  const int64_t inner = shape[nd - 1];
+  int64_t runs = 1;
+  for (int d = 0; d < nd - 1; ++d) runs *= shape[d];
+  const bool par = runs > 1 && runs * inner >= (int64_t(1) << 16);
+#pragma omp parallel for schedule(static) if (par)
+  for (int64_t r = 0; r < runs; ++r) {
+    int64_t rem = r, oa = 0, ob = 0;
+    for (int d = nd - 2; d >= 0; --d) {
+      const int64_t q = rem / shape[d], c = rem - q * shape[d];
+      oa += c * sa[d];
+      ob += c * sb[d];
+      rem = q;
+    }
+    f(r * inner, oa, ob);
+  }
 }
 
 // rows are independent in every kernel here

@@ -229,8 +229,7 @@ def test_binary_reads_operands_through_their_strides(ht):
     out = torch.empty(4, 6)
     ht.binary("sub", a, b, out)
     assert torch.equal(out, a - b)
-    ht.binary("mul", a[:, ::2], b[:, 1::2], out[:, :3].contiguous())   # column slices
-    o2 = torch.empty(4, 3)
+    o2 = torch.empty(4, 3)                                         # column slices
     ht.binary("mul", a[:, ::2], b[:, 1::2], o2)
     assert torch.equal(o2, a[:, ::2] * b[:, 1::2])
     with pytest.raises(ht.HetuError):

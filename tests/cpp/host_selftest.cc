@@ -291,6 +291,108 @@ int main() {
       [&] { hetu::impl::ReduceCuda(a, out, {0}, kSUM, Stream(Device(kCUDA, 0), 1)); }));
   });
 
+  run("host twins of the neighbours: broadcasting arithmetic, broadcasts, norms, losses, batch norm", [] {
+    const Device cpu(kCPU);
+    const Stream st(cpu, 0);
+    // [3, 1, 5] op [4, 1] -> [3, 4, 5], one operand read through a transposed view
+    NDArray a = NDArray::empty({3, 1, 5}, cpu, kFloat32), b = NDArray::empty({1, 4}, cpu, kFloat32);
+    for (int i = 0; i < 15; ++i) a->data_ptr<float>()[i] = float(i + 1);
+    for (int i = 0; i < 4; ++i) b->data_ptr<float>()[i] = float(2 * i + 1);
+    NDArray bt = NDArray::permute(b, {1, 0});   // [4, 1], strides {1, 4}
+    NDArray out = NDArray::empty({3, 4, 5}, cpu, kFloat32);
+    hetu::impl::SubElewiseCpu(a, bt, out, st);
+    hetu::impl::DivElewiseCpu(out, bt, out, st);   // in place
+    for (int i = 0; i < 3; ++i)
+      for (int j = 0; j < 4; ++j)
+        for (int k = 0; k < 5; ++k)
+          CHECK(out->data_ptr<float>()[(i * 4 + j) * 5 + k] == (float(i * 5 + k + 1) - float(2 * j + 1)) / float(2 * j + 1));
+    CHECK(throws<assertion_error>([&] { hetu::impl::AddElewiseCpu(a, NDArray::empty({3}, cpu, kFloat32), out, st); }));
+    // integers wrap, a zero divisor gives zero
+    NDArray i8 = NDArray::empty({4}, cpu, kInt8), j8 = NDArray::empty({4}, cpu, kInt8), o8 = NDArray::empty({4}, cpu, kInt8);
+    const int8_t xs[4] = {127, -128, 100, 7}, ys[4] = {1, -1, 0, -2};
+    for (int i = 0; i < 4; ++i) { i8->data_ptr<int8_t>()[i] = xs[i]; j8->data_ptr<int8_t>()[i] = ys[i]; }
+    hetu::impl::AddElewiseCpu(i8, j8, o8, st);
+    CHECK(o8->data_ptr<int8_t>()[0] == -128 && o8->data_ptr<int8_t>()[1] == 127);
+    hetu::impl::DivElewiseCpu(i8, j8, o8, st);
+    CHECK(o8->data_ptr<int8_t>()[1] == -128 && o8->data_ptr<int8_t>()[2] == 0 && o8->data_ptr<int8_t>()[3] == -3);
+    hetu::impl::OppositeCpu(i8, o8, st);
+    CHECK(o8->data_ptr<int8_t>()[0] == -127 && o8->data_ptr<int8_t>()[1] == -128);
+    CHECK(throws<not_implemented>([&] { hetu::impl::ExpCpu(i8, o8, st); }));
+    // constants: value - x, and a zero divisor is refused
+    NDArray c = NDArray::empty({3, 1, 5}, cpu, kFloat32);
+    hetu::impl::SubConstCpu(a, 20.0, c, st);
+    CHECK(c->data_ptr<float>()[14] == 5.f);
+    CHECK(throws<assertion_error>([&] { hetu::impl::DivConstCpu(a, 0.0, c, st); }, "Divided by 0"));
+    // broadcast [5] -> [2, 5, 3] with the input's dimension in the middle, times a constant
+    NDArray v = NDArray::empty({5}, cpu, kFloat32);
+    for (int i = 0; i < 5; ++i) v->data_ptr<float>()[i] = float(i);
+    NDArray wide = NDArray::empty({2, 5, 3}, cpu, kFloat32);
+    hetu::impl::BroadcastShapeMulCpu(v, 0.5, wide, {0, 2}, st);
+    for (int i = 0; i < 30; ++i) CHECK(wide->data_ptr<float>()[i] == 0.5f * float((i / 3) % 5));
+    CHECK(throws<assertion_error>([&] { hetu::impl::BroadcastShapeCpu(v, wide, {0, 0}, st); }, "twice"));
+    // 3-4-5: the 2-norm over the middle dimension, its gradient, and a zero norm
+    NDArray x = NDArray::zeros({2, 2, 3}, cpu, kFloat32);
+    x->data_ptr<float>()[0] = 3.f; x->data_ptr<float>()[3] = -4.f;   // column (0, :, 0) = (3, -4)
+    NDArray n = NDArray::empty({2, 3}, cpu, kFloat32), g = NDArray::empty({2, 3}, cpu, kFloat32);
+    for (int i = 0; i < 6; ++i) g->data_ptr<float>()[i] = 10.f;
+    hetu::impl::NormCpu(x, n, 1, 2, st);
+    CHECK(n->data_ptr<float>()[0] == 5.f && n->data_ptr<float>()[1] == 0.f);
+    NDArray dx = NDArray::empty({2, 2, 3}, cpu, kFloat32);
+    hetu::impl::NormGradientCpu(x, n, g, dx, 1, 2, st);
+    CHECK(dx->data_ptr<float>()[0] == 6.f && dx->data_ptr<float>()[3] == -8.f && dx->data_ptr<float>()[1] == 0.f);
+    hetu::impl::NormCpu(x, n, -2, 1, st);
+    CHECK(n->data_ptr<float>()[0] == 7.f);
+    CHECK(throws<value_error>([&] { hetu::impl::NormCpu(x, n, 1, 0, st); }));
+    // negative log likelihood: picks, and labels outside the classes
+    NDArray pred = NDArray::empty({3, 4}, cpu, kFloat32), lab = NDArray::empty({3}, cpu, kInt64);
+    for (int i = 0; i < 12; ++i) pred->data_ptr<float>()[i] = float(i);
+    lab->data_ptr<int64_t>()[0] = 2; lab->data_ptr<int64_t>()[1] = -1; lab->data_ptr<int64_t>()[2] = 4;
+    NDArray loss = NDArray::empty({3}, cpu, kFloat32);
+    hetu::impl::NLLLossCpu(pred, lab, loss, st);
+    CHECK(loss->data_ptr<float>()[0] == -2.f && loss->data_ptr<float>()[1] == 0.f && loss->data_ptr<float>()[2] == 0.f);
+    NDArray dp = NDArray::empty({3, 4}, cpu, kFloat32);
+    hetu::impl::NLLLossGradientCpu(pred, lab, loss, dp, st);
+    CHECK(dp->data_ptr<float>()[2] == 8.f && dp->data_ptr<float>()[0] == 0.f && dp->data_ptr<float>()[6] == 0.f);
+    // one-hot dense labels give the sparse loss
+    NDArray oh = NDArray::zeros({3, 4}, cpu, kFloat32), dl = NDArray::empty({3}, cpu, kFloat32);
+    NDArray sl = NDArray::empty({3}, cpu, kFloat32), cls = NDArray::empty({3}, cpu, kInt64);
+    for (int r = 0; r < 3; ++r) { oh->data_ptr<float>()[r * 4 + r] = 1.f; cls->data_ptr<int64_t>()[r] = r; }
+    hetu::impl::SoftmaxCrossEntropyCpu(pred, oh, dl, st);
+    hetu::impl::SoftmaxCrossEntropySparseCpu(pred, cls, sl, -100, st);
+    for (int r = 0; r < 3; ++r) CHECK(std::fabs(dl->data_ptr<float>()[r] - sl->data_ptr<float>()[r]) < 1e-6f);
+    // batch norm of [2, 2, 3]: channel means, inverse deviations, running statistics; then its gradient sums
+    NDArray bx = NDArray::empty({2, 2, 3}, cpu, kFloat32), by = NDArray::empty({2, 2, 3}, cpu, kFloat32);
+    for (int i = 0; i < 12; ++i) bx->data_ptr<float>()[i] = float(i);
+    NDArray sc = NDArray::empty({2}, cpu, kFloat32), bi = NDArray::zeros({2}, cpu, kFloat32);
+    NDArray rm = NDArray::zeros({2}, cpu, kFloat32), rv = NDArray::zeros({2}, cpu, kFloat32);
+    NDArray sm = NDArray::empty({2}, cpu, kFloat32), sv = NDArray::empty({2}, cpu, kFloat32);
+    sc->data_ptr<float>()[0] = sc->data_ptr<float>()[1] = 1.f;
+    hetu::impl::BatchNormCpu(bx, sc, bi, by, 0.5, 0.0, rm, rv, sm, sv, st);
+    // channel 0 holds {0, 1, 2, 6, 7, 8}: mean 4, biased variance 58 / 6, unbiased 58 / 5
+    CHECK(sm->data_ptr<float>()[0] == 4.f && sm->data_ptr<float>()[1] == 7.f);
+    CHECK(std::fabs(sv->data_ptr<float>()[0] - 1.f / std::sqrt(58.f / 6.f)) < 1e-6f);
+    CHECK(rm->data_ptr<float>()[0] == 2.f && std::fabs(rv->data_ptr<float>()[0] - 5.8f) < 1e-6f);
+    float ysum = 0.f;
+    for (int i = 0; i < 12; ++i) ysum += by->data_ptr<float>()[i];
+    CHECK(std::fabs(ysum) < 1e-5f);
+    NDArray bdx = NDArray::empty({2, 2, 3}, cpu, kFloat32), ds = NDArray::empty({2}, cpu, kFloat32),
+            dbias = NDArray::empty({2}, cpu, kFloat32);
+    hetu::impl::BatchNormGradientCpu(by, bx, sc, bdx, ds, dbias, 0.0, sm, sv, st);   // dy = y: dscale = count, dbias = 0
+    CHECK(std::fabs(ds->data_ptr<float>()[0] - 6.f) < 1e-5f && std::fabs(dbias->data_ptr<float>()[1]) < 1e-5f);
+    for (int i = 0; i < 12; ++i) CHECK(std::fabs(bdx->data_ptr<float>()[i]) < 1e-5f);   // y lies in the null space
+    CHECK(throws<assertion_error>(
+      [&] { hetu::impl::BatchNormCpu(bx, NDArray::empty({3}, cpu, kFloat32), bi, by, 0.5, 0.0, rm, rv, sm, sv, st); }));
+    // instance norm = per-plane standardisation
+    NDArray ix = NDArray::empty({1, 2, 2, 3}, cpu, kFloat32), iy = NDArray::empty({1, 2, 2, 3}, cpu, kFloat32);
+    for (int i = 0; i < 12; ++i) ix->data_ptr<float>()[i] = float(i * i);
+    NDArray im = NDArray::empty({1, 2, 1, 1}, cpu, kFloat32), iv = NDArray::empty({1, 2, 1, 1}, cpu, kFloat32);
+    hetu::impl::InstanceNormCpu(ix, im, iv, iy, 0.f, st);
+    float m0 = 0.f, q0 = 0.f;
+    for (int i = 0; i < 6; ++i) { m0 += iy->data_ptr<float>()[i]; q0 += iy->data_ptr<float>()[i] * iy->data_ptr<float>()[i]; }
+    CHECK(std::fabs(m0) < 1e-5f && std::fabs(q0 - 6.f) < 1e-4f);
+    CHECK(std::fabs(im->data_ptr<float>()[0] - 55.f / 6.f) < 1e-5f);
+  });
+
   // ------------------------------------------------------------------ pool policy
   run("pool: rounding, carving small requests from one segment", [] {
     PoolFixture f;

@@ -562,3 +562,9 @@ def memcpy_d2d(dst, src, stream=None):
 def strided_copy(src, dst, stream=None):
     check(lib().hk_strided_copy(dtype_code(src), _ptr(src), _ptr(dst), ctypes.c_int(src.dim()), _arr(src.shape),
                                 _arr(src.stride()), stream if stream is not None else current_stream()))
+
+
+def strided_scatter(src, dst, stream=None):
+    """Lays the dense array `src` over the view `dst` (same shape, any strides)."""
+    check(lib().hk_strided_scatter(dtype_code(dst), _ptr(src), _ptr(dst), ctypes.c_int(dst.dim()), _arr(dst.shape),
+                                   _arr(dst.stride()), stream if stream is not None else current_stream()))

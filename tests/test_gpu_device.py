@@ -45,6 +45,46 @@ def test_copy_and_strided_copy(hk, cuda):
         assert torch.equal(out, view.contiguous()), dt
 
 
+def test_strided_scatter_is_the_inverse_of_the_gather(hk, cuda):
+    """hk_strided_scatter lays a dense array over a view of any strides: the view then reads back as the array,
+    and no element outside the view changes; eight dimensions, empty views and single elements included."""
+    import torch
+    for dt in (torch.float32, torch.bfloat16, torch.int64, torch.uint8, torch.float64):
+        backing = torch.full((7, 12, 5), 99, dtype=dt, device=cuda)
+        view = backing.permute(2, 0, 1)[:, ::2, 1:]
+        dense = (torch.arange(view.numel(), device=cuda) % 90).to(dt).reshape(view.shape)
+        hk.strided_scatter(dense, view)
+        torch.cuda.synchronize()
+        assert torch.equal(view.contiguous(), dense), dt
+        untouched = torch.ones_like(backing, dtype=torch.bool)
+        untouched.permute(2, 0, 1)[:, ::2, 1:] = False
+        assert bool((backing[untouched] == 99).all()), dt
+        back = torch.empty_like(dense)
+        hk.strided_copy(view, back)
+        torch.cuda.synchronize()
+        assert torch.equal(back, dense), dt
+    # eight dimensions, every one permuted; a column slice of a wider array; a single element; nothing at all
+    b8 = torch.zeros((2, 3, 2, 2, 3, 2, 2, 3), dtype=torch.float32, device=cuda)
+    v8 = b8.permute(7, 6, 5, 4, 3, 2, 1, 0)
+    d8 = torch.arange(v8.numel(), dtype=torch.float32, device=cuda).reshape(v8.shape)
+    hk.strided_scatter(d8, v8)
+    wide = torch.zeros((33, 200), dtype=torch.bfloat16, device=cuda)
+    pitched = wide[:, 8:136]
+    dp = torch.randn(33, 128, device=cuda).to(torch.bfloat16)
+    hk.strided_scatter(dp, pitched)
+    one = torch.zeros((), dtype=torch.float32, device=cuda)
+    hk.strided_scatter(torch.full((), 3.0, device=cuda), one)
+    hk.strided_scatter(torch.empty((0, 4), device=cuda), torch.empty((4, 0), device=cuda).t())
+    torch.cuda.synchronize()
+    assert torch.equal(v8.contiguous(), d8)
+    assert torch.equal(pitched.contiguous(), dp) and float(wide[:, :8].abs().sum()) == 0 and float(wide[:, 136:].abs().sum()) == 0
+    assert float(one) == 3.0
+    lib = hk.lib()
+    shape9 = (ctypes.c_int64 * 9)(*([1] * 9))
+    assert lib.hk_strided_scatter(0, ctypes.c_void_p(one.data_ptr()), ctypes.c_void_p(one.data_ptr()), 9, shape9, shape9,
+                                  hk.current_stream()) != 0
+
+
 def test_streams_events_and_ordering(hk, cuda):
     import torch
     lib = hk.lib()

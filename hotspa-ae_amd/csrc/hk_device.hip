@@ -161,6 +161,65 @@ __global__ __launch_bounds__(256) void strided_copy_kernel(const W* __restrict__
   }
 }
 
+// The same copy for a view whose unit-stride dimension is not the last one (a transposed or permuted array):
+// 64 x 64 tiles of the two dimensions that are contiguous on one side each go through LDS, so that both the reads
+// and the writes of a wavefront are consecutive in memory.  u = the view's unit-stride dimension, v = the last
+// dimension (unit stride in the dense array); the other dimensions are walked by the workgroup index.
+struct TransposeMeta {
+  int n_other;
+  int64_t other_shape[6], other_dense[6], other_view[6];
+  int64_t U, V;        // extents of u and v
+  int64_t u_dense;     // stride of u in the dense array
+  int64_t v_view;      // stride of v in the view
+  int64_t tiles_u, tiles_v;
+};
+
+template <typename W, bool SCATTER>
+__global__ __launch_bounds__(256) void strided_transpose_kernel(const W* __restrict__ src, W* __restrict__ dst,
+                                                                TransposeMeta m) {
+  constexpr int TS = 64;
+  __shared__ W tile[TS][TS + 1];
+  int64_t b = blockIdx.x;
+  const int64_t tv = b % m.tiles_v;
+  b /= m.tiles_v;
+  const int64_t tu = b % m.tiles_u;
+  b /= m.tiles_u;
+  int64_t base_dense = 0, base_view = 0;
+  for (int d = m.n_other - 1; d >= 0; --d) {
+    const int64_t q = b / m.other_shape[d], idx = b - q * m.other_shape[d];
+    base_dense += idx * m.other_dense[d];
+    base_view += idx * m.other_view[d];
+    b = q;
+  }
+  const int tx = int(threadIdx.x & 63), ty = int(threadIdx.x >> 6);
+  const int64_t u0 = tu * TS, v0 = tv * TS;
+  const W* dense_in = src + base_dense;
+  const W* view_in = src + base_view;
+  W* dense_out = dst + base_dense;
+  W* view_out = dst + base_view;
+  if constexpr (!SCATTER) {
+    for (int j = ty; j < TS; j += 4) {             // lanes run along u: consecutive in the view
+      const int64_t u = u0 + tx, v = v0 + j;
+      if (u < m.U && v < m.V) tile[j][tx] = view_in[u + v * m.v_view];
+    }
+    __syncthreads();
+    for (int j = ty; j < TS; j += 4) {             // lanes run along v: consecutive in the dense array
+      const int64_t u = u0 + j, v = v0 + tx;
+      if (u < m.U && v < m.V) dense_out[u * m.u_dense + v] = tile[tx][j];
+    }
+  } else {
+    for (int j = ty; j < TS; j += 4) {
+      const int64_t u = u0 + j, v = v0 + tx;
+      if (u < m.U && v < m.V) tile[j][tx] = dense_in[u * m.u_dense + v];
+    }
+    __syncthreads();
+    for (int j = ty; j < TS; j += 4) {
+      const int64_t u = u0 + tx, v = v0 + j;
+      if (u < m.U && v < m.V) view_out[u + v * m.v_view] = tile[tx][j];
+    }
+  }
+}
+
 } // namespace hk
 
 using namespace hk;
@@ -172,22 +231,85 @@ static int strided_copy_any(const char* who, int dtype, const void* src, void* d
   HK_REQUIRE(ndim == 0 || (shape && strides), HK_ERR_INVALID, "%s: null meta", who);
   size_t es = dtype_size(dtype);
   HK_REQUIRE(es != 0, HK_ERR_UNSUPPORTED, "%s: unknown dtype %d", who, dtype);
+  // extents of 1 carry no index; neighbours that the view steps through like one dimension become one
   StridedMeta m;
-  m.ndim = ndim;
+  m.ndim = 0;
   int64_t numel = 1;
   for (int d = 0; d < ndim; ++d) {
     HK_REQUIRE(shape[d] >= 0, HK_ERR_INVALID, "%s: negative extent", who);
-    m.shape[d] = shape[d];
-    m.stride[d] = strides[d];
     numel *= shape[d];
+    if (shape[d] == 1) continue;
+    if (m.ndim > 0 && m.stride[m.ndim - 1] == strides[d] * shape[d]) {
+      m.shape[m.ndim - 1] *= shape[d];
+      m.stride[m.ndim - 1] = strides[d];
+    } else {
+      m.shape[m.ndim] = shape[d];
+      m.stride[m.ndim] = strides[d];
+      ++m.ndim;
+    }
   }
   if (numel == 0) return HK_OK;
   HK_REQUIRE(src && dst, HK_ERR_INVALID, "%s: null pointer", who);
+  hipStream_t s = as_hip(stream);
+
+  // a permuted view: the dimension it is contiguous in is not the last one
+  const int v = m.ndim - 1;
+  int u = -1;
+  if (m.ndim >= 2 && m.stride[v] != 1 && m.shape[v] >= 16) {
+    for (int d = 0; d < v; ++d)
+      if (m.stride[d] == 1 && m.shape[d] >= 16 && (u < 0 || m.shape[d] > m.shape[u])) u = d;
+  }
+  if (u >= 0) {
+    TransposeMeta t;
+    t.n_other = 0;
+    int64_t dense_stride = 1, others = 1;
+    int64_t dense_of[8];
+    for (int d = m.ndim - 1; d >= 0; --d) { dense_of[d] = dense_stride; dense_stride *= m.shape[d]; }
+    t.u_dense = dense_of[u];
+    for (int d = 0; d < m.ndim; ++d) {
+      if (d == u || d == v) continue;
+      t.other_shape[t.n_other] = m.shape[d];
+      t.other_dense[t.n_other] = dense_of[d];
+      t.other_view[t.n_other] = m.stride[d];
+      ++t.n_other;
+      others *= m.shape[d];
+    }
+    t.U = m.shape[u];
+    t.V = m.shape[v];
+    t.v_view = m.stride[v];
+    t.tiles_u = (t.U + 63) / 64;
+    t.tiles_v = (t.V + 63) / 64;
+    const int64_t nblocks = t.tiles_u * t.tiles_v * others;
+    if (nblocks <= 0x7fffffffLL) {
+      dim3 g{unsigned(nblocks)}, b{256};
+      switch (es) {
+        case 1: HK_LAUNCH((strided_transpose_kernel<uint8_t, SCATTER>), g, b, 0, s, (const uint8_t*)src, (uint8_t*)dst, t); break;
+        case 2: HK_LAUNCH((strided_transpose_kernel<uint16_t, SCATTER>), g, b, 0, s, (const uint16_t*)src, (uint16_t*)dst, t); break;
+        case 4: HK_LAUNCH((strided_transpose_kernel<uint32_t, SCATTER>), g, b, 0, s, (const uint32_t*)src, (uint32_t*)dst, t); break;
+        default: HK_LAUNCH((strided_transpose_kernel<uint64_t, SCATTER>), g, b, 0, s, (const uint64_t*)src, (uint64_t*)dst, t); break;
+      }
+      return launch_check("strided_transpose_kernel");
+    }
+  }
+
+  // rows that are contiguous on both sides and made of whole 16-byte vectors move as vectors
+  if (m.ndim >= 1 && m.stride[v] == 1 && es < 16) {
+    const int64_t k = int64_t(16 / es);
+    bool ok = m.shape[v] % k == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
+              reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+    for (int d = 0; d < v; ++d) ok = ok && m.stride[d] % k == 0;
+    if (ok) {
+      m.shape[v] /= k;
+      for (int d = 0; d < v; ++d) m.stride[d] /= k;
+      numel /= k;
+      es = 16;
+    }
+  }
   int64_t blocks = (numel + 255) / 256;
   if (blocks > 65536) blocks = 65536;
   dim3 g{unsigned(blocks)}, b{256};
-  hipStream_t s = as_hip(stream);
   switch (es) {
+    case 16: HK_LAUNCH((strided_copy_kernel<u32x4, SCATTER>), g, b, 0, s, (const u32x4*)src, (u32x4*)dst, m, numel); break;
     case 1: HK_LAUNCH((strided_copy_kernel<uint8_t, SCATTER>), g, b, 0, s, (const uint8_t*)src, (uint8_t*)dst, m, numel); break;
     case 2: HK_LAUNCH((strided_copy_kernel<uint16_t, SCATTER>), g, b, 0, s, (const uint16_t*)src, (uint16_t*)dst, m, numel); break;
     case 4: HK_LAUNCH((strided_copy_kernel<uint32_t, SCATTER>), g, b, 0, s, (const uint32_t*)src, (uint32_t*)dst, m, numel); break;

@@ -85,6 +85,54 @@ def test_strided_scatter_is_the_inverse_of_the_gather(hk, cuda):
                                   hk.current_stream()) != 0
 
 
+@pytest.mark.parametrize("dt", ["uint8", "bfloat16", "float32", "int64"])
+def test_permuted_views_take_the_tiled_path(hk, cuda, dt):
+    """Views whose contiguous dimension is not the last one (every permutation of three and four dimensions, extents
+    around the 64-element tile, sliced and with a dimension of 1) gather into, and scatter from, a dense array
+    exactly as torch's own copy does; nothing outside a scattered view changes."""
+    import itertools
+    import torch
+    td = getattr(torch, dt)
+    cases = []
+    for shape in ((65, 130, 3), (3, 64, 200), (17, 1, 100, 33), (2, 70, 5, 129)):
+        for perm in itertools.permutations(range(len(shape))):
+            cases.append((shape, perm))
+    for shape, perm in cases:
+        n = int(np.prod(shape))
+        base = (torch.arange(n, device=cuda) % 251).to(td).reshape(shape)
+        view = base.permute(perm)
+        out = torch.empty(view.shape, dtype=td, device=cuda)
+        hk.strided_copy(view, out)
+        assert torch.equal(out, view.contiguous()), (shape, perm)
+        backing = torch.zeros(shape, dtype=td, device=cuda)
+        hk.strided_scatter(out, backing.permute(perm))
+        assert torch.equal(backing, base), (shape, perm)
+    # a sliced transposed view: strides that are not products of the extents, and a covered region with holes
+    backing = torch.full((300, 260), 9, dtype=td, device=cuda)
+    view = backing.t()[3:200:2, 10:290]          # [99, 280]: rows step 2 columns of the backing, columns are its rows
+    dense = (torch.arange(view.numel(), device=cuda) % 200).to(td).reshape(view.shape)
+    hk.strided_scatter(dense, view)
+    assert torch.equal(view.contiguous(), dense)
+    covered = torch.zeros_like(backing, dtype=torch.bool)
+    covered.t()[3:200:2, 10:290] = True
+    assert bool((backing[~covered] == 9).all())
+    back = torch.empty_like(dense)
+    hk.strided_copy(view, back)
+    assert torch.equal(back, dense)
+    # rows contiguous on both sides: whole 16-byte vectors when the pitch, the width and the start allow it
+    # (columns 16 .. 144 of a 208-column array), element by element when they do not (columns 3 .. 131)
+    for lo, hi in ((16, 144), (3, 131)):
+        wide = torch.full((5, 37, 208), 9, dtype=td, device=cuda)
+        view = wide.permute(1, 0, 2)[:, :, lo:hi]
+        dense = (torch.arange(view.numel(), device=cuda) % 200).to(td).reshape(view.shape)
+        hk.strided_scatter(dense, view)
+        assert torch.equal(view.contiguous(), dense)
+        assert bool((wide[:, :, :lo] == 9).all()) and bool((wide[:, :, hi:] == 9).all())
+        back = torch.empty_like(dense)
+        hk.strided_copy(view, back)
+        assert torch.equal(back, dense)
+
+
 def test_streams_events_and_ordering(hk, cuda):
     import torch
     lib = hk.lib()

@@ -94,7 +94,7 @@ def test_permuted_views_take_the_tiled_path(hk, cuda, dt):
     import torch
     td = getattr(torch, dt)
     cases = []
-    for shape in ((65, 130, 3), (3, 64, 200), (17, 1, 100, 33), (2, 70, 5, 129)):
+    for shape in ((65, 130, 3), (3, 64, 200), (17, 1, 100, 33), (2, 70, 5, 129), (4, 130, 258)):
         for perm in itertools.permutations(range(len(shape))):
             cases.append((shape, perm))
     for shape, perm in cases:

@@ -68,6 +68,7 @@ static const char* const kTuneNames[] = {
   "reduce_outer_waves_across",  // wavefronts of a column-reduction workgroup side by side across columns
   "reduce_outer_waves",         // wavefronts of a column-reduction workgroup in all
   "norm_fwd_rows",              // rows a workgroup of the forward norm kernel takes (1 or 2)
+  "norm_fwd_resident",         // workgroups of the two-row forward norm kernel resident per compute unit (-1: no cap)
 };
 constexpr int kNumTune = sizeof(kTuneNames) / sizeof(kTuneNames[0]);
 static_assert(kNumTune == TUNE_NUM_KEYS, "tune name table out of sync with TuneKey");

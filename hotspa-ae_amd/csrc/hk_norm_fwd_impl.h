@@ -308,7 +308,13 @@ template <typename T, int NV, bool WAVE_ROW, bool HAS_RES, bool IS_RMS>
 static void launch_norm_fwd_width(const NormFwdArgs& a, int rows_per_block, dim3 grid, dim3 block, hipStream_t s) {
   if constexpr (!WAVE_ROW && max_rows_per_block<T>(NV, HAS_RES) >= 2) {
     if (rows_per_block == 2) {
-      HK_LAUNCH((norm_fwd_kernel<T, NV, false, HAS_RES, IS_RMS, 2>), grid, block, 0, s, a);
+      // two rows of several vectors per thread: fewer workgroups per compute unit than the thread limit admits
+      // stream faster (256 threads: 5 instead of 8, 83.5 against 84.8 us at 4096 bf16 columns; 512 threads: 3
+      // instead of 4, 44.7 against 45.9 us at 4096 fp32 columns; 2 lose again)
+      int resident = tune_get(TUNE_NORM_FWD_RESIDENT);
+      if (resident == 0) resident = block.x == 256 ? 5 : (block.x == 512 ? 3 : 0);
+      const size_t lds = lds_bytes_for_residency(resident, sizeof(float) * 2 * kMaxWaves * 2 * 2);
+      HK_LAUNCH((norm_fwd_kernel<T, NV, false, HAS_RES, IS_RMS, 2>), grid, block, lds, s, a);
       return;
     }
   }

@@ -371,6 +371,22 @@ def case_copy(hk, torch, nsets):
     return (lambda i: hk.copy_kernel(dst[i % nsets], src[i % nsets])), 2 * n, 1
 
 
+def case_strided(hk, torch, nsets, which):
+    """The extra pass an operator pays for an operand that is neither dense nor row-pitched: a permuted view gathered
+    into a dense array (hk_strided_copy), or a dense result laid over such a view (hk_strided_scatter)."""
+    if which == "transposed fp32":
+        shape, perm, dt = (8192, 4096), (1, 0), torch.float32
+    elif which == "swapped bf16":
+        shape, perm, dt = (32, 2048, 2048), (0, 2, 1), torch.bfloat16
+    else:   # rows stay contiguous: [64, 512, 4096] with the first two dimensions swapped
+        shape, perm, dt = (64, 512, 4096), (1, 0, 2), torch.bfloat16
+    srcs = [_randn(torch, shape, dt, 1.0, 961 + k) for k in range(nsets)]
+    views = [x.permute(perm) for x in srcs]
+    outs = [torch.empty(views[0].shape, dtype=dt, device="cuda") for _ in range(nsets)]
+    nbytes = 2 * srcs[0].numel() * srcs[0].element_size()
+    return (lambda i: hk.strided_copy(views[i % nsets], outs[i % nsets])), nbytes, 1
+
+
 def case_fill(hk, torch, nsets):
     import ctypes
     n = 1 << 28
@@ -526,6 +542,11 @@ CASES = [
     ("next: gradient of mean axis1 bf16 [32768x4096] (write only)", lambda hk, t, n: case_reduce_gradient(hk, t, n, 1)),
     ("next: batch norm fwd bf16 [256,256,56,56] (2R+1W, 3 launches)", lambda hk, t, n: case_batch_norm(hk, t, n, "fwd")),
     ("next: batch norm bwd bf16 [256,256,56,56] (4R+1W, 3 launches)", lambda hk, t, n: case_batch_norm(hk, t, n, "bwd")),
+    ("next: gather of a transposed view fp32 [8192x4096]", lambda hk, t, n: case_strided(hk, t, n, "transposed fp32")),
+    ("next: gather of a view with the last two dimensions swapped bf16 [32x2048x2048]",
+     lambda hk, t, n: case_strided(hk, t, n, "swapped bf16")),
+    ("next: gather of a view with the first two dimensions swapped bf16 [64x512x4096]",
+     lambda hk, t, n: case_strided(hk, t, n, "outer bf16")),
     ("C4 rmsnorm fwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "fwd")),
     ("C4 rmsnorm bwd bf16 [32768x4096]", lambda hk, t, n: case_rmsnorm(hk, t, n, "bwd")),
     ("C5 sce fwd bf16 [16384x32000]", lambda hk, t, n: case_sce(hk, t, 2, "fwd")),

@@ -252,6 +252,7 @@ static int strided_copy_any(const char* who, int dtype, const void* src, void* d
   if (numel == 0) return HK_OK;
   HK_REQUIRE(src && dst, HK_ERR_INVALID, "%s: null pointer", who);
   hipStream_t s = as_hip(stream);
+  profile_before(s);
 
   // a permuted view: the dimension it is contiguous in is not the last one
   const int v = m.ndim - 1;
@@ -289,6 +290,7 @@ static int strided_copy_any(const char* who, int dtype, const void* src, void* d
         case 4: HK_LAUNCH((strided_transpose_kernel<uint32_t, SCATTER>), g, b, 0, s, (const uint32_t*)src, (uint32_t*)dst, t); break;
         default: HK_LAUNCH((strided_transpose_kernel<uint64_t, SCATTER>), g, b, 0, s, (const uint64_t*)src, (uint64_t*)dst, t); break;
       }
+      profile_after(s);
       return launch_check("strided_transpose_kernel");
     }
   }
@@ -316,6 +318,7 @@ static int strided_copy_any(const char* who, int dtype, const void* src, void* d
     case 4: HK_LAUNCH((strided_copy_kernel<uint32_t, SCATTER>), g, b, 0, s, (const uint32_t*)src, (uint32_t*)dst, m, numel); break;
     default: HK_LAUNCH((strided_copy_kernel<uint64_t, SCATTER>), g, b, 0, s, (const uint64_t*)src, (uint64_t*)dst, m, numel); break;
   }
+  profile_after(s);
   return launch_check("strided_copy_kernel");
 }
 

@@ -356,7 +356,7 @@ static int launch_norm_fwd_nv(const NormFwdArgs& a, int nv, int rpb, dim3 grid, 
 
 // Picks threads-per-row and vectors-per-thread for a row of `nvec` 16-byte
 // vectors.  Returns false when the row does not fit the register kernels.
-static bool pick_row_shape(int nvec, int forced_threads, int max_nv, int wave_row_max_nv,
+static bool pick_row_shape(int nvec, int forced_threads, int max_nv, int wave_row_max_nv, bool many_rows,
                            int* threads, int* nv) {
   if (forced_threads > 0) {
     int t = std::min(1024, std::max(64, (forced_threads + 63) / 64 * 64));
@@ -378,12 +378,14 @@ static bool pick_row_shape(int nvec, int forced_threads, int max_nv, int wave_ro
   // (5120 bf16 columns = 640 vectors = 128 threads x 5): no idle lanes, and the
   // statistics merge takes its equal-count form.
   // A 512-thread workgroup (two wavefronts on each of the four SIMDs) is as good when it gets by with two vectors
-  // (4096 fp32 columns: 46 us against 49 us for 256 x 4); widths that load the SIMDs unevenly (320, 384) are not.
+  // (4096 fp32 columns: 46 us against 49 us for 256 x 4); widths that load the SIMDs unevenly (320, 384) are not,
+  // except that 320 x 2 beats 128 x 5 once the input is large enough for two rows per workgroup (5120 bf16
+  // columns, 16384 rows: 55.4 against 56.4 us; one row per workgroup: 61.4 against 57.7 us).
   static const int kCounts[] = {2, 3, 4, 5, 6, 8};
   for (int n : kCounts) {
     if (n > max_nv) break;
     int t = ((nvec + n - 1) / n + 63) / 64 * 64;
-    if ((t <= 256 || (t == 512 && n == 2)) && n * t == nvec) {
+    if ((t <= 256 || (t == 512 && n == 2) || (t == 320 && n == 2 && many_rows)) && n * t == nvec) {
       *threads = t;
       *nv = n;
       return true;
@@ -425,7 +427,11 @@ int norm_fwd_typed(NormFwdArgs a, hipStream_t s) {
   // flight next to it)
   const int max_nv = has_res ? std::min(8, 64 / VEC) : 64 / VEC;
   const int wave_nv = has_res ? (VEC == 4 ? 8 : 4) : (VEC == 4 ? 16 : 8);
-  if (vec_ok && pick_row_shape(a.nvec, tune_get(TUNE_NORM_FWD_THREADS), max_nv, wave_nv, &threads, &nv)) {
+  // large inputs take two rows per workgroup (below), which also changes the best width of some rows
+  const int want_rows = tune_get(TUNE_NORM_FWD_ROWS);
+  const bool many_rows = want_rows > 0 ? want_rows >= 2 : a.rows >= 16 * int64_t(device_cu_count());
+  if (vec_ok &&
+      pick_row_shape(a.nvec, tune_get(TUNE_NORM_FWD_THREADS), max_nv, wave_nv, many_rows, &threads, &nv)) {
     if (threads == 64) {
       dim3 grid(unsigned((a.rows + 3) / 4)), block(256);
       return has_res ? launch_norm_fwd_nv<T, true, true>(a, nv, 1, grid, block, s)
@@ -436,10 +442,7 @@ int norm_fwd_typed(NormFwdArgs a, hipStream_t s) {
     int rpb = 1;
     if (threads <= 512) {
       const int most = max_rows_per_block<T>(nv, has_res);
-      const int want = tune_get(TUNE_NORM_FWD_ROWS);
-      if (want > 0) rpb = want >= 2 ? 2 : 1;
-      else rpb = a.rows >= 16 * int64_t(device_cu_count()) ? 2 : 1;
-      rpb = std::min(rpb, most);
+      rpb = std::min(many_rows ? 2 : 1, most);
     }
     dim3 grid{unsigned((a.rows + rpb - 1) / rpb)}, block{unsigned(threads)};
     return has_res ? launch_norm_fwd_nv<T, false, true>(a, nv, rpb, grid, block, s)

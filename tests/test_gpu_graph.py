@@ -160,3 +160,52 @@ def test_graph_replays_match_eager_widened_calls(hk, cuda):
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), "output %d differs on replay %d" % (i, trial)
         assert torch.equal(run_mean, want_running[0]) and torch.equal(run_var, want_running[1])
+
+
+def test_graph_replays_of_the_large_input_forward_launches(hk, cuda):
+    """Inputs tall enough for the forward norm's two-rows-per-workgroup launch (which asks for dynamic LDS to bound
+    the workgroups resident per compute unit) recorded into a graph: RMSNorm at 4096 bf16 columns (256 threads),
+    LayerNorm at 4096 fp32 columns (512 threads) and at 5120 bf16 columns (320 threads); every replay equals eager."""
+    import torch
+    g = torch.Generator(device=cuda).manual_seed(778)
+    bf = torch.bfloat16
+    rows = 8192
+    cases = []
+    for cols, dt, rms in ((4096, bf, True), (4096, torch.float32, False), (5120, bf, False)):
+        x = torch.randn(rows, cols, generator=g, device=cuda).to(dt)
+        w = (torch.rand(cols, generator=g, device=cuda) + 0.5).to(dt)
+        b = None if rms else (torch.randn(cols, generator=g, device=cuda) * 0.1).to(dt)
+        y = torch.empty_like(x)
+        mu, rs = torch.empty(rows, device=cuda), torch.empty(rows, device=cuda)
+        cases.append((x, w, b, y, mu, rs, rms))
+
+    def step():
+        for x, w, b, y, mu, rs, rms in cases:
+            if rms:
+                hk.dropout_add_ln_fwd(x, None, w, None, y, None, mu, rs, 1e-6, True)
+            else:
+                hk.layer_norm_fwd(x, w, b, y, mu, rs, 1e-5, stat_kind=1)
+
+    outs = [t for c in cases for t in (c[3], c[4], c[5])]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for trial in range(3):
+        for c in cases:
+            c[0].copy_(torch.randn(c[0].shape, generator=g, device=cuda).to(c[0].dtype))
+        step()
+        torch.cuda.synchronize()
+        want = [o.clone() for o in outs]
+        for o in outs:
+            o.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(outs, want)):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), "output %d differs on replay %d" % (i, trial)

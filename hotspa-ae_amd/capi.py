@@ -124,9 +124,74 @@ def _pitch(t, cols):
     return t.stride(0) if t.shape[0] > 1 else cols
 
 
+def row_levels(tensors):
+    """The joint row levels of same-shaped operands whose last dimension has unit stride: (level_rows, steps) with
+    level_rows = [n0, n1, n2] innermost first and steps[k] = the three element steps of operand k (None for an absent
+    operand), as the *_strided_rows entry points take them.  Leading dimensions that step together in EVERY operand
+    are merged; returns None when more than three levels remain."""
+    present = [t for t in tensors if t is not None]
+    ref = present[0]
+    nd = ref.dim()
+    for t in present:
+        if tuple(t.shape) != tuple(ref.shape):
+            raise HkError(-1, "operands of one call must have one shape, got %s and %s" % (tuple(ref.shape), tuple(t.shape)))
+        if nd and t.shape[-1] > 1 and t.stride(-1) != 1:
+            raise HkError(-1, "the last dimension must have unit stride, got strides %s" % (tuple(t.stride()),))
+    cols = ref.shape[-1] if nd else 1
+    levels = []                      # (count, [step of every present operand]), innermost first
+    for i in range(nd - 2, -1, -1):
+        n = ref.shape[i]
+        if n == 1:
+            continue
+        steps = [t.stride(i) for t in present]
+        if levels and all(st == levels[-1][0] * ls for st, ls in zip(steps, levels[-1][1])):
+            levels[-1] = (levels[-1][0] * n, levels[-1][1])
+        else:
+            levels.append((n, steps))
+    if len(levels) > 3:
+        return None
+    while len(levels) < 3:
+        levels.append((1, [cols if not levels else 0] * len(present)))
+    counts = [l[0] for l in levels]
+    out, k = [], 0
+    for t in tensors:
+        if t is None:
+            out.append(None)
+        else:
+            out.append([levels[0][1][k], levels[1][1][k], levels[2][1][k]])
+            k += 1
+    return counts, out
+
+
+def _steps(v):
+    return None if v is None else _arr(v)
+
+
+def _multi_level(tensors):
+    """(level_rows, steps) when the operands need the *_strided_rows entry points: some operand is neither dense
+    nor a 2-D row-pitched view.  None when the dense / pitched entry points take them (or nothing does)."""
+    present = [t for t in tensors if t is not None]
+    if all(t.is_contiguous() or t.dim() == 2 for t in present):
+        return None
+    lv = row_levels(tensors)
+    if lv is None:
+        raise HkError(-1, "operands need more than three row levels; make them dense first")
+    return lv
+
+
 def layer_norm_fwd(x, gamma, beta, y, mean, stat, eps, stat_kind=HK_STAT_RSTD, stream=None):
     rows = x.numel() // x.shape[-1] if x.numel() else 0
     cols = x.shape[-1]
+    lv = _multi_level([x, y])
+    if lv is not None:
+        counts, (xs, ys) = lv
+        check(lib().hk_layer_norm_fwd_strided_rows(dtype_code(x), _ptr(x), _steps(xs), _ptr(gamma), _ptr(beta), _ptr(y),
+                                                   _steps(ys), _ptr(mean), _ptr(stat),
+                                                   dtype_code(mean if mean is not None else stat),
+                                                   ctypes.c_int(stat_kind), _arr(counts), _i64(cols),
+                                                   ctypes.c_float(eps),
+                                                   stream if stream is not None else current_stream()))
+        return
     check(lib().hk_layer_norm_fwd_pitched(dtype_code(x), _ptr(x), _i64(_pitch(x, cols)), _ptr(gamma), _ptr(beta),
                                           _ptr(y), _i64(_pitch(y, cols)), _ptr(mean), _ptr(stat),
                                           dtype_code(mean if mean is not None else stat), ctypes.c_int(stat_kind),
@@ -154,6 +219,17 @@ def layer_norm_bwd(dy, x_or_y, gamma, beta, mean, stat, dx, dgamma, dbeta, eps, 
     if workspace is None:
         workspace = _workspace(norm_bwd_workspace_bytes(dtype_code(dy), rows, cols), dy.device)
     wsb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    lv = _multi_level([dy, x_or_y, dx])
+    if lv is not None:
+        counts, (dys, xs, dxs) = lv
+        check(lib().hk_layer_norm_bwd_strided_rows(dtype_code(dy), _ptr(dy), _steps(dys), _ptr(x_or_y), _steps(xs),
+                                                   _ptr(gamma), _ptr(beta), _ptr(mean), _ptr(stat), dtype_code(stat),
+                                                   ctypes.c_int(stat_kind), _ptr(dx), _steps(dxs), _ptr(dgamma),
+                                                   _ptr(dbeta), _arr(counts), _i64(cols), ctypes.c_float(eps),
+                                                   ctypes.c_int(int(memory_efficient)), ctypes.c_int(int(clamp_gamma)),
+                                                   _ptr(workspace), ctypes.c_size_t(wsb),
+                                                   stream if stream is not None else current_stream()))
+        return workspace
     check(lib().hk_layer_norm_bwd_pitched(dtype_code(dy), _ptr(dy), _i64(_pitch(dy, cols)), _ptr(x_or_y),
                                           _i64(_pitch(x_or_y, cols)), _ptr(gamma), _ptr(beta), _ptr(mean),
                                           _ptr(stat), dtype_code(stat), ctypes.c_int(stat_kind), _ptr(dx),
@@ -165,8 +241,19 @@ def layer_norm_bwd(dy, x_or_y, gamma, beta, mean, stat, dx, dgamma, dbeta, eps, 
 
 
 def dropout_add_ln_fwd(x0, residual, gamma, beta, z, x_out, mu, rsigma, eps, is_rms, stream=None):
-    rows, cols = x0.shape
+    cols = x0.shape[-1]
+    rows = x0.numel() // cols if x0.numel() else 0
     rtype = dtype_code(residual) if residual is not None else dtype_code(x0)
+    lv = _multi_level([x0, residual, z, x_out])
+    if lv is not None:
+        counts, (xs, rs_, zs, xos) = lv
+        check(lib().hk_dropout_add_ln_fwd_strided_rows(dtype_code(x0), rtype, dtype_code(gamma), _ptr(x0), _steps(xs),
+                                                       _ptr(residual), _steps(rs_), _ptr(gamma), _ptr(beta), _ptr(z),
+                                                       _steps(zs), _ptr(x_out), _steps(xos), _ptr(mu), _ptr(rsigma),
+                                                       _arr(counts), _i64(cols), ctypes.c_float(eps),
+                                                       ctypes.c_int(int(is_rms)),
+                                                       stream if stream is not None else current_stream()))
+        return
     check(lib().hk_dropout_add_ln_fwd_pitched(dtype_code(x0), rtype, dtype_code(gamma), _ptr(x0),
                                               _i64(_pitch(x0, cols)), _ptr(residual), _i64(_pitch(residual, cols)),
                                               _ptr(gamma), _ptr(beta), _ptr(z), _i64(_pitch(z, cols)), _ptr(x_out),
@@ -177,10 +264,22 @@ def dropout_add_ln_fwd(x0, residual, gamma, beta, z, x_out, mu, rsigma, eps, is_
 
 def dropout_add_ln_bwd(dz, dx_in, x, mu, rsigma, gamma, dx0, dresidual, dgamma, dbeta, is_rms,
                        workspace=None, stream=None):
-    rows, cols = x.shape
+    cols = x.shape[-1]
+    rows = x.numel() // cols if x.numel() else 0
     if workspace is None:
         workspace = _workspace(norm_bwd_workspace_bytes(dtype_code(dz), rows, cols), dz.device)
     wsb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    lv = _multi_level([dz, dx_in, x, dx0, dresidual])
+    if lv is not None:
+        counts, (dzs, dis, xs, dxs, drs) = lv
+        check(lib().hk_dropout_add_ln_bwd_strided_rows(dtype_code(dz), dtype_code(x), dtype_code(gamma), _ptr(dz),
+                                                       _steps(dzs), _ptr(dx_in), _steps(dis), _ptr(x), _steps(xs),
+                                                       _ptr(mu), _ptr(rsigma), _ptr(gamma), _ptr(dx0), _steps(dxs),
+                                                       _ptr(dresidual), _steps(drs), _ptr(dgamma), _ptr(dbeta),
+                                                       _arr(counts), _i64(cols), ctypes.c_int(int(is_rms)),
+                                                       _ptr(workspace), ctypes.c_size_t(wsb),
+                                                       stream if stream is not None else current_stream()))
+        return workspace
     check(lib().hk_dropout_add_ln_bwd_pitched(dtype_code(dz), dtype_code(x), dtype_code(gamma), _ptr(dz),
                                               _i64(_pitch(dz, cols)), _ptr(dx_in), _i64(_pitch(dx_in, cols)),
                                               _ptr(x), _i64(_pitch(x, cols)), _ptr(mu), _ptr(rsigma), _ptr(gamma),
@@ -431,6 +530,14 @@ def _odi(shape, dim):
 
 
 def softmax_fwd(x, y, dim=-1, stream=None):
+    if dim in (-1, x.dim() - 1):
+        lv = _multi_level([x, y])
+        if lv is not None:
+            counts, (xs, ys) = lv
+            check(lib().hk_softmax_fwd_strided_rows(dtype_code(x), _ptr(x), _steps(xs), _ptr(y), _steps(ys),
+                                                    _arr(counts), _i64(x.shape[-1]),
+                                                    stream if stream is not None else current_stream()))
+            return
     if x.dim() == 2 and dim in (-1, 1) and not (x.is_contiguous() and y.is_contiguous()):
         rows, cols = x.shape
         check(lib().hk_softmax_fwd_pitched(dtype_code(x), _ptr(x), _i64(_pitch(x, cols)), _ptr(y),
@@ -443,6 +550,14 @@ def softmax_fwd(x, y, dim=-1, stream=None):
 
 
 def softmax_bwd(y, dy, dx, dim=-1, stream=None):
+    if dim in (-1, y.dim() - 1):
+        lv = _multi_level([y, dy, dx])
+        if lv is not None:
+            counts, (ys, dys, dxs) = lv
+            check(lib().hk_softmax_bwd_strided_rows(dtype_code(y), _ptr(y), _steps(ys), _ptr(dy), _steps(dys), _ptr(dx),
+                                                    _steps(dxs), _arr(counts), _i64(y.shape[-1]),
+                                                    stream if stream is not None else current_stream()))
+            return
     if y.dim() == 2 and dim in (-1, 1) and not (y.is_contiguous() and dy.is_contiguous() and dx.is_contiguous()):
         rows, cols = y.shape
         check(lib().hk_softmax_bwd_pitched(dtype_code(y), _ptr(y), _i64(_pitch(y, cols)), _ptr(dy),
@@ -457,6 +572,13 @@ def softmax_bwd(y, dy, dx, dim=-1, stream=None):
 def sce_sparse_fwd(logits, labels, loss, ignored_index, stream=None):
     cols = logits.shape[-1]
     rows = logits.numel() // cols if logits.numel() else 0
+    lv = _multi_level([logits])
+    if lv is not None:
+        counts, (xs,) = lv
+        check(lib().hk_sce_sparse_fwd_strided_rows(dtype_code(logits), _ptr(logits), _steps(xs), _ptr(labels),
+                                                   _ptr(loss), _arr(counts), _i64(cols), _i64(ignored_index),
+                                                   stream if stream is not None else current_stream()))
+        return
     check(lib().hk_sce_sparse_fwd_pitched(dtype_code(logits), _ptr(logits), _i64(_pitch(logits, cols)), _ptr(labels),
                                           _ptr(loss), _i64(rows), _i64(cols), _i64(ignored_index),
                                           stream if stream is not None else current_stream()))
@@ -465,6 +587,14 @@ def sce_sparse_fwd(logits, labels, loss, ignored_index, stream=None):
 def sce_sparse_bwd(logits, labels, grad_loss, dlogits, ignored_index, stream=None):
     cols = logits.shape[-1]
     rows = logits.numel() // cols if logits.numel() else 0
+    lv = _multi_level([logits, dlogits])
+    if lv is not None:
+        counts, (xs, ds) = lv
+        check(lib().hk_sce_sparse_bwd_strided_rows(dtype_code(logits), _ptr(logits), _steps(xs), _ptr(labels),
+                                                   _ptr(grad_loss), _ptr(dlogits), _steps(ds), _arr(counts),
+                                                   _i64(cols), _i64(ignored_index),
+                                                   stream if stream is not None else current_stream()))
+        return
     check(lib().hk_sce_sparse_bwd_pitched(dtype_code(logits), _ptr(logits), _i64(_pitch(logits, cols)), _ptr(labels),
                                           _ptr(grad_loss), _ptr(dlogits), _i64(_pitch(dlogits, cols)), _i64(rows),
                                           _i64(cols), _i64(ignored_index),

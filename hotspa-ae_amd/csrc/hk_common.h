@@ -204,6 +204,34 @@ __device__ __forceinline__ u32x4 ld16_stream(const void* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }
 
+// Rows on up to three levels.  The leading dimensions of a row-major operand need not step by one constant
+// pitch: a view with permuted leading dimensions (x.permute(0, 2, 1, 3) of a [B, H, S, D] array) numbers its rows
+// r = (i2 * n1 + i1) * n0 + i0 and row r starts i0 * pitch + i1 * p1 + i2 * p2 elements from the base, the three
+// steps being whatever the view's strides are.  A dense or row-pitched array is the one-level case (n0 = rows).
+// The one-shot row kernels get the decomposition for nothing: they are launched on a three-dimensional grid whose
+// x walks the rows of the innermost level and whose y / z are i1 / i2.
+struct LevelSteps {
+  int64_t p1, p2;   // elements between consecutive i1 / i2; the innermost step is the operand's pitch
+};
+// offset of the two outer levels of this workgroup's rows, in elements
+__device__ __forceinline__ int64_t outer_level_offset(const LevelSteps& l) {
+  return int64_t(blockIdx.y) * l.p1 + int64_t(blockIdx.z) * l.p2;
+}
+// number of the row (i0, blockIdx.y, blockIdx.z) in the dense [rows] arrays next to the operand (statistics,
+// labels, losses)
+__device__ __forceinline__ int64_t dense_row_index(int64_t i0, int64_t n0) {
+  return i0 + n0 * (int64_t(blockIdx.y) + int64_t(gridDim.y) * int64_t(blockIdx.z));
+}
+// (i0, i1, i2) of row r for kernels that walk the rows themselves
+__device__ __forceinline__ int64_t level_row_offset(int64_t r, int64_t n0, int64_t n1, int64_t pitch,
+                                                    const LevelSteps& l) {
+  const uint32_t q = uint32_t(r) / uint32_t(n0);
+  const uint32_t i0 = uint32_t(r) - q * uint32_t(n0);
+  const uint32_t i2 = q / uint32_t(n1);
+  const uint32_t i1 = q - i2 * uint32_t(n1);
+  return int64_t(i0) * pitch + int64_t(i1) * l.p1 + int64_t(i2) * l.p2;
+}
+
 // ---------------------------------------------------------------------------
 // wave64 reductions through DPP (no LDS traffic).  After the call every lane
 // holds the result.

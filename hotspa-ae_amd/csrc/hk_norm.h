@@ -24,6 +24,9 @@ struct NormFwdArgs {
   void* stat;
   int64_t rows;
   int64_t x_pitch, res_pitch, y_pitch, xout_pitch;
+  // rows on several levels (see LevelSteps): n0 * n1 * n2 = rows; one level is n0 = rows, n1 = n2 = 1
+  int64_t n0, n1, n2;
+  LevelSteps x_lv, res_lv, y_lv, xout_lv;
   int cols;
   int nvec;
   float eps;
@@ -49,6 +52,9 @@ struct NormBwdArgs {
   float* part_dbeta;    // [grid, cols]
   int64_t rows;
   int64_t dy_pitch, x_pitch, dx_pitch, dxin_pitch, dres_pitch;
+  // rows on several levels (see LevelSteps); the walking kernel splits the row number itself
+  int64_t n0, n1, n2;
+  LevelSteps dy_lv, x_lv, dx_lv, dxin_lv, dres_lv;
   int cols;
   int nvec;
   int tpr;              // threads per row (multiple of 64)

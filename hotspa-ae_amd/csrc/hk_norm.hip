@@ -12,8 +12,9 @@ static int norm_fwd_dispatch(int dtype, NormFwdArgs& a, hipStream_t s, const cha
   HK_REQUIRE(a.rows <= 0x7fffffffLL && a.cols <= 0x3fffffff, HK_ERR_INVALID,
              "%s: shape [%lld, %d] too large", who, (long long)a.rows, a.cols);
   HK_REQUIRE(a.x && a.y, HK_ERR_INVALID, "%s: null input/output", who);
-  HK_REQUIRE(a.x_pitch >= a.cols && a.y_pitch >= a.cols && (!a.residual || a.res_pitch >= a.cols) &&
-             (!a.x_out || a.xout_pitch >= a.cols), HK_ERR_INVALID,
+  if (a.n0 == 0) { a.n0 = a.rows; a.n1 = a.n2 = 1; }   // one level
+  HK_REQUIRE(a.n0 == 1 || (a.x_pitch >= a.cols && a.y_pitch >= a.cols && (!a.residual || a.res_pitch >= a.cols) &&
+                           (!a.x_out || a.xout_pitch >= a.cols)), HK_ERR_INVALID,
              "%s: a row pitch is smaller than the %d columns of a row", who, a.cols);
   a.inv_cols = 1.0f / float(a.cols);
   switch (dtype) {
@@ -35,8 +36,9 @@ static int norm_bwd_dispatch(int dtype, NormBwdArgs& a, int mode, void* dgamma, 
              "%s: shape [%lld, %d] too large", who, (long long)a.rows, a.cols);
   HK_REQUIRE(a.dy && a.x && a.dx && a.stat, HK_ERR_INVALID, "%s: null input/output", who);
   HK_REQUIRE(mode != BWD_LN || a.mean, HK_ERR_INVALID, "%s: mean is required", who);
-  HK_REQUIRE(a.dy_pitch >= a.cols && a.x_pitch >= a.cols && a.dx_pitch >= a.cols &&
-             (!a.dx_in || a.dxin_pitch >= a.cols) && (!a.dres || a.dres_pitch >= a.cols), HK_ERR_INVALID,
+  if (a.n0 == 0) { a.n0 = a.rows; a.n1 = a.n2 = 1; }   // one level
+  HK_REQUIRE(a.n0 == 1 || (a.dy_pitch >= a.cols && a.x_pitch >= a.cols && a.dx_pitch >= a.cols &&
+                           (!a.dx_in || a.dxin_pitch >= a.cols) && (!a.dres || a.dres_pitch >= a.cols)), HK_ERR_INVALID,
              "%s: a row pitch is smaller than the %d columns of a row", who, a.cols);
   a.inv_cols = 1.0f / float(a.cols);
   switch (dtype) {
@@ -49,6 +51,23 @@ static int norm_bwd_dispatch(int dtype, NormBwdArgs& a, int mode, void* dgamma, 
       return HK_ERR_UNSUPPORTED;
   }
 }
+
+// level_rows = {n0, n1, n2} of a *_strided_rows call: every count positive, the outer two within a grid's y / z
+// range, the product within the row limit.  Writes the total.
+static int check_levels(const int64_t level_rows[3], int64_t* rows, const char* who) {
+  HK_REQUIRE(level_rows, HK_ERR_INVALID, "%s: null level_rows", who);
+  const int64_t n0 = level_rows[0], n1 = level_rows[1], n2 = level_rows[2];
+  HK_REQUIRE(n0 >= 0 && n1 >= 0 && n2 >= 0, HK_ERR_INVALID, "%s: negative level count", who);
+  if (n0 == 0 || n1 == 0 || n2 == 0) { *rows = 0; return HK_OK; }
+  HK_REQUIRE(n1 <= 65535 && n2 <= 65535, HK_ERR_UNSUPPORTED,
+             "%s: the two outer levels hold at most 65535 rows each (got %lld, %lld)", who, (long long)n1, (long long)n2);
+  HK_REQUIRE(n0 <= 0x7fffffffLL && n0 * n1 <= 0x7fffffffLL && n0 * n1 * n2 <= 0x7fffffffLL, HK_ERR_INVALID,
+             "%s: too many rows", who);
+  *rows = n0 * n1 * n2;
+  return HK_OK;
+}
+
+static inline LevelSteps outer_steps(const int64_t steps[3]) { return LevelSteps{steps[1], steps[2]}; }
 
 // Scratch memory owned by the library, for the entry point that must not
 // allocate.  The array lives in the code object's global segment, so every
@@ -85,6 +104,31 @@ using namespace hk;
 
 extern "C" {
 
+
+int hk_layer_norm_fwd_strided_rows(int dtype, const void* x, const int64_t x_steps[3], const void* gamma,
+                                   const void* beta, void* y, const int64_t y_steps[3], void* mean, void* stat,
+                                   int stats_dtype, int stat_kind, const int64_t level_rows[3], int64_t cols,
+                                   float eps, hkStream_t stream) {
+  const char* who = "hk_layer_norm_fwd_strided_rows";
+  HK_REQUIRE(x_steps && y_steps, HK_ERR_INVALID, "%s: null steps", who);
+  int64_t rows = 0;
+  int rc = check_levels(level_rows, &rows, who);
+  if (rc != HK_OK) return rc;
+  HK_REQUIRE(stats_dtype == HK_FLOAT32 || stats_dtype == dtype, HK_ERR_INVALID,
+             "%s: stats dtype %d must be fp32 or the data dtype %d", who, stats_dtype, dtype);
+  HK_REQUIRE(stat_kind == HK_STAT_VAR || stat_kind == HK_STAT_RSTD, HK_ERR_INVALID, "%s: bad stat_kind %d", who,
+             stat_kind);
+  HK_REQUIRE(cols >= 0 && cols <= 0x3fffffff, HK_ERR_INVALID, "%s: bad cols", who);
+  HK_REQUIRE(dtype != HK_FLOAT64 || stats_dtype == HK_FLOAT64, HK_ERR_UNSUPPORTED,
+             "%s: fp64 data needs fp64 statistics", who);
+  NormFwdArgs a{};
+  a.x = x; a.gamma = gamma; a.beta = beta; a.y = y; a.mean = mean; a.stat = stat;
+  a.x_pitch = x_steps[0]; a.y_pitch = y_steps[0]; a.x_lv = outer_steps(x_steps); a.y_lv = outer_steps(y_steps);
+  a.n0 = level_rows[0]; a.n1 = level_rows[1]; a.n2 = level_rows[2];
+  a.rows = rows; a.cols = int(cols); a.eps = eps; a.is_rms = 0; a.stat_kind = stat_kind;
+  a.stats_f32 = (stats_dtype == HK_FLOAT32 && dtype != HK_FLOAT64) ? 1 : 0;
+  return norm_fwd_dispatch(dtype, a, as_hip(stream), who);
+}
 
 int hk_layer_norm_fwd_pitched(int dtype, const void* x, int64_t x_pitch, const void* gamma, const void* beta,
                               void* y, int64_t y_pitch, void* mean, void* stat, int stats_dtype, int stat_kind,
@@ -133,6 +177,36 @@ int hk_norm_bwd_workspace_bytes(int dtype, int64_t rows, int64_t cols, size_t* b
   return HK_OK;
 }
 
+int hk_layer_norm_bwd_strided_rows(int dtype, const void* dy, const int64_t dy_steps[3], const void* x_or_y,
+                                   const int64_t x_steps[3], const void* gamma, const void* beta, const void* mean,
+                                   const void* stat, int stats_dtype, int stat_kind, void* dx,
+                                   const int64_t dx_steps[3], void* dgamma, void* dbeta,
+                                   const int64_t level_rows[3], int64_t cols, float eps, int memory_efficient,
+                                   int clamp_gamma, void* workspace, size_t workspace_bytes, hkStream_t stream) {
+  const char* who = "hk_layer_norm_bwd_strided_rows";
+  HK_REQUIRE(dy_steps && x_steps && dx_steps, HK_ERR_INVALID, "%s: null steps", who);
+  int64_t rows = 0;
+  int rc = check_levels(level_rows, &rows, who);
+  if (rc != HK_OK) return rc;
+  HK_REQUIRE(stats_dtype == HK_FLOAT32 || stats_dtype == dtype, HK_ERR_INVALID,
+             "%s: stats dtype %d must be fp32 or the data dtype %d", who, stats_dtype, dtype);
+  HK_REQUIRE(stat_kind == HK_STAT_VAR || stat_kind == HK_STAT_RSTD, HK_ERR_INVALID, "%s: bad stat_kind %d", who,
+             stat_kind);
+  HK_REQUIRE(cols >= 0 && cols <= 0x3fffffff, HK_ERR_INVALID, "%s: bad cols", who);
+  HK_REQUIRE(dtype != HK_FLOAT64 || stats_dtype == HK_FLOAT64, HK_ERR_UNSUPPORTED,
+             "%s: fp64 data needs fp64 statistics", who);
+  NormBwdArgs a{};
+  a.dy = dy; a.x = x_or_y; a.gamma = gamma; a.beta = beta; a.mean = mean; a.stat = stat;
+  a.dy_pitch = dy_steps[0]; a.x_pitch = x_steps[0]; a.dx_pitch = dx_steps[0];
+  a.dy_lv = outer_steps(dy_steps); a.x_lv = outer_steps(x_steps); a.dx_lv = outer_steps(dx_steps);
+  a.n0 = level_rows[0]; a.n1 = level_rows[1]; a.n2 = level_rows[2];
+  a.dx = dx; a.rows = rows; a.cols = int(cols); a.eps = eps; a.stat_kind = stat_kind;
+  a.stats_f32 = (stats_dtype == HK_FLOAT32 && dtype != HK_FLOAT64) ? 1 : 0;
+  a.clamp_gamma = clamp_gamma;
+  return norm_bwd_dispatch(dtype, a, memory_efficient ? BWD_LN_MEMEFF : BWD_LN, dgamma, dbeta, workspace,
+                           workspace_bytes, as_hip(stream), who);
+}
+
 int hk_layer_norm_bwd_pitched(int dtype, const void* dy, int64_t dy_pitch, const void* x_or_y, int64_t x_pitch,
                               const void* gamma, const void* beta, const void* mean, const void* stat,
                               int stats_dtype, int stat_kind, void* dx, int64_t dx_pitch, void* dgamma,
@@ -165,6 +239,74 @@ int hk_layer_norm_bwd(int dtype, const void* dy, const void* x_or_y, const void*
   return hk_layer_norm_bwd_pitched(dtype, dy, cols, x_or_y, cols, gamma, beta, mean, stat, stats_dtype, stat_kind,
                                    dx, cols, dgamma, dbeta, rows, cols, eps, memory_efficient, clamp_gamma,
                                    workspace, workspace_bytes, stream);
+}
+
+static const int64_t kNoSteps[3] = {0, 0, 0};
+
+int hk_dropout_add_ln_fwd_strided_rows(int itype, int rtype, int wtype, const void* x0, const int64_t x0_steps[3],
+                                       const void* residual, const int64_t residual_steps[3], const void* gamma,
+                                       const void* beta, void* z, const int64_t z_steps[3], void* x_out,
+                                       const int64_t x_out_steps[3], void* mu, void* rsigma,
+                                       const int64_t level_rows[3], int64_t cols, float eps, int is_rms_norm,
+                                       hkStream_t stream) {
+  const char* who = "hk_dropout_add_ln_fwd_strided_rows";
+  HK_REQUIRE(x0_steps && z_steps && (!residual || residual_steps) && (!x_out || x_out_steps), HK_ERR_INVALID,
+             "%s: null steps", who);
+  if (!residual_steps) residual_steps = kNoSteps;
+  if (!x_out_steps) x_out_steps = kNoSteps;
+  int64_t rows = 0;
+  int rc = check_levels(level_rows, &rows, who);
+  if (rc != HK_OK) return rc;
+  HK_REQUIRE(itype == rtype && itype == wtype, HK_ERR_UNSUPPORTED,
+             "%s: mixed dtypes (input %d, residual %d, weight %d) are not implemented", who, itype, rtype, wtype);
+  HK_REQUIRE(itype == HK_FLOAT32 || itype == HK_BFLOAT16 || itype == HK_FLOAT16, HK_ERR_UNSUPPORTED,
+             "%s: not implemented for dtype %d", who, itype);
+  HK_REQUIRE(gamma != nullptr, HK_ERR_INVALID, "%s: gamma is required", who);
+  HK_REQUIRE(eps >= 0.f, HK_ERR_INVALID, "%s: epsilon must be >= 0", who);
+  HK_REQUIRE(cols >= 0 && cols <= 0x3fffffff, HK_ERR_INVALID, "%s: bad cols", who);
+  NormFwdArgs a{};
+  a.x = x0; a.residual = residual; a.gamma = gamma; a.beta = beta; a.y = z; a.x_out = x_out;
+  a.x_pitch = x0_steps[0]; a.res_pitch = residual_steps[0]; a.y_pitch = z_steps[0]; a.xout_pitch = x_out_steps[0];
+  a.x_lv = outer_steps(x0_steps); a.res_lv = outer_steps(residual_steps); a.y_lv = outer_steps(z_steps);
+  a.xout_lv = outer_steps(x_out_steps);
+  a.n0 = level_rows[0]; a.n1 = level_rows[1]; a.n2 = level_rows[2];
+  a.mean = mu; a.stat = rsigma; a.rows = rows; a.cols = int(cols); a.eps = eps;
+  a.is_rms = is_rms_norm ? 1 : 0; a.stat_kind = HK_STAT_RSTD; a.stats_f32 = 1;
+  return norm_fwd_dispatch(itype, a, as_hip(stream), who);
+}
+
+int hk_dropout_add_ln_bwd_strided_rows(int itype, int rtype, int wtype, const void* dz, const int64_t dz_steps[3],
+                                       const void* dx_in, const int64_t dx_in_steps[3], const void* x,
+                                       const int64_t x_steps[3], const void* mu, const void* rsigma,
+                                       const void* gamma, void* dx0, const int64_t dx0_steps[3], void* dresidual,
+                                       const int64_t dresidual_steps[3], void* dgamma, void* dbeta,
+                                       const int64_t level_rows[3], int64_t cols, int is_rms_norm, void* workspace,
+                                       size_t workspace_bytes, hkStream_t stream) {
+  const char* who = "hk_dropout_add_ln_bwd_strided_rows";
+  HK_REQUIRE(dz_steps && x_steps && dx0_steps && (!dx_in || dx_in_steps) && (!dresidual || dresidual_steps),
+             HK_ERR_INVALID, "%s: null steps", who);
+  if (!dx_in_steps) dx_in_steps = kNoSteps;
+  if (!dresidual_steps) dresidual_steps = kNoSteps;
+  int64_t rows = 0;
+  int rc = check_levels(level_rows, &rows, who);
+  if (rc != HK_OK) return rc;
+  HK_REQUIRE(itype == rtype && itype == wtype, HK_ERR_UNSUPPORTED,
+             "%s: mixed dtypes (input %d, residual %d, weight %d) are not implemented", who, itype, rtype, wtype);
+  HK_REQUIRE(itype == HK_FLOAT32 || itype == HK_BFLOAT16 || itype == HK_FLOAT16, HK_ERR_UNSUPPORTED,
+             "%s: not implemented for dtype %d", who, itype);
+  HK_REQUIRE(gamma != nullptr, HK_ERR_INVALID, "%s: gamma is required", who);
+  HK_REQUIRE(cols >= 0 && cols <= 0x3fffffff, HK_ERR_INVALID, "%s: bad cols", who);
+  NormBwdArgs a{};
+  a.dy = dz; a.x = x; a.gamma = gamma; a.mean = mu; a.stat = rsigma; a.dx_in = dx_in;
+  a.dy_pitch = dz_steps[0]; a.x_pitch = x_steps[0]; a.dx_pitch = dx0_steps[0]; a.dxin_pitch = dx_in_steps[0];
+  a.dres_pitch = dresidual_steps[0];
+  a.dy_lv = outer_steps(dz_steps); a.x_lv = outer_steps(x_steps); a.dx_lv = outer_steps(dx0_steps);
+  a.dxin_lv = outer_steps(dx_in_steps); a.dres_lv = outer_steps(dresidual_steps);
+  a.n0 = level_rows[0]; a.n1 = level_rows[1]; a.n2 = level_rows[2];
+  a.dx = dx0; a.dres = dresidual; a.rows = rows; a.cols = int(cols); a.eps = 0.f;
+  a.stat_kind = HK_STAT_RSTD; a.stats_f32 = 1; a.clamp_gamma = 0;
+  return norm_bwd_dispatch(itype, a, is_rms_norm ? BWD_RMS : BWD_LN, dgamma, dbeta, workspace, workspace_bytes,
+                           as_hip(stream), who);
 }
 
 int hk_dropout_add_ln_fwd_pitched(int itype, int rtype, int wtype, const void* x0, int64_t x0_pitch,

@@ -111,8 +111,15 @@ void norm_bwd_kernel(NormBwdArgs a) {
     const int64_t rc = r < last_row ? r : last_row;
     if constexpr (MODE == BWD_LN) nmu[d] = meanp[rc];
     nsv[d] = statp[rc];
-    const T* xr = static_cast<const T*>(a.x) + rc * a.x_pitch;
-    const T* dyr = static_cast<const T*>(a.dy) + rc * a.dy_pitch;
+    int64_t xo = rc * a.x_pitch, dyo = rc * a.dy_pitch;
+    if constexpr (EXTRA) {
+      if (a.n0 != a.rows) {   // rows on several levels: uniform
+        xo = level_row_offset(rc, a.n0, a.n1, a.x_pitch, a.x_lv);
+        dyo = level_row_offset(rc, a.n0, a.n1, a.dy_pitch, a.dy_lv);
+      }
+    }
+    const T* xr = static_cast<const T*>(a.x) + xo;
+    const T* dyr = static_cast<const T*>(a.dy) + dyo;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       nx[d][i] = ld16(xr + vidx[i] * VEC);
@@ -202,8 +209,16 @@ void norm_bwd_kernel(NormBwdArgs a) {
       [[maybe_unused]] T* drr = nullptr;
       [[maybe_unused]] const T* dir = nullptr;
       if constexpr (EXTRA) {
-        drr = a.dres ? static_cast<T*>(a.dres) + row * a.dres_pitch : nullptr;
-        dir = a.dx_in ? static_cast<const T*>(a.dx_in) + row * a.dxin_pitch : nullptr;
+        const bool levels = a.n0 != a.rows;   // uniform
+        if (levels) dxr = static_cast<T*>(a.dx) + level_row_offset(row, a.n0, a.n1, a.dx_pitch, a.dx_lv);
+        if (a.dres) {
+          drr = static_cast<T*>(a.dres) +
+                (levels ? level_row_offset(row, a.n0, a.n1, a.dres_pitch, a.dres_lv) : row * a.dres_pitch);
+        }
+        if (a.dx_in) {
+          dir = static_cast<const T*>(a.dx_in) +
+                (levels ? level_row_offset(row, a.n0, a.n1, a.dxin_pitch, a.dxin_lv) : row * a.dxin_pitch);
+        }
       }
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
@@ -337,9 +352,10 @@ template <typename T, typename CT>
 __global__ __launch_bounds__(256)
 void norm_bwd_generic_dx_kernel(NormBwdArgs a, int mode) {
   __shared__ CT lds[256];
-  const int64_t row = blockIdx.x;
-  const T* xr = static_cast<const T*>(a.x) + row * a.x_pitch;
-  const T* dyr = static_cast<const T*>(a.dy) + row * a.dy_pitch;
+  const int64_t i0 = blockIdx.x;                       // row within the innermost level
+  const int64_t row = dense_row_index(i0, a.n0);
+  const T* xr = static_cast<const T*>(a.x) + i0 * a.x_pitch + outer_level_offset(a.x_lv);
+  const T* dyr = static_cast<const T*>(a.dy) + i0 * a.dy_pitch + outer_level_offset(a.dy_lv);
   const T* gp = static_cast<const T*>(a.gamma);
   const T* bp = static_cast<const T*>(a.beta);
   CT mu = 0;
@@ -379,9 +395,9 @@ void norm_bwd_generic_dx_kernel(NormBwdArgs a, int mode) {
   s2 = block_sum_generic<CT>(s2, lds);
   const CT inv = CT(1) / CT(a.cols);
   const CT c1 = s1 * inv, c2 = s2 * inv;
-  T* dxr = static_cast<T*>(a.dx) + row * a.dx_pitch;
-  T* drr = a.dres ? static_cast<T*>(a.dres) + row * a.dres_pitch : nullptr;
-  const T* dir = a.dx_in ? static_cast<const T*>(a.dx_in) + row * a.dxin_pitch : nullptr;
+  T* dxr = static_cast<T*>(a.dx) + i0 * a.dx_pitch + outer_level_offset(a.dx_lv);
+  T* drr = a.dres ? static_cast<T*>(a.dres) + i0 * a.dres_pitch + outer_level_offset(a.dres_lv) : nullptr;
+  const T* dir = a.dx_in ? static_cast<const T*>(a.dx_in) + i0 * a.dxin_pitch + outer_level_offset(a.dxin_lv) : nullptr;
   for (int c = threadIdx.x; c < a.cols; c += blockDim.x) {
     const CT g = gp ? GenericIO<T, CT>::ld(gp + c) : CT(1);
     const CT d = GenericIO<T, CT>::ld(dyr + c);
@@ -411,9 +427,12 @@ void norm_bwd_generic_cols_kernel(NormBwdArgs a, int mode, T* dgamma, T* dbeta) 
       if (g >= CT(0)) kg = g < e ? e : g; else kg = g > -e ? -e : g;
     }
     const CT b = (bp && mode == BWD_LN_MEMEFF) ? GenericIO<T, CT>::ld(bp + c) : CT(0);
+    const bool levels = a.n0 != a.rows;
     for (int64_t r = w; r < a.rows; r += 4) {
-      const CT d = GenericIO<T, CT>::ld(static_cast<const T*>(a.dy) + r * a.dy_pitch + c);
-      const CT xv = GenericIO<T, CT>::ld(static_cast<const T*>(a.x) + r * a.x_pitch + c);
+      const int64_t dyo = levels ? level_row_offset(r, a.n0, a.n1, a.dy_pitch, a.dy_lv) : r * a.dy_pitch;
+      const int64_t xo = levels ? level_row_offset(r, a.n0, a.n1, a.x_pitch, a.x_lv) : r * a.x_pitch;
+      const CT d = GenericIO<T, CT>::ld(static_cast<const T*>(a.dy) + dyo + c);
+      const CT xv = GenericIO<T, CT>::ld(static_cast<const T*>(a.x) + xo + c);
       CT xhat;
       if (mode == BWD_LN_MEMEFF) {
         xhat = (xv - b) / kg;
@@ -503,7 +522,8 @@ static int launch_norm_bwd_inst(const NormBwdArgs& a, const BwdPlan& p, int pf, 
   // the kernel's "extra" instance takes the optional operands behind uniform branches, and the clamp request in
   // the modes that have no instance of their own for it
   const bool want_clamp = a.clamp_gamma != 0 && MODE != BWD_LN_MEMEFF;   // the memory-efficient mode always clamps
-  const bool extra = a.dx_in != nullptr || a.dres != nullptr || (want_clamp && MODE != BWD_LN);
+  // rows on several levels go with them: that instance splits the row number itself
+  const bool extra = a.dx_in != nullptr || a.dres != nullptr || (want_clamp && MODE != BWD_LN) || a.n0 != a.rows;
   // one group that is the whole block, of exactly the bound's size: the instance with a constant group width
   const bool fixed = p.rpb == 1 && p.block == MAXT;
   // the deep ring exists for the plain case only: full rows, no optional operands
@@ -573,14 +593,15 @@ template <typename T>
 int norm_bwd_typed(NormBwdArgs a, int mode, void* dgamma, void* dbeta, void* ws, size_t ws_bytes,
                    hipStream_t s) {
   constexpr int VEC = VecIO<T>::N;
-  auto pitch_ok = [](int64_t p) { return p % VEC == 0; };
+  auto steps_ok = [](int64_t pitch, const LevelSteps& l) { return pitch % VEC == 0 && l.p1 % VEC == 0 && l.p2 % VEC == 0; };
   const bool aligned = aligned16(a.dy) && aligned16(a.x) && aligned16(a.dx) && aligned16(a.gamma) &&
                        aligned16(a.beta) && aligned16(a.dx_in) && aligned16(a.dres) &&
-                       pitch_ok(a.dy_pitch) && pitch_ok(a.x_pitch) && pitch_ok(a.dx_pitch) &&
-                       (!a.dx_in || pitch_ok(a.dxin_pitch)) && (!a.dres || pitch_ok(a.dres_pitch));
+                       steps_ok(a.dy_pitch, a.dy_lv) && steps_ok(a.x_pitch, a.x_lv) && steps_ok(a.dx_pitch, a.dx_lv) &&
+                       (!a.dx_in || steps_ok(a.dxin_pitch, a.dxin_lv)) && (!a.dres || steps_ok(a.dres_pitch, a.dres_lv));
   BwdPlan p = plan_norm_bwd<T>(a.rows, a.cols, aligned);
   if (!p.reg_path) {
-    HK_LAUNCH((norm_bwd_generic_dx_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s, a, mode);
+    HK_LAUNCH((norm_bwd_generic_dx_kernel<T, float>), dim3(unsigned(a.n0), unsigned(a.n1), unsigned(a.n2)), dim3(256),
+              0, s, a, mode);
     int rc = launch_check("norm_bwd_generic_dx_kernel");
     if (rc != HK_OK) return rc;
     if (dgamma || dbeta) {

@@ -42,7 +42,8 @@ void norm_fwd_kernel(NormFwdArgs a) {
   const int64_t row0 = WAVE_ROW
       ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index()
       : int64_t(blockIdx.x) * R;
-  if (WAVE_ROW && row0 >= a.rows) return;  // wave-uniform; no block barrier in this mode
+  // row0 counts within the innermost level of rows; blockIdx.y / z are the outer levels (one level: both 0)
+  if (WAVE_ROW && row0 >= a.n0) return;  // wave-uniform; no block barrier in this mode
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
   auto off = [&](int i) { return uint32_t(i * tpr + t) * 16u; };   // vector i of thread t, in bytes from the row's start
   // long rows: stops the scheduler from unpacking every vector of a pass before the first one is consumed
@@ -54,7 +55,7 @@ void norm_fwd_kernel(NormFwdArgs a) {
   bool live[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    live[r] = r == 0 || row0 + r < a.rows;
+    live[r] = r == 0 || row0 + r < a.n0;
     rowi[r] = live[r] ? row0 + r : row0;
     bytes[r] = live[r] ? uint32_t(a.nvec) * 16u : 0u;
   }
@@ -64,7 +65,8 @@ void norm_fwd_kernel(NormFwdArgs a) {
     u32x4 raw[R][NV];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const BufferRsrc xr = make_rsrc(static_cast<const T*>(a.x) + rowi[r] * a.x_pitch, bytes[r]);
+      const BufferRsrc xr = make_rsrc(static_cast<const T*>(a.x) + rowi[r] * a.x_pitch + outer_level_offset(a.x_lv),
+                                      bytes[r]);
 #pragma unroll
       for (int i = 0; i < NV; ++i) raw[r][i] = buf_ld16<kBufStream>(xr, off(i));
     }
@@ -72,14 +74,16 @@ void norm_fwd_kernel(NormFwdArgs a) {
       u32x4 res[R][NV];
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const BufferRsrc rr = make_rsrc(static_cast<const T*>(a.residual) + rowi[r] * a.res_pitch, bytes[r]);
+        const BufferRsrc rr = make_rsrc(static_cast<const T*>(a.residual) + rowi[r] * a.res_pitch +
+                                        outer_level_offset(a.res_lv), bytes[r]);
 #pragma unroll
         for (int i = 0; i < NV; ++i) res[r][i] = buf_ld16<kBufStream>(rr, off(i));
       }
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         // an absent x_out becomes an empty buffer: its stores are dropped by the bounds check
-        const BufferRsrc xo = make_rsrc(a.x_out ? static_cast<T*>(a.x_out) + rowi[r] * a.xout_pitch
+        const BufferRsrc xo = make_rsrc(a.x_out ? static_cast<T*>(a.x_out) + rowi[r] * a.xout_pitch +
+                                                      outer_level_offset(a.xout_lv)
                                                 : static_cast<T*>(a.y), a.x_out ? bytes[r] : 0u);
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
@@ -185,15 +189,17 @@ void norm_fwd_kernel(NormFwdArgs a) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       if (live[r]) {
-        store_stat<T>(a.mean, rowi[r], mu[r], a.stats_f32);
-        store_stat<T>(a.stat, rowi[r], a.stat_kind == HK_STAT_VAR ? var[r] : rs[r], a.stats_f32);
+        const int64_t dense = dense_row_index(rowi[r], a.n0);
+        store_stat<T>(a.mean, dense, mu[r], a.stats_f32);
+        store_stat<T>(a.stat, dense, a.stat_kind == HK_STAT_VAR ? var[r] : rs[r], a.stats_f32);
       }
     }
   }
 
   BufferRsrc yr[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) yr[r] = make_rsrc(static_cast<T*>(a.y) + rowi[r] * a.y_pitch, bytes[r]);
+  for (int r = 0; r < R; ++r)
+    yr[r] = make_rsrc(static_cast<T*>(a.y) + rowi[r] * a.y_pitch + outer_level_offset(a.y_lv), bytes[r]);
   const uint32_t row_bytes = uint32_t(a.nvec) * 16u;
   // gamma / beta are fetched after the reduction: every fetch holds one of the compute unit's outstanding-request
   // slots until the data is back; issued before the row has arrived they would hold those slots for the whole HBM
@@ -236,10 +242,12 @@ template <typename T, typename CT>
 __global__ __launch_bounds__(256)
 void norm_fwd_generic_kernel(NormFwdArgs a) {
   __shared__ CT lds[256];
-  const int64_t row = blockIdx.x;
-  const T* xr = static_cast<const T*>(a.x) + row * a.x_pitch;
-  const T* rr = a.residual ? static_cast<const T*>(a.residual) + row * a.res_pitch : nullptr;
-  T* xo = a.x_out ? static_cast<T*>(a.x_out) + row * a.xout_pitch : nullptr;
+  const int64_t i0 = blockIdx.x;                       // row within the innermost level
+  const int64_t row = dense_row_index(i0, a.n0);
+  const T* xr = static_cast<const T*>(a.x) + i0 * a.x_pitch + outer_level_offset(a.x_lv);
+  const T* rr = a.residual ? static_cast<const T*>(a.residual) + i0 * a.res_pitch + outer_level_offset(a.res_lv)
+                           : nullptr;
+  T* xo = a.x_out ? static_cast<T*>(a.x_out) + i0 * a.xout_pitch + outer_level_offset(a.xout_lv) : nullptr;
   auto ldx = [&](int c) -> CT {
     CT v = GenericIO<T, CT>::ld(xr + c);
     if (rr) v += GenericIO<T, CT>::ld(rr + c);
@@ -284,7 +292,7 @@ void norm_fwd_generic_kernel(NormFwdArgs a) {
     }
   }
   const CT shift = a.is_rms ? CT(0) : mu;
-  T* yr = static_cast<T*>(a.y) + row * a.y_pitch;
+  T* yr = static_cast<T*>(a.y) + i0 * a.y_pitch + outer_level_offset(a.y_lv);
   const T* gp = static_cast<const T*>(a.gamma);
   const T* bp = static_cast<const T*>(a.beta);
   for (int c = threadIdx.x; c < a.cols; c += blockDim.x) {
@@ -416,10 +424,13 @@ template <typename T>
 int norm_fwd_typed(NormFwdArgs a, hipStream_t s) {
   constexpr int VEC = VecIO<T>::N;
   auto pitch_ok = [](int64_t p) { return p % VEC == 0; };
+  auto steps_ok = [](int64_t pitch, const LevelSteps& l) { return pitch % VEC == 0 && l.p1 % VEC == 0 && l.p2 % VEC == 0; };
+  (void)pitch_ok;
   const bool vec_ok = (a.cols % VEC == 0) && aligned16(a.x) && aligned16(a.y) &&
                       aligned16(a.gamma) && aligned16(a.beta) && aligned16(a.residual) &&
-                      aligned16(a.x_out) && pitch_ok(a.x_pitch) && pitch_ok(a.y_pitch) &&
-                      (!a.residual || pitch_ok(a.res_pitch)) && (!a.x_out || pitch_ok(a.xout_pitch));
+                      aligned16(a.x_out) && steps_ok(a.x_pitch, a.x_lv) && steps_ok(a.y_pitch, a.y_lv) &&
+                      (!a.residual || steps_ok(a.res_pitch, a.res_lv)) &&
+                      (!a.x_out || steps_ok(a.xout_pitch, a.xout_lv));
   int threads = 0, nv = 0;
   a.nvec = a.cols / VEC;
   const bool has_res = a.residual != nullptr;
@@ -433,7 +444,7 @@ int norm_fwd_typed(NormFwdArgs a, hipStream_t s) {
   if (vec_ok &&
       pick_row_shape(a.nvec, tune_get(TUNE_NORM_FWD_THREADS), max_nv, wave_nv, many_rows, &threads, &nv)) {
     if (threads == 64) {
-      dim3 grid(unsigned((a.rows + 3) / 4)), block(256);
+      dim3 grid(unsigned((a.n0 + 3) / 4), unsigned(a.n1), unsigned(a.n2)), block(256);
       return has_res ? launch_norm_fwd_nv<T, true, true>(a, nv, 1, grid, block, s)
                      : launch_norm_fwd_nv<T, true, false>(a, nv, 1, grid, block, s);
     }
@@ -444,11 +455,12 @@ int norm_fwd_typed(NormFwdArgs a, hipStream_t s) {
       const int most = max_rows_per_block<T>(nv, has_res);
       rpb = std::min(many_rows ? 2 : 1, most);
     }
-    dim3 grid{unsigned((a.rows + rpb - 1) / rpb)}, block{unsigned(threads)};
+    dim3 grid{unsigned((a.n0 + rpb - 1) / rpb), unsigned(a.n1), unsigned(a.n2)}, block{unsigned(threads)};
     return has_res ? launch_norm_fwd_nv<T, false, true>(a, nv, rpb, grid, block, s)
                    : launch_norm_fwd_nv<T, false, false>(a, nv, rpb, grid, block, s);
   }
-  HK_LAUNCH((norm_fwd_generic_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
+  HK_LAUNCH((norm_fwd_generic_kernel<T, float>), dim3(unsigned(a.n0), unsigned(a.n1), unsigned(a.n2)), dim3(256), 0,
+            s, a);
   return launch_check("norm_fwd_generic_kernel");
 }
 

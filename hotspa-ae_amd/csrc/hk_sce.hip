@@ -26,6 +26,10 @@ struct SceArgs {
   int64_t rows;
   // elements between the starts of consecutive rows of logits / dense labels / dlogits (0 = dense: cols)
   int64_t x_pitch, lab_pitch, out_pitch;
+  // rows on several levels (see LevelSteps); one level: n0 = rows.  labels, losses, per-row gradients and
+  // statistics are dense [rows] arrays and take the row's number
+  int64_t n0, n1, n2;
+  LevelSteps x_lv, lab_lv, out_lv;
   int cols;
   int nvec;
   int64_t ignored_index;
@@ -50,11 +54,13 @@ __device__ __forceinline__ CT sce_row_grad(const SceArgs& a, int64_t row) {
   return CT(Cvt<T>::load(&rounded));
 }
 
+// i0: the row's place within the innermost level (blockIdx.y / z are the outer levels); row: its number
 template <bool WAVE_ROW>
-__device__ __forceinline__ void row_coords(int& tpr, int& t, int64_t& row, int& nwaves) {
+__device__ __forceinline__ void row_coords(const SceArgs& a, int& tpr, int& t, int64_t& i0, int64_t& row, int& nwaves) {
   tpr = WAVE_ROW ? kWave : int(blockDim.x);
   t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
-  row = WAVE_ROW ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index() : int64_t(blockIdx.x);
+  i0 = WAVE_ROW ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index() : int64_t(blockIdx.x);
+  row = dense_row_index(i0, a.n0);
   nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
 }
 
@@ -65,9 +71,9 @@ void sce_sparse_fwd_kernel(SceArgs a) {
   constexpr int VEC = VecIO<T>::N;
   __shared__ float red[kMaxWaves * 3];
   int tpr, t, nwaves;
-  int64_t row;
-  row_coords<WAVE_ROW>(tpr, t, row, nwaves);
-  if (WAVE_ROW && row >= a.rows) return;
+  int64_t i0, row;
+  row_coords<WAVE_ROW>(a, tpr, t, i0, row, nwaves);
+  if (WAVE_ROW && i0 >= a.n0) return;
 
   T* loss = static_cast<T*>(a.out);
   const int64_t label = a.labels[row];
@@ -83,7 +89,7 @@ void sce_sparse_fwd_kernel(SceArgs a) {
     }
     return;
   }
-  const T* xr = static_cast<const T*>(a.logits) + row * a.x_pitch;
+  const T* xr = static_cast<const T*>(a.logits) + i0 * a.x_pitch + outer_level_offset(a.x_lv);
   // slots past the row's end hold -inf: they change neither the maximum nor the sum
   float f[NV * VEC];
   {
@@ -153,11 +159,11 @@ void sce_sparse_bwd_kernel(SceArgs a) {
   constexpr int VEC = VecIO<T>::N;
   __shared__ float red[kMaxWaves * 2];
   int tpr, t, nwaves;
-  int64_t row;
-  row_coords<WAVE_ROW>(tpr, t, row, nwaves);
-  if (WAVE_ROW && row >= a.rows) return;
+  int64_t i0, row;
+  row_coords<WAVE_ROW>(a, tpr, t, i0, row, nwaves);
+  if (WAVE_ROW && i0 >= a.n0) return;
 
-  T* dxr = static_cast<T*>(a.out) + row * a.out_pitch;
+  T* dxr = static_cast<T*>(a.out) + i0 * a.out_pitch + outer_level_offset(a.out_lv);
   const int64_t label = a.labels[row];
   if (label == a.ignored_index) {
     const u32x4 z = {0, 0, 0, 0};
@@ -170,7 +176,7 @@ void sce_sparse_bwd_kernel(SceArgs a) {
     }
     return;
   }
-  const T* xr = static_cast<const T*>(a.logits) + row * a.x_pitch;
+  const T* xr = static_cast<const T*>(a.logits) + i0 * a.x_pitch + outer_level_offset(a.x_lv);
   // slots past the row's end hold -inf: they change neither the maximum nor the sum
   u32x4 raw[NV];
 #pragma unroll
@@ -230,12 +236,12 @@ void sce_dense_kernel(SceArgs a) {
   __shared__ float red[kMaxWaves * 3];
   __shared__ float red2[kMaxWaves * 2];
   int tpr, t, nwaves;
-  int64_t row;
-  row_coords<WAVE_ROW>(tpr, t, row, nwaves);
-  if (WAVE_ROW && row >= a.rows) return;
+  int64_t i0, row;
+  row_coords<WAVE_ROW>(a, tpr, t, i0, row, nwaves);
+  if (WAVE_ROW && i0 >= a.n0) return;
 
-  const T* xr = static_cast<const T*>(a.logits) + row * a.x_pitch;
-  const T* lr = static_cast<const T*>(a.dlabels) + row * a.lab_pitch;
+  const T* xr = static_cast<const T*>(a.logits) + i0 * a.x_pitch + outer_level_offset(a.x_lv);
+  const T* lr = static_cast<const T*>(a.dlabels) + i0 * a.lab_pitch + outer_level_offset(a.lab_lv);
   u32x4 rx[NV], rl[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -286,7 +292,7 @@ void sce_dense_kernel(SceArgs a) {
     const float g = sce_row_grad<T, float>(a, row);
     const float ML = (p.v[0] == kNegInf) ? 0.f : p.v[0];
     const float inv = 1.0f / p.v[1];
-    T* dxr = static_cast<T*>(a.out) + row * a.out_pitch;
+    T* dxr = static_cast<T*>(a.out) + i0 * a.out_pitch + outer_level_offset(a.out_lv);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = i * tpr + t;
@@ -338,9 +344,10 @@ template <typename T, typename CT, int MODE>
 __global__ __launch_bounds__(256)
 void sce_generic_kernel(SceArgs a) {
   __shared__ CT lds[256];
-  const int64_t row = blockIdx.x;
+  const int64_t i0 = blockIdx.x;
+  const int64_t row = dense_row_index(i0, a.n0);
   const int64_t cols = a.cols;
-  const T* xr = static_cast<const T*>(a.logits) + row * a.x_pitch;
+  const T* xr = static_cast<const T*>(a.logits) + i0 * a.x_pitch + outer_level_offset(a.x_lv);
   int64_t label = 0;
   if (MODE < 2) {
     label = a.labels[row];
@@ -356,7 +363,7 @@ void sce_generic_kernel(SceArgs a) {
           }
         }
       } else {
-        T* dxr = static_cast<T*>(a.out) + row * a.out_pitch;
+        T* dxr = static_cast<T*>(a.out) + i0 * a.out_pitch + outer_level_offset(a.out_lv);
         for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) SceIO<T, CT>::st(dxr + c, CT(0));
       }
       return;
@@ -386,7 +393,7 @@ void sce_generic_kernel(SceArgs a) {
       SceIO<T, CT>::st(static_cast<T*>(a.out) + row, r);
     }
   } else if (MODE == 2) {
-    const T* lr = static_cast<const T*>(a.dlabels) + row * a.lab_pitch;
+    const T* lr = static_cast<const T*>(a.dlabels) + i0 * a.lab_pitch + outer_level_offset(a.lab_lv);
     CT sl = 0, slx = 0;
     for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
       const CT l = SceIO<T, CT>::ld(lr + c);
@@ -400,8 +407,8 @@ void sce_generic_kernel(SceArgs a) {
   } else {
     const CT g = sce_row_grad<T, CT>(a, row);
     const CT inv = CT(1) / s;
-    T* dxr = static_cast<T*>(a.out) + row * a.out_pitch;
-    const T* lr = MODE == 3 ? static_cast<const T*>(a.dlabels) + row * a.lab_pitch : nullptr;
+    T* dxr = static_cast<T*>(a.out) + i0 * a.out_pitch + outer_level_offset(a.out_lv);
+    const T* lr = MODE == 3 ? static_cast<const T*>(a.dlabels) + i0 * a.lab_pitch + outer_level_offset(a.lab_lv) : nullptr;
     for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
       CT pr = sce_exp<CT>(SceIO<T, CT>::ld(xr + c) - m) * inv;
       if (MODE == 1) pr = (c == label) ? (pr * g - g) : pr * g;
@@ -474,9 +481,10 @@ static int launch_sce_nv(const SceArgs& a, int nv, dim3 grid, dim3 block, hipStr
 template <typename T, int MODE>
 static int sce_typed(SceArgs a, hipStream_t s) {
   constexpr int VEC = VecIO<T>::N;
+  auto steps_ok = [](int64_t pitch, const LevelSteps& l) { return pitch % VEC == 0 && l.p1 % VEC == 0 && l.p2 % VEC == 0; };
   const bool vec_ok = a.cols % VEC == 0 && aligned16(a.logits) && aligned16(a.dlabels) &&
-                      (MODE == 0 || MODE == 2 || (aligned16(a.out) && a.out_pitch % VEC == 0)) &&
-                      a.x_pitch % VEC == 0 && (MODE < 2 || a.lab_pitch % VEC == 0);
+                      (MODE == 0 || MODE == 2 || (aligned16(a.out) && steps_ok(a.out_pitch, a.out_lv))) &&
+                      steps_ok(a.x_pitch, a.x_lv) && (MODE < 2 || steps_ok(a.lab_pitch, a.lab_lv));
   a.nvec = a.cols / VEC;
   // sparse forward only keeps the packed row; the others keep 32 floats or two rows
   const int max_nv = (MODE == 0) ? 8 : 32 / VEC;
@@ -484,13 +492,14 @@ static int sce_typed(SceArgs a, hipStream_t s) {
   int threads = 0, nv = 0;
   if (vec_ok && pick_sce_shape(a.nvec, max_nv_wave, max_nv, &threads, &nv)) {
     if (threads == 64) {
-      dim3 grid(unsigned((a.rows + 3) / 4)), block(256);
+      dim3 grid(unsigned((a.n0 + 3) / 4), unsigned(a.n1), unsigned(a.n2)), block(256);
       return launch_sce_nv<T, MODE, true>(a, nv, grid, block, s);
     }
-    dim3 grid{unsigned(a.rows)}, block{unsigned(threads)};
+    dim3 grid{unsigned(a.n0), unsigned(a.n1), unsigned(a.n2)}, block{unsigned(threads)};
     return launch_sce_nv<T, MODE, false>(a, nv, grid, block, s);
   }
-  HK_LAUNCH((sce_generic_kernel<T, float, MODE>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
+  HK_LAUNCH((sce_generic_kernel<T, float, MODE>), dim3(unsigned(a.n0), unsigned(a.n1), unsigned(a.n2)), dim3(256), 0,
+            s, a);
   return launch_check("sce_generic_kernel");
 }
 
@@ -507,14 +516,16 @@ static int sce_dispatch(int dtype, SceArgs& a, hipStream_t s, const char* who) {
   if (a.x_pitch == 0) a.x_pitch = a.cols;
   if (a.lab_pitch == 0) a.lab_pitch = a.cols;
   if (a.out_pitch == 0) a.out_pitch = a.cols;
-  HK_REQUIRE(a.x_pitch >= a.cols && a.lab_pitch >= a.cols && a.out_pitch >= a.cols, HK_ERR_INVALID,
+  if (a.n0 == 0) { a.n0 = a.rows; a.n1 = a.n2 = 1; }   // one level
+  HK_REQUIRE(a.n0 == 1 || (a.x_pitch >= a.cols && a.lab_pitch >= a.cols && a.out_pitch >= a.cols), HK_ERR_INVALID,
              "%s: a row pitch is smaller than the %d columns of a row", who, a.cols);
   switch (dtype) {
     case HK_FLOAT32: return sce_typed<float, MODE>(a, s);
     case HK_BFLOAT16: return sce_typed<bf16, MODE>(a, s);
     case HK_FLOAT16: return sce_typed<fp16, MODE>(a, s);
     case HK_FLOAT64:
-      HK_LAUNCH((sce_generic_kernel<double, double, MODE>), dim3(unsigned(a.rows)), dim3(256), 0, s, a);
+      HK_LAUNCH((sce_generic_kernel<double, double, MODE>), dim3(unsigned(a.n0), unsigned(a.n1), unsigned(a.n2)),
+                dim3(256), 0, s, a);
       return launch_check("sce_generic_kernel<double>");
     default:
       set_last_error("%s: not implemented for dtype %d", who, dtype);
@@ -535,6 +546,53 @@ int hk_sce_sparse_fwd(int dtype, const void* logits, const int64_t* labels, void
   a.logits = logits; a.labels = labels; a.out = loss; a.rows = rows; a.cols = int(cols);
   a.ignored_index = ignored_index;
   return sce_dispatch<0>(dtype, a, as_hip(stream), "hk_sce_sparse_fwd");
+}
+
+static int sce_levels(SceArgs& a, const int64_t level_rows[3], const char* who) {
+  HK_REQUIRE(level_rows, HK_ERR_INVALID, "%s: null level_rows", who);
+  const int64_t n0 = level_rows[0], n1 = level_rows[1], n2 = level_rows[2];
+  HK_REQUIRE(n0 >= 0 && n1 >= 0 && n2 >= 0, HK_ERR_INVALID, "%s: negative level count", who);
+  a.rows = 0;
+  if (n0 == 0 || n1 == 0 || n2 == 0) return HK_OK;
+  HK_REQUIRE(n1 <= 65535 && n2 <= 65535, HK_ERR_UNSUPPORTED,
+             "%s: the two outer levels hold at most 65535 rows each (got %lld, %lld)", who, (long long)n1, (long long)n2);
+  HK_REQUIRE(n0 <= 0x7fffffffLL && n0 * n1 <= 0x7fffffffLL && n0 * n1 * n2 <= 0x7fffffffLL, HK_ERR_INVALID,
+             "%s: too many rows", who);
+  a.rows = n0 * n1 * n2;
+  a.n0 = n0; a.n1 = n1; a.n2 = n2;
+  return HK_OK;
+}
+
+int hk_sce_sparse_fwd_strided_rows(int dtype, const void* logits, const int64_t logits_steps[3],
+                                   const int64_t* labels, void* loss, const int64_t level_rows[3], int64_t cols,
+                                   int64_t ignored_index, hkStream_t stream) {
+  const char* who = "hk_sce_sparse_fwd_strided_rows";
+  HK_REQUIRE(logits_steps, HK_ERR_INVALID, "%s: null steps", who);
+  HK_REQUIRE(cols >= 0 && cols <= 0x3fffffff, HK_ERR_INVALID, "%s: bad cols", who);
+  SceArgs a{};
+  int rc = sce_levels(a, level_rows, who);
+  if (rc != HK_OK) return rc;
+  a.logits = logits; a.labels = labels; a.out = loss; a.cols = int(cols);
+  a.x_pitch = logits_steps[0]; a.x_lv = LevelSteps{logits_steps[1], logits_steps[2]};
+  a.ignored_index = ignored_index;
+  return sce_dispatch<0>(dtype, a, as_hip(stream), who);
+}
+
+int hk_sce_sparse_bwd_strided_rows(int dtype, const void* logits, const int64_t logits_steps[3],
+                                   const int64_t* labels, const void* grad_loss, void* dlogits,
+                                   const int64_t dlogits_steps[3], const int64_t level_rows[3], int64_t cols,
+                                   int64_t ignored_index, hkStream_t stream) {
+  const char* who = "hk_sce_sparse_bwd_strided_rows";
+  HK_REQUIRE(logits_steps && dlogits_steps, HK_ERR_INVALID, "%s: null steps", who);
+  HK_REQUIRE(cols >= 0 && cols <= 0x3fffffff, HK_ERR_INVALID, "%s: bad cols", who);
+  SceArgs a{};
+  int rc = sce_levels(a, level_rows, who);
+  if (rc != HK_OK) return rc;
+  a.logits = logits; a.labels = labels; a.grad_loss = grad_loss; a.out = dlogits; a.cols = int(cols);
+  a.x_pitch = logits_steps[0]; a.x_lv = LevelSteps{logits_steps[1], logits_steps[2]};
+  a.out_pitch = dlogits_steps[0]; a.out_lv = LevelSteps{dlogits_steps[1], dlogits_steps[2]};
+  a.ignored_index = ignored_index;
+  return sce_dispatch<1>(dtype, a, as_hip(stream), who);
 }
 
 int hk_sce_sparse_fwd_pitched(int dtype, const void* logits, int64_t logits_pitch, const int64_t* labels,

@@ -20,6 +20,8 @@ struct SoftmaxArgs {
   void* out;        // forward: y;      backward: dx
   int64_t rows;
   int64_t x_pitch, dy_pitch, out_pitch;   // elements between row starts (== cols for a dense array)
+  int64_t n0, n1, n2;                     // rows on several levels (see LevelSteps); one level: n0 = rows
+  LevelSteps x_lv, dy_lv, out_lv;
   int cols;
   int nvec;
 };
@@ -34,10 +36,10 @@ void softmax_fwd_kernel(SoftmaxArgs a) {
   const int64_t row = WAVE_ROW
       ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index()
       : int64_t(blockIdx.x);
-  if (WAVE_ROW && row >= a.rows) return;
+  if (WAVE_ROW && row >= a.n0) return;   // row counts within the innermost level
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
 
-  const T* xr = static_cast<const T*>(a.x) + row * a.x_pitch;
+  const T* xr = static_cast<const T*>(a.x) + row * a.x_pitch + outer_level_offset(a.x_lv);
   // slots past the row's end hold -inf: they change neither the maximum nor the sum
   u32x4 raw[NV];
 #pragma unroll
@@ -71,7 +73,7 @@ void softmax_fwd_kernel(SoftmaxArgs a) {
   const float ML = (p.v[0] == kNegInf) ? 0.f : p.v[0];
   const float scale = __builtin_amdgcn_exp2f(ml - ML) / p.v[1];
 
-  T* yr = static_cast<T*>(a.out) + row * a.out_pitch;
+  T* yr = static_cast<T*>(a.out) + row * a.out_pitch + outer_level_offset(a.out_lv);
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int v = i * tpr + t;
@@ -94,11 +96,11 @@ void softmax_bwd_kernel(SoftmaxArgs a) {
   const int64_t row = WAVE_ROW
       ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index()
       : int64_t(blockIdx.x);
-  if (WAVE_ROW && row >= a.rows) return;
+  if (WAVE_ROW && row >= a.n0) return;   // row counts within the innermost level
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
 
-  const T* yr = static_cast<const T*>(a.x) + row * a.x_pitch;
-  const T* dyr = static_cast<const T*>(a.dy) + row * a.dy_pitch;
+  const T* yr = static_cast<const T*>(a.x) + row * a.x_pitch + outer_level_offset(a.x_lv);
+  const T* dyr = static_cast<const T*>(a.dy) + row * a.dy_pitch + outer_level_offset(a.dy_lv);
   u32x4 ry[NV], rdy[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -119,7 +121,7 @@ void softmax_bwd_kernel(SoftmaxArgs a) {
   }
   s = WAVE_ROW ? wave_allreduce_tuple(s) : group_allreduce_tuple(s, red, 0, nwaves);
   const float dot = s.v[0];
-  T* dxr = static_cast<T*>(a.out) + row * a.out_pitch;
+  T* dxr = static_cast<T*>(a.out) + row * a.out_pitch + outer_level_offset(a.out_lv);
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int v = i * tpr + t;
@@ -297,8 +299,10 @@ static int launch_softmax_nv(const SoftmaxArgs& a, int nv, dim3 grid, dim3 block
 template <typename T, bool BWD>
 static int softmax_lastdim_typed(SoftmaxArgs a, hipStream_t s) {
   constexpr int VEC = VecIO<T>::N;
+  auto steps_ok = [](int64_t pitch, const LevelSteps& l) { return pitch % VEC == 0 && l.p1 % VEC == 0 && l.p2 % VEC == 0; };
   const bool vec_ok = a.cols % VEC == 0 && aligned16(a.x) && aligned16(a.dy) && aligned16(a.out) &&
-                      a.x_pitch % VEC == 0 && a.out_pitch % VEC == 0 && (!BWD || a.dy_pitch % VEC == 0);
+                      steps_ok(a.x_pitch, a.x_lv) && steps_ok(a.out_pitch, a.out_lv) &&
+                      (!BWD || steps_ok(a.dy_pitch, a.dy_lv));
   a.nvec = a.cols / VEC;
   // forward keeps NV*VEC exponentials per thread: at most 64 floats
   // backward holds y and dy: at most 4 vectors of each per thread
@@ -307,11 +311,15 @@ static int softmax_lastdim_typed(SoftmaxArgs a, hipStream_t s) {
   int threads = 0, nv = 0;
   if (vec_ok && pick_softmax_shape(a.nvec, max_nv_wave, max_nv, BWD, &threads, &nv)) {
     if (threads == 64) {
-      dim3 grid(unsigned((a.rows + 3) / 4)), block(256);
+      dim3 grid(unsigned((a.n0 + 3) / 4), unsigned(a.n1), unsigned(a.n2)), block(256);
       return launch_softmax_nv<T, BWD, true>(a, nv, grid, block, s);
     }
-    dim3 grid{unsigned(a.rows)}, block{unsigned(threads)};
+    dim3 grid{unsigned(a.n0), unsigned(a.n1), unsigned(a.n2)}, block{unsigned(threads)};
     return launch_softmax_nv<T, BWD, false>(a, nv, grid, block, s);
+  }
+  if (a.n0 != a.rows) {
+    set_last_error("softmax: rows on several levels need 16-byte aligned rows and steps");
+    return HK_ERR_UNSUPPORTED;
   }
   if constexpr (BWD) {
     HK_LAUNCH((softmax_bwd_longrow_kernel<T, float>), dim3(unsigned(a.rows)), dim3(256), 0, s,
@@ -355,17 +363,22 @@ static int softmax_strided_typed(const void* x, const void* dy, void* out, int64
 
 // x_pitch / dy_pitch / out_pitch: elements between the starts of consecutive rows when inner == 1 (0: dense, the
 // row's own length); a dimension other than the last (inner > 1) only exists for dense arrays.
+struct SoftmaxLevels {
+  int64_t n0, n1, n2;
+  LevelSteps x, dy, out;
+};
+
 template <bool BWD>
 static int softmax_dispatch(int dtype, const void* x, const void* dy, void* out, int64_t outer,
                             int64_t dim, int64_t inner, int64_t x_pitch, int64_t dy_pitch, int64_t out_pitch,
-                            hipStream_t s, const char* who) {
+                            hipStream_t s, const char* who, const SoftmaxLevels* levels = nullptr) {
   HK_REQUIRE(outer >= 0 && dim >= 0 && inner >= 0, HK_ERR_INVALID, "%s: negative extent", who);
   if (outer == 0 || dim == 0 || inner == 0) return HK_OK;
   HK_REQUIRE(x && out && (!BWD || dy), HK_ERR_INVALID, "%s: null input/output", who);
   if (x_pitch == 0) x_pitch = dim;
   if (dy_pitch == 0) dy_pitch = dim;
   if (out_pitch == 0) out_pitch = dim;
-  HK_REQUIRE(x_pitch >= dim && out_pitch >= dim && dy_pitch >= dim, HK_ERR_INVALID,
+  HK_REQUIRE((levels && levels->n0 == 1) || (x_pitch >= dim && out_pitch >= dim && dy_pitch >= dim), HK_ERR_INVALID,
              "%s: a row pitch is smaller than the %lld columns of a row", who, (long long)dim);
   HK_REQUIRE(inner == 1 || (x_pitch == dim && dy_pitch == dim && out_pitch == dim), HK_ERR_INVALID,
              "%s: row pitches only apply to the last dimension", who);
@@ -375,12 +388,21 @@ static int softmax_dispatch(int dtype, const void* x, const void* dy, void* out,
     SoftmaxArgs a{};
     a.x = x; a.dy = dy; a.out = out; a.rows = outer; a.cols = int(dim);
     a.x_pitch = x_pitch; a.dy_pitch = dy_pitch; a.out_pitch = out_pitch;
+    a.n0 = outer; a.n1 = a.n2 = 1;
+    if (levels) {
+      a.n0 = levels->n0; a.n1 = levels->n1; a.n2 = levels->n2;
+      a.x_lv = levels->x; a.dy_lv = levels->dy; a.out_lv = levels->out;
+    }
     switch (dtype) {
       case HK_FLOAT32: return softmax_lastdim_typed<float, BWD>(a, s);
       case HK_BFLOAT16: return softmax_lastdim_typed<bf16, BWD>(a, s);
       case HK_FLOAT16: return softmax_lastdim_typed<fp16, BWD>(a, s);
       default: break;
     }
+  }
+  if (levels && levels->n0 != outer) {
+    set_last_error("%s: rows on several levels are not implemented for dtype %d", who, dtype);
+    return HK_ERR_UNSUPPORTED;
   }
   switch (dtype) {
     case HK_FLOAT32: return softmax_strided_typed<float, float, BWD>(x, dy, out, outer, dim, inner, x_pitch, dy_pitch, out_pitch, s);
@@ -409,6 +431,49 @@ int hk_softmax_fwd_pitched(int dtype, const void* x, int64_t x_pitch, void* y, i
   HK_REQUIRE(x_pitch > 0 && y_pitch > 0, HK_ERR_INVALID, "hk_softmax_fwd_pitched: a row pitch must be positive");
   return softmax_dispatch<false>(dtype, x, nullptr, y, rows, cols, 1, x_pitch, x_pitch, y_pitch, as_hip(stream),
                                  "hk_softmax_fwd_pitched");
+}
+
+static int softmax_levels(const int64_t level_rows[3], const int64_t* x_steps, const int64_t* dy_steps,
+                          const int64_t* out_steps, SoftmaxLevels* lv, int64_t* rows, const char* who) {
+  HK_REQUIRE(level_rows && x_steps && out_steps, HK_ERR_INVALID, "%s: null level_rows / steps", who);
+  const int64_t n0 = level_rows[0], n1 = level_rows[1], n2 = level_rows[2];
+  HK_REQUIRE(n0 >= 0 && n1 >= 0 && n2 >= 0, HK_ERR_INVALID, "%s: negative level count", who);
+  *rows = 0;
+  if (n0 == 0 || n1 == 0 || n2 == 0) return HK_OK;
+  HK_REQUIRE(n1 <= 65535 && n2 <= 65535, HK_ERR_UNSUPPORTED,
+             "%s: the two outer levels hold at most 65535 rows each (got %lld, %lld)", who, (long long)n1, (long long)n2);
+  HK_REQUIRE(n0 <= 0x7fffffffLL && n0 * n1 <= 0x7fffffffLL && n0 * n1 * n2 <= 0x7fffffffLL, HK_ERR_INVALID,
+             "%s: too many rows", who);
+  *rows = n0 * n1 * n2;
+  lv->n0 = n0; lv->n1 = n1; lv->n2 = n2;
+  lv->x = LevelSteps{x_steps[1], x_steps[2]};
+  lv->out = LevelSteps{out_steps[1], out_steps[2]};
+  lv->dy = dy_steps ? LevelSteps{dy_steps[1], dy_steps[2]} : LevelSteps{0, 0};
+  return HK_OK;
+}
+
+int hk_softmax_fwd_strided_rows(int dtype, const void* x, const int64_t x_steps[3], void* y, const int64_t y_steps[3],
+                                const int64_t level_rows[3], int64_t cols, hkStream_t stream) {
+  const char* who = "hk_softmax_fwd_strided_rows";
+  SoftmaxLevels lv{};
+  int64_t rows = 0;
+  int rc = softmax_levels(level_rows, x_steps, nullptr, y_steps, &lv, &rows, who);
+  if (rc != HK_OK || rows == 0) return rc;
+  return softmax_dispatch<false>(dtype, x, nullptr, y, rows, cols, 1, x_steps[0], x_steps[0], y_steps[0],
+                                 as_hip(stream), who, &lv);
+}
+
+int hk_softmax_bwd_strided_rows(int dtype, const void* y, const int64_t y_steps[3], const void* dy,
+                                const int64_t dy_steps[3], void* dx, const int64_t dx_steps[3],
+                                const int64_t level_rows[3], int64_t cols, hkStream_t stream) {
+  const char* who = "hk_softmax_bwd_strided_rows";
+  HK_REQUIRE(dy_steps, HK_ERR_INVALID, "%s: null steps", who);
+  SoftmaxLevels lv{};
+  int64_t rows = 0;
+  int rc = softmax_levels(level_rows, y_steps, dy_steps, dx_steps, &lv, &rows, who);
+  if (rc != HK_OK || rows == 0) return rc;
+  return softmax_dispatch<true>(dtype, y, dy, dx, rows, cols, 1, y_steps[0], dy_steps[0], dx_steps[0],
+                                as_hip(stream), who, &lv);
 }
 
 int hk_softmax_bwd(int dtype, const void* y, const void* dy, void* dx, int64_t outer, int64_t dim,

@@ -28,7 +28,6 @@ void FusedLayerNormCuda(const NDArray& in_arr, const NDArray& ln_scale, const ND
 
   int64_t rows, cols;
   SplitRows(in_arr, reduce_dims, rows, cols);
-  int64_t x_pitch = cols;
   HT_ASSERT(int64_t(ln_scale->numel()) == cols && int64_t(ln_bias->numel()) == cols)
     << "scale " << ln_scale->shape() << " / bias " << ln_bias->shape() << " do not match " << cols << " columns";
   HT_ASSERT(int64_t(mean_arr->numel()) == rows && int64_t(var_arr->numel()) == rows)
@@ -37,15 +36,18 @@ void FusedLayerNormCuda(const NDArray& in_arr, const NDArray& ln_scale, const ND
 
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
-  NDArray x = RowOperand(in_arr, reduce_dims, stream, &x_pitch);
+  // row-pitched arrays and views with permuted leading dimensions are read and written in place
+  RowPlan plan(reduce_dims, stream);
+  RowPlan::Slot& x = plan.Input(in_arr);
+  RowPlan::Slot& y = plan.Output(out_arr);
+  plan.Resolve();
   NDArray g = Dense(ln_scale, stream), b = Dense(ln_bias, stream);
-  RowOutput y(out_arr, reduce_dims, stream);
-  HK_CALL(hk_layer_norm_fwd_pitched(int(in_arr->dtype()), x->raw_data_ptr(), x_pitch, g->raw_data_ptr(),
-                                    b->raw_data_ptr(), y.ptr(), y.pitch(), mean_arr->raw_data_ptr(),
-                                    var_arr->raw_data_ptr(), HK_FLOAT32, HK_STAT_RSTD, rows, cols, eps,
-                                    hip_stream));
-  NDArray::MarkUsedBy({x, g, b, mean_arr, var_arr, y.array()}, stream);
-  y.Commit();
+  HK_CALL(hk_layer_norm_fwd_strided_rows(int(in_arr->dtype()), x.ptr(), x.steps, g->raw_data_ptr(),
+                                         b->raw_data_ptr(), y.ptr(), y.steps, mean_arr->raw_data_ptr(),
+                                         var_arr->raw_data_ptr(), HK_FLOAT32, HK_STAT_RSTD, plan.level_rows(), cols,
+                                         eps, hip_stream));
+  NDArray::MarkUsedBy({x.array, g, b, mean_arr, var_arr, y.array}, stream);
+  plan.Commit();
 }
 
 void FusedLayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr, const NDArray& ln_scale,
@@ -75,7 +77,6 @@ void FusedLayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr,
 
   int64_t rows, cols;
   SplitRows(in_arr, reduce_dims, rows, cols);
-  int64_t dy_pitch = cols, x_pitch = cols;
   HT_ASSERT(int64_t(ln_scale->numel()) == cols && int64_t(grad_scale->numel()) == cols &&
             int64_t(grad_bias->numel()) == cols)
     << "scale / grad_scale / grad_bias must hold " << cols << " values";
@@ -94,22 +95,25 @@ void FusedLayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr,
     }
     return;
   }
-  NDArray dy = RowOperand(out_grads, reduce_dims, stream, &dy_pitch);
-  NDArray xy = RowOperand(in_arr, reduce_dims, stream, &x_pitch), g = Dense(ln_scale, stream);
+  RowPlan plan(reduce_dims, stream);
+  RowPlan::Slot& dy = plan.Input(out_grads);
+  RowPlan::Slot& xy = plan.Input(in_arr);
+  RowPlan::Slot& dx = plan.Output(grad_arr);
+  plan.Resolve();
+  NDArray g = Dense(ln_scale, stream);
   NDArray b = Dense(ln_bias, stream), mean = Dense(mean_arr, stream), rstd = Dense(var_arr, stream);
   size_t ws_bytes = 0;
   HK_CALL(hk_norm_bwd_workspace_bytes(dt, rows, cols, &ws_bytes));
   NDArray ws = Scratch(ws_bytes, in_arr->device(), stream);
-  RowOutput dx(grad_arr, reduce_dims, stream);
   // gamma enters dx through clamp_by_magnitude(gamma, eps) in both modes
   // (FusedLayerNorm.cu:911-938)
-  HK_CALL(hk_layer_norm_bwd_pitched(dt, dy->raw_data_ptr(), dy_pitch, xy->raw_data_ptr(), x_pitch, g->raw_data_ptr(),
-                                    PtrOrNull(b), mean->raw_data_ptr(), rstd->raw_data_ptr(), HK_FLOAT32,
-                                    HK_STAT_RSTD, dx.ptr(), dx.pitch(), grad_scale->raw_data_ptr(),
-                                    grad_bias->raw_data_ptr(), rows, cols, eps, inplace ? 1 : 0, /*clamp_gamma=*/1,
-                                    MutPtrOrNull(ws), ws_bytes, hip_stream));
-  NDArray::MarkUsedBy({dy, xy, g, b, mean, rstd, dx.array(), grad_scale, grad_bias, ws}, stream);
-  dx.Commit();
+  HK_CALL(hk_layer_norm_bwd_strided_rows(dt, dy.ptr(), dy.steps, xy.ptr(), xy.steps, g->raw_data_ptr(), PtrOrNull(b),
+                                         mean->raw_data_ptr(), rstd->raw_data_ptr(), HK_FLOAT32, HK_STAT_RSTD,
+                                         dx.ptr(), dx.steps, grad_scale->raw_data_ptr(), grad_bias->raw_data_ptr(),
+                                         plan.level_rows(), cols, eps, inplace ? 1 : 0, /*clamp_gamma=*/1,
+                                         MutPtrOrNull(ws), ws_bytes, hip_stream));
+  NDArray::MarkUsedBy({dy.array, xy.array, g, b, mean, rstd, dx.array, grad_scale, grad_bias, ws}, stream);
+  plan.Commit();
 }
 
 } // namespace impl

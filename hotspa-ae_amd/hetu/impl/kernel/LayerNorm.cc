@@ -2,8 +2,9 @@
 // hetu/impl/kernel/LayerNorm.cu:66-121 and :235-337 of the reference (statistics
 // are mean and VARIANCE, stored in the data dtype), run by the gfx950 kernels
 // behind hk_layer_norm_fwd / hk_layer_norm_bwd.  The operator takes non-contiguous
-// arrays (hetu/graph/ops/LayerNorm.h:78-80): row-pitched inputs and outputs go to
-// the kernels as they are, any other input layout through a dense copy.
+// arrays (hetu/graph/ops/LayerNorm.h:78-80): row-pitched arrays and views with permuted
+// leading dimensions go to the kernels as they are (RowPlan), any other layout through
+// a dense copy (inputs) or a dense stand-in laid over the strides afterwards (outputs).
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/kernel/kernel_utils.h"
 #include "hetu/impl/utils/cpu_utils.h"
@@ -33,7 +34,6 @@ void LayerNormCuda(const NDArray& in_arr, const NDArray& ln_scale, const NDArray
 
   int64_t rows, cols;
   SplitRows(in_arr, reduce_dims, rows, cols);
-  int64_t x_pitch = cols;
   HT_ASSERT(int64_t(ln_scale->numel()) == cols && int64_t(ln_bias->numel()) == cols)
     << "scale " << ln_scale->shape() << " / bias " << ln_bias->shape() << " do not match " << cols << " columns";
   HT_ASSERT(int64_t(mean_arr->numel()) == rows && int64_t(var_arr->numel()) == rows)
@@ -42,15 +42,17 @@ void LayerNormCuda(const NDArray& in_arr, const NDArray& ln_scale, const NDArray
 
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
-  NDArray x = RowOperand(in_arr, reduce_dims, stream, &x_pitch);
+  RowPlan plan(reduce_dims, stream);
+  RowPlan::Slot& x = plan.Input(in_arr);
+  RowPlan::Slot& y = plan.Output(out_arr);
+  plan.Resolve();
   NDArray g = Dense(ln_scale, stream), b = Dense(ln_bias, stream);
-  RowOutput y(out_arr, reduce_dims, stream);
   const int dt = int(in_arr->dtype());
-  HK_CALL(hk_layer_norm_fwd_pitched(dt, x->raw_data_ptr(), x_pitch, g->raw_data_ptr(), b->raw_data_ptr(),
-                                    y.ptr(), y.pitch(), mean_arr->raw_data_ptr(),
-                                    var_arr->raw_data_ptr(), dt, HK_STAT_VAR, rows, cols, eps, hip_stream));
-  NDArray::MarkUsedBy({x, g, b, mean_arr, var_arr, y.array()}, stream);
-  y.Commit();
+  HK_CALL(hk_layer_norm_fwd_strided_rows(dt, x.ptr(), x.steps, g->raw_data_ptr(), b->raw_data_ptr(), y.ptr(), y.steps,
+                                         mean_arr->raw_data_ptr(), var_arr->raw_data_ptr(), dt, HK_STAT_VAR,
+                                         plan.level_rows(), cols, eps, hip_stream));
+  NDArray::MarkUsedBy({x.array, g, b, mean_arr, var_arr, y.array}, stream);
+  plan.Commit();
 }
 
 void LayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr, const NDArray& ln_scale,
@@ -78,7 +80,6 @@ void LayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr, cons
 
   int64_t rows, cols;
   SplitRows(in_arr, reduce_dims, rows, cols);
-  int64_t dy_pitch = cols, x_pitch = cols;
   HT_ASSERT(int64_t(ln_scale->numel()) == cols && int64_t(grad_scale->numel()) == cols &&
             int64_t(grad_bias->numel()) == cols)
     << "scale / grad_scale / grad_bias must hold " << cols << " values";
@@ -98,20 +99,24 @@ void LayerNormGradientCuda(const NDArray& out_grads, const NDArray& in_arr, cons
     }
     return;
   }
-  NDArray dy = RowOperand(out_grads, reduce_dims, stream, &dy_pitch);
-  NDArray x = RowOperand(in_arr, reduce_dims, stream, &x_pitch), g = Dense(ln_scale, stream);
+  RowPlan plan(reduce_dims, stream);
+  RowPlan::Slot& dy = plan.Input(out_grads);
+  RowPlan::Slot& x = plan.Input(in_arr);
+  RowPlan::Slot& dx = plan.Output(grad_arr);
+  plan.Resolve();
+  NDArray g = Dense(ln_scale, stream);
   NDArray mean = Dense(mean_arr, stream), var = Dense(var_arr, stream);
   size_t ws_bytes = 0;
   HK_CALL(hk_norm_bwd_workspace_bytes(dt, rows, cols, &ws_bytes));
   NDArray ws = Scratch(ws_bytes, in_arr->device(), stream);
-  RowOutput dx(grad_arr, reduce_dims, stream);
-  HK_CALL(hk_layer_norm_bwd_pitched(dt, dy->raw_data_ptr(), dy_pitch, x->raw_data_ptr(), x_pitch, g->raw_data_ptr(),
-                                    /*beta=*/nullptr, mean->raw_data_ptr(), var->raw_data_ptr(), dt, HK_STAT_VAR,
-                                    dx.ptr(), dx.pitch(), grad_scale->raw_data_ptr(),
-                                    grad_bias->raw_data_ptr(), rows, cols, eps, /*memory_efficient=*/0,
-                                    /*clamp_gamma=*/0, MutPtrOrNull(ws), ws_bytes, hip_stream));
-  NDArray::MarkUsedBy({dy, x, g, mean, var, dx.array(), grad_scale, grad_bias, ws}, stream);
-  dx.Commit();
+  HK_CALL(hk_layer_norm_bwd_strided_rows(dt, dy.ptr(), dy.steps, x.ptr(), x.steps, g->raw_data_ptr(),
+                                         /*beta=*/nullptr, mean->raw_data_ptr(), var->raw_data_ptr(), dt,
+                                         HK_STAT_VAR, dx.ptr(), dx.steps, grad_scale->raw_data_ptr(),
+                                         grad_bias->raw_data_ptr(), plan.level_rows(), cols, eps,
+                                         /*memory_efficient=*/0, /*clamp_gamma=*/0, MutPtrOrNull(ws), ws_bytes,
+                                         hip_stream));
+  NDArray::MarkUsedBy({dy.array, x.array, g, mean, var, dx.array, grad_scale, grad_bias, ws}, stream);
+  plan.Commit();
 }
 
 // ---------------------------------------------------------------------------------------------------------

@@ -37,13 +37,15 @@ void SoftmaxCuda(const NDArray& input, NDArray& output, int64_t dim, const Strea
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
   if (inner == 1) {
-    int64_t x_pitch = extent;
-    NDArray x = RowOperand(input, 1, stream, &x_pitch);
-    RowOutput y(output, 1, stream);
-    HK_CALL(hk_softmax_fwd_pitched(int(input->dtype()), x->raw_data_ptr(), x_pitch, y.ptr(), y.pitch(),
-                                   outer, extent, hip_stream));
-    NDArray::MarkUsedBy({x, y.array()}, stream);
-    y.Commit();
+    // row-pitched arrays and views with permuted leading dimensions are read and written in place
+    RowPlan plan(1, stream);
+    RowPlan::Slot& x = plan.Input(input);
+    RowPlan::Slot& y = plan.Output(output);
+    plan.Resolve(/*vector_rows_only=*/true);
+    HK_CALL(hk_softmax_fwd_strided_rows(int(input->dtype()), x.ptr(), x.steps, y.ptr(), y.steps, plan.level_rows(),
+                                        extent, hip_stream));
+    NDArray::MarkUsedBy({x.array, y.array}, stream);
+    plan.Commit();
     return;
   }
   NDArray x = Dense(input, stream);
@@ -69,13 +71,15 @@ void SoftmaxGradientCuda(const NDArray& input_Y, const NDArray& output_grad, NDA
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
   if (inner == 1) {
-    int64_t y_pitch = extent, dy_pitch = extent;
-    NDArray y = RowOperand(input_Y, 1, stream, &y_pitch), dy = RowOperand(output_grad, 1, stream, &dy_pitch);
-    RowOutput dx(input_grad, 1, stream);
-    HK_CALL(hk_softmax_bwd_pitched(int(input_Y->dtype()), y->raw_data_ptr(), y_pitch, dy->raw_data_ptr(), dy_pitch,
-                                   dx.ptr(), dx.pitch(), outer, extent, hip_stream));
-    NDArray::MarkUsedBy({y, dy, dx.array()}, stream);
-    dx.Commit();
+    RowPlan plan(1, stream);
+    RowPlan::Slot& y = plan.Input(input_Y);
+    RowPlan::Slot& dy = plan.Input(output_grad);
+    RowPlan::Slot& dx = plan.Output(input_grad);
+    plan.Resolve(/*vector_rows_only=*/true);
+    HK_CALL(hk_softmax_bwd_strided_rows(int(input_Y->dtype()), y.ptr(), y.steps, dy.ptr(), dy.steps, dx.ptr(), dx.steps,
+                                        plan.level_rows(), extent, hip_stream));
+    NDArray::MarkUsedBy({y.array, dy.array, dx.array}, stream);
+    plan.Commit();
     return;
   }
   NDArray y = Dense(input_Y, stream), dy = Dense(output_grad, stream);

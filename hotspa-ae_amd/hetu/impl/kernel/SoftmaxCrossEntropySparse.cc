@@ -37,11 +37,14 @@ void SoftmaxCrossEntropySparseCuda(const NDArray& pred, const NDArray& label, ND
 
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
-  int64_t p_pitch = cols;
-  NDArray p = RowOperand(pred, 1, stream, &p_pitch), l = Dense(label, stream);
-  HK_CALL(hk_sce_sparse_fwd_pitched(int(pred->dtype()), p->raw_data_ptr(), p_pitch, l->data_ptr<int64_t>(),
-                                    loss->raw_data_ptr(), rows, cols, ignored_index, hip_stream));
-  NDArray::MarkUsedBy({p, l, loss}, stream);
+  // row-pitched logits and views with permuted leading dimensions are read in place
+  RowPlan plan(1, stream);
+  RowPlan::Slot& p = plan.Input(pred);
+  plan.Resolve();
+  NDArray l = Dense(label, stream);
+  HK_CALL(hk_sce_sparse_fwd_strided_rows(int(pred->dtype()), p.ptr(), p.steps, l->data_ptr<int64_t>(),
+                                         loss->raw_data_ptr(), plan.level_rows(), cols, ignored_index, hip_stream));
+  NDArray::MarkUsedBy({p.array, l, loss}, stream);
 }
 
 namespace {
@@ -59,7 +62,6 @@ void SparseGradient(const NDArray& pred, const NDArray& label, const NDArray& gr
   HT_ASSERT(label->dtype() == kInt64) << "labels must be int64 class ids, got " << label->dtype();
   int64_t rows, cols;
   RowsCols(pred, rows, cols);
-  int64_t p_pitch = cols;
   HT_ASSERT(int64_t(label->numel()) == rows) << "labels " << label->shape() << " must hold one value per row of "
                                              << pred->shape();
   if (scale) {
@@ -73,20 +75,27 @@ void SparseGradient(const NDArray& pred, const NDArray& label, const NDArray& gr
 
   HIPStream hip_stream(stream);
   hip::DeviceGuard guard(hip_stream.device_id());
-  NDArray p = scale ? Dense(pred, stream) : RowOperand(pred, 1, stream, &p_pitch);
   NDArray l = Dense(label, stream), g = Dense(grad_loss, stream);
-  RowOutput out(output, scale ? -1 : 1, stream);
   if (scale) {
+    NDArray p = Dense(pred, stream);
+    RowOutput out(output, -1, stream);
     HK_CALL(hk_sce_sparse_bwd_reduced(int(pred->dtype()), p->raw_data_ptr(), l->data_ptr<int64_t>(),
                                       g->raw_data_ptr(), *scale, out.ptr(), rows, cols, ignored_index,
                                       hip_stream));
-  } else {
-    HK_CALL(hk_sce_sparse_bwd_pitched(int(pred->dtype()), p->raw_data_ptr(), p_pitch, l->data_ptr<int64_t>(),
-                                      g->raw_data_ptr(), out.ptr(), out.pitch(), rows, cols,
-                                      ignored_index, hip_stream));
+    NDArray::MarkUsedBy({p, l, g, out.array()}, stream);
+    out.Commit();
+    return;
   }
-  NDArray::MarkUsedBy({p, l, g, out.array()}, stream);
-  out.Commit();
+  // row-pitched arrays and views with permuted leading dimensions are read and written in place
+  RowPlan plan(1, stream);
+  RowPlan::Slot& p = plan.Input(pred);
+  RowPlan::Slot& out = plan.Output(output);
+  plan.Resolve();
+  HK_CALL(hk_sce_sparse_bwd_strided_rows(int(pred->dtype()), p.ptr(), p.steps, l->data_ptr<int64_t>(),
+                                         g->raw_data_ptr(), out.ptr(), out.steps, plan.level_rows(), cols,
+                                         ignored_index, hip_stream));
+  NDArray::MarkUsedBy({p.array, l, g, out.array}, stream);
+  plan.Commit();
 }
 } // namespace
 

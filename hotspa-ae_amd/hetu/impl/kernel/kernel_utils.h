@@ -92,6 +92,155 @@ class RowOutput {
   int64_t pitch_ = 0;
 };
 
+// The row operands of ONE kernel call on joint levels, for the *_strided_rows entry points.  A view whose leading
+// dimensions are permuted (x.permute(0, 2, 1, 3): rows contiguous, leading dimensions not on one pitch) keeps its
+// rows on up to three levels, row r = (i2 * n1 + i1) * n0 + i0 starting i0 * s0 + i1 * s1 + i2 * s2 elements from
+// the base; the kernels take that as it is, so such an operand is read / written in place where the reference
+// walks it through its OffsetCalculator (hetu/impl/utils/offset_calculator.cuh:16-68).  Leading dimensions are
+// merged where they step together in EVERY operand of the call, since all operands share one numbering of the
+// rows.  What does not fit (trailing dimensions that are not dense, more than three levels, more than 65535 rows
+// on an outer level) falls back operand by operand: an input is gathered into a dense copy, an output is written
+// dense into pool memory and laid over its strides by Commit().
+class RowPlan {
+ public:
+  struct Slot {
+    NDArray array;              // what the kernel reads or writes
+    NDArray* target = nullptr;  // outputs: the caller's array
+    int64_t steps[3] = {0, 0, 0};
+    bool defined() const { return array.is_defined(); }
+    void* ptr() { return array.is_defined() ? array->raw_data_ptr() : nullptr; }
+    const int64_t* steps_or_null() const { return array.is_defined() ? steps : nullptr; }
+    bool staged() const { return target != nullptr && array->raw_data_ptr() != (*target)->raw_data_ptr(); }
+  };
+
+  RowPlan(int64_t inner_dims, const Stream& stream) : inner_dims_(inner_dims), stream_(stream) {}
+
+  // an undefined array is an absent optional operand
+  Slot& Input(const NDArray& a) {
+    slots_[count_].array = a;
+    return slots_[count_++];
+  }
+  Slot& Output(NDArray& a) {
+    slots_[count_].array = a;
+    slots_[count_].target = a.is_defined() ? &a : nullptr;
+    return slots_[count_++];
+  }
+
+  // call once after every operand has been added.  vector_rows_only: the kernels behind the call take several
+  // levels on their 128-bit path only (softmax, cross-entropy), so rows and steps that are not whole 16-byte
+  // vectors go dense as well
+  void Resolve(bool vector_rows_only = false) {
+    // an operand whose trailing dimensions are not dense has no 128-bit row at all
+    for (int k = 0; k < count_; ++k)
+      if (slots_[k].defined() && !TrailingDense(slots_[k].array)) MakeDense(slots_[k]);
+    if (!JointLevels() || (vector_rows_only && level_rows_[1] * level_rows_[2] > 1 && !WholeVectors())) {
+      // too many levels: everything that is not on one pitch by itself goes dense, which leaves one level
+      for (int k = 0; k < count_; ++k) {
+        int64_t pitch = 0;
+        if (slots_[k].defined() && !RowPitch(slots_[k].array, inner_dims_, &pitch)) MakeDense(slots_[k]);
+      }
+      const bool ok = JointLevels();
+      HT_ASSERT(ok) << "row operands do not reduce to one level";
+    }
+  }
+
+  const int64_t* level_rows() const { return level_rows_; }
+
+  // after the kernel call, on the same stream
+  void Commit() {
+    for (int k = 0; k < count_; ++k) {
+      Slot& sl = slots_[k];
+      if (!sl.defined() || !sl.staged()) continue;
+      HIPStream hip_stream(stream_);
+      const HTShape& shape = (*sl.target)->shape();
+      const HTStride& stride = (*sl.target)->stride();
+      HK_CALL(hk_strided_scatter(int((*sl.target)->dtype()), sl.array->raw_data_ptr(), (*sl.target)->raw_data_ptr(),
+                                 int(shape.size()), shape.data(), stride.data(), hip_stream));
+      NDArray::MarkUsedBy({sl.array, *sl.target}, stream_);
+    }
+  }
+
+  // every array a kernel call touches, for NDArray::MarkUsedBy
+  NDArrayList arrays() const {
+    NDArrayList out;
+    for (int k = 0; k < count_; ++k)
+      if (slots_[k].defined()) out.push_back(slots_[k].array);
+    return out;
+  }
+
+ private:
+  bool TrailingDense(const NDArray& a) const {
+    const int64_t nd = int64_t(a->ndim());
+    int64_t expect = 1;
+    for (int64_t i = nd - 1; i >= nd - inner_dims_; --i) {
+      if (a->shape(i) != 1 && a->stride(i) != expect) return false;
+      expect *= a->shape(i);
+    }
+    return true;
+  }
+  // every base address and every step a whole number of 16-byte vectors
+  bool WholeVectors() const {
+    for (int k = 0; k < count_; ++k) {
+      if (!slots_[k].defined()) continue;
+      const size_t es = DataType2Size(slots_[k].array->dtype());
+      if (reinterpret_cast<uintptr_t>(slots_[k].array->raw_data_ptr()) % 16 != 0) return false;
+      for (int j = 0; j < 3; ++j)
+        if ((size_t(slots_[k].steps[j]) * es) % 16 != 0) return false;
+    }
+    return true;
+  }
+  void MakeDense(Slot& sl) {
+    if (sl.target == nullptr) {
+      sl.array = NDArray::contiguous(sl.array, stream_.stream_index());
+    } else {
+      sl.array = NDArray::empty((*sl.target)->shape(), (*sl.target)->device(), (*sl.target)->dtype(),
+                                stream_.stream_index());
+    }
+  }
+  // merges the leading dimensions over all operands; false when more than three levels remain or an outer
+  // level is too long for a grid's y / z
+  bool JointLevels() {
+    const Slot* ref = nullptr;
+    for (int k = 0; k < count_; ++k)
+      if (slots_[k].defined()) { ref = &slots_[k]; break; }
+    int64_t counts[3] = {1, 1, 1};
+    int64_t steps[kMaxSlots][3];
+    int levels = 0;
+    const int64_t nd = ref ? int64_t(ref->array->ndim()) : 0;
+    int64_t cols = 1;
+    for (int64_t i = nd - inner_dims_; i < nd; ++i) cols *= ref->array->shape(i);
+    for (int k = 0; k < count_; ++k) { steps[k][0] = cols; steps[k][1] = steps[k][2] = 0; }
+    for (int64_t i = nd - inner_dims_ - 1; i >= 0; --i) {
+      const int64_t n = ref->array->shape(i);
+      if (n == 1) continue;
+      bool merges = levels > 0;
+      for (int k = 0; k < count_ && merges; ++k)
+        if (slots_[k].defined() && slots_[k].array->stride(i) != counts[levels - 1] * steps[k][levels - 1]) merges = false;
+      if (merges) {
+        counts[levels - 1] *= n;
+        continue;
+      }
+      if (levels == 3) return false;
+      counts[levels] = n;
+      for (int k = 0; k < count_; ++k)
+        if (slots_[k].defined()) steps[k][levels] = slots_[k].array->stride(i);
+      ++levels;
+    }
+    if (counts[1] > 65535 || counts[2] > 65535) return false;
+    for (int j = 0; j < 3; ++j) level_rows_[j] = counts[j];
+    for (int k = 0; k < count_; ++k)
+      for (int j = 0; j < 3; ++j) slots_[k].steps[j] = steps[k][j];
+    return true;
+  }
+
+  static constexpr int kMaxSlots = 8;
+  Slot slots_[kMaxSlots];
+  int count_ = 0;
+  int64_t inner_dims_;
+  Stream stream_;
+  int64_t level_rows_[3] = {1, 1, 1};
+};
+
 inline const void* PtrOrNull(const NDArray& a) {
   return a.is_defined() ? a->raw_data_ptr() : nullptr;
 }

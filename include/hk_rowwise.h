@@ -170,6 +170,26 @@ HK_API int hk_layer_norm_fwd_pitched(int dtype, const void* x, int64_t x_pitch, 
                                      int stats_dtype, int stat_kind, int64_t rows, int64_t cols,
                                      float eps, hkStream_t stream);
 
+/* The same on rows laid out on up to THREE LEVELS: what a view with permuted leading dimensions presents, e.g.
+ * x.permute(0, 2, 1, 3) of a dense [B, H, S, D] array normalised over D.  Rows are numbered
+ *   r = (i2 * level_rows[1] + i1) * level_rows[0] + i0,   0 <= i_k < level_rows[k]
+ * (the view's own row-major order) and row r of an operand starts
+ *   i0 * steps[0] + i1 * steps[1] + i2 * steps[2]   ELEMENTS
+ * from its base, every operand with its own steps (the strides of the view's leading dimensions, merged where
+ * neighbours step together; a dense operand is {cols, level_rows[0] * cols, level_rows[0] * level_rows[1] * cols});
+ * mean / stat stay dense [rows] arrays indexed by r.  The last dimension must have unit stride.  The row kernels
+ * run on a three-dimensional grid whose y / z are i1 / i2, so such a view is read and written IN PLACE with the
+ * 128-bit kernels (steps that are whole 16-byte vectors), no gather or scatter pass: the traffic is the dense
+ * call's.  level_rows[1], level_rows[2] <= 65535 (HK_ERR_UNSUPPORTED beyond; the caller then gathers).
+ * Replaces, for such views, the per-element OffsetCalculator of the reference
+ * (hetu/impl/utils/offset_calculator.cuh:16-68, .cu:31-65), on which its LayerNorm / Softmax operators run
+ * because they accept non-contiguous inputs (hetu/graph/ops/LayerNorm.h:78-80, Softmax.h:52-54). */
+HK_API int hk_layer_norm_fwd_strided_rows(int dtype, const void* x, const int64_t x_steps[3], const void* gamma,
+                                          const void* beta, void* y, const int64_t y_steps[3], void* mean,
+                                          void* stat, int stats_dtype, int stat_kind,
+                                          const int64_t level_rows[3], int64_t cols, float eps,
+                                          hkStream_t stream);
+
 /* Bytes of scratch hk_layer_norm_bwd / hk_dropout_add_ln_bwd need for the
  * column-sum partials of dgamma / dbeta. */
 HK_API int hk_norm_bwd_workspace_bytes(int dtype, int64_t rows, int64_t cols, size_t* bytes);
@@ -197,6 +217,17 @@ HK_API int hk_layer_norm_bwd_pitched(int dtype, const void* dy, int64_t dy_pitch
                                      void* dx, int64_t dx_pitch, void* dgamma, void* dbeta, int64_t rows,
                                      int64_t cols, float eps, int memory_efficient, int clamp_gamma,
                                      void* workspace, size_t workspace_bytes, hkStream_t stream);
+
+/* hk_layer_norm_bwd on operands whose rows lie on up to three levels (see hk_layer_norm_fwd_strided_rows); the
+ * workspace is that of hk_norm_bwd_workspace_bytes for rows = the product of level_rows.  The walking kernel
+ * splits each row number itself (two integer divisions per row and workgroup), in its general instance. */
+HK_API int hk_layer_norm_bwd_strided_rows(int dtype, const void* dy, const int64_t dy_steps[3], const void* x_or_y,
+                                          const int64_t x_steps[3], const void* gamma, const void* beta,
+                                          const void* mean, const void* stat, int stats_dtype, int stat_kind,
+                                          void* dx, const int64_t dx_steps[3], void* dgamma, void* dbeta,
+                                          const int64_t level_rows[3], int64_t cols, float eps,
+                                          int memory_efficient, int clamp_gamma, void* workspace,
+                                          size_t workspace_bytes, hkStream_t stream);
 
 /* ======================================================================== *
  * Dropout-add-LayerNorm / RMSNorm (flash-attention layer_norm path).
@@ -240,6 +271,25 @@ HK_API int hk_dropout_add_ln_bwd_pitched(int itype, int rtype, int wtype, const 
                                          int64_t dresidual_pitch, void* dgamma, void* dbeta, int64_t rows,
                                          int64_t cols, int is_rms_norm, void* workspace,
                                          size_t workspace_bytes, hkStream_t stream);
+
+/* The same two calls on operands whose rows lie on up to three levels (see hk_layer_norm_fwd_strided_rows);
+ * the steps of an absent optional operand may be NULL. */
+HK_API int hk_dropout_add_ln_fwd_strided_rows(int itype, int rtype, int wtype, const void* x0,
+                                              const int64_t x0_steps[3], const void* residual,
+                                              const int64_t residual_steps[3], const void* gamma,
+                                              const void* beta, void* z, const int64_t z_steps[3], void* x_out,
+                                              const int64_t x_out_steps[3], void* mu, void* rsigma,
+                                              const int64_t level_rows[3], int64_t cols, float eps,
+                                              int is_rms_norm, hkStream_t stream);
+HK_API int hk_dropout_add_ln_bwd_strided_rows(int itype, int rtype, int wtype, const void* dz,
+                                              const int64_t dz_steps[3], const void* dx_in,
+                                              const int64_t dx_in_steps[3], const void* x,
+                                              const int64_t x_steps[3], const void* mu, const void* rsigma,
+                                              const void* gamma, void* dx0, const int64_t dx0_steps[3],
+                                              void* dresidual, const int64_t dresidual_steps[3], void* dgamma,
+                                              void* dbeta, const int64_t level_rows[3], int64_t cols,
+                                              int is_rms_norm, void* workspace, size_t workspace_bytes,
+                                              hkStream_t stream);
 
 /* hk_dropout_add_ln_bwd for callers that cannot allocate device memory and so have no workspace to
  * pass: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
@@ -404,6 +454,16 @@ HK_API int hk_softmax_fwd_pitched(int dtype, const void* x, int64_t x_pitch, voi
 HK_API int hk_softmax_bwd_pitched(int dtype, const void* y, int64_t y_pitch, const void* dy, int64_t dy_pitch,
                                   void* dx, int64_t dx_pitch, int64_t rows, int64_t cols, hkStream_t stream);
 
+/* Last-dimension softmax of operands whose rows lie on up to three levels (see hk_layer_norm_fwd_strided_rows):
+ * a view with permuted leading dimensions is read and written in place.  Rows must be whole 16-byte vectors
+ * (HK_ERR_UNSUPPORTED otherwise; the caller then gathers). */
+HK_API int hk_softmax_fwd_strided_rows(int dtype, const void* x, const int64_t x_steps[3], void* y,
+                                       const int64_t y_steps[3], const int64_t level_rows[3], int64_t cols,
+                                       hkStream_t stream);
+HK_API int hk_softmax_bwd_strided_rows(int dtype, const void* y, const int64_t y_steps[3], const void* dy,
+                                       const int64_t dy_steps[3], void* dx, const int64_t dx_steps[3],
+                                       const int64_t level_rows[3], int64_t cols, hkStream_t stream);
+
 /* ======================================================================== *
  * Fused softmax cross-entropy, sparse int64 labels.
  * logits: [rows, cols]; labels: [rows] int64; loss: [rows] `dtype`.
@@ -432,6 +492,16 @@ HK_API int hk_sce_sparse_bwd_pitched(int dtype, const void* logits, int64_t logi
                                      const int64_t* labels, const void* grad_loss, void* dlogits,
                                      int64_t dlogits_pitch, int64_t rows, int64_t cols,
                                      int64_t ignored_index, hkStream_t stream);
+
+/* The same on logits / dlogits whose rows lie on up to three levels (see hk_layer_norm_fwd_strided_rows);
+ * labels, loss and grad_loss stay dense [rows] arrays indexed by the row's number. */
+HK_API int hk_sce_sparse_fwd_strided_rows(int dtype, const void* logits, const int64_t logits_steps[3],
+                                          const int64_t* labels, void* loss, const int64_t level_rows[3],
+                                          int64_t cols, int64_t ignored_index, hkStream_t stream);
+HK_API int hk_sce_sparse_bwd_strided_rows(int dtype, const void* logits, const int64_t logits_steps[3],
+                                          const int64_t* labels, const void* grad_loss, void* dlogits,
+                                          const int64_t dlogits_steps[3], const int64_t level_rows[3],
+                                          int64_t cols, int64_t ignored_index, hkStream_t stream);
 
 /* The same with the gradient of a REDUCED loss: grad_output holds one value and every row uses
  * round_dtype(grad_output[0] * round_dtype(scale)) -- what BroadcastShapeMul(grad, 1/rows) into a [rows]

@@ -1028,3 +1028,97 @@ def test_batch_norm_entry_points(ops, cuda, dtype):
             ops.batch_norm(tx, ts.bfloat16(), tb, ty, 0.1, 1e-5, trm, trv, sm, sv)
     with pytest.raises(ops.AssertionError_, match="one value per channel"):
         ops.batch_norm(tx, ts[:11].contiguous(), tb, ty, 0.1, 1e-5, trm, trv, sm, sv)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_permuted_views_run_in_place(ops, cuda, dtype):
+    """x.permute(0, 2, 1, 3) of a dense [B, H, S, D] array as input AND output of the norm / softmax / cross-entropy
+    operators: the values equal the dense call's bit for bit, and the operator takes nothing from the pool for the
+    forward calls (no gather of the input, no stand-in for the output: the reference reads such views through its
+    OffsetCalculator, this layer through the row levels of the kernels)."""
+    import torch
+    B, H, S, D = 2, 3, 5, 256
+    x = helpers.draw(951, (B, S, H, D), dtype=dtype)           # the VIEW's logical contents
+    dy = helpers.draw(952, (B, S, H, D), dtype=dtype)
+    g = helpers.draw(953, (D,), "uniform", 0.5, 1.5, dtype)
+    b = helpers.draw(954, (D,), "normal", 0.0, 0.1, dtype)
+    tg, tb = helpers.to_torch(g, dtype, cuda), helpers.to_torch(b, dtype, cuda)
+    td = tg.dtype
+    rows = B * S * H
+
+    def permuted(values):
+        stored = helpers.to_torch(np.ascontiguousarray(np.transpose(values, (0, 2, 1, 3))), dtype, cuda)   # [B, H, S, D]
+        return stored.permute(0, 2, 1, 3)
+
+    def empty_view():
+        return torch.full((B, H, S, D), 7.0, dtype=td, device=cuda).permute(0, 2, 1, 3)
+
+    vx, vdy = permuted(x), permuted(dy)
+    dx_dense, dy_dense = vx.contiguous(), vdy.contiguous()
+    assert not vx.is_contiguous()
+
+    def both(run, what, allocs=0, exact=True):
+        """run(x_like, dy_like, out) on dense arrays, then on the views; allocs = pool allocations the call may make;
+        exact=False where the view takes another instance of the kernel than the dense array (the walking backward
+        kernel splits row numbers in its general instance only), whose results may differ in the last bit"""
+        dense = torch.empty((B, S, H, D), dtype=td, device=cuda)
+        _sync_in()
+        run(dx_dense, dy_dense, dense)
+        ops.stream_sync()
+        view = empty_view()
+        _sync_in()
+        before = ops.pool_stats()["alloc_cnt"]
+        run(vx, vdy, view)
+        ops.stream_sync()
+        assert ops.pool_stats()["alloc_cnt"] - before == allocs, what + ": pool allocations for a permuted view"
+        if exact:
+            assert torch.equal(view.contiguous(), dense), what
+        else:
+            helpers.assert_close(view.contiguous(), helpers.to_numpy(dense).astype(np.float64), dtype, what)
+
+    mean = torch.empty(rows, dtype=torch.float32, device=cuda)
+    rstd = torch.empty(rows, dtype=torch.float32, device=cuda)
+    both(lambda a, d, out: ops.fused_layer_norm(a, tg, tb, mean, rstd, out, 1, 1e-5), "fused layer norm")
+    ey, em, _, ers = oracle.layernorm_fwd(x.reshape(rows, D), g, b, 1e-5)
+    helpers.assert_close(rstd, ers, "fp32", "rstd")
+    dg, db = torch.empty_like(tg), torch.empty_like(tg)
+    # the backward takes its column-sum partials from the pool: one allocation, views or not
+    both(lambda a, d, out: ops.fused_layer_norm_gradient(d, a, tg, tb, out, dg, db, mean, rstd, 1, 1e-5, False),
+         "fused layer norm gradient", allocs=1, exact=False)
+    edx, _, _ = oracle.layernorm_bwd(dy.reshape(rows, D), x.reshape(rows, D), g, helpers.to_numpy(mean),
+                                     helpers.to_numpy(rstd), eps=1e-5, clamp_gamma=True)
+    view = empty_view()
+    _sync_in()
+    ops.fused_layer_norm_gradient(vdy, vx, tg, tb, view, dg, db, mean, rstd, 1, 1e-5, False)
+    ops.stream_sync()
+    helpers.assert_close(view.reshape(rows, D), edx, dtype, "dx")
+    mean_t, var_t = torch.empty(rows, dtype=td, device=cuda), torch.empty(rows, dtype=td, device=cuda)
+    both(lambda a, d, out: ops.layer_norm(a, tg, tb, mean_t, var_t, out, 1, 1e-5), "layer norm")
+    both(lambda a, d, out: ops.layer_norm_gradient(d, a, tg, out, dg, db, mean_t, var_t, 1, 1e-5), "layer norm gradient",
+         allocs=1, exact=False)
+    both(lambda a, d, out: ops.softmax(a, out, -1), "softmax")
+    ty = torch.empty((B, S, H, D), dtype=td, device=cuda)
+    _sync_in()
+    ops.softmax(dx_dense, ty, -1)
+    ops.stream_sync()
+    vy = permuted(helpers.to_numpy(ty))
+    dense = torch.empty((B, S, H, D), dtype=td, device=cuda)
+    view = empty_view()
+    _sync_in()
+    ops.softmax_gradient(ty, dy_dense, dense, -1)
+    before = ops.pool_stats()["alloc_cnt"]
+    ops.softmax_gradient(vy, vdy, view, -1)
+    ops.stream_sync()
+    assert ops.pool_stats()["alloc_cnt"] == before and torch.equal(view.contiguous(), dense), "softmax gradient"
+    labels = torch.randint(0, D, (B, S, H), device=cuda, dtype=torch.int64)
+    labels[0, 1, 2] = -100
+    gl = helpers.to_torch(helpers.draw(955, (B, S, H), dtype=dtype), dtype, cuda)
+    loss_d = torch.empty((B, S, H), dtype=td, device=cuda)
+    loss_v = torch.empty((B, S, H), dtype=td, device=cuda)
+    _sync_in()
+    ops.softmax_cross_entropy_sparse(dx_dense, labels, loss_d, -100)
+    before = ops.pool_stats()["alloc_cnt"]
+    ops.softmax_cross_entropy_sparse(vx, labels, loss_v, -100)
+    ops.stream_sync()
+    assert ops.pool_stats()["alloc_cnt"] == before and torch.equal(loss_v, loss_d), "sparse CE"
+    both(lambda a, d, out: ops.softmax_cross_entropy_sparse_gradient(a, labels, gl, out, -100), "sparse CE gradient")

@@ -131,6 +131,55 @@ def case_rmsnorm_pitched(hk, torch, nsets, which):
         3 * rows * cols * 2 + rows * 4 + cols * 2 + 2 * cols * 2, rows
 
 
+def case_rmsnorm_permuted(hk, torch, nsets, which):
+    """The headline shape as a view with permuted leading dimensions: arrays stored [2048, 16, 4096] (sequence first)
+    and used as [16, 2048, 4096] (batch first) through permute(1, 0, 2), inputs and outputs alike.  Rows stay contiguous,
+    the leading dimensions lie on two levels; the kernels take the steps, nothing is gathered or scattered."""
+    S, B, cols, eps = 2048, 16, 4096, 1e-6
+    rows = S * B
+    bf = torch.bfloat16
+    sets = []
+    for i in range(nsets):
+        st = {k: torch.empty((S, B, cols), dtype=bf, device="cuda") for k in ("x", "dz", "z", "dx")}
+        st["x"].copy_(_randn(torch, (S, B, cols), bf, 1.0, 402 + 10 * i))
+        st["dz"].copy_(_randn(torch, (S, B, cols), bf, 1.0, 404 + 10 * i))
+        s = {k: v.permute(1, 0, 2) for k, v in st.items()}
+        s["mu"], s["rs"] = torch.empty(rows, device="cuda"), torch.empty(rows, device="cuda")
+        sets.append(s)
+    w = _uniform(torch, (cols,), bf, 0.8, 1.2, 403)
+    dg, db = torch.empty_like(w), torch.empty_like(w)
+    ws = torch.empty(max(1, hk.norm_bwd_workspace_bytes(8, rows, cols) // 4), device="cuda")
+    for s in sets:
+        hk.dropout_add_ln_fwd(s["x"], None, w, None, s["z"], None, s["mu"], s["rs"], eps, True)
+    if which == "fwd":
+        return (lambda i: hk.dropout_add_ln_fwd(sets[i % nsets]["x"], None, w, None, sets[i % nsets]["z"], None,
+                                                sets[i % nsets]["mu"], sets[i % nsets]["rs"], eps, True)), \
+            2 * rows * cols * 2 + cols * 2 + rows * 8, rows
+    return (lambda i: hk.dropout_add_ln_bwd(sets[i % nsets]["dz"], None, sets[i % nsets]["x"], sets[i % nsets]["mu"],
+                                            sets[i % nsets]["rs"], w, sets[i % nsets]["dx"], None, dg, db, True,
+                                            workspace=ws)), \
+        3 * rows * cols * 2 + rows * 4 + cols * 2 + 2 * cols * 2, rows
+
+
+def case_softmax_permuted(hk, torch, nsets, which):
+    """Softmax over the last dimension of attention scores stored [4, 2048, 32, 2048] (batch, query, head, key) and used
+    as [4, 32, 2048, 2048] through permute(0, 2, 1, 3): three levels of rows, read and written in place."""
+    B, H, S = 4, 32, 2048
+    bf = torch.bfloat16
+    n = B * H * S * S
+    sets = []
+    for i in range(nsets):
+        st = {k: torch.empty((B, S, H, S), dtype=bf, device="cuda") for k in ("x", "y", "dy", "dx")}
+        st["x"].copy_(_randn(torch, (B, S, H, S), bf, 3.0, 201 + 10 * i))
+        st["dy"].copy_(_randn(torch, (B, S, H, S), bf, 1.0, 202 + 10 * i))
+        s = {k: v.permute(0, 2, 1, 3) for k, v in st.items()}
+        hk.softmax_fwd(s["x"], s["y"])
+        sets.append(s)
+    if which == "fwd":
+        return (lambda i: hk.softmax_fwd(sets[i % nsets]["x"], sets[i % nsets]["y"])), 2 * n * 2, B * H * S
+    return (lambda i: hk.softmax_bwd(sets[i % nsets]["y"], sets[i % nsets]["dy"], sets[i % nsets]["dx"])), 3 * n * 2, B * H * S
+
+
 def case_layernorm(hk, torch, nsets, which, cfg):
     if cfg == "C1":
         rows, cols, dt, eps = 8192, 4096, torch.float32, 1e-5
@@ -522,6 +571,14 @@ CASES = [
      lambda hk, t, n: case_rmsnorm_pitched(hk, t, n, "fwd")),
     ("next: rmsnorm bwd bf16 on a [32768x4096] slice of [32768x4608] (row-pitched in and out)",
      lambda hk, t, n: case_rmsnorm_pitched(hk, t, n, "bwd")),
+    ("next: rmsnorm fwd bf16 on a [16,2048,4096] view of a [2048,16,4096] array (leading dimensions permuted, in and out)",
+     lambda hk, t, n: case_rmsnorm_permuted(hk, t, n, "fwd")),
+    ("next: rmsnorm bwd bf16 on a [16,2048,4096] view of a [2048,16,4096] array (leading dimensions permuted, in and out)",
+     lambda hk, t, n: case_rmsnorm_permuted(hk, t, n, "bwd")),
+    ("next: softmax fwd bf16 on a [4,32,2048,2048] view of a [4,2048,32,2048] array (leading dimensions permuted, in and out)",
+     lambda hk, t, n: case_softmax_permuted(hk, t, 2, "fwd")),
+    ("next: softmax bwd bf16 on a [4,32,2048,2048] view of a [4,2048,32,2048] array (leading dimensions permuted, in and out)",
+     lambda hk, t, n: case_softmax_permuted(hk, t, 2, "bwd")),
     ("next: reduce max axis0 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (0,), "max")),
     ("next: reduce max axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "max")),
     ("next: reduce prod axis1 bf16 [32768x4096]", lambda hk, t, n: case_reduce(hk, t, n, (1,), "prod")),

@@ -206,30 +206,47 @@ __device__ __forceinline__ u32x4 ld16_stream(const void* p) {
 
 // Rows on up to three levels.  The leading dimensions of a row-major operand need not step by one constant
 // pitch: a view with permuted leading dimensions (x.permute(0, 2, 1, 3) of a [B, H, S, D] array) numbers its rows
-// r = (i2 * n1 + i1) * n0 + i0 and row r starts i0 * pitch + i1 * p1 + i2 * p2 elements from the base, the three
-// steps being whatever the view's strides are.  A dense or row-pitched array is the one-level case (n0 = rows).
-// The one-shot row kernels get the decomposition for nothing: they are launched on a three-dimensional grid whose
-// x walks the rows of the innermost level and whose y / z are i1 / i2.
+// r = (i2 * c1 + i1) * c0 + i0 and row r starts i0 * s0 + i1 * s1 + i2 * s2 elements from the base, the three
+// steps being whatever the view's strides are.  A dense or row-pitched array is the one-level case.
+//
+// A launch WALKS the levels in an order of its own choosing (plan_row_walk below puts the level with the smallest
+// steps first, so that neighbouring workgroups touch neighbouring memory whatever the view's own order is): walk
+// index (j0, j1, j2), j_k < n_k, is the row whose operands start j0 * pitch + j1 * p1 + j2 * p2 elements from their
+// bases (the operand's steps in walk order) and whose NUMBER, the index into the dense [rows] arrays next to the
+// operands (statistics, labels, losses), is j0 * rn0 + j1 * rn1 + j2 * rn2.  The one-shot row kernels get the
+// decomposition for nothing: they run on a three-dimensional grid whose x walks j0 and whose y / z are j1 / j2.
+// One level is n = {rows, 1, 1}, rn = {1, 0, 0}.
 struct LevelSteps {
-  int64_t p1, p2;   // elements between consecutive i1 / i2; the innermost step is the operand's pitch
+  int64_t p1, p2;   // elements between consecutive j1 / j2; the step of j0 is the operand's pitch
 };
-// offset of the two outer levels of this workgroup's rows, in elements
+struct RowNumbering {
+  int64_t rn0, rn1, rn2;
+};
+// offset of this workgroup's rows along the two outer walk levels, in elements
 __device__ __forceinline__ int64_t outer_level_offset(const LevelSteps& l) {
   return int64_t(blockIdx.y) * l.p1 + int64_t(blockIdx.z) * l.p2;
 }
-// number of the row (i0, blockIdx.y, blockIdx.z) in the dense [rows] arrays next to the operand (statistics,
-// labels, losses)
-__device__ __forceinline__ int64_t dense_row_index(int64_t i0, int64_t n0) {
-  return i0 + n0 * (int64_t(blockIdx.y) + int64_t(gridDim.y) * int64_t(blockIdx.z));
+// number of the row (j0, blockIdx.y, blockIdx.z)
+__device__ __forceinline__ int64_t dense_row_index(int64_t j0, const RowNumbering& rn) {
+  return j0 * rn.rn0 + int64_t(blockIdx.y) * rn.rn1 + int64_t(blockIdx.z) * rn.rn2;
 }
-// (i0, i1, i2) of row r for kernels that walk the rows themselves
-__device__ __forceinline__ int64_t level_row_offset(int64_t r, int64_t n0, int64_t n1, int64_t pitch,
-                                                    const LevelSteps& l) {
+// (j0, j1, j2) of walk index r, for kernels that walk the rows themselves
+struct RowSplit {
+  uint32_t j0, j1, j2;
+};
+__device__ __forceinline__ RowSplit split_row(int64_t r, int64_t n0, int64_t n1) {
+  RowSplit s;
   const uint32_t q = uint32_t(r) / uint32_t(n0);
-  const uint32_t i0 = uint32_t(r) - q * uint32_t(n0);
-  const uint32_t i2 = q / uint32_t(n1);
-  const uint32_t i1 = q - i2 * uint32_t(n1);
-  return int64_t(i0) * pitch + int64_t(i1) * l.p1 + int64_t(i2) * l.p2;
+  s.j0 = uint32_t(r) - q * uint32_t(n0);
+  s.j2 = q / uint32_t(n1);
+  s.j1 = q - s.j2 * uint32_t(n1);
+  return s;
+}
+__device__ __forceinline__ int64_t split_offset(const RowSplit& s, int64_t pitch, const LevelSteps& l) {
+  return int64_t(s.j0) * pitch + int64_t(s.j1) * l.p1 + int64_t(s.j2) * l.p2;
+}
+__device__ __forceinline__ int64_t split_number(const RowSplit& s, const RowNumbering& rn) {
+  return int64_t(s.j0) * rn.rn0 + int64_t(s.j1) * rn.rn1 + int64_t(s.j2) * rn.rn2;
 }
 
 // ---------------------------------------------------------------------------
@@ -535,6 +552,61 @@ inline double round_to_dtype(int dtype, double c) {
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// The order in which a launch walks the levels of its rows (see LevelSteps).  level_rows = the counts in the
+// rows' own numbering (innermost first); key = per level, the sum of the operands' steps.  Levels are taken by
+// ascending key, levels of a single row last.  on_grid: the walk rides on a grid (x = walk level 0 carries up to
+// four rows per workgroup, y / z hold at most 65535): level 0 is then the first level in that order with at least
+// eight rows, if there is one; an order whose y / z do not fit gives way to the rows' own order, then to the
+// longest level on x.  The caller checks n[1], n[2] against the grid's limits (walk_fits_grid).  perm[k] = the level
+// walked k-th.
+struct RowWalk {
+  int perm[3];
+  int64_t n[3];
+  RowNumbering rn;
+};
+inline RowWalk plan_row_walk(const int64_t level_rows[3], const int64_t key[3], bool on_grid) {
+  int order[3] = {0, 1, 2};
+  auto before = [&](int a, int b) {
+    const bool ea = level_rows[a] == 1, eb = level_rows[b] == 1;
+    if (ea != eb) return eb;
+    if (key[a] != key[b]) return key[a] < key[b];
+    return a < b;
+  };
+  for (int i = 0; i < 3; ++i)
+    for (int j = i + 1; j < 3; ++j)
+      if (before(order[j], order[i])) { const int t = order[i]; order[i] = order[j]; order[j] = t; }
+  if (on_grid) {
+    int first = -1;
+    for (int k = 0; k < 3 && first < 0; ++k)
+      if (level_rows[order[k]] >= 8) first = k;
+    if (first > 0) {
+      const int lead = order[first];
+      for (int k = first; k > 0; --k) order[k] = order[k - 1];
+      order[0] = lead;
+    }
+    auto fits = [&] { return level_rows[order[1]] <= 65535 && level_rows[order[2]] <= 65535; };
+    if (!fits()) { order[0] = 0; order[1] = 1; order[2] = 2; }
+    if (!fits()) {
+      int longest = 0;
+      for (int k = 1; k < 3; ++k)
+        if (level_rows[k] > level_rows[longest]) longest = k;
+      order[0] = longest; order[1] = longest == 0 ? 1 : 0; order[2] = longest == 2 ? 1 : 2;
+    }
+  }
+  const int64_t number[3] = {1, level_rows[0], level_rows[0] * level_rows[1]};
+  RowWalk w;
+  for (int k = 0; k < 3; ++k) { w.perm[k] = order[k]; w.n[k] = level_rows[order[k]]; }
+  w.rn = RowNumbering{number[order[0]], number[order[1]], number[order[2]]};
+  return w;
+}
+inline bool walk_fits_grid(const RowWalk& w) { return w.n[0] <= 0x7fffffffLL && w.n[1] <= 65535 && w.n[2] <= 65535; }
+// an operand's steps in walk order
+inline void walk_steps(const RowWalk& w, const int64_t steps[3], int64_t* pitch, LevelSteps* lv) {
+  *pitch = steps[w.perm[0]];
+  lv->p1 = steps[w.perm[1]];
+  lv->p2 = steps[w.perm[2]];
+}
 
 inline hipStream_t as_hip(hkStream_t s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -24,8 +24,9 @@ struct NormFwdArgs {
   void* stat;
   int64_t rows;
   int64_t x_pitch, res_pitch, y_pitch, xout_pitch;
-  // rows on several levels (see LevelSteps): n0 * n1 * n2 = rows; one level is n0 = rows, n1 = n2 = 1
+  // rows on several levels (see LevelSteps), in walk order: n0 * n1 * n2 = rows; one level is n0 = rows
   int64_t n0, n1, n2;
+  RowNumbering rn;
   LevelSteps x_lv, res_lv, y_lv, xout_lv;
   int cols;
   int nvec;
@@ -52,8 +53,10 @@ struct NormBwdArgs {
   float* part_dbeta;    // [grid, cols]
   int64_t rows;
   int64_t dy_pitch, x_pitch, dx_pitch, dxin_pitch, dres_pitch;
-  // rows on several levels (see LevelSteps); the walking kernel splits the row number itself
+  // rows on several levels (see LevelSteps), in walk order; the walking kernel splits its walk index itself
   int64_t n0, n1, n2;
+  RowNumbering rn;
+  uint32_t ws0, ws1, ws2;   // the walking kernel's row stride (its grid size) split over the walk levels
   LevelSteps dy_lv, x_lv, dx_lv, dxin_lv, dres_lv;
   int cols;
   int nvec;

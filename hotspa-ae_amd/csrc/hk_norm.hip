@@ -12,7 +12,7 @@ static int norm_fwd_dispatch(int dtype, NormFwdArgs& a, hipStream_t s, const cha
   HK_REQUIRE(a.rows <= 0x7fffffffLL && a.cols <= 0x3fffffff, HK_ERR_INVALID,
              "%s: shape [%lld, %d] too large", who, (long long)a.rows, a.cols);
   HK_REQUIRE(a.x && a.y, HK_ERR_INVALID, "%s: null input/output", who);
-  if (a.n0 == 0) { a.n0 = a.rows; a.n1 = a.n2 = 1; }   // one level
+  if (a.n0 == 0) { a.n0 = a.rows; a.n1 = a.n2 = 1; a.rn = RowNumbering{1, 0, 0}; }   // one level
   HK_REQUIRE(a.n0 == 1 || (a.x_pitch >= a.cols && a.y_pitch >= a.cols && (!a.residual || a.res_pitch >= a.cols) &&
                            (!a.x_out || a.xout_pitch >= a.cols)), HK_ERR_INVALID,
              "%s: a row pitch is smaller than the %d columns of a row", who, a.cols);
@@ -36,7 +36,7 @@ static int norm_bwd_dispatch(int dtype, NormBwdArgs& a, int mode, void* dgamma, 
              "%s: shape [%lld, %d] too large", who, (long long)a.rows, a.cols);
   HK_REQUIRE(a.dy && a.x && a.dx && a.stat, HK_ERR_INVALID, "%s: null input/output", who);
   HK_REQUIRE(mode != BWD_LN || a.mean, HK_ERR_INVALID, "%s: mean is required", who);
-  if (a.n0 == 0) { a.n0 = a.rows; a.n1 = a.n2 = 1; }   // one level
+  if (a.n0 == 0) { a.n0 = a.rows; a.n1 = a.n2 = 1; a.rn = RowNumbering{1, 0, 0}; }   // one level
   HK_REQUIRE(a.n0 == 1 || (a.dy_pitch >= a.cols && a.x_pitch >= a.cols && a.dx_pitch >= a.cols &&
                            (!a.dx_in || a.dxin_pitch >= a.cols) && (!a.dres || a.dres_pitch >= a.cols)), HK_ERR_INVALID,
              "%s: a row pitch is smaller than the %d columns of a row", who, a.cols);
@@ -52,22 +52,24 @@ static int norm_bwd_dispatch(int dtype, NormBwdArgs& a, int mode, void* dgamma, 
   }
 }
 
-// level_rows = {n0, n1, n2} of a *_strided_rows call: every count positive, the outer two within a grid's y / z
-// range, the product within the row limit.  Writes the total.
+// level_rows = {n0, n1, n2} of a *_strided_rows call: no count negative, the product within the row limit.
+// Writes the total.
 static int check_levels(const int64_t level_rows[3], int64_t* rows, const char* who) {
   HK_REQUIRE(level_rows, HK_ERR_INVALID, "%s: null level_rows", who);
   const int64_t n0 = level_rows[0], n1 = level_rows[1], n2 = level_rows[2];
   HK_REQUIRE(n0 >= 0 && n1 >= 0 && n2 >= 0, HK_ERR_INVALID, "%s: negative level count", who);
   if (n0 == 0 || n1 == 0 || n2 == 0) { *rows = 0; return HK_OK; }
-  HK_REQUIRE(n1 <= 65535 && n2 <= 65535, HK_ERR_UNSUPPORTED,
-             "%s: the two outer levels hold at most 65535 rows each (got %lld, %lld)", who, (long long)n1, (long long)n2);
   HK_REQUIRE(n0 <= 0x7fffffffLL && n0 * n1 <= 0x7fffffffLL && n0 * n1 * n2 <= 0x7fffffffLL, HK_ERR_INVALID,
              "%s: too many rows", who);
   *rows = n0 * n1 * n2;
   return HK_OK;
 }
 
-static inline LevelSteps outer_steps(const int64_t steps[3]) { return LevelSteps{steps[1], steps[2]}; }
+// per level, the sum of the steps of the operands that are there: what the walk order is chosen by
+static void add_steps(int64_t key[3], const void* operand, const int64_t steps[3]) {
+  if (operand == nullptr || steps == nullptr) return;
+  for (int k = 0; k < 3; ++k) key[k] += steps[k];
+}
 
 // Scratch memory owned by the library, for the entry point that must not
 // allocate.  The array lives in the code object's global segment, so every
@@ -123,8 +125,16 @@ int hk_layer_norm_fwd_strided_rows(int dtype, const void* x, const int64_t x_ste
              "%s: fp64 data needs fp64 statistics", who);
   NormFwdArgs a{};
   a.x = x; a.gamma = gamma; a.beta = beta; a.y = y; a.mean = mean; a.stat = stat;
-  a.x_pitch = x_steps[0]; a.y_pitch = y_steps[0]; a.x_lv = outer_steps(x_steps); a.y_lv = outer_steps(y_steps);
-  a.n0 = level_rows[0]; a.n1 = level_rows[1]; a.n2 = level_rows[2];
+  int64_t key[3] = {0, 0, 0};
+  add_steps(key, x, x_steps);
+  add_steps(key, y, y_steps);
+  const RowWalk w = plan_row_walk(level_rows, key, /*on_grid=*/true);
+  walk_steps(w, x_steps, &a.x_pitch, &a.x_lv);
+  walk_steps(w, y_steps, &a.y_pitch, &a.y_lv);
+  a.n0 = w.n[0]; a.n1 = w.n[1]; a.n2 = w.n[2]; a.rn = w.rn;
+  HK_REQUIRE(rows == 0 || walk_fits_grid(w), HK_ERR_UNSUPPORTED,
+             "%s: two of the three levels must hold at most 65535 rows each (got %lld, %lld, %lld)", who,
+             (long long)level_rows[0], (long long)level_rows[1], (long long)level_rows[2]);
   a.rows = rows; a.cols = int(cols); a.eps = eps; a.is_rms = 0; a.stat_kind = stat_kind;
   a.stats_f32 = (stats_dtype == HK_FLOAT32 && dtype != HK_FLOAT64) ? 1 : 0;
   return norm_fwd_dispatch(dtype, a, as_hip(stream), who);
@@ -197,9 +207,19 @@ int hk_layer_norm_bwd_strided_rows(int dtype, const void* dy, const int64_t dy_s
              "%s: fp64 data needs fp64 statistics", who);
   NormBwdArgs a{};
   a.dy = dy; a.x = x_or_y; a.gamma = gamma; a.beta = beta; a.mean = mean; a.stat = stat;
-  a.dy_pitch = dy_steps[0]; a.x_pitch = x_steps[0]; a.dx_pitch = dx_steps[0];
-  a.dy_lv = outer_steps(dy_steps); a.x_lv = outer_steps(x_steps); a.dx_lv = outer_steps(dx_steps);
-  a.n0 = level_rows[0]; a.n1 = level_rows[1]; a.n2 = level_rows[2];
+  int64_t key[3] = {0, 0, 0};
+  add_steps(key, dy, dy_steps);
+  add_steps(key, x_or_y, x_steps);
+  add_steps(key, dx, dx_steps);
+  // the register kernel walks the rows itself; its fallback rides on a grid, whose limits the levels' own order meets
+  const RowWalk w = plan_row_walk(level_rows, key, /*on_grid=*/true);
+  walk_steps(w, dy_steps, &a.dy_pitch, &a.dy_lv);
+  walk_steps(w, x_steps, &a.x_pitch, &a.x_lv);
+  walk_steps(w, dx_steps, &a.dx_pitch, &a.dx_lv);
+  a.n0 = w.n[0]; a.n1 = w.n[1]; a.n2 = w.n[2]; a.rn = w.rn;
+  HK_REQUIRE(rows == 0 || walk_fits_grid(w), HK_ERR_UNSUPPORTED,
+             "%s: two of the three levels must hold at most 65535 rows each (got %lld, %lld, %lld)", who,
+             (long long)level_rows[0], (long long)level_rows[1], (long long)level_rows[2]);
   a.dx = dx; a.rows = rows; a.cols = int(cols); a.eps = eps; a.stat_kind = stat_kind;
   a.stats_f32 = (stats_dtype == HK_FLOAT32 && dtype != HK_FLOAT64) ? 1 : 0;
   a.clamp_gamma = clamp_gamma;
@@ -266,10 +286,20 @@ int hk_dropout_add_ln_fwd_strided_rows(int itype, int rtype, int wtype, const vo
   HK_REQUIRE(cols >= 0 && cols <= 0x3fffffff, HK_ERR_INVALID, "%s: bad cols", who);
   NormFwdArgs a{};
   a.x = x0; a.residual = residual; a.gamma = gamma; a.beta = beta; a.y = z; a.x_out = x_out;
-  a.x_pitch = x0_steps[0]; a.res_pitch = residual_steps[0]; a.y_pitch = z_steps[0]; a.xout_pitch = x_out_steps[0];
-  a.x_lv = outer_steps(x0_steps); a.res_lv = outer_steps(residual_steps); a.y_lv = outer_steps(z_steps);
-  a.xout_lv = outer_steps(x_out_steps);
-  a.n0 = level_rows[0]; a.n1 = level_rows[1]; a.n2 = level_rows[2];
+  int64_t key[3] = {0, 0, 0};
+  add_steps(key, x0, x0_steps);
+  add_steps(key, residual, residual_steps);
+  add_steps(key, z, z_steps);
+  add_steps(key, x_out, x_out_steps);
+  const RowWalk w = plan_row_walk(level_rows, key, /*on_grid=*/true);
+  walk_steps(w, x0_steps, &a.x_pitch, &a.x_lv);
+  walk_steps(w, residual_steps, &a.res_pitch, &a.res_lv);
+  walk_steps(w, z_steps, &a.y_pitch, &a.y_lv);
+  walk_steps(w, x_out_steps, &a.xout_pitch, &a.xout_lv);
+  a.n0 = w.n[0]; a.n1 = w.n[1]; a.n2 = w.n[2]; a.rn = w.rn;
+  HK_REQUIRE(rows == 0 || walk_fits_grid(w), HK_ERR_UNSUPPORTED,
+             "%s: two of the three levels must hold at most 65535 rows each (got %lld, %lld, %lld)", who,
+             (long long)level_rows[0], (long long)level_rows[1], (long long)level_rows[2]);
   a.mean = mu; a.stat = rsigma; a.rows = rows; a.cols = int(cols); a.eps = eps;
   a.is_rms = is_rms_norm ? 1 : 0; a.stat_kind = HK_STAT_RSTD; a.stats_f32 = 1;
   return norm_fwd_dispatch(itype, a, as_hip(stream), who);
@@ -298,11 +328,22 @@ int hk_dropout_add_ln_bwd_strided_rows(int itype, int rtype, int wtype, const vo
   HK_REQUIRE(cols >= 0 && cols <= 0x3fffffff, HK_ERR_INVALID, "%s: bad cols", who);
   NormBwdArgs a{};
   a.dy = dz; a.x = x; a.gamma = gamma; a.mean = mu; a.stat = rsigma; a.dx_in = dx_in;
-  a.dy_pitch = dz_steps[0]; a.x_pitch = x_steps[0]; a.dx_pitch = dx0_steps[0]; a.dxin_pitch = dx_in_steps[0];
-  a.dres_pitch = dresidual_steps[0];
-  a.dy_lv = outer_steps(dz_steps); a.x_lv = outer_steps(x_steps); a.dx_lv = outer_steps(dx0_steps);
-  a.dxin_lv = outer_steps(dx_in_steps); a.dres_lv = outer_steps(dresidual_steps);
-  a.n0 = level_rows[0]; a.n1 = level_rows[1]; a.n2 = level_rows[2];
+  int64_t key[3] = {0, 0, 0};
+  add_steps(key, dz, dz_steps);
+  add_steps(key, dx_in, dx_in_steps);
+  add_steps(key, x, x_steps);
+  add_steps(key, dx0, dx0_steps);
+  add_steps(key, dresidual, dresidual_steps);
+  const RowWalk w = plan_row_walk(level_rows, key, /*on_grid=*/true);
+  walk_steps(w, dz_steps, &a.dy_pitch, &a.dy_lv);
+  walk_steps(w, x_steps, &a.x_pitch, &a.x_lv);
+  walk_steps(w, dx0_steps, &a.dx_pitch, &a.dx_lv);
+  walk_steps(w, dx_in_steps, &a.dxin_pitch, &a.dxin_lv);
+  walk_steps(w, dresidual_steps, &a.dres_pitch, &a.dres_lv);
+  a.n0 = w.n[0]; a.n1 = w.n[1]; a.n2 = w.n[2]; a.rn = w.rn;
+  HK_REQUIRE(rows == 0 || walk_fits_grid(w), HK_ERR_UNSUPPORTED,
+             "%s: two of the three levels must hold at most 65535 rows each (got %lld, %lld, %lld)", who,
+             (long long)level_rows[0], (long long)level_rows[1], (long long)level_rows[2]);
   a.dx = dx0; a.dres = dresidual; a.rows = rows; a.cols = int(cols); a.eps = 0.f;
   a.stat_kind = HK_STAT_RSTD; a.stats_f32 = 1; a.clamp_gamma = 0;
   return norm_bwd_dispatch(itype, a, is_rms_norm ? BWD_RMS : BWD_LN, dgamma, dbeta, workspace, workspace_bytes,

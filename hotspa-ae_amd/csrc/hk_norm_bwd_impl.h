@@ -45,10 +45,17 @@ __device__ __forceinline__ float clamp_by_magnitude(float g, float eps) {
 // arithmetic otherwise, whose merge costs one register move per live value per row);
 // without EXTRA, CLAMP says at compile time whether gamma enters dx clamped (the fused
 // LayerNorm's backward does that in both of its modes, the plain one never).
+//
+// LEVELS (FIXED instances without optional operands only): the rows lie on several levels (see LevelSteps).  The
+// loads are issued in strictly increasing row order, one grid size apart, so the walk index of the next row to
+// issue is kept as a running (j0, j1, j2) in scalar registers and advanced by the split grid size with two
+// carries: no division in the loop, nothing on the vector unit.  The general instance takes levels too, with
+// optional operands, by splitting each row number with two divisions.
 template <typename T, int NV, int MODE, int PF, bool EXACT, bool STATS_F32, bool EXTRA, int MAXT, bool FIXED,
-          bool CLAMP>
+          bool CLAMP, bool LEVELS = false>
 __global__ __launch_bounds__(MAXT)
 void norm_bwd_kernel(NormBwdArgs a) {
+  static_assert(!LEVELS || (FIXED && !EXTRA && EXACT), "the running walk index is built for the lean instances");
   constexpr int VEC = VecIO<T>::N;
   constexpr int NE = NV * VEC;
   constexpr int KS = (MODE == BWD_RMS) ? 1 : 2;   // row sums to reduce: RMSNorm has no mean term
@@ -105,19 +112,47 @@ void norm_bwd_kernel(NormBwdArgs a) {
   StatT nmu[PF], nsv[PF];
   const StatT* meanp = static_cast<const StatT*>(a.mean);
   const StatT* statp = static_cast<const StatT*>(a.stat);
+  // LEVELS: walk index of the next row to issue, and where each slot's dx row goes
+  [[maybe_unused]] uint32_t wj0 = 0, wj1 = 0, wj2 = 0;
+  [[maybe_unused]] int64_t dxo[PF];
+  if constexpr (LEVELS) {
+    const RowSplit first = split_row(int64_t(blockIdx.x), a.n0, a.n1);
+    wj0 = __builtin_amdgcn_readfirstlane(first.j0);
+    wj1 = __builtin_amdgcn_readfirstlane(first.j1);
+    wj2 = __builtin_amdgcn_readfirstlane(first.j2);
+  }
   // loads of row r into slot d; r past the end re-reads the last row (its results are never used)
   auto issue = [&](auto slot, int64_t r) {
     constexpr int d = decltype(slot)::value;
     const int64_t rc = r < last_row ? r : last_row;
-    if constexpr (MODE == BWD_LN) nmu[d] = meanp[rc];
-    nsv[d] = statp[rc];
-    int64_t xo = rc * a.x_pitch, dyo = rc * a.dy_pitch;
+    int64_t xo = rc * a.x_pitch, dyo = rc * a.dy_pitch, number = rc;
+    if constexpr (LEVELS) {
+      // a row past the end reads row 0 instead (any row will do)
+      const bool ok = r <= last_row;
+      const RowSplit sp{ok ? wj0 : 0u, ok ? wj1 : 0u, ok ? wj2 : 0u};
+      xo = split_offset(sp, a.x_pitch, a.x_lv);
+      dyo = split_offset(sp, a.dy_pitch, a.dy_lv);
+      number = split_number(sp, a.rn);
+      dxo[d] = split_offset(sp, a.dx_pitch, a.dx_lv);
+      // the next row to issue lies one grid size further on
+      wj0 += a.ws0;
+      uint32_t carry = wj0 >= uint32_t(a.n0) ? 1u : 0u;
+      wj0 -= carry ? uint32_t(a.n0) : 0u;
+      wj1 += a.ws1 + carry;
+      carry = wj1 >= uint32_t(a.n1) ? 1u : 0u;
+      wj1 -= carry ? uint32_t(a.n1) : 0u;
+      wj2 += a.ws2 + carry;
+    }
     if constexpr (EXTRA) {
       if (a.n0 != a.rows) {   // rows on several levels: uniform
-        xo = level_row_offset(rc, a.n0, a.n1, a.x_pitch, a.x_lv);
-        dyo = level_row_offset(rc, a.n0, a.n1, a.dy_pitch, a.dy_lv);
+        const RowSplit sp = split_row(rc, a.n0, a.n1);
+        xo = split_offset(sp, a.x_pitch, a.x_lv);
+        dyo = split_offset(sp, a.dy_pitch, a.dy_lv);
+        number = split_number(sp, a.rn);
       }
     }
+    if constexpr (MODE == BWD_LN) nmu[d] = meanp[number];
+    nsv[d] = statp[number];
     const T* xr = static_cast<const T*>(a.x) + xo;
     const T* dyr = static_cast<const T*>(a.dy) + dyo;
 #pragma unroll
@@ -151,6 +186,8 @@ void norm_bwd_kernel(NormBwdArgs a) {
     const float sv = Cvt<StatT>::to_float(nsv[d]);
     // RMSNorm keeps the inverse root mean square, never a variance
     const float rs = (MODE != BWD_RMS && a.stat_kind == HK_STAT_VAR) ? 1.0f / sqrtf(sv + a.eps) : sv;
+    [[maybe_unused]] int64_t dx_offset = 0;
+    if constexpr (LEVELS) dx_offset = dxo[d];   // the refill below reuses the slot
     // the slot is free again: refill it with the row PF steps ahead
     issue(slot, row + int64_t(PF) * stride);
 
@@ -205,19 +242,19 @@ void norm_bwd_kernel(NormBwdArgs a) {
         rc1 = (MODE == BWD_RMS) ? 0.f : s.v[0] * a.inv_cols;
         k3 = rs * rs * s_prod * a.inv_cols;
       }
-      T* dxr = static_cast<T*>(a.dx) + row * a.dx_pitch;
+      T* dxr = static_cast<T*>(a.dx) + (LEVELS ? dx_offset : row * a.dx_pitch);
       [[maybe_unused]] T* drr = nullptr;
       [[maybe_unused]] const T* dir = nullptr;
       if constexpr (EXTRA) {
         const bool levels = a.n0 != a.rows;   // uniform
-        if (levels) dxr = static_cast<T*>(a.dx) + level_row_offset(row, a.n0, a.n1, a.dx_pitch, a.dx_lv);
-        if (a.dres) {
-          drr = static_cast<T*>(a.dres) +
-                (levels ? level_row_offset(row, a.n0, a.n1, a.dres_pitch, a.dres_lv) : row * a.dres_pitch);
+        RowSplit sp{};
+        if (levels) {
+          sp = split_row(row, a.n0, a.n1);
+          dxr = static_cast<T*>(a.dx) + split_offset(sp, a.dx_pitch, a.dx_lv);
         }
+        if (a.dres) drr = static_cast<T*>(a.dres) + (levels ? split_offset(sp, a.dres_pitch, a.dres_lv) : row * a.dres_pitch);
         if (a.dx_in) {
-          dir = static_cast<const T*>(a.dx_in) +
-                (levels ? level_row_offset(row, a.n0, a.n1, a.dxin_pitch, a.dxin_lv) : row * a.dxin_pitch);
+          dir = static_cast<const T*>(a.dx_in) + (levels ? split_offset(sp, a.dxin_pitch, a.dxin_lv) : row * a.dxin_pitch);
         }
       }
 #pragma unroll
@@ -353,7 +390,7 @@ __global__ __launch_bounds__(256)
 void norm_bwd_generic_dx_kernel(NormBwdArgs a, int mode) {
   __shared__ CT lds[256];
   const int64_t i0 = blockIdx.x;                       // row within the innermost level
-  const int64_t row = dense_row_index(i0, a.n0);
+  const int64_t row = dense_row_index(i0, a.rn);
   const T* xr = static_cast<const T*>(a.x) + i0 * a.x_pitch + outer_level_offset(a.x_lv);
   const T* dyr = static_cast<const T*>(a.dy) + i0 * a.dy_pitch + outer_level_offset(a.dy_lv);
   const T* gp = static_cast<const T*>(a.gamma);
@@ -429,21 +466,26 @@ void norm_bwd_generic_cols_kernel(NormBwdArgs a, int mode, T* dgamma, T* dbeta) 
     const CT b = (bp && mode == BWD_LN_MEMEFF) ? GenericIO<T, CT>::ld(bp + c) : CT(0);
     const bool levels = a.n0 != a.rows;
     for (int64_t r = w; r < a.rows; r += 4) {
-      const int64_t dyo = levels ? level_row_offset(r, a.n0, a.n1, a.dy_pitch, a.dy_lv) : r * a.dy_pitch;
-      const int64_t xo = levels ? level_row_offset(r, a.n0, a.n1, a.x_pitch, a.x_lv) : r * a.x_pitch;
+      int64_t dyo = r * a.dy_pitch, xo = r * a.x_pitch, number = r;
+      if (levels) {
+        const RowSplit sp = split_row(r, a.n0, a.n1);
+        dyo = split_offset(sp, a.dy_pitch, a.dy_lv);
+        xo = split_offset(sp, a.x_pitch, a.x_lv);
+        number = split_number(sp, a.rn);
+      }
       const CT d = GenericIO<T, CT>::ld(static_cast<const T*>(a.dy) + dyo + c);
       const CT xv = GenericIO<T, CT>::ld(static_cast<const T*>(a.x) + xo + c);
       CT xhat;
       if (mode == BWD_LN_MEMEFF) {
         xhat = (xv - b) / kg;
       } else {
-        const CT sv = a.stats_f32 ? CT(static_cast<const float*>(a.stat)[r])
-                                  : GenericIO<T, CT>::ld(static_cast<const T*>(a.stat) + r);
+        const CT sv = a.stats_f32 ? CT(static_cast<const float*>(a.stat)[number])
+                                  : GenericIO<T, CT>::ld(static_cast<const T*>(a.stat) + number);
         const CT rs = a.stat_kind == HK_STAT_VAR ? CT(1) / sqrt(sv + CT(a.eps)) : sv;
         CT mu = 0;
         if (mode == BWD_LN)
-          mu = a.stats_f32 ? CT(static_cast<const float*>(a.mean)[r])
-                           : GenericIO<T, CT>::ld(static_cast<const T*>(a.mean) + r);
+          mu = a.stats_f32 ? CT(static_cast<const float*>(a.mean)[number])
+                           : GenericIO<T, CT>::ld(static_cast<const T*>(a.mean) + number);
         xhat = rs * (xv - mu);
       }
       sg += d * xhat;
@@ -522,25 +564,31 @@ static int launch_norm_bwd_inst(const NormBwdArgs& a, const BwdPlan& p, int pf, 
   // the kernel's "extra" instance takes the optional operands behind uniform branches, and the clamp request in
   // the modes that have no instance of their own for it
   const bool want_clamp = a.clamp_gamma != 0 && MODE != BWD_LN_MEMEFF;   // the memory-efficient mode always clamps
-  // rows on several levels go with them: that instance splits the row number itself
-  const bool extra = a.dx_in != nullptr || a.dres != nullptr || (want_clamp && MODE != BWD_LN) || a.n0 != a.rows;
   // one group that is the whole block, of exactly the bound's size: the instance with a constant group width
   const bool fixed = p.rpb == 1 && p.block == MAXT;
+  // rows on several levels: the lean fixed instances keep a running walk index; every other case splits each row
+  // number in the general instance
+  const bool levels = a.n0 != a.rows;
+  const bool optional = a.dx_in != nullptr || a.dres != nullptr || (want_clamp && MODE != BWD_LN);
+  const bool extra = optional || (levels && !(fixed && exact));
   // the deep ring exists for the plain case only: full rows, no optional operands
   if (!exact || extra) pf = 1;
-#define HK_BWD_LAUNCH(P, E, F, X, FX, C) \
-  HK_LAUNCH((norm_bwd_kernel<T, NV, MODE, P, E, F, X, MAXT, FX, C>), grid, block, p.lds_bytes, s, a)
-#define HK_BWD_LEAN(P, F, FX)                                               \
+#define HK_BWD_LAUNCH_L(P, E, F, X, FX, C, L) \
+  HK_LAUNCH((norm_bwd_kernel<T, NV, MODE, P, E, F, X, MAXT, FX, C, L>), grid, block, p.lds_bytes, s, a)
+#define HK_BWD_LAUNCH(P, E, F, X, FX, C) HK_BWD_LAUNCH_L(P, E, F, X, FX, C, false)
+#define HK_BWD_LEAN_L(P, F, FX, L)                                          \
   do {                                                                      \
     if constexpr (MODE == BWD_LN) {                                         \
-      if (want_clamp) HK_BWD_LAUNCH(P, true, F, false, FX, true); else HK_BWD_LAUNCH(P, true, F, false, FX, false); \
+      if (want_clamp) HK_BWD_LAUNCH_L(P, true, F, false, FX, true, L); else HK_BWD_LAUNCH_L(P, true, F, false, FX, false, L); \
     } else {                                                                \
-      HK_BWD_LAUNCH(P, true, F, false, FX, false);                          \
+      HK_BWD_LAUNCH_L(P, true, F, false, FX, false, L);                     \
     }                                                                       \
   } while (0)
+#define HK_BWD_LEAN(P, F, FX) HK_BWD_LEAN_L(P, F, FX, false)
 #define HK_BWD_F(F)                                                         \
   do {                                                                      \
-    if (exact && !extra && fixed) { if (pf >= 2) HK_BWD_LEAN(2, F, true); else HK_BWD_LEAN(1, F, true); } \
+    if (exact && !extra && fixed && levels) { if (pf >= 2) HK_BWD_LEAN_L(2, F, true, true); else HK_BWD_LEAN_L(1, F, true, true); } \
+    else if (exact && !extra && fixed) { if (pf >= 2) HK_BWD_LEAN(2, F, true); else HK_BWD_LEAN(1, F, true); } \
     else if (exact && !extra) { if (pf >= 2) HK_BWD_LEAN(2, F, false); else HK_BWD_LEAN(1, F, false); } \
     else if (exact) HK_BWD_LAUNCH(1, true, F, true, false, false);          \
     else if (!extra && !want_clamp) HK_BWD_LAUNCH(1, false, F, false, false, false); \
@@ -553,7 +601,9 @@ static int launch_norm_bwd_inst(const NormBwdArgs& a, const BwdPlan& p, int pf, 
   }
 #undef HK_BWD_F
 #undef HK_BWD_LEAN
+#undef HK_BWD_LEAN_L
 #undef HK_BWD_LAUNCH
+#undef HK_BWD_LAUNCH_L
   return HK_OK;
 }
 
@@ -624,6 +674,14 @@ int norm_bwd_typed(NormBwdArgs a, int mode, void* dgamma, void* dbeta, void* ws,
   }
   a.tpr = p.tpr;
   a.nvec = a.cols / VecIO<T>::N;
+  {
+    // the walking kernel's row stride, split over the walk levels (used by the instances with a running walk index)
+    const uint64_t stride = uint64_t(p.grid) * uint64_t(p.rpb);
+    const uint64_t q = stride / uint64_t(a.n0);
+    a.ws0 = uint32_t(stride - q * uint64_t(a.n0));
+    a.ws1 = uint32_t(q % uint64_t(a.n1));
+    a.ws2 = uint32_t(q / uint64_t(a.n1));
+  }
   int rc;
   switch (mode) {
     case BWD_LN: rc = launch_norm_bwd_nv<T, BWD_LN>(a, p, s); break;

@@ -42,7 +42,7 @@ void norm_fwd_kernel(NormFwdArgs a) {
   const int64_t row0 = WAVE_ROW
       ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index()
       : int64_t(blockIdx.x) * R;
-  // row0 counts within the innermost level of rows; blockIdx.y / z are the outer levels (one level: both 0)
+  // row0 counts along the first walk level; blockIdx.y / z are the other two (one level: both 0)
   if (WAVE_ROW && row0 >= a.n0) return;  // wave-uniform; no block barrier in this mode
   const int nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
   auto off = [&](int i) { return uint32_t(i * tpr + t) * 16u; };   // vector i of thread t, in bytes from the row's start
@@ -189,7 +189,7 @@ void norm_fwd_kernel(NormFwdArgs a) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       if (live[r]) {
-        const int64_t dense = dense_row_index(rowi[r], a.n0);
+        const int64_t dense = dense_row_index(rowi[r], a.rn);
         store_stat<T>(a.mean, dense, mu[r], a.stats_f32);
         store_stat<T>(a.stat, dense, a.stat_kind == HK_STAT_VAR ? var[r] : rs[r], a.stats_f32);
       }
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256)
 void norm_fwd_generic_kernel(NormFwdArgs a) {
   __shared__ CT lds[256];
   const int64_t i0 = blockIdx.x;                       // row within the innermost level
-  const int64_t row = dense_row_index(i0, a.n0);
+  const int64_t row = dense_row_index(i0, a.rn);
   const T* xr = static_cast<const T*>(a.x) + i0 * a.x_pitch + outer_level_offset(a.x_lv);
   const T* rr = a.residual ? static_cast<const T*>(a.residual) + i0 * a.res_pitch + outer_level_offset(a.res_lv)
                            : nullptr;

@@ -29,6 +29,7 @@ struct SceArgs {
   // rows on several levels (see LevelSteps); one level: n0 = rows.  labels, losses, per-row gradients and
   // statistics are dense [rows] arrays and take the row's number
   int64_t n0, n1, n2;
+  RowNumbering rn;
   LevelSteps x_lv, lab_lv, out_lv;
   int cols;
   int nvec;
@@ -60,7 +61,7 @@ __device__ __forceinline__ void row_coords(const SceArgs& a, int& tpr, int& t, i
   tpr = WAVE_ROW ? kWave : int(blockDim.x);
   t = WAVE_ROW ? int(threadIdx.x & 63) : int(threadIdx.x);
   i0 = WAVE_ROW ? int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_index() : int64_t(blockIdx.x);
-  row = dense_row_index(i0, a.n0);
+  row = dense_row_index(i0, a.rn);
   nwaves = WAVE_ROW ? 1 : int(blockDim.x >> 6);
 }
 
@@ -345,7 +346,7 @@ __global__ __launch_bounds__(256)
 void sce_generic_kernel(SceArgs a) {
   __shared__ CT lds[256];
   const int64_t i0 = blockIdx.x;
-  const int64_t row = dense_row_index(i0, a.n0);
+  const int64_t row = dense_row_index(i0, a.rn);
   const int64_t cols = a.cols;
   const T* xr = static_cast<const T*>(a.logits) + i0 * a.x_pitch + outer_level_offset(a.x_lv);
   int64_t label = 0;
@@ -516,7 +517,7 @@ static int sce_dispatch(int dtype, SceArgs& a, hipStream_t s, const char* who) {
   if (a.x_pitch == 0) a.x_pitch = a.cols;
   if (a.lab_pitch == 0) a.lab_pitch = a.cols;
   if (a.out_pitch == 0) a.out_pitch = a.cols;
-  if (a.n0 == 0) { a.n0 = a.rows; a.n1 = a.n2 = 1; }   // one level
+  if (a.n0 == 0) { a.n0 = a.rows; a.n1 = a.n2 = 1; a.rn = RowNumbering{1, 0, 0}; }   // one level
   HK_REQUIRE(a.n0 == 1 || (a.x_pitch >= a.cols && a.lab_pitch >= a.cols && a.out_pitch >= a.cols), HK_ERR_INVALID,
              "%s: a row pitch is smaller than the %d columns of a row", who, a.cols);
   switch (dtype) {
@@ -548,18 +549,26 @@ int hk_sce_sparse_fwd(int dtype, const void* logits, const int64_t* labels, void
   return sce_dispatch<0>(dtype, a, as_hip(stream), "hk_sce_sparse_fwd");
 }
 
-static int sce_levels(SceArgs& a, const int64_t level_rows[3], const char* who) {
+// logits_steps / out_steps (out_steps may be null): the operands' steps in the rows' own order
+static int sce_levels(SceArgs& a, const int64_t level_rows[3], const int64_t* logits_steps, const int64_t* out_steps,
+                      const char* who) {
   HK_REQUIRE(level_rows, HK_ERR_INVALID, "%s: null level_rows", who);
   const int64_t n0 = level_rows[0], n1 = level_rows[1], n2 = level_rows[2];
   HK_REQUIRE(n0 >= 0 && n1 >= 0 && n2 >= 0, HK_ERR_INVALID, "%s: negative level count", who);
   a.rows = 0;
   if (n0 == 0 || n1 == 0 || n2 == 0) return HK_OK;
-  HK_REQUIRE(n1 <= 65535 && n2 <= 65535, HK_ERR_UNSUPPORTED,
-             "%s: the two outer levels hold at most 65535 rows each (got %lld, %lld)", who, (long long)n1, (long long)n2);
   HK_REQUIRE(n0 <= 0x7fffffffLL && n0 * n1 <= 0x7fffffffLL && n0 * n1 * n2 <= 0x7fffffffLL, HK_ERR_INVALID,
              "%s: too many rows", who);
   a.rows = n0 * n1 * n2;
-  a.n0 = n0; a.n1 = n1; a.n2 = n2;
+  int64_t key[3] = {0, 0, 0};
+  for (int k = 0; k < 3; ++k) key[k] = logits_steps[k] + (out_steps ? out_steps[k] : 0);
+  const RowWalk w = plan_row_walk(level_rows, key, /*on_grid=*/true);
+  HK_REQUIRE(walk_fits_grid(w), HK_ERR_UNSUPPORTED,
+             "%s: two of the three levels must hold at most 65535 rows each (got %lld, %lld, %lld)", who,
+             (long long)n0, (long long)n1, (long long)n2);
+  a.n0 = w.n[0]; a.n1 = w.n[1]; a.n2 = w.n[2]; a.rn = w.rn;
+  walk_steps(w, logits_steps, &a.x_pitch, &a.x_lv);
+  if (out_steps) walk_steps(w, out_steps, &a.out_pitch, &a.out_lv);
   return HK_OK;
 }
 
@@ -570,10 +579,9 @@ int hk_sce_sparse_fwd_strided_rows(int dtype, const void* logits, const int64_t 
   HK_REQUIRE(logits_steps, HK_ERR_INVALID, "%s: null steps", who);
   HK_REQUIRE(cols >= 0 && cols <= 0x3fffffff, HK_ERR_INVALID, "%s: bad cols", who);
   SceArgs a{};
-  int rc = sce_levels(a, level_rows, who);
+  int rc = sce_levels(a, level_rows, logits_steps, nullptr, who);
   if (rc != HK_OK) return rc;
   a.logits = logits; a.labels = labels; a.out = loss; a.cols = int(cols);
-  a.x_pitch = logits_steps[0]; a.x_lv = LevelSteps{logits_steps[1], logits_steps[2]};
   a.ignored_index = ignored_index;
   return sce_dispatch<0>(dtype, a, as_hip(stream), who);
 }
@@ -586,11 +594,9 @@ int hk_sce_sparse_bwd_strided_rows(int dtype, const void* logits, const int64_t 
   HK_REQUIRE(logits_steps && dlogits_steps, HK_ERR_INVALID, "%s: null steps", who);
   HK_REQUIRE(cols >= 0 && cols <= 0x3fffffff, HK_ERR_INVALID, "%s: bad cols", who);
   SceArgs a{};
-  int rc = sce_levels(a, level_rows, who);
+  int rc = sce_levels(a, level_rows, logits_steps, dlogits_steps, who);
   if (rc != HK_OK) return rc;
   a.logits = logits; a.labels = labels; a.grad_loss = grad_loss; a.out = dlogits; a.cols = int(cols);
-  a.x_pitch = logits_steps[0]; a.x_lv = LevelSteps{logits_steps[1], logits_steps[2]};
-  a.out_pitch = dlogits_steps[0]; a.out_lv = LevelSteps{dlogits_steps[1], dlogits_steps[2]};
   a.ignored_index = ignored_index;
   return sce_dispatch<1>(dtype, a, as_hip(stream), who);
 }

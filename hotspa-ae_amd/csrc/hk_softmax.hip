@@ -20,7 +20,7 @@ struct SoftmaxArgs {
   void* out;        // forward: y;      backward: dx
   int64_t rows;
   int64_t x_pitch, dy_pitch, out_pitch;   // elements between row starts (== cols for a dense array)
-  int64_t n0, n1, n2;                     // rows on several levels (see LevelSteps); one level: n0 = rows
+  int64_t n0, n1, n2;                     // rows on several levels in walk order (see LevelSteps); one level: n0 = rows
   LevelSteps x_lv, dy_lv, out_lv;
   int cols;
   int nvec;
@@ -364,7 +364,8 @@ static int softmax_strided_typed(const void* x, const void* dy, void* out, int64
 // x_pitch / dy_pitch / out_pitch: elements between the starts of consecutive rows when inner == 1 (0: dense, the
 // row's own length); a dimension other than the last (inner > 1) only exists for dense arrays.
 struct SoftmaxLevels {
-  int64_t n0, n1, n2;
+  int64_t n0, n1, n2;          // in walk order
+  int64_t x_pitch, dy_pitch, out_pitch;
   LevelSteps x, dy, out;
 };
 
@@ -440,15 +441,21 @@ static int softmax_levels(const int64_t level_rows[3], const int64_t* x_steps, c
   HK_REQUIRE(n0 >= 0 && n1 >= 0 && n2 >= 0, HK_ERR_INVALID, "%s: negative level count", who);
   *rows = 0;
   if (n0 == 0 || n1 == 0 || n2 == 0) return HK_OK;
-  HK_REQUIRE(n1 <= 65535 && n2 <= 65535, HK_ERR_UNSUPPORTED,
-             "%s: the two outer levels hold at most 65535 rows each (got %lld, %lld)", who, (long long)n1, (long long)n2);
   HK_REQUIRE(n0 <= 0x7fffffffLL && n0 * n1 <= 0x7fffffffLL && n0 * n1 * n2 <= 0x7fffffffLL, HK_ERR_INVALID,
              "%s: too many rows", who);
   *rows = n0 * n1 * n2;
-  lv->n0 = n0; lv->n1 = n1; lv->n2 = n2;
-  lv->x = LevelSteps{x_steps[1], x_steps[2]};
-  lv->out = LevelSteps{out_steps[1], out_steps[2]};
-  lv->dy = dy_steps ? LevelSteps{dy_steps[1], dy_steps[2]} : LevelSteps{0, 0};
+  int64_t key[3] = {0, 0, 0};
+  for (int k = 0; k < 3; ++k) key[k] = x_steps[k] + out_steps[k] + (dy_steps ? dy_steps[k] : 0);
+  const RowWalk w = plan_row_walk(level_rows, key, /*on_grid=*/true);
+  HK_REQUIRE(walk_fits_grid(w), HK_ERR_UNSUPPORTED,
+             "%s: two of the three levels must hold at most 65535 rows each (got %lld, %lld, %lld)", who,
+             (long long)n0, (long long)n1, (long long)n2);
+  lv->n0 = w.n[0]; lv->n1 = w.n[1]; lv->n2 = w.n[2];
+  walk_steps(w, x_steps, &lv->x_pitch, &lv->x);
+  walk_steps(w, out_steps, &lv->out_pitch, &lv->out);
+  lv->dy_pitch = lv->x_pitch;
+  lv->dy = lv->x;
+  if (dy_steps) walk_steps(w, dy_steps, &lv->dy_pitch, &lv->dy);
   return HK_OK;
 }
 
@@ -459,7 +466,7 @@ int hk_softmax_fwd_strided_rows(int dtype, const void* x, const int64_t x_steps[
   int64_t rows = 0;
   int rc = softmax_levels(level_rows, x_steps, nullptr, y_steps, &lv, &rows, who);
   if (rc != HK_OK || rows == 0) return rc;
-  return softmax_dispatch<false>(dtype, x, nullptr, y, rows, cols, 1, x_steps[0], x_steps[0], y_steps[0],
+  return softmax_dispatch<false>(dtype, x, nullptr, y, rows, cols, 1, lv.x_pitch, lv.dy_pitch, lv.out_pitch,
                                  as_hip(stream), who, &lv);
 }
 
@@ -472,7 +479,7 @@ int hk_softmax_bwd_strided_rows(int dtype, const void* y, const int64_t y_steps[
   int64_t rows = 0;
   int rc = softmax_levels(level_rows, y_steps, dy_steps, dx_steps, &lv, &rows, who);
   if (rc != HK_OK || rows == 0) return rc;
-  return softmax_dispatch<true>(dtype, y, dy, dx, rows, cols, 1, y_steps[0], dy_steps[0], dx_steps[0],
+  return softmax_dispatch<true>(dtype, y, dy, dx, rows, cols, 1, lv.x_pitch, lv.dy_pitch, lv.out_pitch,
                                 as_hip(stream), who, &lv);
 }
 

@@ -98,9 +98,9 @@ class RowOutput {
 // the base; the kernels take that as it is, so such an operand is read / written in place where the reference
 // walks it through its OffsetCalculator (hetu/impl/utils/offset_calculator.cuh:16-68).  Leading dimensions are
 // merged where they step together in EVERY operand of the call, since all operands share one numbering of the
-// rows.  What does not fit (trailing dimensions that are not dense, more than three levels, more than 65535 rows
-// on an outer level) falls back operand by operand: an input is gathered into a dense copy, an output is written
-// dense into pool memory and laid over its strides by Commit().
+// rows.  What does not fit (trailing dimensions that are not dense, more than three levels) falls back operand
+// by operand: an input is gathered into a dense copy, an output is written dense into pool memory and laid over
+// its strides by Commit().
 class RowPlan {
  public:
   struct Slot {
@@ -197,8 +197,7 @@ class RowPlan {
                                 stream_.stream_index());
     }
   }
-  // merges the leading dimensions over all operands; false when more than three levels remain or an outer
-  // level is too long for a grid's y / z
+  // merges the leading dimensions over all operands; false when more than three levels remain
   bool JointLevels() {
     const Slot* ref = nullptr;
     for (int k = 0; k < count_; ++k)
@@ -226,7 +225,6 @@ class RowPlan {
         if (slots_[k].defined()) steps[k][levels] = slots_[k].array->stride(i);
       ++levels;
     }
-    if (counts[1] > 65535 || counts[2] > 65535) return false;
     for (int j = 0; j < 3; ++j) level_rows_[j] = counts[j];
     for (int k = 0; k < count_; ++k)
       for (int j = 0; j < 3; ++j) slots_[k].steps[j] = steps[k][j];

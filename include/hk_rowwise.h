@@ -178,9 +178,10 @@ HK_API int hk_layer_norm_fwd_pitched(int dtype, const void* x, int64_t x_pitch, 
  * from its base, every operand with its own steps (the strides of the view's leading dimensions, merged where
  * neighbours step together; a dense operand is {cols, level_rows[0] * cols, level_rows[0] * level_rows[1] * cols});
  * mean / stat stay dense [rows] arrays indexed by r.  The last dimension must have unit stride.  The row kernels
- * run on a three-dimensional grid whose y / z are i1 / i2, so such a view is read and written IN PLACE with the
- * 128-bit kernels (steps that are whole 16-byte vectors), no gather or scatter pass: the traffic is the dense
- * call's.  level_rows[1], level_rows[2] <= 65535 (HK_ERR_UNSUPPORTED beyond; the caller then gathers).
+ * run on a three-dimensional grid, one level per grid dimension, so such a view is read and written IN PLACE with
+ * the 128-bit kernels (steps that are whole 16-byte vectors), no gather or scatter pass: the traffic is the dense
+ * call's.  The launch walks the levels in the order of their steps, smallest first (neighbouring workgroups then
+ * touch neighbouring memory whatever order the view numbers its rows in); results do not depend on that order.
  * Replaces, for such views, the per-element OffsetCalculator of the reference
  * (hetu/impl/utils/offset_calculator.cuh:16-68, .cu:31-65), on which its LayerNorm / Softmax operators run
  * because they accept non-contiguous inputs (hetu/graph/ops/LayerNorm.h:78-80, Softmax.h:52-54). */

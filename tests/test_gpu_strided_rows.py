@@ -17,7 +17,9 @@ SENTINEL = 12288.0          # exactly representable in bf16
 #   [B, H, S, D] -> [B, S, H, D]: three levels;  [S, H, D] -> [H, S, D]: two levels;
 #   [A, B, C, D] -> [C, B, A, D]: three levels, all reversed;  row counts that are odd and one that is 1
 VIEWS = [((2, 4, 6, 1024), (0, 2, 1)), ((5, 3, 4096), (1, 0)), ((3, 2, 5, 512), (2, 1, 0)), ((1, 7, 3, 2048), (0, 2, 1)),
-         ((2, 3, 1, 5120), (1, 0, 2)), ((4, 33, 256), (1, 0)), ((2, 2, 3, 264), (0, 2, 1))]
+         ((2, 3, 1, 5120), (1, 0, 2)), ((4, 33, 256), (1, 0)), ((2, 2, 3, 264), (0, 2, 1)),
+         # more rows than the walking backward kernel has workgroups times ring slots: its steady loop and its tail
+         ((40, 33, 4096), (1, 0)), ((3, 7, 61, 2048), (0, 2, 1))]
 
 
 def _view(values, perm, dt, dev, pad=0):
@@ -206,14 +208,22 @@ def test_sparse_cross_entropy_on_permuted_views(hk, cuda, dt, case):
     assert bool((vd.reshape(rows, cols)[tl == -100].float() == 0).all())
 
 
-def test_levels_beyond_a_grid_are_refused(hk, cuda):
-    """The outer two levels ride on a grid's y / z: more than 65535 rows on one of them is refused by name
-    (the operator layer then gathers)."""
-    import ctypes
+def test_walk_order_does_not_change_results(hk, cuda):
+    """The launch walks the levels by ascending step; a view whose longest level has the smallest step (and one
+    whose row count on a level exceeds a grid's y / z range) still gets every row's statistics in the row's own
+    number."""
     import torch
-    x = torch.zeros(8, device=cuda)
-    steps = (ctypes.c_int64 * 3)(8, 8, 8)
-    counts = (ctypes.c_int64 * 3)(1, 70000, 1)
-    rc = hk.lib().hk_softmax_fwd_strided_rows(6, ctypes.c_void_p(x.data_ptr()), steps, ctypes.c_void_p(x.data_ptr()),
-                                              steps, counts, ctypes.c_int64(8), None)
-    assert rc == -2 and b"65535" in hk.lib().hk_last_error()
+    dt = "fp32"
+    S, B, D = 70000, 2, 64                       # stored [S, B, D], used as [B, S, D]: level 0 = S rows, 128 apart
+    x = helpers.draw(81, (B, S, D), dtype=dt)
+    sx, vx = _view(x, (1, 0), dt, cuda)
+    g = helpers.draw(82, (D,), "uniform", 0.5, 1.5, dt)
+    tg = helpers.to_torch(g, dt, cuda)
+    y = torch.empty((B, S, D), device=cuda)
+    mean, rstd = torch.empty(B * S, device=cuda), torch.empty(B * S, device=cuda)
+    hk.layer_norm_fwd(vx, tg, None, y, mean, rstd, 1e-5, stat_kind=1)
+    torch.cuda.synchronize()
+    ey, em, _, ers = oracle.layernorm_fwd(x.reshape(B * S, D), g, np.zeros(D), 1e-5)
+    helpers.assert_close(y.reshape(B * S, D), ey, dt, "y")
+    helpers.assert_close(mean, em, dt, "mean", scale=1.0)
+    helpers.assert_close(rstd, ers, dt, "rstd")

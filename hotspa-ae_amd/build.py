@@ -1,6 +1,7 @@
 """Builds the native libraries of this package in-tree.
 
   lib/libhk_rowwise.so   C-ABI device layer + HIP kernels (hipcc, gfx950)
+  lib/libhk_bench.so     the streaming yardstick bench.py measures against (hipcc, gfx950); not an operator
   lib/libhetu_rowwise.so C++ host layer mirroring Hetu's operator interface (g++)
 
 Run as ``python hotspa-ae_amd/build.py`` or through ``__graft_entry__.build()``.
@@ -21,7 +22,9 @@ INCLUDE = os.path.join(ROOT, "include")
 
 HIP_SOURCES = ["hk_norm_bwd_bf16.hip", "hk_norm_bwd_f32.hip", "hk_norm_bwd_f16.hip", "hk_norm_fwd_bf16.hip",
                "hk_norm_fwd_f32.hip", "hk_norm_fwd_f16.hip", "hk_device.hip", "hk_norm.hip", "hk_softmax.hip", "hk_sce.hip", "hk_reduce.hip", "hk_nll.hip",
-               "hk_dropout_ln.hip", "hk_elementwise.hip", "hk_vocab_ce.hip", "hk_batchnorm.hip", "hk_stream_probe.hip"]
+               "hk_dropout_ln.hip", "hk_elementwise.hip", "hk_vocab_ce.hip", "hk_batchnorm.hip"]
+# measurement tools, a library of their own
+BENCH_SOURCES = [os.path.join("bench", "hk_bench_probe.hip")]
 
 HIPCC_FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -65,8 +68,8 @@ def build_device(verbose=True, incremental=False):
     os.makedirs(LIB, exist_ok=True)
     os.makedirs(OBJ, exist_ok=True)
     hipcc = _hipcc()
-    sources = [s for s in HIP_SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    objs = [os.path.join(OBJ, s.replace(".hip", ".o")) for s in sources]
+    sources = [s for s in HIP_SOURCES + BENCH_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    objs = [os.path.join(OBJ, os.path.basename(s).replace(".hip", ".o")) for s in sources]
 
     def one(pair):
         src, obj = pair
@@ -80,9 +83,15 @@ def build_device(verbose=True, incremental=False):
             if verbose:
                 print("[build] compiled", src, flush=True)
     out = os.path.join(LIB, "libhk_rowwise.so")
-    _run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", out] + objs)
+    main_objs = [o for s, o in zip(sources, objs) if s in HIP_SOURCES]
+    _run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", out] + main_objs)
     if verbose:
         print("[build] linked", out, flush=True)
+    bench = os.path.join(LIB, "libhk_bench.so")
+    _run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", bench] +
+         [o for s, o in zip(sources, objs) if s in BENCH_SOURCES])
+    if verbose:
+        print("[build] linked", bench, flush=True)
     return out
 
 

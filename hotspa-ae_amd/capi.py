@@ -29,6 +29,21 @@ def lib_path():
     return _LIB
 
 
+_BENCH_LIB = os.path.join(_HERE, "lib", "libhk_bench.so")
+_bench_lib = None
+
+
+def bench_lib():
+    """Loads libhk_bench.so (the streaming yardstick of include/hk_bench.h); raises if it has not been built."""
+    global _bench_lib
+    if _bench_lib is None:
+        if not os.path.exists(_BENCH_LIB):
+            raise HkError(-100, "native library %s is missing: run __graft_entry__.build() first" % _BENCH_LIB)
+        _bench_lib = ctypes.CDLL(_BENCH_LIB)
+        _bench_lib.hk_bench_last_error.restype = ctypes.c_char_p
+    return _bench_lib
+
+
 def lib():
     """Loads libhk_rowwise.so; raises if it has not been built."""
     global _lib
@@ -677,11 +692,14 @@ def stream_probe(dsts, srcs, block_threads=256, vectors_per_thread=1, nt_loads=T
     nbytes = ref.numel() * ref.element_size()
     d = list(dsts) + [None, None]
     r = list(srcs) + [None, None]
-    check(lib().hk_stream_probe(_ptr(d[0]), _ptr(d[1]), _ptr(r[0]), _ptr(r[1]), ctypes.c_int(len(srcs)),
-                                ctypes.c_int(len(dsts)), ctypes.c_size_t(nbytes), ctypes.c_int(block_threads),
-                                ctypes.c_int(vectors_per_thread), ctypes.c_int(int(nt_loads)),
-                                ctypes.c_int(int(nt_stores)), ctypes.c_int(workgroups_per_cu),
-                                stream if stream is not None else current_stream()))
+    rc = bench_lib().hk_bench_stream_probe(_ptr(d[0]), _ptr(d[1]), _ptr(r[0]), _ptr(r[1]), ctypes.c_int(len(srcs)),
+                                           ctypes.c_int(len(dsts)), ctypes.c_size_t(nbytes),
+                                           ctypes.c_int(block_threads), ctypes.c_int(vectors_per_thread),
+                                           ctypes.c_int(int(nt_loads)), ctypes.c_int(int(nt_stores)),
+                                           ctypes.c_int(workgroups_per_cu),
+                                           stream if stream is not None else current_stream())
+    if rc != 0:
+        raise HkError(rc, bench_lib().hk_bench_last_error().decode("utf-8", "replace"))
 
 
 def memcpy_d2d(dst, src, stream=None):

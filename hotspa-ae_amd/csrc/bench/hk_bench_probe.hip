@@ -3,9 +3,41 @@
 // fixed number of workgroups per compute unit walking the array, non-temporal hint on the loads and / or the
 // stores).  What the best shape of a mix reaches is the roof the operator kernels with that mix are held against.
 // The hints are template arguments: as run-time flags the compiler merges the two branches into a plain access.
+//
+// This file is a library of its own (libhk_bench.so, include/hk_bench.h) that bench.py loads: a measurement tool, kept
+// out of the operator library.  It shares hk_common.h's device-side types with the kernels and nothing else.
 #include "hk_common.h"
+#include "hk_bench.h"
+
+#include <algorithm>
+#include <stdarg.h>
+#include <stdio.h>
 
 namespace hk {
+
+static thread_local char g_bench_error[512] = "";
+
+// this library's own error text (the operator library's is not shared with it)
+void set_last_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_bench_error, sizeof(g_bench_error), fmt, ap);
+  va_end(ap);
+}
+
+static int bench_launch_check(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return HK_OK;
+  set_last_error("%s: launch failed: %s", what, hipGetErrorString(e));
+  return HK_ERR_HIP;
+}
+
+static int bench_cu_count() {
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+  return n;
+}
 
 struct ProbeArgs {
   const u32x4* src[2];
@@ -66,13 +98,13 @@ template <int BS, int U, int NR, int NW>
 static int probe_nt(const ProbeArgs& a, int ntl, int nts, unsigned grid, hipStream_t s) {
   if (NR == 0) ntl = 0;
   if (NW == 0) nts = 0;
-  profile_before(s);
-  if (ntl && nts) HK_LAUNCH((stream_probe_kernel<BS, U, NR, NW, NR != 0, NW != 0>), dim3(grid), dim3(BS), 0, s, a);
-  else if (ntl) HK_LAUNCH((stream_probe_kernel<BS, U, NR, NW, NR != 0, false>), dim3(grid), dim3(BS), 0, s, a);
-  else if (nts) HK_LAUNCH((stream_probe_kernel<BS, U, NR, NW, false, NW != 0>), dim3(grid), dim3(BS), 0, s, a);
-  else HK_LAUNCH((stream_probe_kernel<BS, U, NR, NW, false, false>), dim3(grid), dim3(BS), 0, s, a);
-  profile_after(s);
-  return launch_check("stream_probe_kernel");
+#define HK_PROBE(L, S) hipLaunchKernelGGL((stream_probe_kernel<BS, U, NR, NW, L, S>), dim3(grid), dim3(BS), 0, s, a)
+  if (ntl && nts) HK_PROBE(NR != 0, NW != 0);
+  else if (ntl) HK_PROBE(NR != 0, false);
+  else if (nts) HK_PROBE(false, NW != 0);
+  else HK_PROBE(false, false);
+#undef HK_PROBE
+  return bench_launch_check("stream_probe_kernel");
 }
 
 template <int BS, int U>
@@ -82,7 +114,7 @@ static int probe_mix(const ProbeArgs& a, int nr, int nw, int ntl, int nts, unsig
   if (nr == 1 && nw == 2) return probe_nt<BS, U, 1, 2>(a, ntl, nts, grid, s);
   if (nr == 1 && nw == 0) return probe_nt<BS, U, 1, 0>(a, ntl, nts, grid, s);
   if (nr == 0 && nw == 1) return probe_nt<BS, U, 0, 1>(a, ntl, nts, grid, s);
-  set_last_error("hk_stream_probe: no kernel for %d reads : %d writes", nr, nw);
+  set_last_error("hk_bench_stream_probe: no kernel for %d reads : %d writes", nr, nw);
   return HK_ERR_UNSUPPORTED;
 }
 
@@ -93,7 +125,7 @@ static int probe_unroll(const ProbeArgs& a, int unroll, int nr, int nw, int ntl,
     case 2: return probe_mix<BS, 2>(a, nr, nw, ntl, nts, grid, s);
     case 4: return probe_mix<BS, 4>(a, nr, nw, ntl, nts, grid, s);
     default:
-      set_last_error("hk_stream_probe: 1, 2 or 4 vectors per thread, got %d", unroll);
+      set_last_error("hk_bench_stream_probe: 1, 2 or 4 vectors per thread, got %d", unroll);
       return HK_ERR_UNSUPPORTED;
   }
 }
@@ -104,38 +136,43 @@ using namespace hk;
 
 extern "C" {
 
-int hk_stream_probe(void* dst0, void* dst1, const void* src0, const void* src1, int reads, int writes, size_t bytes,
-                    int block_threads, int vectors_per_thread, int nt_loads, int nt_stores, int workgroups_per_cu,
-                    hkStream_t stream) {
-  HK_REQUIRE(bytes % 16 == 0 && bytes > 0, HK_ERR_INVALID, "hk_stream_probe: size must be a positive multiple of 16");
+const char* hk_bench_last_error(void) { return g_bench_error; }
+
+int hk_bench_stream_probe(void* dst0, void* dst1, const void* src0, const void* src1, int reads, int writes,
+                          size_t bytes, int block_threads, int vectors_per_thread, int nt_loads, int nt_stores,
+                          int workgroups_per_cu, hkStream_t stream) {
+  const char* who = "hk_bench_stream_probe";
+  HK_REQUIRE(block_threads == 64 || block_threads == 128 || block_threads == 256 || block_threads == 512 ||
+             block_threads == 1024, HK_ERR_UNSUPPORTED, "%s: workgroups of 64, 128, 256, 512 or 1024 threads, got %d",
+             who, block_threads);
+  HK_REQUIRE(vectors_per_thread == 1 || vectors_per_thread == 2 || vectors_per_thread == 4, HK_ERR_UNSUPPORTED,
+             "%s: 1, 2 or 4 vectors per thread, got %d", who, vectors_per_thread);
+  HK_REQUIRE(bytes % 16 == 0 && bytes > 0, HK_ERR_INVALID, "%s: size must be a positive multiple of 16", who);
   HK_REQUIRE(reads >= 0 && reads <= 2 && writes >= 0 && writes <= 2 && reads + writes > 0, HK_ERR_INVALID,
-             "hk_stream_probe: 0..2 reads and 0..2 writes, not both 0");
+             "%s: 0..2 reads and 0..2 writes, not both 0", who);
   HK_REQUIRE((reads < 1 || src0) && (reads < 2 || src1) && (writes < 1 || dst0) && (writes < 2 || dst1),
-             HK_ERR_INVALID, "hk_stream_probe: null array");
+             HK_ERR_INVALID, "%s: null array", who);
   HK_REQUIRE(aligned16(src0) && aligned16(src1) && aligned16(dst0) && aligned16(dst1), HK_ERR_INVALID,
-             "hk_stream_probe: arrays must be 16-byte aligned");
+             "%s: arrays must be 16-byte aligned", who);
   HK_REQUIRE(workgroups_per_cu >= 0 && workgroups_per_cu <= 64, HK_ERR_INVALID,
-             "hk_stream_probe: 0 (one-shot grid) to 64 workgroups per compute unit");
+             "%s: 0 (one-shot grid) to 64 workgroups per compute unit", who);
   ProbeArgs a{};
   a.src[0] = static_cast<const u32x4*>(src0); a.src[1] = static_cast<const u32x4*>(src1);
   a.dst[0] = static_cast<u32x4*>(dst0); a.dst[1] = static_cast<u32x4*>(dst1);
   a.nvec = bytes / 16;
   a.sink = nullptr;
-  const size_t tile = size_t(block_threads) * size_t(vectors_per_thread > 0 ? vectors_per_thread : 1);
+  const size_t tile = size_t(block_threads) * size_t(vectors_per_thread);
   const size_t tiles = (a.nvec + tile - 1) / tile;
-  HK_REQUIRE(tiles <= 0x7fffffffu, HK_ERR_INVALID, "hk_stream_probe: size too large");
+  HK_REQUIRE(tiles <= 0x7fffffffu, HK_ERR_INVALID, "%s: size too large", who);
   const unsigned grid = workgroups_per_cu == 0 ? unsigned(tiles)
-                                               : unsigned(std::min<size_t>(tiles, size_t(device_cu_count()) * workgroups_per_cu));
+                                               : unsigned(std::min<size_t>(tiles, size_t(bench_cu_count()) * workgroups_per_cu));
   hipStream_t s = as_hip(stream);
   switch (block_threads) {
     case 64: return probe_unroll<64>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
     case 128: return probe_unroll<128>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
     case 256: return probe_unroll<256>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
     case 512: return probe_unroll<512>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
-    case 1024: return probe_unroll<1024>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
-    default:
-      set_last_error("hk_stream_probe: workgroups of 64, 128, 256, 512 or 1024 threads, got %d", block_threads);
-      return HK_ERR_UNSUPPORTED;
+    default: return probe_unroll<1024>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
   }
 }
 

@@ -630,6 +630,7 @@ enum TuneKey {
 };
 int tune_get(int key);
 int device_cu_count();
+void device_lds_bytes(size_t* per_cu, size_t* per_block);
 
 inline size_t dtype_size(int dtype) {
   switch (dtype) {
@@ -653,15 +654,21 @@ void profile_after(hipStream_t s);
 bool profile_claim(hipEvent_t* before, hipEvent_t* after);
 
 // Dynamic LDS to ask for so that at most `workgroups` workgroups of a kernel are resident on a compute unit
-// (160 KB of LDS each; `static_bytes` = the kernel's own __shared__ arrays): half way between the size that would
-// let one more in and the size that would keep one out, so the allocation granule does not matter.  A streaming
-// kernel whose threads hold several vectors in flight moves more with fewer workgroups per compute unit than the
-// thread limit allows (RMSNorm forward, 256-thread workgroups: 8 resident 84.8 us, 5 resident 83.5 us).
-static inline size_t lds_bytes_for_residency(int workgroups, size_t static_bytes) {
-  if (workgroups <= 0) return 0;
-  const size_t total = 160 * 1024;
+// (`static_bytes` = the kernel's own __shared__ arrays; the compute unit's LDS as the device reports it): half way
+// between the size that would let one more in and the size that would keep one out, so the allocation granule does
+// not matter.  A streaming kernel whose threads hold several vectors in flight moves more with fewer workgroups
+// per compute unit than the thread limit allows (RMSNorm forward, 256-thread workgroups: 8 resident 84.8 us, 5
+// resident 83.5 us).  Returns false when one workgroup may not ask for that much (a residency the device cannot be
+// held to this way).
+static inline bool lds_bytes_for_residency(int workgroups, size_t static_bytes, size_t* bytes) {
+  *bytes = 0;
+  if (workgroups <= 0) return true;
+  size_t total = 0, per_block = 0;
+  device_lds_bytes(&total, &per_block);
   const size_t want = (total / size_t(workgroups + 1) + total / size_t(workgroups)) / 2;
-  return want > static_bytes ? want - static_bytes : 0;
+  if (want > per_block) return false;
+  *bytes = want > static_bytes ? want - static_bytes : 0;
+  return true;
 }
 
 #define HK_LAUNCH(kernel, grid, block, lds_bytes, stream, ...)                                                  \

@@ -91,6 +91,29 @@ int device_cu_count() {
   return cached[dev];
 }
 
+// LDS of the current device, cached per device index: bytes one compute unit holds and bytes one workgroup may ask
+// for.  What the device reports is used; the figures of this part (160 KB, 64 KB) only stand in when the query fails.
+void device_lds_bytes(size_t* per_cu, size_t* per_block) {
+  static size_t cached_cu[64] = {0}, cached_block[64] = {0};
+  int dev = 0;
+  size_t cu = 160 * 1024, block = 64 * 1024;
+  if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
+    if (cached_cu[dev] == 0) {
+      int a = 0, b = 0;
+      if (hipDeviceGetAttribute(&a, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) != hipSuccess || a <= 0)
+        a = int(cu);
+      if (hipDeviceGetAttribute(&b, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess || b <= 0)
+        b = int(block);
+      cached_cu[dev] = size_t(a);
+      cached_block[dev] = size_t(b);
+    }
+    cu = cached_cu[dev];
+    block = cached_block[dev];
+  }
+  *per_cu = cu;
+  *per_block = block;
+}
+
 // ---------------------------------------------------------------------------
 // utility kernels
 // ---------------------------------------------------------------------------
@@ -462,6 +485,16 @@ int hk_mem_get_info(size_t* free_bytes, size_t* total_bytes) {
 int hk_device_cu_count(int device, int* cus) {
   HK_REQUIRE(cus, HK_ERR_INVALID, "hk_device_cu_count: null output");
   HK_CHECK_HIP(hipDeviceGetAttribute(cus, hipDeviceAttributeMultiprocessorCount, device));
+  return HK_OK;
+}
+
+int hk_device_lds_bytes(int device, size_t* per_cu, size_t* per_block) {
+  HK_REQUIRE(per_cu && per_block, HK_ERR_INVALID, "hk_device_lds_bytes: null output");
+  int a = 0, b = 0;
+  HK_CHECK_HIP(hipDeviceGetAttribute(&a, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, device));
+  HK_CHECK_HIP(hipDeviceGetAttribute(&b, hipDeviceAttributeMaxSharedMemoryPerBlock, device));
+  *per_cu = size_t(a);
+  *per_block = size_t(b);
   return HK_OK;
 }
 

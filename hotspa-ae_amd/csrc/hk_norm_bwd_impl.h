@@ -609,7 +609,6 @@ static int launch_norm_bwd_inst(const NormBwdArgs& a, const BwdPlan& p, int pf, 
 
 template <typename T, int MODE>
 static int launch_norm_bwd_nv(const NormBwdArgs& a, const BwdPlan& p, hipStream_t s) {
-  profile_before(s);
   int pf = tune_get(TUNE_NORM_BWD_PREFETCH);
   // two rows in flight per thread group pay at 512 threads per row (4096 bf16 columns: 134 against 139 us for
   // RMSNorm, 134 against 141 us for LayerNorm) and cost at 640 (5120 columns: 93.7 against 91.0 us)
@@ -620,6 +619,14 @@ static int launch_norm_bwd_nv(const NormBwdArgs& a, const BwdPlan& p, hipStream_
     return HK_ERR_INVALID;
   }
   const int bound = bound_for(p.block);
+  const bool have_kernel = p.nv == 1 || p.nv == 2 || (p.nv == 4 && VecIO<T>::N == 4);
+  if (!have_kernel) {
+    set_last_error("norm_bwd: no kernel for %d vectors per thread", p.nv);
+    return HK_ERR_UNSUPPORTED;
+  }
+  // every argument check has passed: only now are the timing events of a measurement handed to the launch, so an
+  // early return never leaves them for an unrelated launch to claim
+  profile_before(s);
   int rc = HK_ERR_UNSUPPORTED;
   if (p.nv == 1) {
     if (bound == 512) rc = launch_norm_bwd_inst<T, MODE, 1, 512>(a, p, pf, s);
@@ -631,11 +638,8 @@ static int launch_norm_bwd_nv(const NormBwdArgs& a, const BwdPlan& p, hipStream_
   } else if (p.nv == 4) {
     if constexpr (VecIO<T>::N == 4) rc = launch_norm_bwd_inst<T, MODE, 4, 512>(a, p, pf, s);
   }
-  if (rc == HK_ERR_UNSUPPORTED) {
-    set_last_error("norm_bwd: no kernel for %d vectors per thread", p.nv);
-    return rc;
-  }
   profile_after(s);
+  if (rc != HK_OK) return rc;
   return launch_check("norm_bwd_kernel");
 }
 

@@ -313,7 +313,7 @@ static constexpr int max_rows_per_block(int nv, bool has_res) {
 
 // rows_per_block: 1 or 2 (one-wavefront rows always 1)
 template <typename T, int NV, bool WAVE_ROW, bool HAS_RES, bool IS_RMS>
-static void launch_norm_fwd_width(const NormFwdArgs& a, int rows_per_block, dim3 grid, dim3 block, hipStream_t s) {
+static int launch_norm_fwd_width(const NormFwdArgs& a, int rows_per_block, dim3 grid, dim3 block, hipStream_t s) {
   if constexpr (!WAVE_ROW && max_rows_per_block<T>(NV, HAS_RES) >= 2) {
     if (rows_per_block == 2) {
       // two rows of several vectors per thread: fewer workgroups per compute unit than the thread limit admits
@@ -321,30 +321,39 @@ static void launch_norm_fwd_width(const NormFwdArgs& a, int rows_per_block, dim3
       // instead of 4, 44.7 against 45.9 us at 4096 fp32 columns; 2 lose again)
       int resident = tune_get(TUNE_NORM_FWD_RESIDENT);
       if (resident == 0) resident = block.x == 256 ? 5 : (block.x == 512 ? 3 : 0);
-      const size_t lds = lds_bytes_for_residency(resident, sizeof(float) * 2 * kMaxWaves * 2 * 2);
+      size_t lds = 0;
+      HK_REQUIRE(lds_bytes_for_residency(resident, sizeof(float) * 2 * kMaxWaves * 2 * 2, &lds), HK_ERR_INVALID,
+                 "norm_fwd: 'norm_fwd_resident' = %d needs more dynamic LDS than one workgroup may ask for", resident);
+      profile_before(s);
       HK_LAUNCH((norm_fwd_kernel<T, NV, false, HAS_RES, IS_RMS, 2>), grid, block, lds, s, a);
-      return;
+      profile_after(s);
+      return HK_OK;
     }
   }
+  profile_before(s);
   HK_LAUNCH((norm_fwd_kernel<T, NV, WAVE_ROW, HAS_RES, IS_RMS, 1>), grid, block, 0, s, a);
+  profile_after(s);
+  return HK_OK;
 }
 
 template <typename T, bool WAVE_ROW, bool HAS_RES, bool IS_RMS>
 static int launch_norm_fwd_rms(const NormFwdArgs& a, int nv, int rpb, dim3 grid, dim3 block, hipStream_t s) {
-  profile_before(s);
+  // the timing events of a measurement are handed to the launch only once every argument check has passed
+  // (launch_norm_fwd_width), so an early return never leaves them for an unrelated launch to claim
+  int rc = HK_ERR_UNSUPPORTED;
   switch (nv) {
-    case 1: launch_norm_fwd_width<T, 1, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
-    case 2: launch_norm_fwd_width<T, 2, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
-    case 3: launch_norm_fwd_width<T, 3, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
-    case 4: launch_norm_fwd_width<T, 4, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
-    case 5: launch_norm_fwd_width<T, 5, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
-    case 6: launch_norm_fwd_width<T, 6, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
-    case 8: launch_norm_fwd_width<T, 8, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 1: rc = launch_norm_fwd_width<T, 1, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 2: rc = launch_norm_fwd_width<T, 2, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 3: rc = launch_norm_fwd_width<T, 3, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 4: rc = launch_norm_fwd_width<T, 4, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 5: rc = launch_norm_fwd_width<T, 5, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 6: rc = launch_norm_fwd_width<T, 6, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
+    case 8: rc = launch_norm_fwd_width<T, 8, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s); break;
     case 16:
       // sixteen vectors are 64 fp32 registers only for fp32 data; with a residual two packed rows of that length
       // are in flight on top
       if constexpr (sizeof(T) == 4 && !WAVE_ROW && !HAS_RES) {
-        launch_norm_fwd_width<T, 16, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s);
+        rc = launch_norm_fwd_width<T, 16, WAVE_ROW, HAS_RES, IS_RMS>(a, rpb, grid, block, s);
         break;
       }
       [[fallthrough]];
@@ -352,7 +361,7 @@ static int launch_norm_fwd_rms(const NormFwdArgs& a, int nv, int rpb, dim3 grid,
       set_last_error("norm_fwd: no kernel for %d vectors per thread", nv);
       return HK_ERR_UNSUPPORTED;
   }
-  profile_after(s);
+  if (rc != HK_OK) return rc;
   return launch_check("norm_fwd_kernel");
 }
 

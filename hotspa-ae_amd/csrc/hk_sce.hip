@@ -137,7 +137,9 @@ void sce_sparse_fwd_kernel(SceArgs a) {
       // sum exp(x - M) = S * 2^(ML - M * log2e); the fma recovers the rounding of ML exactly
       const float M = p.v[2];
       const float log2s = __builtin_amdgcn_logf(p.v[1]) - fmaf(M, kLog2e, -p.v[0]);
-      r = (log2s * kLn2 + M) - xl;
+      // M - xl first: the difference of two logits is (nearly) exact however large their common offset is, and
+      // the sum then rounds at the size of the loss, not of the logits
+      r = log2s * kLn2 + (M - xl);
     } else {
       r = __builtin_nanf("");  // label outside [0, cols): no logit to gather
     }
@@ -389,7 +391,7 @@ void sce_generic_kernel(SceArgs a) {
   } else if (MODE == 0) {
     if (threadIdx.x == 0) {
       CT r;
-      if (label >= 0 && label < cols) r = (sce_log<CT>(s) + m) - SceIO<T, CT>::ld(xr + label);
+      if (label >= 0 && label < cols) r = sce_log<CT>(s) + (m - SceIO<T, CT>::ld(xr + label));
       else r = CT(__builtin_nanf(""));
       SceIO<T, CT>::st(static_cast<T*>(a.out) + row, r);
     }

@@ -77,6 +77,9 @@ HK_API int hk_get_device(int* device);
 HK_API int hk_device_sync(void);
 HK_API int hk_mem_get_info(size_t* free_bytes, size_t* total_bytes);
 HK_API int hk_device_cu_count(int device, int* cus);    /* Device::dprop().multiProcessorCount */
+/* LDS bytes of one compute unit and the most one workgroup may ask for, as the device reports them
+ * (Device::dprop().maxSharedMemoryPerMultiProcessor / sharedMemPerBlock) */
+HK_API int hk_device_lds_bytes(int device, size_t* per_cu, size_t* per_block);
 
 HK_API int hk_malloc(void** ptr, size_t bytes);         /* CUDACachingMemoryPool.cu: cudaMalloc */
 HK_API int hk_free(void* ptr);
@@ -120,15 +123,6 @@ HK_API int hk_profile_next_kernel(hkEvent_t before, hkEvent_t after);
 /* Plain streaming copy kernel of `bytes` (multiple of 16, 16-byte aligned):
  * calibration reference for bandwidth counters and timings. */
 HK_API int hk_copy_kernel(void* dst, const void* src, size_t bytes, hkStream_t stream);
-
-/* Streaming yardstick (no counterpart in the reference): moves `bytes` per array, `reads` arrays in (0..2) and
- * `writes` arrays out (0..2), with workgroups of `block_threads` (64 .. 1024), `vectors_per_thread` 16-byte vectors
- * in flight per thread (1, 2, 4), the non-temporal hint on loads / stores, and either a one-shot grid
- * (`workgroups_per_cu` 0) or that many workgroups per compute unit walking the arrays.  The best shape of a
- * read : write mix is the roof the operator kernels with that mix are measured against (bench.py --all). */
-HK_API int hk_stream_probe(void* dst0, void* dst1, const void* src0, const void* src1, int reads, int writes,
-                           size_t bytes, int block_threads, int vectors_per_thread, int nt_loads, int nt_stores,
-                           int workgroups_per_cu, hkStream_t stream);
 
 /* Gathers a strided view into a dense row-major array (what the reference's
  * OffsetCalculator does per element, hetu/impl/utils/offset_calculator.cuh:16-68).
@@ -301,7 +295,9 @@ HK_API int hk_dropout_add_ln_bwd_strided_rows(int itype, int rtype, int wtype, c
  * row the register kernel takes (8192 columns) needs on 256 persistent workgroups; a plan that needs
  * more (hk_norm_bwd_workspace_bytes > 16 MiB: a device with more compute units, or a raised
  * "norm_bwd_blocks") is refused with HK_ERR_WORKSPACE.  All calls on one device share the array: calls that overlap on one
- * device (different streams, or threads) race and must be ordered by the caller. */
+ * device (different streams, or threads) race and must be ordered by the caller.  The first call on a device looks
+ * the array's address up (hipGetSymbolAddress, once per device): make that call before a capture begins; calls
+ * recorded after it replay like any other kernel launch. */
 HK_API int hk_dropout_add_ln_bwd_static(int itype, int rtype, int wtype, const void* dz,
                                         const void* dx_in, const void* x, const void* mu,
                                         const void* rsigma, const void* gamma, void* dx0,

@@ -44,7 +44,10 @@ def pytest_terminal_summary(terminalreporter):
         return
     tr = terminalreporter
     tr.section("strict relative error |a - e| / |e| over elements with |e| >= %.0e rms(e)" % helpers.STRICT_FLOOR)
-    tr.write_line("%-34s %-22s %-5s %11s %9s %11s %6s" % ("test file", "quantity", "dtype", "strict", "bound",
-                                                          "gate", "calls"))
-    for (f, what, dt), (strict, bound, gate, n) in sorted(helpers.STRICT_LOG.items()):
-        tr.write_line("%-34s %-22s %-5s %11.3e %9.1e %11.3e %6d" % (f, what[:22], dt, strict, bound, gate, n))
+    tr.write_line("ordinary: the same over elements with |e| >= %.1f rms(e), held to the dtype's own tolerance"
+                  % helpers.ORDINARY_FLOOR)
+    tr.write_line("%-34s %-22s %-5s %11s %9s %11s %9s %11s %6s" % ("test file", "quantity", "dtype", "ordinary", "bound",
+                                                                   "strict", "bound", "gate", "calls"))
+    for (f, what, dt), (strict, bound, gate, n, ordinary, obound) in sorted(helpers.STRICT_LOG.items()):
+        tr.write_line("%-34s %-22s %-5s %11.3e %9.1e %11.3e %9.1e %11.3e %6d" % (f, what[:22], dt, ordinary, obound,
+                                                                                 strict, bound, gate, n))

@@ -13,7 +13,10 @@ if ROOT not in sys.path:
 import oracle  # noqa: E402  (test infrastructure)
 
 # Tolerances of the parity bar: fp32 within 1e-5 relative, bf16 / fp16 within
-# 1e-2 relative (fp32 accumulation).  Two figures are formed for every comparison:
+# 1e-2 relative (fp32 accumulation).  Three figures are formed for every comparison:
+#   * the ordinary figure: |a - e| / |e| over the elements of ordinary size, |e| >= 0.1 rms(e).  It is held to the
+#     dtype's OWN tolerance (fp32 1e-5) for every quantity, loosened only where a call states why (`rtol`; or
+#     `scale`, the size of the terms a sum was formed from when that is larger than the sum);
 #   * the gate: |a - e| / (|e| + rms(e)), over every element.  Elements that cancel to ~0 are judged against
 #     the tensor's scale instead of their own vanishing magnitude;
 #   * the strict figure: |a - e| / |e| alone, over the elements that are not near zero (|e| >= 1e-3 rms(e)).
@@ -21,6 +24,7 @@ import oracle  # noqa: E402  (test infrastructure)
 #     worst value per test file and quantity is printed at the end of the run.
 RTOL = {"fp32": 1e-5, "bf16": 1e-2, "fp16": 1e-2, "fp64": 1e-12}
 STRICT_FLOOR = 1e-3          # an element counts as "not near zero" from this multiple of rms(expected)
+ORDINARY_FLOOR = 0.1         # an element is "of ordinary size" from this multiple of rms(expected)
 # Bounds of the strict figure.
 #   * Quantities formed without cancellation (inverse standard deviations, variances, single element-wise
 #     operations, sums of one sign) meet the dtype's own tolerance element by element: STRICT_RTOL.
@@ -33,13 +37,21 @@ STRICT_FLOOR = 1e-3          # an element counts as "not near zero" from this mu
 #     itself fp64 arithmetic with its own rounding, so two correct results differ by a few thousand ulp there.
 STRICT_RTOL = {"fp32": 1e-5, "bf16": 1e-2, "fp16": 1e-2, "fp64": 1e-12}
 STRICT_RTOL_SUMS = {"fp32": 2e-4, "bf16": 1e-2, "fp16": 1e-2, "fp64": 1e-9}
+# The gradient of a softmax, dx = y * (dy - sum(dy * y)), carries the factor (dy - dot): where dy is close to the
+# row's dot product that factor cancels, while y (which spans orders of magnitude within a row) may still make
+# |dx| an element of ordinary size.  The dot product of a row of n terms is known to about sqrt(n) * 2^-24 of the
+# terms' size, so such an element cannot be held to 1e-5 of its own size in fp32: the ordinary figure is held to
+# 1e-4 there, the strict one to 1e-3 for rows of thousands of terms.
+SOFTMAX_GRADIENT_ORDINARY_RTOL = 1e-4
+SOFTMAX_GRADIENT_STRICT_RTOL = 1e-3
 NO_CANCELLATION = ("rs", "rstd", "var", "save_invstd", "running_var", "exp", "log", "sqrt", "mul", "div", "add",
                    "sub", "neg", "reduce", "ln_rstd", "rms_rs", "rms_z", "sm_y")
 # fp16 stores magnitudes under 2^-14 as subnormals with fewer than 11 significant bits: such outputs are outside
 # the strict figure (the gate still covers them)
 MIN_NORMAL = {"fp16": 6.103515625e-05}
 
-# (test file, quantity, dtype) -> [worst strict figure, its bound, worst gate figure, comparisons]
+# (test file, quantity, dtype) -> [worst strict figure, its bound, worst gate figure, comparisons,
+#                                   worst ordinary figure, its bound]
 STRICT_LOG = {}
 
 
@@ -74,14 +86,16 @@ def rel_error(actual, expected, scale=None):
     return np.abs(actual - expected) / denom
 
 
-def strict_error(actual, expected, dtype="fp32"):
-    """max |a - e| / |e| over the finite elements with |e| >= STRICT_FLOOR * rms(e); 0.0 when there is none."""
+def strict_error(actual, expected, dtype="fp32", floor=None):
+    """max |a - e| / |e| over the finite elements with |e| >= floor * rms(e) (STRICT_FLOOR when not given); 0.0
+    when there is none."""
+    floor = STRICT_FLOOR if floor is None else floor
     actual = np.asarray(actual, dtype=np.float64).ravel()
     expected = np.asarray(expected, dtype=np.float64).ravel()
     if expected.size == 0:
         return 0.0
     rms = float(np.sqrt(np.mean(np.square(expected))))
-    keep = np.abs(expected) >= STRICT_FLOOR * rms if rms > 0.0 else np.zeros(expected.shape, dtype=bool)
+    keep = np.abs(expected) >= floor * rms if rms > 0.0 else np.zeros(expected.shape, dtype=bool)
     if dtype in MIN_NORMAL:
         keep &= np.abs(expected) >= MIN_NORMAL[dtype]
     if not keep.any():
@@ -89,19 +103,21 @@ def strict_error(actual, expected, dtype="fp32"):
     return float(np.max(np.abs(actual[keep] - expected[keep]) / np.abs(expected[keep])))
 
 
-def _log_strict(what, dtype, strict, bound, gate):
+def _log_strict(what, dtype, strict, bound, gate, ordinary=0.0, ordinary_bound=0.0):
     test = os.environ.get("PYTEST_CURRENT_TEST", "")
     key = (test.split("::")[0].split("/")[-1], what.split(" ")[0] if what else "", dtype)
-    rec = STRICT_LOG.setdefault(key, [0.0, bound, 0.0, 0])
+    rec = STRICT_LOG.setdefault(key, [0.0, bound, 0.0, 0, 0.0, ordinary_bound])
     rec[0] = max(rec[0], strict)
     rec[1] = max(rec[1], bound)
     rec[2] = max(rec[2], gate)
     rec[3] += 1
+    rec[4] = max(rec[4], ordinary)
+    rec[5] = max(rec[5], ordinary_bound)
 
 
-def assert_close(actual, expected, dtype, what="", scale=None, rtol=None, strict_rtol=None):
+def assert_close(actual, expected, dtype, what="", scale=None, rtol=None, strict_rtol=None, ordinary_rtol=None):
     """actual: torch tensor or numpy; expected: float64 numpy (oracle).  `scale` replaces rms(expected) in the
-    gate; `rtol` / `strict_rtol` replace the dtype's bounds (a call that loosens one says why)."""
+    gate; `rtol` / `strict_rtol` / `ordinary_rtol` replace the dtype's bounds (a call that loosens one says why)."""
     if hasattr(actual, "detach"):
         actual = to_numpy(actual)
     actual = np.asarray(actual, dtype=np.float64).reshape(np.asarray(expected).shape)
@@ -125,9 +141,25 @@ def assert_close(actual, expected, dtype, what="", scale=None, rtol=None, strict
             rms = float(np.sqrt(np.mean(np.square(e)))) if e.size else 0.0
             if rms > 0.0:
                 strict_rtol *= max(1.0, float(scale) / rms)
-    _log_strict(what, dtype, strict, strict_rtol, worst)
+    # elements of ordinary size: the dtype's own tolerance, loosened only by what the call itself states (a looser
+    # `rtol`; a `scale` larger than the result, i.e. terms larger than their sum)
+    ordinary = strict_error(actual[fin], np.asarray(expected)[fin], dtype, ORDINARY_FLOOR)
+    stated = ordinary_rtol
+    ordinary_rtol = RTOL[dtype] * max(1.0, tol / RTOL[dtype])
+    if stated is not None:
+        ordinary_rtol = max(ordinary_rtol, stated) if dtype in ("fp32", "fp64") else ordinary_rtol
+    if scale is not None and dtype in ("fp32", "fp64"):
+        e = np.asarray(expected, dtype=np.float64)[fin]
+        rms = float(np.sqrt(np.mean(np.square(e)))) if e.size else 0.0
+        if rms > 0.0:
+            ordinary_rtol *= max(1.0, float(scale) / rms)
+    if dtype == "fp64":
+        ordinary_rtol = max(ordinary_rtol, 1e-10)   # the oracle is fp64 arithmetic itself
+    _log_strict(what, dtype, strict, strict_rtol, worst, ordinary, ordinary_rtol)
     assert strict <= strict_rtol, ("%s: max strictly element-relative error %.3e (elements with |e| >= %.0e rms) "
                                    "exceeds %.1e" % (what, strict, STRICT_FLOOR, strict_rtol))
+    assert ordinary <= ordinary_rtol, ("%s: max element-relative error %.3e over elements of ordinary size "
+                                       "(|e| >= %.1f rms) exceeds %.1e" % (what, ordinary, ORDINARY_FLOOR, ordinary_rtol))
     return worst
 
 

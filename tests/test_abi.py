@@ -19,6 +19,27 @@ def test_library_exports_every_declared_symbol(hk):
     assert not missing, missing
 
 
+def test_bench_library_is_separate(hk):
+    """The streaming yardstick lives in a library of its own: libhk_bench.so exports what include/hk_bench.h
+    declares, the operator library exports none of it, and bad arguments come back as codes before anything is
+    computed from them (no GPU needed)."""
+    import importlib
+    capi = importlib.import_module("hotspa-ae_amd.capi")
+    text = open(os.path.join(helpers.ROOT, "include", "hk_bench.h")).read()
+    names = sorted(set(re.findall(r"HK_API\s+[\w\s\*]+?\b(hk_\w+)\s*\(", text)))
+    assert names == ["hk_bench_last_error", "hk_bench_stream_probe"]
+    bench = capi.bench_lib()
+    for n in names:
+        assert hasattr(bench, n) and not hasattr(hk.lib(), n)
+    assert not hasattr(hk.lib(), "hk_stream_probe")
+    buf = ctypes.create_string_buffer(64)
+    addr = ctypes.c_void_p((ctypes.addressof(buf) + 15) // 16 * 16)
+    for threads, vectors in ((0, 1), (-64, 1), (96, 1), (256, 0), (256, 3)):
+        rc = bench.hk_bench_stream_probe(addr, None, addr, None, 1, 1, ctypes.c_size_t(32), threads, vectors, 1, 1, 0, None)
+        assert rc == -2, (threads, vectors, rc)
+        assert b"threads" in bench.hk_bench_last_error() or b"vectors" in bench.hk_bench_last_error()
+
+
 def test_no_torch_types_in_the_boundary():
     text = open(os.path.join(helpers.ROOT, "include", "hk_rowwise.h")).read()
     assert "torch" not in text and "at::" not in text and 'extern "C"' in text

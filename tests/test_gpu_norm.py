@@ -284,7 +284,10 @@ def test_layer_norm_statistics_conditioning(hk, cuda, dtype, cols):
     # The strict figure is left out of the bound here on purpose: in the outlier rows the regular elements come out
     # as |y| ~ 1e-3 (the outlier owns the variance) from x - mean with mean ~ 0.6..300, so the half ulp of the mean
     # alone is percents of such an element, in any fp32 arithmetic.  It is still printed with the others.
-    helpers.assert_close(ty, ey, dtype, "y", rtol=1e-4 if dtype == "fp32" else None, strict_rtol=1e-1)
+    # The ordinary figure is loosened for the same reason: in the offset rows |x - mean| ~ 1 against a mean near 300,
+    # half an ulp of which (1.5e-5) is 1e-5 .. 1e-3 of elements that are of ordinary size in y.
+    helpers.assert_close(ty, ey, dtype, "y", rtol=1e-4 if dtype == "fp32" else None, strict_rtol=1e-1,
+                         ordinary_rtol=1e-3)
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])

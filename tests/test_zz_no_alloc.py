@@ -94,3 +94,74 @@ def test_static_scratch_refuses_what_does_not_fit(hk, cuda):
     hk.dropout_add_ln_bwd_static(x, None, x, st, st, w, dx, None, dg, db, True)
     torch.cuda.synchronize()
     assert float(dx.float().abs().max()) == 0.0
+
+
+def test_static_scratch_allocates_nothing(hk, cuda):
+    """The property the entry point exists for: after the first call on the device (which looks the scratch's
+    address up), repeated calls leave the device's free memory where it was, through the driver's own count and
+    through torch's caching allocator, and the library's device pool, neither of which is asked for a byte."""
+    import torch
+    rows, cols, dt = 1024, 4096, "bf16"
+    x, dz, w = _inputs(rows, cols, dt, cuda, 77)
+    mu, rs, z = torch.empty(rows, device=cuda), torch.empty(rows, device=cuda), torch.empty_like(x)
+    hk.dropout_add_ln_fwd(x, None, w, None, z, None, mu, rs, 1e-6, True)
+    dx, dg, db = torch.empty_like(x), torch.empty_like(w), torch.empty_like(w)
+    hk.dropout_add_ln_bwd_static(dz, None, x, mu, rs, w, dx, None, dg, db, True)      # first call on the device
+    torch.cuda.synchronize()
+    free0 = ctypes.c_size_t()
+    total = ctypes.c_size_t()
+    hk.check(hk.lib().hk_mem_get_info(ctypes.byref(free0), ctypes.byref(total)))
+    stats0 = torch.cuda.memory_stats()
+    for _ in range(20):
+        hk.dropout_add_ln_bwd_static(dz, None, x, mu, rs, w, dx, None, dg, db, True)
+    torch.cuda.synchronize()
+    free1 = ctypes.c_size_t()
+    hk.check(hk.lib().hk_mem_get_info(ctypes.byref(free1), ctypes.byref(total)))
+    stats1 = torch.cuda.memory_stats()
+    assert free1.value == free0.value, "device free memory moved across static calls"
+    for key in ("allocation.all.allocated", "segment.all.allocated", "num_alloc_retries"):
+        assert stats1.get(key, 0) == stats0.get(key, 0), key
+
+
+def test_static_scratch_under_graph_capture(hk, cuda):
+    """Recorded into a HIP graph after a first call outside the capture (the address look-up of the scratch is
+    made once per device and not again), the static call replays: every replay, with new inputs written in place
+    and eager work and synchronisations between replays, equals the eager workspace call bit for bit."""
+    import torch
+    rows, cols, bf = 768, 4096, torch.bfloat16
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(rows, cols, generator=g, device=cuda).to(bf)
+    dz = torch.randn(rows, cols, generator=g, device=cuda).to(bf)
+    w = (torch.rand(cols, generator=g, device=cuda) * 0.4 + 0.8).to(bf)
+    mu, rs, z = torch.empty(rows, device=cuda), torch.empty(rows, device=cuda), torch.empty_like(x)
+    dx, dg, db = torch.empty_like(x), torch.empty_like(w), torch.empty_like(w)
+    ws = torch.empty(hk.norm_bwd_workspace_bytes(hk.dtype_code(x), rows, cols) // 4 + 4, device=cuda)
+
+    def step():
+        hk.dropout_add_ln_fwd(x, None, w, None, z, None, mu, rs, 1e-6, True)
+        hk.dropout_add_ln_bwd_static(dz, None, x, mu, rs, w, dx, None, dg, db, True)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                      # first call on the device, outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for trial in range(4):
+        x.copy_(torch.randn(rows, cols, generator=g, device=cuda).to(bf))
+        dz.copy_(torch.randn(rows, cols, generator=g, device=cuda).to(bf))
+        # eager reference through the workspace call
+        edx, edg, edb = torch.empty_like(x), torch.empty_like(w), torch.empty_like(w)
+        emu, ers, ez = torch.empty_like(mu), torch.empty_like(rs), torch.empty_like(z)
+        hk.dropout_add_ln_fwd(x, None, w, None, ez, None, emu, ers, 1e-6, True)
+        hk.dropout_add_ln_bwd(dz, None, x, emu, ers, w, edx, None, edg, edb, True, workspace=ws)
+        torch.cuda.synchronize()
+        for t in (dx, dg, db):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dx, edx) and torch.equal(dg, edg) and torch.equal(db, edb), "replay %d" % trial

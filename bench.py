@@ -246,10 +246,18 @@ def case_sce(hk, torch, nsets, which):
     loss = torch.empty(rows, dtype=bf, device="cuda")
     gl = torch.full((rows,), 1.0 / rows, dtype=bf, device="cuda")
     n = rows * cols * 2
+    # rows whose label is the ignored index are not read (their loss is 0, their gradient row is zeros): the bytes
+    # really moved are the algorithmic ones less one logits row per such row
+    ignored = int(drop.sum().item())
     if which == "fwd":
-        return (lambda i: hk.sce_sparse_fwd(sets[i % nsets]["x"], labels, loss, IGNORE)), n + rows * 8 + rows * 2, rows
-    return (lambda i: hk.sce_sparse_bwd(sets[i % nsets]["x"], labels, gl, sets[i % nsets]["dx"], IGNORE)), \
-        2 * n + rows * 8 + rows * 2, rows
+        launch = lambda i: hk.sce_sparse_fwd(sets[i % nsets]["x"], labels, loss, IGNORE)
+        nbytes = n + rows * 8 + rows * 2
+    else:
+        launch = lambda i: hk.sce_sparse_bwd(sets[i % nsets]["x"], labels, gl, sets[i % nsets]["dx"], IGNORE)
+        nbytes = 2 * n + rows * 8 + rows * 2
+    launch.bytes_moved = nbytes - ignored * cols * 2
+    launch.ignored_rows = ignored
+    return launch, nbytes, rows
 
 
 def case_nll_bwd(hk, torch, nsets):
@@ -671,15 +679,25 @@ def _cpu_cores():
     return min(int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1), 64)
 
 
-def cpu_baseline(rows=32768, cols=4096, budget_s=3.0):
-    """fp32 CPU port of the headline step (oracle's refcpu_rmsnorm_*) on all host threads: the full workload,
-    repeated for about `budget_s` seconds of CPU work; the mean over the repetitions is reported."""
+def _timed_cpu(fn, budget_s):
+    fn()                                    # pages the outputs in, warms whatever the call warms
+    reps, t0 = 0, time.perf_counter()
+    while reps < 2 or time.perf_counter() - t0 < budget_s:
+        fn()
+        reps += 1
+    return (time.perf_counter() - t0) / reps, reps
+
+
+def cpu_baseline(rows=32768, cols=4096, budget_s=2.0):
+    """The headline step on the host: `value` is the fp32 CPU port of it (oracle's refcpu_rmsnorm_*) on all host
+    threads over the full workload, repeated for about `budget_s` seconds; beside it the same port on ONE thread (the
+    reference's scalar loops are serial and its build never enables OpenMP, CMakeLists.txt:33-36) on a quarter of the
+    rows, and torch's own CPU operators (F.rms_norm and its autograd; MKL / oneDNN-class kernels) on all threads."""
     import ctypes
     import numpy as np
     import oracle
     lib = oracle.lib()
     cores = _cpu_cores()
-    lib.refcpu_set_num_threads(ctypes.c_int(cores))
     g = np.random.default_rng(402)
     # a 1024-row random block repeated down the array: the values do not change the timing
     reps_of_block = (rows + 1023) // 1024
@@ -691,32 +709,60 @@ def cpu_baseline(rows=32768, cols=4096, budget_s=3.0):
     fp = ctypes.POINTER(ctypes.c_float)
     P = lambda a: a.ctypes.data_as(fp)
 
-    def step():
-        lib.refcpu_rmsnorm_fwd_f32(P(x), P(w), ctypes.c_int64(rows), ctypes.c_int64(cols), ctypes.c_float(1e-6), P(z), P(rs))
-        lib.refcpu_rmsnorm_bwd_f32(P(dz), P(x), P(w), P(rs), ctypes.c_int64(rows), ctypes.c_int64(cols), P(dx), P(dg))
+    def step(n):
+        lib.refcpu_rmsnorm_fwd_f32(P(x), P(w), ctypes.c_int64(n), ctypes.c_int64(cols), ctypes.c_float(1e-6), P(z), P(rs))
+        lib.refcpu_rmsnorm_bwd_f32(P(dz), P(x), P(w), P(rs), ctypes.c_int64(n), ctypes.c_int64(cols), P(dx), P(dg))
 
-    step()  # page in the outputs
-    reps, t0 = 0, time.perf_counter()
-    while reps < 2 or time.perf_counter() - t0 < budget_s:
-        step()
-        reps += 1
-    dt = (time.perf_counter() - t0) / reps
-    algo = rows * (5 * cols * 2 + 12)  # same bf16 accounting as the GPU step, per row
-    return {"value": round(algo / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": "all %d rows, fwd+bwd in fp32, %d repetitions over %.1f s, mean; bytes counted as for the GPU step "
-                      "(bf16 storage); RMSNorm has no CPU kernel in the reference, this is the oracle's fp32 port of the "
-                      "formula" % (rows, reps, reps * dt)}
+    per_row = 5 * cols * 2 + 12             # same bf16 accounting as the GPU step
+    lib.refcpu_set_num_threads(ctypes.c_int(cores))
+    dt, reps = _timed_cpu(lambda: step(rows), budget_s)
+    out = {"value": round(rows * per_row / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+           "sample": "all %d rows, fwd+bwd in fp32, %d repetitions over %.1f s, mean; bytes counted as for the GPU step "
+                     "(bf16 storage); RMSNorm has no CPU kernel in the reference, this is the oracle's fp32 port of the "
+                     "formula" % (rows, reps, reps * dt)}
+    # one thread, a quarter of the rows
+    lib.refcpu_set_num_threads(ctypes.c_int(1))
+    n1 = rows // 4
+    dt1, reps1 = _timed_cpu(lambda: step(n1), 1.0)
+    lib.refcpu_set_num_threads(ctypes.c_int(cores))
+    out["one_thread"] = {"value": round(n1 * per_row / dt1 / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                         "sample": "%d of %d rows, %d repetitions, mean" % (n1, rows, reps1)}
+    # torch's CPU operators on the same shape in bf16 (forward, then forward + backward through autograd)
+    import torch
+    torch.set_num_threads(cores)
+    nt = rows // 16
+    tx = torch.from_numpy(x[:nt]).to(torch.bfloat16).requires_grad_(True)
+    tdz = torch.from_numpy(dz[:nt]).to(torch.bfloat16)
+    tw = torch.from_numpy(w).to(torch.bfloat16).requires_grad_(True)
+
+    def torch_step():
+        tx.grad = None
+        tw.grad = None
+        torch.nn.functional.rms_norm(tx, (cols,), tw, 1e-6).backward(tdz)
+
+    dtt, repst = _timed_cpu(torch_step, 1.0)
+    out["torch_cpu"] = {"value": round(nt * per_row / dtt / 1e9, 3), "unit": "GB/s", "cores": cores,
+                        "kind": "torch-cpu (oneDNN-class)",
+                        "sample": "F.rms_norm forward + autograd backward, bf16, %d of %d rows, %d repetitions, mean"
+                                  % (nt, rows, repst)}
+    return out
 
 
-def cpu_baselines(budget_s=1.2):
-    """One entry per BASELINE configuration kernel: the host twins of the kernels (LayerNormCpu /
-    LayerNormGradientCpu, SoftmaxCpu / SoftmaxGradientCpu, SoftmaxCrossEntropySparseCpu / ...GradientCpu, ReduceCpu:
-    the reference's CPU pass structure as fp32 loops, OpenMP over rows), called through the same operator entry
-    points and device dispatch as the accelerator kernels, on a bounded sample of the configuration's rows in the
-    configuration's storage type.  `value` counts the same algorithmic bytes per row as the GPU entry of that
-    configuration, so the two columns compare like with like."""
+def cpu_baselines(budget_s=0.5):
+    """Per BASELINE configuration kernel, three host figures on a bounded sample of the configuration's rows, in the
+    configuration's storage type, counting the same algorithmic bytes per row as the GPU entry:
+      * kind "port": the host twin of the kernel (LayerNormCpu / LayerNormGradientCpu, SoftmaxCpu / SoftmaxGradientCpu,
+        SoftmaxCrossEntropySparseCpu / ...GradientCpu, ReduceCpu: the reference's CPU pass structure as fp32 loops,
+        OpenMP over rows), called through the same operator entry points and device dispatch as the accelerator
+        kernels, on all host threads;
+      * kind "port (1 thread)": the same on one thread -- the reference's own scalar loops are serial and its build
+        never enables OpenMP (CMakeLists.txt:33-36);
+      * kind "torch-cpu (oneDNN-class)": torch's CPU operator of the same mathematics on all threads (MKL / oneDNN
+        inside), standing in for the oneDNN primitives the reference calls (hetu/impl/kernel/Softmax.cc:31-45,
+        Reduce.cc:41-68, LayerNorm.cc:89-129), whose library is not part of the reference's sources."""
     import importlib
     import torch
+    import torch.nn.functional as F
     importlib.import_module("hotspa-ae_amd")
     ops = importlib.import_module("hotspa-ae_amd.hetu_ops")
     cores = _cpu_cores()
@@ -728,66 +774,91 @@ def cpu_baselines(budget_s=1.2):
         b = torch.randn(min(rows, 512), cols, generator=g)
         return b.repeat((rows + b.shape[0] - 1) // b.shape[0], 1)[:rows].to(dt).contiguous()
 
-    def timed(fn):
-        fn()
-        reps, t0 = 0, time.perf_counter()
-        while reps < 2 or time.perf_counter() - t0 < budget_s:
-            fn()
-            reps += 1
-        return (time.perf_counter() - t0) / reps, reps
-
     out = []
 
-    def add(config, case, fn, algo_bytes, sample_rows, full_rows, arith="fp32"):
-        dt, reps = timed(fn)
-        out.append({"config": config, "case": case, "value": round(algo_bytes / dt / 1e9, 3), "unit": "GB/s",
-                    "us": round(dt * 1e6, 1), "cores": cores, "kind": "port",
-                    "sample": "%d of %d rows, %s arithmetic, %d repetitions, mean" % (sample_rows, full_rows, arith, reps)})
+    def add(config, case, port_fn, torch_fn, algo_bytes, sample_rows, full_rows, torch_what, torch_bytes=None):
+        def rec(kind, n_cores, dt, reps, nbytes, what):
+            out.append({"config": config, "case": case, "value": round(nbytes / dt / 1e9, 3), "unit": "GB/s",
+                        "us": round(dt * 1e6, 1), "cores": n_cores, "kind": kind,
+                        "sample": "%d of %d rows, %s, %d repetitions, mean" % (sample_rows, full_rows, what, reps)})
+        # the team size is set through the operator library itself: whichever OpenMP runtime it is bound to in this
+        # process (torch ships one of its own) is the one that counts
+        assert ops.set_host_threads(cores) == cores
+        dt, reps = _timed_cpu(port_fn, budget_s)
+        rec("port", cores, dt, reps, algo_bytes, "fp32 arithmetic")
+        assert ops.set_host_threads(1) == 1
+        dt, reps = _timed_cpu(port_fn, budget_s)
+        rec("port (1 thread)", 1, dt, reps, algo_bytes, "fp32 arithmetic")
+        ops.set_host_threads(cores)
+        if torch_fn is not None:
+            with torch.no_grad():
+                dt, reps = _timed_cpu(torch_fn, budget_s)
+            rec("torch-cpu (oneDNN-class)", cores, dt, reps, torch_bytes or algo_bytes, torch_what)
 
-    # C1: the whole configuration, fp32 storage
-    rows, cols = 8192, 4096
+    # C1: a quarter of the configuration, fp32 storage
+    rows, cols = 2048, 4096
     x = block(rows, cols, torch.float32); y = torch.empty_like(x)
     gm, bt = torch.ones(cols), torch.zeros(cols)
     mean, var = torch.empty(rows, 1), torch.empty(rows, 1)
     add("C1", "layernorm fwd fp32 [8192x4096] (LayerNormCpu)",
-        lambda: ops.layer_norm(x, gm, bt, mean, var, y, 1, 1e-5), rows * (2 * cols * 4 + 8), rows, rows)
-    # C5 layer norm at 5120 columns, forward and gradient, 1/4 of the rows, bf16 storage
-    rows, cols = 4096, 5120
-    x = block(rows, cols, bf); y = torch.empty_like(x); dy = block(rows, cols, bf); dx = torch.empty_like(x)
-    gm, bt = torch.ones(cols, dtype=bf), torch.zeros(cols, dtype=bf)
-    mean, var = torch.empty(rows, 1, dtype=bf), torch.empty(rows, 1, dtype=bf)
+        lambda: ops.layer_norm(x, gm, bt, mean, var, y, 1, 1e-5),
+        lambda: torch.ops.aten.native_layer_norm(x, [cols], gm, bt, 1e-5),
+        rows * (2 * cols * 4 + 8), rows, 8192, "torch native_layer_norm")
+    # C5 layer norm at 5120 columns, forward and gradient, 1/8 of the rows, bf16 storage
+    rows, cols = 2048, 5120
+    x5 = block(rows, cols, bf); y5 = torch.empty_like(x5); dy5 = block(rows, cols, bf); dx5 = torch.empty_like(x5)
+    gm5, bt5 = torch.ones(cols, dtype=bf), torch.zeros(cols, dtype=bf)
+    mean5, var5 = torch.empty(rows, 1, dtype=bf), torch.empty(rows, 1, dtype=bf)
     dgm, dbt = torch.empty(cols, dtype=bf), torch.empty(cols, dtype=bf)
+    _, tmean, trstd = torch.ops.aten.native_layer_norm(x5, [cols], gm5, bt5, 1e-5)
     add("C5", "layernorm fwd bf16 [16384x5120] (LayerNormCpu)",
-        lambda: ops.layer_norm(x, gm, bt, mean, var, y, 1, 1e-5), rows * (2 * cols * 2 + 8), rows, 16384)
+        lambda: ops.layer_norm(x5, gm5, bt5, mean5, var5, y5, 1, 1e-5),
+        lambda: torch.ops.aten.native_layer_norm(x5, [cols], gm5, bt5, 1e-5),
+        rows * (2 * cols * 2 + 8), rows, 16384, "torch native_layer_norm")
     add("C5", "layernorm bwd bf16 [16384x5120] (LayerNormGradientCpu)",
-        lambda: ops.layer_norm_gradient(dy, x, gm, dx, dgm, dbt, mean, var, 1, 1e-5),
-        rows * (3 * cols * 2 + 8), rows, 16384)
-    # C2: 1/16 of the rows
-    rows, cols = 16384, 2048
-    x = block(rows, cols, bf); y = torch.empty_like(x); dx = torch.empty_like(x)
-    add("C2", "softmax fwd bf16 [4,32,2048,2048] (SoftmaxCpu)", lambda: ops.softmax(x, y, 1),
-        2 * rows * cols * 2, rows, 262144)
-    add("C2", "softmax bwd bf16 [4,32,2048,2048] (SoftmaxGradientCpu)", lambda: ops.softmax_gradient(y, x, dx, 1),
-        3 * rows * cols * 2, rows, 262144)
-    # C3: 1/4 of the rows
-    rows, cols = 8192, 4096
-    x = block(rows, cols, bf); o0 = torch.empty(cols, dtype=bf); o1 = torch.empty(rows, dtype=bf)
+        lambda: ops.layer_norm_gradient(dy5, x5, gm5, dx5, dgm, dbt, mean5, var5, 1, 1e-5),
+        lambda: torch.ops.aten.native_layer_norm_backward(dy5, x5, [cols], tmean, trstd, gm5, bt5, [True, True, True]),
+        rows * (3 * cols * 2 + 8), rows, 16384, "torch native_layer_norm_backward")
+    # C2: 1/64 of the rows
+    rows, cols = 4096, 2048
+    x2 = block(rows, cols, bf); y2 = torch.empty_like(x2); dx2 = torch.empty_like(x2)
+    add("C2", "softmax fwd bf16 [4,32,2048,2048] (SoftmaxCpu)", lambda: ops.softmax(x2, y2, 1),
+        lambda: torch.softmax(x2, -1), 2 * rows * cols * 2, rows, 262144, "torch.softmax")
+    add("C2", "softmax bwd bf16 [4,32,2048,2048] (SoftmaxGradientCpu)", lambda: ops.softmax_gradient(y2, x2, dx2, 1),
+        lambda: torch.ops.aten._softmax_backward_data(x2, y2, -1, bf), 3 * rows * cols * 2, rows, 262144,
+        "torch _softmax_backward_data")
+    # C3: 1/8 of the rows
+    rows, cols = 4096, 4096
+    x3 = block(rows, cols, bf); o0 = torch.empty(cols, dtype=bf); o1 = torch.empty(rows, dtype=bf)
     for name, axes, o in (("axis 1", [1], o1), ("axis 0", [0], o0)):
         for red in ("sum", "mean"):
+            tfn = (lambda a=axes[0]: torch.sum(x3, a)) if red == "sum" else (lambda a=axes[0]: torch.mean(x3, a))
             add("C3", "reduce %s %s bf16 [32768x4096] (ReduceCpu)%s" % (
                 red, name, "; also the merged axes (0,1) of [64x512x4096]" if (axes == [0] and red == "sum") else ""),
-                (lambda axes=axes, o=o, red=red: ops.reduce(x, o, axes, red)), rows * cols * 2, rows, 32768)
-    # C5 cross-entropy: 1/16 of the rows
-    rows, cols = 1024, 32000
-    x = block(rows, cols, bf); loss = torch.empty(rows, dtype=bf); dx = torch.empty_like(x)
+                (lambda axes=axes, o=o, red=red: ops.reduce(x3, o, axes, red)), tfn, rows * cols * 2, rows, 32768,
+                "torch.%s" % red)
+    # C5 cross-entropy: 1/64 of the rows
+    rows, cols = 256, 32000
+    xc = block(rows, cols, bf); loss = torch.empty(rows, dtype=bf); dxc = torch.empty_like(xc)
     gl = torch.full((rows,), 1.0 / 16384, dtype=bf)
     lab = (torch.arange(rows, dtype=torch.int64) * 31) % cols
     lab[::20] = IGNORE
     add("C5", "cross-entropy fwd bf16 [16384x32000] (SoftmaxCrossEntropySparseCpu)",
-        lambda: ops.softmax_cross_entropy_sparse(x, lab, loss, IGNORE), rows * (cols * 2 + 10), rows, 16384)
+        lambda: ops.softmax_cross_entropy_sparse(xc, lab, loss, IGNORE),
+        lambda: F.cross_entropy(xc, lab, ignore_index=IGNORE, reduction="none"),
+        rows * (cols * 2 + 10), rows, 16384, "torch F.cross_entropy")
+    xg = xc.clone().requires_grad_(True)
+
+    def torch_ce_fwd_bwd():
+        with torch.enable_grad():
+            xg.grad = None
+            F.cross_entropy(xg, lab, ignore_index=IGNORE, reduction="sum").backward()
+
     add("C5", "cross-entropy bwd bf16 [16384x32000] (SoftmaxCrossEntropySparseGradientCpu)",
-        lambda: ops.softmax_cross_entropy_sparse_gradient(x, lab, gl, dx, IGNORE),
-        rows * (2 * cols * 2 + 10), rows, 16384)
+        lambda: ops.softmax_cross_entropy_sparse_gradient(xc, lab, gl, dxc, IGNORE), torch_ce_fwd_bwd,
+        rows * (2 * cols * 2 + 10), rows, 16384,
+        "torch F.cross_entropy forward + autograd backward (bytes of forward and backward counted)",
+        torch_bytes=rows * (3 * cols * 2 + 20))
     return out
 
 
@@ -893,6 +964,13 @@ def main():
                "GBps": round(nbytes / kms / 1e6, 1), "frac": round(nbytes / kms / 1e6 / HBM_PEAK_GBS, 4),
                "main_kernel_frac": round(getattr(launch, "main_bytes", nbytes) / main_us / 1e3 / HBM_PEAK_GBS, 4),
                "rows_per_s": round(nrows / kms * 1e3), "bytes": nbytes}
+        if hasattr(launch, "bytes_moved"):
+            # the algorithmic bytes count every row; this kernel skips the reads of ignored rows, so the rate at
+            # which bytes really moved is frac * bytes_moved_frac
+            rec["bytes_moved"] = launch.bytes_moved
+            rec["bytes_moved_frac"] = round(launch.bytes_moved / nbytes, 4)
+            rec["ignored_rows"] = launch.ignored_rows
+            rec["frac_of_bytes_moved"] = round(launch.bytes_moved / kms / 1e6 / HBM_PEAK_GBS, 4)
         kernels.append(rec)
         print("%-46s %9.2f us (main %8.2f us) %8.1f GB/s  %5.1f%% (main %5.1f%%)" % (
             name, rec["us"], rec["main_kernel_us"], rec["GBps"], 100 * rec["frac"],
@@ -927,8 +1005,9 @@ def main():
     if not args.no_cpu and not args.no_kernels:
         out["cpu_baselines"] = cpu_baselines()
         for rec in out["cpu_baselines"]:
-            print("cpu  %-3s %-66s %10.1f us %8.2f GB/s (%d threads)" % (rec["config"], rec["case"], rec["us"], rec["value"],
-                                                                        rec["cores"]), file=sys.stderr, flush=True)
+            print("cpu  %-3s %-66s %-26s %10.1f us %8.2f GB/s (%d threads)" % (
+                rec["config"], rec["case"][:66], rec["kind"], rec["us"], rec["value"], rec["cores"]), file=sys.stderr,
+                flush=True)
     print(json.dumps(out), flush=True)
 
 

@@ -1,4 +1,7 @@
 // extern "C" face of the operator layer (declared in hetu_ops_c.h).
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 #include "hetu_ops_c.h"
 
 #include <cstring>
@@ -558,6 +561,16 @@ int ht_stream_sync(int device_index, int stream_index) {
 
 int ht_synchronize_all(void) {
   return guarded([&] { SynchronizeAllStreams(); });
+}
+
+int ht_set_host_threads(int threads) {
+#ifdef _OPENMP
+  if (threads > 0) omp_set_num_threads(threads);
+  return omp_get_max_threads();
+#else
+  (void)threads;
+  return 1;
+#endif
 }
 
 int ht_pool_alloc(int device_index, size_t bytes, int stream_index, void** ptr, uint64_t* id,

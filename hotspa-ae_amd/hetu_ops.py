@@ -121,6 +121,11 @@ def stream_sync(stream=DEFAULT_STREAM, device=0):
     check(lib().ht_stream_sync(ctypes.c_int(device), ctypes.c_int(stream)))
 
 
+def set_host_threads(n):
+    """OpenMP team size of the host twins; returns the size now in force (n <= 0 only asks)."""
+    return int(lib().ht_set_host_threads(ctypes.c_int(int(n))))
+
+
 def synchronize_all():
     check(lib().ht_synchronize_all())
 

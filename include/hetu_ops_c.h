@@ -179,6 +179,10 @@ HT_API int ht_sceloss_gradient(const HtArray* preds, const HtArray* labels, cons
 /* ---- streams and the device memory pool ---- */
 HT_API int ht_stream_sync(int device_index, int stream_index);
 HT_API int ht_synchronize_all(void);
+/* OpenMP team size of the host twins (the ...Cpu kernels), set on the calling thread through the library's own
+ * OpenMP runtime; threads <= 0 only asks.  Returns the team size now in force.  For the CPU baseline legs of the
+ * benchmark (all threads / one thread). */
+HT_API int ht_set_host_threads(int threads);
 HT_API int ht_pool_alloc(int device_index, size_t bytes, int stream_index, void** ptr, uint64_t* id,
                          size_t* granted_bytes);
 HT_API int ht_pool_free(int device_index, void* ptr, uint64_t id, size_t granted_bytes);

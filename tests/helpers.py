@@ -177,6 +177,14 @@ def draw(seed, shape, dist="normal", a=0.0, b=1.0, dtype="fp32"):
     return oracle.round_to(v, dtype)
 
 
+def sample_rows(seed, rows, count):
+    """`count` rows drawn at random plus the first two and the last two: the ends of the array are where a launch's
+    first and last workgroups (the odd tail of a two-rows-per-workgroup launch, a clamped last row) work."""
+    picked = set(rng(seed).choice(rows, min(count, rows), replace=False).tolist())
+    picked.update(r for r in (0, 1, rows - 2, rows - 1) if 0 <= r < rows)
+    return np.array(sorted(picked), dtype=np.int64)
+
+
 def packed_lengths(seed=401, total=32768, mu=6.5, sigma=1.0, lo=128, hi=16384):
     """Variable-length sequences packed until `total` tokens (the boundaries do
     not enter the row-wise kernels; recorded for completeness)."""

@@ -230,7 +230,7 @@ def test_full_size_configs(hk, cuda, cfg):
     tdx, tdg, tdb = torch.empty_like(tx), torch.empty_like(tg), torch.empty_like(tg)
     hk.dropout_add_ln_bwd(tdz, None, tx, tmu, trs, tg, tdx, None, tdg, tdb, is_rms)
     torch.cuda.synchronize()
-    sel = np.sort(helpers.rng(5).choice(rows, 48, replace=False))
+    sel = helpers.sample_rows(5, rows, 48)
     ez, _, emu, ers = oracle.dropout_add_ln_fwd(x[sel], None, gamma, None if is_rms else beta, eps, is_rms)
     helpers.assert_close(tz[sel], ez, dtype, "z")
     helpers.assert_close(trs[sel], ers, "fp32", "rsigma")

@@ -121,9 +121,7 @@ def test_sce_full_size_bf16(hk, cuda):
     tdx = torch.empty_like(tx)
     hk.sce_sparse_bwd(tx, tl, tg, tdx, IGN)
     torch.cuda.synchronize()
-    sel = np.sort(helpers.rng(4).choice(rows, 24, replace=False))
-    sel[0] = int(np.nonzero(lab == IGN)[0][0])
-    sel = np.sort(sel)
+    sel = np.unique(np.append(helpers.sample_rows(4, rows, 24), int(np.nonzero(lab == IGN)[0][0])))
     xs = helpers.to_numpy(tx[torch.from_numpy(sel).to(cuda)])
     eloss = oracle.sce_sparse_fwd(xs, lab[sel], IGN)
     helpers.assert_close(tloss[torch.from_numpy(sel).to(cuda)], eloss, "bf16", "loss")

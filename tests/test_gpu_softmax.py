@@ -67,7 +67,7 @@ def test_softmax_full_size_bf16(hk, cuda):
     hk.softmax_bwd(ty, tdy, tdx)
     torch.cuda.synchronize()
     rows = 4 * 32 * 2048
-    sel = torch.from_numpy(np.sort(helpers.rng(3).choice(rows, 64, replace=False))).to(cuda)
+    sel = torch.from_numpy(helpers.sample_rows(3, rows, 64)).to(cuda)
     x2, y2, dy2, dx2 = (t.view(rows, 2048)[sel] for t in (tx, ty, tdy, tdx))
     ey = oracle.softmax_fwd(helpers.to_numpy(x2))
     helpers.assert_close(y2, ey, "bf16", "y")

@@ -303,6 +303,28 @@ void norm_bwd_kernel(NormBwdArgs a) {
 
   // fold the row groups of this block, then write one partial row per block
   float* outs[2] = {a.part_dgamma, a.part_dbeta};
+  if constexpr (FIXED) {
+    // one group: every thread writes its own sums, as 16-byte streaming stores (the partial rows are read by the
+    // fold kernel, never again by this one; left in the cache they would only wait for the write-back at the
+    // kernel's end)
+    static_assert(VEC % 4 == 0, "whole float4 vectors per 16-byte vector of the data type");
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+      if (outs[which] == nullptr) continue;
+      const float* acc = which == 0 ? dg : db;
+      float* dst = outs[which] + int64_t(blockIdx.x) * a.cols;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+#pragma unroll
+        for (int j = 0; j < VEC; j += 4) {
+          const u32x4 pk = {f2u(acc[i * VEC + j]), f2u(acc[i * VEC + j + 1]), f2u(acc[i * VEC + j + 2]),
+                            f2u(acc[i * VEC + j + 3])};
+          st16_stream(dst + vidx[i] * VEC + j, pk);
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int which = 0; which < 2; ++which) {
     if (outs[which] == nullptr) continue;
@@ -610,8 +632,11 @@ static int launch_norm_bwd_inst(const NormBwdArgs& a, const BwdPlan& p, int pf, 
 template <typename T, int MODE>
 static int launch_norm_bwd_nv(const NormBwdArgs& a, const BwdPlan& p, hipStream_t s) {
   int pf = tune_get(TUNE_NORM_BWD_PREFETCH);
-  // two rows in flight per thread group pay at 512 threads per row (4096 bf16 columns: 134 against 139 us for
-  // RMSNorm, 134 against 141 us for LayerNorm) and cost at 640 (5120 columns: 93.7 against 91.0 us)
+  // Rows in flight per thread group, measured on the lean instances: at 512 threads per row (4096 bf16 columns,
+  // RMSNorm, main kernel) depth 1 / 2 / 3 / 4 / 6 run 134.8 / 130.4 / 133.0 / 134.0 / 136.5 us; at 640 threads
+  // (5120 columns, LayerNorm) depth 1 / 2 / 3 run 85.2 / 85.7 / 87.6 us and depths 4 and 6 collapse (252 / 371 us).
+  // More bytes in flight than two rows of a 512-thread group (32 KB per compute unit) only lose, as they do for a
+  // plain copy kernel; deeper instances than 2 are therefore not built.
   if (pf <= 0) pf = p.block <= 512 ? 2 : 1;
   // statistics in the data dtype only ever come with the plain LayerNorm backward
   if (!a.stats_f32 && MODE != BWD_LN) {

@@ -245,6 +245,7 @@ struct OuterArgs {
   int wx;               // wavefronts of a workgroup side by side across columns (the others stack over rows)
   float factor;
   int is_mean;
+  int split_major;      // grid = (row splits, column tiles, batch) instead of (column tiles, row splits, batch)
 };
 
 template <typename T, typename OUT_T, typename R>
@@ -259,10 +260,15 @@ void reduce_outer_vec_kernel(OuterArgs a) {
   const int wc = wave % wx;        // this wavefront's place across columns ...
   const int w = wave / wx;         // ... and over rows
   const int wy = int(blockDim.x >> 6) / wx;
-  const int64_t cv = (int64_t(blockIdx.x) * wx + wc) * kWave + lane;   // column vector index
+  // Row splits along the grid's x (whenever the column tiles fit its y): workgroups are dealt to the XCDs round
+  // robin in x-major order, so the workgroups of one XCD then take whole runs of rows (every column tile of a few
+  // row splits) rather than one column tile of every row split -- the same bytes in flight at any time, 1 % faster
+  // (32768 x 4096 bf16: 42.5 against 42.9 us, both orders measured alternately)
+  const int split = a.split_major ? blockIdx.x : blockIdx.y;
+  const int64_t tile = a.split_major ? blockIdx.y : blockIdx.x;
+  const int64_t cv = (tile * wx + wc) * kWave + lane;   // column vector index
   const int64_t c = cv * VEC;
   const bool col_ok = c < a.C;                              // C is a multiple of VEC here
-  const int split = blockIdx.y;
   const int64_t b = blockIdx.z;
   const int64_t r0 = int64_t(split) * a.rows_per_split;
   const int64_t r1 = (r0 + a.rows_per_split < a.R) ? r0 + a.rows_per_split : a.R;
@@ -620,7 +626,9 @@ static int reduce_fast(const ReducePlan& p, const void* in, void* out, float fac
     }
     HK_REQUIRE(p.B <= 65535, HK_ERR_UNSUPPORTED, "hk_reduce: batch extent %lld too large for the column kernel", (long long)p.B);
     const int64_t col_tiles = ((p.C / VEC + 63) / 64 + s.wx - 1) / s.wx;
+    a.split_major = col_tiles <= 65535 ? 1 : 0;
     dim3 grid(unsigned(col_tiles), unsigned(s.rsplit), unsigned(p.B)), block{unsigned(64 * s.wy * s.wx)};
+    if (a.split_major) grid = dim3(unsigned(s.rsplit), unsigned(col_tiles), unsigned(p.B));
     const size_t lds = size_t(s.wy) * s.wx * 64 * VEC * sizeof(float);
     profile_before(st);
     HK_LAUNCH((reduce_outer_vec_kernel<T, OUT_T, R>), grid, block, lds, st, a);

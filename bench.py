@@ -635,9 +635,9 @@ CASES = [
 
 
 # HBM bytes one launch of the RMSNorm backward kernel moves at the headline shape: rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE read 262868.3 and 270336.0 KiB per dispatch; a 256 MiB copy kernel calibrates the counters at
-# x1.99986 (FETCH_SIZE reads 131081.5 KiB for 262144 KiB fetched) and x1.000 (WRITE_SIZE).
-NORM_BWD_TRAFFIC_BYTES = int((262868.3 * 1.99986 + 270336.0 * 1.0) * 1024)
+# --pmc WRITE_SIZE read 262841.3 and 270792.1 KiB per dispatch; a 256 MiB copy kernel calibrates the counters at
+# x1.99993 (FETCH_SIZE reads 131076.5 KiB for 262144 KiB fetched) and x1.00000 (WRITE_SIZE reads 262146.3).
+NORM_BWD_TRAFFIC_BYTES = int((262841.3 * 1.99993 + 270792.1 * 1.0) * 1024)
 
 
 def preroll(torch, launch, min_steps=PREROLL_MIN_STEPS, min_seconds=PREROLL_MIN_SECONDS):

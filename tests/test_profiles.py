@@ -33,7 +33,9 @@ def test_backward_kernel_traffic_constant_matches_the_counter_profile():
     from the committed table, it must agree with bench.py's constant to 0.5 %."""
     text, rows = _traffic_table()
     # the headline launch: mode 1 (RMSNorm), 512-thread groups, 256 workgroups of 512 work-items
-    hits = [r for name, rs in rows.items() if name.startswith("norm_bwd_kernel<bf16, 1, 1, 2,") for r in rs
+    # (last template argument false: rows on one level, the dense call)
+    hits = [r for name, rs in rows.items()
+            if name.startswith("norm_bwd_kernel<bf16, 1, 1, 2,") and name.endswith(", false>") for r in rs
             if r["grid"] == 256 * 512 and r["wg"] == 512]
     assert len(hits) == 1, hits
     copies = [r for name, rs in rows.items() if name.startswith("copy16_kernel") for r in rs]

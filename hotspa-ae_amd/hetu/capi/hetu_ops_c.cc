@@ -4,14 +4,15 @@
 #endif
 #include "hetu_ops_c.h"
 
+#include <atomic>
 #include <cstring>
-
 #include <string>
 
 #include "hetu/graph/ops/gradient_compute.h"
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/random/CPURandomState.h"
 #include "hetu/impl/memory/CachingMemoryPool.h"
+#include "hetu/impl/stream/CPUStream.h"
 #include "hetu/impl/stream/HIPStream.h"
 
 using namespace hetu;
@@ -20,10 +21,31 @@ namespace {
 
 thread_local std::string g_error;
 
+// Host arrays are borrowed from the caller, so by default a call on them has finished when it returns: whatever it
+// put on a host stream is waited for.  ht_set_host_async(1) leaves the waiting to the caller (ht_host_stream_sync).
+std::atomic<bool> g_host_async{false};
+
+struct HostDrain {
+  // on the way out of a failed call: nothing may still be reading the caller's buffers
+  ~HostDrain() {
+    if (armed && !g_host_async.load(std::memory_order_relaxed) && hetu::impl::AnyCPUStreamBusy()) {
+      try {
+        hetu::impl::SynchronizeAllCPUStreams();
+      } catch (...) {
+      }
+    }
+  }
+  bool armed = true;
+};
+
 template <typename F>
 int guarded(F&& fn) {
   try {
+    HostDrain drain;
     fn();
+    if (!g_host_async.load(std::memory_order_relaxed) && hetu::impl::AnyCPUStreamBusy())
+      hetu::impl::SynchronizeAllCPUStreams();   // a host kernel that failed on its stream fails the call
+    drain.armed = false;
     g_error.clear();
     return HT_OK;
   } catch (const hetu::not_implemented& e) {
@@ -71,8 +93,12 @@ void copy_out(const NDArray& result, HtArray* out, const Stream& stream) {
     << "result " << result->meta() << " does not fit the buffer " << dst->meta();
   if (result->numel() == 0) return;
   NDArray src = NDArray::contiguous(result, stream.stream_index());
-  if (stream.device().is_cpu()) {   // host result (the host twins ran in this thread): a plain copy
-    std::memcpy(dst->raw_data_ptr(), src->raw_data_ptr(), src->numel() * DataType2Size(src->dtype()));
+  if (stream.device().is_cpu()) {   // host result: a plain copy, on the stream that still has to produce it
+    hetu::impl::CPUStream(stream).EnqueueTask(
+      [src, dst]() {
+        std::memcpy(dst->raw_data_ptr(), src->raw_data_ptr(), src->numel() * DataType2Size(src->dtype()));
+      },
+      "CopyOut");
     return;
   }
   hetu::impl::HIPStream hs(stream);
@@ -563,13 +589,21 @@ int ht_synchronize_all(void) {
   return guarded([&] { SynchronizeAllStreams(); });
 }
 
+int ht_host_stream_sync(int stream_index) {
+  return guarded([&] { Stream(Device(kCPU), StreamIndex(stream_index)).Sync(); });
+}
+
+int ht_set_host_async(int on) {
+  const bool before = g_host_async.exchange(on != 0);
+  return before ? 1 : 0;
+}
+
 int ht_set_host_threads(int threads) {
+  hetu::impl::SetHostKernelThreads(threads);
 #ifdef _OPENMP
-  if (threads > 0) omp_set_num_threads(threads);
-  return omp_get_max_threads();
+  return threads > 0 ? threads : omp_get_max_threads();
 #else
-  (void)threads;
-  return 1;
+  return threads > 0 ? threads : 1;
 #endif
 }
 

@@ -5,6 +5,7 @@
 #include <numeric>
 
 #include "hetu/graph/ops/kernel_links.h"
+#include "hetu/impl/stream/CPUStream.h"
 #include "hetu/impl/stream/HIPStream.h"
 #include "hetu/impl/utils/hip_utils.h"
 
@@ -141,18 +142,23 @@ NDArray NDArray::contiguous(const NDArray& input, StreamIndex stream_id) {
   NDArray out = empty(input->shape(), input->device(), input->dtype(), stream_id);
   if (input->numel() == 0) return out;
   if (input->is_cpu()) {
-    const size_t es = DataType2Size(input->dtype());
-    const auto* src = static_cast<const uint8_t*>(input->raw_data_ptr());
-    auto* dst = static_cast<uint8_t*>(out->raw_data_ptr());
-    const int64_t n = int64_t(input->numel()), nd = int64_t(input->ndim());
-    for (int64_t i = 0; i < n; ++i) {
-      int64_t rem = i, off = 0;
-      for (int64_t d = nd - 1; d >= 0; --d) {
-        off += (rem % input->shape(d)) * input->stride(d);
-        rem /= input->shape(d);
-      }
-      std::memcpy(dst + i * es, src + off * es, es);
-    }
+    // on the host stream, behind whatever still has to write the input
+    hetu::impl::CPUStream(Stream(input->device(), stream_id)).EnqueueTask(
+      [input, out]() {
+        const size_t es = DataType2Size(input->dtype());
+        const auto* src = static_cast<const uint8_t*>(input->raw_data_ptr());
+        auto* dst = static_cast<uint8_t*>(out->raw_data_ptr());
+        const int64_t n = int64_t(input->numel()), nd = int64_t(input->ndim());
+        for (int64_t i = 0; i < n; ++i) {
+          int64_t rem = i, off = 0;
+          for (int64_t d = nd - 1; d >= 0; --d) {
+            off += (rem % input->shape(d)) * input->stride(d);
+            rem /= input->shape(d);
+          }
+          std::memcpy(dst + i * es, src + off * es, es);
+        }
+      },
+      "Contiguous");
     return out;
   }
   HT_NOT_IMPLEMENTED_IF(input->ndim() > 8) << "contiguous supports up to 8 dimensions on the device";
@@ -168,6 +174,8 @@ NDArray NDArray::contiguous(const NDArray& input, StreamIndex stream_id) {
 NDArray NDArray::to(const NDArray& input, const Device& device, StreamIndex stream_id) {
   if (device == input->device()) return input;
   NDArray src = contiguous(input, stream_id);
+  // a host source may still be the output of work on the host stream of the same index
+  if (src->is_cpu()) Stream(src->device(), stream_id).Sync();
   NDArray out = empty(src->shape(), device, src->dtype(), stream_id);
   const size_t bytes = src->numel() * DataType2Size(src->dtype());
   if (bytes == 0) return out;

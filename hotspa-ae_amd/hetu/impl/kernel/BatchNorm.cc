@@ -126,46 +126,48 @@ void BatchNormCpu(const NDArray& input_X, const NDArray& bn_scale, const NDArray
   CheckParam(save_mean, input_X, pt, C, "save_mean");
   CheckParam(save_var, input_X, pt, C, "save_var");
   if (input_X->numel() == 0) return;
-  NDArray x = Dense(input_X, stream);
   HT_DISPATCH_FLOATING_TYPES(input_X->dtype(), spec_t, "BatchNormCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;   // also the parameters' storage type
-    const spec_t* xp = x->data_ptr<spec_t>();
-    spec_t* yp = output_Y->data_ptr<spec_t>();
-    const A* scale = bn_scale->data_ptr<A>();
-    const A* bias = bn_bias->data_ptr<A>();
-    A* rm = running_mean->data_ptr<A>();
-    A* rv = running_var->data_ptr<A>();
-    A* sm = save_mean->data_ptr<A>();
-    A* sv = save_var->data_ptr<A>();
-    const int64_t m = N * HW;
-    cpu::parallel_rows(C, m, [&](int64_t c) {
-      A sum = A(0);
-      for (int64_t n = 0; n < N; ++n) {
-        const spec_t* plane = xp + (n * C + c) * HW;
-        sum += cpu::blocked_sum<A>(HW, [&](int64_t i) { return cpu::ld<spec_t, A>(plane + i); });
-      }
-      const A mean = sum / A(m);
-      A sq = A(0);
-      for (int64_t n = 0; n < N; ++n) {
-        const spec_t* plane = xp + (n * C + c) * HW;
-        sq += cpu::blocked_sum<A>(HW, [&](int64_t i) {
-          const A d = cpu::ld<spec_t, A>(plane + i) - mean;
-          return d * d;
-        });
-      }
-      const A var = sq / A(m);
-      const A invstd = A(1) / std::sqrt(var + A(eps));
-      const A unbiased = m > 1 ? sq / A(m - 1) : var;
-      sm[c] = mean;
-      sv[c] = invstd;
-      rm[c] = A((1.0 - momentum) * double(rm[c]) + momentum * double(mean));
-      rv[c] = A((1.0 - momentum) * double(rv[c]) + momentum * double(unbiased));
-      const A w = invstd * scale[c], b = bias[c];
-      for (int64_t n = 0; n < N; ++n) {
-        const spec_t* plane = xp + (n * C + c) * HW;
-        spec_t* out = yp + (n * C + c) * HW;
-        for (int64_t i = 0; i < HW; ++i) cpu::st<spec_t, A>(out + i, (cpu::ld<spec_t, A>(plane + i) - mean) * w + b);
-      }
+    cpu::on_stream(stream, "BatchNormCpu", [=]() {
+      NDArray x = Dense(input_X, stream);
+      using A = typename cpu::Arith<spec_t>::type;   // also the parameters' storage type
+      const spec_t* xp = x->data_ptr<spec_t>();
+      spec_t* yp = output_Y->data_ptr<spec_t>();
+      const A* scale = bn_scale->data_ptr<A>();
+      const A* bias = bn_bias->data_ptr<A>();
+      A* rm = running_mean->data_ptr<A>();
+      A* rv = running_var->data_ptr<A>();
+      A* sm = save_mean->data_ptr<A>();
+      A* sv = save_var->data_ptr<A>();
+      const int64_t m = N * HW;
+      cpu::parallel_rows(C, m, [&](int64_t c) {
+        A sum = A(0);
+        for (int64_t n = 0; n < N; ++n) {
+          const spec_t* plane = xp + (n * C + c) * HW;
+          sum += cpu::blocked_sum<A>(HW, [&](int64_t i) { return cpu::ld<spec_t, A>(plane + i); });
+        }
+        const A mean = sum / A(m);
+        A sq = A(0);
+        for (int64_t n = 0; n < N; ++n) {
+          const spec_t* plane = xp + (n * C + c) * HW;
+          sq += cpu::blocked_sum<A>(HW, [&](int64_t i) {
+            const A d = cpu::ld<spec_t, A>(plane + i) - mean;
+            return d * d;
+          });
+        }
+        const A var = sq / A(m);
+        const A invstd = A(1) / std::sqrt(var + A(eps));
+        const A unbiased = m > 1 ? sq / A(m - 1) : var;
+        sm[c] = mean;
+        sv[c] = invstd;
+        rm[c] = A((1.0 - momentum) * double(rm[c]) + momentum * double(mean));
+        rv[c] = A((1.0 - momentum) * double(rv[c]) + momentum * double(unbiased));
+        const A w = invstd * scale[c], b = bias[c];
+        for (int64_t n = 0; n < N; ++n) {
+          const spec_t* plane = xp + (n * C + c) * HW;
+          spec_t* out = yp + (n * C + c) * HW;
+          for (int64_t i = 0; i < HW; ++i) cpu::st<spec_t, A>(out + i, (cpu::ld<spec_t, A>(plane + i) - mean) * w + b);
+        }
+      });
     });
   });
 }
@@ -191,41 +193,43 @@ void BatchNormGradientCpu(const NDArray& gradient_Y, const NDArray& input_X, con
   CheckParam(save_mean, input_X, pt, C, "save_mean");
   CheckParam(save_var, input_X, pt, C, "save_var");
   if (input_X->numel() == 0) return;
-  NDArray x = Dense(input_X, stream), dy = Dense(gradient_Y, stream);
   HT_DISPATCH_FLOATING_TYPES(input_X->dtype(), spec_t, "BatchNormGradientCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* xp = x->data_ptr<spec_t>();
-    const spec_t* dyp = dy->data_ptr<spec_t>();
-    spec_t* dxp = gradient_X->data_ptr<spec_t>();
-    const A* scale = bn_scale->data_ptr<A>();
-    const A* sm = save_mean->data_ptr<A>();
-    const A* sv = save_var->data_ptr<A>();
-    A* dscale = gradient_bn_scale->data_ptr<A>();
-    A* dbias = gradient_bn_bias->data_ptr<A>();
-    const int64_t m = N * HW;
-    cpu::parallel_rows(C, m, [&](int64_t c) {
-      const A mean = sm[c], invstd = sv[c];
-      A sum_dy = A(0), sum_dy_xhat = A(0);
-      for (int64_t n = 0; n < N; ++n) {
-        const spec_t* xr = xp + (n * C + c) * HW;
-        const spec_t* dr = dyp + (n * C + c) * HW;
-        sum_dy += cpu::blocked_sum<A>(HW, [&](int64_t i) { return cpu::ld<spec_t, A>(dr + i); });
-        sum_dy_xhat += cpu::blocked_sum<A>(HW, [&](int64_t i) {
-          return cpu::ld<spec_t, A>(dr + i) * (cpu::ld<spec_t, A>(xr + i) - mean) * invstd;
-        });
-      }
-      dscale[c] = sum_dy_xhat;
-      dbias[c] = sum_dy;
-      const A w = scale[c] * invstd, k1 = sum_dy / A(m), k2 = sum_dy_xhat / A(m);
-      for (int64_t n = 0; n < N; ++n) {
-        const spec_t* xr = xp + (n * C + c) * HW;
-        const spec_t* dr = dyp + (n * C + c) * HW;
-        spec_t* out = dxp + (n * C + c) * HW;
-        for (int64_t i = 0; i < HW; ++i) {
-          const A xh = (cpu::ld<spec_t, A>(xr + i) - mean) * invstd;
-          cpu::st<spec_t, A>(out + i, w * (cpu::ld<spec_t, A>(dr + i) - k1 - xh * k2));
+    cpu::on_stream(stream, "BatchNormGradientCpu", [=]() {
+      NDArray x = Dense(input_X, stream), dy = Dense(gradient_Y, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* xp = x->data_ptr<spec_t>();
+      const spec_t* dyp = dy->data_ptr<spec_t>();
+      spec_t* dxp = gradient_X->data_ptr<spec_t>();
+      const A* scale = bn_scale->data_ptr<A>();
+      const A* sm = save_mean->data_ptr<A>();
+      const A* sv = save_var->data_ptr<A>();
+      A* dscale = gradient_bn_scale->data_ptr<A>();
+      A* dbias = gradient_bn_bias->data_ptr<A>();
+      const int64_t m = N * HW;
+      cpu::parallel_rows(C, m, [&](int64_t c) {
+        const A mean = sm[c], invstd = sv[c];
+        A sum_dy = A(0), sum_dy_xhat = A(0);
+        for (int64_t n = 0; n < N; ++n) {
+          const spec_t* xr = xp + (n * C + c) * HW;
+          const spec_t* dr = dyp + (n * C + c) * HW;
+          sum_dy += cpu::blocked_sum<A>(HW, [&](int64_t i) { return cpu::ld<spec_t, A>(dr + i); });
+          sum_dy_xhat += cpu::blocked_sum<A>(HW, [&](int64_t i) {
+            return cpu::ld<spec_t, A>(dr + i) * (cpu::ld<spec_t, A>(xr + i) - mean) * invstd;
+          });
         }
-      }
+        dscale[c] = sum_dy_xhat;
+        dbias[c] = sum_dy;
+        const A w = scale[c] * invstd, k1 = sum_dy / A(m), k2 = sum_dy_xhat / A(m);
+        for (int64_t n = 0; n < N; ++n) {
+          const spec_t* xr = xp + (n * C + c) * HW;
+          const spec_t* dr = dyp + (n * C + c) * HW;
+          spec_t* out = dxp + (n * C + c) * HW;
+          for (int64_t i = 0; i < HW; ++i) {
+            const A xh = (cpu::ld<spec_t, A>(xr + i) - mean) * invstd;
+            cpu::st<spec_t, A>(out + i, w * (cpu::ld<spec_t, A>(dr + i) - k1 - xh * k2));
+          }
+        }
+      });
     });
   });
 }

@@ -53,13 +53,15 @@ void BinaryConstHost(int op, const char* who, const NDArray& input, double value
   HT_ASSERT_SAME_DTYPE(input, output);
   HT_ASSERT_CONTIGUOUS(output);
   if (input->numel() == 0) return;
-  NDArray x = Dense(input, stream);
   const int64_t n = int64_t(input->numel());
   HT_DISPATCH_INTEGER_AND_FLOATING_TYPES(input->dtype(), spec_t, who, [&]() {
-    const spec_t* px = x->data_ptr<spec_t>();
-    spec_t* po = output->data_ptr<spec_t>();
-    const spec_t c = static_cast<spec_t>(value);   // the constant in the array's type, as the accelerator path
-    cpu::parallel_for(n, [&](int64_t i) { po[i] = cpu::binary_op<spec_t>(op, c, px[i]); });
+    cpu::on_stream(stream, who, [=]() {
+      NDArray x = Dense(input, stream);
+      const spec_t* px = x->data_ptr<spec_t>();
+      spec_t* po = output->data_ptr<spec_t>();
+      const spec_t c = static_cast<spec_t>(value);   // the constant in the array's type, as the accelerator path
+      cpu::parallel_for(n, [&](int64_t i) { po[i] = cpu::binary_op<spec_t>(op, c, px[i]); });
+    });
   });
 }
 } // namespace

@@ -73,7 +73,8 @@ void DivElewiseCuda(const NDArray& inputA, const NDArray& inputB, NDArray& outpu
 // float64) and round once; the integer types wrap in their own width, a division by zero gives 0 instead of a trap.
 // ---------------------------------------------------------------------------------------------------------
 namespace {
-void BinaryElewiseHost(int op, const char* who, const NDArray& inputA, const NDArray& inputB, NDArray& output) {
+void BinaryElewiseHost(int op, const char* who, const NDArray& inputA, const NDArray& inputB, NDArray& output,
+                       const Stream& stream) {
   HT_ASSERT_CPU_DEVICE(inputA);
   HT_ASSERT_SAME_DEVICE(inputA, output);
   HT_ASSERT_SAME_DEVICE(inputB, output);
@@ -92,29 +93,31 @@ void BinaryElewiseHost(int op, const char* who, const NDArray& inputA, const NDA
   const std::vector<int64_t> shape(output->shape().begin(), output->shape().end());
   const int nd = int(shape.size());
   HT_DISPATCH_INTEGER_AND_FLOATING_TYPES(output->dtype(), spec_t, who, [&]() {
-    const spec_t* pa = inputA->data_ptr<spec_t>();
-    const spec_t* pb = inputB->data_ptr<spec_t>();
-    spec_t* po = output->data_ptr<spec_t>();
-    const int64_t n = nd ? shape[size_t(nd - 1)] : 1;
-    const int64_t ia = nd ? sa[size_t(nd - 1)] : 0, ib = nd ? sb[size_t(nd - 1)] : 0;
-    cpu::for_each_run(nd, shape.data(), sa.data(), sb.data(), [&](int64_t o, int64_t oa, int64_t ob) {
-      for (int64_t i = 0; i < n; ++i) po[o + i] = cpu::binary_op<spec_t>(op, pa[oa + i * ia], pb[ob + i * ib]);
+    cpu::on_stream(stream, who, [=]() {   // the stride vectors travel with the task
+      const spec_t* pa = inputA->data_ptr<spec_t>();
+      const spec_t* pb = inputB->data_ptr<spec_t>();
+      spec_t* po = output->data_ptr<spec_t>();
+      const int64_t n = nd ? shape[size_t(nd - 1)] : 1;
+      const int64_t ia = nd ? sa[size_t(nd - 1)] : 0, ib = nd ? sb[size_t(nd - 1)] : 0;
+      cpu::for_each_run(nd, shape.data(), sa.data(), sb.data(), [&](int64_t o, int64_t oa, int64_t ob) {
+        for (int64_t i = 0; i < n; ++i) po[o + i] = cpu::binary_op<spec_t>(op, pa[oa + i * ia], pb[ob + i * ib]);
+      });
     });
   });
 }
 } // namespace
 
-void AddElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream&) {
-  BinaryElewiseHost(HK_BINARY_ADD, "AddElewiseCpu", inputA, inputB, output);
+void AddElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream& stream) {
+  BinaryElewiseHost(HK_BINARY_ADD, "AddElewiseCpu", inputA, inputB, output, stream);
 }
-void SubElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream&) {
-  BinaryElewiseHost(HK_BINARY_SUB, "SubElewiseCpu", inputA, inputB, output);
+void SubElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream& stream) {
+  BinaryElewiseHost(HK_BINARY_SUB, "SubElewiseCpu", inputA, inputB, output, stream);
 }
-void MulElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream&) {
-  BinaryElewiseHost(HK_BINARY_MUL, "MulElewiseCpu", inputA, inputB, output);
+void MulElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream& stream) {
+  BinaryElewiseHost(HK_BINARY_MUL, "MulElewiseCpu", inputA, inputB, output, stream);
 }
-void DivElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream&) {
-  BinaryElewiseHost(HK_BINARY_DIV, "DivElewiseCpu", inputA, inputB, output);
+void DivElewiseCpu(const NDArray& inputA, const NDArray& inputB, NDArray& output, const Stream& stream) {
+  BinaryElewiseHost(HK_BINARY_DIV, "DivElewiseCpu", inputA, inputB, output, stream);
 }
 
 } // namespace impl

@@ -88,33 +88,35 @@ void BroadcastShapeMulCuda(const NDArray& input, double const_value, NDArray& ou
 // the constant rounded to the array's type) one run along the last dimension at a time.
 namespace {
 void BroadcastHost(const char* who, const NDArray& input, bool multiply, double const_value, NDArray& output,
-                   const HTShape& add_axes) {
+                   const HTShape& add_axes, const Stream& stream) {
   HT_ASSERT_CPU_DEVICE(input);
   int64_t out_shape[8], in_strides[8], none[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   if (!BroadcastLayout(who, input, output, add_axes, out_shape, in_strides)) return;
   const int nd = int(output->ndim());
   HT_DISPATCH_INTEGER_AND_FLOATING_TYPES(output->dtype(), spec_t, who, [&]() {
-    const spec_t* pi = input->data_ptr<spec_t>();
-    spec_t* po = output->data_ptr<spec_t>();
-    const spec_t c = static_cast<spec_t>(const_value);
-    const int64_t n = nd ? out_shape[nd - 1] : 1, step = nd ? in_strides[nd - 1] : 0;
-    cpu::for_each_run(nd, out_shape, in_strides, none, [&](int64_t o, int64_t oi, int64_t) {
-      if (multiply) {
-        for (int64_t i = 0; i < n; ++i) po[o + i] = cpu::binary_op<spec_t>(2, pi[oi + i * step], c);
-      } else {
-        for (int64_t i = 0; i < n; ++i) po[o + i] = pi[oi + i * step];
-      }
+    cpu::on_stream(stream, who, [=]() {   // the layout arrays are copied into the task
+      const spec_t* pi = input->data_ptr<spec_t>();
+      spec_t* po = output->data_ptr<spec_t>();
+      const spec_t c = static_cast<spec_t>(const_value);
+      const int64_t n = nd ? out_shape[nd - 1] : 1, step = nd ? in_strides[nd - 1] : 0;
+      cpu::for_each_run(nd, out_shape, in_strides, none, [&](int64_t o, int64_t oi, int64_t) {
+        if (multiply) {
+          for (int64_t i = 0; i < n; ++i) po[o + i] = cpu::binary_op<spec_t>(2, pi[oi + i * step], c);
+        } else {
+          for (int64_t i = 0; i < n; ++i) po[o + i] = pi[oi + i * step];
+        }
+      });
     });
   });
 }
 } // namespace
 
-void BroadcastShapeCpu(const NDArray& input, NDArray& output, const HTShape& add_axes, const Stream&) {
-  BroadcastHost("BroadcastShape", input, false, 1.0, output, add_axes);
+void BroadcastShapeCpu(const NDArray& input, NDArray& output, const HTShape& add_axes, const Stream& stream) {
+  BroadcastHost("BroadcastShape", input, false, 1.0, output, add_axes, stream);
 }
 void BroadcastShapeMulCpu(const NDArray& input, double const_value, NDArray& output, const HTShape& add_axes,
-                          const Stream&) {
-  BroadcastHost("BroadcastShapeMul", input, true, const_value, output, add_axes);
+                          const Stream& stream) {
+  BroadcastHost("BroadcastShapeMul", input, true, const_value, output, add_axes, stream);
 }
 
 } // namespace impl

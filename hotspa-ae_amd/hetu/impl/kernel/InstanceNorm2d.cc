@@ -104,26 +104,28 @@ void InstanceNormCpu(const NDArray& in_arr, NDArray& mean_arr, NDArray& var_arr,
   HT_ASSERT(int64_t(mean_arr->numel()) == rows && int64_t(var_arr->numel()) == rows)
     << "statistics must hold one value per plane (" << rows << ")";
   if (in_arr->numel() == 0) return;
-  NDArray x = Dense(in_arr, stream);
   HT_DISPATCH_FLOATING_TYPES(in_arr->dtype(), spec_t, "InstanceNormCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* xp = x->data_ptr<spec_t>();
-    spec_t* mp = mean_arr->data_ptr<spec_t>();
-    spec_t* vp = var_arr->data_ptr<spec_t>();
-    spec_t* yp = out_arr->data_ptr<spec_t>();
-    const A inv = A(1) / A(cols);
-    cpu::parallel_rows(rows, cols, [&](int64_t r) {
-      const spec_t* xr = xp + r * cols;
-      const A mean = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); }) * inv;
-      const A var = cpu::blocked_sum<A>(cols, [&](int64_t i) {
-        const A d = cpu::ld<spec_t, A>(xr + i) - mean;
-        return d * d;
-      }) * inv;
-      cpu::st<spec_t, A>(mp + r, mean);
-      cpu::st<spec_t, A>(vp + r, var);
-      const A rstd = A(1) / std::sqrt(var + A(eps));
-      spec_t* yr = yp + r * cols;
-      for (int64_t i = 0; i < cols; ++i) cpu::st<spec_t, A>(yr + i, (cpu::ld<spec_t, A>(xr + i) - mean) * rstd);
+    cpu::on_stream(stream, "InstanceNormCpu", [=]() {
+      NDArray x = Dense(in_arr, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* xp = x->data_ptr<spec_t>();
+      spec_t* mp = mean_arr->data_ptr<spec_t>();
+      spec_t* vp = var_arr->data_ptr<spec_t>();
+      spec_t* yp = out_arr->data_ptr<spec_t>();
+      const A inv = A(1) / A(cols);
+      cpu::parallel_rows(rows, cols, [&](int64_t r) {
+        const spec_t* xr = xp + r * cols;
+        const A mean = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); }) * inv;
+        const A var = cpu::blocked_sum<A>(cols, [&](int64_t i) {
+          const A d = cpu::ld<spec_t, A>(xr + i) - mean;
+          return d * d;
+        }) * inv;
+        cpu::st<spec_t, A>(mp + r, mean);
+        cpu::st<spec_t, A>(vp + r, var);
+        const A rstd = A(1) / std::sqrt(var + A(eps));
+        spec_t* yr = yp + r * cols;
+        for (int64_t i = 0; i < cols; ++i) cpu::st<spec_t, A>(yr + i, (cpu::ld<spec_t, A>(xr + i) - mean) * rstd);
+      });
     });
   });
 }
@@ -147,30 +149,32 @@ void InstanceNormGradientCpu(const NDArray& out_grads, const NDArray& in_arr, ND
   HT_ASSERT(int64_t(mean_arr->numel()) == rows && int64_t(var_arr->numel()) == rows)
     << "statistics must hold one value per plane (" << rows << ")";
   if (in_arr->numel() == 0) return;
-  NDArray dy = Dense(out_grads, stream), x = Dense(in_arr, stream);
-  NDArray mean = Dense(mean_arr, stream), var = Dense(var_arr, stream);
   HT_DISPATCH_FLOATING_TYPES(in_arr->dtype(), spec_t, "InstanceNormGradientCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* dyp = dy->data_ptr<spec_t>();
-    const spec_t* xp = x->data_ptr<spec_t>();
-    const spec_t* mp = mean->data_ptr<spec_t>();
-    const spec_t* vp = var->data_ptr<spec_t>();
-    spec_t* dxp = grad_arr->data_ptr<spec_t>();
-    const A inv = A(1) / A(cols);
-    cpu::parallel_rows(rows, cols, [&](int64_t r) {
-      const A m = cpu::ld<spec_t, A>(mp + r);
-      const A rstd = A(1) / std::sqrt(cpu::ld<spec_t, A>(vp + r) + A(eps));
-      const spec_t* dyr = dyp + r * cols;
-      const spec_t* xr = xp + r * cols;
-      const A s1 = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(dyr + i); }) * inv;
-      const A s2 = cpu::blocked_sum<A>(cols, [&](int64_t i) {
-        return cpu::ld<spec_t, A>(dyr + i) * (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
-      }) * inv;
-      spec_t* dxr = dxp + r * cols;
-      for (int64_t i = 0; i < cols; ++i) {
-        const A xh = (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
-        cpu::st<spec_t, A>(dxr + i, rstd * (cpu::ld<spec_t, A>(dyr + i) - s1 - xh * s2));
-      }
+    cpu::on_stream(stream, "InstanceNormGradientCpu", [=]() {
+      NDArray dy = Dense(out_grads, stream), x = Dense(in_arr, stream);
+      NDArray mean = Dense(mean_arr, stream), var = Dense(var_arr, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* dyp = dy->data_ptr<spec_t>();
+      const spec_t* xp = x->data_ptr<spec_t>();
+      const spec_t* mp = mean->data_ptr<spec_t>();
+      const spec_t* vp = var->data_ptr<spec_t>();
+      spec_t* dxp = grad_arr->data_ptr<spec_t>();
+      const A inv = A(1) / A(cols);
+      cpu::parallel_rows(rows, cols, [&](int64_t r) {
+        const A m = cpu::ld<spec_t, A>(mp + r);
+        const A rstd = A(1) / std::sqrt(cpu::ld<spec_t, A>(vp + r) + A(eps));
+        const spec_t* dyr = dyp + r * cols;
+        const spec_t* xr = xp + r * cols;
+        const A s1 = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(dyr + i); }) * inv;
+        const A s2 = cpu::blocked_sum<A>(cols, [&](int64_t i) {
+          return cpu::ld<spec_t, A>(dyr + i) * (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
+        }) * inv;
+        spec_t* dxr = dxp + r * cols;
+        for (int64_t i = 0; i < cols; ++i) {
+          const A xh = (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
+          cpu::st<spec_t, A>(dxr + i, rstd * (cpu::ld<spec_t, A>(dyr + i) - s1 - xh * s2));
+        }
+      });
     });
   });
 }

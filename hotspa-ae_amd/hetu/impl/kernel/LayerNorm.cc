@@ -152,30 +152,32 @@ void LayerNormCpu(const NDArray& in_arr, const NDArray& ln_scale, const NDArray&
   HT_ASSERT(int64_t(mean_arr->numel()) == rows && int64_t(var_arr->numel()) == rows)
     << "statistics must hold one value per row (" << rows << ")";
   if (in_arr->numel() == 0) return;
-  NDArray x = Dense(in_arr, stream), g = Dense(ln_scale, stream), b = Dense(ln_bias, stream);
   HT_DISPATCH_FLOATING_TYPES(in_arr->dtype(), spec_t, "LayerNormCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* xp = x->data_ptr<spec_t>();
-    const spec_t* gp = g->data_ptr<spec_t>();
-    const spec_t* bp = b->data_ptr<spec_t>();
-    spec_t* mp = mean_arr->data_ptr<spec_t>();
-    spec_t* vp = var_arr->data_ptr<spec_t>();
-    spec_t* yp = out_arr->data_ptr<spec_t>();
-    const A inv = A(1) / A(cols);
-    cpu::parallel_rows(rows, cols, [&](int64_t r) {
-      const spec_t* xr = xp + r * cols;
-      const A mean = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); }) * inv;
-      const A var = cpu::blocked_sum<A>(cols, [&](int64_t i) {
-        const A d = cpu::ld<spec_t, A>(xr + i) - mean;
-        return d * d;
-      }) * inv;
-      cpu::st<spec_t, A>(mp + r, mean);
-      cpu::st<spec_t, A>(vp + r, var);
-      const A rstd = A(1) / std::sqrt(var + A(eps));
-      spec_t* yr = yp + r * cols;
-      for (int64_t i = 0; i < cols; ++i)
-        cpu::st<spec_t, A>(yr + i, (cpu::ld<spec_t, A>(xr + i) - mean) * rstd * cpu::ld<spec_t, A>(gp + i) +
-                                     cpu::ld<spec_t, A>(bp + i));
+    cpu::on_stream(stream, "LayerNormCpu", [=]() {
+      NDArray x = Dense(in_arr, stream), g = Dense(ln_scale, stream), b = Dense(ln_bias, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* xp = x->data_ptr<spec_t>();
+      const spec_t* gp = g->data_ptr<spec_t>();
+      const spec_t* bp = b->data_ptr<spec_t>();
+      spec_t* mp = mean_arr->data_ptr<spec_t>();
+      spec_t* vp = var_arr->data_ptr<spec_t>();
+      spec_t* yp = out_arr->data_ptr<spec_t>();
+      const A inv = A(1) / A(cols);
+      cpu::parallel_rows(rows, cols, [&](int64_t r) {
+        const spec_t* xr = xp + r * cols;
+        const A mean = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); }) * inv;
+        const A var = cpu::blocked_sum<A>(cols, [&](int64_t i) {
+          const A d = cpu::ld<spec_t, A>(xr + i) - mean;
+          return d * d;
+        }) * inv;
+        cpu::st<spec_t, A>(mp + r, mean);
+        cpu::st<spec_t, A>(vp + r, var);
+        const A rstd = A(1) / std::sqrt(var + A(eps));
+        spec_t* yr = yp + r * cols;
+        for (int64_t i = 0; i < cols; ++i)
+          cpu::st<spec_t, A>(yr + i, (cpu::ld<spec_t, A>(xr + i) - mean) * rstd * cpu::ld<spec_t, A>(gp + i) +
+                                       cpu::ld<spec_t, A>(bp + i));
+      });
     });
   });
 }
@@ -210,60 +212,62 @@ void LayerNormGradientCpu(const NDArray& out_grads, const NDArray& in_arr, const
     << "scale / grad_scale / grad_bias must hold " << cols << " values";
   HT_ASSERT(int64_t(mean_arr->numel()) == rows && int64_t(var_arr->numel()) == rows)
     << "statistics must hold one value per row (" << rows << ")";
-  NDArray dy = Dense(out_grads, stream), x = Dense(in_arr, stream), g = Dense(ln_scale, stream);
-  NDArray mean = Dense(mean_arr, stream), var = Dense(var_arr, stream);
   HT_DISPATCH_FLOATING_TYPES(in_arr->dtype(), spec_t, "LayerNormGradientCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* dyp = dy->data_ptr<spec_t>();
-    const spec_t* xp = x->data_ptr<spec_t>();
-    const spec_t* gp = g->data_ptr<spec_t>();
-    const spec_t* mp = mean->data_ptr<spec_t>();
-    const spec_t* vp = var->data_ptr<spec_t>();
-    spec_t* dxp = grad_arr->data_ptr<spec_t>();
-    spec_t* dgp = grad_scale->data_ptr<spec_t>();
-    spec_t* dbp = grad_bias->data_ptr<spec_t>();
-    // column sums, a band of columns per thread: every thread walks all rows of its band
-    constexpr int64_t kBand = 64;
-    const int64_t bands = (cols + kBand - 1) / kBand;
-    cpu::parallel_rows(bands, rows * kBand, [&](int64_t band) {
-      const int64_t c0 = band * kBand, c1 = std::min(cols, c0 + kBand);
-      A sg[kBand], sb[kBand];
-      for (int64_t c = 0; c < kBand; ++c) sg[c] = sb[c] = A(0);
-      for (int64_t r = 0; r < rows; ++r) {
+    cpu::on_stream(stream, "LayerNormGradientCpu", [=]() {
+      NDArray dy = Dense(out_grads, stream), x = Dense(in_arr, stream), g = Dense(ln_scale, stream);
+      NDArray mean = Dense(mean_arr, stream), var = Dense(var_arr, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* dyp = dy->data_ptr<spec_t>();
+      const spec_t* xp = x->data_ptr<spec_t>();
+      const spec_t* gp = g->data_ptr<spec_t>();
+      const spec_t* mp = mean->data_ptr<spec_t>();
+      const spec_t* vp = var->data_ptr<spec_t>();
+      spec_t* dxp = grad_arr->data_ptr<spec_t>();
+      spec_t* dgp = grad_scale->data_ptr<spec_t>();
+      spec_t* dbp = grad_bias->data_ptr<spec_t>();
+      // column sums, a band of columns per thread: every thread walks all rows of its band
+      constexpr int64_t kBand = 64;
+      const int64_t bands = (cols + kBand - 1) / kBand;
+      cpu::parallel_rows(bands, rows * kBand, [&](int64_t band) {
+        const int64_t c0 = band * kBand, c1 = std::min(cols, c0 + kBand);
+        A sg[kBand], sb[kBand];
+        for (int64_t c = 0; c < kBand; ++c) sg[c] = sb[c] = A(0);
+        for (int64_t r = 0; r < rows; ++r) {
+          const A m = cpu::ld<spec_t, A>(mp + r);
+          const A rstd = A(1) / std::sqrt(cpu::ld<spec_t, A>(vp + r) + A(eps));
+          const spec_t* dyr = dyp + r * cols;
+          const spec_t* xr = xp + r * cols;
+          for (int64_t c = c0; c < c1; ++c) {
+            const A d = cpu::ld<spec_t, A>(dyr + c);
+            sb[c - c0] += d;
+            sg[c - c0] += d * (cpu::ld<spec_t, A>(xr + c) - m) * rstd;
+          }
+        }
+        for (int64_t c = c0; c < c1; ++c) {
+          cpu::st<spec_t, A>(dgp + c, sg[c - c0]);
+          cpu::st<spec_t, A>(dbp + c, sb[c - c0]);
+        }
+      });
+      if (in_arr->numel() == 0) return;
+      const A inv = A(1) / A(cols);
+      cpu::parallel_rows(rows, cols, [&](int64_t r) {
         const A m = cpu::ld<spec_t, A>(mp + r);
         const A rstd = A(1) / std::sqrt(cpu::ld<spec_t, A>(vp + r) + A(eps));
         const spec_t* dyr = dyp + r * cols;
         const spec_t* xr = xp + r * cols;
-        for (int64_t c = c0; c < c1; ++c) {
-          const A d = cpu::ld<spec_t, A>(dyr + c);
-          sb[c - c0] += d;
-          sg[c - c0] += d * (cpu::ld<spec_t, A>(xr + c) - m) * rstd;
+        const A s1 = cpu::blocked_sum<A>(cols, [&](int64_t i) {
+          return cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i);
+        }) * inv;
+        const A s2 = cpu::blocked_sum<A>(cols, [&](int64_t i) {
+          return cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i) * (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
+        }) * inv;
+        spec_t* dxr = dxp + r * cols;
+        for (int64_t i = 0; i < cols; ++i) {
+          const A xh = (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
+          const A t = cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i);
+          cpu::st<spec_t, A>(dxr + i, rstd * (t - s1 - xh * s2));
         }
-      }
-      for (int64_t c = c0; c < c1; ++c) {
-        cpu::st<spec_t, A>(dgp + c, sg[c - c0]);
-        cpu::st<spec_t, A>(dbp + c, sb[c - c0]);
-      }
-    });
-    if (in_arr->numel() == 0) return;
-    const A inv = A(1) / A(cols);
-    cpu::parallel_rows(rows, cols, [&](int64_t r) {
-      const A m = cpu::ld<spec_t, A>(mp + r);
-      const A rstd = A(1) / std::sqrt(cpu::ld<spec_t, A>(vp + r) + A(eps));
-      const spec_t* dyr = dyp + r * cols;
-      const spec_t* xr = xp + r * cols;
-      const A s1 = cpu::blocked_sum<A>(cols, [&](int64_t i) {
-        return cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i);
-      }) * inv;
-      const A s2 = cpu::blocked_sum<A>(cols, [&](int64_t i) {
-        return cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i) * (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
-      }) * inv;
-      spec_t* dxr = dxp + r * cols;
-      for (int64_t i = 0; i < cols; ++i) {
-        const A xh = (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
-        const A t = cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i);
-        cpu::st<spec_t, A>(dxr + i, rstd * (t - s1 - xh * s2));
-      }
+      });
     });
   });
 }

@@ -79,17 +79,19 @@ void NLLLossCpu(const NDArray& pred, const NDArray& label, NDArray& loss, const 
   for (size_t i = 0; i < label->ndim(); i++) rows *= label->shape(i);
   const int64_t cols = pred->shape(pred->ndim() - 1);
   if (rows == 0) return;
-  NDArray p = Dense(pred, stream), l = Dense(label, stream);
   HT_DISPATCH_FLOATING_TYPES(pred->dtype(), spec_t, "NLLLossCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* pp = p->data_ptr<spec_t>();
-    const int64_t* lp = l->data_ptr<int64_t>();
-    spec_t* out = loss->data_ptr<spec_t>();
-    for (int64_t r = 0; r < rows; ++r) {
-      const int64_t lab = lp[r];
-      const bool ok = lab >= 0 && lab < cols;
-      cpu::st<spec_t, A>(out + r, ok ? -cpu::ld<spec_t, A>(pp + r * cols + lab) : A(0));
-    }
+    cpu::on_stream(stream, "NLLLossCpu", [=]() {
+      NDArray p = Dense(pred, stream), l = Dense(label, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* pp = p->data_ptr<spec_t>();
+      const int64_t* lp = l->data_ptr<int64_t>();
+      spec_t* out = loss->data_ptr<spec_t>();
+      for (int64_t r = 0; r < rows; ++r) {
+        const int64_t lab = lp[r];
+        const bool ok = lab >= 0 && lab < cols;
+        cpu::st<spec_t, A>(out + r, ok ? -cpu::ld<spec_t, A>(pp + r * cols + lab) : A(0));
+      }
+    });
   });
 }
 
@@ -112,17 +114,19 @@ void NLLLossGradientCpu(const NDArray& pred, const NDArray& label, const NDArray
     << "labels " << label->shape() << " / grad_loss " << grad_loss->shape() << " must hold one value per row of "
     << pred->shape();
   if (rows == 0 || cols == 0) return;
-  NDArray l = Dense(label, stream), g = Dense(grad_loss, stream);
   HT_DISPATCH_FLOATING_TYPES(pred->dtype(), spec_t, "NLLLossGradientCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const int64_t* lp = l->data_ptr<int64_t>();
-    const spec_t* gp = g->data_ptr<spec_t>();
-    spec_t* out = output->data_ptr<spec_t>();
-    cpu::parallel_rows(rows, cols, [&](int64_t r) {
-      spec_t* dr = out + r * cols;
-      for (int64_t c = 0; c < cols; ++c) cpu::st<spec_t, A>(dr + c, A(0));
-      const int64_t lab = lp[r];
-      if (lab >= 0 && lab < cols) cpu::st<spec_t, A>(dr + lab, -cpu::ld<spec_t, A>(gp + r) * A(cols));
+    cpu::on_stream(stream, "NLLLossGradientCpu", [=]() {
+      NDArray l = Dense(label, stream), g = Dense(grad_loss, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const int64_t* lp = l->data_ptr<int64_t>();
+      const spec_t* gp = g->data_ptr<spec_t>();
+      spec_t* out = output->data_ptr<spec_t>();
+      cpu::parallel_rows(rows, cols, [&](int64_t r) {
+        spec_t* dr = out + r * cols;
+        for (int64_t c = 0; c < cols; ++c) cpu::st<spec_t, A>(dr + c, A(0));
+        const int64_t lab = lp[r];
+        if (lab >= 0 && lab < cols) cpu::st<spec_t, A>(dr + lab, -cpu::ld<spec_t, A>(gp + r) * A(cols));
+      });
     });
   });
 }

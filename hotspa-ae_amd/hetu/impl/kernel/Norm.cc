@@ -103,17 +103,19 @@ void NormCpu(const NDArray& input, NDArray& output, int64_t dim, int64_t p, cons
     << "output " << output->shape() << " does not hold the " << before * after << " norms of " << input->shape()
     << " over dimension " << dim;
   if (before * after == 0) return;
-  NDArray x = Dense(input, stream);
   HT_DISPATCH_FLOATING_TYPES(input->dtype(), spec_t, "NormCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* px = x->data_ptr<spec_t>();
-    spec_t* po = output->data_ptr<spec_t>();
-    cpu::parallel_rows(before * after, reduce_size, [&](int64_t o) {
-      const spec_t* base = px + (o / after) * reduce_size * after + (o % after);
-      const A sum = cpu::blocked_sum<A>(reduce_size, [&](int64_t k) {
-        return AbsPow<A>(cpu::ld<spec_t, A>(base + k * after), p);
+    cpu::on_stream(stream, "NormCpu", [=]() {
+      NDArray x = Dense(input, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* px = x->data_ptr<spec_t>();
+      spec_t* po = output->data_ptr<spec_t>();
+      cpu::parallel_rows(before * after, reduce_size, [&](int64_t o) {
+        const spec_t* base = px + (o / after) * reduce_size * after + (o % after);
+        const A sum = cpu::blocked_sum<A>(reduce_size, [&](int64_t k) {
+          return AbsPow<A>(cpu::ld<spec_t, A>(base + k * after), p);
+        });
+        cpu::st<spec_t, A>(po + o, p == 1 ? sum : p == 2 ? std::sqrt(sum) : std::pow(sum, A(1) / A(p)));
       });
-      cpu::st<spec_t, A>(po + o, p == 1 ? sum : p == 2 ? std::sqrt(sum) : std::pow(sum, A(1) / A(p)));
     });
   });
 }
@@ -142,25 +144,27 @@ void NormGradientCpu(const NDArray& input, const NDArray& output, const NDArray&
     << "norm " << output->shape() << " and its gradient " << output_grad->shape() << " must hold " << before * after
     << " values for " << input->shape() << " over dimension " << dim;
   if (input->numel() == 0) return;
-  NDArray x = Dense(input, stream), n = Dense(output, stream), g = Dense(output_grad, stream);
   HT_DISPATCH_FLOATING_TYPES(input->dtype(), spec_t, "NormGradientCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* px = x->data_ptr<spec_t>();
-    const spec_t* pn = n->data_ptr<spec_t>();
-    const spec_t* pg = g->data_ptr<spec_t>();
-    spec_t* pd = input_grad->data_ptr<spec_t>();
-    cpu::parallel_rows(before * reduce_size, after, [&](int64_t row) {
-      const int64_t b = row / reduce_size;
-      for (int64_t a = 0; a < after; ++a) {
-        const A v = cpu::ld<spec_t, A>(px + row * after + a);
-        const A nv = cpu::ld<spec_t, A>(pn + b * after + a), gv = cpu::ld<spec_t, A>(pg + b * after + a);
-        A r;
-        if (p == 1) r = (v > A(0) ? A(1) : v < A(0) ? A(-1) : A(0)) * gv;
-        else if (nv == A(0)) r = A(0);
-        else if (p == 2) r = gv * v / nv;
-        else r = v * std::pow(std::fabs(v), A(p - 2)) * gv / std::pow(nv, A(p - 1));
-        cpu::st<spec_t, A>(pd + row * after + a, r);
-      }
+    cpu::on_stream(stream, "NormGradientCpu", [=]() {
+      NDArray x = Dense(input, stream), n = Dense(output, stream), g = Dense(output_grad, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* px = x->data_ptr<spec_t>();
+      const spec_t* pn = n->data_ptr<spec_t>();
+      const spec_t* pg = g->data_ptr<spec_t>();
+      spec_t* pd = input_grad->data_ptr<spec_t>();
+      cpu::parallel_rows(before * reduce_size, after, [&](int64_t row) {
+        const int64_t b = row / reduce_size;
+        for (int64_t a = 0; a < after; ++a) {
+          const A v = cpu::ld<spec_t, A>(px + row * after + a);
+          const A nv = cpu::ld<spec_t, A>(pn + b * after + a), gv = cpu::ld<spec_t, A>(pg + b * after + a);
+          A r;
+          if (p == 1) r = (v > A(0) ? A(1) : v < A(0) ? A(-1) : A(0)) * gv;
+          else if (nv == A(0)) r = A(0);
+          else if (p == 2) r = gv * v / nv;
+          else r = v * std::pow(std::fabs(v), A(p - 2)) * gv / std::pow(nv, A(p - 1));
+          cpu::st<spec_t, A>(pd + row * after + a, r);
+        }
+      });
     });
   });
 }

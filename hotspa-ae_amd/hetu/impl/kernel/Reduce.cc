@@ -141,7 +141,7 @@ template <typename T, typename A> inline void host_st(T* p, A v) {
 }
 
 template <typename T, typename O>
-void HostReduce(const NDArray& in, NDArray& out, const std::vector<bool>& reduced, int op) {
+void HostReduce(const NDArray& in, const NDArray& out, const std::vector<bool>& reduced, int op) {
   using A = typename HostArith<T>::type;
   const int64_t nd = int64_t(in->ndim());
   // kept and reduced extents with their input strides, outermost first
@@ -222,7 +222,7 @@ void HostReduce(const NDArray& in, NDArray& out, const std::vector<bool>& reduce
 }
 
 void HostReduceEntry(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax, int op,
-                     const char* who) {
+                     const char* who, const Stream& stream) {
   HT_ASSERT_CPU_DEVICE(in_arr);
   HT_ASSERT_SAME_DEVICE(in_arr, out_arr);
   HT_ASSERT_CONTIGUOUS(out_arr);
@@ -244,30 +244,37 @@ void HostReduceEntry(const NDArray& in_arr, NDArray& out_arr, const int64_t* axe
     << who << ": the output is of the input's type, or float32 for a 16-bit floating-point input";
   HT_NOT_IMPLEMENTED_IF(widened && (op == HK_REDUCE_MAX || op == HK_REDUCE_MIN)) << who << ": max / min have no widened output";
   HT_DISPATCH_INTEGER_AND_FLOATING_TYPES(in_arr->dtype(), spec_t, who, [&]() {
-    if (widened) {
-      if constexpr (std::is_same<spec_t, bfloat16>::value || std::is_same<spec_t, float16>::value)
-        HostReduce<spec_t, float>(in_arr, out_arr, reduced, op);
-    } else {
-      HostReduce<spec_t, spec_t>(in_arr, out_arr, reduced, op);
-    }
+    cpu::on_stream(stream, who, [=]() {   // the axis flags travel with the task; the caller's axis list is not kept
+      if (widened) {
+        if constexpr (std::is_same<spec_t, bfloat16>::value || std::is_same<spec_t, float16>::value)
+          HostReduce<spec_t, float>(in_arr, out_arr, reduced, op);
+      } else {
+        HostReduce<spec_t, spec_t>(in_arr, out_arr, reduced, op);
+      }
+    });
   });
 }
 } // namespace
 
-void ReduceSumCpu(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax, const Stream&) {
-  HostReduceEntry(in_arr, out_arr, axes, num_ax, HK_REDUCE_SUM, "ReduceSumCpu");
+void ReduceSumCpu(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax,
+                  const Stream& stream) {
+  HostReduceEntry(in_arr, out_arr, axes, num_ax, HK_REDUCE_SUM, "ReduceSumCpu", stream);
 }
-void ReduceMeanCpu(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax, const Stream&) {
-  HostReduceEntry(in_arr, out_arr, axes, num_ax, HK_REDUCE_MEAN, "ReduceMeanCpu");
+void ReduceMeanCpu(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax,
+                   const Stream& stream) {
+  HostReduceEntry(in_arr, out_arr, axes, num_ax, HK_REDUCE_MEAN, "ReduceMeanCpu", stream);
 }
-void ReduceMaxCpu(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax, const Stream&) {
-  HostReduceEntry(in_arr, out_arr, axes, num_ax, HK_REDUCE_MAX, "ReduceMaxCpu");
+void ReduceMaxCpu(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax,
+                  const Stream& stream) {
+  HostReduceEntry(in_arr, out_arr, axes, num_ax, HK_REDUCE_MAX, "ReduceMaxCpu", stream);
 }
-void ReduceMinCpu(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax, const Stream&) {
-  HostReduceEntry(in_arr, out_arr, axes, num_ax, HK_REDUCE_MIN, "ReduceMinCpu");
+void ReduceMinCpu(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax,
+                  const Stream& stream) {
+  HostReduceEntry(in_arr, out_arr, axes, num_ax, HK_REDUCE_MIN, "ReduceMinCpu", stream);
 }
-void ReduceProdCpu(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax, const Stream&) {
-  HostReduceEntry(in_arr, out_arr, axes, num_ax, HK_REDUCE_PROD, "ReduceProdCpu");
+void ReduceProdCpu(const NDArray& in_arr, NDArray& out_arr, const int64_t* axes, int64_t num_ax,
+                   const Stream& stream) {
+  HostReduceEntry(in_arr, out_arr, axes, num_ax, HK_REDUCE_PROD, "ReduceProdCpu", stream);
 }
 
 void ReduceCpu(const NDArray& input, NDArray& output, const HTAxes& axes, ReductionType red_type,

@@ -112,22 +112,24 @@ void SoftmaxCrossEntropyCpu(const NDArray& input, const NDArray& label, NDArray&
   const int64_t cols = input->shape(indim - 1);
   HT_ASSERT(int64_t(output->numel()) == rows) << "loss " << output->shape() << " must hold one value per row";
   if (rows * cols == 0) return;
-  NDArray x = Dense(input, stream), l = Dense(label, stream);
   HT_DISPATCH_FLOATING_TYPES(input->dtype(), spec_t, "SoftmaxCrossEntropyCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* xp = x->data_ptr<spec_t>();
-    const spec_t* lp = l->data_ptr<spec_t>();
-    spec_t* out = output->data_ptr<spec_t>();
-    cpu::parallel_rows(rows, cols, [&](int64_t r) {
-      const spec_t* xr = xp + r * cols;
-      const spec_t* lr = lp + r * cols;
-      const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
-      const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
-      const A lse = m + std::log(sum);
-      const A acc = cpu::blocked_sum<A>(cols, [&](int64_t i) {
-        return cpu::ld<spec_t, A>(lr + i) * (lse - cpu::ld<spec_t, A>(xr + i));
+    cpu::on_stream(stream, "SoftmaxCrossEntropyCpu", [=]() {
+      NDArray x = Dense(input, stream), l = Dense(label, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* xp = x->data_ptr<spec_t>();
+      const spec_t* lp = l->data_ptr<spec_t>();
+      spec_t* out = output->data_ptr<spec_t>();
+      cpu::parallel_rows(rows, cols, [&](int64_t r) {
+        const spec_t* xr = xp + r * cols;
+        const spec_t* lr = lp + r * cols;
+        const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
+        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+        const A lse = m + std::log(sum);
+        const A acc = cpu::blocked_sum<A>(cols, [&](int64_t i) {
+          return cpu::ld<spec_t, A>(lr + i) * (lse - cpu::ld<spec_t, A>(xr + i));
+        });
+        cpu::st<spec_t, A>(out + r, acc);
       });
-      cpu::st<spec_t, A>(out + r, acc);
     });
   });
 }
@@ -151,22 +153,24 @@ void SoftmaxCrossEntropyGradientCpu(const NDArray& input_y, const NDArray& label
   const int64_t cols = input_y->shape(indim - 1);
   HT_ASSERT(int64_t(grad->numel()) == rows) << "grad " << grad->shape() << " must hold one value per row";
   if (rows * cols == 0) return;
-  NDArray x = Dense(input_y, stream), l = Dense(label, stream), g = Dense(grad, stream);
   HT_DISPATCH_FLOATING_TYPES(input_y->dtype(), spec_t, "SoftmaxCrossEntropyGradientCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* xp = x->data_ptr<spec_t>();
-    const spec_t* lp = l->data_ptr<spec_t>();
-    const spec_t* gp = g->data_ptr<spec_t>();
-    spec_t* out = output->data_ptr<spec_t>();
-    cpu::parallel_rows(rows, cols, [&](int64_t r) {
-      const spec_t* xr = xp + r * cols;
-      const spec_t* lr = lp + r * cols;
-      spec_t* dr = out + r * cols;
-      const A gr = cpu::ld<spec_t, A>(gp + r);
-      const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
-      const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
-      for (int64_t i = 0; i < cols; ++i)
-        cpu::st<spec_t, A>(dr + i, (std::exp(cpu::ld<spec_t, A>(xr + i) - m) / sum - cpu::ld<spec_t, A>(lr + i)) * gr);
+    cpu::on_stream(stream, "SoftmaxCrossEntropyGradientCpu", [=]() {
+      NDArray x = Dense(input_y, stream), l = Dense(label, stream), g = Dense(grad, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* xp = x->data_ptr<spec_t>();
+      const spec_t* lp = l->data_ptr<spec_t>();
+      const spec_t* gp = g->data_ptr<spec_t>();
+      spec_t* out = output->data_ptr<spec_t>();
+      cpu::parallel_rows(rows, cols, [&](int64_t r) {
+        const spec_t* xr = xp + r * cols;
+        const spec_t* lr = lp + r * cols;
+        spec_t* dr = out + r * cols;
+        const A gr = cpu::ld<spec_t, A>(gp + r);
+        const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
+        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+        for (int64_t i = 0; i < cols; ++i)
+          cpu::st<spec_t, A>(dr + i, (std::exp(cpu::ld<spec_t, A>(xr + i) - m) / sum - cpu::ld<spec_t, A>(lr + i)) * gr);
+      });
     });
   });
 }

@@ -134,20 +134,22 @@ void SoftmaxCrossEntropySparseCpu(const NDArray& pred, const NDArray& label, NDA
     << pred->shape();
   if (rows == 0) return;
   HT_VALUE_ERROR_IF(cols == 0) << "cross entropy over zero classes";
-  NDArray p = Dense(pred, stream), l = Dense(label, stream);
   HT_DISPATCH_FLOATING_TYPES(pred->dtype(), spec_t, "SoftmaxCrossEntropySparseCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* pp = p->data_ptr<spec_t>();
-    const int64_t* lp = l->data_ptr<int64_t>();
-    spec_t* out = loss->data_ptr<spec_t>();
-    cpu::parallel_rows(rows, cols, [&](int64_t r) {
-      const int64_t lab = lp[r];
-      if (lab == ignored_index) { cpu::st<spec_t, A>(out + r, A(0)); return; }
-      if (lab < 0 || lab >= cols) { cpu::st<spec_t, A>(out + r, std::numeric_limits<A>::quiet_NaN()); return; }
-      const spec_t* xr = pp + r * cols;
-      const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
-      const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
-      cpu::st<spec_t, A>(out + r, std::log(sum) - (cpu::ld<spec_t, A>(xr + lab) - m));
+    cpu::on_stream(stream, "SoftmaxCrossEntropySparseCpu", [=]() {
+      NDArray p = Dense(pred, stream), l = Dense(label, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* pp = p->data_ptr<spec_t>();
+      const int64_t* lp = l->data_ptr<int64_t>();
+      spec_t* out = loss->data_ptr<spec_t>();
+      cpu::parallel_rows(rows, cols, [&](int64_t r) {
+        const int64_t lab = lp[r];
+        if (lab == ignored_index) { cpu::st<spec_t, A>(out + r, A(0)); return; }
+        if (lab < 0 || lab >= cols) { cpu::st<spec_t, A>(out + r, std::numeric_limits<A>::quiet_NaN()); return; }
+        const spec_t* xr = pp + r * cols;
+        const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
+        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+        cpu::st<spec_t, A>(out + r, std::log(sum) - (cpu::ld<spec_t, A>(xr + lab) - m));
+      });
     });
   });
 }
@@ -169,33 +171,35 @@ void SoftmaxCrossEntropySparseGradientCpu(const NDArray& pred, const NDArray& la
     << "labels " << label->shape() << " / grad_loss " << grad_loss->shape()
     << " must hold one value per row of " << pred->shape();
   if (pred->numel() == 0) return;
-  NDArray p = Dense(pred, stream), l = Dense(label, stream), gl = Dense(grad_loss, stream);
   HT_DISPATCH_FLOATING_TYPES(pred->dtype(), spec_t, "SoftmaxCrossEntropySparseGradientCpu", [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* pp = p->data_ptr<spec_t>();
-    const int64_t* lp = l->data_ptr<int64_t>();
-    const spec_t* gp = gl->data_ptr<spec_t>();
-    spec_t* out = output->data_ptr<spec_t>();
-    cpu::parallel_rows(rows, cols, [&](int64_t r) {
-      const int64_t lab = lp[r];
-      spec_t* dr = out + r * cols;
-      if (lab == ignored_index) {
-        for (int64_t i = 0; i < cols; ++i) cpu::st<spec_t, A>(dr + i, A(0));
-        return;
-      }
-      if (lab < 0 || lab >= cols) {
-        for (int64_t i = 0; i < cols; ++i) cpu::st<spec_t, A>(dr + i, std::numeric_limits<A>::quiet_NaN());
-        return;
-      }
-      const spec_t* xr = pp + r * cols;
-      const A g = cpu::ld<spec_t, A>(gp + r);
-      const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
-      const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
-      const A scale = g / sum;
-      for (int64_t i = 0; i < cols; ++i) {
-        const A pr = std::exp(cpu::ld<spec_t, A>(xr + i) - m) * scale;
-        cpu::st<spec_t, A>(dr + i, i == lab ? pr - g : pr);
-      }
+    cpu::on_stream(stream, "SoftmaxCrossEntropySparseGradientCpu", [=]() {
+      NDArray p = Dense(pred, stream), l = Dense(label, stream), gl = Dense(grad_loss, stream);
+      using A = typename cpu::Arith<spec_t>::type;
+      const spec_t* pp = p->data_ptr<spec_t>();
+      const int64_t* lp = l->data_ptr<int64_t>();
+      const spec_t* gp = gl->data_ptr<spec_t>();
+      spec_t* out = output->data_ptr<spec_t>();
+      cpu::parallel_rows(rows, cols, [&](int64_t r) {
+        const int64_t lab = lp[r];
+        spec_t* dr = out + r * cols;
+        if (lab == ignored_index) {
+          for (int64_t i = 0; i < cols; ++i) cpu::st<spec_t, A>(dr + i, A(0));
+          return;
+        }
+        if (lab < 0 || lab >= cols) {
+          for (int64_t i = 0; i < cols; ++i) cpu::st<spec_t, A>(dr + i, std::numeric_limits<A>::quiet_NaN());
+          return;
+        }
+        const spec_t* xr = pp + r * cols;
+        const A g = cpu::ld<spec_t, A>(gp + r);
+        const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
+        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+        const A scale = g / sum;
+        for (int64_t i = 0; i < cols; ++i) {
+          const A pr = std::exp(cpu::ld<spec_t, A>(xr + i) - m) * scale;
+          cpu::st<spec_t, A>(dr + i, i == lab ? pr - g : pr);
+        }
+      });
     });
   });
 }

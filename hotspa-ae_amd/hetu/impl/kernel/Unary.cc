@@ -45,23 +45,28 @@ void UnaryHost(int op, const char* who, const NDArray& input, NDArray& output, c
   HT_ASSERT_SAME_DTYPE(input, output);
   HT_ASSERT_CONTIGUOUS(output);
   if (input->numel() == 0) return;
-  NDArray x = Dense(input, stream);
   const int64_t n = int64_t(input->numel());
   if (op == HK_UNARY_NEG) {
     HT_DISPATCH_INTEGER_AND_FLOATING_TYPES(input->dtype(), spec_t, who, [&]() {
-      const spec_t* px = x->data_ptr<spec_t>();
-      spec_t* po = output->data_ptr<spec_t>();
-      cpu::parallel_for(n, [&](int64_t i) { po[i] = cpu::negate<spec_t>(px[i]); });
+      cpu::on_stream(stream, who, [=]() {
+        NDArray x = Dense(input, stream);
+        const spec_t* px = x->data_ptr<spec_t>();
+        spec_t* po = output->data_ptr<spec_t>();
+        cpu::parallel_for(n, [&](int64_t i) { po[i] = cpu::negate<spec_t>(px[i]); });
+      });
     });
     return;
   }
   HT_DISPATCH_FLOATING_TYPES(input->dtype(), spec_t, who, [&]() {
-    using A = typename cpu::Arith<spec_t>::type;
-    const spec_t* px = x->data_ptr<spec_t>();
-    spec_t* po = output->data_ptr<spec_t>();
-    cpu::parallel_for(n, [&](int64_t i) {
-      const A v = cpu::ld<spec_t, A>(px + i);
-      cpu::st<spec_t, A>(po + i, op == HK_UNARY_EXP ? std::exp(v) : op == HK_UNARY_LOG ? std::log(v) : std::sqrt(v));
+    cpu::on_stream(stream, who, [=]() {
+      using A = typename cpu::Arith<spec_t>::type;
+      NDArray x = Dense(input, stream);
+      const spec_t* px = x->data_ptr<spec_t>();
+      spec_t* po = output->data_ptr<spec_t>();
+      cpu::parallel_for(n, [&](int64_t i) {
+        const A v = cpu::ld<spec_t, A>(px + i);
+        cpu::st<spec_t, A>(po + i, op == HK_UNARY_EXP ? std::exp(v) : op == HK_UNARY_LOG ? std::log(v) : std::sqrt(v));
+      });
     });
   });
 }

@@ -1,4 +1,5 @@
 #include "hetu/impl/stream/HIPStream.h"
+#include "hetu/impl/stream/CPUStream.h"
 
 #include <mutex>
 
@@ -92,12 +93,16 @@ int64_t HIPEvent::TimeSince(const Event& event) const {
 
 void Stream::Sync() const {
   if (_device.is_cuda()) hetu::impl::SyncStream(*this);
+  else if (_device.is_cpu()) hetu::impl::CPUStream(*this).Sync();
 }
 
 void SynchronizeAllStreams(const Device& device) {
   if (device.is_cuda()) {
     hetu::impl::SyncAllStreams(device);
+  } else if (device.is_cpu()) {
+    hetu::impl::SynchronizeAllCPUStreams();
   } else if (device.is_undetermined()) {
+    hetu::impl::SynchronizeAllCPUStreams();
     int n = 0;
     if (hk_device_count(&n) != HK_OK) return;
     for (int i = 0; i < n && i < HT_MAX_DEVICE_INDEX; ++i) hetu::impl::SyncAllStreams(Device(kCUDA, DeviceIndex(i)));

@@ -9,16 +9,42 @@
 
 #include "hetu/core/dtype.h"
 #include "hetu/core/ndarray.h"
+#include "hetu/impl/stream/CPUStream.h"
 
 #include <cmath>
 #include <cstdint>
 #include <limits>
 #include <type_traits>
+#include <utility>
 #include <vector>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 
 namespace hetu {
 namespace impl {
 namespace cpu {
+
+// The computing part of a host kernel goes onto its stream: it runs after whatever the stream was given before and
+// the call returns at once (stream index 0: in the calling thread, before the call returns), as the reference's
+// host kernels do with CPUStream::EnqueueTask (hetu/impl/kernel/Softmax.cc:31-45 of the reference).  The task owns
+// copies of the array handles it works on.  Argument checks stay in front of it, in the calling thread.
+template <typename F>
+inline void on_stream(const Stream& stream, const char* name, F&& body) {
+  CPUStream(stream).EnqueueTask(std::function<void()>(std::forward<F>(body)), name);
+}
+
+// size of the OpenMP team of a host kernel: what SetHostKernelThreads asked for, else the runtime's default for
+// the thread the kernel runs on
+inline int team_size() {
+  const int asked = HostKernelThreads();
+#ifdef _OPENMP
+  return asked > 0 ? asked : omp_get_max_threads();
+#else
+  return asked > 0 ? asked : 1;
+#endif
+}
 
 // arithmetic type of a storage type
 template <typename T> struct Arith { using type = float; };
@@ -107,7 +133,7 @@ inline T negate(T x) {
 // f(i) for i in [0, n), shared out over the OpenMP team when there is enough of it
 template <typename F>
 inline void parallel_for(int64_t n, F f) {
-#pragma omp parallel for schedule(static) if (n >= (int64_t(1) << 16))
+#pragma omp parallel for schedule(static) num_threads(team_size()) if (n >= (int64_t(1) << 16))
   for (int64_t i = 0; i < n; ++i) f(i);
 }
 
@@ -122,7 +148,7 @@ inline void for_each_run(int nd, const int64_t* shape, const int64_t* sa, const 
   int64_t runs = 1;
   for (int d = 0; d < nd - 1; ++d) runs *= shape[d];
   const bool par = runs > 1 && runs * inner >= (int64_t(1) << 16);
-#pragma omp parallel for schedule(static) if (par)
+#pragma omp parallel for schedule(static) num_threads(team_size()) if (par)
   for (int64_t r = 0; r < runs; ++r) {
     int64_t rem = r, oa = 0, ob = 0;
     for (int d = nd - 2; d >= 0; --d) {
@@ -139,7 +165,7 @@ inline void for_each_run(int nd, const int64_t* shape, const int64_t* sa, const 
 template <typename F>
 inline void parallel_rows(int64_t rows, int64_t work_per_row, F f) {
   const bool par = rows > 1 && rows * work_per_row >= (int64_t(1) << 16);
-#pragma omp parallel for schedule(static) if (par)
+#pragma omp parallel for schedule(static) num_threads(team_size()) if (par)
   for (int64_t r = 0; r < rows; ++r) f(r);
 }
 

@@ -121,6 +121,17 @@ def stream_sync(stream=DEFAULT_STREAM, device=0):
     check(lib().ht_stream_sync(ctypes.c_int(device), ctypes.c_int(stream)))
 
 
+def host_stream_sync(stream=DEFAULT_STREAM):
+    """Waits for the host stream of that index and raises what a host kernel on it failed with."""
+    check(lib().ht_host_stream_sync(ctypes.c_int(stream)))
+
+
+def set_host_async(on):
+    """Host calls return once their work is on its stream (True) or once it has finished (False, the default);
+    returns the previous setting.  While on, the caller keeps the arrays alive until host_stream_sync."""
+    return bool(lib().ht_set_host_async(ctypes.c_int(int(bool(on)))))
+
+
 def set_host_threads(n):
     """OpenMP team size of the host twins; returns the size now in force (n <= 0 only asks)."""
     return int(lib().ht_set_host_threads(ctypes.c_int(int(n))))

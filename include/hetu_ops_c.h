@@ -179,9 +179,17 @@ HT_API int ht_sceloss_gradient(const HtArray* preds, const HtArray* labels, cons
 /* ---- streams and the device memory pool ---- */
 HT_API int ht_stream_sync(int device_index, int stream_index);
 HT_API int ht_synchronize_all(void);
-/* OpenMP team size of the host twins (the ...Cpu kernels), set on the calling thread through the library's own
- * OpenMP runtime; threads <= 0 only asks.  Returns the team size now in force.  For the CPU baseline legs of the
- * benchmark (all threads / one thread). */
+/* Host streams (Device(kCPU), index 1..15) are task queues with one worker thread each, as in
+ * hetu/impl/stream/CPUStream.cc:15-48 of the reference; index 0 runs in the calling thread.  Arrays handed to this C
+ * face are borrowed, so by default every call on host arrays has finished when it returns.  ht_set_host_async(1)
+ * makes host calls return as soon as their work is on its stream; the caller then keeps the buffers alive and
+ * unchanged until ht_host_stream_sync (or ht_synchronize_all), which also reports a failure of such work.  Returns
+ * the previous setting. */
+HT_API int ht_set_host_async(int on);
+HT_API int ht_host_stream_sync(int stream_index);
+/* OpenMP team size of the host twins (the ...Cpu kernels), whichever thread runs them; threads <= 0 goes back to
+ * the OpenMP runtime's default.  Returns the team size now in force.  For the CPU baseline legs of the benchmark
+ * (all threads / one thread). */
 HT_API int ht_set_host_threads(int threads);
 HT_API int ht_pool_alloc(int device_index, size_t bytes, int stream_index, void** ptr, uint64_t* id,
                          size_t* granted_bytes);

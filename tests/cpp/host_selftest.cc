@@ -5,14 +5,19 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <atomic>
 #include <functional>
+#include <future>
 #include <set>
 #include <string>
+#include <thread>
+#include <vector>
 
 #include "hetu/core/ndarray.h"
 #include "hetu/graph/ops/kernel_links.h"
 #include "hetu/impl/memory/CachingMemoryPool.h"
 #include "hetu/impl/random/CPURandomState.h"
+#include "hetu/impl/stream/CPUStream.h"
 #include "hetu/impl/utils/dispatch.h"
 
 using namespace hetu;
@@ -244,7 +249,8 @@ int main() {
     CHECK(throws<value_error>([&] { NDArray::view(a, {5, -1}); }));
     NDArray t = NDArray::permute(a, {2, 0, 1});
     CHECK((t->shape() == HTShape{4, 2, 3}) && (t->stride() == HTStride{1, 12, 4}) && !t->is_contiguous());
-    NDArray tc = NDArray::contiguous(t);
+    NDArray tc = NDArray::contiguous(t);   // on the host computing stream: a task, waited for before reading
+    SynchronizeAllStreams(Device(kCPU));
     CHECK(tc->is_contiguous() && tc->data_ptr<float>() != p);
     // tc[k][i][j] = a[i][j][k]
     for (int k = 0; k < 4; ++k)
@@ -268,14 +274,17 @@ int main() {
     for (int i = 0; i < 32; ++i) a->data_ptr<float>()[i] = float(i % 8);
     for (int i = 0; i < 8; ++i) g->data_ptr<float>()[i] = 1.f;
     NDArray sm = NDArray::softmax(a, 1);
+    Stream(Device(kCPU), kComputingStream).Sync();
     for (int r = 0; r < 4; ++r) {
       float s = 0.f;
       for (int c = 0; c < 8; ++c) s += sm->data_ptr<float>()[r * 8 + c];
       CHECK(std::fabs(s - 1.f) < 1e-6f);
     }
     NDArray cs = NDArray::sum(a, {0});
+    Stream(Device(kCPU), kComputingStream).Sync();
     for (int c = 0; c < 8; ++c) CHECK(cs->data_ptr<float>()[c] == 4.f * float(c));
     NDArrayList ln = NDArray::layernorm(a, g, NDArray::zeros({8}, Device(kCPU), kFloat32), {8});
+    Stream(Device(kCPU), kComputingStream).Sync();
     CHECK(std::fabs(ln[1]->data_ptr<float>()[0] - 3.5f) < 1e-6f);     // mean of 0..7
     CHECK(std::fabs(ln[2]->data_ptr<float>()[0] - 5.25f) < 1e-5f);    // variance of 0..7
     // the fused variant exists for the accelerator only: the switch itself refuses
@@ -283,12 +292,153 @@ int main() {
     NDArray lab = NDArray::zeros({4}, Device(kCPU), kInt64);
     lab->data_ptr<int64_t>()[1] = -1;   // ignored
     NDArray loss = NDArray::sceloss(a, lab, int64_t(-1), kNONE);
+    Stream(Device(kCPU), kComputingStream).Sync();
     CHECK(loss->data_ptr<float>()[1] == 0.f && loss->data_ptr<float>()[0] > 7.f);
     // an accelerator kernel handed host arrays fails its device assertion
     NDArray out = NDArray::empty_like(a);
     CHECK(throws<assertion_error>([&] { hetu::impl::SoftmaxCuda(a, out, 1, Stream(Device(kCUDA, 0), 1)); }));
     CHECK(throws<assertion_error>(
       [&] { hetu::impl::ReduceCuda(a, out, {0}, kSUM, Stream(Device(kCUDA, 0), 1)); }));
+  });
+
+  run("host streams: a worker per stream, order within a stream, events across streams, failures at Sync", [] {
+    using hetu::impl::CPUEvent;
+    using hetu::impl::CPUStream;
+    using hetu::impl::GetCPUStream;
+    const Device cpu(kCPU);
+    // the blocking stream runs in the calling thread, before EnqueueTask returns, and throws to the caller
+    std::thread::id ran_on;
+    GetCPUStream(kBlockingStream).EnqueueTask([&] { ran_on = std::this_thread::get_id(); });
+    CHECK(ran_on == std::this_thread::get_id());
+    CHECK(throws<value_error>([] { GetCPUStream(kBlockingStream).EnqueueTask([] { HT_VALUE_ERROR << "now"; }); }, "now"));
+    // any other stream has its own thread and keeps the order of its tasks
+    std::vector<int> order;
+    std::thread::id worker3, worker4;
+    std::promise<void> gate;
+    std::shared_future<void> open = gate.get_future().share();
+    CPUStream s3 = GetCPUStream(3), s4 = GetCPUStream(4);
+    const uint64_t before = s3.num_enqueued_tasks();
+    s3.EnqueueTask([&, open] { open.wait(); worker3 = std::this_thread::get_id(); order.push_back(1); }, "first");
+    for (int i = 2; i <= 50; ++i) s3.EnqueueTask([&order, i] { order.push_back(i); });
+    CHECK(s3.num_enqueued_tasks() == before + 50 && s3.num_completed_tasks() == before);   // nothing ran: the call returned
+    CHECK(hetu::impl::AnyCPUStreamBusy());
+    s4.EnqueueTask([&] { worker4 = std::this_thread::get_id(); });
+    s4.Sync();                         // stream 4 does not wait for stream 3
+    CHECK(order.empty());
+    gate.set_value();
+    Stream(cpu, 3).Sync();             // through the device-independent handle
+    CHECK(order.size() == 50);
+    for (int i = 0; i < 50; ++i) CHECK(order[size_t(i)] == i + 1);
+    CHECK(worker3 != std::this_thread::get_id() && worker4 != std::this_thread::get_id() && worker3 != worker4);
+    CHECK(s3.num_completed_tasks() == before + 50);
+    // a task enqueued from the stream's own worker runs inside the running task, not behind it
+    std::vector<int> nested;
+    s3.EnqueueTask([&] {
+      nested.push_back(1);
+      GetCPUStream(3).EnqueueTask([&] { nested.push_back(2); });
+      GetCPUStream(3).Sync();          // from the worker: nothing to wait for
+      nested.push_back(3);
+    });
+    s3.Sync();
+    CHECK((nested == std::vector<int>{1, 2, 3}));
+    // events: stream 4 waits for a point of stream 3
+    std::promise<void> gate2;
+    std::shared_future<void> open2 = gate2.get_future().share();
+    std::atomic<int> stage{0};
+    CPUEvent start, reached;
+    CHECK(!reached.IsRecorded());
+    CHECK(throws<assertion_error>([&] { reached.Sync(); }));
+    start.Record(Stream(cpu, 3));
+    s3.EnqueueTask([&, open2] { open2.wait(); stage = 1; });
+    reached.Record(Stream(cpu, 3));
+    reached.Block(Stream(cpu, 4));
+    int seen_by_4 = -1;
+    s4.EnqueueTask([&] { seen_by_4 = stage.load(); });
+    CHECK(seen_by_4 == -1);
+    gate2.set_value();
+    reached.Sync();
+    s4.Sync();
+    CHECK(seen_by_4 == 1);
+    CHECK(reached.TimeSince(start) >= 0);
+    {   // an event may go away while its stream still has to reach it
+      std::promise<void> gate3;
+      std::shared_future<void> open3 = gate3.get_future().share();
+      s3.EnqueueTask([open3] { open3.wait(); });
+      { CPUEvent gone; gone.Record(Stream(cpu, 3)); }
+      gate3.set_value();
+      s3.Sync();
+    }
+    // a task that throws: its future carries the failure, and the next Sync on the stream reports the first one, once
+    std::future<void> failed = s3.EnqueueTask([] { HT_VALUE_ERROR << "task one"; }, "one");
+    s3.EnqueueTask([] { HT_RUNTIME_ERROR << "task two"; }, "two");
+    int after = 0;
+    s3.EnqueueTask([&] { after = 7; });
+    CHECK(throws<value_error>([&] { s3.Sync(); }, "task one"));
+    CHECK(after == 7);                 // the stream went on
+    CHECK(throws<value_error>([&] { failed.get(); }, "task one"));
+    s3.Sync();                         // reported once
+    s3.EnqueueTask([] { HT_VALUE_ERROR << "again"; });
+    CHECK(throws<value_error>([] { SynchronizeAllStreams(Device(kCPU)); }, "again"));
+    CHECK(!hetu::impl::AnyCPUStreamBusy());
+    CHECK(throws<assertion_error>([] { CPUStream(Stream(Device(kCUDA, 0), 1)); }));
+  });
+
+  run("host twins on a stream: argument checks at the call, the work in stream order, results after Sync", [] {
+    const Device cpu(kCPU);
+    const Stream st(cpu, 5);
+    const int64_t rows = 64, cols = 96;
+    NDArray x = NDArray::empty({rows, cols}, cpu, kFloat32);
+    for (int64_t i = 0; i < rows * cols; ++i) x->data_ptr<float>()[i] = float((i * 37) % 101) * 0.05f - 2.f;
+    // the same chain on the blocking stream (in this thread) and on stream 5 behind a gate
+    auto chain = [&](const Stream& s, NDArray& y, NDArray& e, NDArray& sum) {
+      hetu::impl::SoftmaxCpu(x, y, 1, s);
+      hetu::impl::ExpCpu(y, e, s);                           // reads what the task before it writes
+      hetu::impl::ReduceCpu(e, sum, {1}, kSUM, s);
+    };
+    NDArray y0 = NDArray::empty_like(x), e0 = NDArray::empty_like(x), s0 = NDArray::empty({rows}, cpu, kFloat32);
+    chain(Stream(cpu, kBlockingStream), y0, e0, s0);
+    NDArray y1 = NDArray::zeros({rows, cols}, cpu, kFloat32), e1 = NDArray::zeros({rows, cols}, cpu, kFloat32);
+    NDArray s1 = NDArray::zeros({rows}, cpu, kFloat32);
+    std::promise<void> gate;
+    std::shared_future<void> open = gate.get_future().share();
+    hetu::impl::CPUStream(st).EnqueueTask([open] { open.wait(); });
+    chain(st, y1, e1, s1);
+    CHECK(s1->data_ptr<float>()[0] == 0.f && y1->data_ptr<float>()[0] == 0.f);   // nothing has run yet
+    // a bad argument is refused at the call, in this thread, while the stream is still held
+    NDArray wrong = NDArray::empty({rows, cols + 1}, cpu, kFloat32);
+    CHECK(throws<assertion_error>([&] { hetu::impl::SoftmaxCpu(x, wrong, 1, st); }));
+    CHECK(throws<not_implemented>([&] {
+      NDArray xi = NDArray::zeros({4, 4}, cpu, kInt32), yi = NDArray::zeros({4, 4}, cpu, kInt32);
+      hetu::impl::SoftmaxCpu(xi, yi, 1, st);
+    }));
+    gate.set_value();
+    st.Sync();
+    CHECK(std::memcmp(y0->raw_data_ptr(), y1->raw_data_ptr(), size_t(rows * cols) * 4) == 0);
+    CHECK(std::memcmp(e0->raw_data_ptr(), e1->raw_data_ptr(), size_t(rows * cols) * 4) == 0);
+    CHECK(std::memcmp(s0->raw_data_ptr(), s1->raw_data_ptr(), size_t(rows) * 4) == 0);
+    // a strided input is gathered inside the task, after the task that fills it
+    NDArray base = NDArray::zeros({cols, rows}, cpu, kFloat32);
+    NDArray xt = NDArray::permute(base, {1, 0});             // [rows, cols] view, not dense
+    std::promise<void> gate2;
+    std::shared_future<void> open2 = gate2.get_future().share();
+    hetu::impl::CPUStream(st).EnqueueTask([open2, base, x, rows, cols] {
+      open2.wait();
+      for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c) base->data_ptr<float>()[c * rows + r] = x->data_ptr<float>()[r * cols + c];
+    });
+    NDArray y2 = NDArray::empty_like(x);
+    hetu::impl::SoftmaxCpu(xt, y2, 1, st);
+    gate2.set_value();
+    st.Sync();
+    CHECK(std::memcmp(y0->raw_data_ptr(), y2->raw_data_ptr(), size_t(rows * cols) * 4) == 0);
+    // the team size set through the library reaches the stream's worker
+    hetu::impl::SetHostKernelThreads(1);
+    NDArray big = NDArray::zeros({512, 512}, cpu, kFloat32), bigy = NDArray::empty({512, 512}, cpu, kFloat32);
+    hetu::impl::SoftmaxCpu(big, bigy, 1, st);
+    st.Sync();
+    CHECK(std::fabs(bigy->data_ptr<float>()[0] - 1.f / 512.f) < 1e-7f);
+    hetu::impl::SetHostKernelThreads(0);
+    CHECK(hetu::impl::HostKernelThreads() == 0);
   });
 
   run("host twins of the neighbours: broadcasting arithmetic, broadcasts, norms, losses, batch norm", [] {

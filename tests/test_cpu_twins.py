@@ -474,3 +474,39 @@ def test_ndarray_arithmetic_statics_on_host_arrays(ht):
     ht.ndarray_sceloss(a, lab, loss, "sum")
     want = oracle.sce_dense_fwd(a.numpy(), lab.numpy()).sum()
     assert abs(float(loss) - want) <= 1e-5 * abs(want)
+
+
+def test_host_calls_on_a_stream_run_in_order_and_report_failures_at_sync(ht):
+    """Host streams 1..15 are task queues with a worker thread each (the blocking stream 0 runs in the caller).  With
+    the C face switched to asynchronous host calls, a chain of dependent kernels on one stream gives the bits of the
+    same chain run call by call, and the first failure of a task comes out of the stream's sync."""
+    import torch
+    x = _t(_draw(71, (256, 384), "fp32"), "fp32")
+
+    def chain(stream):
+        y, e = torch.zeros_like(x), torch.zeros_like(x)
+        s = torch.zeros((256,), dtype=x.dtype)
+        ht.softmax(x, y, 1, stream=stream)
+        ht.unary("exp", y, e, stream=stream)
+        ht.reduce(e, s, [1], "sum", stream=stream)
+        return y, e, s
+
+    want = chain(0)
+    was = ht.set_host_async(True)
+    try:
+        assert was is False
+        got = chain(7)
+        ht.host_stream_sync(7)
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+        # argument checks still fail the call itself
+        with pytest.raises(ht.HetuError):
+            ht.softmax(x, torch.zeros((256, 385)), 1, stream=7)
+        ht.host_stream_sync(7)
+    finally:
+        ht.set_host_async(False)
+        ht.synchronize_all()
+    # default mode: the call has finished when it returns, whatever the stream
+    y = torch.zeros_like(x)
+    ht.softmax(x, y, 1, stream=9)
+    assert torch.equal(y, want[0])

@@ -107,7 +107,7 @@ def build_host(verbose=True):
     objdir = os.path.join(OBJ, "host")
     os.makedirs(objdir, exist_ok=True)
     # OpenMP: the host twins of the kernels share their rows out over the cores
-    cxx = ["g++", "-O3", "-std=c++17", "-fPIC", "-pthread", "-fopenmp", "-I" + INCLUDE, "-I" + HERE]
+    cxx = ["g++", "-O3", "-fno-trapping-math", "-std=c++17", "-fPIC", "-pthread", "-fopenmp", "-I" + INCLUDE, "-I" + HERE]
     srcs = sorted(srcs)
     objs = [os.path.join(objdir, os.path.relpath(s, HOST).replace(os.sep, "_")[:-3] + ".o") for s in srcs]
 

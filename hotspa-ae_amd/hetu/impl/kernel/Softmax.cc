@@ -110,18 +110,20 @@ void SoftmaxCpu(const NDArray& input, NDArray& output, int64_t dim, const Stream
       using A = typename cpu::Arith<spec_t>::type;
       const spec_t* xp = x->data_ptr<spec_t>();
       spec_t* yp = output->data_ptr<spec_t>();
-      cpu::parallel_rows(outer * inner, extent, [&](int64_t line) {
-        const int64_t o = line / inner, i = line - o * inner;
-        const spec_t* xl = xp + o * extent * inner + i;
-        spec_t* yl = yp + o * extent * inner + i;
-        const A m = cpu::blocked_max<A>(extent, [&](int64_t k) { return cpu::ld<spec_t, A>(xl + k * inner); });
-        // a line of -inf only: exp(-inf - -inf) is NaN, as on the accelerator
-        const A sum = cpu::blocked_sum<A>(extent, [&](int64_t k) {
-          return std::exp(cpu::ld<spec_t, A>(xl + k * inner) - m);
+      cpu::with_step(inner, [&](auto step) {
+        cpu::parallel_rows(outer * inner, extent, [&](int64_t line) {
+          const int64_t o = line / inner, i = line - o * inner;
+          const spec_t* xl = xp + o * extent * inner + i;
+          spec_t* yl = yp + o * extent * inner + i;
+          const A m = cpu::blocked_max<A>(extent, [&](int64_t k) { return cpu::ld<spec_t, A>(xl + k * step()); });
+          // a line of -inf only: exp(-inf - -inf) is NaN, as on the accelerator
+          const A sum = cpu::blocked_sum<A>(extent, [&](int64_t k) {
+            return cpu::exp_(cpu::ld<spec_t, A>(xl + k * step()) - m);
+          });
+          const A inv = A(1) / sum;
+          for (int64_t k = 0; k < extent; ++k)
+            cpu::st<spec_t, A>(yl + k * step(), cpu::exp_(cpu::ld<spec_t, A>(xl + k * step()) - m) * inv);
         });
-        const A inv = A(1) / sum;
-        for (int64_t k = 0; k < extent; ++k)
-          cpu::st<spec_t, A>(yl + k * inner, std::exp(cpu::ld<spec_t, A>(xl + k * inner) - m) * inv);
       });
     });
   });
@@ -147,16 +149,19 @@ void SoftmaxGradientCpu(const NDArray& input_Y, const NDArray& output_grad, NDAr
       const spec_t* yp = y->data_ptr<spec_t>();
       const spec_t* dyp = dy->data_ptr<spec_t>();
       spec_t* dxp = input_grad->data_ptr<spec_t>();
-      cpu::parallel_rows(outer * inner, extent, [&](int64_t line) {
-        const int64_t o = line / inner, i = line - o * inner;
-        const int64_t base = o * extent * inner + i;
-        const A dot = cpu::blocked_sum<A>(extent, [&](int64_t k) {
-          return cpu::ld<spec_t, A>(yp + base + k * inner) * cpu::ld<spec_t, A>(dyp + base + k * inner);
+      cpu::with_step(inner, [&](auto step) {
+        cpu::parallel_rows(outer * inner, extent, [&](int64_t line) {
+          const int64_t o = line / inner, i = line - o * inner;
+          const spec_t* yl = yp + o * extent * inner + i;
+          const spec_t* dyl = dyp + o * extent * inner + i;
+          spec_t* dxl = dxp + o * extent * inner + i;
+          const A dot = cpu::blocked_sum<A>(extent, [&](int64_t k) {
+            return cpu::ld<spec_t, A>(yl + k * step()) * cpu::ld<spec_t, A>(dyl + k * step());
+          });
+          for (int64_t k = 0; k < extent; ++k)
+            cpu::st<spec_t, A>(dxl + k * step(),
+                               cpu::ld<spec_t, A>(yl + k * step()) * (cpu::ld<spec_t, A>(dyl + k * step()) - dot));
         });
-        for (int64_t k = 0; k < extent; ++k) {
-          const int64_t e = base + k * inner;
-          cpu::st<spec_t, A>(dxp + e, cpu::ld<spec_t, A>(yp + e) * (cpu::ld<spec_t, A>(dyp + e) - dot));
-        }
       });
     });
   });

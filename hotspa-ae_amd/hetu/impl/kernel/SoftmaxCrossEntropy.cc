@@ -123,7 +123,7 @@ void SoftmaxCrossEntropyCpu(const NDArray& input, const NDArray& label, NDArray&
         const spec_t* xr = xp + r * cols;
         const spec_t* lr = lp + r * cols;
         const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
-        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m); });
         const A lse = m + std::log(sum);
         const A acc = cpu::blocked_sum<A>(cols, [&](int64_t i) {
           return cpu::ld<spec_t, A>(lr + i) * (lse - cpu::ld<spec_t, A>(xr + i));
@@ -167,9 +167,9 @@ void SoftmaxCrossEntropyGradientCpu(const NDArray& input_y, const NDArray& label
         spec_t* dr = out + r * cols;
         const A gr = cpu::ld<spec_t, A>(gp + r);
         const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
-        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m); });
         for (int64_t i = 0; i < cols; ++i)
-          cpu::st<spec_t, A>(dr + i, (std::exp(cpu::ld<spec_t, A>(xr + i) - m) / sum - cpu::ld<spec_t, A>(lr + i)) * gr);
+          cpu::st<spec_t, A>(dr + i, (cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m) / sum - cpu::ld<spec_t, A>(lr + i)) * gr);
       });
     });
   });

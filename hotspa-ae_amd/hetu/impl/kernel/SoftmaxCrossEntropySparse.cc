@@ -147,7 +147,7 @@ void SoftmaxCrossEntropySparseCpu(const NDArray& pred, const NDArray& label, NDA
         if (lab < 0 || lab >= cols) { cpu::st<spec_t, A>(out + r, std::numeric_limits<A>::quiet_NaN()); return; }
         const spec_t* xr = pp + r * cols;
         const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
-        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m); });
         cpu::st<spec_t, A>(out + r, std::log(sum) - (cpu::ld<spec_t, A>(xr + lab) - m));
       });
     });
@@ -193,10 +193,10 @@ void SoftmaxCrossEntropySparseGradientCpu(const NDArray& pred, const NDArray& la
         const spec_t* xr = pp + r * cols;
         const A g = cpu::ld<spec_t, A>(gp + r);
         const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
-        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return std::exp(cpu::ld<spec_t, A>(xr + i) - m); });
+        const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m); });
         const A scale = g / sum;
         for (int64_t i = 0; i < cols; ++i) {
-          const A pr = std::exp(cpu::ld<spec_t, A>(xr + i) - m) * scale;
+          const A pr = cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m) * scale;
           cpu::st<spec_t, A>(dr + i, i == lab ? pr - g : pr);
         }
       });

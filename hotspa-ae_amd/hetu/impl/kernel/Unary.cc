@@ -63,10 +63,14 @@ void UnaryHost(int op, const char* who, const NDArray& input, NDArray& output, c
       NDArray x = Dense(input, stream);
       const spec_t* px = x->data_ptr<spec_t>();
       spec_t* po = output->data_ptr<spec_t>();
-      cpu::parallel_for(n, [&](int64_t i) {
-        const A v = cpu::ld<spec_t, A>(px + i);
-        cpu::st<spec_t, A>(po + i, op == HK_UNARY_EXP ? std::exp(v) : op == HK_UNARY_LOG ? std::log(v) : std::sqrt(v));
-      });
+      // one loop per operation: the choice stays outside, the exp and sqrt loops vectorise
+      if (op == HK_UNARY_EXP) {
+        cpu::parallel_for(n, [&](int64_t i) { cpu::st<spec_t, A>(po + i, cpu::exp_(cpu::ld<spec_t, A>(px + i))); });
+      } else if (op == HK_UNARY_LOG) {
+        cpu::parallel_for(n, [&](int64_t i) { cpu::st<spec_t, A>(po + i, std::log(cpu::ld<spec_t, A>(px + i))); });
+      } else {
+        cpu::parallel_for(n, [&](int64_t i) { cpu::st<spec_t, A>(po + i, std::sqrt(cpu::ld<spec_t, A>(px + i))); });
+      }
     });
   });
 }

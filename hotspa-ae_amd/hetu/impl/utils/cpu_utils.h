@@ -13,6 +13,7 @@
 
 #include <cmath>
 #include <cstdint>
+#include <cstring>
 #include <limits>
 #include <type_traits>
 #include <utility>
@@ -68,25 +69,83 @@ inline A blocked_sum(int64_t n, F f) {
   A acc[kLanes];
   for (int k = 0; k < kLanes; ++k) acc[k] = A(0);
   int64_t i = 0;
-  for (; i + kLanes <= n; i += kLanes)
-    for (int k = 0; k < kLanes; ++k) acc[k] += f(i + k);
+  for (; i + kLanes <= n; i += kLanes) {
+    A v[kLanes];   // the terms first, then the sums: two loops of constant length, each of which vectorises
+    for (int k = 0; k < kLanes; ++k) v[k] = f(i + k);
+    for (int k = 0; k < kLanes; ++k) acc[k] += v[k];
+  }
   for (int k = 0; i < n; ++i, ++k) acc[k] += f(i);
   for (int w = kLanes / 2; w > 0; w >>= 1)
     for (int k = 0; k < w; ++k) acc[k] += acc[k + w];
   return acc[0];
 }
 
+// Maximum of f(i), i in [0, n), NaN if any term is: kLanes running maxima and NaN flags side by side (selects
+// between lanes, which vectorise where a single running maximum would not), combined at the end.
 template <typename A, typename F>
 inline A blocked_max(int64_t n, F f) {
-  A m = -std::numeric_limits<A>::infinity();
-  bool nan = false;
-  for (int64_t i = 0; i < n; ++i) {
-    const A v = f(i);
-    nan |= v != v;
-    m = v > m ? v : m;
+  A mx[kLanes];
+  int bad[kLanes];
+  for (int k = 0; k < kLanes; ++k) { mx[k] = -std::numeric_limits<A>::infinity(); bad[k] = 0; }
+  int64_t i = 0;
+  for (; i + kLanes <= n; i += kLanes) {
+    A v[kLanes];
+    for (int k = 0; k < kLanes; ++k) v[k] = f(i + k);
+    for (int k = 0; k < kLanes; ++k) {
+      bad[k] |= v[k] != v[k] ? 1 : 0;
+      mx[k] = v[k] > mx[k] ? v[k] : mx[k];
+    }
   }
+  for (int k = 0; i < n; ++i, ++k) {
+    const A v = f(i);
+    bad[k] |= v != v ? 1 : 0;
+    mx[k] = v > mx[k] ? v : mx[k];
+  }
+  A m = mx[0];
+  int nan = bad[0];
+  for (int k = 1; k < kLanes; ++k) { m = mx[k] > m ? mx[k] : m; nan |= bad[k]; }
   return nan ? std::numeric_limits<A>::quiet_NaN() : m;
 }
+
+// A loop body written once for a run-time element step and compiled a second time for step 1, the case whose
+// loads and stores are contiguous and vectorise: f receives a callable that returns the step.
+struct UnitStep { constexpr int64_t operator()() const { return 1; } };
+struct AnyStep { int64_t value; int64_t operator()() const { return value; } };
+template <typename F>
+inline void with_step(int64_t step, F f) {
+  if (step == 1) f(UnitStep{});
+  else f(AnyStep{step});
+}
+
+// exp for the float arithmetic of the host kernels, written without a branch or a library call so that the loops
+// around it vectorise: x = n ln2 + r with |r| <= ln2 / 2 (n rounded by the 1.5 * 2^23 trick, ln2 split in two so
+// that n * ln2_hi is exact), a degree-6 polynomial in r, and 2^n applied through the exponent bits in two factors,
+// which keeps gradual underflow.  Within 2 units in the last place of the exact value; exp(-inf) = 0, overflow
+// gives +inf, NaN stays NaN.  float64 data keeps std::exp.
+inline float exp_(float x) {
+  const float lo = -104.f, hi = 89.f;
+  const float xc = x < lo ? lo : (x > hi ? hi : x);          // NaN passes through
+  const float xs = xc == xc ? xc : 0.f;                      // the exponent is taken from a number
+  const float magic = 12582912.f;                            // 1.5 * 2^23
+  const float nf = (xs * 1.44269504088896341f + magic) - magic;
+  float r = xc - nf * 0.693359375f;                          // ln2_hi: 10 significant bits
+  r = r - nf * -2.12194440e-4f;                              // ln2_lo
+  float p = 1.9875691500e-4f;
+  p = p * r + 1.3981999507e-3f;
+  p = p * r + 8.3334519073e-3f;
+  p = p * r + 4.1665795894e-2f;
+  p = p * r + 1.6666665459e-1f;
+  p = p * r + 5.0000001201e-1f;
+  p = p * (r * r) + r + 1.f;
+  const int32_t n = int32_t(nf);
+  const int32_t n1 = n >> 1, n2 = n - n1;                    // both within [-75, 65]
+  const uint32_t b1 = uint32_t(n1 + 127) << 23, b2 = uint32_t(n2 + 127) << 23;
+  float s1, s2;
+  std::memcpy(&s1, &b1, 4);
+  std::memcpy(&s2, &b2, 4);
+  return p * s1 * s2;
+}
+inline double exp_(double x) { return std::exp(x); }
 
 // x op y on one element of storage type T, op being 0 add, 1 subtract, 2 multiply, 3 divide (the values of the
 // HK_BINARY_* constants).  Floating-point types compute in their arithmetic type and round once; integers wrap in

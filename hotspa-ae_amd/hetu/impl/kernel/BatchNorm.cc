@@ -165,7 +165,9 @@ void BatchNormCpu(const NDArray& input_X, const NDArray& bn_scale, const NDArray
         for (int64_t n = 0; n < N; ++n) {
           const spec_t* plane = xp + (n * C + c) * HW;
           spec_t* out = yp + (n * C + c) * HW;
-          for (int64_t i = 0; i < HW; ++i) cpu::st<spec_t, A>(out + i, (cpu::ld<spec_t, A>(plane + i) - mean) * w + b);
+          cpu::for_range(0, HW, [&](int64_t i) {
+            cpu::st<spec_t, A>(out + i, (cpu::ld<spec_t, A>(plane + i) - mean) * w + b);
+          });
         }
       });
     });
@@ -224,10 +226,10 @@ void BatchNormGradientCpu(const NDArray& gradient_Y, const NDArray& input_X, con
           const spec_t* xr = xp + (n * C + c) * HW;
           const spec_t* dr = dyp + (n * C + c) * HW;
           spec_t* out = dxp + (n * C + c) * HW;
-          for (int64_t i = 0; i < HW; ++i) {
+          cpu::for_range(0, HW, [&](int64_t i) {
             const A xh = (cpu::ld<spec_t, A>(xr + i) - mean) * invstd;
             cpu::st<spec_t, A>(out + i, w * (cpu::ld<spec_t, A>(dr + i) - k1 - xh * k2));
-          }
+          });
         }
       });
     });

@@ -124,7 +124,9 @@ void InstanceNormCpu(const NDArray& in_arr, NDArray& mean_arr, NDArray& var_arr,
         cpu::st<spec_t, A>(vp + r, var);
         const A rstd = A(1) / std::sqrt(var + A(eps));
         spec_t* yr = yp + r * cols;
-        for (int64_t i = 0; i < cols; ++i) cpu::st<spec_t, A>(yr + i, (cpu::ld<spec_t, A>(xr + i) - mean) * rstd);
+        cpu::for_range(0, cols, [&](int64_t i) {
+          cpu::st<spec_t, A>(yr + i, (cpu::ld<spec_t, A>(xr + i) - mean) * rstd);
+        });
       });
     });
   });
@@ -170,10 +172,10 @@ void InstanceNormGradientCpu(const NDArray& out_grads, const NDArray& in_arr, ND
           return cpu::ld<spec_t, A>(dyr + i) * (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
         }) * inv;
         spec_t* dxr = dxp + r * cols;
-        for (int64_t i = 0; i < cols; ++i) {
+        cpu::for_range(0, cols, [&](int64_t i) {
           const A xh = (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
           cpu::st<spec_t, A>(dxr + i, rstd * (cpu::ld<spec_t, A>(dyr + i) - s1 - xh * s2));
-        }
+        });
       });
     });
   });

@@ -174,9 +174,10 @@ void LayerNormCpu(const NDArray& in_arr, const NDArray& ln_scale, const NDArray&
         cpu::st<spec_t, A>(vp + r, var);
         const A rstd = A(1) / std::sqrt(var + A(eps));
         spec_t* yr = yp + r * cols;
-        for (int64_t i = 0; i < cols; ++i)
+        cpu::for_range(0, cols, [&](int64_t i) {
           cpu::st<spec_t, A>(yr + i, (cpu::ld<spec_t, A>(xr + i) - mean) * rstd * cpu::ld<spec_t, A>(gp + i) +
                                        cpu::ld<spec_t, A>(bp + i));
+        });
       });
     });
   });
@@ -237,11 +238,11 @@ void LayerNormGradientCpu(const NDArray& out_grads, const NDArray& in_arr, const
           const A rstd = A(1) / std::sqrt(cpu::ld<spec_t, A>(vp + r) + A(eps));
           const spec_t* dyr = dyp + r * cols;
           const spec_t* xr = xp + r * cols;
-          for (int64_t c = c0; c < c1; ++c) {
+          cpu::for_range(c0, c1, [&](int64_t c) {
             const A d = cpu::ld<spec_t, A>(dyr + c);
             sb[c - c0] += d;
             sg[c - c0] += d * (cpu::ld<spec_t, A>(xr + c) - m) * rstd;
-          }
+          });
         }
         for (int64_t c = c0; c < c1; ++c) {
           cpu::st<spec_t, A>(dgp + c, sg[c - c0]);
@@ -262,11 +263,11 @@ void LayerNormGradientCpu(const NDArray& out_grads, const NDArray& in_arr, const
           return cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i) * (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
         }) * inv;
         spec_t* dxr = dxp + r * cols;
-        for (int64_t i = 0; i < cols; ++i) {
+        cpu::for_range(0, cols, [&](int64_t i) {
           const A xh = (cpu::ld<spec_t, A>(xr + i) - m) * rstd;
           const A t = cpu::ld<spec_t, A>(dyr + i) * cpu::ld<spec_t, A>(gp + i);
           cpu::st<spec_t, A>(dxr + i, rstd * (t - s1 - xh * s2));
-        }
+        });
       });
     });
   });

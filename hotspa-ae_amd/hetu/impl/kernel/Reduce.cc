@@ -206,7 +206,7 @@ void HostReduce(const NDArray& in, const NDArray& out, const std::vector<bool>& 
       for (int64_t c = 0; c < kBand; ++c) acc[c] = HostRed<A>::identity(op);
       for (int64_t r = 0; r < n_red; ++r) {
         const T* row = base + offset_of(r, rs, rst);
-        if (sum_like) for (int64_t c = c0; c < c1; ++c) acc[c - c0] += host_ld<T, A>(row + c);
+        if (sum_like) cpu::for_range(c0, c1, [&](int64_t c) { acc[c - c0] += host_ld<T, A>(row + c); });
         else for (int64_t c = c0; c < c1; ++c) acc[c - c0] = HostRed<A>::apply(op, acc[c - c0], host_ld<T, A>(row + c));
       }
       for (int64_t c = c0; c < c1; ++c) host_st<O, A>(op_ + ob * C + c, HostRed<A>::finish(op, acc[c - c0], factor));

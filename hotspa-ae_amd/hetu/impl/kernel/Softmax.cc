@@ -121,8 +121,9 @@ void SoftmaxCpu(const NDArray& input, NDArray& output, int64_t dim, const Stream
             return cpu::exp_(cpu::ld<spec_t, A>(xl + k * step()) - m);
           });
           const A inv = A(1) / sum;
-          for (int64_t k = 0; k < extent; ++k)
+          cpu::for_range(0, extent, [&](int64_t k) {
             cpu::st<spec_t, A>(yl + k * step(), cpu::exp_(cpu::ld<spec_t, A>(xl + k * step()) - m) * inv);
+          });
         });
       });
     });
@@ -158,9 +159,10 @@ void SoftmaxGradientCpu(const NDArray& input_Y, const NDArray& output_grad, NDAr
           const A dot = cpu::blocked_sum<A>(extent, [&](int64_t k) {
             return cpu::ld<spec_t, A>(yl + k * step()) * cpu::ld<spec_t, A>(dyl + k * step());
           });
-          for (int64_t k = 0; k < extent; ++k)
+          cpu::for_range(0, extent, [&](int64_t k) {
             cpu::st<spec_t, A>(dxl + k * step(),
                                cpu::ld<spec_t, A>(yl + k * step()) * (cpu::ld<spec_t, A>(dyl + k * step()) - dot));
+          });
         });
       });
     });

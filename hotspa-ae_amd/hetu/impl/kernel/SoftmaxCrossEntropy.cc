@@ -168,8 +168,9 @@ void SoftmaxCrossEntropyGradientCpu(const NDArray& input_y, const NDArray& label
         const A gr = cpu::ld<spec_t, A>(gp + r);
         const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
         const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m); });
-        for (int64_t i = 0; i < cols; ++i)
+        cpu::for_range(0, cols, [&](int64_t i) {
           cpu::st<spec_t, A>(dr + i, (cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m) / sum - cpu::ld<spec_t, A>(lr + i)) * gr);
+        });
       });
     });
   });

@@ -195,10 +195,10 @@ void SoftmaxCrossEntropySparseGradientCpu(const NDArray& pred, const NDArray& la
         const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
         const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m); });
         const A scale = g / sum;
-        for (int64_t i = 0; i < cols; ++i) {
+        cpu::for_range(0, cols, [&](int64_t i) {
           const A pr = cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m) * scale;
           cpu::st<spec_t, A>(dr + i, i == lab ? pr - g : pr);
-        }
+        });
       });
     });
   });

@@ -11,8 +11,10 @@
 #include "hetu/core/ndarray.h"
 #include "hetu/impl/stream/CPUStream.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <type_traits>
@@ -61,29 +63,71 @@ inline void st(T* p, A v) { *p = T(float(v)); }
 template <> inline void st<double, double>(double* p, double v) { *p = v; }
 template <> inline void st<float, float>(float* p, float v) { *p = v; }
 
+// The inner loops of the host kernels exist three times: for the baseline x86-64 instruction set, for AVX2 + FMA
+// and for AVX-512, picked once per process from what the processor reports (HETU_HOST_ISA=0 / 1 / 2 caps the
+// choice, for tests).  A loop is written once, as a body that is inlined into three thin functions, each compiled
+// for its instruction set; the callable it applies (a lambda of the calling kernel) is inlined with it.
+inline int detect_isa_level() {
+  int level = 0;
+#if defined(__x86_64__)
+  __builtin_cpu_init();
+  if (__builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma") && __builtin_cpu_supports("f16c")) level = 1;
+  if (level == 1 && __builtin_cpu_supports("avx512f") && __builtin_cpu_supports("avx512bw") &&
+      __builtin_cpu_supports("avx512vl") && __builtin_cpu_supports("avx512dq"))
+    level = 2;
+#endif
+  if (const char* cap = std::getenv("HETU_HOST_ISA")) {
+    const int c = std::atoi(cap);
+    if (c >= 0 && c < level) level = c;
+  }
+  return level;
+}
+inline int isa_level() {
+  static const int level = detect_isa_level();
+  return level;
+}
+#if defined(__x86_64__)
+#define HT_HOST_ISA_V3 __attribute__((target("avx2,fma,f16c")))
+#define HT_HOST_ISA_V4 __attribute__((target("avx512f,avx512bw,avx512vl,avx512dq,avx2,fma,f16c")))
+#else
+#define HT_HOST_ISA_V3
+#define HT_HOST_ISA_V4
+#endif
+#define HT_HOST_LOOP_BODY __attribute__((always_inline)) inline
+
+// Defines NAME(args) as the choice between three compilations of BODY(args).
+#define HT_HOST_ISA_VARIANTS(RET, NAME, BODY, PARAMS, ARGS)                                  \
+  template <typename A, typename F> HT_HOST_ISA_V3 RET NAME##_v3 PARAMS { return BODY<A> ARGS; } \
+  template <typename A, typename F> HT_HOST_ISA_V4 RET NAME##_v4 PARAMS { return BODY<A> ARGS; } \
+  template <typename A, typename F> inline RET NAME PARAMS {                                 \
+    switch (isa_level()) {                                                                   \
+      case 2: return NAME##_v4<A> ARGS;                                                      \
+      case 1: return NAME##_v3<A> ARGS;                                                      \
+      default: return BODY<A> ARGS;                                                          \
+    }                                                                                        \
+  }
+
 // Sum of f(i), i in [0, n), in kLanes independent running sums that are combined pairwise at the end: the loop
 // vectorises, and the rounding error grows with n / kLanes instead of n.
 constexpr int kLanes = 16;
 template <typename A, typename F>
-inline A blocked_sum(int64_t n, F f) {
+HT_HOST_LOOP_BODY A blocked_sum_body(int64_t n, F& f) {
   A acc[kLanes];
   for (int k = 0; k < kLanes; ++k) acc[k] = A(0);
   int64_t i = 0;
-  for (; i + kLanes <= n; i += kLanes) {
-    A v[kLanes];   // the terms first, then the sums: two loops of constant length, each of which vectorises
-    for (int k = 0; k < kLanes; ++k) v[k] = f(i + k);
-    for (int k = 0; k < kLanes; ++k) acc[k] += v[k];
-  }
+  for (; i + kLanes <= n; i += kLanes)
+    for (int k = 0; k < kLanes; ++k) acc[k] += f(i + k);
   for (int k = 0; i < n; ++i, ++k) acc[k] += f(i);
   for (int w = kLanes / 2; w > 0; w >>= 1)
     for (int k = 0; k < w; ++k) acc[k] += acc[k + w];
   return acc[0];
 }
+HT_HOST_ISA_VARIANTS(A, blocked_sum, blocked_sum_body, (int64_t n, F f), (n, f))
 
 // Maximum of f(i), i in [0, n), NaN if any term is: kLanes running maxima and NaN flags side by side (selects
 // between lanes, which vectorise where a single running maximum would not), combined at the end.
 template <typename A, typename F>
-inline A blocked_max(int64_t n, F f) {
+HT_HOST_LOOP_BODY A blocked_max_body(int64_t n, F& f) {
   A mx[kLanes];
   int bad[kLanes];
   for (int k = 0; k < kLanes; ++k) { mx[k] = -std::numeric_limits<A>::infinity(); bad[k] = 0; }
@@ -106,6 +150,16 @@ inline A blocked_max(int64_t n, F f) {
   for (int k = 1; k < kLanes; ++k) { m = mx[k] > m ? mx[k] : m; nan |= bad[k]; }
   return nan ? std::numeric_limits<A>::quiet_NaN() : m;
 }
+HT_HOST_ISA_VARIANTS(A, blocked_max, blocked_max_body, (int64_t n, F f), (n, f))
+
+// f(i) for i in [begin, end), in order, in the calling thread: the element-wise loop of a kernel's row
+template <typename A, typename F>
+HT_HOST_LOOP_BODY void for_range_body(int64_t begin, int64_t end, F& f) {
+  for (int64_t i = begin; i < end; ++i) f(i);
+}
+HT_HOST_ISA_VARIANTS(void, for_range_any, for_range_body, (int64_t begin, int64_t end, F f), (begin, end, f))
+template <typename F>
+inline void for_range(int64_t begin, int64_t end, F f) { for_range_any<void>(begin, end, f); }
 
 // A loop body written once for a run-time element step and compiled a second time for step 1, the case whose
 // loads and stores are contiguous and vectorise: f receives a callable that returns the step.
@@ -192,8 +246,11 @@ inline T negate(T x) {
 // f(i) for i in [0, n), shared out over the OpenMP team when there is enough of it
 template <typename F>
 inline void parallel_for(int64_t n, F f) {
+  // pieces of 8192 elements, each a plain loop in the instruction set of the processor
+  constexpr int64_t kPiece = 8192;
+  const int64_t pieces = (n + kPiece - 1) / kPiece;
 #pragma omp parallel for schedule(static) num_threads(team_size()) if (n >= (int64_t(1) << 16))
-  for (int64_t i = 0; i < n; ++i) f(i);
+  for (int64_t p = 0; p < pieces; ++p) for_range(p * kPiece, std::min(n, (p + 1) * kPiece), f);
 }
 
 // Walks a dense row-major array of `nd` dimensions run by run along the last dimension: f(out_offset, a_offset,

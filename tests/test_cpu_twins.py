@@ -510,3 +510,20 @@ def test_host_calls_on_a_stream_run_in_order_and_report_failures_at_sync(ht):
     y = torch.zeros_like(x)
     ht.softmax(x, y, 1, stream=9)
     assert torch.equal(y, want[0])
+
+
+@pytest.mark.parametrize("level", [0, 1])
+def test_every_instruction_set_variant_of_the_host_loops(level):
+    """The inner loops of the host kernels are compiled for baseline x86-64, AVX2 + FMA and AVX-512 and chosen once
+    per process; the rest of this file runs the best the processor has.  The lower levels are forced through
+    HETU_HOST_ISA in a process of their own, on the tests that cover every loop helper (sums, maxima, element-wise
+    passes with and without exp)."""
+    import os
+    import subprocess
+    import sys
+    env = dict(os.environ, HETU_HOST_ISA=str(level))
+    picked = ("test_layer_norm_and_gradient or test_softmax_and_gradient or test_sparse_cross_entropy_and_gradient "
+              "or test_reduce_every_axis_subset or test_unary_and_constants or test_batch_norm_and_gradient")
+    run = subprocess.run([sys.executable, "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-k", picked,
+                          "-p", "no:cacheprovider"], env=env, cwd=helpers.ROOT, capture_output=True, text=True)
+    assert run.returncode == 0, run.stdout[-3000:] + run.stderr[-2000:]

@@ -195,10 +195,11 @@ void SoftmaxCrossEntropySparseGradientCpu(const NDArray& pred, const NDArray& la
         const A m = cpu::blocked_max<A>(cols, [&](int64_t i) { return cpu::ld<spec_t, A>(xr + i); });
         const A sum = cpu::blocked_sum<A>(cols, [&](int64_t i) { return cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m); });
         const A scale = g / sum;
+        // the row without its label term (a loop with nothing but arithmetic in it), then the one element again
         cpu::for_range(0, cols, [&](int64_t i) {
-          const A pr = cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m) * scale;
-          cpu::st<spec_t, A>(dr + i, i == lab ? pr - g : pr);
+          cpu::st<spec_t, A>(dr + i, cpu::exp_(cpu::ld<spec_t, A>(xr + i) - m) * scale);
         });
+        cpu::st<spec_t, A>(dr + lab, cpu::exp_(cpu::ld<spec_t, A>(xr + lab) - m) * scale - g);
       });
     });
   });

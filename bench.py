@@ -909,6 +909,26 @@ def stream_sweep(hk, torch, steps=40):
                 best = (gbs, name, d)
         res["%dR:%dW" % (nr, nw)] = {"best_shape": best[1], "us": round(best[2] * 1e6, 2), "GBps": round(best[0], 1),
                                      "frac": round(best[0] / HBM_PEAK_GBS, 4)}
+    # the persistent 2R:1W walk with a ring of tiles in flight per thread and a barrier per tile: the design of the
+    # backward norm kernels with the arithmetic taken out
+    best = None
+    for bs in (256, 512, 1024):
+        for w in (1, 2):
+            for depth in (1, 2, 3, 4):
+                for barrier in (0, 1):
+                    def fn(i, bs=bs, w=w, depth=depth, barrier=barrier):
+                        o = (3 * i) % 8
+                        hk.ring_probe(bufs[(o + 2) % 8], bufs[o], bufs[(o + 1) % 8], bs, depth, bool(barrier), w)
+                    d = timed(fn)
+                    gbs = 3 * n / d / 1e9
+                    name = "%4d threads, ring depth %d, barrier %d, %d workgroups per CU" % (bs, depth, barrier, w)
+                    print("ring   %-8s %-58s %8.2f us %7.1f GB/s %5.1f%%" % ("2R:1W", name, d * 1e6, gbs,
+                                                                           gbs / HBM_PEAK_GBS * 100), file=sys.stderr, flush=True)
+                    if barrier and (best is None or gbs > best[0]):
+                        best = (gbs, name, d)
+    res["2R:1W pipelined persistent, barrier per tile"] = {"best_shape": best[1], "us": round(best[2] * 1e6, 2),
+                                                           "GBps": round(best[0], 1),
+                                                           "frac": round(best[0] / HBM_PEAK_GBS, 4)}
     del bufs
     torch.cuda.empty_cache()
     return res

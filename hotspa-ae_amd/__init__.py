@@ -22,6 +22,6 @@ from .capi import (  # noqa: F401
     vocab_parallel_ce_stats, vocab_parallel_ce_combine, vocab_parallel_ce_bwd_fused, UNARY_OPS, BINARY_OPS,
     softmax_fwd, softmax_bwd,
     sce_sparse_fwd, sce_sparse_bwd, sce_dense_fwd, sce_dense_bwd, nll_loss_fwd, nll_loss_bwd,
-    reduce, reduce_workspace_bytes, norm, norm_bwd, batch_norm_fwd, batch_norm_bwd, batch_norm_workspace_bytes, tune_set, copy_kernel, strided_copy, strided_scatter, stream_probe, memcpy_d2d,
+    reduce, reduce_workspace_bytes, norm, norm_bwd, batch_norm_fwd, batch_norm_bwd, batch_norm_workspace_bytes, tune_set, copy_kernel, strided_copy, strided_scatter, stream_probe, ring_probe, memcpy_d2d,
     Event, current_stream,
 )

@@ -702,6 +702,17 @@ def stream_probe(dsts, srcs, block_threads=256, vectors_per_thread=1, nt_loads=T
         raise HkError(rc, bench_lib().hk_bench_last_error().decode("utf-8", "replace"))
 
 
+def ring_probe(dst, src0, src1, block_threads=512, depth=2, barrier=True, workgroups_per_cu=1, stream=None):
+    """Pipelined persistent yardstick: two arrays read, one written, a ring of `depth` tiles in flight per thread."""
+    nbytes = dst.numel() * dst.element_size()
+    rc = bench_lib().hk_bench_ring_probe(_ptr(dst), _ptr(src0), _ptr(src1), ctypes.c_size_t(nbytes),
+                                         ctypes.c_int(block_threads), ctypes.c_int(depth), ctypes.c_int(int(barrier)),
+                                         ctypes.c_int(workgroups_per_cu),
+                                         stream if stream is not None else current_stream())
+    if rc != 0:
+        raise HkError(rc, bench_lib().hk_bench_last_error().decode("utf-8", "replace"))
+
+
 def memcpy_d2d(dst, src, stream=None):
     check(lib().hk_memcpy_d2d(_ptr(dst), _ptr(src), ctypes.c_size_t(src.numel() * src.element_size()),
                               stream if stream is not None else current_stream()))

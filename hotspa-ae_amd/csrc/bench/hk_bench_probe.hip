@@ -130,6 +130,87 @@ static int probe_unroll(const ProbeArgs& a, int unroll, int nr, int nw, int ntl,
   }
 }
 
+// The persistent 2R:1W walk once more, software-pipelined the way the backward norm kernels are: a workgroup owns
+// every gridDim.x-th tile of BS vectors, keeps a ring of PF tiles of both input arrays in flight per thread (a slot is
+// refilled as soon as it has been consumed, loads past the end re-read the last tile), and optionally goes through one
+// workgroup barrier with a small LDS exchange per tile, which is what a row reduction across the wavefronts costs.
+// What the best depth reaches is the ceiling of that kernel design, whatever arithmetic is put into it.
+struct RingArgs {
+  const u32x4* a;
+  const u32x4* b;
+  u32x4* d;
+  long ntiles;
+};
+
+template <int BS, int PF, bool BARRIER>
+__global__ __launch_bounds__(BS)
+void ring_probe_kernel(RingArgs p) {
+  __shared__ uint32_t red[2][16];
+  u32x4 va[PF], vb[PF];
+  const long G = gridDim.x;
+  const long last = p.ntiles - 1;
+  long t0 = blockIdx.x;
+  auto issue = [&](auto slot, long t) {
+    constexpr int s = decltype(slot)::value;
+    const long tc = t < last ? t : last;
+    va[s] = __builtin_nontemporal_load(p.a + tc * BS + threadIdx.x);
+    vb[s] = __builtin_nontemporal_load(p.b + tc * BS + threadIdx.x);
+  };
+  static_for<PF>([&](auto slot) { issue(slot, t0 + decltype(slot)::value * G); });
+  int parity = 0;
+  auto step = [&](auto slot, auto guarded) {
+    constexpr int s = decltype(slot)::value;
+    const long t = t0 + s * G;
+    u32x4 r = va[s] ^ vb[s];
+    issue(slot, t + PF * G);
+    if constexpr (BARRIER) {
+      uint32_t v = r.x + r.y;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) v += uint32_t(__shfl_xor(int(v), o));
+      if ((threadIdx.x & 63) == 0) red[parity][threadIdx.x >> 6] = v;
+      __syncthreads();
+      uint32_t total = 0;
+#pragma unroll
+      for (int w = 0; w < BS / 64; ++w) total += red[parity][w];
+      parity ^= 1;
+      r.w ^= total;
+    }
+    if (!decltype(guarded)::value || t < p.ntiles) __builtin_nontemporal_store(r, p.d + t * BS + threadIdx.x);
+  };
+  long base = blockIdx.x;
+  const long round = long(PF) * G;
+#pragma nounroll
+  for (; base + long(PF - 1) * G < p.ntiles; base += round) {
+    static_for<PF>([&](auto slot) { step(slot, std::false_type{}); });
+    t0 += round;
+  }
+#pragma nounroll
+  for (; base < p.ntiles; base += round) {
+    static_for<PF>([&](auto slot) { step(slot, std::true_type{}); });
+    t0 += round;
+  }
+}
+
+template <int BS, int PF>
+static int ring_barrier(const RingArgs& a, int barrier, unsigned grid, hipStream_t s) {
+  if (barrier) hipLaunchKernelGGL((ring_probe_kernel<BS, PF, true>), dim3(grid), dim3(BS), 0, s, a);
+  else hipLaunchKernelGGL((ring_probe_kernel<BS, PF, false>), dim3(grid), dim3(BS), 0, s, a);
+  return bench_launch_check("ring_probe_kernel");
+}
+
+template <int BS>
+static int ring_depth(const RingArgs& a, int depth, int barrier, unsigned grid, hipStream_t s) {
+  switch (depth) {
+    case 1: return ring_barrier<BS, 1>(a, barrier, grid, s);
+    case 2: return ring_barrier<BS, 2>(a, barrier, grid, s);
+    case 3: return ring_barrier<BS, 3>(a, barrier, grid, s);
+    case 4: return ring_barrier<BS, 4>(a, barrier, grid, s);
+    default:
+      set_last_error("hk_bench_ring_probe: ring depth 1 to 4, got %d", depth);
+      return HK_ERR_UNSUPPORTED;
+  }
+}
+
 } // namespace hk
 
 using namespace hk;
@@ -173,6 +254,34 @@ int hk_bench_stream_probe(void* dst0, void* dst1, const void* src0, const void* 
     case 256: return probe_unroll<256>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
     case 512: return probe_unroll<512>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
     default: return probe_unroll<1024>(a, vectors_per_thread, reads, writes, nt_loads, nt_stores, grid, s);
+  }
+}
+
+int hk_bench_ring_probe(void* dst, const void* src0, const void* src1, size_t bytes, int block_threads, int depth,
+                        int barrier, int workgroups_per_cu, hkStream_t stream) {
+  const char* who = "hk_bench_ring_probe";
+  HK_REQUIRE(block_threads == 256 || block_threads == 512 || block_threads == 1024, HK_ERR_UNSUPPORTED,
+             "%s: workgroups of 256, 512 or 1024 threads, got %d", who, block_threads);
+  HK_REQUIRE(depth >= 1 && depth <= 4, HK_ERR_UNSUPPORTED, "%s: ring depth 1 to 4, got %d", who, depth);
+  HK_REQUIRE(workgroups_per_cu >= 1 && workgroups_per_cu <= 8, HK_ERR_INVALID,
+             "%s: 1 to 8 workgroups per compute unit, got %d", who, workgroups_per_cu);
+  HK_REQUIRE(dst && src0 && src1, HK_ERR_INVALID, "%s: null array", who);
+  HK_REQUIRE(aligned16(dst) && aligned16(src0) && aligned16(src1), HK_ERR_INVALID,
+             "%s: arrays must be 16-byte aligned", who);
+  const size_t tile_bytes = size_t(block_threads) * 16;
+  HK_REQUIRE(bytes > 0 && bytes % tile_bytes == 0, HK_ERR_INVALID,
+             "%s: size must be a positive multiple of %zu bytes (whole tiles)", who, tile_bytes);
+  RingArgs a{};
+  a.a = static_cast<const u32x4*>(src0);
+  a.b = static_cast<const u32x4*>(src1);
+  a.d = static_cast<u32x4*>(dst);
+  a.ntiles = long(bytes / tile_bytes);
+  const unsigned grid = unsigned(std::min<size_t>(size_t(a.ntiles), size_t(bench_cu_count()) * workgroups_per_cu));
+  hipStream_t s = as_hip(stream);
+  switch (block_threads) {
+    case 256: return ring_depth<256>(a, depth, barrier, grid, s);
+    case 512: return ring_depth<512>(a, depth, barrier, grid, s);
+    default: return ring_depth<1024>(a, depth, barrier, grid, s);
   }
 }
 

@@ -21,6 +21,15 @@ HK_API int hk_bench_stream_probe(void* dst0, void* dst1, const void* src0, const
                                  size_t bytes, int block_threads, int vectors_per_thread, int nt_loads,
                                  int nt_stores, int workgroups_per_cu, hkStream_t stream);
 
+/* The persistent two-in / one-out walk of hk_bench_stream_probe, software-pipelined the way the backward norm kernels
+ * are: `workgroups_per_cu` (1..8) workgroups of `block_threads` (256, 512, 1024) per compute unit each own every n-th
+ * tile of block_threads vectors and keep a ring of `depth` (1..4) tiles of both inputs in flight per thread; with
+ * `barrier` != 0 every tile also goes through one workgroup barrier and a small LDS exchange (the cost of a row
+ * reduction across wavefronts).  `bytes` per array, a whole number of tiles.  The best depth is the ceiling of that
+ * kernel design whatever arithmetic is put into it. */
+HK_API int hk_bench_ring_probe(void* dst, const void* src0, const void* src1, size_t bytes, int block_threads,
+                               int depth, int barrier, int workgroups_per_cu, hkStream_t stream);
+
 /* Text of the last error this library returned on the calling thread. */
 HK_API const char* hk_bench_last_error(void);
 

@@ -27,7 +27,7 @@ def test_bench_library_is_separate(hk):
     capi = importlib.import_module("hotspa-ae_amd.capi")
     text = open(os.path.join(helpers.ROOT, "include", "hk_bench.h")).read()
     names = sorted(set(re.findall(r"HK_API\s+[\w\s\*]+?\b(hk_\w+)\s*\(", text)))
-    assert names == ["hk_bench_last_error", "hk_bench_stream_probe"]
+    assert names == ["hk_bench_last_error", "hk_bench_ring_probe", "hk_bench_stream_probe"]
     bench = capi.bench_lib()
     for n in names:
         assert hasattr(bench, n) and not hasattr(hk.lib(), n)

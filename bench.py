@@ -86,7 +86,7 @@ def case_rmsnorm(hk, torch, nsets, which):
     for s in sets:
         hk.dropout_add_ln_fwd(s["x"], None, w, None, s["z"], None, s["mu"], s["rs"], eps, True)
     fwd_bytes = 2 * rows * cols * 2 + cols * 2 + rows * 4 + rows * 4
-    bwd_bytes = 3 * rows * cols * 2 + rows * 4 + cols * 2 + 2 * cols * 2
+    bwd_bytes = 3 * rows * cols * 2 + rows * 4 + cols * 2 + cols * 2
 
     def fwd(i):
         s = sets[i % nsets]
@@ -94,7 +94,8 @@ def case_rmsnorm(hk, torch, nsets, which):
 
     def bwd(i):
         s = sets[i % nsets]
-        hk.dropout_add_ln_bwd(s["dz"], None, s["x"], s["mu"], s["rs"], w, s["dx"], None, dg, db, True, workspace=ws)
+        # an RMSNorm has no bias: dx and dgamma are what its backward is asked for
+        hk.dropout_add_ln_bwd(s["dz"], None, s["x"], s["mu"], s["rs"], w, s["dx"], None, dg, None, True, workspace=ws)
 
     if which == "fwd":
         return fwd, fwd_bytes, rows
@@ -126,9 +127,9 @@ def case_rmsnorm_pitched(hk, torch, nsets, which):
                                                 sets[i % nsets]["mu"], sets[i % nsets]["rs"], eps, True)), \
             2 * rows * cols * 2 + cols * 2 + rows * 8, rows
     return (lambda i: hk.dropout_add_ln_bwd(sets[i % nsets]["dz"], None, sets[i % nsets]["x"], sets[i % nsets]["mu"],
-                                            sets[i % nsets]["rs"], w, sets[i % nsets]["dx"], None, dg, db, True,
+                                            sets[i % nsets]["rs"], w, sets[i % nsets]["dx"], None, dg, None, True,
                                             workspace=ws)), \
-        3 * rows * cols * 2 + rows * 4 + cols * 2 + 2 * cols * 2, rows
+        3 * rows * cols * 2 + rows * 4 + cols * 2 + cols * 2, rows
 
 
 def case_rmsnorm_permuted(hk, torch, nsets, which):
@@ -156,9 +157,9 @@ def case_rmsnorm_permuted(hk, torch, nsets, which):
                                                 sets[i % nsets]["mu"], sets[i % nsets]["rs"], eps, True)), \
             2 * rows * cols * 2 + cols * 2 + rows * 8, rows
     return (lambda i: hk.dropout_add_ln_bwd(sets[i % nsets]["dz"], None, sets[i % nsets]["x"], sets[i % nsets]["mu"],
-                                            sets[i % nsets]["rs"], w, sets[i % nsets]["dx"], None, dg, db, True,
+                                            sets[i % nsets]["rs"], w, sets[i % nsets]["dx"], None, dg, None, True,
                                             workspace=ws)), \
-        3 * rows * cols * 2 + rows * 4 + cols * 2 + 2 * cols * 2, rows
+        3 * rows * cols * 2 + rows * 4 + cols * 2 + cols * 2, rows
 
 
 def case_softmax_permuted(hk, torch, nsets, which):

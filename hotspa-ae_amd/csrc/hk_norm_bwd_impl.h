@@ -46,6 +46,10 @@ __device__ __forceinline__ float clamp_by_magnitude(float g, float eps) {
 // without EXTRA, CLAMP says at compile time whether gamma enters dx clamped (the fused
 // LayerNorm's backward does that in both of its modes, the plain one never).
 //
+// The lean RMSNorm instances (MODE == BWD_RMS without EXTRA) form no column sums of dy: an RMSNorm has no bias, and
+// eight additions and eight registers per row and thread are a tenth of the loop.  A caller that asks for dbeta
+// under RMSNorm all the same (the dropout-add-norm interface allows it) is served by the general instance.
+//
 // LEVELS (FIXED instances without optional operands only): the rows lie on several levels (see LevelSteps).  The
 // loads are issued in strictly increasing row order, one grid size apart, so the walk index of the next row to
 // issue is kept as a running (j0, j1, j2) in scalar registers and advanced by the split grid size with two
@@ -59,6 +63,7 @@ void norm_bwd_kernel(NormBwdArgs a) {
   constexpr int VEC = VecIO<T>::N;
   constexpr int NE = NV * VEC;
   constexpr int KS = (MODE == BWD_RMS) ? 1 : 2;   // row sums to reduce: RMSNorm has no mean term
+  constexpr bool WITH_DB = EXTRA || MODE != BWD_RMS;   // column sums of dy (dbeta)
   using StatT = typename std::conditional<STATS_F32, float, T>::type;
   using RowSums = SumTuple<KS>;
   extern __shared__ float lds[];            // [rows_per_block, cols] column-sum staging
@@ -206,7 +211,7 @@ void norm_bwd_kernel(NormBwdArgs a) {
           s.v[0] = fmaf(dz, gm[e], s.v[0]);
           s_prod = fmaf(dz, yb, s_prod);
           dg[e] = fmaf(dz, xhat, dg[e]);
-          db[e] += dz;
+          if constexpr (WITH_DB) db[e] += dz;
           xs[e] = xhat;
           ts[e] = dz * kg;
         } else {
@@ -216,7 +221,7 @@ void norm_bwd_kernel(NormBwdArgs a) {
           s_prod = fmaf(q, xc, s_prod);
           if constexpr (MODE != BWD_RMS) s.v[0] += q;
           dg[e] = fmaf(dzr, xc, dg[e]);
-          db[e] += dz;
+          if constexpr (WITH_DB) db[e] += dz;
           xs[e] = xc;
           // the per-element term of dx uses the clamped gamma when asked to
           if constexpr (decltype(clamped)::value) ts[e] = dzr * clamp_by_magnitude(gm[e], a.eps);
@@ -309,7 +314,7 @@ void norm_bwd_kernel(NormBwdArgs a) {
     // kernel's end)
     static_assert(VEC % 4 == 0, "whole float4 vectors per 16-byte vector of the data type");
 #pragma unroll
-    for (int which = 0; which < 2; ++which) {
+    for (int which = 0; which < (WITH_DB ? 2 : 1); ++which) {
       if (outs[which] == nullptr) continue;
       const float* acc = which == 0 ? dg : db;
       float* dst = outs[which] + int64_t(blockIdx.x) * a.cols;
@@ -326,7 +331,7 @@ void norm_bwd_kernel(NormBwdArgs a) {
     return;
   }
 #pragma unroll
-  for (int which = 0; which < 2; ++which) {
+  for (int which = 0; which < (WITH_DB ? 2 : 1); ++which) {
     if (outs[which] == nullptr) continue;
     float* acc = which == 0 ? dg : db;
     __syncthreads();
@@ -591,7 +596,9 @@ static int launch_norm_bwd_inst(const NormBwdArgs& a, const BwdPlan& p, int pf, 
   // rows on several levels: the lean fixed instances keep a running walk index; every other case splits each row
   // number in the general instance
   const bool levels = a.n0 != a.rows;
-  const bool optional = a.dx_in != nullptr || a.dres != nullptr || (want_clamp && MODE != BWD_LN);
+  // (dbeta under RMSNorm counts as optional: the lean RMSNorm instances do not form it)
+  const bool optional = a.dx_in != nullptr || a.dres != nullptr || (want_clamp && MODE != BWD_LN) ||
+                        (MODE == BWD_RMS && a.part_dbeta != nullptr);
   const bool extra = optional || (levels && !(fixed && exact));
   // the deep ring exists for the plain case only: full rows, no optional operands
   if (!exact || extra) pf = 1;

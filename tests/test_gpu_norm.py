@@ -158,6 +158,37 @@ def test_dropout_add_ln(hk, cuda, dtype, shape, is_rms, residual):
     helpers.assert_close(tdb, edb, dtype, "dbeta")
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("rows,cols", [(1, 4096), (37, 4096), (300, 4096), (515, 2048), (64, 5120), (33, 8192),
+                                       (40, 1000), (7, 264)])
+def test_rmsnorm_bwd_without_dbeta(hk, cuda, dtype, rows, cols):
+    """An RMSNorm has no bias: its backward is asked for dx and dgamma only, and takes the instances that form no
+    column sums of dy.  Against the oracle, and against the same call with dbeta (the general instance)."""
+    import torch
+    eps = 1e-6
+    x, gamma, _, dz = _inputs(rows, cols, dtype, 5100 + cols + rows)
+    tx, tg, tdz = (helpers.to_torch(v, dtype, cuda) for v in (x, gamma, dz))
+    tz, tmu, trs = torch.empty_like(tx), torch.empty(rows, device=cuda), torch.empty(rows, device=cuda)
+    hk.dropout_add_ln_fwd(tx, None, tg, None, tz, None, tmu, trs, eps, True)
+    tdx, tdg = torch.empty_like(tx), torch.empty_like(tg)
+    hk.dropout_add_ln_bwd(tdz, None, tx, tmu, trs, tg, tdx, None, tdg, None, True)
+    tdx2, tdg2, tdb2 = torch.empty_like(tx), torch.empty_like(tg), torch.empty_like(tg)
+    hk.dropout_add_ln_bwd(tdz, None, tx, tmu, trs, tg, tdx2, None, tdg2, tdb2, True)
+    # dx alone: no column sums at all
+    tdx3 = torch.empty_like(tx)
+    hk.dropout_add_ln_bwd(tdz, None, tx, tmu, trs, tg, tdx3, None, None, None, True)
+    torch.cuda.synchronize()
+    mu32, rs32 = helpers.to_numpy(tmu), helpers.to_numpy(trs)
+    edx, edg, edb = oracle.dropout_add_ln_bwd(dz, None, x, mu32, rs32, gamma, True)
+    helpers.assert_close(tdx, edx, dtype, "dx0")
+    helpers.assert_close(tdg, edg, dtype, "dgamma")
+    helpers.assert_close(tdx2, edx, dtype, "dx0")
+    helpers.assert_close(tdg2, edg, dtype, "dgamma")
+    helpers.assert_close(tdb2, edb, dtype, "dbeta")
+    helpers.assert_close(tdx3, edx, dtype, "dx0")
+    assert torch.equal(tdx3, tdx)
+
+
 def test_rmsnorm_bwd_identity(hk, cuda):
     """sum_cols dx*x = eps * rs^3 * sum_cols (gamma*dz)*x per row: pins where eps sits."""
     import torch
@@ -229,6 +260,10 @@ def test_full_size_configs(hk, cuda, cfg):
     hk.dropout_add_ln_fwd(tx, None, tg, None if is_rms else tb, tz, None, tmu, trs, eps, is_rms)
     tdx, tdg, tdb = torch.empty_like(tx), torch.empty_like(tg), torch.empty_like(tg)
     hk.dropout_add_ln_bwd(tdz, None, tx, tmu, trs, tg, tdx, None, tdg, tdb, is_rms)
+    if is_rms:
+        # what an RMSNorm layer asks for: no bias, so no dbeta; the instance that forms no column sums of dy
+        tdx_nb, tdg_nb = torch.empty_like(tx), torch.empty_like(tg)
+        hk.dropout_add_ln_bwd(tdz, None, tx, tmu, trs, tg, tdx_nb, None, tdg_nb, None, True)
     torch.cuda.synchronize()
     sel = helpers.sample_rows(5, rows, 48)
     ez, _, emu, ers = oracle.dropout_add_ln_fwd(x[sel], None, gamma, None if is_rms else beta, eps, is_rms)
@@ -242,6 +277,9 @@ def test_full_size_configs(hk, cuda, cfg):
     yhat = (xd - (0.0 if is_rms else mu32.astype(np.float64)[:, None])) * rs32.astype(np.float64)[:, None]
     helpers.assert_close(tdg, (dzd * yhat).sum(0), dtype, "dgamma")
     helpers.assert_close(tdb, dzd.sum(0), dtype, "dbeta")
+    if is_rms:
+        helpers.assert_close(tdx_nb[sel], edx, dtype, "dx")
+        helpers.assert_close(tdg_nb, (dzd * yhat).sum(0), dtype, "dgamma")
     # per-row invariant of LayerNorm: sum_cols dx == 0 (up to rounding of the stored dx)
     if not is_rms:
         rowsum = tdx.float().sum(1).abs().max().item()

@@ -145,6 +145,17 @@ def test_rmsnorm_on_permuted_views(hk, cuda, case):
     assert torch.equal(vdx0, tdr)
     helpers.assert_close(dg, edg, dt, "dgamma", scale=float(np.sqrt(rows)))
     assert _padding_untouched(wdx0, cols)
+    # the plain backward of an RMSNorm layer on the same views: dx and dgamma only, no residual stream (the lean
+    # instances, with a running walk index where the rows lie on several levels)
+    wdx1, vdx1 = _out_view(vshape, perm, dt, cuda, pad=16)
+    dg1 = torch.empty_like(tw)
+    hk.dropout_add_ln_bwd(vdz, None, vxo, mu, rs, tw, vdx1, None, dg1, None, True)
+    torch.cuda.synchronize()
+    edx1, edg1, _ = oracle.dropout_add_ln_bwd(dz.reshape(rows, cols), None, xsum, helpers.to_numpy(mu),
+                                              helpers.to_numpy(rs), w, True)
+    helpers.assert_close(vdx1.reshape(rows, cols), edx1, dt, "dx0")
+    helpers.assert_close(dg1, edg1, dt, "dgamma", scale=float(np.sqrt(rows)))
+    assert _padding_untouched(wdx1, cols)
 
 
 @pytest.mark.parametrize("dt", ["bf16", "fp32"])

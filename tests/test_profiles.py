@@ -48,7 +48,7 @@ def test_backward_kernel_traffic_constant_matches_the_counter_profile():
     quoted = _bench().NORM_BWD_TRAFFIC_BYTES
     assert abs(quoted - traffic) <= 0.005 * traffic, (quoted, traffic)
     # and the traffic is the algorithmic bytes plus the partial rows, not a re-read: within 2 % above
-    algorithmic = 32768 * (3 * 4096 * 2 + 4) + 3 * 4096 * 2
+    algorithmic = 32768 * (3 * 4096 * 2 + 4) + 2 * 4096 * 2
     assert 1.0 <= traffic / algorithmic < 1.02, traffic / algorithmic
 
 

@@ -636,9 +636,9 @@ CASES = [
 
 
 # HBM bytes one launch of the RMSNorm backward kernel moves at the headline shape: rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE read 262841.3 and 270792.1 KiB per dispatch; a 256 MiB copy kernel calibrates the counters at
-# x1.99993 (FETCH_SIZE reads 131076.5 KiB for 262144 KiB fetched) and x1.00000 (WRITE_SIZE reads 262146.3).
-NORM_BWD_TRAFFIC_BYTES = int((262841.3 * 1.99993 + 270792.1 * 1.0) * 1024)
+# --pmc WRITE_SIZE read 262834.3 and 266598.8 KiB per dispatch; a 256 MiB copy kernel calibrates the counters at
+# x1.99993 (FETCH_SIZE reads 131076.5 KiB for 262144 KiB fetched) and x1.00000 (WRITE_SIZE reads 262145.9).
+NORM_BWD_TRAFFIC_BYTES = int((262834.3 * 1.99993 + 266598.8 * 1.0) * 1024)
 
 
 def preroll(torch, launch, min_steps=PREROLL_MIN_STEPS, min_seconds=PREROLL_MIN_SECONDS):
@@ -1011,7 +1011,7 @@ def main():
         "config": {"workload": "C4 RMSNorm fwd+bwd bf16 [32768 packed tokens x 4096], eps 1e-6, weight U(0.8,1.2)",
                    "rows": rows, "hidden": 4096, "storage": "bf16", "accumulate": "fp32", "us_fwd_plus_bwd": round(ms * 1000, 2),
                    "rows_per_s": round(rows / ms * 1e3), "frac_of_hbm_peak": round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)},
-        "roofline": {"bound": "hbm", "kernel": "norm_bwd_kernel<bf16> (RMSNorm backward, dx + dgamma/dbeta partials)",
+        "roofline": {"bound": "hbm", "kernel": "norm_bwd_kernel<bf16> (RMSNorm backward, dx + dgamma partials)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": NORM_BWD_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_us": round(bwd_us, 2)},

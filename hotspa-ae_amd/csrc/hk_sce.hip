@@ -201,12 +201,14 @@ void sce_sparse_bwd_kernel(SceArgs a) {
 #pragma unroll
   for (int k = 2; k < NV * VEC; k += 2) m = max3(m, e[k], e[k + 1]);
   const float ml = (m == kNegInf) ? 0.f : m * kLog2e;
-  float s = 0.f;
+  // four independent chains, as in the forward kernel
+  float s4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int k = 0; k < NV * VEC; ++k) {
     e[k] = __builtin_amdgcn_exp2f(fmaf(e[k], kLog2e, -ml));
-    s += e[k];
+    s4[k & 3] += e[k];
   }
+  const float s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
   MaxSumTuple p;
   p.v[0] = (m == kNegInf) ? kNegInf : ml; p.v[1] = s;
   p = WAVE_ROW ? wave_allreduce_tuple(p) : group_allreduce_tuple(p, red, 0, nwaves);

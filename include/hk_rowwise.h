@@ -244,7 +244,10 @@ HK_API int hk_dropout_add_ln_fwd(int itype, int rtype, int wtype, const void* x0
 /* dz: [rows, cols] `itype`; dx_in (optional): upstream gradient of the
  * pre-norm sum (`rtype`), added to dx; x: [rows, cols] `rtype`; dx0: [rows,
  * cols] `itype`; dresidual (optional): `rtype`; dgamma, dbeta: [cols] `wtype`
- * (dbeta may be NULL).  (ln_bwd_kernels.cuh:126-221, finalize :301-442) */
+ * (either may be NULL).  An RMSNorm layer has no bias and passes dbeta = NULL, as the reference's RMSNorm operator
+ * does when it was given no beta (hetu/graph/ops/RMSNorm.cc:156): that call takes the instances that form no
+ * column sums of dy; dbeta under is_rms_norm is computed all the same when asked for, by a more general and
+ * slightly slower instance.  (ln_bwd_kernels.cuh:126-221, finalize :301-442) */
 HK_API int hk_dropout_add_ln_bwd(int itype, int rtype, int wtype, const void* dz,
                                  const void* dx_in, const void* x, const void* mu,
                                  const void* rsigma, const void* gamma, void* dx0,

@@ -523,7 +523,37 @@ def test_every_instruction_set_variant_of_the_host_loops(level):
     import sys
     env = dict(os.environ, HETU_HOST_ISA=str(level))
     picked = ("test_layer_norm_and_gradient or test_softmax_and_gradient or test_sparse_cross_entropy_and_gradient "
-              "or test_reduce_every_axis_subset or test_unary_and_constants or test_batch_norm_and_gradient")
+              "or test_reduce_every_axis_subset or test_unary_and_constants or test_batch_norm_and_gradient "
+              "or test_special_values_go_through_the_vector_loops")
     run = subprocess.run([sys.executable, "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-k", picked,
                           "-p", "no:cacheprovider"], env=env, cwd=helpers.ROOT, capture_output=True, text=True)
     assert run.returncode == 0, run.stdout[-3000:] + run.stderr[-2000:]
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_special_values_go_through_the_vector_loops(ht, dtype):
+    """-inf elements, a row of -inf only, +inf, NaN, a large common offset and an overflowing exponent: the
+    branch-free exp and the lane-wise maxima give what the scalar library calls give."""
+    import torch
+    inf, nan = float("inf"), float("nan")
+    dt = torch.float32 if dtype == "fp32" else torch.bfloat16
+    x = torch.from_numpy(_draw(91, (6, 200), "fp32")).to(dt)
+    x[0, 3] = -inf
+    x[1, :] = -inf
+    x[2, 5] = inf
+    x[3, 7] = nan
+    x[4, :] += 1e4
+    x[5, 0] = 200.0
+    y = torch.empty_like(x)
+    ht.softmax(x, y, 1)
+    ref = torch.softmax(x.double(), 1)
+    assert torch.equal(torch.isnan(y), torch.isnan(ref))
+    tol = 1e-5 if dtype == "fp32" else 1e-2
+    assert torch.allclose(torch.nan_to_num(y.double()), torch.nan_to_num(ref), rtol=tol, atol=1e-7)
+    e = torch.empty_like(x)
+    ht.unary("exp", x, e)
+    re = torch.exp(x.double()).to(dt)          # overflow where the type overflows
+    assert torch.equal(torch.isnan(e), torch.isnan(re)) and torch.equal(torch.isinf(e), torch.isinf(re))
+    fin = torch.isfinite(re)
+    assert torch.allclose(e[fin].double(), re[fin].double(), rtol=tol, atol=0)
+    assert float(e[1].abs().max()) == 0.0      # exp(-inf) is exactly 0

@@ -750,8 +750,9 @@ def cpu_baseline(rows=32768, cols=4096, budget_s=2.0):
 
 
 def cpu_baselines(budget_s=0.5):
-    """Per BASELINE configuration kernel, three host figures on a bounded sample of the configuration's rows, in the
-    configuration's storage type, counting the same algorithmic bytes per row as the GPU entry:
+    """Per BASELINE configuration kernel, three host figures on a bounded sample of the configuration's rows (at least
+    128 MB of input each, so that the sample does not sit in the last-level cache), in the configuration's storage
+    type, counting the same algorithmic bytes per row as the GPU entry:
       * kind "port": the host twin of the kernel (LayerNormCpu / LayerNormGradientCpu, SoftmaxCpu / SoftmaxGradientCpu,
         SoftmaxCrossEntropySparseCpu / ...GradientCpu, ReduceCpu: the reference's CPU pass structure as fp32 loops,
         OpenMP over rows), called through the same operator entry points and device dispatch as the accelerator
@@ -796,8 +797,8 @@ def cpu_baselines(budget_s=0.5):
                 dt, reps = _timed_cpu(torch_fn, budget_s)
             rec("torch-cpu (oneDNN-class)", cores, dt, reps, torch_bytes or algo_bytes, torch_what)
 
-    # C1: a quarter of the configuration, fp32 storage
-    rows, cols = 2048, 4096
+    # C1: the whole configuration, fp32 storage
+    rows, cols = 8192, 4096
     x = block(rows, cols, torch.float32); y = torch.empty_like(x)
     gm, bt = torch.ones(cols), torch.zeros(cols)
     mean, var = torch.empty(rows, 1), torch.empty(rows, 1)
@@ -805,8 +806,8 @@ def cpu_baselines(budget_s=0.5):
         lambda: ops.layer_norm(x, gm, bt, mean, var, y, 1, 1e-5),
         lambda: torch.ops.aten.native_layer_norm(x, [cols], gm, bt, 1e-5),
         rows * (2 * cols * 4 + 8), rows, 8192, "torch native_layer_norm")
-    # C5 layer norm at 5120 columns, forward and gradient, 1/8 of the rows, bf16 storage
-    rows, cols = 2048, 5120
+    # C5 layer norm at 5120 columns, forward and gradient, 3/4 of the rows, bf16 storage
+    rows, cols = 12288, 5120
     x5 = block(rows, cols, bf); y5 = torch.empty_like(x5); dy5 = block(rows, cols, bf); dx5 = torch.empty_like(x5)
     gm5, bt5 = torch.ones(cols, dtype=bf), torch.zeros(cols, dtype=bf)
     mean5, var5 = torch.empty(rows, 1, dtype=bf), torch.empty(rows, 1, dtype=bf)
@@ -820,16 +821,16 @@ def cpu_baselines(budget_s=0.5):
         lambda: ops.layer_norm_gradient(dy5, x5, gm5, dx5, dgm, dbt, mean5, var5, 1, 1e-5),
         lambda: torch.ops.aten.native_layer_norm_backward(dy5, x5, [cols], tmean, trstd, gm5, bt5, [True, True, True]),
         rows * (3 * cols * 2 + 8), rows, 16384, "torch native_layer_norm_backward")
-    # C2: 1/64 of the rows
-    rows, cols = 4096, 2048
+    # C2: 1/8 of the rows
+    rows, cols = 32768, 2048
     x2 = block(rows, cols, bf); y2 = torch.empty_like(x2); dx2 = torch.empty_like(x2)
     add("C2", "softmax fwd bf16 [4,32,2048,2048] (SoftmaxCpu)", lambda: ops.softmax(x2, y2, 1),
         lambda: torch.softmax(x2, -1), 2 * rows * cols * 2, rows, 262144, "torch.softmax")
     add("C2", "softmax bwd bf16 [4,32,2048,2048] (SoftmaxGradientCpu)", lambda: ops.softmax_gradient(y2, x2, dx2, 1),
         lambda: torch.ops.aten._softmax_backward_data(x2, y2, -1, bf), 3 * rows * cols * 2, rows, 262144,
         "torch _softmax_backward_data")
-    # C3: 1/8 of the rows
-    rows, cols = 4096, 4096
+    # C3: half of the rows
+    rows, cols = 16384, 4096
     x3 = block(rows, cols, bf); o0 = torch.empty(cols, dtype=bf); o1 = torch.empty(rows, dtype=bf)
     for name, axes, o in (("axis 1", [1], o1), ("axis 0", [0], o0)):
         for red in ("sum", "mean"):
@@ -838,8 +839,8 @@ def cpu_baselines(budget_s=0.5):
                 red, name, "; also the merged axes (0,1) of [64x512x4096]" if (axes == [0] and red == "sum") else ""),
                 (lambda axes=axes, o=o, red=red: ops.reduce(x3, o, axes, red)), tfn, rows * cols * 2, rows, 32768,
                 "torch.%s" % red)
-    # C5 cross-entropy: 1/64 of the rows
-    rows, cols = 256, 32000
+    # C5 cross-entropy: 1/8 of the rows
+    rows, cols = 2048, 32000
     xc = block(rows, cols, bf); loss = torch.empty(rows, dtype=bf); dxc = torch.empty_like(xc)
     gl = torch.full((rows,), 1.0 / 16384, dtype=bf)
     lab = (torch.arange(rows, dtype=torch.int64) * 31) % cols
